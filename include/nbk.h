@@ -1,0 +1,305 @@
+/*
+ * nbk.h -- C ABI of libnbk.so, the gfx950 kernel library behind the nabla_amd
+ * execution backend.
+ *
+ * The reference (nabla-ml/nabla) has no native code of its own: every
+ * Operation.kernel() calls a `max.graph.ops.*` builder and the engine hands the
+ * finished graph to `InferenceSession.load(graph)` / `model(*buffers)`
+ * (nabla/core/graph/engine.py:656-663).  This header is what replaces those
+ * MAX call sites on one MI355X.  Each entry point cites the reference call site
+ * whose arithmetic it takes over.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; device pointers are raw HIP addresses
+ *   - every launch goes onto the hipStream_t passed as `void* stream`
+ *     (NULL = the legacy default stream)
+ *   - kernels never allocate: the caller owns inputs, outputs and workspace
+ *   - return value: 0 on success, negative nbk_status otherwise;
+ *     nbk_last_error() returns a thread-local message for the last failure
+ *   - the library keeps no mutable global state besides that message
+ */
+#ifndef NBK_H_
+#define NBK_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ status */
+enum nbk_status {
+  NBK_OK = 0,
+  NBK_ERR_INVALID = -1,   /* bad argument (shape, dtype, alignment, limits) */
+  NBK_ERR_LAUNCH = -2,    /* HIP reported a launch / runtime error          */
+  NBK_ERR_UNSUPPORTED = -3
+};
+
+/* ------------------------------------------------------------------ dtypes */
+enum nbk_dtype {
+  NBK_F32 = 0,
+  NBK_BF16 = 1,
+  NBK_F16 = 2,
+  NBK_I32 = 3,
+  NBK_I64 = 4,
+  NBK_U8 = 5    /* also bool: 0 / 1 */
+};
+
+/* --------------------------------------------------------------- lifecycle */
+/* Select the device, query it, and make sure it is a gfx950 part.
+ * Replaces the session singleton of nabla/core/common/context.py:120-139. */
+int nbk_init(int device);
+const char* nbk_last_error(void);
+/* ABI version of this header; the ctypes shim refuses a mismatch. */
+int nbk_abi_version(void);
+#define NBK_ABI_VERSION 3
+
+/* ===================================================================== */
+/*  Row programs: fused elementwise chains + last-axis reductions         */
+/* ===================================================================== */
+/*
+ * One kernel family executes every fused group of elementwise ops
+ * (nabla/ops/binary.py:18-156, unary.py:20-697, comparison.py:63-130,
+ * control_flow.py:21-141 WhereOp, creation.py fills/arange/tril) together
+ * with the single-axis keepdims reductions over the LAST axis that the
+ * reference emits as ops.sum / ops.mean / ops._reduce_max
+ * (nabla/ops/reduction.py:147-245), including softmax / logsoftmax
+ * (unary.py:192-230, 598-632) and layer_norm (nn/functional/layers.py:38-56)
+ * once the lowering pass has fused their primitive ops.
+ *
+ * Iteration domain: rows x C, rows = prod(lead_dim[0..n_lead)).
+ * An operand is addressed as
+ *     ptr[ sum_k lead_idx[k]*lead_stride[k] + col*col_stride ]   (elements)
+ * so broadcasts (stride 0), row vectors (col_stride 0), column vectors
+ * (all lead strides 0) and transposed views are all the same thing.
+ *
+ * The program is a stream of 8-byte instructions interpreted by every lane.
+ * Registers: 16 vector registers (4 consecutive columns each) numbered 0..15
+ * and 16 per-row scalar registers numbered 16..31.  A program is
+ *     { prologue ; BODY n ; n body instructions } ... HALT
+ * Prologue instructions run once per row on scalar registers; body
+ * instructions run once per 4-column chunk.
+ */
+#define NBK_RP_MAX_OPERANDS 20
+#define NBK_RP_MAX_INS 224
+#define NBK_RP_MAX_IMM 24
+#define NBK_RP_MAX_LEAD 4
+#define NBK_RP_NVEC 16
+#define NBK_RP_NSCL 16
+#define NBK_RP_NACC 4
+#define NBK_RP_MAX_STAGE 4
+
+typedef struct nbk_operand {
+  void* ptr;                           /* device address of element 0          */
+  int64_t lead_stride[NBK_RP_MAX_LEAD];/* element strides of the leading dims  */
+  int32_t col_stride;                  /* element stride along the row axis    */
+  int32_t dtype;                       /* nbk_dtype                            */
+  int32_t vec_ok;                      /* 1: 4 columns can move as one access  */
+  int32_t stage_slot;                  /* >=0: row is pre-loaded into LDS slot */
+} nbk_operand;
+
+typedef struct nbk_ins {
+  uint8_t op;    /* nbk_rp_op                                         */
+  uint8_t dst;   /* register, accumulator index or operand index      */
+  uint8_t a, b, c; /* source registers / operand index / immediate id */
+  uint8_t pad;
+  uint16_t aux;  /* BODY: number of body instructions                 */
+} nbk_ins;
+
+enum nbk_rp_op {
+  NBK_OP_HALT = 0,
+  /* structure */
+  NBK_OP_BODY = 1,     /* aux = body length                                    */
+  /* memory (a = operand index) */
+  NBK_OP_LDG = 2,      /* body: vreg dst <- operand a, 4 columns               */
+  NBK_OP_STG = 3,      /* body: operand dst <- vreg a                          */
+  NBK_OP_LDR = 4,      /* prologue: sreg dst <- operand a at column 0          */
+  NBK_OP_STR = 5,      /* prologue: operand dst <- sreg a (column 0, 1 lane)   */
+  NBK_OP_IMM = 6,      /* prologue: sreg dst <- imm[a]                         */
+  NBK_OP_COLIDX = 7,   /* body: vreg dst <- column index as float              */
+  NBK_OP_LEADIDX = 8,  /* prologue: sreg dst <- index along leading dim a      */
+  /* reductions over the row */
+  NBK_OP_ACCINIT = 9,  /* prologue: acc dst <- identity of kind a              */
+  NBK_OP_ACC = 10,     /* body: acc dst <- combine(acc, vreg a), kind b        */
+  NBK_OP_RED = 11,     /* prologue: sreg dst <- block-reduce(acc a), kind b    */
+  /* unary  dst <- f(a) */
+  NBK_OP_MOV = 16, NBK_OP_NEG = 17, NBK_OP_RELU = 18, NBK_OP_EXP = 19,
+  NBK_OP_LOG = 20, NBK_OP_SQRT = 21, NBK_OP_RSQRT = 22, NBK_OP_ERF = 23,
+  NBK_OP_GELU = 24, NBK_OP_TANH = 25, NBK_OP_SIGMOID = 26, NBK_OP_ABS = 27,
+  NBK_OP_RBF16 = 28,   /* round to bf16 and back                               */
+  NBK_OP_NOT = 29,     /* 1 - a  on 0/1 values                                 */
+  NBK_OP_TRUNC = 30,   /* round toward zero (float -> integer casts)           */
+  NBK_OP_NEZ = 31,     /* a != 0 -> 1/0 (casts to bool)                        */
+  /* binary dst <- f(a, b) */
+  NBK_OP_ADD = 32, NBK_OP_SUB = 33, NBK_OP_MUL = 34, NBK_OP_DIV = 35,
+  NBK_OP_MAX = 36, NBK_OP_MIN = 37, NBK_OP_GT = 38, NBK_OP_GE = 39,
+  NBK_OP_EQ = 40, NBK_OP_NE = 41, NBK_OP_LT = 42, NBK_OP_LE = 43,
+  NBK_OP_POW = 44, NBK_OP_AND = 45, NBK_OP_OR = 46,
+  /* ternary */
+  NBK_OP_WHERE = 48,   /* dst <- a != 0 ? b : c                                */
+  NBK_OP_FMA = 49      /* dst <- a * b + c                                     */
+};
+
+enum nbk_red_kind { NBK_RED_SUM = 0, NBK_RED_MAX = 1, NBK_RED_MIN = 2 };
+
+typedef struct nbk_rowprog {
+  int64_t lead_dim[NBK_RP_MAX_LEAD];
+  int64_t C;              /* row length                                        */
+  int32_t n_lead;
+  int32_t n_operands;
+  int32_t n_ins;
+  int32_t n_imm;
+  int32_t has_reduce;     /* 0: flat launch, 1: one workgroup per row          */
+  int32_t block;          /* workgroup size for has_reduce=1 (64..512, pow2)   */
+  int32_t n_stage;        /* operands pre-loaded into LDS (has_reduce=1 only)  */
+  int32_t reserved;
+  float imm[NBK_RP_MAX_IMM];
+  nbk_operand operand[NBK_RP_MAX_OPERANDS];
+  nbk_ins ins[NBK_RP_MAX_INS];
+} nbk_rowprog;
+
+int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream);
+
+/* ===================================================================== */
+/*  Reductions over a middle / leading axis                               */
+/* ===================================================================== */
+/* in: contiguous [outer, red, inner] -> out: contiguous [outer, inner].
+ * Covers the inner>1 cases of nabla/ops/reduction.py:147-245 that the
+ * autodiff un-broadcast emits (nabla/core/autograd/backward.py:31-54),
+ * e.g. bias and layer-norm weight gradients.  kind: nbk_red_kind. */
+int nbk_reduce_mid(const void* in, void* out, int32_t dtype_in, int32_t dtype_out,
+                   int64_t outer, int64_t red, int64_t inner, int32_t kind,
+                   void* stream);
+
+/* ===================================================================== */
+/*  Strided copy (materialise a view)                                     */
+/* ===================================================================== */
+/* dst (contiguous, row-major over shape) <- src viewed with src_stride.
+ * Serves permute / swap_axes / broadcast_to / slice_tensor / pad /
+ * concatenate / slice_update when a consumer cannot fold the view
+ * (nabla/ops/view/shape.py:56-158, 586-980, 1313-1398; view/axes.py:43-868).
+ * dst_stride may also be strided (writes into a window of a larger buffer). */
+#define NBK_MAX_RANK 8
+int nbk_copy_strided(const void* src, void* dst, int32_t dtype_src, int32_t dtype_dst,
+                     int32_t rank, const int64_t* shape, const int64_t* src_stride,
+                     const int64_t* dst_stride, void* stream);
+/* Fill a contiguous buffer with a constant (creation.py:50-93). */
+int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void* stream);
+
+/* ===================================================================== */
+/*  GEMM                                                                  */
+/* ===================================================================== */
+/* C[b] = alpha * op(A[b]) @ op(B[b]) (+ bias) (+ residual) with optional
+ * activation; replaces ops.matmul at nabla/ops/binary.py:198 for the forward
+ * product and for both backward products of MatmulOp.vjp_rule
+ * (binary.py:303-314), whose swap_axes are folded into the strides here.
+ * A is M x K with element strides (a_rs, a_cs), B is K x N with (b_rs, b_cs);
+ * one of the two strides of each must be 1.  C is row-major with leading
+ * dimension ldc.  Batches are strided (stride 0 = broadcast).
+ * `batch_reduce` != 0 sums the products of all batches into ONE C
+ * (dW of a 3-D activation against a 2-D weight: backward.py:36-41).
+ * dtype_ab: NBK_F32 or NBK_BF16; accumulation is always fp32. */
+enum nbk_gemm_act { NBK_ACT_NONE = 0, NBK_ACT_RELU = 1, NBK_ACT_GELU = 2 };
+typedef struct nbk_gemm_desc {
+  const void* A; const void* B; void* C;
+  const void* bias;      /* NULL or [N] (dtype_c), added to every row        */
+  const void* residual;  /* NULL or same layout as C, added after activation */
+  int64_t M, N, K;
+  int64_t a_rs, a_cs, b_rs, b_cs, ldc;
+  int64_t batch, a_bs, b_bs, c_bs;
+  int32_t dtype_ab, dtype_c;
+  int32_t act;
+  int32_t batch_reduce;
+  float alpha;
+  int32_t reserved;
+} nbk_gemm_desc;
+int nbk_gemm(const nbk_gemm_desc* d, void* stream);
+
+/* ===================================================================== */
+/*  Convolution / pooling (NHWC x HWIO)                                   */
+/* ===================================================================== */
+/* Replaces ops.conv2d at nabla/ops/convolution.py:252 and the two products
+ * of Conv2DOp.vjp_rule (convolution.py:309-392): dgrad (the conv2d_transpose
+ * + pad + slice sequence) and wgrad (the conv of permuted tensors).
+ * x [N,H,W,Cin], w [R,S,Cin,Cout], y [N,Ho,Wo,Cout]; fp32; dilation 1,
+ * groups 1 as the reference validates (convolution.py:602-696). */
+typedef struct nbk_conv_desc {
+  int64_t N, H, W, Cin, R, S, Cout, Ho, Wo;
+  int32_t stride_h, stride_w;
+  int32_t pad_t, pad_b, pad_l, pad_r;
+  int32_t dtype;      /* NBK_F32 */
+  int32_t reserved;
+} nbk_conv_desc;
+int nbk_conv2d_fwd(const nbk_conv_desc* d, const void* x, const void* w,
+                   const void* bias, void* y, void* stream);
+int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const void* w,
+                     void* dx, void* stream);
+int nbk_conv2d_wgrad(const nbk_conv_desc* d, const void* x, const void* dy,
+                     void* dw, void* stream);
+
+/* max_pool2d forward/backward; replaces the per-window slice + reduce_max +
+ * stack graph of nabla/ops/pooling.py:53-137.  Backward follows the
+ * reduce_max tie rule (reduction.py:219-230): every element equal to the
+ * window maximum receives the full cotangent.  Windows are clipped at the
+ * padded border (pooling.py:111-130). */
+typedef struct nbk_pool_desc {
+  int64_t N, H, W, C, Ho, Wo;
+  int32_t kh, kw, stride_h, stride_w, pad_t, pad_l;
+  int32_t dtype;
+  int32_t reserved;
+} nbk_pool_desc;
+int nbk_maxpool2d_fwd(const nbk_pool_desc* d, const void* x, void* y, void* stream);
+int nbk_maxpool2d_bwd(const nbk_pool_desc* d, const void* x, const void* y,
+                      const void* dy, void* dx, void* stream);
+
+/* ===================================================================== */
+/*  Index ops (bit-exact)                                                 */
+/* ===================================================================== */
+/* out[o, j, i] = table[o, idx[j], i]; replaces ops.gather at
+ * nabla/ops/view/indexing.py:171 (embedding: nn/functional/layers.py:84-98).
+ * Negative indices wrap once; out-of-range indices are an error reported
+ * through `status` (a device int32 the caller zeroes; set to 1 on error). */
+int nbk_gather(const void* table, const void* idx, void* out, int32_t dtype,
+               int32_t idx_dtype, int64_t outer, int64_t axis_len, int64_t n_idx,
+               int64_t inner, int32_t* status, void* stream);
+/* out[r] = index of the first maximum of in[r, 0..C) as int64; replaces
+ * ops.argmax at nabla/ops/reduction.py:745-765. */
+int nbk_argmax_rows(const void* in, int64_t* out, int32_t dtype, int64_t rows,
+                    int64_t C, int32_t want_min, void* stream);
+
+/* ===================================================================== */
+/*  Custom kernels                                                        */
+/* ===================================================================== */
+/* Contract of a user kernel library loaded by call_custom_kernel
+ * (nabla/ops/utils.py:765-824; tests/mojo/kernels/custom_kernel.mojo:12-26):
+ * a shared object exporting, per registered name,
+ *     int <name>(const nbk_tensor* in, int n_in,
+ *                nbk_tensor* out, int n_out, void* stream);
+ * nbk_custom() resolves and calls it, and verifies the symbol exists. */
+typedef struct nbk_tensor {
+  void* ptr;
+  int32_t dtype;
+  int32_t rank;
+  int64_t shape[NBK_MAX_RANK];
+  int64_t stride[NBK_MAX_RANK];
+} nbk_tensor;
+typedef int (*nbk_custom_fn)(const nbk_tensor* in, int n_in, nbk_tensor* out,
+                             int n_out, void* stream);
+int nbk_custom(const char* library_path, const char* name, const nbk_tensor* in,
+               int n_in, nbk_tensor* out, int n_out, void* stream);
+
+/* ===================================================================== */
+/*  Measurement helpers                                                   */
+/* ===================================================================== */
+/* HIP events on the caller's stream, so that bench code can time the very
+ * stream the kernels run on. */
+int nbk_event_create(void** ev);
+int nbk_event_record(void* ev, void* stream);
+int nbk_event_elapsed_ms(void* start, void* stop, float* ms); /* syncs stop */
+int nbk_event_destroy(void* ev);
+int nbk_stream_sync(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NBK_H_ */

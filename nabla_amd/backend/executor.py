@@ -1,0 +1,322 @@
+"""Plan execution on the GPU through libnbk.so.
+
+``HipExecutor`` is the product path: it binds the plan's buffers to device
+addresses (inputs and outputs are torch allocations used as plain memory,
+intermediates live in one arena per plan) and issues every step as a call
+into the C ABI of include/nbk.h on the current HIP stream.  It refuses to
+work without the built library and a gfx950 device -- there is no CPU path
+in this package.  The executor is replaceable (``set_executor``) only so that
+host-side logic can be unit-tested against a reference interpreter of the
+same launch records.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Any, Sequence
+
+import torch
+
+from ..core.dtype import DType
+from . import isa, lib
+from .planner import Plan, Step, ViewRef
+
+_RED = {"sum": 0, "max": 1, "min": 2}
+
+
+class BoundPlan:
+    """A plan with its ctypes launch records prepared once.
+
+    Only the addresses of plan inputs and outputs change from run to run; they
+    are patched into the prepared records before launch."""
+
+    def __init__(self, plan: Plan, ex: "HipExecutor"):
+        self.plan = plan
+        self.ex = ex
+        self.arena = None
+        if plan.arena_bytes > 0:
+            self.arena = torch.empty(plan.arena_bytes, dtype=torch.uint8, device=ex.torch_device)
+        self.base: list[int] = [0] * len(plan.bufs)
+        if self.arena is not None:
+            a0 = self.arena.data_ptr()
+            for b in plan.bufs:
+                if b.role == "temp" and b.offset >= 0:
+                    self.base[b.id] = a0 + b.offset
+        self.dynamic = [b.id for b in plan.bufs if b.role in ("input", "output")]
+        self.calls: list[tuple] = []  # (fn, args tuple, patch list)
+        self._prepare()
+
+    # -- address helpers -------------------------------------------------------
+    def _addr(self, ref: ViewRef) -> int:
+        return self.base[ref.buf] + ref.offset * ref.dtype.size_in_bytes
+
+    def _prepare(self) -> None:
+        L = self.ex.lib
+        plan = self.plan
+        dyn = set(self.dynamic)
+        for st in plan.steps:
+            a = st.attrs
+            k = st.kind
+            patches: list = []  # (setter(addr_of_buf)) closures
+
+            def ptr_field(obj, field, buf: int, byte_off: int):
+                """Set obj.field = base[buf] + byte_off now, and again per run if dynamic."""
+                setattr(obj, field, self.base[buf] + byte_off)
+                if buf in dyn:
+                    patches.append((obj, field, buf, byte_off))
+
+            if k == "rowprog":
+                rp = lib.RowProg()
+                lead = a["lead"]
+                rp.n_lead = len(lead)
+                for i, d in enumerate(lead):
+                    rp.lead_dim[i] = d
+                rp.C = a["C"]
+                rp.n_operands = len(a["operands"])
+                rp.n_ins = len(a["ins"])
+                rp.n_imm = len(a["imm"])
+                rp.has_reduce = 1 if a["has_reduce"] else 0
+                rp.block = a["block"]
+                rp.n_stage = a["n_stage"]
+                for i, v in enumerate(a["imm"]):
+                    rp.imm[i] = v
+                for i, o in enumerate(a["operands"]):
+                    od = rp.operand[i]
+                    for j, s in enumerate(o.lead_strides):
+                        od.lead_stride[j] = s
+                    od.col_stride = o.col_stride
+                    od.dtype = o.dtype.abi
+                    od.vec_ok = 1 if o.vec_ok else 0
+                    od.stage_slot = o.stage_slot
+                    ptr_field(od, "ptr", o.buf, o.offset * o.dtype.size_in_bytes)
+                for i, ins in enumerate(a["ins"]):
+                    d = rp.ins[i]
+                    d.op, d.dst, d.a, d.b, d.c, d.aux = ins[0], ins[1], ins[2], ins[3], ins[4], ins[5]
+                self.calls.append((L.nbk_rowprog_launch, [C.byref(rp)], patches, rp))
+            elif k == "copy":
+                src, dst = a["src"], a["dst"]
+                rank = len(src.shape)
+                shape = (C.c_int64 * max(rank, 1))(*src.shape)
+                ss = (C.c_int64 * max(rank, 1))(*src.strides)
+                ds = (C.c_int64 * max(rank, 1))(*dst.strides)
+                holder = _Ptrs(2)
+                ptr_field(holder, "p0", src.buf, src.offset * src.dtype.size_in_bytes)
+                ptr_field(holder, "p1", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                self.calls.append((L.nbk_copy_strided,
+                                   [holder, ("p0", "p1"), src.dtype.abi, dst.dtype.abi, rank, shape,
+                                    ss, ds], patches, None))
+            elif k == "fill":
+                holder = _Ptrs(1)
+                ptr_field(holder, "p0", a["buf"], 0)
+                self.calls.append((L.nbk_fill, [holder, ("p0",), a["dtype"].abi, a["numel"],
+                                                float(a["value"])], patches, None))
+            elif k == "reduce_mid":
+                src, dst = a["src"], a["dst"]
+                holder = _Ptrs(2)
+                ptr_field(holder, "p0", src.buf, src.offset * src.dtype.size_in_bytes)
+                ptr_field(holder, "p1", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                self.calls.append((L.nbk_reduce_mid,
+                                   [holder, ("p0", "p1"), src.dtype.abi, dst.dtype.abi, a["outer"],
+                                    a["red"], a["inner"], _RED[a["fn"]]], patches, None))
+            elif k == "gemm":
+                d = lib.GemmDesc()
+                ra, rb, rc = a["a"], a["b"], a["dst"]
+                ptr_field(d, "A", ra.buf, ra.offset * ra.dtype.size_in_bytes)
+                ptr_field(d, "B", rb.buf, rb.offset * rb.dtype.size_in_bytes)
+                ptr_field(d, "C", rc.buf, rc.offset * rc.dtype.size_in_bytes)
+                d.bias = None
+                d.residual = None
+                d.M, d.N, d.K = a["M"], a["N"], a["K"]
+                d.a_rs, d.a_cs, d.b_rs, d.b_cs = a["a_rs"], a["a_cs"], a["b_rs"], a["b_cs"]
+                d.ldc = a["ldc"]
+                d.batch, d.a_bs, d.b_bs, d.c_bs = a["batch"], a["a_bs"], a["b_bs"], a["c_bs"]
+                if ra.dtype is not rb.dtype:
+                    raise TypeError(f"matmul operands differ in dtype: {ra.dtype} vs {rb.dtype}")
+                d.dtype_ab = ra.dtype.abi
+                d.dtype_c = rc.dtype.abi
+                d.act = 0
+                d.batch_reduce = 0
+                d.alpha = a.get("alpha", 1.0)
+                self.calls.append((L.nbk_gemm, [C.byref(d)], patches, d))
+            elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
+                d = lib.ConvDesc()
+                xs, ws, ys = a["x_shape"], a["w_shape"], a["y_shape"]
+                d.N, d.H, d.W, d.Cin = xs
+                d.R, d.S, _, d.Cout = ws
+                d.Ho, d.Wo = ys[1], ys[2]
+                d.stride_h, d.stride_w = a["stride"]
+                d.pad_t, d.pad_b, d.pad_l, d.pad_r = a["padding"]
+                d.dtype = a["dst"].dtype.abi
+                n_ptr = 4 if k == "conv2d" else 3
+                holder = _Ptrs(4)
+                refs = list(a["ins"])
+                if k == "conv2d" and not a["has_bias"]:
+                    refs.append(None)
+                refs.append(a["dst"])
+                names = []
+                for i, r in enumerate(refs):
+                    nm = f"p{i}"
+                    names.append(nm)
+                    if r is None:
+                        setattr(holder, nm, None)
+                    else:
+                        ptr_field(holder, nm, r.buf, r.offset * r.dtype.size_in_bytes)
+                fn = {"conv2d": L.nbk_conv2d_fwd, "conv2d_dgrad": L.nbk_conv2d_dgrad,
+                      "conv2d_wgrad": L.nbk_conv2d_wgrad}[k]
+                self.calls.append((fn, [C.byref(d), holder, tuple(names[:n_ptr])], patches, d))
+            elif k in ("maxpool2d", "maxpool2d_bwd"):
+                d = lib.PoolDesc()
+                xs, ys = a["x_shape"], a["y_shape"]
+                d.N, d.H, d.W, d.C = xs
+                d.Ho, d.Wo = ys[1], ys[2]
+                d.kh, d.kw = a["kernel"]
+                d.stride_h, d.stride_w = a["stride"]
+                d.pad_t, d.pad_l = a["padding"][0], a["padding"][2]
+                d.dtype = a["dst"].dtype.abi
+                refs = list(a["ins"]) + [a["dst"]]
+                holder = _Ptrs(4)
+                names = []
+                for i, r in enumerate(refs):
+                    nm = f"p{i}"
+                    names.append(nm)
+                    ptr_field(holder, nm, r.buf, r.offset * r.dtype.size_in_bytes)
+                fn = L.nbk_maxpool2d_fwd if k == "maxpool2d" else L.nbk_maxpool2d_bwd
+                self.calls.append((fn, [C.byref(d), holder, tuple(names)], patches, d))
+            elif k == "gather":
+                t, ix, dst = a["table"], a["idx"], a["dst"]
+                holder = _Ptrs(3)
+                ptr_field(holder, "p0", t.buf, t.offset * t.dtype.size_in_bytes)
+                ptr_field(holder, "p1", ix.buf, ix.offset * ix.dtype.size_in_bytes)
+                ptr_field(holder, "p2", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                self.calls.append((L.nbk_gather,
+                                   [holder, ("p0", "p1", "p2"), t.dtype.abi, ix.dtype.abi, a["outer"],
+                                    a["axis_len"], a["n_idx"], a["inner"],
+                                    C.c_void_p(self.ex.status_flag.data_ptr())], patches, None))
+            elif k == "argreduce":
+                src, dst = a["src"], a["dst"]
+                holder = _Ptrs(2)
+                ptr_field(holder, "p0", src.buf, src.offset * src.dtype.size_in_bytes)
+                ptr_field(holder, "p1", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                self.calls.append((L.nbk_argmax_rows,
+                                   [holder, ("p0", "p1"), src.dtype.abi, a["rows"], a["C"],
+                                    1 if a["fn"] == "min" else 0], patches, None))
+            elif k == "custom":
+                ins = (lib.TensorDesc * max(len(a["ins"]), 1))()
+                outs = (lib.TensorDesc * len(a["dsts"]))()
+                for arr, refs in ((ins, a["ins"]), (outs, a["dsts"])):
+                    for i, r in enumerate(refs):
+                        t = arr[i]
+                        t.dtype = r.dtype.abi
+                        t.rank = len(r.shape)
+                        for j, (d_, s_) in enumerate(zip(r.shape, r.strides)):
+                            t.shape[j] = d_
+                            t.stride[j] = s_
+                        ptr_field(t, "ptr", r.buf, r.offset * r.dtype.size_in_bytes)
+                self.calls.append((L.nbk_custom,
+                                   [a["library"].encode(), a["name"].encode(), ins, len(a["ins"]),
+                                    outs, len(a["dsts"])], patches, (ins, outs)))
+            else:
+                raise NotImplementedError(f"executor: unknown step kind '{k}'")
+
+    def run(self, inputs: Sequence[torch.Tensor]) -> list[torch.Tensor]:
+        plan = self.plan
+        ex = self.ex
+        if len(inputs) != plan.n_inputs:
+            raise ValueError(f"plan expects {plan.n_inputs} inputs, got {len(inputs)}")
+        keep = []
+        outs: list[torch.Tensor] = [None] * len(plan.outputs)  # type: ignore
+        out_by_buf = {}
+        for oi, (bid, shape, dtype) in enumerate(plan.outputs):
+            if bid not in out_by_buf:
+                out_by_buf[bid] = torch.empty(shape, dtype=dtype.to_torch(), device=ex.torch_device)
+            outs[oi] = out_by_buf[bid]
+        for b in plan.bufs:
+            if b.role == "input":
+                t = inputs[b.index]
+                if t.device != ex.torch_device:
+                    raise ValueError(f"input {b.index} lives on {t.device}, expected {ex.torch_device}")
+                if not t.is_contiguous() or (t.data_ptr() % 16) != 0:
+                    t = t.contiguous().clone()
+                    keep.append(t)
+                self.base[b.id] = t.data_ptr()
+            elif b.role == "output":
+                self.base[b.id] = out_by_buf[b.id].data_ptr()
+        stream = C.c_void_p(ex.current_stream())
+        base = self.base
+        check = lib.check
+        for fn, args, patches, _keep in self.calls:
+            for obj, fieldname, buf, off in patches:
+                setattr(obj, fieldname, base[buf] + off)
+            if len(args) >= 2 and isinstance(args[0], _Ptrs):
+                h = args[0]
+                call_args = [C.c_void_p(getattr(h, n)) for n in args[1]] + list(args[2:])
+            elif len(args) >= 3 and isinstance(args[1], _Ptrs):
+                h = args[1]
+                call_args = [args[0]] + [C.c_void_p(getattr(h, n)) for n in args[2]] + list(args[3:])
+            else:
+                call_args = args
+            check(fn(*call_args, stream))
+        del keep
+        return outs
+
+
+class _Ptrs:
+    """Mutable holder for raw addresses that are patched per run."""
+
+    __slots__ = ("p0", "p1", "p2", "p3")
+
+    def __init__(self, n: int):
+        self.p0 = self.p1 = self.p2 = self.p3 = None
+
+
+class HipExecutor:
+    """Runs plans on one gfx950 GPU.  Construction fails without it."""
+
+    name = "hip"
+
+    def __init__(self, device: int = 0):
+        self.lib = lib.load()
+        if not torch.cuda.is_available():
+            raise RuntimeError(
+                "nabla_amd needs a ROCm GPU: torch.cuda.is_available() is False and the "
+                "package has no CPU execution path"
+            )
+        lib.check(self.lib.nbk_init(device))
+        self.torch_device = torch.device("cuda", device)
+        self.status_flag = torch.zeros(1, dtype=torch.int32, device=self.torch_device)
+
+    def current_stream(self) -> int:
+        return torch.cuda.current_stream(self.torch_device).cuda_stream
+
+    def bind(self, plan: Plan) -> BoundPlan:
+        return BoundPlan(plan, self)
+
+    def synchronize(self) -> None:
+        torch.cuda.current_stream(self.torch_device).synchronize()
+
+    def check_status(self) -> None:
+        """Raise if a kernel flagged a data-dependent error (out-of-range gather index)."""
+        if int(self.status_flag.item()) != 0:
+            self.status_flag.zero_()
+            raise IndexError("gather: index out of range")
+
+
+_EXECUTOR: Any = None
+
+
+def get_executor():
+    global _EXECUTOR
+    if _EXECUTOR is None:
+        _EXECUTOR = HipExecutor(0)
+    return _EXECUTOR
+
+
+def set_executor(ex) -> Any:
+    """Install another executor (used by host-logic tests); returns the previous one."""
+    global _EXECUTOR
+    prev = _EXECUTOR
+    _EXECUTOR = ex
+    from ..core import engine
+    engine.clear_plan_cache()
+    from ..core import tensor as _t
+    _t._SCALAR_CACHE.clear()
+    return prev

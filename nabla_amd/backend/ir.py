@@ -1,0 +1,355 @@
+"""Lowering IR: what ``Operation.kernel`` emits instead of MAX graph ops.
+
+In the reference every ``kernel(args, kwargs)`` receives MAX ``TensorValue``s
+and calls ``max.graph.ops.*`` (nabla/ops/base.py:127-137, engine.py:832-847).
+Here it receives ``Value``s and calls the builder functions of this module;
+the result is a small SSA graph that the planner turns into kernel launches.
+
+Node kinds
+    input                       a realized leaf buffer
+    ew        fn, n inputs      elementwise, all tensor inputs have the output shape
+    reduce    fn, axis          single axis, keepdims (reduction.py:147-245)
+    reshape / broadcast / permute / slice      pure views
+    fill / iota                 generators
+    tril                        keep the lower triangle (creation.py:225-274)
+    matmul, conv2d, conv2d_dgrad, conv2d_wgrad, maxpool2d, maxpool2d_bwd,
+    gather, argreduce, pad, concat, slice_update, custom
+"""
+from __future__ import annotations
+
+from contextvars import ContextVar
+from typing import Any, Sequence
+
+from ..core.dtype import DType, promote
+
+
+class Value:
+    __slots__ = ("shape", "dtype", "node", "index", "id")
+
+    def __init__(self, shape, dtype: DType, node: "Node", index: int, vid: int):
+        self.shape = tuple(int(d) for d in shape)
+        self.dtype = dtype
+        self.node = node
+        self.index = index
+        self.id = vid
+
+    @property
+    def rank(self) -> int:
+        return len(self.shape)
+
+    @property
+    def type(self):
+        """(shape, dtype) pair; what ``call_custom_kernel`` takes as an out_type."""
+        return (self.shape, self.dtype)
+
+    def numel(self) -> int:
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+    def __repr__(self) -> str:
+        return f"%{self.id}:{self.dtype.name}{list(self.shape)}"
+
+
+class Node:
+    __slots__ = ("kind", "fn", "inputs", "attrs", "outputs", "pos")
+
+    def __init__(self, kind: str, fn: str | None, inputs: Sequence[Value], attrs: dict, pos: int):
+        self.kind = kind
+        self.fn = fn
+        self.inputs = list(inputs)
+        self.attrs = attrs
+        self.outputs: list[Value] = []
+        self.pos = pos
+
+    def __repr__(self) -> str:
+        fn = f".{self.fn}" if self.fn else ""
+        return f"{self.outputs} = {self.kind}{fn}({self.inputs}) {self.attrs or ''}"
+
+
+class Builder:
+    def __init__(self) -> None:
+        self.nodes: list[Node] = []
+        self.inputs: list[Value] = []
+        self._n_values = 0
+
+    def add(self, kind: str, inputs: Sequence[Value], outs: Sequence[tuple], fn: str | None = None,
+            **attrs: Any) -> list[Value]:
+        node = Node(kind, fn, inputs, attrs, len(self.nodes))
+        for i, (shape, dtype) in enumerate(outs):
+            node.outputs.append(Value(shape, dtype, node, i, self._n_values))
+            self._n_values += 1
+        self.nodes.append(node)
+        return node.outputs
+
+
+_CURRENT: ContextVar[Builder | None] = ContextVar("nbk_ir_builder", default=None)
+
+
+def current() -> Builder:
+    b = _CURRENT.get()
+    if b is None:
+        raise RuntimeError("no lowering in progress: kernel() may only run inside evaluate()")
+    return b
+
+
+class building:
+    """Context manager that makes ``builder`` the target of the functions below."""
+
+    def __init__(self, builder: Builder):
+        self.builder = builder
+
+    def __enter__(self) -> Builder:
+        self._tok = _CURRENT.set(self.builder)
+        return self.builder
+
+    def __exit__(self, *exc) -> None:
+        _CURRENT.reset(self._tok)
+
+
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+# ---- leaves ---------------------------------------------------------------------
+def input(shape, dtype: DType) -> Value:  # noqa: A001 - mirrors graph "input"
+    b = current()
+    v = b.add("input", [], [(shape, dtype)])[0]
+    b.inputs.append(v)
+    return v
+
+
+# ---- elementwise ------------------------------------------------------------------
+UNARY_FNS = {"mov", "neg", "relu", "exp", "log", "sqrt", "rsqrt", "erf", "gelu", "tanh", "sigmoid",
+             "abs", "not", "trunc", "nez"}
+BINARY_FNS = {"add", "sub", "mul", "div", "max", "min", "gt", "ge", "eq", "ne", "lt", "le", "pow",
+              "and", "or"}
+TERNARY_FNS = {"where", "fma"}
+BOOL_FNS = {"gt", "ge", "eq", "ne", "lt", "le", "and", "or", "not", "nez"}
+
+
+def ew(fn: str, *xs: Value | float | int, dtype: DType | None = None) -> Value:
+    """Elementwise ``fn``.  Tensor inputs must already share one shape (the
+    reference makes broadcasts explicit before the op, base.py:645-652);
+    Python numbers are immediates."""
+    tensors = [x for x in xs if isinstance(x, Value)]
+    if not tensors:
+        raise ValueError(f"ew.{fn}: needs at least one tensor input")
+    shape = tensors[0].shape
+    for t in tensors[1:]:
+        if t.shape != shape:
+            raise ValueError(f"ew.{fn}: operand shapes differ: {[t.shape for t in tensors]}")
+    arity = 1 if fn in UNARY_FNS else 2 if fn in BINARY_FNS else 3 if fn in TERNARY_FNS else 0
+    if arity == 0:
+        raise ValueError(f"ew: unknown function '{fn}'")
+    if len(xs) != arity:
+        raise ValueError(f"ew.{fn}: expected {arity} operands, got {len(xs)}")
+    if dtype is None:
+        if fn in BOOL_FNS:
+            dtype = DType.bool
+        elif fn == "where":
+            vals = [x.dtype for x in xs[1:] if isinstance(x, Value)]
+            dtype = vals[0] if len(vals) == 1 else promote(vals[0], vals[1]) if vals else DType.float32
+        else:
+            dtype = tensors[0].dtype
+            for t in tensors[1:]:
+                dtype = promote(dtype, t.dtype)
+    operands = tuple(x if isinstance(x, Value) else float(x) for x in xs)
+    return current().add("ew", tensors, [(shape, dtype)], fn=fn, operands=operands)[0]
+
+
+def cast(x: Value, dtype: DType) -> Value:
+    if x.dtype is dtype:
+        return x
+    if dtype is DType.bool:
+        return ew("nez", x, dtype=dtype)
+    if dtype.is_integral() and x.dtype.is_float():
+        return ew("trunc", x, dtype=dtype)
+    return ew("mov", x, dtype=dtype)
+
+
+def tril(x: Value, k: int = 0, upper: bool = False) -> Value:
+    """Zero everything above (below, if ``upper``) the k-th diagonal of the last two axes."""
+    if x.rank < 2:
+        raise ValueError("tril/triu needs rank >= 2")
+    return current().add("tril", [x], [(x.shape, x.dtype)], k=int(k), upper=bool(upper))[0]
+
+
+# ---- reductions ---------------------------------------------------------------------
+def reduce(fn: str, x: Value, axis: int) -> Value:  # noqa: A001
+    """Single-axis keepdims reduction; ``fn`` in {sum, max, min}."""
+    if fn not in ("sum", "max", "min"):
+        raise ValueError(f"reduce: unknown kind '{fn}'")
+    if axis < 0:
+        axis += x.rank
+    if not 0 <= axis < x.rank:
+        raise ValueError(f"reduce: axis {axis} out of range for rank {x.rank}")
+    shape = x.shape[:axis] + (1,) + x.shape[axis + 1:]
+    return current().add("reduce", [x], [(shape, x.dtype)], fn=fn, axis=axis)[0]
+
+
+def argreduce(fn: str, x: Value, axis: int) -> Value:
+    """Index (int64) of the first max / min along ``axis``, keepdims."""
+    if axis < 0:
+        axis += x.rank
+    shape = x.shape[:axis] + (1,) + x.shape[axis + 1:]
+    return current().add("argreduce", [x], [(shape, DType.int64)], fn=fn, axis=axis)[0]
+
+
+# ---- views --------------------------------------------------------------------------
+def reshape(x: Value, shape) -> Value:
+    shape = tuple(int(d) for d in shape)
+    if -1 in shape:
+        known = _numel([d for d in shape if d != -1])
+        shape = tuple(x.numel() // max(known, 1) if d == -1 else d for d in shape)
+    if _numel(shape) != x.numel():
+        raise ValueError(f"reshape: cannot view {x.shape} as {shape}")
+    if shape == x.shape:
+        return x
+    return current().add("reshape", [x], [(shape, x.dtype)])[0]
+
+
+def broadcast_to(x: Value, shape) -> Value:
+    shape = tuple(int(d) for d in shape)
+    if shape == x.shape:
+        return x
+    if len(shape) < x.rank:
+        raise ValueError(f"broadcast_to: cannot broadcast {x.shape} to {shape}")
+    for a, b in zip(x.shape[::-1], shape[::-1]):
+        if a != b and a != 1:
+            raise ValueError(f"broadcast_to: cannot broadcast {x.shape} to {shape}")
+    return current().add("broadcast", [x], [(shape, x.dtype)])[0]
+
+
+def permute(x: Value, perm) -> Value:
+    perm = tuple(int(p) % max(x.rank, 1) for p in perm)
+    if sorted(perm) != list(range(x.rank)):
+        raise ValueError(f"permute: {perm} is not a permutation of rank {x.rank}")
+    if perm == tuple(range(x.rank)):
+        return x
+    shape = tuple(x.shape[p] for p in perm)
+    return current().add("permute", [x], [(shape, x.dtype)], perm=perm)[0]
+
+
+def slice(x: Value, starts, stops, steps=None) -> Value:  # noqa: A001
+    steps = tuple(steps) if steps is not None else (1,) * x.rank
+    starts, stops = tuple(starts), tuple(stops)
+    shape = []
+    for d, a, b, s in zip(x.shape, starts, stops, steps):
+        if s <= 0 or not (0 <= a <= b <= d):
+            raise ValueError(f"slice: bad range [{a}:{b}:{s}] for extent {d}")
+        shape.append((b - a + s - 1) // s)
+    shape = tuple(shape)
+    if shape == x.shape and all(s == 1 for s in steps):
+        return x
+    return current().add("slice", [x], [(shape, x.dtype)], starts=starts, steps=steps)[0]
+
+
+# ---- generators -----------------------------------------------------------------------
+def fill(shape, dtype: DType, value: float) -> Value:
+    return current().add("fill", [], [(tuple(shape), dtype)], value=float(value))[0]
+
+
+def iota(n: int, dtype: DType, start: float = 0.0, step: float = 1.0) -> Value:
+    return current().add("iota", [], [((int(n),), dtype)], start=float(start), step=float(step))[0]
+
+
+# ---- contractions ---------------------------------------------------------------------
+def matmul(a: Value, b: Value) -> Value:
+    """``(..., M, K) @ (..., K, N)`` with identical leading dims (binary.py:197-287)."""
+    if a.rank < 2 or b.rank < 2:
+        raise ValueError("matmul: operands must have rank >= 2 (promote 1-D operands first)")
+    if a.shape[-1] != b.shape[-2]:
+        raise ValueError(f"matmul: contraction mismatch {a.shape} @ {b.shape}")
+    if a.shape[:-2] != b.shape[:-2]:
+        raise ValueError(f"matmul: batch dims differ {a.shape} vs {b.shape}")
+    shape = a.shape[:-1] + (b.shape[-1],)
+    return current().add("matmul", [a, b], [(shape, promote(a.dtype, b.dtype))])[0]
+
+
+def conv_out_size(n: int, k: int, stride: int, pad_lo: int, pad_hi: int) -> int:
+    return (n + pad_lo + pad_hi - k) // stride + 1
+
+
+def conv2d(x: Value, w: Value, bias: Value | None, stride, padding) -> Value:
+    """NHWC x HWIO correlation; padding = (top, bottom, left, right)."""
+    n, h, wd, cin = x.shape
+    r, s, cin2, cout = w.shape
+    if cin != cin2:
+        raise ValueError(f"conv2d: input channels {cin} vs filter {cin2}")
+    ho = conv_out_size(h, r, stride[0], padding[0], padding[1])
+    wo = conv_out_size(wd, s, stride[1], padding[2], padding[3])
+    ins = [x, w] + ([bias] if bias is not None else [])
+    return current().add("conv2d", ins, [((n, ho, wo, cout), x.dtype)], stride=tuple(stride),
+                         padding=tuple(padding), has_bias=bias is not None)[0]
+
+
+def conv2d_dgrad(dy: Value, w: Value, x_shape, stride, padding) -> Value:
+    return current().add("conv2d_dgrad", [dy, w], [(tuple(x_shape), dy.dtype)], stride=tuple(stride),
+                         padding=tuple(padding))[0]
+
+
+def conv2d_wgrad(x: Value, dy: Value, w_shape, stride, padding) -> Value:
+    return current().add("conv2d_wgrad", [x, dy], [(tuple(w_shape), x.dtype)], stride=tuple(stride),
+                         padding=tuple(padding))[0]
+
+
+def maxpool2d(x: Value, kernel, stride, padding) -> Value:
+    n, h, w, c = x.shape
+    ho = (h + padding[0] + padding[1] - kernel[0]) // stride[0] + 1
+    wo = (w + padding[2] + padding[3] - kernel[1]) // stride[1] + 1
+    return current().add("maxpool2d", [x], [((n, ho, wo, c), x.dtype)], kernel=tuple(kernel),
+                         stride=tuple(stride), padding=tuple(padding))[0]
+
+
+def maxpool2d_bwd(x: Value, y: Value, dy: Value, kernel, stride, padding) -> Value:
+    return current().add("maxpool2d_bwd", [x, y, dy], [(x.shape, x.dtype)], kernel=tuple(kernel),
+                         stride=tuple(stride), padding=tuple(padding))[0]
+
+
+# ---- indexing / movement ------------------------------------------------------------------
+def gather(table: Value, idx: Value, axis: int) -> Value:
+    if axis < 0:
+        axis += table.rank
+    shape = table.shape[:axis] + idx.shape + table.shape[axis + 1:]
+    return current().add("gather", [table, idx], [(shape, table.dtype)], axis=axis)[0]
+
+
+def pad(x: Value, lo, hi, value: float = 0.0) -> Value:
+    shape = tuple(d + a + b for d, a, b in zip(x.shape, lo, hi))
+    if shape == x.shape:
+        return x
+    return current().add("pad", [x], [(shape, x.dtype)], lo=tuple(lo), hi=tuple(hi),
+                         value=float(value))[0]
+
+
+def concat(xs: Sequence[Value], axis: int) -> Value:
+    xs = list(xs)
+    if axis < 0:
+        axis += xs[0].rank
+    base = xs[0].shape
+    total = 0
+    dtype = xs[0].dtype
+    for x in xs:
+        if x.shape[:axis] != base[:axis] or x.shape[axis + 1:] != base[axis + 1:]:
+            raise ValueError(f"concat: shapes differ off-axis: {[v.shape for v in xs]}")
+        total += x.shape[axis]
+        dtype = promote(dtype, x.dtype)
+    shape = base[:axis] + (total,) + base[axis + 1:]
+    if len(xs) == 1:
+        return xs[0]
+    return current().add("concat", xs, [(shape, dtype)], axis=axis)[0]
+
+
+def slice_update(x: Value, update: Value, starts) -> Value:
+    """Copy of ``x`` with the window at ``starts`` replaced by ``update``."""
+    return current().add("slice_update", [x, update], [(x.shape, x.dtype)], starts=tuple(starts))[0]
+
+
+def custom(name: str, library: str, inputs: Sequence[Value], out_types: Sequence[tuple]) -> list[Value]:
+    return current().add("custom", list(inputs), [(tuple(s), d) for s, d in out_types], name=name,
+                         library=str(library))

@@ -1,0 +1,38 @@
+"""Row-program instruction set shared by the assembler, the HIP interpreter
+(nabla_amd/csrc/rowprog.hip) and the numpy emulator used by the CPU tests.
+Numbers must match ``enum nbk_rp_op`` in include/nbk.h (a test compares them).
+"""
+from __future__ import annotations
+
+HALT, BODY, LDG, STG, LDR, STR, IMM, COLIDX, LEADIDX, ACCINIT, ACC, RED = range(12)
+
+UNARY = {
+    "mov": 16, "neg": 17, "relu": 18, "exp": 19, "log": 20, "sqrt": 21, "rsqrt": 22, "erf": 23,
+    "gelu": 24, "tanh": 25, "sigmoid": 26, "abs": 27, "rbf16": 28, "not": 29, "trunc": 30,
+    "nez": 31,
+}
+BINARY = {
+    "add": 32, "sub": 33, "mul": 34, "div": 35, "max": 36, "min": 37, "gt": 38, "ge": 39,
+    "eq": 40, "ne": 41, "lt": 42, "le": 43, "pow": 44, "and": 45, "or": 46,
+}
+TERNARY = {"where": 48, "fma": 49}
+EW = {**UNARY, **BINARY, **TERNARY}
+EW_NAME = {v: k for k, v in EW.items()}
+
+RED_KIND = {"sum": 0, "max": 1, "min": 2}
+
+MAX_OPERANDS = 20
+MAX_INS = 224
+MAX_IMM = 24
+MAX_LEAD = 4
+NVEC = 16
+NSCL = 16
+NACC = 4
+MAX_STAGE = 4
+STAGE_BYTES = 64 * 1024
+MAX_BLOCK = 512
+
+STRUCT_NAMES = {
+    "HALT": HALT, "BODY": BODY, "LDG": LDG, "STG": STG, "LDR": LDR, "STR": STR, "IMM": IMM,
+    "COLIDX": COLIDX, "LEADIDX": LEADIDX, "ACCINIT": ACCINIT, "ACC": ACC, "RED": RED,
+}

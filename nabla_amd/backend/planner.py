@@ -1,0 +1,1320 @@
+"""Lowering pass: IR graph -> launch plan.
+
+This is the step that replaces "replay the trace into a MAX graph and let
+``InferenceSession.load`` compile it" (nabla/core/graph/engine.py:575-663).
+
+Passes
+  1. dead-code elimination from the requested outputs;
+  2. fusion: elementwise ops, last-axis reductions, tril masks and iotas that
+     share an iteration domain ``lead x C`` are grouped into one row program
+     each (softmax, layer_norm, cross-entropy and their backward graphs fuse
+     this way without being pattern-matched); a node joins the group of one of
+     its producers unless that would make the group graph cyclic;
+  3. view folding: reshape / broadcast / permute / slice never run as kernels;
+     they become offsets and strides of the consumers' operands.  A strided
+     copy is inserted only where a consumer cannot take the view;
+  4. code generation of row programs (phases, recomputation instead of
+     spilling, register allocation, LDS staging of rows read in several phases);
+  5. buffer assignment: intermediate buffers live in one arena with
+     liveness-based offsets, outputs get allocations of their own.
+"""
+from __future__ import annotations
+
+import heapq
+import math
+from dataclasses import dataclass, field
+from typing import Any, Sequence
+
+from ..core.dtype import DType
+from . import ir, isa
+
+FUSABLE = ("ew", "reduce", "tril", "iota")
+VIEW_KINDS = ("reshape", "broadcast", "permute", "slice")
+
+
+class FusionLimit(Exception):
+    """A fused group does not fit the row-program limits; planning retries smaller."""
+
+
+# --------------------------------------------------------------------------- data
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def contiguous_strides(shape) -> tuple[int, ...]:
+    st = []
+    acc = 1
+    for d in reversed(shape):
+        st.append(acc)
+        acc *= max(d, 1)
+    return tuple(reversed(st))
+
+
+@dataclass
+class Buf:
+    id: int
+    numel: int
+    dtype: DType
+    role: str  # 'input' | 'temp' | 'output'
+    index: int = -1  # input / output position
+    shape: tuple = ()
+    offset: int = -1  # byte offset in the arena (temps)
+    first: int = 1 << 60
+    last: int = -1
+
+    @property
+    def nbytes(self) -> int:
+        return max(self.numel, 1) * self.dtype.size_in_bytes
+
+
+@dataclass(frozen=True)
+class ViewRef:
+    buf: int
+    offset: int
+    shape: tuple
+    strides: tuple
+    dtype: DType
+
+    def is_contiguous(self) -> bool:
+        exp = 1
+        for d, s in zip(reversed(self.shape), reversed(self.strides)):
+            if d == 1:
+                continue
+            if s != exp:
+                return False
+            exp *= d
+        return True
+
+
+@dataclass(frozen=True)
+class Const:
+    value: float
+    shape: tuple
+    dtype: DType
+
+
+@dataclass
+class OperandSpec:
+    buf: int
+    offset: int
+    lead_strides: tuple
+    col_stride: int
+    dtype: DType
+    vec_ok: bool
+    stage_slot: int = -1
+    is_output: bool = False
+
+
+@dataclass
+class Step:
+    kind: str
+    reads: list = field(default_factory=list)
+    writes: list = field(default_factory=list)
+    attrs: dict = field(default_factory=dict)
+
+
+@dataclass
+class Plan:
+    bufs: list
+    steps: list
+    n_inputs: int
+    outputs: list  # per plan output: (buf id, shape, dtype)
+    arena_bytes: int = 0
+    stats: dict = field(default_factory=dict)
+
+
+# --------------------------------------------------------------------- view algebra
+def _reshape_strides(old_shape, old_strides, new_shape):
+    """Strides that view the same memory as ``new_shape``, or None (numpy's
+    no-copy reshape rule)."""
+    if _numel(old_shape) != _numel(new_shape):
+        return None
+    if _numel(new_shape) == 0:
+        return contiguous_strides(new_shape)
+    olds = [(d, s) for d, s in zip(old_shape, old_strides) if d != 1]
+    new_strides = [0] * len(new_shape)
+    oi = 0
+    ni = 0
+    n_old = len(olds)
+    n_new = len(new_shape)
+    while ni < n_new and new_shape[ni] == 1:
+        ni += 1
+    while oi < n_old and ni < n_new:
+        # grow both sides until their element counts match
+        np_ = new_shape[ni]
+        op_ = olds[oi][0]
+        oj, nj = oi + 1, ni + 1
+        while np_ != op_:
+            if np_ < op_:
+                while nj < n_new and new_shape[nj] == 1:
+                    nj += 1
+                if nj >= n_new:
+                    return None
+                np_ *= new_shape[nj]
+                nj += 1
+            else:
+                if oj >= n_old:
+                    return None
+                op_ *= olds[oj][0]
+                oj += 1
+        # old dims oi..oj must be mutually contiguous
+        for k in range(oi, oj - 1):
+            if olds[k][1] != olds[k + 1][1] * olds[k + 1][0]:
+                return None
+        st = olds[oj - 1][1]
+        for k in range(nj - 1, ni - 1, -1):
+            if new_shape[k] == 1:
+                new_strides[k] = 0
+                continue
+            new_strides[k] = st
+            st *= new_shape[k]
+        oi, ni = oj, nj
+        while ni < n_new and new_shape[ni] == 1:
+            ni += 1
+    if oi != n_old:
+        return None
+    return tuple(new_strides)
+
+
+def _derive_view(node: ir.Node, base: ViewRef) -> ViewRef | None:
+    """View of ``base`` after the view node; None if it needs a copy (reshape only)."""
+    out = node.outputs[0]
+    if node.kind == "broadcast":
+        pad = len(out.shape) - len(base.shape)
+        strides = [0] * pad + [0 if (d == 1 and o != 1) else s
+                               for d, s, o in zip(base.shape, base.strides, out.shape[pad:])]
+        return ViewRef(base.buf, base.offset, out.shape, tuple(strides), base.dtype)
+    if node.kind == "permute":
+        perm = node.attrs["perm"]
+        return ViewRef(base.buf, base.offset, out.shape, tuple(base.strides[p] for p in perm),
+                       base.dtype)
+    if node.kind == "slice":
+        off = base.offset + sum(a * s for a, s in zip(node.attrs["starts"], base.strides))
+        strides = tuple(s * st for s, st in zip(base.strides, node.attrs["steps"]))
+        return ViewRef(base.buf, off, out.shape, strides, base.dtype)
+    if node.kind == "reshape":
+        st = _reshape_strides(base.shape, base.strides, out.shape)
+        if st is None:
+            return None
+        return ViewRef(base.buf, base.offset, out.shape, st, base.dtype)
+    raise AssertionError(node.kind)
+
+
+# ------------------------------------------------------------------------- grouping
+class Unit:
+    __slots__ = ("id", "nodes", "node_pos", "first_pos", "last_pos", "preds", "fused", "lead", "C",
+                 "n_reduce", "ext", "hard", "alias")
+
+    def __init__(self, uid: int, node: ir.Node, fused: bool):
+        self.id = uid
+        self.nodes = [node]
+        self.node_pos = {node.pos}
+        self.first_pos = node.pos
+        self.last_pos = node.pos
+        self.preds: set = set()
+        self.fused = fused
+        self.lead = None
+        self.C = None
+        self.n_reduce = 0
+        self.ext: set = set()
+        self.hard: set = set()   # preds that can never be merged into this unit
+        self.alias = None        # set when this unit was merged into another
+
+    def add(self, node: ir.Node) -> None:
+        self.nodes.append(node)
+        self.node_pos.add(node.pos)
+        self.last_pos = max(self.last_pos, node.pos)
+
+
+def _shape2(shape):
+    return tuple(shape) if len(shape) > 0 else (1,)
+
+
+class Planner:
+    def __init__(self, builder: ir.Builder, outputs: Sequence[ir.Value], max_members: int = 28):
+        self.b = builder
+        self.outputs = list(outputs)
+        self.max_members = max_members
+        self.max_ext = 12
+        self.bufs: list[Buf] = []
+        self.steps: list[Step] = []
+        self.loc: dict[int, Any] = {}  # value id -> ViewRef | Const
+        self.unit_of: dict[int, Unit] = {}  # node pos -> unit
+        self.alias_nodes: set[int] = set()  # broadcast nodes fused as row->full aliases
+
+    # ................................................................ liveness
+    def _live_nodes(self) -> list[ir.Node]:
+        live: set[int] = set()
+        stack = [v.node for v in self.outputs]
+        while stack:
+            n = stack.pop()
+            if n.pos in live:
+                continue
+            live.add(n.pos)
+            for i in n.inputs:
+                if i.node.pos not in live:
+                    stack.append(i.node)
+        return [n for n in self.b.nodes if n.pos in live]
+
+    # ................................................................ helpers
+    def _base(self, v: ir.Value) -> ir.Value:
+        """Strip non-fused view nodes."""
+        while v.node.kind in VIEW_KINDS and v.node.pos not in self.alias_nodes:
+            v = v.node.inputs[0]
+        return v
+
+    @staticmethod
+    def _find(u: "Unit | None") -> "Unit | None":
+        while u is not None and u.alias is not None:
+            u = u.alias
+        return u
+
+    def _unit(self, pos: int) -> "Unit | None":
+        return self._find(self.unit_of.get(pos))
+
+    def _producer_unit(self, v: ir.Value) -> "Unit | None":
+        return self._unit(self._base(v).node.pos)
+
+    def _is_member_value(self, v: ir.Value) -> bool:
+        return v.node.kind in FUSABLE or v.node.pos in self.alias_nodes
+
+    def _depends(self, u: Unit, g: Unit, skip: "Unit | None" = None) -> bool:
+        """Does unit ``u`` (transitively) need ``g`` to have run?  Paths through
+        ``skip`` are ignored (used when ``skip`` is about to be merged with g)."""
+        if u is g:
+            return True
+        seen = {u.id}
+        stack = [u]
+        while stack:
+            x = stack.pop()
+            for p in x.preds:
+                p = self._find(p)
+                if p is g:
+                    return True
+                if p is skip or p.id in seen or p.last_pos < g.first_pos:
+                    continue
+                seen.add(p.id)
+                stack.append(p)
+        return False
+
+    # ................................................................ fusion
+    def _group(self, nodes: list[ir.Node]) -> list[Unit]:
+        units: list[Unit] = []
+        by_root: dict[int, list[Unit]] = {}  # external root value id -> fused units reading it
+
+        def new_unit(node, fused) -> Unit:
+            u = Unit(len(units), node, fused)
+            units.append(u)
+            self.unit_of[node.pos] = u
+            return u
+
+        def classify_inputs(node, g):
+            """(soft preds, hard preds) of ``node`` seen from group ``g``; None if
+            ``node`` cannot run inside ``g``.  A hard pred is read through a
+            strided view or is not a row program, so it can never be merged in."""
+            soft, hard = [], []
+            for i in node.inputs:
+                if self._is_member_value(i) and self._unit(i.node.pos) is g:
+                    continue
+                pu = self._producer_unit(i)
+                if pu is None:
+                    continue
+                if pu is g:  # a strided view of a member: needs a trip through memory
+                    return None
+                if self._depends(pu, g):
+                    return None
+                (soft if (self._is_member_value(i) and pu.fused) else hard).append(pu)
+            return soft, hard
+
+        def dom_ok(g, kind, lead, last) -> bool:
+            if g.lead != lead:
+                return False
+            if kind == "reduce":
+                return (g.C is None or g.C == last) and g.n_reduce < 8
+            return last == 1 or g.C is None or g.C == last
+
+        def ext_ids(node, g):
+            return {self._base(i).id for i in node.inputs
+                    if not (self._is_member_value(i) and self._unit(i.node.pos) is g)}
+
+        def join(g, node, kind, last, soft, hard):
+            if kind == "reduce" or last != 1:
+                g.C = last
+            g.add(node)
+            self.unit_of[node.pos] = g
+            g.preds.update(soft)
+            g.preds.update(hard)
+            g.hard.update(hard)
+            for e in ext_ids(node, g):
+                if e not in g.ext:
+                    g.ext.add(e)
+                    by_root.setdefault(e, []).append(g)
+            if kind == "reduce":
+                g.n_reduce += 1
+
+        def try_merge(g1: Unit, g2: Unit) -> bool:
+            """Fold g2 into g1 when no third unit sits between them."""
+            if g1 is g2 or not (g1.fused and g2.fused) or g1.lead != g2.lead:
+                return False
+            if g1.C is not None and g2.C is not None and g1.C != g2.C:
+                return False
+            if len(g1.nodes) + len(g2.nodes) > self.max_members or g1.n_reduce + g2.n_reduce > 8:
+                return False
+            if any(self._find(h) is g2 for h in g1.hard) or any(self._find(h) is g1 for h in g2.hard):
+                return False
+            if len(g1.ext | g2.ext) > self.max_ext + 4:
+                return False
+            for a, b in ((g1, g2), (g2, g1)):
+                for p in a.preds:
+                    p = self._find(p)
+                    if p is b or p is a:
+                        continue
+                    if self._depends(p, b, skip=a):
+                        return False
+            g2.alias = g1
+            for n in g2.nodes:
+                g1.add(n)
+            g1.first_pos = min(g1.first_pos, g2.first_pos)
+            g1.preds = {self._find(p) for p in (g1.preds | g2.preds)} - {g1, g2}
+            g1.hard = {self._find(p) for p in (g1.hard | g2.hard)} - {g1, g2}
+            g1.ext |= g2.ext
+            for e in g2.ext:
+                by_root.setdefault(e, []).append(g1)
+            g1.n_reduce += g2.n_reduce
+            if g1.C is None:
+                g1.C = g2.C
+            return True
+
+        for node in nodes:
+            kind = node.kind
+            if kind == "input" or kind == "fill":
+                continue
+            if kind in VIEW_KINDS:
+                # row -> full broadcast of a fused value stays inside the group
+                if kind == "broadcast":
+                    src = node.inputs[0]
+                    out = node.outputs[0]
+                    g = self._unit(src.node.pos)
+                    if (g is not None and g.fused and self._is_member_value(src) and
+                            len(src.shape) == len(out.shape) and len(out.shape) >= 1 and
+                            src.shape[:-1] == out.shape[:-1] and src.shape[-1] == 1 and
+                            tuple(out.shape[:-1]) == g.lead and g.C in (None, out.shape[-1]) and
+                            len(g.nodes) < self.max_members):
+                        g.C = out.shape[-1]
+                        g.add(node)
+                        self.unit_of[node.pos] = g
+                        self.alias_nodes.add(node.pos)
+                continue
+            if kind not in FUSABLE or (kind == "reduce" and node.attrs["axis"] != node.inputs[0].rank - 1):
+                u = new_unit(node, False)
+                for i in node.inputs:
+                    pu = self._producer_unit(i)
+                    if pu is not None:
+                        u.preds.add(pu)
+                        u.hard.add(pu)
+                continue
+
+            # fusable node: find its domain
+            out = node.outputs[0]
+            dom_shape = _shape2(node.inputs[0].shape if kind == "reduce" else out.shape)
+            lead, last = tuple(dom_shape[:-1]), dom_shape[-1]
+            home = None
+            if kind != "iota" and not (kind == "tril" and len(lead) == 0):
+                cands: list[Unit] = []
+                for i in node.inputs:
+                    if self._is_member_value(i):
+                        g = self._unit(i.node.pos)
+                        if g is not None and g.fused and g not in cands:
+                            cands.append(g)
+                # groups that read one of the same external tensors over the same domain
+                sib: list[Unit] = []
+                for i in node.inputs:
+                    for g in by_root.get(self._base(i).id, ()):
+                        g = self._find(g)
+                        if g.fused and g not in cands and g not in sib:
+                            sib.append(g)
+                cands.sort(key=lambda g: -g.last_pos)
+                sib.sort(key=lambda g: -g.last_pos)
+                for g in cands + sib[:4]:
+                    if not dom_ok(g, kind, lead, last) or len(g.nodes) >= self.max_members:
+                        continue
+                    cl = classify_inputs(node, g)
+                    if cl is None:
+                        continue
+                    if len(g.ext | ext_ids(node, g)) > self.max_ext:
+                        continue
+                    join(g, node, kind, last, *cl)
+                    home = g
+                    break
+                if home is not None:
+                    # producers that live in other groups: try to pull those groups in
+                    for g2 in cands:
+                        g2 = self._find(g2)
+                        if g2 is not home and dom_ok(g2, "ew", lead, 1):
+                            try_merge(home, g2)
+            if home is None:
+                g = new_unit(node, True)
+                g.lead = lead
+                g.C = last if (kind == "reduce" or last != 1) else None
+                g.n_reduce = 1 if kind == "reduce" else 0
+                for i in node.inputs:
+                    pu = self._producer_unit(i)
+                    if pu is not None and pu is not g:
+                        g.preds.add(pu)
+                        if not (self._is_member_value(i) and pu.fused):
+                            g.hard.add(pu)
+                    e = self._base(i).id
+                    g.ext.add(e)
+                    by_root.setdefault(e, []).append(g)
+        live_units = [u for u in units if u.alias is None]
+        for u in live_units:
+            u.preds = {self._find(p) for p in u.preds} - {u}
+        return live_units
+
+    # ................................................................ ordering
+    def _order(self, units: list[Unit]) -> list[Unit]:
+        indeg = {u.id: 0 for u in units}
+        succs: dict[int, list[Unit]] = {u.id: [] for u in units}
+        for u in units:
+            for p in u.preds:
+                if p is u:
+                    continue
+                indeg[u.id] += 1
+                succs[p.id].append(u)
+        heap = [(u.first_pos, u.id) for u in units if indeg[u.id] == 0]
+        heapq.heapify(heap)
+        by_id = {u.id: u for u in units}
+        out = []
+        while heap:
+            _, uid = heapq.heappop(heap)
+            u = by_id[uid]
+            out.append(u)
+            for s in succs[uid]:
+                indeg[s.id] -= 1
+                if indeg[s.id] == 0:
+                    heapq.heappush(heap, (s.first_pos, s.id))
+        if len(out) != len(units):
+            raise RuntimeError("lowering: fusion produced a cyclic group graph")
+        return out
+
+    # ................................................................ buffers
+    def _new_buf(self, shape, dtype: DType, role: str = "temp", index: int = -1) -> Buf:
+        b = Buf(len(self.bufs), _numel(shape), dtype, role, index, tuple(shape))
+        self.bufs.append(b)
+        return b
+
+    def _emit(self, step: Step) -> None:
+        idx = len(self.steps)
+        for r in step.reads:
+            b = self.bufs[r]
+            b.last = max(b.last, idx)
+            b.first = min(b.first, idx)
+        for w in step.writes:
+            b = self.bufs[w]
+            b.first = min(b.first, idx)
+            b.last = max(b.last, idx)
+        self.steps.append(step)
+
+    def _alloc_value(self, v: ir.Value) -> ViewRef:
+        """Fresh contiguous storage for value ``v`` (an output allocation if it
+        is a plan output that is not claimed yet)."""
+        role, index = "temp", -1
+        if v.id in self._out_pending:
+            role, index = "output", self._out_pending.pop(v.id)
+        b = self._new_buf(v.shape, v.dtype, role, index)
+        ref = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
+        self.loc[v.id] = ref
+        if role == "output":
+            self._out_done[index] = b.id
+        return ref
+
+    def _resolve(self, v: ir.Value):
+        """Location (ViewRef | Const) of a value, folding view chains."""
+        got = self.loc.get(v.id)
+        if got is not None:
+            return got
+        n = v.node
+        if n.kind == "fill":
+            c = Const(n.attrs["value"], v.shape, v.dtype)
+            self.loc[v.id] = c
+            return c
+        if n.kind in VIEW_KINDS and n.pos not in self.alias_nodes:
+            base = self._resolve(n.inputs[0])
+            if isinstance(base, Const):
+                r = Const(base.value, v.shape, v.dtype)
+            else:
+                r = _derive_view(n, base)
+                if r is None:  # reshape of a non-collapsible view
+                    cont = self._materialize(base)
+                    r = _derive_view(n, cont)
+            self.loc[v.id] = r
+            return r
+        raise RuntimeError(f"lowering: value {v} used before it was produced ({n.kind})")
+
+    def _materialize(self, src) -> ViewRef:
+        """Contiguous copy of a view or constant in a fresh temp."""
+        if isinstance(src, Const):
+            b = self._new_buf(src.shape, src.dtype)
+            self._emit(Step("fill", [], [b.id], dict(buf=b.id, numel=_numel(src.shape),
+                                                      value=src.value, dtype=src.dtype)))
+            return ViewRef(b.id, 0, src.shape, contiguous_strides(src.shape), src.dtype)
+        if src.is_contiguous():
+            return src
+        b = self._new_buf(src.shape, src.dtype)
+        dst = ViewRef(b.id, 0, src.shape, contiguous_strides(src.shape), src.dtype)
+        self._emit(Step("copy", [src.buf], [b.id], dict(src=src, dst=dst)))
+        return dst
+
+    def _contig(self, v: ir.Value) -> ViewRef:
+        return self._materialize(self._resolve(v))
+
+    # ................................................................ build
+    def build(self) -> Plan:
+        nodes = self._live_nodes()
+        for i, v in enumerate(self.b.inputs):
+            b = self._new_buf(v.shape, v.dtype, "input", i)
+            self.loc[v.id] = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
+        units = self._group(nodes)
+        order = self._order(units)
+
+        # consumers outside the producing unit decide what must be stored
+        self.need_store: set[int] = set()
+        for n in nodes:
+            cu = self._unit(n.pos)
+            for i in n.inputs:
+                if n.kind in VIEW_KINDS and n.pos not in self.alias_nodes:
+                    # a view forces its source into memory unless that is a view too
+                    self.need_store.add(i.id)
+                    continue
+                pu = self._unit(i.node.pos)
+                if pu is None or pu is not cu or not cu.fused:
+                    self.need_store.add(i.id)
+        # plan outputs: the first output that names a unit-produced value owns
+        # that value's allocation; everything else is copied at the end
+        self._out_pending: dict[int, int] = {}
+        self._out_done: dict[int, int] = {}
+        for oi, v in enumerate(self.outputs):
+            self.need_store.add(v.id)
+            if v.node.kind not in VIEW_KINDS + ("input", "fill") or v.node.pos in self.alias_nodes:
+                if v.id not in self._out_pending:
+                    self._out_pending[v.id] = oi
+
+        for u in order:
+            if u.fused:
+                self._lower_group(u)
+            else:
+                self._lower_single(u.nodes[0])
+
+        outs = []
+        for oi, v in enumerate(self.outputs):
+            if oi in self._out_done:
+                outs.append((self._out_done[oi], v.shape, v.dtype))
+                continue
+            src = self._resolve(v)
+            b = self._new_buf(v.shape, v.dtype, "output", oi)
+            if isinstance(src, Const):
+                self._emit(Step("fill", [], [b.id], dict(buf=b.id, numel=_numel(v.shape),
+                                                          value=src.value, dtype=v.dtype)))
+            else:
+                dst = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
+                self._emit(Step("copy", [src.buf], [b.id], dict(src=src, dst=dst)))
+            outs.append((b.id, v.shape, v.dtype))
+        arena = self._assign_arena()
+        stats = {"steps": len(self.steps), "units": len(units),
+                 "fused_groups": sum(1 for u in units if u.fused)}
+        for s in self.steps:
+            stats[s.kind] = stats.get(s.kind, 0) + 1
+        return Plan(self.bufs, self.steps, len(self.b.inputs), outs, arena, stats)
+
+    def _assign_arena(self) -> int:
+        """First-fit offsets for temps whose live ranges overlap."""
+        temps = [b for b in self.bufs if b.role == "temp" and b.last >= 0]
+        temps.sort(key=lambda b: (b.first, -b.nbytes))
+        placed: list[Buf] = []
+        top = 0
+        for b in temps:
+            size = (b.nbytes + 255) & ~255
+            busy = sorted((p.offset, p.offset + ((p.nbytes + 255) & ~255)) for p in placed
+                          if not (p.last < b.first or p.first > b.last))
+            off = 0
+            for lo, hi in busy:
+                if off + size <= lo:
+                    break
+                off = max(off, hi)
+            b.offset = off
+            top = max(top, off + size)
+            placed.append(b)
+        return top
+
+    # ................................................................ singles
+    def _lower_single(self, n: ir.Node) -> None:
+        k = n.kind
+        out = n.outputs[0]
+        if k == "matmul":
+            self._lower_matmul(n)
+        elif k == "reduce":
+            self._lower_reduce_mid(n)
+        elif k == "argreduce":
+            x = n.inputs[0]
+            axis = n.attrs["axis"]
+            src = self._resolve(x)
+            if axis != x.rank - 1:
+                raise NotImplementedError("argmax/argmin lower only along the last axis; "
+                                          "the op permutes other axes first")
+            src = self._materialize(src)
+            dst = self._alloc_value(out)
+            self._emit(Step("argreduce", [src.buf], [dst.buf], dict(
+                src=src, dst=dst, rows=_numel(x.shape[:-1]), C=x.shape[-1], fn=n.fn)))
+        elif k == "gather":
+            table, idx = n.inputs
+            axis = n.attrs["axis"]
+            t = self._contig(table)
+            ix = self._contig(idx)
+            dst = self._alloc_value(out)
+            self._emit(Step("gather", [t.buf, ix.buf], [dst.buf], dict(
+                table=t, idx=ix, dst=dst, outer=_numel(table.shape[:axis]),
+                axis_len=table.shape[axis], n_idx=idx.numel(),
+                inner=_numel(table.shape[axis + 1:]))))
+        elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
+            ins = [self._contig(i) for i in n.inputs]
+            dst = self._alloc_value(out)
+            if k == "conv2d":
+                xs, ws = n.inputs[0].shape, n.inputs[1].shape
+                ys = out.shape
+            elif k == "conv2d_dgrad":
+                xs, ws, ys = out.shape, n.inputs[1].shape, n.inputs[0].shape
+            else:
+                xs, ws, ys = n.inputs[0].shape, out.shape, n.inputs[1].shape
+            self._emit(Step(k, [i.buf for i in ins], [dst.buf], dict(
+                ins=ins, dst=dst, x_shape=xs, w_shape=ws, y_shape=ys, stride=n.attrs["stride"],
+                padding=n.attrs["padding"], has_bias=n.attrs.get("has_bias", False))))
+        elif k in ("maxpool2d", "maxpool2d_bwd"):
+            ins = [self._contig(i) for i in n.inputs]
+            dst = self._alloc_value(out)
+            xs = n.inputs[0].shape
+            ys = out.shape if k == "maxpool2d" else n.inputs[1].shape
+            self._emit(Step(k, [i.buf for i in ins], [dst.buf], dict(
+                ins=ins, dst=dst, x_shape=xs, y_shape=ys, kernel=n.attrs["kernel"],
+                stride=n.attrs["stride"], padding=n.attrs["padding"])))
+        elif k == "pad":
+            src = self._resolve(n.inputs[0])
+            dst = self._alloc_value(out)
+            self._emit(Step("fill", [], [dst.buf], dict(buf=dst.buf, numel=out.numel(),
+                                                         value=n.attrs["value"], dtype=out.dtype)))
+            self._copy_into(src, dst, n.attrs["lo"], n.inputs[0].shape)
+        elif k == "concat":
+            dst = self._alloc_value(out)
+            axis = n.attrs["axis"]
+            pos = 0
+            for i in n.inputs:
+                src = self._resolve(i)
+                starts = [0] * out.rank
+                starts[axis] = pos
+                self._copy_into(src, dst, starts, i.shape)
+                pos += i.shape[axis]
+        elif k == "slice_update":
+            x = self._resolve(n.inputs[0])
+            upd = self._resolve(n.inputs[1])
+            dst = self._alloc_value(out)
+            self._copy_into(x, dst, [0] * out.rank, out.shape)
+            self._copy_into(upd, dst, n.attrs["starts"], n.inputs[1].shape)
+        elif k == "custom":
+            ins = [self._contig(i) for i in n.inputs]
+            dsts = [self._alloc_value(o) for o in n.outputs]
+            self._emit(Step("custom", [i.buf for i in ins], [d.buf for d in dsts], dict(
+                ins=ins, dsts=dsts, name=n.attrs["name"], library=n.attrs["library"])))
+        else:
+            raise NotImplementedError(f"lowering: no rule for node kind '{k}'")
+
+    def _copy_into(self, src, dst: ViewRef, starts, shape) -> None:
+        off = dst.offset + sum(a * s for a, s in zip(starts, dst.strides))
+        window = ViewRef(dst.buf, off, tuple(shape), dst.strides, dst.dtype)
+        if isinstance(src, Const):
+            src = self._materialize(src)
+        self._emit(Step("copy", [src.buf], [dst.buf], dict(src=src, dst=window)))
+
+    def _lower_reduce_mid(self, n: ir.Node) -> None:
+        x = n.inputs[0]
+        axis = n.attrs["axis"]
+        out = n.outputs[0]
+        src = self._contig(x)
+        outer, red, inner = _numel(x.shape[:axis]), x.shape[axis], _numel(x.shape[axis + 1:])
+        kind = n.fn
+        # few output columns and a long axis: split the axis so the launch has
+        # enough workgroups, then reduce the partials
+        blocks = outer * ((inner + 63) // 64)
+        split = 1
+        if blocks < 256 and red >= 256:
+            want = min(64, max(1, 1024 // max(blocks, 1)))
+            for s in range(want, 1, -1):
+                if red % s == 0 and red // s >= 16 and outer * s <= 65535:
+                    split = s
+                    break
+        if split > 1:
+            tmp = self._new_buf((outer, split, inner), DType.float32)
+            tref = ViewRef(tmp.id, 0, (outer, split, inner),
+                           contiguous_strides((outer, split, inner)), DType.float32)
+            self._emit(Step("reduce_mid", [src.buf], [tmp.id], dict(
+                src=src, dst=tref, outer=outer * split, red=red // split, inner=inner, fn=kind)))
+            dst = self._alloc_value(out)
+            self._emit(Step("reduce_mid", [tmp.id], [dst.buf], dict(
+                src=tref, dst=dst, outer=outer, red=split, inner=inner, fn=kind)))
+            return
+        dst = self._alloc_value(out)
+        self._emit(Step("reduce_mid", [src.buf], [dst.buf], dict(
+            src=src, dst=dst, outer=outer, red=red, inner=inner, fn=kind)))
+
+    # ................................................................ matmul
+    @staticmethod
+    def _mat_operand(ref: ViewRef):
+        """(batch_stride, row_stride, col_stride) if the view is a strided batch
+        of matrices the GEMM can read directly, else None."""
+        shape, st = ref.shape, ref.strides
+        rs, cs = st[-2], st[-1]
+        r, c = shape[-2], shape[-1]
+        if r == 1:
+            rs = c * cs if cs else 1
+        if c == 1:
+            cs = 1 if rs != 1 else (r * rs)
+        if rs != 1 and cs != 1:
+            return None
+        if rs < 0 or cs < 0:
+            return None
+        bdims = [(d, s) for d, s in zip(shape[:-2], st[:-2]) if d != 1]
+        if not bdims:
+            return (0, rs, cs)
+        if all(s == 0 for _, s in bdims):
+            return (0, rs, cs)
+        for (d0, s0), (d1, s1) in zip(bdims[:-1], bdims[1:]):
+            if s0 != s1 * d1:
+                return None
+        return (bdims[-1][1], rs, cs)
+
+    def _lower_matmul(self, n: ir.Node) -> None:
+        a, b = n.inputs
+        out = n.outputs[0]
+        ra, rb = self._resolve(a), self._resolve(b)
+        if isinstance(ra, Const):
+            ra = self._materialize(ra)
+        if isinstance(rb, Const):
+            rb = self._materialize(rb)
+        pa = self._mat_operand(ra)
+        if pa is None:
+            ra = self._materialize(ra)
+            pa = self._mat_operand(ra)
+        pb = self._mat_operand(rb)
+        if pb is None:
+            rb = self._materialize(rb)
+            pb = self._mat_operand(rb)
+        M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
+        batch = _numel(out.shape[:-2])
+        dst = self._alloc_value(out)
+        self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
+            a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch,
+            a_bs=pa[0], a_rs=pa[1], a_cs=pa[2], b_bs=pb[0], b_rs=pb[1], b_cs=pb[2],
+            ldc=N, c_bs=M * N, alpha=1.0)))
+
+    # ................................................................ groups
+    def _lower_group(self, g: Unit) -> None:
+        gen = _RowCodegen(self, g)
+        step = gen.generate()
+        self._emit(step)
+
+
+# ------------------------------------------------------------------ row codegen
+class _VReg:
+    __slots__ = ("kind", "id")
+
+    def __init__(self, kind: str, vid: int):
+        self.kind = kind  # 'v' vector | 's' scalar
+        self.id = vid
+
+
+class _RowCodegen:
+    """Turns one fused group into a row program (see include/nbk.h for the ISA)."""
+
+    def __init__(self, planner: Planner, g: Unit):
+        self.p = planner
+        self.g = g
+
+    # --- domain ------------------------------------------------------------
+    def _setup_domain(self):
+        g = self.g
+        lead, C = tuple(g.lead), g.C
+        self.drop_last = False
+        if C is None:
+            # every member is a row scalar: iterate over the last leading dim instead
+            if len(lead) >= 1:
+                C = lead[-1]
+                lead = lead[:-1]
+                self.drop_last = True
+            else:
+                C = 1
+        self.lead = lead
+        self.C = C
+
+    def _dom_strides(self, ref: ViewRef):
+        """(lead strides, column stride) of an operand shaped like a member value."""
+        shape, st = _shape2(ref.shape), ref.strides if ref.shape else (0,)
+        if self.drop_last:
+            shape, st = shape[:-1], st[:-1]
+            if len(shape) == 0:
+                return (), 0
+        lead_st = tuple(0 if d == 1 else s for d, s in zip(shape[:-1], st[:-1]))
+        col = 0 if shape[-1] == 1 else st[-1]
+        return lead_st, col
+
+    def _cls_of_shape(self, shape) -> str:
+        shape = _shape2(shape)
+        if self.drop_last:
+            shape = shape[:-1] if len(shape) > 1 else shape
+        return "F" if (shape[-1] == self.C and self.C != 1) or self.C == 1 else "R"
+
+    # --- main ----------------------------------------------------------------
+    def generate(self) -> Step:
+        p, g = self.p, self.g
+        self._setup_domain()
+        members = sorted(g.nodes, key=lambda n: n.pos)
+        member_pos = g.node_pos
+        has_reduce = any(n.kind == "reduce" for n in members)
+        has_tril = any(n.kind == "tril" for n in members)
+
+        # classes and in-group test
+        cls: dict[int, str] = {}
+        for n in members:
+            o = n.outputs[0]
+            if n.kind == "reduce":
+                cls[o.id] = "R"
+            else:
+                cls[o.id] = self._cls_of_shape(o.shape)
+
+        def in_group(v: ir.Value) -> bool:
+            return v.node.pos in member_pos and (v.node.kind in FUSABLE or v.node.pos in p.alias_nodes)
+
+        # ---- operands ----------------------------------------------------------
+        operands: list[OperandSpec] = []
+        op_index: dict[tuple, int] = {}
+        op_cls: list[str] = []
+
+        def ext_operand(v: ir.Value):
+            """('imm', value) or ('op', index, class) for an external input."""
+            loc = p._resolve(v)
+            if isinstance(loc, Const):
+                return ("imm", float(loc.value))
+            lead_st, col = self._dom_strides(loc)
+            key = (loc.buf, loc.offset, lead_st, col)
+            idx = op_index.get(key)
+            if idx is None:
+                idx = len(operands)
+                op_index[key] = idx
+                operands.append(OperandSpec(loc.buf, loc.offset, lead_st, col, loc.dtype, False))
+                if all(s == 0 for s in lead_st) and col == 0:
+                    op_cls.append("U")
+                elif col == 0 and self.C != 1:
+                    op_cls.append("R")
+                else:
+                    op_cls.append("F")
+            return ("op", idx, op_cls[idx])
+
+        # ---- phases ------------------------------------------------------------
+        ph: dict[int, int] = {}      # value id -> phase it is computed in
+        avail: dict[int, int] = {}   # row values: first phase whose prologue can read them
+        for n in members:
+            o = n.outputs[0]
+            if n.kind == "reduce":
+                x = n.inputs[0]
+                pin = ph[x.id] if in_group(x) else 0
+                ph[o.id] = pin
+                avail[o.id] = pin + 1
+                continue
+            m = 0
+            for i in n.inputs:
+                if in_group(i):
+                    m = max(m, avail[i.id] if cls[i.id] == "R" else ph[i.id])
+            ph[o.id] = m
+            if cls[o.id] == "R":
+                avail[o.id] = m
+        n_phase = max([0] + [avail.get(n.outputs[0].id, ph[n.outputs[0].id]) for n in members]) + 1
+
+        need_store = p.need_store
+        by_id = {n.outputs[0].id: n for n in members}
+
+        # ---- instruction stream with virtual registers -----------------------------
+        stream: list[list] = []  # [op, dst, a, b, c, aux]; registers are _VReg
+        n_vregs = [0]
+        imm_vals: list[float] = []
+
+        def new_v(kind: str) -> _VReg:
+            n_vregs[0] += 1
+            return _VReg(kind, n_vregs[0])
+
+        sreg_of: dict[Any, _VReg] = {}   # row value id / ('op', idx) / ('imm', value) -> sreg
+        out_operand: dict[int, int] = {}
+
+        def store_operand(v: ir.Value) -> int:
+            idx = out_operand.get(v.id)
+            if idx is None:
+                ref = p._alloc_value(v)
+                lead_st, col = self._dom_strides(ref)
+                idx = len(operands)
+                operands.append(OperandSpec(ref.buf, ref.offset, lead_st, col, ref.dtype, False,
+                                            is_output=True))
+                op_cls.append("O")
+                out_operand[v.id] = idx
+            return idx
+
+        def imm_index(val: float) -> int:
+            for i, x in enumerate(imm_vals):
+                if x == val or (x != x and val != val):
+                    if math.copysign(1.0, x) == math.copysign(1.0, val) or x != x:
+                        return i
+            imm_vals.append(val)
+            return len(imm_vals) - 1
+
+        prologue: list[list] = []
+
+        def scalar_for(key, emit) -> _VReg:
+            r = sreg_of.get(key)
+            if r is None:
+                r = new_v("s")
+                sreg_of[key] = r
+                emit(r)
+            return r
+
+        def scalar_imm(val: float) -> _VReg:
+            return scalar_for(("imm", val), lambda r: prologue.append(
+                [isa.IMM, r, imm_index(val), 0, 0, 0]))
+
+        def scalar_ext(idx: int) -> _VReg:
+            return scalar_for(("op", idx), lambda r: prologue.append([isa.LDR, r, idx, 0, 0, 0]))
+
+        def resolve_alias(v: ir.Value) -> ir.Value:
+            while v.node.pos in p.alias_nodes and v.node.pos in member_pos:
+                v = v.node.inputs[0]
+            return v
+
+        def tril_setup(n: ir.Node) -> _VReg:
+            """Scalar register holding (matrix row index + k)."""
+            key = ("tril", n.attrs["k"])
+            r = sreg_of.get(key)
+            if r is None:
+                row = new_v("s")
+                prologue.append([isa.LEADIDX, row, len(self.lead) - 1, 0, 0, 0])
+                kreg = scalar_imm(float(n.attrs["k"]))
+                r = new_v("s")
+                prologue.append([isa.EW["add"], r, row, kreg, 0, 0])
+                sreg_of[key] = r
+            return r
+
+        acc_slots: dict[int, int] = {}
+        for phase in range(n_phase):
+            prologue = []
+            body: list[list] = []
+            vreg_of: dict[Any, _VReg] = {}
+
+            # 1. reductions finished by the previous body
+            for n in members:
+                if n.kind == "reduce" and avail[n.outputs[0].id] == phase:
+                    r = new_v("s")
+                    sreg_of[n.outputs[0].id] = r
+                    prologue.append([isa.RED, r, acc_slots[n.outputs[0].id],
+                                     isa.RED_KIND[n.fn], 0, 0])
+            acc_slots_phase: dict[int, int] = {}
+
+            # 2. sinks of this phase and the set of full values to (re)compute
+            sinks: list[ir.Value] = []
+            for n in members:
+                o = n.outputs[0]
+                if n.kind == "reduce":
+                    if ph[o.id] == phase:
+                        x = n.inputs[0]
+                        if len(acc_slots_phase) >= isa.NACC:
+                            raise FusionLimit("more than 4 reductions in one phase")
+                        acc_slots_phase[o.id] = len(acc_slots_phase)
+                        if in_group(x):
+                            sinks.append(resolve_alias(x))
+                elif cls[o.id] == "F" and ph[o.id] == phase and o.id in need_store:
+                    sinks.append(o)
+            needed: set[int] = set()
+            stack = [s for s in sinks if in_group(s) and cls.get(s.id) == "F"]
+            while stack:
+                v = stack.pop()
+                if v.id in needed:
+                    continue
+                needed.add(v.id)
+                for i in v.node.inputs:
+                    if in_group(i):
+                        i2 = resolve_alias(i) if i.id not in need_store else i
+                        if cls.get(i2.id) == "F" and in_group(i2):
+                            stack.append(i2)
+
+            # 3. row-scalar ops that become computable in this phase
+            def scalar_operand(x, emit_list):
+                """Register of a row-class operand of a scalar op."""
+                if not isinstance(x, ir.Value):
+                    return scalar_imm(float(x))
+                if in_group(x):
+                    x2 = resolve_alias(x)
+                    return sreg_of[x2.id]
+                e = ext_operand(x)
+                if e[0] == "imm":
+                    return scalar_imm(e[1])
+                return scalar_ext(e[1])
+
+            for n in members:
+                o = n.outputs[0]
+                if n.kind in ("reduce",) or cls[o.id] != "R" or ph[o.id] != phase:
+                    continue
+                if n.pos in p.alias_nodes:
+                    continue
+                if n.kind != "ew":
+                    raise FusionLimit(f"row-class node of kind {n.kind}")
+                regs = [scalar_operand(x, prologue) for x in n.attrs["operands"]]
+                r = new_v("s")
+                sreg_of[o.id] = r
+                regs += [0] * (3 - len(regs))
+                prologue.append([isa.EW[n.fn], r, regs[0], regs[1], regs[2], 0])
+            # stores of row values that became available in this phase
+            for n in members:
+                o = n.outputs[0]
+                if cls[o.id] == "R" and avail[o.id] == phase and o.id in need_store and \
+                        n.pos not in p.alias_nodes:
+                    prologue.append([isa.STR, store_operand(o), sreg_of[o.id], 0, 0, 0])
+
+            # 4. body: full-class ops in topological order
+            def vec_operand(x):
+                if not isinstance(x, ir.Value):
+                    return scalar_imm(float(x))
+                if in_group(x):
+                    x2 = resolve_alias(x) if x.id not in vreg_of else x
+                    if cls.get(x2.id) == "R":
+                        return sreg_of[x2.id]
+                    return vreg_of[x2.id]
+                e = ext_operand(x)
+                if e[0] == "imm":
+                    return scalar_imm(e[1])
+                _, idx, c = e
+                if c in ("U", "R"):
+                    return scalar_ext(idx)
+                key = ("op", idx)
+                r = vreg_of.get(key)
+                if r is None:
+                    r = new_v("v")
+                    vreg_of[key] = r
+                    body.append([isa.LDG, r, idx, 0, 0, 0])
+                return r
+
+            for n in members:
+                o = n.outputs[0]
+                if n.kind == "reduce":
+                    if ph[o.id] == phase:
+                        x = n.inputs[0]
+                        src = vec_operand(x)
+                        if src.kind == "s":  # reducing a row scalar broadcast: materialise it
+                            t = new_v("v")
+                            body.append([isa.EW["mov"], t, src, 0, 0, 0])
+                            src = t
+                        body.append([isa.ACC, acc_slots_phase[o.id], src, isa.RED_KIND[n.fn], 0, 0])
+                    continue
+                if o.id not in needed:
+                    continue
+                if n.pos in p.alias_nodes:
+                    src = vec_operand(n.inputs[0])
+                    r = new_v("v")
+                    body.append([isa.EW["mov"], r, src, 0, 0, 0])
+                elif n.kind == "ew":
+                    regs = [vec_operand(x) for x in n.attrs["operands"]]
+                    regs += [0] * (3 - len(regs))
+                    r = new_v("v")
+                    body.append([isa.EW[n.fn], r, regs[0], regs[1], regs[2], 0])
+                elif n.kind == "tril":
+                    lim = tril_setup(n)
+                    x = vec_operand(n.inputs[0])
+                    zero = scalar_imm(0.0)
+                    c = new_v("v")
+                    body.append([isa.COLIDX, c, 0, 0, 0, 0])
+                    m = new_v("v")
+                    body.append([isa.EW["ge" if n.attrs["upper"] else "le"], m, c, lim, 0, 0])
+                    r = new_v("v")
+                    body.append([isa.EW["where"], r, m, x, zero, 0])
+                elif n.kind == "iota":
+                    c = new_v("v")
+                    body.append([isa.COLIDX, c, 0, 0, 0, 0])
+                    r = new_v("v")
+                    body.append([isa.EW["fma"], r, c, scalar_imm(n.attrs["step"]),
+                                 scalar_imm(n.attrs["start"]), 0])
+                else:
+                    raise AssertionError(n.kind)
+                vreg_of[o.id] = r
+                if o.id in need_store and ph[o.id] == phase:
+                    body.append([isa.STG, store_operand(o), r, 0, 0, 0])
+
+            for oid, slot in acc_slots_phase.items():
+                prologue.append([isa.ACCINIT, slot, isa.RED_KIND[by_id[oid].fn], 0, 0, 0])
+            acc_slots.update(acc_slots_phase)
+            stream.extend(prologue)
+            if body:
+                stream.append([isa.BODY, 0, 0, 0, 0, len(body)])
+                stream.extend(body)
+        stream.append([isa.HALT, 0, 0, 0, 0, 0])
+
+        ins = self._allocate(stream)
+        if len(ins) > isa.MAX_INS:
+            raise FusionLimit(f"{len(ins)} instructions")
+        if len(operands) > isa.MAX_OPERANDS:
+            raise FusionLimit(f"{len(operands)} operands")
+        if len(imm_vals) > isa.MAX_IMM:
+            raise FusionLimit(f"{len(imm_vals)} immediates")
+
+        lead, C = self._finish_domain(operands, has_reduce, has_tril, stream, op_cls)
+        # LDS staging of rows that are read in more than one phase
+        n_stage = 0
+        if has_reduce:
+            loads: dict[int, int] = {}
+            for i in ins:
+                if i[0] == isa.LDG:
+                    loads[i[2]] = loads.get(i[2], 0) + 1
+            c_pad = (C + 3) & ~3
+            for idx, cnt in sorted(loads.items()):
+                if cnt >= 2 and n_stage < isa.MAX_STAGE and (n_stage + 1) * c_pad * 4 <= isa.STAGE_BYTES:
+                    operands[idx].stage_slot = n_stage
+                    n_stage += 1
+        chunks = (C + 3) // 4
+        block = 64
+        while block < isa.MAX_BLOCK and block * 2 < chunks:
+            block *= 2
+        reads = sorted({o.buf for o in operands if not o.is_output})
+        writes = sorted({o.buf for o in operands if o.is_output})
+        return Step("rowprog", reads, writes, dict(
+            lead=lead, C=C, has_reduce=has_reduce, block=block, n_stage=n_stage,
+            operands=operands, ins=ins, imm=imm_vals,
+            members=[f"{n.kind}.{n.fn}" if n.fn else n.kind for n in members]))
+
+    # --- domain collapse -----------------------------------------------------------
+    def _finish_domain(self, operands, has_reduce, has_tril, stream, op_cls):
+        lead = list(self.lead)
+        C = self.C
+        sts = [list(o.lead_strides) for o in operands]
+        uses_leadidx = any(i[0] == isa.LEADIDX for i in stream)
+        # drop unit leading dims, merge adjacent ones that every operand walks linearly
+        k = 0
+        while k < len(lead):
+            if lead[k] == 1 and not (uses_leadidx and k == len(lead) - 1):
+                del lead[k]
+                for s in sts:
+                    del s[k]
+                continue
+            k += 1
+        if not uses_leadidx:
+            k = 0
+            while k + 1 < len(lead):
+                if all(s[k] == s[k + 1] * lead[k + 1] for s in sts):
+                    lead[k] = lead[k] * lead[k + 1]
+                    del lead[k + 1]
+                    for s in sts:
+                        s[k] = s[k + 1]
+                        del s[k + 1]
+                    continue
+                k += 1
+        per_row = any(i[0] in (isa.LDR, isa.STR, isa.LEADIDX) for i in stream)
+        row_ops = {i[2] for i in stream if i[0] == isa.LDR} | {i[1] for i in stream if i[0] == isa.STR}
+        uniform_only = all(all(x == 0 for x in sts[j]) and operands[j].col_stride == 0
+                           for j in row_ops)
+        if not has_reduce and not has_tril and (not per_row or uniform_only):
+            # pure elementwise: fold leading dims into the row while every
+            # operand stays linear
+            while lead:
+                ok = all((o.col_stride == 1 and s[-1] == C) or
+                         (o.col_stride == 0 and all(x == 0 for x in s))
+                         for o, s in zip(operands, sts))
+                if not ok:
+                    break
+                C *= lead[-1]
+                lead.pop()
+                for s in sts:
+                    s.pop()
+        if len(lead) > isa.MAX_LEAD:
+            raise FusionLimit(f"{len(lead)} leading dims after collapse")
+        for o, s in zip(operands, sts):
+            o.lead_strides = tuple(s)
+            o.vec_ok = bool(o.col_stride == 1 and o.offset % 4 == 0 and all(x % 4 == 0 for x in s))
+        return tuple(lead), C
+
+    # --- register allocation -------------------------------------------------------
+    def _allocate(self, stream):
+        """Map virtual registers to the 16 vector + 16 scalar physical ones.
+
+        Vector registers live inside one body; scalar registers live across the
+        program, and one that is read inside a body stays reserved until the
+        body's last instruction (the body runs once per chunk)."""
+        def regs_of(ins):
+            op = ins[0]
+            dst = None
+            if op in (isa.IMM, isa.LDR, isa.LEADIDX, isa.RED, isa.LDG, isa.COLIDX) or op >= 16:
+                dst = ins[1]
+            srcs = [x for x in ins[2:5] if isinstance(x, _VReg)]
+            return dst, srcs
+
+        body_end: dict[int, int] = {}
+        i = 0
+        while i < len(stream):
+            if stream[i][0] == isa.BODY:
+                end = i + stream[i][5]
+                for q in range(i + 1, end + 1):
+                    body_end[q] = end
+                i = end + 1
+            else:
+                i += 1
+        last: dict[int, int] = {}
+        reg_by_id: dict[int, _VReg] = {}
+        for idx, ins in enumerate(stream):
+            dst, srcs = regs_of(ins)
+            for r in srcs + ([dst] if dst is not None else []):
+                pos = body_end.get(idx, idx) if r.kind == "s" else idx
+                last[r.id] = max(last.get(r.id, -1), pos)
+                reg_by_id[r.id] = r
+        free_at: dict[int, list[_VReg]] = {}
+        for rid, pos in last.items():
+            free_at.setdefault(pos, []).append(reg_by_id[rid])
+
+        free_s = list(range(isa.NVEC + isa.NSCL - 1, isa.NVEC - 1, -1))
+        free_v = list(range(isa.NVEC - 1, -1, -1))
+        phys: dict[int, int] = {}
+        out = []
+        for idx, ins in enumerate(stream):
+            if ins[0] == isa.BODY:
+                free_v = list(range(isa.NVEC - 1, -1, -1))
+            dst, srcs = regs_of(ins)
+            enc = list(ins)
+            for k in range(2, 5):
+                if isinstance(enc[k], _VReg):
+                    enc[k] = phys[enc[k].id]
+            dying = free_at.get(idx, [])
+            for r in dying:  # sources that die here may be reused by the destination
+                if r.id in phys and (dst is None or r.id != dst.id):
+                    (free_v if r.kind == "v" else free_s).append(phys[r.id])
+            if dst is not None:
+                pool = free_v if dst.kind == "v" else free_s
+                if dst.id not in phys:
+                    if not pool:
+                        raise FusionLimit("out of registers")
+                    phys[dst.id] = pool.pop()
+                enc[1] = phys[dst.id]
+                if any(r.id == dst.id for r in dying):
+                    pool.append(phys[dst.id])
+            out.append(tuple(int(x) for x in enc))
+        return out
+
+
+def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
+    """Plan with shrinking fusion limits until every group fits a row program."""
+    last = None
+    for limit in (28, 16, 8, 4, 1):
+        try:
+            return Planner(builder, outputs, max_members=limit).build()
+        except FusionLimit as e:  # retry with smaller groups
+            last = e
+    raise RuntimeError(f"lowering failed even without fusion: {last}")

@@ -1,0 +1,61 @@
+"""Context-scoped flags (mirrors nabla/config.py:26-109).
+
+``EAGER_MAX_GRAPH`` keeps its reference name: when set, every op call is
+lowered immediately into the graph under construction instead of being
+deferred; ``compile`` sets it while it traces.  ``VERIFY_EAGER_SHAPES`` checks
+the lowering's shapes against ``compute_physical_shape``.
+"""
+from __future__ import annotations
+
+import contextlib
+import os
+from contextvars import ContextVar
+
+
+def _env_flag(name: str, default: bool = False) -> bool:
+    return os.environ.get(name, "1" if default else "0") in {"1", "true", "TRUE", "True"}
+
+
+_EAGER_MAX_GRAPH: ContextVar[bool] = ContextVar("EAGER_MAX_GRAPH", default=_env_flag("EAGER_MAX_GRAPH"))
+_VERIFY_EAGER_SHAPES: ContextVar[bool] = ContextVar(
+    "VERIFY_EAGER_SHAPES", default=_env_flag("VERIFY_EAGER_SHAPES")
+)
+_TRACING: ContextVar[bool] = ContextVar("TRACING", default=False)
+
+_FLAGS = {
+    "EAGER_MAX_GRAPH": _EAGER_MAX_GRAPH,
+    "VERIFY_EAGER_SHAPES": _VERIFY_EAGER_SHAPES,
+    "TRACING": _TRACING,
+}
+
+
+def __getattr__(name: str):
+    var = _FLAGS.get(name)
+    if var is None:
+        raise AttributeError(name)
+    return var.get()
+
+
+def set_flag(name: str, value: bool):
+    return _FLAGS[name].set(bool(value))
+
+
+def reset_flag(name: str, token) -> None:
+    _FLAGS[name].reset(token)
+
+
+@contextlib.contextmanager
+def flag(name: str, value: bool):
+    tok = set_flag(name, value)
+    try:
+        yield
+    finally:
+        reset_flag(name, tok)
+
+
+def eager_mode(value: bool = True):
+    return flag("EAGER_MAX_GRAPH", value)
+
+
+def verify_eager_shapes(value: bool = True):
+    return flag("VERIFY_EAGER_SHAPES", value)

@@ -1,0 +1,444 @@
+// GEMM for gfx950: C[b] = alpha * A[b] @ B[b] (+bias) (act) (+residual).
+//
+// bf16 path (fp32 accumulate): v_mfma_f32_32x32x16_bf16.  A workgroup of four
+// waves (2 x 2) owns a BM x BN tile of C; K advances in steps of 64 through two
+// LDS buffers.  Both operands sit in LDS as [row][64 k] with 128-byte rows whose
+// eight 16-byte chunks are XOR-swizzled by (row % 8) ^ (row / 8 % 8), which makes
+// the 16-byte fragment reads of the MFMA (32 consecutive rows, one chunk) and
+// both kinds of tile writes below conflict-free without padding.
+//   * an operand that is contiguous along K is copied 16 bytes at a time;
+//   * an operand that is contiguous along its row index (the transposed operand
+//     of the two backward products, and B of the forward product) is read as
+//     8 x 8 blocks and transposed in registers before it is written, so the
+//     swap_axes of the backward GEMMs never touches memory.
+// fp32 path: v_mfma_f32_32x32x2f32 with a 128 x 128 x 16 tile, operands kept
+// k-major in LDS.
+#include "nbk_common.h"
+
+#include <utility>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Compile-time loop: accumulator tiles must be indexed with constants or they
+// leave the register file.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+struct GemmArgs {
+  const void* A; const void* B; void* C; const void* bias; const void* residual;
+  int64_t M, N, K;
+  int64_t a_rs, a_cs, b_rs, b_cs, ldc;
+  int64_t a_bs, b_bs, c_bs;
+  int32_t dtype_c, act;
+  float alpha;
+  int32_t tiles_m, tiles_n;
+  int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
+};
+
+__device__ __forceinline__ float gemm_act(float v, int act) {
+  if (act == NBK_ACT_RELU) return fmaxf(v, 0.f);
+  if (act == NBK_ACT_GELU) return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
+  return v;
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// Re-number them so that every XCD works on one contiguous run of tiles, then
+// walk that run in groups of 8 tile-rows per tile-column: workgroups that share
+// an L2 also share the A and B panels they read.
+__device__ __forceinline__ void gemm_tile_coords(int bid, int tiles_m, int tiles_n, int& tm,
+                                                 int& tn) {
+  {
+    const int n = tiles_m * tiles_n;
+    const int xcd = bid & 7, local = bid >> 3;
+    const int per = n >> 3, rem = n & 7;
+    bid = xcd < rem ? xcd * (per + 1) + local : rem * (per + 1) + (xcd - rem) * per + local;
+  }
+  const int group = 8;
+  const int per_group = group * tiles_n;
+  const int g = bid / per_group;
+  const int first_m = g * group;
+  const int gsize = min(group, tiles_m - first_m);
+  const int r = bid - g * per_group;
+  tm = first_m + r % gsize;
+  tn = r / gsize;
+}
+
+// ---------------------------------------------------------------------------- bf16
+__device__ __forceinline__ int swz(int row, int chunk) {
+  return row * 8 + (chunk ^ (row & 7) ^ ((row >> 3) & 7));
+}
+
+// 16-byte guarded load of 8 consecutive bf16 along the unit-stride axis.
+__device__ __forceinline__ uint4 ld8_bf16(const uint16_t* p, int64_t valid, bool vec) {
+  uint4 r = make_uint4(0, 0, 0, 0);
+  if (valid >= 8 && vec) return *(const uint4*)p;
+  if (valid <= 0) return r;
+  uint16_t t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = i < valid ? p[i] : (uint16_t)0;
+  r.x = t[0] | ((uint32_t)t[1] << 16);
+  r.y = t[2] | ((uint32_t)t[3] << 16);
+  r.z = t[4] | ((uint32_t)t[5] << 16);
+  r.w = t[6] | ((uint32_t)t[7] << 16);
+  return r;
+}
+
+template <int ROWS, bool KC>
+struct TileLoader {
+  // KC : operand contiguous along K   -> ROWS*8 chunk tasks, ROWS/32 per lane
+  // !KC: operand contiguous along rows -> ROWS (8x8 block) tasks, <=1 per lane
+  static constexpr int NREG = KC ? ROWS / 32 : 8;
+  uint4 reg[NREG];
+
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t rs, int64_t cs, int64_t row0,
+                                       int64_t rows_total, int64_t k0, int64_t K, bool vec) {
+    const int tid = threadIdx.x;
+    if (KC) {
+#pragma unroll
+      for (int s = 0; s < NREG; ++s) {
+        const int t = tid + s * 256;
+        const int row = t >> 3, c = t & 7;
+        const int64_t gr = row0 + row, gk = k0 + c * 8;
+        if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
+        else reg[s] = make_uint4(0, 0, 0, 0);
+      }
+    } else {
+      constexpr int NC = ROWS / 8;
+      const int nc = tid % NC, kg = tid / NC;
+      if (kg < 8) {
+        const int64_t gr = row0 + nc * 8;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const int64_t gk = k0 + kg * 8 + r;
+          if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
+          else reg[r] = make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(uint4* lds) {
+    const int tid = threadIdx.x;
+    if (KC) {
+#pragma unroll
+      for (int s = 0; s < NREG; ++s) {
+        const int t = tid + s * 256;
+        lds[swz(t >> 3, t & 7)] = reg[s];
+      }
+    } else {
+      constexpr int NC = ROWS / 8;
+      const int nc = tid % NC, kg = tid / NC;
+      if (kg < 8) {
+        // 8x8 transpose of 16-bit elements: out[j] holds k = 0..7 of column j
+        const uint32_t* in = (const uint32_t*)reg;  // in[r*4 + d]
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int d = j >> 1;
+          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+          uint4 o;
+          o.x = __builtin_amdgcn_perm(in[1 * 4 + d], in[0 * 4 + d], sel);
+          o.y = __builtin_amdgcn_perm(in[3 * 4 + d], in[2 * 4 + d], sel);
+          o.z = __builtin_amdgcn_perm(in[5 * 4 + d], in[4 * 4 + d], sel);
+          o.w = __builtin_amdgcn_perm(in[7 * 4 + d], in[6 * 4 + d], sel);
+          lds[swz(nc * 8 + j, kg)] = o;
+        }
+      }
+    }
+  }
+};
+
+extern __shared__ __align__(16) uint4 gemm_lds[];
+
+template <int BM, int BN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
+  constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int TILE_CHUNKS = (BM + BN) * 8;
+  int tm_i, tn_i;
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
+  const int64_t b = blockIdx.y;
+  const uint16_t* A = (const uint16_t*)g.A + b * g.a_bs;
+  const uint16_t* B = (const uint16_t*)g.B + b * g.b_bs;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int li = lane & 31, kg = lane >> 5;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
+
+  TileLoader<BM, A_KC> la;
+  TileLoader<BN, B_KC> lb;
+  const int64_t nk = (g.K + 63) / 64;
+  // A is rows = m; for the loader a K-contiguous operand has (rs = row stride, k unit),
+  // a row-contiguous one has (cs = k stride, row unit).
+  la.load(A, g.a_rs, g.a_cs, m0, g.M, 0, g.K, g.a_vec);
+  lb.load(B, g.b_cs, g.b_rs, n0, g.N, 0, g.K, g.b_vec);
+  la.store(gemm_lds);
+  lb.store(gemm_lds + BM * 8);
+  __syncthreads();
+
+  for (int64_t kt = 0; kt < nk; ++kt) {
+    const uint4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
+    uint4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.load(A, g.a_rs, g.a_cs, m0, g.M, (kt + 1) * 64, g.K, g.a_vec);
+      lb.load(B, g.b_cs, g.b_rs, n0, g.N, (kt + 1) * 64, g.K, g.b_vec);
+    }
+    const uint4* As = cur;
+    const uint4* Bs = cur + BM * 8;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int kc = ks * 2 + kg;
+      bf16x8 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        uint4 u = As[swz(wm + i * 32 + li, kc)];
+        fa[i] = *(bf16x8*)&u;
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        uint4 u = Bs[swz(wn + j * 32 + li, kc)];
+        fb[j] = *(bf16x8*)&u;
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      la.store(nxt);
+      lb.store(nxt + BM * 8);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: D[i][j] of a 32x32 tile lives in lane (j, (i / 4) % 2), register
+  // (i / 8) * 4 + i % 4.
+  char* Cb = (char*)g.C;
+  const bool out_f32 = g.dtype_c == NBK_F32;
+  static_for<TM * TN>([&](auto t) {
+    constexpr int i = decltype(t)::value / TN, j = decltype(t)::value % TN;
+    const int64_t col = n0 + wn + j * 32 + li;
+    const bool col_ok = col < g.N;
+    float bv = 0.f;
+    if (g.bias && col_ok) bv = nbk_load_as_f32(g.bias, col, g.dtype_c);
+    const f32x16 a = acc[i][j];
+    const int64_t row_base = m0 + wm + i * 32 + kg * 4;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t row = row_base + (r >> 2) * 8 + (r & 3);
+      if (col_ok && row < g.M) {
+        float v = a[r] * g.alpha + bv;
+        v = gemm_act(v, g.act);
+        const int64_t idx = b * g.c_bs + row * g.ldc + col;
+        if (g.residual) v += nbk_load_as_f32(g.residual, idx, g.dtype_c);
+        if (out_f32) ((float*)Cb)[idx] = v;
+        else ((uint16_t*)Cb)[idx] = nbk_f32_to_bf16(v);
+      }
+    }
+  });
+}
+
+// ---------------------------------------------------------------------------- fp32
+// 128 x 128 x 16 tile, LDS k-major ([k][rows], rows padded by 4 floats).
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
+  constexpr int BM = 128, BN = 128, BK = 16, LD = 128 + 4;
+  __shared__ float As[2][BK][LD];
+  __shared__ float Bs[2][BK][LD];
+  int tm_i, tn_i;
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
+  const int64_t b = blockIdx.y;
+  const float* A = (const float*)g.A + b * g.a_bs;
+  const float* B = (const float*)g.B + b * g.b_bs;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int li = lane & 31, kg = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x16)(0.f);
+
+  // each lane stages 8 floats of A and 8 of B per k-tile (128*16 / 256)
+  float ra[8], rb[8];
+  auto load_tile = [&](const float* P, int64_t rs, int64_t cs, int64_t row0, int64_t rows_total,
+                       int64_t k0, bool kc, bool vec, float* r) {
+    if (kc) {
+      // unit stride along k: lane -> (row = tid/2, 8 consecutive k)
+      const int row = tid >> 1, kk = (tid & 1) * 8;
+      const int64_t gr = row0 + row;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int64_t gk = k0 + kk + e;
+        r[e] = (gr < rows_total && gk < g.K) ? P[gr * rs + gk] : 0.f;
+      }
+    } else {
+      // unit stride along rows: lane -> (k = tid/16, 8 consecutive rows)
+      const int kk = tid >> 4, rr = (tid & 15) * 8;
+      const int64_t gk = k0 + kk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int64_t gr = row0 + rr + e;
+        r[e] = (gr < rows_total && gk < g.K) ? P[gk * cs + gr] : 0.f;
+      }
+    }
+  };
+  auto store_tile = [&](float (*S)[LD], bool kc, const float* r) {
+    if (kc) {
+      const int row = tid >> 1, kk = (tid & 1) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) S[kk + e][row] = r[e];
+    } else {
+      const int kk = tid >> 4, rr = (tid & 15) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) S[kk][rr + e] = r[e];
+    }
+  };
+
+  const int64_t nk = (g.K + BK - 1) / BK;
+  load_tile(A, g.a_rs, g.a_cs, m0, g.M, 0, A_KC, g.a_vec, ra);
+  load_tile(B, g.b_cs, g.b_rs, n0, g.N, 0, B_KC, g.b_vec, rb);
+  store_tile(As[0], A_KC, ra);
+  store_tile(Bs[0], B_KC, rb);
+  __syncthreads();
+  for (int64_t kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      load_tile(A, g.a_rs, g.a_cs, m0, g.M, (kt + 1) * BK, A_KC, g.a_vec, ra);
+      load_tile(B, g.b_cs, g.b_rs, n0, g.N, (kt + 1) * BK, B_KC, g.b_vec, rb);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 2; ++ks) {
+      const int k = ks * 2 + kg;
+      float fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = As[cur][k][wm + i * 32 + li];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = Bs[cur][k][wn + j * 32 + li];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      store_tile(As[cur ^ 1], A_KC, ra);
+      store_tile(Bs[cur ^ 1], B_KC, rb);
+    }
+    __syncthreads();
+  }
+  float* C = (float*)g.C;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t col = n0 + wn + j * 32 + li;
+      if (col >= g.N) continue;
+      float bv = g.bias ? ((const float*)g.bias)[col] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t row = m0 + wm + i * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
+        if (row >= g.M) continue;
+        float v = gemm_act(acc[i][j][r] * g.alpha + bv, g.act);
+        const int64_t idx = b * g.c_bs + row * g.ldc + col;
+        if (g.residual) v += ((const float*)g.residual)[idx];
+        C[idx] = v;
+      }
+    }
+}
+
+// ------------------------------------------------------------------------- dispatch
+template <int BM, int BN>
+static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
+  GemmArgs g = a;
+  g.tiles_m = (int)((a.M + BM - 1) / BM);
+  g.tiles_n = (int)((a.N + BN - 1) / BN);
+  dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
+  const size_t lds = 2 * (size_t)(BM + BN) * 8 * sizeof(uint4);
+#define NBK_LAUNCH_BF16(AK, BK_)                                                              \
+  do {                                                                                        \
+    auto kern = gemm_bf16_kernel<BM, BN, AK, BK_>;                                            \
+    static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
+    if (!attr_set) {                                                                          \
+      NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                  (int)lds));                                                 \
+      attr_set = true;                                                                        \
+    }                                                                                         \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, g);                                    \
+  } while (0)
+  if (akc && bkc) NBK_LAUNCH_BF16(true, true);
+  else if (akc && !bkc) NBK_LAUNCH_BF16(true, false);
+  else if (!akc && bkc) NBK_LAUNCH_BF16(false, true);
+  else NBK_LAUNCH_BF16(false, false);
+#undef NBK_LAUNCH_BF16
+  return nbk_check_launch("gemm_bf16_kernel");
+}
+
+extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
+  NBK_REQUIRE(d != nullptr, "gemm: null descriptor");
+  NBK_REQUIRE(d->A && d->B && d->C, "gemm: null operand pointer");
+  NBK_REQUIRE(d->M > 0 && d->N > 0 && d->K > 0, "gemm: empty problem %lld x %lld x %lld",
+              (long long)d->M, (long long)d->N, (long long)d->K);
+  NBK_REQUIRE(d->batch >= 1 && d->batch <= 65535, "gemm: batch %lld out of range",
+              (long long)d->batch);
+  NBK_REQUIRE(d->dtype_ab == NBK_F32 || d->dtype_ab == NBK_BF16, "gemm: operand dtype %d",
+              d->dtype_ab);
+  NBK_REQUIRE(d->dtype_c == NBK_F32 || d->dtype_c == NBK_BF16, "gemm: result dtype %d",
+              d->dtype_c);
+  NBK_REQUIRE(d->dtype_ab == NBK_BF16 || d->dtype_c == NBK_F32,
+              "gemm: fp32 operands need an fp32 result");
+  NBK_REQUIRE(d->a_rs == 1 || d->a_cs == 1, "gemm: A needs a unit stride (rs=%lld, cs=%lld)",
+              (long long)d->a_rs, (long long)d->a_cs);
+  NBK_REQUIRE(d->b_rs == 1 || d->b_cs == 1, "gemm: B needs a unit stride (rs=%lld, cs=%lld)",
+              (long long)d->b_rs, (long long)d->b_cs);
+  NBK_REQUIRE(d->ldc >= d->N, "gemm: ldc %lld < N %lld", (long long)d->ldc, (long long)d->N);
+  NBK_REQUIRE(d->batch_reduce == 0, "gemm: batch_reduce is folded into K by the caller");
+  hipStream_t st = (hipStream_t)stream;
+  GemmArgs a;
+  a.A = d->A; a.B = d->B; a.C = d->C; a.bias = d->bias; a.residual = d->residual;
+  a.M = d->M; a.N = d->N; a.K = d->K;
+  a.a_rs = d->a_rs; a.a_cs = d->a_cs; a.b_rs = d->b_rs; a.b_cs = d->b_cs; a.ldc = d->ldc;
+  a.a_bs = d->a_bs; a.b_bs = d->b_bs; a.c_bs = d->c_bs;
+  a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
+  // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
+  const bool akc = d->a_cs == 1;
+  const bool bkc = d->b_rs == 1;
+  const int esz = d->dtype_ab == NBK_F32 ? 4 : 2;
+  auto vec_ok = [&](const void* p, int64_t other_stride, int64_t bs) {
+    const int64_t q = 16 / esz;
+    return ((uintptr_t)p % 16 == 0) && (other_stride % q == 0) && (bs % q == 0);
+  };
+  a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs);
+  a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs);
+  if (d->dtype_ab == NBK_BF16) {
+    const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
+    if (big_tiles >= 384 && d->M >= 256 && d->N >= 256)
+      return launch_bf16<256, 256>(a, akc, bkc, d->batch, st);
+    return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);
+  }
+  a.tiles_m = (int)((d->M + 127) / 128);
+  a.tiles_n = (int)((d->N + 127) / 128);
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)d->batch);
+  if (akc && bkc) hipLaunchKernelGGL((gemm_f32_kernel<true, true>), grid, dim3(256), 0, st, a);
+  else if (akc) hipLaunchKernelGGL((gemm_f32_kernel<true, false>), grid, dim3(256), 0, st, a);
+  else if (bkc) hipLaunchKernelGGL((gemm_f32_kernel<false, true>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((gemm_f32_kernel<false, false>), grid, dim3(256), 0, st, a);
+  return nbk_check_launch("gemm_f32_kernel");
+}

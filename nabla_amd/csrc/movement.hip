@@ -1,0 +1,203 @@
+// Data-movement kernels: strided copy (materialise a view), fill, and the
+// reduction over a middle axis.
+#include "nbk_common.h"
+
+struct CopyDesc {
+  int rank;
+  int64_t shape[NBK_MAX_RANK];
+  int64_t sstride[NBK_MAX_RANK];
+  int64_t dstride[NBK_MAX_RANK];
+};
+
+// Generic path: one lane per element, index decomposed innermost-first.
+template <typename T_SRC, typename T_DST, bool CONVERT>
+__global__ __launch_bounds__(256) void copy_strided_kernel(const void* __restrict__ src,
+                                                           void* __restrict__ dst, CopyDesc d,
+                                                           int64_t total, int dts, int dtd) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    int64_t rem = i, so = 0, dof = 0;
+    for (int k = d.rank - 1; k >= 0; --k) {
+      int64_t q = rem / d.shape[k];
+      int64_t r = rem - q * d.shape[k];
+      so += r * d.sstride[k];
+      dof += r * d.dstride[k];
+      rem = q;
+    }
+    if (CONVERT) {
+      nbk_store_from_f32(dst, dof, dtd, nbk_load_as_f32(src, so, dts));
+    } else {
+      ((T_DST*)dst)[dof] = ((const T_SRC*)src)[so];
+    }
+  }
+}
+
+// 2-D transpose-style tile through LDS for the case where the source is
+// unit-stride along some axis other than the last: both sides stay coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void copy_tile_kernel(const T* __restrict__ src,
+                                                        T* __restrict__ dst, CopyDesc d,
+                                                        int ax_s /* src-contiguous axis */) {
+  // tile over (ax_s, last); the remaining axes are enumerated by blockIdx.z
+  __shared__ T tile[64][65];
+  const int last = d.rank - 1;
+  const int64_t n_s = d.shape[ax_s], n_l = d.shape[last];
+  int64_t rem = blockIdx.z, so = 0, dof = 0;
+  for (int k = d.rank - 1; k >= 0; --k) {
+    if (k == ax_s || k == last) continue;
+    int64_t q = rem / d.shape[k];
+    int64_t r = rem - q * d.shape[k];
+    so += r * d.sstride[k];
+    dof += r * d.dstride[k];
+    rem = q;
+  }
+  const int64_t s0 = (int64_t)blockIdx.y * 64, l0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  // read: lanes run along ax_s (unit stride in src)
+  for (int j = ty; j < 64; j += 4) {
+    int64_t s = s0 + tx, l = l0 + j;
+    if (s < n_s && l < n_l) tile[j][tx] = src[so + s * d.sstride[ax_s] + l * d.sstride[last]];
+  }
+  __syncthreads();
+  // write: lanes run along the last axis (unit stride in dst)
+  for (int j = ty; j < 64; j += 4) {
+    int64_t s = s0 + j, l = l0 + tx;
+    if (s < n_s && l < n_l) dst[dof + s * d.dstride[ax_s] + l * d.dstride[last]] = tile[tx][j];
+  }
+}
+
+extern "C" int nbk_copy_strided(const void* src, void* dst, int32_t dts, int32_t dtd, int32_t rank,
+                                const int64_t* shape, const int64_t* sstride,
+                                const int64_t* dstride, void* stream) {
+  NBK_REQUIRE(src && dst, "copy_strided: null pointer");
+  NBK_REQUIRE(rank >= 0 && rank <= NBK_MAX_RANK, "copy_strided: rank %d exceeds %d", rank,
+              NBK_MAX_RANK);
+  NBK_REQUIRE(nbk_dtype_size(dts) > 0 && nbk_dtype_size(dtd) > 0, "copy_strided: bad dtype");
+  CopyDesc d;
+  d.rank = rank;
+  int64_t total = 1;
+  for (int k = 0; k < rank; ++k) {
+    NBK_REQUIRE(shape[k] >= 0, "copy_strided: negative extent");
+    d.shape[k] = shape[k];
+    d.sstride[k] = sstride[k];
+    d.dstride[k] = dstride[k];
+    total *= shape[k];
+  }
+  if (total == 0) return NBK_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const int es = nbk_dtype_size(dts);
+  if (dts == dtd && rank >= 2 && d.dstride[rank - 1] == 1 && d.sstride[rank - 1] != 1 &&
+      (es == 4 || es == 2)) {
+    int ax = -1;
+    for (int k = rank - 2; k >= 0; --k)
+      if (d.sstride[k] == 1 && d.shape[k] >= 16) { ax = k; break; }
+    if (ax >= 0 && d.shape[rank - 1] >= 16) {
+      int64_t nz = total / (d.shape[ax] * d.shape[rank - 1]);
+      int64_t gx = (d.shape[rank - 1] + 63) / 64, gy = (d.shape[ax] + 63) / 64;
+      if (nz <= 65535 && gy <= 65535) {
+        dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)nz);
+        if (es == 4)
+          hipLaunchKernelGGL(copy_tile_kernel<uint32_t>, grid, dim3(256), 0, st,
+                             (const uint32_t*)src, (uint32_t*)dst, d, ax);
+        else
+          hipLaunchKernelGGL(copy_tile_kernel<uint16_t>, grid, dim3(256), 0, st,
+                             (const uint16_t*)src, (uint16_t*)dst, d, ax);
+        return nbk_check_launch("copy_tile_kernel");
+      }
+    }
+  }
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 1 << 20) blocks = 1 << 20;
+  dim3 grid((unsigned)blocks);
+  if (dts != dtd) {
+    hipLaunchKernelGGL((copy_strided_kernel<float, float, true>), grid, dim3(256), 0, st, src, dst,
+                       d, total, dts, dtd);
+  } else if (es == 4) {
+    hipLaunchKernelGGL((copy_strided_kernel<uint32_t, uint32_t, false>), grid, dim3(256), 0, st,
+                       src, dst, d, total, dts, dtd);
+  } else if (es == 2) {
+    hipLaunchKernelGGL((copy_strided_kernel<uint16_t, uint16_t, false>), grid, dim3(256), 0, st,
+                       src, dst, d, total, dts, dtd);
+  } else if (es == 8) {
+    hipLaunchKernelGGL((copy_strided_kernel<uint64_t, uint64_t, false>), grid, dim3(256), 0, st,
+                       src, dst, d, total, dts, dtd);
+  } else {
+    hipLaunchKernelGGL((copy_strided_kernel<uint8_t, uint8_t, false>), grid, dim3(256), 0, st, src,
+                       dst, d, total, dts, dtd);
+  }
+  return nbk_check_launch("copy_strided_kernel");
+}
+
+// ---- fill -------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fill_kernel(void* dst, int dt, int64_t n, float v,
+                                                   int64_t iv) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    if (dt == NBK_I64) ((int64_t*)dst)[i] = iv;
+    else if (dt == NBK_I32) ((int32_t*)dst)[i] = (int32_t)iv;
+    else nbk_store_from_f32(dst, i, dt, v);
+  }
+}
+extern "C" int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void* stream) {
+  NBK_REQUIRE(dst || n == 0, "fill: null pointer");
+  NBK_REQUIRE(nbk_dtype_size(dtype) > 0, "fill: bad dtype %d", dtype);
+  if (n <= 0) return NBK_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, dst,
+                     dtype, n, (float)value, (int64_t)value);
+  return nbk_check_launch("fill_kernel");
+}
+
+// ---- reduction over a middle axis ---------------------------------------------
+// in [outer, red, inner] -> out [outer, inner].  Lanes run along `inner`
+// (coalesced); each workgroup owns a 64-column strip and splits `red` over its
+// four waves, then combines the four partials through LDS.  Two-level split of
+// `red` across workgroups goes through fp32 atomics only for sums of long axes.
+__device__ __forceinline__ float red_comb(float a, float b, int kind) {
+  return kind == NBK_RED_SUM ? a + b : (kind == NBK_RED_MAX ? fmaxf(a, b) : fminf(a, b));
+}
+__global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict__ in,
+                                                         void* __restrict__ out, int dti, int dto,
+                                                         int64_t red, int64_t inner, int kind) {
+  __shared__ float part[4][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t o = blockIdx.y;
+  const int64_t col = (int64_t)blockIdx.x * 64 + lane;
+  float acc = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
+  if (col < inner) {
+    const int64_t base = o * red * inner + col;
+    // four accumulators keep four loads in flight
+    float a0 = acc, a1 = acc, a2 = acc, a3 = acc;
+    int64_t r = w;
+    for (; r + 12 < red; r += 16) {
+      float v0 = nbk_load_as_f32(in, base + r * inner, dti);
+      float v1 = nbk_load_as_f32(in, base + (r + 4) * inner, dti);
+      float v2 = nbk_load_as_f32(in, base + (r + 8) * inner, dti);
+      float v3 = nbk_load_as_f32(in, base + (r + 12) * inner, dti);
+      a0 = red_comb(a0, v0, kind); a1 = red_comb(a1, v1, kind);
+      a2 = red_comb(a2, v2, kind); a3 = red_comb(a3, v3, kind);
+    }
+    for (; r < red; r += 4) a0 = red_comb(a0, nbk_load_as_f32(in, base + r * inner, dti), kind);
+    acc = red_comb(red_comb(a0, a1, kind), red_comb(a2, a3, kind), kind);
+  }
+  part[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && col < inner) {
+    float v = red_comb(red_comb(part[0][lane], part[1][lane], kind),
+                       red_comb(part[2][lane], part[3][lane], kind), kind);
+    nbk_store_from_f32(out, o * inner + col, dto, v);
+  }
+}
+
+extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
+                              int64_t red, int64_t inner, int32_t kind, void* stream) {
+  NBK_REQUIRE(in && out, "reduce_mid: null pointer");
+  NBK_REQUIRE(outer > 0 && red > 0 && inner > 0, "reduce_mid: empty extent");
+  NBK_REQUIRE(kind >= NBK_RED_SUM && kind <= NBK_RED_MIN, "reduce_mid: kind %d", kind);
+  NBK_REQUIRE(nbk_dtype_size(dti) > 0 && nbk_dtype_size(dto) > 0, "reduce_mid: bad dtype");
+  NBK_REQUIRE(outer <= 65535, "reduce_mid: outer %lld exceeds the grid limit", (long long)outer);
+  dim3 grid((unsigned)((inner + 63) / 64), (unsigned)outer);
+  hipLaunchKernelGGL(reduce_mid_kernel, grid, dim3(256), 0, (hipStream_t)stream, in, out, dti, dto,
+                     red, inner, kind);
+  return nbk_check_launch("reduce_mid_kernel");
+}

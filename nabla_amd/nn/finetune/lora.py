@@ -1,0 +1,41 @@
+"""LoRA helpers (nabla/nn/finetune/lora.py): init_lora_adapter 16-52,
+lora_delta 55-69 = ``(A @ B) * (alpha / rank)``, lora_linear 72-79 =
+``x @ W + x @ delta`` exactly as written there, merge / unmerge."""
+from __future__ import annotations
+
+from ...core.dtype import DType
+from ...core.tensor import Tensor
+from ...ops.creation import zeros
+from ..functional.init import normal
+
+
+def init_lora_adapter(weight: Tensor, rank: int, init_std: float = 0.01,
+                      dtype: DType | None = None) -> dict[str, Tensor]:
+    if len(weight.shape) != 2:
+        raise ValueError("init_lora_adapter expects a 2D weight tensor")
+    if rank <= 0:
+        raise ValueError("rank must be > 0")
+    in_features, out_features = int(weight.shape[0]), int(weight.shape[1])
+    adapter_dtype = dtype or weight.dtype
+    A = normal((in_features, rank), 0.0, init_std, dtype=adapter_dtype)
+    B = zeros((rank, out_features), dtype=adapter_dtype, device=weight.device)
+    return {"A": A, "B": B}
+
+
+def lora_delta(adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
+    A, B = adapter["A"], adapter["B"]
+    rank = int(A.shape[1])
+    return (A @ B) * (alpha / float(rank))
+
+
+def lora_linear(x: Tensor, frozen_weight: Tensor, adapter: dict[str, Tensor],
+                alpha: float = 1.0) -> Tensor:
+    return (x @ frozen_weight) + (x @ lora_delta(adapter, alpha=alpha))
+
+
+def merge_lora_weight(frozen_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
+    return frozen_weight + lora_delta(adapter, alpha=alpha)
+
+
+def unmerge_lora_weight(merged_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
+    return merged_weight - lora_delta(adapter, alpha=alpha)

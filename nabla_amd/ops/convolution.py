@@ -1,0 +1,178 @@
+"""2-D convolution, NHWC x HWIO (nabla/ops/convolution.py).
+
+``Conv2DOp`` mirrors 220-416.  Its VJP has the meaning of 309-392 -- input
+gradient = transposed convolution of the cotangent, cropped by the padding;
+filter gradient = correlation of the padded input with the cotangent; bias
+gradient = sum over N, H, W -- but emits the two dedicated gradient kernels
+instead of the conv2d_transpose + pad + slice and permute + conv2d + permute
+sequences.  Validation and its messages follow 602-696.
+"""
+from __future__ import annotations
+
+from typing import Any
+
+from ..backend import ir
+from ..core.tensor import Tensor
+from .base import Operation, ensure_tensor
+
+
+def _normalize_2tuple(value, name: str) -> tuple[int, int]:
+    if isinstance(value, int):
+        return (value, value)
+    if isinstance(value, (tuple, list)) and len(value) == 2:
+        return (int(value[0]), int(value[1]))
+    raise ValueError(f"{name} must be int or tuple/list of length 2, got {value}")
+
+
+def _normalize_4padding(padding) -> tuple[int, int, int, int]:
+    if isinstance(padding, int):
+        p = int(padding)
+        return (p, p, p, p)
+    if isinstance(padding, (tuple, list)):
+        if len(padding) == 2:
+            ph, pw = int(padding[0]), int(padding[1])
+            return (ph, ph, pw, pw)
+        if len(padding) == 4:
+            return tuple(int(v) for v in padding)
+    raise ValueError(
+        "padding must be int, (pad_h, pad_w), or (pad_top, pad_bottom, pad_left, pad_right)"
+    )
+
+
+def _require_all_positive_2tuple(value, name: str) -> None:
+    if value[0] <= 0 or value[1] <= 0:
+        raise ValueError(f"{name} values must be > 0, got {value}")
+
+
+def _require_all_nonnegative(value, name: str) -> None:
+    if any(v < 0 for v in value):
+        raise ValueError(f"{name} values must be >= 0, got {value}")
+
+
+def _out_hw(x_shape, w_shape, stride, padding) -> tuple[int, int]:
+    ho = ir.conv_out_size(x_shape[1], w_shape[0], stride[0], padding[0], padding[1])
+    wo = ir.conv_out_size(x_shape[2], w_shape[1], stride[1], padding[2], padding[3])
+    if ho <= 0 or wo <= 0:
+        raise ValueError(f"Non-positive conv2d output size H={ho}, W={wo}")
+    return ho, wo
+
+
+class Conv2DOp(Operation):
+    @property
+    def name(self) -> str:
+        return "conv2d"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x, w = args[0], args[1]
+        ho, wo = _out_hw(x.shape, w.shape, kwargs["stride"], kwargs["padding"])
+        return [(x.shape[0], ho, wo, w.shape[3])], [x.dtype], [x.device]
+
+    def kernel(self, args, kwargs):
+        x, w = args[0], args[1]
+        bias = args[2] if len(args) > 2 else None
+        return [ir.conv2d(x, w, bias, kwargs["stride"], kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        from .reduction import reduce_sum
+        x, w = primals[0], primals[1]
+        g = cotangents[0]
+        kw = {"stride": kwargs["stride"], "padding": kwargs["padding"]}
+        gx = _conv2d_dgrad_op([g, w], dict(kw, x_shape=tuple(x.shape)))[0]
+        gw = _conv2d_wgrad_op([x, g], dict(kw, w_shape=tuple(w.shape)))[0]
+        grads = [gx, gw]
+        if len(primals) > 2:
+            grads.append(reduce_sum(g, axis=[0, 1, 2]))
+        return grads
+
+
+class Conv2DInputGradOp(Operation):
+    """dX of conv2d: ``dy`` [N,Ho,Wo,Cout] and ``w`` [R,S,Cin,Cout] -> [N,H,W,Cin]."""
+
+    @property
+    def name(self) -> str:
+        return "conv2d_input_grad"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        return [tuple(kwargs["x_shape"])], [args[0].dtype], [args[0].device]
+
+    def kernel(self, args, kwargs):
+        return [ir.conv2d_dgrad(args[0], args[1], kwargs["x_shape"], kwargs["stride"],
+                                kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        # linear in both operands: d/d(dy) is a forward convolution, d/dw a filter gradient
+        dy, w = primals
+        g = cotangents[0]
+        kw = {"stride": kwargs["stride"], "padding": kwargs["padding"]}
+        g_dy = _conv2d_op([g, w], dict(kw))[0]
+        g_w = _conv2d_wgrad_op([g, dy], dict(kw, w_shape=tuple(w.shape)))[0]
+        return [g_dy, g_w]
+
+
+class Conv2DFilterGradOp(Operation):
+    """dW of conv2d: ``x`` [N,H,W,Cin] and ``dy`` [N,Ho,Wo,Cout] -> [R,S,Cin,Cout]."""
+
+    @property
+    def name(self) -> str:
+        return "conv2d_filter_grad"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        return [tuple(kwargs["w_shape"])], [args[0].dtype], [args[0].device]
+
+    def kernel(self, args, kwargs):
+        return [ir.conv2d_wgrad(args[0], args[1], kwargs["w_shape"], kwargs["stride"],
+                                kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        x, dy = primals
+        g = cotangents[0]  # [R,S,Cin,Cout]
+        kw = {"stride": kwargs["stride"], "padding": kwargs["padding"]}
+        g_x = _conv2d_dgrad_op([dy, g], dict(kw, x_shape=tuple(x.shape)))[0]
+        g_dy = _conv2d_op([x, g], dict(kw))[0]
+        return [g_x, g_dy]
+
+
+_conv2d_op = Conv2DOp()
+_conv2d_dgrad_op = Conv2DInputGradOp()
+_conv2d_wgrad_op = Conv2DFilterGradOp()
+
+
+def conv2d(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0, 0, 0), groups: int = 1,
+           bias=None, input_layout: Any = None, filter_layout: Any = None) -> Tensor:  # noqa: A002
+    x = ensure_tensor(x)
+    filter = ensure_tensor(filter)
+    bias_t = ensure_tensor(bias) if bias is not None else None
+    if len(x.shape) != 4 or len(filter.shape) != 4:
+        raise ValueError(
+            f"conv2d expects rank-4 tensors, got x={tuple(x.shape)}, filter={tuple(filter.shape)}"
+        )
+    if input_layout is not None or filter_layout is not None:
+        raise ValueError("conv2d currently supports only the default NHWC/RSCF layouts")
+    norm_stride = _normalize_2tuple(stride, "stride")
+    norm_dilation = _normalize_2tuple(dilation, "dilation")
+    norm_padding = _normalize_4padding(padding)
+    groups_i = int(groups)
+    _require_all_positive_2tuple(norm_stride, "stride")
+    _require_all_positive_2tuple(norm_dilation, "dilation")
+    _require_all_nonnegative(norm_padding, "padding")
+    if groups_i <= 0:
+        raise ValueError(f"groups must be > 0, got {groups_i}")
+    if norm_dilation != (1, 1):
+        raise ValueError("conv2d currently supports only dilation=(1, 1)")
+    if groups_i != 1:
+        raise ValueError("conv2d grouped mode is not exposed")
+    c_in, c_in_w, c_out = x.shape[-1], filter.shape[2], filter.shape[3]
+    if c_in != c_in_w * groups_i:
+        raise ValueError(
+            f"Input channels ({c_in}) must match filter channels*groups ({c_in_w * groups_i})"
+        )
+    if bias_t is not None:
+        if len(bias_t.shape) != 1:
+            raise ValueError(f"conv2d bias must be rank-1 [C_out], got shape={tuple(bias_t.shape)}")
+        if bias_t.shape[0] != c_out:
+            raise ValueError(
+                f"conv2d bias size ({bias_t.shape[0]}) must match filter C_out ({c_out})"
+            )
+    kwargs = {"stride": norm_stride, "padding": norm_padding}
+    args = [x, filter] if bias_t is None else [x, filter, bias_t]
+    return _conv2d_op(args, kwargs)[0]

@@ -1,0 +1,80 @@
+"""max_pool2d over NHWC (nabla/ops/pooling.py:53-137, 177-211).
+
+The reference unrolls pooling in Python -- one slice + reduce_max per output
+pixel, then stack -- which makes a 32x32 feature map cost hundreds of graph
+nodes.  Here it is one op with one kernel each way.  Semantics kept: windows
+are clipped at the padded border (111-130), and the gradient follows the
+reduce_max tie rule (reduction.py:219-230): every element equal to its
+window's maximum receives that window's full cotangent.
+"""
+from __future__ import annotations
+
+from ..backend import ir
+from ..core.tensor import Tensor
+from .base import Operation, ensure_tensor
+from .convolution import (_normalize_2tuple, _normalize_4padding, _require_all_nonnegative,
+                          _require_all_positive_2tuple)
+
+
+class MaxPool2DOp(Operation):
+    @property
+    def name(self) -> str:
+        return "max_pool2d"
+
+    @staticmethod
+    def _out_shape(x_shape, kernel, stride, padding):
+        n, h, w, c = x_shape
+        ho = (h + padding[0] + padding[1] - kernel[0]) // stride[0] + 1
+        wo = (w + padding[2] + padding[3] - kernel[1]) // stride[1] + 1
+        if ho <= 0 or wo <= 0:
+            raise ValueError(
+                f"Non-positive pool2d output size H={ho}, W={wo}. Input={(h, w)}, "
+                f"kernel={tuple(kernel)}, stride={tuple(stride)}, padding={tuple(padding)}."
+            )
+        return (n, ho, wo, c)
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x = args[0]
+        return ([self._out_shape(x.shape, kwargs["kernel_size"], kwargs["stride"], kwargs["padding"])],
+                [x.dtype], [x.device])
+
+    def kernel(self, args, kwargs):
+        return [ir.maxpool2d(args[0], kwargs["kernel_size"], kwargs["stride"], kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        return [_max_pool2d_grad_op([primals[0], outputs[0], cotangents[0]], dict(kwargs))[0]]
+
+
+class MaxPool2DGradOp(Operation):
+    @property
+    def name(self) -> str:
+        return "max_pool2d_grad"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x = args[0]
+        return [tuple(x.shape)], [x.dtype], [x.device]
+
+    def kernel(self, args, kwargs):
+        x, y, dy = args
+        return [ir.maxpool2d_bwd(x, y, dy, kwargs["kernel_size"], kwargs["stride"],
+                                 kwargs["padding"])]
+
+
+_max_pool2d_op = MaxPool2DOp()
+_max_pool2d_grad_op = MaxPool2DGradOp()
+
+
+def max_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Tensor:
+    x = ensure_tensor(x)
+    if len(x.shape) != 4:
+        raise ValueError(f"max_pool2d expects an NHWC rank-4 tensor, got shape {tuple(x.shape)}")
+    kernel = _normalize_2tuple(kernel_size, "kernel_size")
+    stride_n = _normalize_2tuple(stride if stride is not None else kernel, "stride")
+    padding_n = _normalize_4padding(padding)
+    dil = _normalize_2tuple(dilation, "dilation")
+    _require_all_positive_2tuple(kernel, "kernel_size")
+    _require_all_positive_2tuple(stride_n, "stride")
+    _require_all_nonnegative(padding_n, "padding")
+    if dil != (1, 1):
+        raise ValueError("pool2d currently supports only dilation=(1, 1)")
+    return _max_pool2d_op([x], {"kernel_size": kernel, "stride": stride_n, "padding": padding_n})[0]

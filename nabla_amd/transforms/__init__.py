@@ -1,0 +1,3 @@
+from .compile import CompilationStats, CompiledFunction, compile
+from .grad import grad, value_and_grad
+from .vjp import vjp

@@ -1,0 +1,338 @@
+"""TEST INFRASTRUCTURE -- not part of the product.
+
+A numpy/torch-CPU interpreter of the launch records that the lowering pass
+produces (row programs, strided copies, GEMM / conv / pool / gather records).
+It exists so that the host-side logic -- tracing, autodiff replay, fusion,
+view folding, register allocation, buffer planning -- can be checked on a
+machine without a GPU, and so that the HIP interpreter can be compared with a
+second implementation of the same instruction set.  Only tests may install it
+(``nabla_amd.backend.executor.set_executor``); the package itself never does.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+from scipy import special as _sp
+
+from nabla_amd.backend import isa
+from nabla_amd.backend.planner import Plan, ViewRef
+from nabla_amd.core.dtype import DType
+
+_F32 = np.float32
+
+
+def _round_bf16(a: np.ndarray) -> np.ndarray:
+    t = torch.from_numpy(np.ascontiguousarray(a.astype(np.float32)))
+    return t.to(torch.bfloat16).to(torch.float32).numpy()
+
+
+_UNARY = {
+    "mov": lambda a: a,
+    "neg": lambda a: -a,
+    "relu": lambda a: np.maximum(a, _F32(0)),
+    "exp": lambda a: np.exp(a),
+    "log": lambda a: np.log(a),
+    "sqrt": lambda a: np.sqrt(a),
+    "rsqrt": lambda a: (_F32(1) / np.sqrt(a)).astype(_F32),
+    "erf": lambda a: _sp.erf(a.astype(np.float64)).astype(_F32),
+    "gelu": lambda a: (0.5 * a.astype(np.float64) * (1.0 + _sp.erf(a.astype(np.float64) / np.sqrt(2.0)))).astype(_F32),
+    "tanh": lambda a: np.tanh(a),
+    "sigmoid": lambda a: (_F32(1) / (_F32(1) + np.exp(-a))).astype(_F32),
+    "abs": lambda a: np.abs(a),
+    "rbf16": _round_bf16,
+    "not": lambda a: (a == 0).astype(_F32),
+    "trunc": lambda a: np.trunc(a),
+    "nez": lambda a: (a != 0).astype(_F32),
+}
+_BINARY = {
+    "add": lambda a, b: a + b,
+    "sub": lambda a, b: a - b,
+    "mul": lambda a, b: a * b,
+    "div": lambda a, b: a / b,
+    "max": lambda a, b: np.maximum(a, b),
+    "min": lambda a, b: np.minimum(a, b),
+    "gt": lambda a, b: (a > b).astype(_F32),
+    "ge": lambda a, b: (a >= b).astype(_F32),
+    "eq": lambda a, b: (a == b).astype(_F32),
+    "ne": lambda a, b: (a != b).astype(_F32),
+    "lt": lambda a, b: (a < b).astype(_F32),
+    "le": lambda a, b: (a <= b).astype(_F32),
+    "pow": lambda a, b: np.power(a, b),
+    "and": lambda a, b: ((a != 0) & (b != 0)).astype(_F32),
+    "or": lambda a, b: ((a != 0) | (b != 0)).astype(_F32),
+}
+
+
+def _as_f32(t: torch.Tensor) -> np.ndarray:
+    if t.dtype == torch.bfloat16 or t.dtype == torch.float16:
+        return t.float().numpy()
+    if t.dtype == torch.bool:
+        return t.numpy().astype(_F32)
+    return t.numpy().astype(_F32)
+
+
+def _store(flat: torch.Tensor, idx: np.ndarray, vals: np.ndarray) -> None:
+    """flat[idx] = vals with the destination's rounding."""
+    v = torch.from_numpy(np.ascontiguousarray(vals.astype(_F32)))
+    if flat.dtype == torch.bool:
+        v = v != 0
+    elif flat.dtype in (torch.int32, torch.int64):
+        v = v.to(flat.dtype)  # truncation, as the kernel's float->int conversion
+    else:
+        v = v.to(flat.dtype)
+    flat[torch.from_numpy(idx.reshape(-1))] = v.reshape(-1)
+
+
+def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
+    lead, C = a["lead"], a["C"]
+    R = int(np.prod(lead)) if lead else 1
+    ops = a["operands"]
+    imm = a["imm"]
+    # per-row leading indices
+    lead_idx = np.stack(np.unravel_index(np.arange(R), lead), axis=0) if lead else np.zeros((0, R), np.int64)
+
+    def row_off(o):
+        off = np.full(R, o.offset, dtype=np.int64)
+        for k, s in enumerate(o.lead_strides):
+            off = off + lead_idx[k].astype(np.int64) * s
+        return off
+
+    cols = np.arange(C, dtype=np.int64)
+    V = {}
+    S = {}
+    ACC = {}
+    ins = a["ins"]
+
+    def rd(r):
+        if r < isa.NVEC:
+            return V[r]
+        return S[r][:, None]
+
+    def rs(r):
+        return S[r]
+
+    pc = 0
+    while pc < len(ins):
+        op, dst, x, y, z, aux = ins[pc]
+        if op == isa.HALT:
+            break
+        if op == isa.BODY:
+            for q in range(pc + 1, pc + 1 + aux):
+                bop, bd, bx, by, bz, _ = ins[q]
+                if bop == isa.LDG:
+                    o = ops[bx]
+                    idx = row_off(o)[:, None] + cols[None, :] * o.col_stride
+                    V[bd] = _as_f32(mem[o.buf][torch.from_numpy(idx.reshape(-1))]).reshape(R, C)
+                elif bop == isa.STG:
+                    o = ops[bd]
+                    idx = row_off(o)[:, None] + cols[None, :] * o.col_stride
+                    _store(mem[o.buf], idx, np.broadcast_to(rd(bx), (R, C)))
+                elif bop == isa.ACC:
+                    v = np.broadcast_to(rd(bx), (R, C)).astype(_F32)
+                    red = {0: np.sum, 1: np.max, 2: np.min}[by]
+                    part = red(v, axis=1).astype(_F32)
+                    ACC[bd] = {0: np.add, 1: np.maximum, 2: np.minimum}[by](ACC[bd], part).astype(_F32)
+                elif bop == isa.COLIDX:
+                    V[bd] = np.broadcast_to(cols.astype(_F32)[None, :], (R, C)).copy()
+                elif bop in isa.EW_NAME:
+                    name = isa.EW_NAME[bop]
+                    with np.errstate(all="ignore"):
+                        if name in _UNARY:
+                            r = _UNARY[name](np.broadcast_to(rd(bx), (R, C)).astype(_F32))
+                        elif name in _BINARY:
+                            r = _BINARY[name](rd(bx).astype(_F32), rd(by).astype(_F32))
+                        elif name == "where":
+                            r = np.where(rd(bx) != 0, rd(by), rd(bz))
+                        else:  # fma
+                            r = (rd(bx).astype(np.float64) * rd(by) + rd(bz))
+                    V[bd] = np.broadcast_to(np.asarray(r, dtype=_F32), (R, C)).copy()
+                else:
+                    raise AssertionError(f"opcode {bop} in a body")
+            pc += 1 + aux
+            continue
+        if op == isa.IMM:
+            S[dst] = np.full(R, imm[x], dtype=_F32)
+        elif op == isa.LDR:
+            o = ops[x]
+            S[dst] = _as_f32(mem[o.buf][torch.from_numpy(row_off(o))])
+        elif op == isa.STR:
+            o = ops[dst]
+            _store(mem[o.buf], row_off(o), rs(x))
+        elif op == isa.LEADIDX:
+            S[dst] = lead_idx[x].astype(_F32)
+        elif op == isa.ACCINIT:
+            ACC[dst] = np.full(R, {0: 0.0, 1: -np.inf, 2: np.inf}[x], dtype=_F32)
+        elif op == isa.RED:
+            S[dst] = ACC[x].astype(_F32)
+        elif op in isa.EW_NAME:
+            name = isa.EW_NAME[op]
+            with np.errstate(all="ignore"):
+                if name in _UNARY:
+                    S[dst] = np.asarray(_UNARY[name](rs(x)), dtype=_F32)
+                elif name in _BINARY:
+                    S[dst] = np.asarray(_BINARY[name](rs(x), rs(y)), dtype=_F32)
+                elif name == "where":
+                    S[dst] = np.where(rs(x) != 0, rs(y), rs(z)).astype(_F32)
+                else:
+                    S[dst] = (rs(x).astype(np.float64) * rs(y) + rs(z)).astype(_F32)
+        else:
+            raise AssertionError(f"opcode {op} in a prologue")
+        pc += 1
+
+
+def _view(mem, ref: ViewRef) -> torch.Tensor:
+    return torch.as_strided(mem[ref.buf], ref.shape, ref.strides, ref.offset)
+
+
+def _gemm(a, mem):
+    def mat(ref, bs, rs, cs, rows, cols):
+        base = mem[ref.buf]
+        return torch.as_strided(base, (a["batch"], rows, cols), (bs, rs, cs), ref.offset).float()
+    A = mat(a["a"], a["a_bs"], a["a_rs"], a["a_cs"], a["M"], a["K"])
+    B = mat(a["b"], a["b_bs"], a["b_rs"], a["b_cs"], a["K"], a["N"])
+    C = torch.matmul(A.double(), B.double()).float() * a.get("alpha", 1.0)
+    dst = a["dst"]
+    out = torch.as_strided(mem[dst.buf], (a["batch"], a["M"], a["N"]), (a["c_bs"], a["ldc"], 1), dst.offset)
+    out.copy_(C.to(out.dtype))
+
+
+def _conv(kind, a, mem):
+    import torch.nn.functional as F
+    pt, pb, pl, pr = a["padding"]
+    sh, sw = a["stride"]
+    ins = [_view(mem, r).float() for r in a["ins"]]
+    dst = _view(mem, a["dst"])
+    if kind == "conv2d":
+        x, w = ins[0], ins[1]
+        xp = F.pad(x.permute(0, 3, 1, 2), (pl, pr, pt, pb))
+        y = F.conv2d(xp.double(), w.permute(3, 2, 0, 1).double(), stride=(sh, sw)).float()
+        y = y.permute(0, 2, 3, 1)
+        if a["has_bias"]:
+            y = y + ins[2]
+        dst.copy_(y.to(dst.dtype))
+        return
+    xs, ws = a["x_shape"], a["w_shape"]
+    x = (ins[0] if kind == "conv2d_wgrad" else torch.zeros(xs)).double().requires_grad_(True)
+    w = (ins[1] if kind == "conv2d_dgrad" else torch.zeros(ws)).double().requires_grad_(True)
+    dy = (ins[0] if kind == "conv2d_dgrad" else ins[1]).double()
+    xp = F.pad(x.permute(0, 3, 1, 2), (pl, pr, pt, pb))
+    y = F.conv2d(xp, w.permute(3, 2, 0, 1), stride=(sh, sw)).permute(0, 2, 3, 1)
+    (g,) = torch.autograd.grad(y, x if kind == "conv2d_dgrad" else w, dy)
+    dst.copy_(g.float().to(dst.dtype))
+
+
+def _pool(kind, a, mem):
+    kh, kw = a["kernel"]
+    sh, sw = a["stride"]
+    pt, _, pl, _ = a["padding"]
+    x = _view(mem, a["ins"][0]).float().numpy()
+    N, H, W, C = x.shape
+    _, Ho, Wo, _ = a["y_shape"]
+    dst = _view(mem, a["dst"])
+    if kind == "maxpool2d":
+        y = np.full((N, Ho, Wo, C), -np.inf, dtype=_F32)
+        for i in range(Ho):
+            for j in range(Wo):
+                h0, h1 = max(0, i * sh - pt), min(H, i * sh - pt + kh)
+                w0, w1 = max(0, j * sw - pl), min(W, j * sw - pl + kw)
+                if h0 < h1 and w0 < w1:
+                    y[:, i, j, :] = x[:, h0:h1, w0:w1, :].max(axis=(1, 2))
+        dst.copy_(torch.from_numpy(y).to(dst.dtype))
+        return
+    y = _view(mem, a["ins"][1]).float().numpy()
+    dy = _view(mem, a["ins"][2]).float().numpy()
+    dx = np.zeros_like(x)
+    for i in range(Ho):
+        for j in range(Wo):
+            h0, h1 = max(0, i * sh - pt), min(H, i * sh - pt + kh)
+            w0, w1 = max(0, j * sw - pl), min(W, j * sw - pl + kw)
+            if h0 < h1 and w0 < w1:
+                win = x[:, h0:h1, w0:w1, :]
+                mask = (win == y[:, i:i + 1, j:j + 1, :]).astype(_F32)
+                dx[:, h0:h1, w0:w1, :] += mask * dy[:, i:i + 1, j:j + 1, :]
+    dst.copy_(torch.from_numpy(dx).to(dst.dtype))
+
+
+class EmulatedPlan:
+    def __init__(self, plan: Plan):
+        self.plan = plan
+
+    def run(self, inputs):
+        plan = self.plan
+        mem: list = [None] * len(plan.bufs)
+        outs = [None] * len(plan.outputs)
+        for b in plan.bufs:
+            if b.role == "input":
+                mem[b.id] = inputs[b.index].contiguous().reshape(-1)
+            else:
+                # poison temporaries so that reads of unwritten memory show up
+                t = torch.empty(max(b.numel, 1), dtype=b.dtype.to_torch())
+                if t.dtype.is_floating_point:
+                    t.fill_(float("nan"))
+                else:
+                    t.zero_()
+                mem[b.id] = t
+        for st in plan.steps:
+            a, k = st.attrs, st.kind
+            if k == "rowprog":
+                run_rowprog(a, mem)
+            elif k == "copy":
+                src = _view(mem, a["src"])
+                dst = _view(mem, a["dst"])
+                dst.copy_(src.to(dst.dtype))
+            elif k == "fill":
+                v = a["value"]
+                t = mem[a["buf"]]
+                t.fill_(bool(v) if t.dtype == torch.bool else (int(v) if not t.dtype.is_floating_point else v))
+            elif k == "reduce_mid":
+                src = mem[a["src"].buf][a["src"].offset:a["src"].offset + a["outer"] * a["red"] * a["inner"]]
+                x = _as_f32(src).reshape(a["outer"], a["red"], a["inner"])
+                r = {"sum": x.sum(axis=1, dtype=np.float64), "max": x.max(axis=1), "min": x.min(axis=1)}[a["fn"]]
+                d = a["dst"]
+                _store(mem[d.buf], d.offset + np.arange(a["outer"] * a["inner"]), np.asarray(r, dtype=_F32))
+            elif k == "gemm":
+                _gemm(a, mem)
+            elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
+                _conv(k, a, mem)
+            elif k in ("maxpool2d", "maxpool2d_bwd"):
+                _pool(k, a, mem)
+            elif k == "gather":
+                t = _view(mem, a["table"]).reshape(a["outer"], a["axis_len"], a["inner"])
+                ix = _view(mem, a["idx"]).reshape(-1).long()
+                if bool(((ix < -a["axis_len"]) | (ix >= a["axis_len"])).any()):
+                    raise IndexError("gather: index out of range")
+                ix = torch.where(ix < 0, ix + a["axis_len"], ix)
+                _view(mem, a["dst"]).copy_(t.index_select(1, ix).reshape(a["dst"].shape))
+            elif k == "argreduce":
+                x = _as_f32(_view(mem, a["src"])).reshape(a["rows"], a["C"])
+                r = np.argmin(x, axis=1) if a["fn"] == "min" else np.argmax(x, axis=1)
+                _view(mem, a["dst"]).copy_(torch.from_numpy(r.astype(np.int64)).reshape(a["dst"].shape))
+            else:
+                raise NotImplementedError(f"emulator: step kind '{k}'")
+        by_buf = {}
+        for oi, (bid, shape, dtype) in enumerate(plan.outputs):
+            if bid not in by_buf:
+                by_buf[bid] = mem[bid].reshape(shape)
+            outs[oi] = by_buf[bid]
+        return outs
+
+
+class EmulatorExecutor:
+    """Drop-in for the HIP executor in CPU tests of the host logic."""
+
+    name = "emulator"
+
+    def __init__(self):
+        self.torch_device = torch.device("cpu")
+
+    def bind(self, plan: Plan) -> EmulatedPlan:
+        return EmulatedPlan(plan)
+
+    def current_stream(self) -> int:
+        return 0
+
+    def synchronize(self) -> None:
+        pass
+
+    def check_status(self) -> None:
+        pass
