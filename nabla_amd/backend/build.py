@@ -64,5 +64,25 @@ def build(force: bool = True, jobs: int = 8, verbose: bool = False) -> Path:
     return LIB
 
 
+def build_examples(force: bool = True) -> list[Path]:
+    """Compile the example custom-kernel libraries under tests/custom_kernels:
+    every ``<name>.hip`` becomes ``lib<name>.so`` next to it."""
+    out = []
+    for src in sorted((ROOT / "tests" / "custom_kernels").glob("*.hip")):
+        lib = src.parent / f"lib{src.stem}.so"
+        if not force and lib.exists() and lib.stat().st_mtime > src.stat().st_mtime:
+            out.append(lib)
+            continue
+        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               f"-I{INCLUDE}", str(src), "-o", str(lib)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src.name}:\n{res.stderr[-4000:]}")
+        out.append(lib)
+    return out
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv, verbose=True)
+    build_examples(force=True)

@@ -383,13 +383,36 @@ class GatherOp(AxisOp):
         return [ir.gather(x, idx, self._norm_axis(kwargs.get("axis", 0), x.rank))]
 
     def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        # the reference scatters the cotangent into zeros (indexing.py:173-182); the
+        # node stays lazy and is dropped as dead code unless the table gradient is
+        # actually requested
+        from .creation import zeros_like
+        x, idx = primals
+        return [_scatter_op([zeros_like(x), idx, cotangents[0]], dict(kwargs))[0], None]
+
+
+class ScatterOp(AxisOp):
+    """``x`` with the rows selected by ``indices`` along ``axis`` replaced by
+    ``updates`` (indexing.py:185-447).  Recorded so that gather stays
+    differentiable in the trace; it has no kernel in this backend."""
+
+    @property
+    def name(self) -> str:
+        return "scatter"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x = args[0]
+        return [tuple(x.shape)], [x.dtype], [x.device]
+
+    def kernel(self, args, kwargs):
         raise NotImplementedError(
-            "gather: the gradient w.r.t. the table needs scatter, which is outside the "
-            "op set of this backend; treat the table as a constant"
+            "scatter (the gradient of gather w.r.t. its table) is outside the op set of "
+            "this backend; treat the table as a constant"
         )
 
 
 _gather_op = GatherOp()
+_scatter_op = ScatterOp()
 
 
 def gather(x: Tensor, indices: Tensor | None = None, axis: int = 0) -> Tensor:

@@ -1,0 +1,175 @@
+"""First GPU bring-up checks: every kernel family against torch-CPU fp64."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def T(a, dtype=None):
+    import nabla_amd as nb
+    return nb.Tensor.constant(a, dtype=dtype)
+
+
+def test_elementwise_chain(hip):
+    import nabla_amd as nb
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((37, 130)).astype(np.float32)
+    y = rng.standard_normal((37, 130)).astype(np.float32)
+    z = nb.relu(T(x) * T(y) + 1.0) - nb.exp(T(x) * 0.1)
+    ref = np.maximum(x * y + 1, 0) - np.exp(x * np.float32(0.1))
+    np.testing.assert_allclose(z.numpy(), ref, rtol=1e-6, atol=1e-6)
+
+
+def test_row_reduce_and_grad(hip):
+    import nabla_amd as nb
+    rng = np.random.default_rng(1)
+    for shape in [(8, 16), (33, 1000), (5, 4096 + 12)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        y = rng.standard_normal(shape).astype(np.float32)
+
+        def f(X, Y):
+            p = X * Y
+            m = nb.reduce_max(p, axis=1, keepdims=True)
+            return nb.reduce_sum(nb.exp(p - m) * nb.relu(X), axis=1)
+
+        X, Y = T(x), T(y)
+        out = f(X, Y)
+        g = nb.grad(lambda X, Y: nb.reduce_sum(f(X, Y)), realize=True, create_graph=False)(X, Y)
+        xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+        yt = torch.tensor(y, dtype=torch.float64)
+        pt = xt * yt
+        ot = (torch.exp(pt - pt.max(1, keepdim=True).values) * torch.relu(xt)).sum(1)
+        ot.sum().backward()
+        np.testing.assert_allclose(out.numpy(), ot.detach().numpy(), rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(g.numpy(), xt.grad.numpy(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (200, 136, 72), (512, 384, 256), (64, 10, 256),
+                                   (1024, 1024, 512)])
+def test_gemm(hip, dtype, layout, shape):
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(2)
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    A = torch.tensor(rng.standard_normal((M, K)), dtype=tdt)
+    B = torch.tensor(rng.standard_normal((K, N)), dtype=tdt)
+    ref = (A.double() @ B.double()).numpy()
+    a_dev = (A if layout[0] == "n" else A.t().contiguous()).cuda()
+    b_dev = (B if layout[1] == "n" else B.t().contiguous()).cuda()
+    c_dev = torch.empty((M, N), dtype=tdt, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs = (K, 1) if layout[0] == "n" else (1, M)
+    d.b_rs, d.b_cs = (N, 1) if layout[1] == "n" else (1, K)
+    d.ldc = N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
+    d.dtype_ab = d.dtype_c = 0 if dtype == "f32" else 1
+    d.alpha = 1.0
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    tol = 1e-5 if dtype == "f32" else 1e-2
+    scale = np.sqrt(K)
+    assert np.abs(got - ref).max() <= tol * scale, np.abs(got - ref).max()
+
+
+def test_mlp_grads(hip):
+    import nabla_amd as nb
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-0.05, 0.05, (128, 784)).astype(np.float32)
+    W1 = rng.uniform(-0.05, 0.05, (784, 256)).astype(np.float32)
+    W2 = rng.uniform(-0.05, 0.05, (256, 10)).astype(np.float32)
+    b1 = np.zeros((1, 256), np.float32)
+    b2 = np.zeros((1, 10), np.float32)
+
+    def loss_fn(W1, b1, W2, b2, x):
+        return nb.mean(nb.relu(x @ W1 + b1) @ W2 + b2)
+
+    args = [T(a) for a in (W1, b1, W2, b2, x)]
+    loss, grads = nb.value_and_grad(loss_fn, argnums=(0, 1, 2, 3))(*args)
+    nb.realize_all(loss, *grads)
+    ta = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (W1, b1, W2, b2)]
+    tl = (torch.relu(torch.tensor(x, dtype=torch.float64) @ ta[0] + ta[1]) @ ta[2] + ta[3]).mean()
+    tl.backward()
+    assert abs(loss.item() - tl.item()) <= 1e-5 * abs(tl.item()) + 1e-9
+    for g, t in zip(grads, ta):
+        ref = t.grad.numpy()
+        assert np.abs(g.numpy() - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-9
+
+
+def test_layernorm_softmax_grads(hip):
+    import nabla_amd as nb
+    F = nb.nn.functional
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((4, 6, 256)).astype(np.float32)
+    w = rng.standard_normal((256,)).astype(np.float32)
+    b = rng.standard_normal((256,)).astype(np.float32)
+
+    def loss_fn(x, w, b):
+        y = F.layer_norm(x, w, b)
+        return nb.mean(nb.softmax(y, axis=-1) * y)
+
+    l, gs = nb.value_and_grad(loss_fn, argnums=(0, 1, 2))(T(x), T(w), T(b))
+    nb.realize_all(l, *gs)
+    tx, tw, tb = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (x, w, b)]
+    ty = torch.nn.functional.layer_norm(tx, (256,), tw, tb)
+    tl = (torch.softmax(ty, -1) * ty).mean()
+    tl.backward()
+    assert abs(l.item() - tl.item()) < 1e-5
+    for g, t in zip(gs, (tx, tw, tb)):
+        ref = t.grad.numpy()
+        assert np.abs(g.numpy() - ref).max() <= 2e-5 * np.abs(ref).max() + 1e-8
+
+
+def test_conv_pool_grads(hip):
+    import nabla_amd as nb
+    rng = np.random.default_rng(4)
+    x = rng.uniform(0, 1, (4, 12, 12, 3)).astype(np.float32)
+    w1 = (rng.standard_normal((3, 3, 3, 8)) * 0.3).astype(np.float32)
+    b1 = (rng.standard_normal((8,)) * 0.1).astype(np.float32)
+    w2 = (rng.standard_normal((3, 3, 8, 16)) * 0.2).astype(np.float32)
+
+    def loss_fn(w1, b1, w2, x):
+        h = nb.relu(nb.conv2d(x, w1, stride=(1, 1), padding=1, bias=b1))
+        h = nb.max_pool2d(h, kernel_size=2)
+        h = nb.conv2d(h, w2, stride=(2, 1), padding=(1, 0, 2, 1))
+        return nb.mean(h * h)
+
+    l, gs = nb.value_and_grad(loss_fn, argnums=(0, 1, 2, 3))(T(w1), T(b1), T(w2), T(x))
+    nb.realize_all(l, *gs)
+    import torch.nn.functional as TF
+    tw1, tb1, tw2, tx = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (w1, b1, w2, x)]
+    h = TF.conv2d(tx.permute(0, 3, 1, 2), tw1.permute(3, 2, 0, 1), tb1, padding=1)
+    h = TF.max_pool2d(torch.relu(h), 2)
+    h = TF.conv2d(TF.pad(h, (2, 1, 1, 0)), tw2.permute(3, 2, 0, 1), stride=(2, 1))
+    tl = (h * h).mean()
+    tl.backward()
+    assert abs(l.item() - tl.item()) <= 1e-5 * abs(tl.item())
+    for g, t in zip(gs, (tw1, tb1, tw2, tx)):
+        ref = t.grad.numpy()
+        assert np.abs(g.numpy() - ref).max() <= 2e-5 * np.abs(ref).max() + 1e-8
+
+
+def test_gather_argmax_views(hip):
+    import nabla_amd as nb
+    rng = np.random.default_rng(5)
+    table = rng.standard_normal((50, 24)).astype(np.float32)
+    idx = rng.integers(0, 50, (3, 7)).astype(np.int64)
+    out = nb.gather(T(table), T(idx), axis=0)
+    assert np.array_equal(out.numpy(), table[idx])
+    logits = rng.standard_normal((9, 33)).astype(np.float32)
+    assert np.array_equal(nb.argmax(T(logits), axis=-1).numpy(), logits.argmax(-1))
+    x = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    y = nb.permute(T(x), (2, 0, 1)) * 2.0
+    np.testing.assert_array_equal(y.numpy(), x.transpose(2, 0, 1) * 2)
+    z = nb.pad(T(x), [(1, 0), (0, 2), (1, 1)], value=-1.0)
+    np.testing.assert_array_equal(z.numpy(), np.pad(x, [(1, 0), (0, 2), (1, 1)], constant_values=-1))
+    c = nb.concatenate([T(x), T(x) + 1.0], axis=1)
+    np.testing.assert_array_equal(c.numpy(), np.concatenate([x, x + 1], 1))
