@@ -1,0 +1,256 @@
+"""Benchmark of the hot path on one MI355X.
+
+Default workload: the elementwise + reduction stress configuration
+(x, y [8192, 8192] fp32; out = sum(exp(x*y - max(x*y)) * relu(x), axis=1) and
+the gradient of sum(out) w.r.t. x), one compiled step per iteration with the
+inputs already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+
+
+class KernelTimer:
+    """Brackets chosen plan steps with HIP events on the launch stream."""
+
+    def __init__(self, lib, kinds):
+        self.lib = lib
+        self.kinds = set(kinds)
+        self.pairs = []  # (step index, kind, start event, stop event)
+
+    def __call__(self, si, kind, stream):
+        if kind not in self.kinds:
+            return None
+        a, b = C.c_void_p(), C.c_void_p()
+        self.lib.nbk_event_create(C.byref(a))
+        self.lib.nbk_event_create(C.byref(b))
+        self.lib.nbk_event_record(a, stream)
+        self.pairs.append((si, kind, a, b))
+        return lambda: self.lib.nbk_event_record(b, stream)
+
+    def durations_ms(self):
+        out = {}
+        ms = C.c_float()
+        for si, kind, a, b in self.pairs:
+            self.lib.nbk_event_elapsed_ms(a, b, C.byref(ms))
+            out.setdefault((si, kind), []).append(ms.value)
+            self.lib.nbk_event_destroy(a)
+            self.lib.nbk_event_destroy(b)
+        self.pairs = []
+        return out
+
+
+def sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def compiled_plan(nb, fn, args):
+    """Trace + lower ``fn`` once; returns (bound plan, input buffers, call that
+    replays it).  The replay is what a cached ``@compile`` call executes."""
+    cf = nb.compile(fn)
+    out = cf(*args)
+    spec = next(iter(next(iter(cf._cache.values())).specializations.values()))
+    flat, _ = nb.tree_flatten((args, {}))
+
+    def bufs():
+        return [flat[v]._impl._buffer if kind == "arg" else v for kind, v in spec.input_plan]
+
+    return cf, spec, bufs, out
+
+
+# ------------------------------------------------------------------ workloads
+def workload_c2(nb, oc, rows=8192, cols=8192):
+    inp = oc.c2_inputs(rows, cols, seed=0)
+    X, Y = nb.Tensor.constant(inp["x"]), nb.Tensor.constant(inp["y"])
+
+    def step(X, Y):
+        return oc.c2_program(nb, X, Y)
+
+    algo_bytes = 3 * rows * cols * 4 + 2 * rows * 4
+    return dict(name=f"c2 elementwise+reduction fwd+grad, x,y[{rows},{cols}] fp32", fn=step,
+                args=(X, Y), dtype="f32", bound="hbm", algo=algo_bytes, dominant="rowprog",
+                cpu=lambda: cpu_c2(oc, rows, cols))
+
+
+def cpu_c2(oc, rows, cols):
+    sample_rows = max(64, rows // 16)
+    inp = oc.c2_inputs(sample_rows, cols, seed=0)
+    t0 = time.perf_counter()
+    oc.c2_reference(inp["x"], inp["y"], dtype=np.float32)
+    dt = time.perf_counter() - t0
+    return dict(value=1.0 / (dt * rows / sample_rows), unit="steps/s", cores=1, kind="port",
+                sample=f"{sample_rows} of {rows} rows, numpy fp32 oracle, scaled by rows")
+
+
+def workload_c1(nb, oc):
+    inp = oc.c1_inputs()
+    t = {k: nb.Tensor.constant(v) for k, v in inp.items()}
+
+    def step(t):
+        return oc.c1_program(nb, t)
+
+    def cpu():
+        t0 = time.perf_counter()
+        n = 20
+        for _ in range(n):
+            oc.c1_reference(**inp, dtype=np.float32)
+        return dict(value=n / (time.perf_counter() - t0), unit="steps/s", cores=os.cpu_count(),
+                    kind="port", sample=f"{n} full steps, numpy fp32 oracle")
+
+    return dict(name="c1 2-layer MLP fwd+grad fp32, x[128,784]", fn=step, args=(t,), dtype="f32",
+                bound="mfma", algo=104.7e6, dominant="gemm", cpu=cpu)
+
+
+def workload_c3(nb, oc, batch=8, seq=1024, d=1024, ff=4096):
+    inp = oc.c3_inputs(batch, seq, d, ff, seed=0, bf16=True)
+    t = oc.upload(nb, inp, dtype=nb.DType.bfloat16)
+
+    def step(t):
+        return oc.c3_program(nb, t, num_heads=16)
+
+    T = batch * seq
+    hd = d // 16
+    qkvo = 4 * 2 * T * d * d
+    mlp = 2 * 2 * T * d * ff
+    attn_causal = 2 * 2 * batch * 16 * seq * seq * hd / 2
+    flops = 3 * (qkvo + mlp + attn_causal)
+
+    def cpu():
+        small = oc.c3_inputs(1, 128, d, ff, seed=0, bf16=True)
+        t0 = time.perf_counter()
+        oc.c3_reference(small, num_heads=16, dtype=np.float32)
+        dt = time.perf_counter() - t0
+        scale = T / 128.0
+        return dict(value=1.0 / (dt * scale), unit="steps/s", cores=os.cpu_count(), kind="port",
+                    sample="1 x 128 tokens of 8 x 1024, numpy fp32 oracle, scaled by tokens "
+                           "(attention cost per token is under-counted)")
+
+    return dict(name=f"c3 pre-LN transformer block fwd+bwd bf16, B{batch} S{seq} D{d} FF{ff}",
+                fn=step, args=(t,), dtype="bf16", bound="mfma", algo=flops, dominant="gemm", cpu=cpu)
+
+
+def workload_c4(nb, oc):
+    inp = oc.c4_inputs()
+    t = oc.upload(nb, inp)
+
+    def step(t):
+        return oc.c4_program(nb, t)
+
+    def cpu():
+        small = oc.c4_inputs(batch=4)
+        t0 = time.perf_counter()
+        oc.c4_reference(small, dtype=np.float32)
+        dt = time.perf_counter() - t0
+        return dict(value=1.0 / (dt * 16), unit="steps/s", cores=os.cpu_count(), kind="port",
+                    sample="4 of 64 images, numpy fp32 oracle, scaled by batch")
+
+    return dict(name="c4 CNN step fp32, img[64,32,32,3]", fn=step, args=(t,), dtype="f32",
+                bound="mfma", algo=58.4e9, dominant="conv", cpu=cpu)
+
+
+def workload_c5(nb, oc, layers=12):
+    inp = oc.c5_inputs(layers=layers, seed=0, b_zero=True, bf16=True)
+    t = oc.upload(nb, inp, dtype=nb.DType.bfloat16)
+
+    def step(t):
+        return oc.c5_program(nb, t, num_heads=16)
+
+    def cpu():
+        return dict(value=None, unit="steps/s", cores=os.cpu_count(), kind="port",
+                    sample="not run: one step is ~27 TFLOP on the host")
+
+    return dict(name=f"c5 LoRA step bf16, {layers} layers D2048 S2048 B4", fn=step, args=(t,),
+                dtype="bf16", bound="mfma", algo=24.5e12 * layers / 12, dominant="gemm", cpu=cpu)
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4,
+             "c5": workload_c5}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import nabla_amd as nb
+    from nabla_amd.backend import lib as nbk_lib
+    from nabla_amd.backend.executor import get_executor
+    from oracle import configs as oc
+
+    ex = get_executor()  # raises without libnbk.so or without a gfx950 GPU
+    L = nbk_lib.load()
+    w = WORKLOADS[a.workload](nb, oc)
+    cf, spec, bufs, first = compiled_plan(nb, w["fn"], w["args"])
+    plan = spec.bound.plan
+    inputs = bufs()
+
+    for _ in range(a.warmup):
+        spec.bound.run(inputs)
+    sync()
+    dominant_kinds = {"rowprog": ["rowprog"], "gemm": ["gemm"],
+                      "conv": ["conv2d", "conv2d_dgrad", "conv2d_wgrad"]}[w["dominant"]]
+    timer = KernelTimer(L, dominant_kinds)
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        spec.bound.run(inputs, timer=timer)
+    sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / a.steps * 1e3
+    dur = timer.durations_ms()
+    per_step_total = {}
+    for (si, kind), v in dur.items():
+        per_step_total[(si, kind)] = sum(v) / len(v)
+    dom_ms = sum(per_step_total.values())
+    # the single longest launch of the dominant kind
+    top = max(per_step_total.items(), key=lambda kv: kv[1]) if per_step_total else None
+
+    if w["bound"] == "hbm":
+        achieved = w["algo"] / (dom_ms * 1e-3) / 1e9 if dom_ms else 0.0
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = w["algo"] / (dom_ms * 1e-3) / 1e12 if dom_ms else 0.0
+        peak, unit = MFMA_PEAK_TFLOPS[w["dtype"]], "TFLOP/s"
+    roofline = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                "frac": round(achieved / peak, 4), "traffic": None,
+                "kernel": w["dominant"], "kernel_ms_per_step": round(dom_ms, 4),
+                "launches_per_step": len(per_step_total)}
+    cpu = None if a.no_cpu else w["cpu"]()
+    line = {
+        "metric": "train steps/sec fwd+bwd at 1 MI355X; GEMM % MFMA peak; fused-op % HBM BW",
+        "value": round(a.steps / wall, 3), "unit": "steps/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["name"], "step": "compiled replay of forward + gradients",
+                   "plan": plan.stats},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

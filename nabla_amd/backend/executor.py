@@ -217,7 +217,10 @@ class BoundPlan:
             else:
                 raise NotImplementedError(f"executor: unknown step kind '{k}'")
 
-    def run(self, inputs: Sequence[torch.Tensor]) -> list[torch.Tensor]:
+    def run(self, inputs: Sequence[torch.Tensor], timer=None) -> list[torch.Tensor]:
+        """Launch every step on the current stream.  ``timer(step_index, kind)``,
+        if given, is called before each launch and may return a callable to be
+        invoked right after it (used to bracket kernels with HIP events)."""
         plan = self.plan
         ex = self.ex
         if len(inputs) != plan.n_inputs:
@@ -243,7 +246,8 @@ class BoundPlan:
         stream = C.c_void_p(ex.current_stream())
         base = self.base
         check = lib.check
-        for fn, args, patches, _keep in self.calls:
+        for si, (fn, args, patches, _keep) in enumerate(self.calls):
+            after = timer(si, plan.steps[si].kind, stream) if timer is not None else None
             for obj, fieldname, buf, off in patches:
                 setattr(obj, fieldname, base[buf] + off)
             if len(args) >= 2 and isinstance(args[0], _Ptrs):
@@ -255,6 +259,8 @@ class BoundPlan:
             else:
                 call_args = args
             check(fn(*call_args, stream))
+            if after is not None:
+                after()
         del keep
         return outs
 

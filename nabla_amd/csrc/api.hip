@@ -15,6 +15,19 @@ void nbk_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+static int g_num_cus = 0;  // written once with the same value by whoever gets there first
+int nbk_num_cus(void) {
+  if (g_num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_num_cus = n;
+    else
+      g_num_cus = 256;
+  }
+  return g_num_cus;
+}
+
 extern "C" const char* nbk_last_error(void) { return g_err; }
 extern "C" int nbk_abi_version(void) { return NBK_ABI_VERSION; }
 

@@ -9,6 +9,8 @@
 
 // ---- error reporting (thread-local message, C ABI status codes) ----------
 void nbk_set_error(const char* fmt, ...);
+// Compute units of the current device (256 on MI355X); set by nbk_init, lazily otherwise.
+int nbk_num_cus(void);
 
 #define NBK_REQUIRE(cond, ...)            \
   do {                                    \

@@ -13,6 +13,7 @@
 // (one per chunk component) indexed with a wave-uniform index, which the
 // compiler turns into VGPR-relative moves instead of scratch memory.
 #include "nbk_common.h"
+#include <stddef.h>
 
 typedef float vf16 __attribute__((ext_vector_type(16)));
 typedef float vf4 __attribute__((ext_vector_type(4)));
@@ -176,20 +177,24 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
   }
 }
 
-// Offset of the current row inside one operand.
+__device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead);
+
+// Offset of the current row inside one operand.  Strides and indices beyond
+// n_lead are zero, so all four terms can be added unconditionally (constant
+// indices keep both arrays in registers).
 template <typename IDX>
 __device__ __forceinline__ int64_t rp_row_offset(const nbk_operand& o, const IDX* lead_idx,
                                                  int n_lead) {
-  int64_t off = 0;
-  for (int k = 0; k < n_lead; ++k) off += (int64_t)lead_idx[k] * o.lead_stride[k];
-  return off;
+  (void)n_lead;
+  return (int64_t)lead_idx[0] * o.lead_stride[0] + (int64_t)lead_idx[1] * o.lead_stride[1] +
+         (int64_t)lead_idx[2] * o.lead_stride[2] + (int64_t)lead_idx[3] * o.lead_stride[3];
 }
 
 // One body instruction on one chunk.
 template <typename IDX>
 __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins in, RpRegs& R,
                                              const IDX* lead_idx, int64_t col, int valid,
-                                             const float* stage, int64_t c_pad) {
+                                             const float* stage, int64_t c_pad, int n_lead) {
   const int op = in.op;
   if (op >= NBK_OP_ADD && op < NBK_OP_WHERE) {
     float4 a = rp_read(R, in.a), b = rp_read(R, in.b), r;
@@ -208,17 +213,17 @@ __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins
                            rp_unary(op, a.w));
     rp_write(R, in.dst, r);
   } else if (op == NBK_OP_LDG) {
-    const nbk_operand& o = P.operand[in.a];
+    const nbk_operand o = rp_operand(P, in.a, n_lead);
     float4 r;
     if (o.stage_slot >= 0 && stage != nullptr) {
       r = *(const float4*)(stage + o.stage_slot * c_pad + col);
     } else {
-      r = rp_load4(o, rp_row_offset(o, lead_idx, P.n_lead), col, valid);
+      r = rp_load4(o, rp_row_offset(o, lead_idx, n_lead), col, valid);
     }
     rp_write(R, in.dst, r);
   } else if (op == NBK_OP_STG) {
-    const nbk_operand& o = P.operand[in.dst];
-    rp_store4(o, rp_row_offset(o, lead_idx, P.n_lead), col, valid, rp_read(R, in.a));
+    const nbk_operand o = rp_operand(P, in.dst, n_lead);
+    rp_store4(o, rp_row_offset(o, lead_idx, n_lead), col, valid, rp_read(R, in.a));
   } else if (op == NBK_OP_ACC) {
     float4 a = rp_read(R, in.a);
     const int kind = in.b;
@@ -260,22 +265,24 @@ __device__ __forceinline__ float rp_block_reduce(float v, int kind, float* red_b
 // Prologue (per-row, scalar-register) instruction.  Returns through R.
 template <typename IDX>
 __device__ __forceinline__ void rp_exec_scalar(const nbk_rowprog& P, const nbk_ins in, RpRegs& R,
-                                               const IDX* lead_idx, bool writer, float* red_buf) {
+                                               const IDX* lead_idx, bool writer, float* red_buf,
+                                               int n_lead) {
   const int op = in.op;
   const int d = in.dst - NBK_RP_NVEC;
   if (op == NBK_OP_IMM) {
-    R.s[d] = P.imm[in.a];
+    R.s[d] = __uint_as_float(rp_sgpr(__float_as_uint(P.imm[in.a])));
   } else if (op == NBK_OP_LDR) {
-    const nbk_operand& o = P.operand[in.a];
-    R.s[d] = nbk_load_as_f32(o.ptr, rp_row_offset(o, lead_idx, P.n_lead), o.dtype);
+    const nbk_operand o = rp_operand(P, in.a, n_lead);
+    R.s[d] = nbk_load_as_f32(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype);
   } else if (op == NBK_OP_STR) {
+    const nbk_operand o = rp_operand(P, in.dst, n_lead);
     if (writer) {
-      const nbk_operand& o = P.operand[in.dst];
-      nbk_store_from_f32(o.ptr, rp_row_offset(o, lead_idx, P.n_lead), o.dtype,
+      nbk_store_from_f32(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype,
                          R.s[in.a - NBK_RP_NVEC]);
     }
   } else if (op == NBK_OP_LEADIDX) {
-    R.s[d] = (float)lead_idx[in.a];
+    const int k = in.a;
+    R.s[d] = (float)(k == 0 ? lead_idx[0] : k == 1 ? lead_idx[1] : k == 2 ? lead_idx[2] : lead_idx[3]);
   } else if (op == NBK_OP_ACCINIT) {
     R.acc[in.dst] = rp_identity(in.a);
   } else if (op == NBK_OP_RED) {
@@ -291,128 +298,212 @@ __device__ __forceinline__ void rp_exec_scalar(const nbk_rowprog& P, const nbk_i
   }
 }
 
+// ---------------------------------------------------------------- program staging
+// Kernel arguments live in uncached memory: a scalar load from them costs a full
+// memory round trip, far too slow for an instruction stream that is re-read for
+// every chunk.  Each workgroup therefore copies the program into LDS once and
+// then walks rows persistently; the interpreter fetches instructions and operand
+// descriptors from LDS and turns them into scalars with readfirstlane.
+#define RP_WORDS ((int)(sizeof(nbk_rowprog) / 4))
+static_assert(sizeof(nbk_rowprog) % 4 == 0, "program is copied word by word");
+static_assert(sizeof(nbk_operand) % 8 == 0 && offsetof(nbk_rowprog, operand) % 8 == 0 &&
+                  offsetof(nbk_operand, col_stride) % 8 == 0 && offsetof(nbk_operand, vec_ok) % 8 == 0,
+              "operand descriptors are read from LDS with 8-byte accesses");
+static_assert(sizeof(nbk_ins) == 8 && offsetof(nbk_rowprog, ins) % 8 == 0,
+              "instructions are read from LDS with 8-byte accesses");
+
+__device__ __forceinline__ void rp_copy_program(const nbk_rowprog& P, uint32_t* dst) {
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(&P);
+  for (int i = threadIdx.x; i < RP_WORDS; i += blockDim.x) dst[i] = src[i];
+  __syncthreads();
+}
+
+// readfirstlane returns a SIGNED int: widening it directly to 64 bits would
+// sign-extend and corrupt the high half of a pointer, so go through uint32_t.
+__device__ __forceinline__ uint32_t rp_sgpr(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane(v);
+}
+__device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
+  return (uint64_t)rp_sgpr(v.x) | ((uint64_t)rp_sgpr(v.y) << 32);
+}
+
+__device__ __forceinline__ nbk_ins rp_fetch(const nbk_rowprog& S, int q) {
+  const uint2 u = *reinterpret_cast<const uint2*>(&S.ins[q]);
+  const uint32_t lo = rp_sgpr(u.x);
+  const uint32_t hi = rp_sgpr(u.y);
+  nbk_ins in;
+  in.op = lo & 0xff; in.dst = (lo >> 8) & 0xff; in.a = (lo >> 16) & 0xff; in.b = lo >> 24;
+  in.c = hi & 0xff; in.pad = 0; in.aux = (uint16_t)(hi >> 16);
+  return in;
+}
+
+// Scalar copy of one operand descriptor out of LDS.
+__device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead) {
+  const nbk_operand& o = S.operand[i];
+  nbk_operand r;
+  r.ptr = reinterpret_cast<void*>(rp_sgpr64(*reinterpret_cast<const uint2*>(&o.ptr)));
+  // descriptors are 56 bytes apart, so only 8-byte alignment is guaranteed here
+  const uint2 t0 = *reinterpret_cast<const uint2*>(&o.col_stride);
+  const uint2 t1 = *reinterpret_cast<const uint2*>(&o.vec_ok);
+  r.col_stride = (int32_t)rp_sgpr(t0.x);
+  r.dtype = (int32_t)rp_sgpr(t0.y);
+  r.vec_ok = (int32_t)rp_sgpr(t1.x);
+  r.stage_slot = (int32_t)rp_sgpr(t1.y);
+  // the host zero-fills strides beyond n_lead
+  (void)n_lead;
+#pragma unroll
+  for (int k = 0; k < NBK_RP_MAX_LEAD; ++k) {
+    r.lead_stride[k] = (int64_t)rp_sgpr64(*reinterpret_cast<const uint2*>(&o.lead_stride[k]));
+  }
+  return r;
+}
+
 // ---------------------------------------------------------------- block mode
 extern __shared__ __align__(16) float rp_stage_lds[];
 
-__global__ __launch_bounds__(512) void rp_block_kernel(const nbk_rowprog P) {
+__global__ __launch_bounds__(512) void rp_block_kernel(const nbk_rowprog P, int64_t rows) {
   __shared__ float red_buf[16];
+  __shared__ __align__(16) uint32_t prog_lds[RP_WORDS];
+  rp_copy_program(P, prog_lds);
+  const nbk_rowprog& S = *reinterpret_cast<const nbk_rowprog*>(prog_lds);
   RpRegs R;
   R.acc = (vf4)(0.f);
   const int64_t C = P.C;
   const int64_t c_pad = (C + 3) & ~(int64_t)3;
   const int64_t n_chunks = c_pad >> 2;
   const int n_lead = P.n_lead;
-  const float* stage = P.n_stage > 0 ? rp_stage_lds : nullptr;
+  const int n_ins = P.n_ins;
+  const int n_operands = P.n_operands;
+  const int n_stage = P.n_stage;
+  int64_t lead_dim[NBK_RP_MAX_LEAD];
+#pragma unroll
+  for (int k = 0; k < NBK_RP_MAX_LEAD; ++k) lead_dim[k] = P.lead_dim[k];
+  const float* stage = n_stage > 0 ? rp_stage_lds : nullptr;
+  const bool writer = threadIdx.x == 0;
 
-  // decompose the row index over the leading dims (wave-uniform)
-  int64_t lead_idx[NBK_RP_MAX_LEAD];
-  {
-    int64_t rem = blockIdx.x;
-    for (int k = n_lead - 1; k > 0; --k) {
-      int64_t d = P.lead_dim[k];
-      int64_t q = rem / d;
-      lead_idx[k] = rem - q * d;
-      rem = q;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    // decompose the row index over the leading dims (wave-uniform)
+    // unused leading dims have extent 1, so the same three divisions serve every n_lead
+    int64_t lead_idx[NBK_RP_MAX_LEAD];
+    {
+      int64_t rem = row, q;
+      q = rem / lead_dim[3]; lead_idx[3] = rem - q * lead_dim[3]; rem = q;
+      q = rem / lead_dim[2]; lead_idx[2] = rem - q * lead_dim[2]; rem = q;
+      q = rem / lead_dim[1]; lead_idx[1] = rem - q * lead_dim[1]; rem = q;
+      lead_idx[0] = rem;
     }
-    if (n_lead > 0) lead_idx[0] = rem;
-  }
 
-  // pre-load staged operands: every lane stages exactly the chunks it will
-  // later read back, so no barrier is needed between the two.
-  if (P.n_stage > 0) {
-    for (int oi = 0; oi < P.n_operands; ++oi) {
-      const nbk_operand& o = P.operand[oi];
-      if (o.stage_slot < 0) continue;
-      const int64_t off = rp_row_offset(o, lead_idx, n_lead);
-      float* dst = rp_stage_lds + o.stage_slot * c_pad;
-      if (o.vec_ok && o.dtype == NBK_F32 && (C & 3) == 0) {
-        const float4* src = (const float4*)((const float*)o.ptr + off);
-        int64_t ch = threadIdx.x;
-        // four independent 16-byte loads in flight per lane
-        for (; ch + 3 * (int64_t)blockDim.x < n_chunks; ch += 4 * (int64_t)blockDim.x) {
-          float4 v0 = src[ch], v1 = src[ch + blockDim.x], v2 = src[ch + 2 * blockDim.x],
-                 v3 = src[ch + 3 * blockDim.x];
-          ((float4*)dst)[ch] = v0;
-          ((float4*)dst)[ch + blockDim.x] = v1;
-          ((float4*)dst)[ch + 2 * blockDim.x] = v2;
-          ((float4*)dst)[ch + 3 * blockDim.x] = v3;
+    // pre-load staged operands: every lane stages exactly the chunks it will
+    // later read back, so no barrier is needed between the two.
+    if (n_stage > 0) {
+      for (int oi = 0; oi < n_operands; ++oi) {
+        const nbk_operand o = rp_operand(S, oi, n_lead);
+        if (o.stage_slot < 0) continue;
+        const int64_t off = rp_row_offset(o, lead_idx, n_lead);
+        float* dst = rp_stage_lds + o.stage_slot * c_pad;
+        if (o.vec_ok && o.dtype == NBK_F32 && (C & 3) == 0) {
+          const float4* src = (const float4*)((const float*)o.ptr + off);
+          int64_t ch = threadIdx.x;
+          const int64_t bd = blockDim.x;
+          // four independent 16-byte loads in flight per lane
+          for (; ch + 3 * bd < n_chunks; ch += 4 * bd) {
+            const float4 v0 = src[ch], v1 = src[ch + bd], v2 = src[ch + 2 * bd],
+                         v3 = src[ch + 3 * bd];
+            ((float4*)dst)[ch] = v0;
+            ((float4*)dst)[ch + bd] = v1;
+            ((float4*)dst)[ch + 2 * bd] = v2;
+            ((float4*)dst)[ch + 3 * bd] = v3;
+          }
+          for (; ch < n_chunks; ch += bd) ((float4*)dst)[ch] = src[ch];
+        } else {
+          for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
+            const int64_t col = ch << 2;
+            const int64_t left = C - col;
+            ((float4*)dst)[ch] = rp_load4(o, off, col, left >= 4 ? 4 : (int)left);
+          }
         }
-        for (; ch < n_chunks; ch += blockDim.x) ((float4*)dst)[ch] = src[ch];
-      } else {
+      }
+    }
+
+    int pc = 0;
+    while (pc < n_ins) {
+      const nbk_ins in = rp_fetch(S, pc);
+      if (in.op == NBK_OP_HALT) break;
+      if (in.op == NBK_OP_BODY) {
+        const int b0 = pc + 1, b1 = pc + 1 + in.aux;
         for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
           const int64_t col = ch << 2;
           const int64_t left = C - col;
-          ((float4*)dst)[ch] = rp_load4(o, off, col, left >= 4 ? 4 : (int)left);
-        }
-      }
-    }
-  }
-
-  const bool writer = threadIdx.x == 0;
-  int pc = 0;
-  const int n_ins = P.n_ins;
-  while (pc < n_ins) {
-    const nbk_ins in = P.ins[pc];
-    if (in.op == NBK_OP_HALT) break;
-    if (in.op == NBK_OP_BODY) {
-      const int b0 = pc + 1, b1 = pc + 1 + in.aux;
-      for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
-        const int64_t col = ch << 2;
-        const int64_t left = C - col;
-        const int valid = left >= 4 ? 4 : (int)left;
+          const int valid = left >= 4 ? 4 : (int)left;
+          nbk_ins nxt = rp_fetch(S, b0);
 #pragma unroll 1
-        for (int q = b0; q < b1; ++q)
-          rp_exec_body(P, P.ins[q], R, lead_idx, col, valid, stage, c_pad);
+          for (int q = b0; q < b1; ++q) {
+            const nbk_ins cur = nxt;
+            if (q + 1 < b1) nxt = rp_fetch(S, q + 1);  // fetch ahead of the decode
+            rp_exec_body(S, cur, R, lead_idx, col, valid, stage, c_pad, n_lead);
+          }
+        }
+        pc = b1;
+      } else {
+        rp_exec_scalar(S, in, R, lead_idx, writer, red_buf, n_lead);
+        ++pc;
       }
-      pc = b1;
-    } else {
-      rp_exec_scalar(P, in, R, lead_idx, writer, red_buf);
-      ++pc;
     }
+    // rows reuse the staging buffer and red_buf; RED already ends with a barrier,
+    // the staging area is private per lane, so no extra barrier is needed here
   }
 }
 
 // ----------------------------------------------------------------- flat mode
 __global__ __launch_bounds__(256) void rp_flat_kernel(const nbk_rowprog P, uint32_t cpr,
                                                       uint64_t total_chunks) {
-  const uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x;
-  if (g >= total_chunks) return;
+  __shared__ __align__(16) uint32_t prog_lds[RP_WORDS];
+  rp_copy_program(P, prog_lds);
+  const nbk_rowprog& S = *reinterpret_cast<const nbk_rowprog*>(prog_lds);
   RpRegs R;
   R.acc = (vf4)(0.f);
   const int n_lead = P.n_lead;
-  uint32_t row, cc;
-  if (cpr == 1) { row = (uint32_t)g; cc = 0; }
-  else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }
-  else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }
-  uint32_t lead_idx[NBK_RP_MAX_LEAD];
-  {
-    uint32_t rem = row;
-    for (int k = n_lead - 1; k > 0; --k) {
-      uint32_t d = (uint32_t)P.lead_dim[k];
-      uint32_t q = rem / d;
-      lead_idx[k] = rem - q * d;
-      rem = q;
-    }
-    if (n_lead > 0) lead_idx[0] = rem;
-  }
-  const int64_t col = (int64_t)cc << 2;
-  const int64_t left = P.C - col;
-  const int valid = left >= 4 ? 4 : (int)left;
-  int pc = 0;
   const int n_ins = P.n_ins;
-  while (pc < n_ins) {
-    const nbk_ins in = P.ins[pc];
-    if (in.op == NBK_OP_HALT) break;
-    if (in.op == NBK_OP_BODY) {
-      const int b1 = pc + 1 + in.aux;
+  const int64_t C = P.C;
+  uint32_t lead_dim[NBK_RP_MAX_LEAD];
+#pragma unroll
+  for (int k = 0; k < NBK_RP_MAX_LEAD; ++k) lead_dim[k] = (uint32_t)P.lead_dim[k];
+  const uint64_t stride = (uint64_t)gridDim.x * 256u;
+  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {
+    uint32_t row, cc;
+    if (cpr == 1) { row = (uint32_t)g; cc = 0; }
+    else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }
+    else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }
+    uint32_t lead_idx[NBK_RP_MAX_LEAD] = {0, 0, 0, 0};
+    if (n_lead > 0) {
+      uint32_t rem = row, q;
+      q = rem / lead_dim[3]; lead_idx[3] = rem - q * lead_dim[3]; rem = q;
+      q = rem / lead_dim[2]; lead_idx[2] = rem - q * lead_dim[2]; rem = q;
+      q = rem / lead_dim[1]; lead_idx[1] = rem - q * lead_dim[1]; rem = q;
+      lead_idx[0] = rem;
+    }
+    const int64_t col = (int64_t)cc << 2;
+    const int64_t left = C - col;
+    const int valid = left >= 4 ? 4 : (int)left;
+    int pc = 0;
+    while (pc < n_ins) {
+      const nbk_ins in = rp_fetch(S, pc);
+      if (in.op == NBK_OP_HALT) break;
+      if (in.op == NBK_OP_BODY) {
+        const int b1 = pc + 1 + in.aux;
+        nbk_ins nxt = rp_fetch(S, pc + 1);
 #pragma unroll 1
-      for (int q = pc + 1; q < b1; ++q)
-        rp_exec_body(P, P.ins[q], R, lead_idx, col, valid, nullptr, 0);
-      pc = b1;
-    } else {
-      // one lane per row writes row scalars: the lane that owns chunk 0
-      rp_exec_scalar(P, in, R, lead_idx, cc == 0, nullptr);
-      ++pc;
+        for (int q = pc + 1; q < b1; ++q) {
+          const nbk_ins cur = nxt;
+          if (q + 1 < b1) nxt = rp_fetch(S, q + 1);
+          rp_exec_body(S, cur, R, lead_idx, col, valid, nullptr, 0, n_lead);
+        }
+        pc = b1;
+      } else {
+        // one lane per row writes row scalars: the lane that owns chunk 0
+        rp_exec_scalar(S, in, R, lead_idx, cc == 0, nullptr, n_lead);
+        ++pc;
+      }
     }
   }
 }
@@ -510,9 +601,17 @@ static int rp_validate(const nbk_rowprog* p) {
   return NBK_OK;
 }
 
-extern "C" int nbk_rowprog_launch(const nbk_rowprog* p, void* stream) {
-  int rc = rp_validate(p);
+extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
+  int rc = rp_validate(prog);
   if (rc != NBK_OK) return rc;
+  // normalised copy: unused leading dims get extent 1 and stride 0 so the kernels
+  // can index all four unconditionally
+  nbk_rowprog norm = *prog;
+  for (int k = norm.n_lead; k < NBK_RP_MAX_LEAD; ++k) {
+    norm.lead_dim[k] = 1;
+    for (int i = 0; i < norm.n_operands; ++i) norm.operand[i].lead_stride[k] = 0;
+  }
+  const nbk_rowprog* p = &norm;
   hipStream_t st = (hipStream_t)stream;
   int64_t rows = 1;
   for (int k = 0; k < p->n_lead; ++k) rows *= p->lead_dim[k];
@@ -526,7 +625,20 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* p, void* stream) {
     NBK_REQUIRE(p->n_stage >= 0 && p->n_stage <= NBK_RP_MAX_STAGE, "rowprog: n_stage %d",
                 p->n_stage);
     NBK_REQUIRE(lds <= 64 * 1024, "rowprog: staging %zu bytes of LDS exceeds 64 KiB", lds);
-    hipLaunchKernelGGL(rp_block_kernel, dim3((unsigned)rows), dim3(block), lds, st, *p);
+    if (lds > 32 * 1024) {
+      // static (program copy) + dynamic (staging) LDS exceeds the 64 KiB default cap
+      static bool attr_set = false;  // idempotent, a race only repeats the call
+      if (!attr_set) {
+        NBK_HIP(hipFuncSetAttribute((const void*)rp_block_kernel,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        attr_set = true;
+      }
+    }
+    // persistent workgroups: enough to fill every CU at this block size / LDS use
+    const int per_cu = lds > 48 * 1024 ? 2 : (block >= 512 ? 2 : (block >= 256 ? 4 : 8));
+    int64_t grid = (int64_t)nbk_num_cus() * per_cu;
+    if (grid > rows) grid = rows;
+    hipLaunchKernelGGL(rp_block_kernel, dim3((unsigned)grid), dim3(block), lds, st, *p, rows);
     return nbk_check_launch("rp_block_kernel");
   }
   NBK_REQUIRE(rows <= 0xffffffffLL, "rowprog: %lld rows exceed 2^32", (long long)rows);
@@ -535,8 +647,9 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* p, void* stream) {
   const uint64_t cpr = (uint64_t)((p->C + 3) >> 2);
   NBK_REQUIRE(cpr <= 0xffffffffULL, "rowprog: row too long for a flat launch");
   const uint64_t total = (uint64_t)rows * cpr;
-  const uint64_t blocks = (total + 255) / 256;
-  NBK_REQUIRE(blocks <= 0x7fffffffULL, "rowprog: flat launch too large");
+  uint64_t blocks = (total + 255) / 256;
+  const uint64_t cap = (uint64_t)nbk_num_cus() * 8;
+  if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(rp_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, *p, (uint32_t)cpr,
                      total);
   return nbk_check_launch("rp_flat_kernel");
