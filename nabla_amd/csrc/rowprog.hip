@@ -177,6 +177,15 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
   }
 }
 
+// readfirstlane returns a SIGNED int: widening it directly to 64 bits would
+// sign-extend and corrupt the high half of a pointer, so go through uint32_t.
+__device__ __forceinline__ uint32_t rp_sgpr(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane(v);
+}
+__device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
+  return (uint64_t)rp_sgpr(v.x) | ((uint64_t)rp_sgpr(v.y) << 32);
+}
+
 __device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead);
 
 // Offset of the current row inside one operand.  Strides and indices beyond
@@ -316,15 +325,6 @@ __device__ __forceinline__ void rp_copy_program(const nbk_rowprog& P, uint32_t* 
   const uint32_t* src = reinterpret_cast<const uint32_t*>(&P);
   for (int i = threadIdx.x; i < RP_WORDS; i += blockDim.x) dst[i] = src[i];
   __syncthreads();
-}
-
-// readfirstlane returns a SIGNED int: widening it directly to 64 bits would
-// sign-extend and corrupt the high half of a pointer, so go through uint32_t.
-__device__ __forceinline__ uint32_t rp_sgpr(uint32_t v) {
-  return (uint32_t)__builtin_amdgcn_readfirstlane(v);
-}
-__device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
-  return (uint64_t)rp_sgpr(v.x) | ((uint64_t)rp_sgpr(v.y) << 32);
 }
 
 __device__ __forceinline__ nbk_ins rp_fetch(const nbk_rowprog& S, int q) {
