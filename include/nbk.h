@@ -159,6 +159,10 @@ typedef struct nbk_rowprog {
 } nbk_rowprog;
 
 int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream);
+/* 1 if the library carries a straight-line (ahead-of-time specialised) kernel
+ * for this program, 0 if the interpreter will run it.  Results are the same
+ * either way; setting NBK_ROWPROG_INTERPRET=1 forces the interpreter. */
+int nbk_rowprog_is_specialized(const nbk_rowprog* prog);
 
 /* ===================================================================== */
 /*  Reductions over a middle / leading axis                               */

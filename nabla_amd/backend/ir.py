@@ -73,15 +73,40 @@ class Builder:
         self.nodes: list[Node] = []
         self.inputs: list[Value] = []
         self._n_values = 0
+        self._cse: dict = {}
 
     def add(self, kind: str, inputs: Sequence[Value], outs: Sequence[tuple], fn: str | None = None,
             **attrs: Any) -> list[Value]:
+        # common-subexpression elimination: the same pure op on the same values is
+        # emitted once (a forward chain traced twice -- once for its value, once
+        # under grad -- collapses to one)
+        key = None
+        if kind not in ("input", "custom"):
+            try:
+                key = (kind, fn, tuple(v.id for v in inputs),
+                       tuple(sorted((k, _hashable(v)) for k, v in attrs.items())),
+                       tuple((tuple(s), d) for s, d in outs))
+                hit = self._cse.get(key)
+                if hit is not None:
+                    return hit.outputs
+            except TypeError:
+                key = None
         node = Node(kind, fn, inputs, attrs, len(self.nodes))
         for i, (shape, dtype) in enumerate(outs):
             node.outputs.append(Value(shape, dtype, node, i, self._n_values))
             self._n_values += 1
         self.nodes.append(node)
+        if key is not None:
+            self._cse[key] = node
         return node.outputs
+
+
+def _hashable(v):
+    if isinstance(v, Value):
+        return ("%", v.id)
+    if isinstance(v, (list, tuple)):
+        return tuple(_hashable(x) for x in v)
+    return v
 
 
 _CURRENT: ContextVar[Builder | None] = ContextVar("nbk_ir_builder", default=None)

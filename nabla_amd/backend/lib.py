@@ -102,6 +102,7 @@ _SIGNATURES = {
     "nbk_last_error": ([], C.c_char_p),
     "nbk_abi_version": ([], C.c_int),
     "nbk_rowprog_launch": ([C.POINTER(RowProg), C.c_void_p], C.c_int),
+    "nbk_rowprog_is_specialized": ([C.POINTER(RowProg)], C.c_int),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
                         C.c_int64, C.c_int32, C.c_void_p], C.c_int),
     "nbk_copy_strided": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,

@@ -1,0 +1,325 @@
+"""Ahead-of-time specialisation of row programs.
+
+The interpreter in ``csrc/rowprog.hip`` runs any fused group, but it pays a
+decode cost per instruction.  For the row programs that the lowering pass emits
+for the five benchmark steps, this module turns the instruction stream into
+straight-line HIP (same skeleton: persistent workgroups, 16-byte coalesced
+chunks, LDS staging of rows that are read in several phases, wavefront-shuffle +
+LDS-tree reductions) and writes them to ``csrc/rowprog_spec_gen*.hip`` together
+with a lookup table keyed by a hash of the program.  ``nbk_rowprog_launch``
+hashes the program it is given and uses the specialised kernel when one exists.
+
+    python -m nabla_amd.backend.specialize          # regenerate the sources
+
+Generation needs no GPU: the steps are traced with uninitialised host tensors
+and planned; nothing is executed.
+"""
+from __future__ import annotations
+
+import struct
+from pathlib import Path
+
+import torch
+
+from . import isa
+from .planner import Plan
+
+CSRC = Path(__file__).resolve().parents[1] / "csrc"
+N_FILES = 4  # generated sources are split so that they compile in parallel
+
+_FNV_OFFSET = 0xCBF29CE484222325
+_FNV_PRIME = 0x100000001B3
+
+
+def cs_class(col_stride: int) -> int:
+    return 0 if col_stride == 0 else 1 if col_stride == 1 else 2
+
+
+def program_bytes(a: dict) -> bytes:
+    """Canonical byte string of a row program; must match rp_program_hash() in
+    csrc/rowprog.hip."""
+    ops = a["operands"]
+    out = struct.pack("<BBHBB", 1 if a["has_reduce"] else 0, len(ops), len(a["ins"]), len(a["imm"]),
+                      a["n_stage"])
+    for o in ops:
+        out += struct.pack("<BBBb", o.dtype.abi, cs_class(o.col_stride), 1 if o.vec_ok else 0,
+                           o.stage_slot)
+    for i in a["ins"]:
+        out += struct.pack("<BBBBBBH", i[0], i[1], i[2], i[3], i[4], 0, i[5])
+    for v in a["imm"]:
+        out += struct.pack("<f", v)
+    return out
+
+
+def program_hash(a: dict) -> int:
+    h = _FNV_OFFSET
+    for b in program_bytes(a):
+        h = ((h ^ b) * _FNV_PRIME) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+# ------------------------------------------------------------------------ codegen
+def _reg(r: int) -> str:
+    return f"v{r}" if r < isa.NVEC else f"s{r}"
+
+
+def _as_vec(r: int) -> str:
+    return f"v{r}" if r < isa.NVEC else f"rp_splat(s{r})"
+
+
+def _ew_vec(op: int, dst: int, a: int, b: int, c: int) -> str:
+    name = isa.EW_NAME[op]
+    if name in isa.UNARY:
+        return f"v{dst} = rp_un4<{op}>({_as_vec(a)});"
+    if name in isa.BINARY:
+        return f"v{dst} = rp_bin4<{op}>({_as_vec(a)}, {_as_vec(b)});"
+    if name == "where":
+        return f"v{dst} = rp_where4({_as_vec(a)}, {_as_vec(b)}, {_as_vec(c)});"
+    return f"v{dst} = rp_fma4({_as_vec(a)}, {_as_vec(b)}, {_as_vec(c)});"
+
+
+def _ew_scalar(op: int, dst: int, a: int, b: int, c: int) -> str:
+    name = isa.EW_NAME[op]
+    if name in isa.UNARY:
+        return f"s{dst} = rp_unary({op}, s{a});"
+    if name in isa.BINARY:
+        return f"s{dst} = rp_binary({op}, s{a}, s{b});"
+    if name == "where":
+        return f"s{dst} = s{a} != 0.f ? s{b} : s{c};"
+    return f"s{dst} = fmaf(s{a}, s{b}, s{c});"
+
+
+def generate_kernel(a: dict, name: str) -> str:
+    """HIP source of one specialised kernel for the row program ``a``."""
+    ops = a["operands"]
+    ins = a["ins"]
+    block_mode = bool(a["has_reduce"])
+    L: list[str] = []
+    w = L.append
+    if block_mode:
+        w(f"__global__ __launch_bounds__(512) void {name}(const nbk_rowprog P, int64_t rows) {{")
+        w("  __shared__ float red_buf[16];")
+        w("  const int64_t C = P.C, c_pad = (C + 3) & ~(int64_t)3, n_chunks = c_pad >> 2;")
+        w("  const bool writer = threadIdx.x == 0;")
+    else:
+        w(f"__global__ __launch_bounds__(256) void {name}(const nbk_rowprog P, uint32_t cpr, "
+          "uint64_t total_chunks) {")
+        w("  const int64_t C = P.C;")
+    w("  (void)C;")
+    # operand descriptors with the specialised fields folded to constants
+    for k, o in enumerate(ops):
+        w(f"  nbk_operand o{k} = P.operand[{k}]; o{k}.dtype = {o.dtype.abi}; "
+          f"o{k}.vec_ok = {1 if o.vec_ok else 0}; o{k}.stage_slot = {o.stage_slot};"
+          + (f" o{k}.col_stride = {o.col_stride};" if o.col_stride in (0, 1) else ""))
+    w("  const int64_t ld1 = P.lead_dim[1], ld2 = P.lead_dim[2], ld3 = P.lead_dim[3];")
+    used_s = sorted({r for i in ins for r in (i[1], i[2], i[3], i[4]) if isa.NVEC <= r < 32})
+    if block_mode:
+        w("  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {")
+        w("    int64_t lead_idx[4];")
+        w("    { int64_t rem = row, q; q = rem / ld3; lead_idx[3] = rem - q * ld3; rem = q;"
+          " q = rem / ld2; lead_idx[2] = rem - q * ld2; rem = q;"
+          " q = rem / ld1; lead_idx[1] = rem - q * ld1; rem = q; lead_idx[0] = rem; }")
+    else:
+        w("  const uint64_t stride = (uint64_t)gridDim.x * 256u;")
+        w("  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {")
+        w("    uint32_t row, cc;")
+        w("    if (cpr == 1) { row = (uint32_t)g; cc = 0; }")
+        w("    else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }")
+        w("    else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }")
+        w("    uint32_t lead_idx[4] = {0, 0, 0, 0};")
+        w("    if (P.n_lead > 0) { uint32_t rem = row, q; const uint32_t d1 = (uint32_t)ld1, "
+          "d2 = (uint32_t)ld2, d3 = (uint32_t)ld3;"
+          " q = rem / d3; lead_idx[3] = rem - q * d3; rem = q; q = rem / d2; lead_idx[2] = rem - q * d2; rem = q;"
+          " q = rem / d1; lead_idx[1] = rem - q * d1; rem = q; lead_idx[0] = rem; }")
+        w("    const bool writer = cc == 0;")
+        w("    const int64_t col = (int64_t)cc << 2;")
+        w("    const int64_t left = C - col;")
+        w("    const int valid = left >= 4 ? 4 : (int)left;")
+    for k in range(len(ops)):
+        w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
+    if block_mode and a["n_stage"] > 0:
+        for k, o in enumerate(ops):
+            if o.stage_slot >= 0:
+                w(f"    rp_stage_row(o{k}, off{k}, rp_stage_lds + {o.stage_slot} * c_pad, C, n_chunks);")
+    if used_s:
+        w("    float " + ", ".join(f"s{r} = 0.f" for r in used_s) + ";")
+    w("    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;")
+    w("    (void)acc0; (void)acc1; (void)acc2; (void)acc3; (void)writer;")
+
+    pc = 0
+    while pc < len(ins):
+        op, dst, x, y, z, aux = ins[pc]
+        if op == isa.HALT:
+            break
+        if op == isa.BODY:
+            body = ins[pc + 1:pc + 1 + aux]
+            ind = "      " if block_mode else "    "
+            if block_mode:
+                w("    for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {")
+                w("      const int64_t col = ch << 2;")
+                w("      const int64_t left = C - col;")
+                w("      const int valid = left >= 4 ? 4 : (int)left;")
+            else:
+                w("    {")
+            used_v = sorted({r for i in body for r in (i[1], i[2], i[3], i[4])
+                             if r < isa.NVEC and i[0] not in (isa.STG,)} |
+                            {i[2] for i in body if i[0] in (isa.STG, isa.ACC) and i[2] < isa.NVEC})
+            if used_v:
+                w(ind + "float4 " + ", ".join(f"v{r}" for r in used_v) + ";")
+            for bop, bd, bx, by, bz, _ in body:
+                if bop == isa.LDG:
+                    o = ops[bx]
+                    if block_mode and o.stage_slot >= 0:
+                        w(ind + f"v{bd} = *(const float4*)(rp_stage_lds + {o.stage_slot} * c_pad + col);")
+                    else:
+                        w(ind + f"v{bd} = rp_load4(o{bx}, off{bx}, col, valid);")
+                elif bop == isa.STG:
+                    w(ind + f"rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
+                elif bop == isa.ACC:
+                    w(ind + f"acc{bd} = rp_acc4(acc{bd}, {_as_vec(bx)}, {by}, valid);")
+                elif bop == isa.COLIDX:
+                    w(ind + f"v{bd} = make_float4((float)col, (float)col + 1.f, (float)col + 2.f, "
+                      "(float)col + 3.f);")
+                else:
+                    w(ind + _ew_vec(bop, bd, bx, by, bz))
+            w("    }")
+            pc += 1 + aux
+            continue
+        if op == isa.IMM:
+            w(f"    s{dst} = P.imm[{x}];")
+        elif op == isa.LDR:
+            w(f"    s{dst} = nbk_load_as_f32(o{x}.ptr, off{x}, o{x}.dtype);")
+        elif op == isa.STR:
+            w(f"    if (writer) nbk_store_from_f32(o{dst}.ptr, off{dst}, o{dst}.dtype, s{x});")
+        elif op == isa.LEADIDX:
+            w(f"    s{dst} = (float)lead_idx[{x}];")
+        elif op == isa.ACCINIT:
+            w(f"    acc{dst} = rp_identity({x});")
+        elif op == isa.RED:
+            w(f"    s{dst} = rp_block_reduce(acc{x}, {y}, red_buf);")
+        else:
+            w("    " + _ew_scalar(op, dst, x, y, z))
+        pc += 1
+    w("  }")
+    w("}")
+    return "\n".join(L)
+
+
+_PRELUDE = '''// GENERATED by nabla_amd/backend/specialize.py -- do not edit.
+// Straight-line versions of the row programs of the benchmark steps; the
+// interpreter in rowprog.hip runs everything that is not listed here.
+#include "rowprog_device.h"
+#include "rowprog_spec.h"
+
+extern __shared__ __align__(16) float rp_stage_lds[];
+'''
+
+
+def collect_programs() -> dict[int, dict]:
+    """Plan the five benchmark steps at full size and return {hash: rowprog attrs}."""
+    import nabla_amd as nb
+    from nabla_amd import workloads as W
+    from nabla_amd.backend import executor
+    from nabla_amd.core.engine import _PLAN_CACHE, clear_plan_cache
+
+    class _PlanOnly:
+        """Executor that plans but computes nothing (outputs stay uninitialised)."""
+
+        name = "plan-only"
+        torch_device = torch.device("cpu")
+
+        def bind(self, plan: Plan):
+            ex = self
+
+            class _B:
+                def __init__(self):
+                    self.plan = plan
+
+                def run(self, inputs, timer=None):
+                    return [torch.empty(s, dtype=d.to_torch()) for _, s, d in plan.outputs]
+
+            return _B()
+
+        def current_stream(self):
+            return 0
+
+        def synchronize(self):
+            pass
+
+        def check_status(self):
+            pass
+
+    def leaves(shapes, dtype):
+        if isinstance(shapes, dict):
+            return {k: leaves(v, dtype) for k, v in shapes.items()}
+        if isinstance(shapes, list):
+            return [leaves(v, dtype) for v in shapes]
+        return nb.Tensor._from_torch(torch.empty(shapes, dtype=dtype))
+
+    prev = executor.set_executor(_PlanOnly())
+    programs: dict[int, dict] = {}
+    try:
+        f32, bf16, i64 = torch.float32, torch.bfloat16, torch.int64
+        jobs = []
+        t = leaves(W.c1_shapes(), f32)
+        jobs.append(lambda: W.c1_step(t))
+        t2 = leaves(W.c2_shapes(), f32)
+        jobs.append(lambda: W.c2_step(t2["x"], t2["y"]))
+        t3 = leaves(W.c3_shapes(), bf16)
+        jobs.append(lambda: W.c3_step(t3))
+        s4 = W.c4_shapes()
+        t4 = leaves({k: v for k, v in s4.items() if k != "labels"}, f32)
+        t4["labels"] = nb.Tensor._from_torch(torch.zeros(s4["labels"], dtype=i64))
+        jobs.append(lambda: W.c4_step(t4))
+        s5 = W.c5_shapes(layers=2)
+        t5 = leaves({k: v for k, v in s5.items() if k != "ids"}, bf16)
+        t5["ids"] = nb.Tensor._from_torch(torch.zeros(s5["ids"], dtype=i64))
+        jobs.append(lambda: W.c5_step(t5))
+        for job in jobs:
+            clear_plan_cache()
+            res = job()
+            flat = [x for x in nb.tree_leaves(res) if isinstance(x, nb.Tensor)]
+            nb.realize_all(*flat)
+            for bound in _PLAN_CACHE.values():
+                for st in bound.plan.steps:
+                    if st.kind == "rowprog":
+                        programs.setdefault(program_hash(st.attrs), st.attrs)
+    finally:
+        executor.set_executor(prev)
+    return programs
+
+
+def write_sources(programs: dict[int, dict]) -> list[Path]:
+    for old in CSRC.glob("rowprog_spec_gen*.hip"):
+        old.unlink()
+    items = sorted(programs.items())
+    files = []
+    for fi in range(N_FILES):
+        chunk = items[fi::N_FILES]
+        src = [_PRELUDE]
+        for h, a in chunk:
+            src.append(f"// members: {' '.join(a.get('members', []))}")
+            src.append(generate_kernel(a, f"rp_spec_{h:016x}"))
+            src.append("")
+        src.append(f"extern const rp_spec_entry rp_spec_table_{fi}[] = {{")
+        for h, a in chunk:
+            kind = "block" if a["has_reduce"] else "flat"
+            src.append(f"  {{0x{h:016x}ULL, (const void*)rp_spec_{h:016x}, {1 if a['has_reduce'] else 0}}},  // {kind}")
+        src.append("  {0ULL, nullptr, 0}};")
+        src.append(f"extern const int rp_spec_count_{fi} = {len(chunk)};")
+        path = CSRC / f"rowprog_spec_gen{fi}.hip"
+        path.write_text("\n".join(src) + "\n")
+        files.append(path)
+    return files
+
+
+def main() -> None:
+    programs = collect_programs()
+    files = write_sources(programs)
+    n_block = sum(1 for a in programs.values() if a["has_reduce"])
+    print(f"specialised {len(programs)} row programs ({n_block} with reductions) into "
+          f"{len(files)} files")
+
+
+if __name__ == "__main__":
+    main()

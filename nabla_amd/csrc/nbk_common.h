@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <stdlib.h>
 #include "nbk.h"
 
 // ---- error reporting (thread-local message, C ABI status codes) ----------

@@ -13,7 +13,11 @@
 // (one per chunk component) indexed with a wave-uniform index, which the
 // compiler turns into VGPR-relative moves instead of scratch memory.
 #include "nbk_common.h"
+#include "rowprog_device.h"
+#include "rowprog_spec.h"
 #include <stddef.h>
+#include <mutex>
+#include <unordered_map>
 
 typedef float vf16 __attribute__((ext_vector_type(16)));
 typedef float vf4 __attribute__((ext_vector_type(4)));
@@ -35,148 +39,6 @@ __device__ __forceinline__ void rp_write(RpRegs& R, int i, float4 v) {
   R.x[i] = v.x; R.y[i] = v.y; R.z[i] = v.z; R.w[i] = v.w;
 }
 
-__device__ __forceinline__ float rp_combine(float a, float b, int kind) {
-  if (kind == NBK_RED_SUM) return a + b;
-  if (kind == NBK_RED_MAX) return fmaxf(a, b);
-  return fminf(a, b);
-}
-__device__ __forceinline__ float rp_identity(int kind) {
-  if (kind == NBK_RED_SUM) return 0.0f;
-  if (kind == NBK_RED_MAX) return -INFINITY;
-  return INFINITY;
-}
-
-// ---- chunk load / store ----------------------------------------------------
-__device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, int64_t col,
-                                           int valid) {
-  const int dt = o.dtype;
-  const int64_t cs = o.col_stride;
-  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (o.vec_ok && valid == 4) {
-    const int64_t e = off + col;
-    if (dt == NBK_F32) {
-      r = *(const float4*)((const float*)o.ptr + e);
-    } else if (dt == NBK_BF16) {
-      uint2 u = *(const uint2*)((const uint16_t*)o.ptr + e);
-      r.x = __uint_as_float(u.x << 16);
-      r.y = __uint_as_float(u.x & 0xffff0000u);
-      r.z = __uint_as_float(u.y << 16);
-      r.w = __uint_as_float(u.y & 0xffff0000u);
-    } else if (dt == NBK_F16) {
-      const __half* h = (const __half*)o.ptr + e;
-      uint2 u = *(const uint2*)h;
-      __half2 a = *(__half2*)&u.x, b = *(__half2*)&u.y;
-      float2 fa = __half22float2(a), fb = __half22float2(b);
-      r = make_float4(fa.x, fa.y, fb.x, fb.y);
-    } else if (dt == NBK_I32) {
-      int4 u = *(const int4*)((const int32_t*)o.ptr + e);
-      r = make_float4((float)u.x, (float)u.y, (float)u.z, (float)u.w);
-    } else if (dt == NBK_I64) {
-      const int64_t* p = (const int64_t*)o.ptr + e;
-      longlong2 u0 = *(const longlong2*)p, u1 = *(const longlong2*)(p + 2);
-      r = make_float4((float)u0.x, (float)u0.y, (float)u1.x, (float)u1.y);
-    } else {
-      uint32_t u = *(const uint32_t*)((const uint8_t*)o.ptr + e);
-      r = make_float4((float)(u & 0xff), (float)((u >> 8) & 0xff), (float)((u >> 16) & 0xff),
-                      (float)(u >> 24));
-    }
-    return r;
-  }
-  const int64_t e0 = off + col * cs;
-  if (valid > 0) r.x = nbk_load_as_f32(o.ptr, e0, dt);
-  if (cs == 0) {
-    r.y = r.z = r.w = r.x;
-    return r;
-  }
-  if (valid > 1) r.y = nbk_load_as_f32(o.ptr, e0 + cs, dt);
-  if (valid > 2) r.z = nbk_load_as_f32(o.ptr, e0 + 2 * cs, dt);
-  if (valid > 3) r.w = nbk_load_as_f32(o.ptr, e0 + 3 * cs, dt);
-  return r;
-}
-
-__device__ __forceinline__ void rp_store4(const nbk_operand& o, int64_t off, int64_t col,
-                                          int valid, float4 v) {
-  const int dt = o.dtype;
-  const int64_t cs = o.col_stride;
-  if (o.vec_ok && valid == 4) {
-    const int64_t e = off + col;
-    if (dt == NBK_F32) {
-      *(float4*)((float*)o.ptr + e) = v;
-    } else if (dt == NBK_BF16) {
-      uint2 u;
-      u.x = (uint32_t)nbk_f32_to_bf16(v.x) | ((uint32_t)nbk_f32_to_bf16(v.y) << 16);
-      u.y = (uint32_t)nbk_f32_to_bf16(v.z) | ((uint32_t)nbk_f32_to_bf16(v.w) << 16);
-      *(uint2*)((uint16_t*)o.ptr + e) = u;
-    } else if (dt == NBK_F16) {
-      __half2 a = __floats2half2_rn(v.x, v.y), b = __floats2half2_rn(v.z, v.w);
-      uint2 u;
-      u.x = *(uint32_t*)&a;
-      u.y = *(uint32_t*)&b;
-      *(uint2*)((__half*)o.ptr + e) = u;
-    } else if (dt == NBK_I32) {
-      *(int4*)((int32_t*)o.ptr + e) = make_int4((int)v.x, (int)v.y, (int)v.z, (int)v.w);
-    } else if (dt == NBK_I64) {
-      int64_t* p = (int64_t*)o.ptr + e;
-      p[0] = (int64_t)v.x; p[1] = (int64_t)v.y; p[2] = (int64_t)v.z; p[3] = (int64_t)v.w;
-    } else {
-      uint32_t u = (uint32_t)(v.x != 0.f) | ((uint32_t)(v.y != 0.f) << 8) |
-                   ((uint32_t)(v.z != 0.f) << 16) | ((uint32_t)(v.w != 0.f) << 24);
-      *(uint32_t*)((uint8_t*)o.ptr + e) = u;
-    }
-    return;
-  }
-  const int64_t e0 = off + col * cs;
-  if (valid > 0) nbk_store_from_f32(o.ptr, e0, dt, v.x);
-  if (valid > 1) nbk_store_from_f32(o.ptr, e0 + cs, dt, v.y);
-  if (valid > 2) nbk_store_from_f32(o.ptr, e0 + 2 * cs, dt, v.z);
-  if (valid > 3) nbk_store_from_f32(o.ptr, e0 + 3 * cs, dt, v.w);
-}
-
-// ---- elementwise functions --------------------------------------------------
-
-
-__device__ __forceinline__ float rp_unary(int op, float a) {
-  switch (op) {
-    case NBK_OP_MOV: return a;
-    case NBK_OP_NEG: return -a;
-    case NBK_OP_RELU: return fmaxf(a, 0.0f);
-    case NBK_OP_EXP: return expf(a);
-    case NBK_OP_LOG: return logf(a);
-    case NBK_OP_SQRT: return sqrtf(a);
-    case NBK_OP_RSQRT: return 1.0f / sqrtf(a);
-    case NBK_OP_ERF: return erff(a);
-    case NBK_OP_GELU: return 0.5f * a * (1.0f + erff(a * 0.70710678118654752440f));
-    case NBK_OP_TANH: return tanhf(a);
-    case NBK_OP_SIGMOID: return 1.0f / (1.0f + expf(-a));
-    case NBK_OP_ABS: return fabsf(a);
-    case NBK_OP_RBF16: return nbk_bf16_to_f32(nbk_f32_to_bf16(a));
-    case NBK_OP_NOT: return a != 0.0f ? 0.0f : 1.0f;
-    case NBK_OP_TRUNC: return truncf(a);
-    case NBK_OP_NEZ: return a != 0.0f ? 1.0f : 0.0f;
-    default: return a;
-  }
-}
-__device__ __forceinline__ float rp_binary(int op, float a, float b) {
-  switch (op) {
-    case NBK_OP_ADD: return a + b;
-    case NBK_OP_SUB: return a - b;
-    case NBK_OP_MUL: return a * b;
-    case NBK_OP_DIV: return a / b;
-    case NBK_OP_MAX: return fmaxf(a, b);
-    case NBK_OP_MIN: return fminf(a, b);
-    case NBK_OP_GT: return a > b ? 1.0f : 0.0f;
-    case NBK_OP_GE: return a >= b ? 1.0f : 0.0f;
-    case NBK_OP_EQ: return a == b ? 1.0f : 0.0f;
-    case NBK_OP_NE: return a != b ? 1.0f : 0.0f;
-    case NBK_OP_LT: return a < b ? 1.0f : 0.0f;
-    case NBK_OP_LE: return a <= b ? 1.0f : 0.0f;
-    case NBK_OP_POW: return powf(a, b);
-    case NBK_OP_AND: return (a != 0.0f && b != 0.0f) ? 1.0f : 0.0f;
-    case NBK_OP_OR: return (a != 0.0f || b != 0.0f) ? 1.0f : 0.0f;
-    default: return a;
-  }
-}
-
 // readfirstlane returns a SIGNED int: widening it directly to 64 bits would
 // sign-extend and corrupt the high half of a pointer, so go through uint32_t.
 __device__ __forceinline__ uint32_t rp_sgpr(uint32_t v) {
@@ -187,17 +49,6 @@ __device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
 }
 
 __device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead);
-
-// Offset of the current row inside one operand.  Strides and indices beyond
-// n_lead are zero, so all four terms can be added unconditionally (constant
-// indices keep both arrays in registers).
-template <typename IDX>
-__device__ __forceinline__ int64_t rp_row_offset(const nbk_operand& o, const IDX* lead_idx,
-                                                 int n_lead) {
-  (void)n_lead;
-  return (int64_t)lead_idx[0] * o.lead_stride[0] + (int64_t)lead_idx[1] * o.lead_stride[1] +
-         (int64_t)lead_idx[2] * o.lead_stride[2] + (int64_t)lead_idx[3] * o.lead_stride[3];
-}
 
 // One body instruction on one chunk.
 template <typename IDX>
@@ -254,21 +105,6 @@ __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins
     float c0 = (float)col;
     rp_write(R, in.dst, make_float4(c0, c0 + 1.f, c0 + 2.f, c0 + 3.f));
   }
-}
-
-// Block-wide reduction of one float: wavefront shuffles, then an LDS tree.
-__device__ __forceinline__ float rp_block_reduce(float v, int kind, float* red_buf) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = rp_combine(v, __shfl_xor(v, off, 64), kind);
-  const int nw = blockDim.x >> 6;
-  if (nw == 1) return v;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  if (lane == 0) red_buf[w] = v;
-  __syncthreads();
-  float r = red_buf[0];
-  for (int i = 1; i < nw; ++i) r = rp_combine(r, red_buf[i], kind);
-  __syncthreads();
-  return r;
 }
 
 // Prologue (per-row, scalar-register) instruction.  Returns through R.
@@ -399,29 +235,8 @@ __global__ __launch_bounds__(512) void rp_block_kernel(const nbk_rowprog P, int6
       for (int oi = 0; oi < n_operands; ++oi) {
         const nbk_operand o = rp_operand(S, oi, n_lead);
         if (o.stage_slot < 0) continue;
-        const int64_t off = rp_row_offset(o, lead_idx, n_lead);
-        float* dst = rp_stage_lds + o.stage_slot * c_pad;
-        if (o.vec_ok && o.dtype == NBK_F32 && (C & 3) == 0) {
-          const float4* src = (const float4*)((const float*)o.ptr + off);
-          int64_t ch = threadIdx.x;
-          const int64_t bd = blockDim.x;
-          // four independent 16-byte loads in flight per lane
-          for (; ch + 3 * bd < n_chunks; ch += 4 * bd) {
-            const float4 v0 = src[ch], v1 = src[ch + bd], v2 = src[ch + 2 * bd],
-                         v3 = src[ch + 3 * bd];
-            ((float4*)dst)[ch] = v0;
-            ((float4*)dst)[ch + bd] = v1;
-            ((float4*)dst)[ch + 2 * bd] = v2;
-            ((float4*)dst)[ch + 3 * bd] = v3;
-          }
-          for (; ch < n_chunks; ch += bd) ((float4*)dst)[ch] = src[ch];
-        } else {
-          for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {
-            const int64_t col = ch << 2;
-            const int64_t left = C - col;
-            ((float4*)dst)[ch] = rp_load4(o, off, col, left >= 4 ? 4 : (int)left);
-          }
-        }
+        rp_stage_row(o, rp_row_offset(o, lead_idx, n_lead), rp_stage_lds + o.stage_slot * c_pad, C,
+                     n_chunks);
       }
     }
 
@@ -601,6 +416,73 @@ static int rp_validate(const nbk_rowprog* p) {
   return NBK_OK;
 }
 
+// ---- specialised kernels -------------------------------------------------------
+// FNV-1a over the canonical bytes of a program (same bytes as program_bytes() in
+// nabla_amd/backend/specialize.py): header, per-operand (dtype, stride class,
+// vec_ok, stage slot), instructions, immediates.  Extents and addresses are not
+// part of it -- a specialised kernel serves every size.
+static uint64_t rp_program_hash(const nbk_rowprog* p) {
+  uint64_t h = 0xCBF29CE484222325ULL;
+  auto eat = [&](const void* data, size_t n) {
+    const uint8_t* b = (const uint8_t*)data;
+    for (size_t i = 0; i < n; ++i) h = (h ^ b[i]) * 0x100000001B3ULL;
+  };
+  const uint8_t head[6] = {(uint8_t)(p->has_reduce ? 1 : 0), (uint8_t)p->n_operands,
+                           (uint8_t)(p->n_ins & 0xff), (uint8_t)(p->n_ins >> 8),
+                           (uint8_t)p->n_imm, (uint8_t)p->n_stage};
+  eat(head, 6);
+  for (int i = 0; i < p->n_operands; ++i) {
+    const nbk_operand& o = p->operand[i];
+    const uint8_t ob[4] = {(uint8_t)o.dtype,
+                           (uint8_t)(o.col_stride == 0 ? 0 : (o.col_stride == 1 ? 1 : 2)),
+                           (uint8_t)(o.vec_ok ? 1 : 0), (uint8_t)(int8_t)o.stage_slot};
+    eat(ob, 4);
+  }
+  for (int i = 0; i < p->n_ins; ++i) {
+    const nbk_ins& in = p->ins[i];
+    const uint8_t ib[8] = {in.op, in.dst, in.a, in.b, in.c, 0, (uint8_t)(in.aux & 0xff),
+                           (uint8_t)(in.aux >> 8)};
+    eat(ib, 8);
+  }
+  eat(p->imm, sizeof(float) * (size_t)p->n_imm);
+  return h;
+}
+
+struct RpSpec { const void* kernel; int block_mode; bool lds_attr_set; };
+static std::mutex g_spec_mu;
+static std::unordered_map<uint64_t, RpSpec>* g_specs = nullptr;
+
+static RpSpec* rp_find_spec(uint64_t h) {
+  std::lock_guard<std::mutex> lk(g_spec_mu);
+  if (!g_specs) {
+    g_specs = new std::unordered_map<uint64_t, RpSpec>();
+    const rp_spec_entry* tabs[NBK_RP_SPEC_FILES] = {rp_spec_table_0, rp_spec_table_1,
+                                                   rp_spec_table_2, rp_spec_table_3};
+    const int counts[NBK_RP_SPEC_FILES] = {rp_spec_count_0, rp_spec_count_1, rp_spec_count_2,
+                                           rp_spec_count_3};
+    for (int t = 0; t < NBK_RP_SPEC_FILES; ++t)
+      for (int i = 0; i < counts[t]; ++i)
+        (*g_specs)[tabs[t][i].hash] = RpSpec{tabs[t][i].kernel, tabs[t][i].block_mode, false};
+  }
+  auto it = g_specs->find(h);
+  return it == g_specs->end() ? nullptr : &it->second;
+}
+
+// 1: interpreter only (debug / comparison); read once.
+static bool rp_specs_disabled() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("NBK_ROWPROG_INTERPRET");
+    v = (e && e[0] == '1') ? 1 : 0;
+  }
+  return v == 1;
+}
+
+extern "C" int nbk_rowprog_is_specialized(const nbk_rowprog* prog) {
+  if (rp_validate(prog) != NBK_OK) return 0;
+  return (!rp_specs_disabled() && rp_find_spec(rp_program_hash(prog)) != nullptr) ? 1 : 0;
+}
+
 extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
   int rc = rp_validate(prog);
   if (rc != NBK_OK) return rc;
@@ -612,6 +494,8 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     for (int i = 0; i < norm.n_operands; ++i) norm.operand[i].lead_stride[k] = 0;
   }
   const nbk_rowprog* p = &norm;
+  RpSpec* spec = rp_specs_disabled() ? nullptr : rp_find_spec(rp_program_hash(prog));
+  if (spec && spec->block_mode != (p->has_reduce ? 1 : 0)) spec = nullptr;
   hipStream_t st = (hipStream_t)stream;
   int64_t rows = 1;
   for (int k = 0; k < p->n_lead; ++k) rows *= p->lead_dim[k];
@@ -638,6 +522,17 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     const int per_cu = lds > 48 * 1024 ? 2 : (block >= 512 ? 2 : (block >= 256 ? 4 : 8));
     int64_t grid = (int64_t)nbk_num_cus() * per_cu;
     if (grid > rows) grid = rows;
+    if (spec) {
+      if (lds > 32 * 1024 && !spec->lds_attr_set) {
+        NBK_HIP(hipFuncSetAttribute(spec->kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    64 * 1024));
+        spec->lds_attr_set = true;
+      }
+      int64_t rows_arg = rows;
+      void* args[2] = {(void*)p, (void*)&rows_arg};
+      NBK_HIP(hipLaunchKernel(spec->kernel, dim3((unsigned)grid), dim3(block), args, lds, st));
+      return NBK_OK;
+    }
     hipLaunchKernelGGL(rp_block_kernel, dim3((unsigned)grid), dim3(block), lds, st, *p, rows);
     return nbk_check_launch("rp_block_kernel");
   }
@@ -650,6 +545,13 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
   uint64_t blocks = (total + 255) / 256;
   const uint64_t cap = (uint64_t)nbk_num_cus() * 8;
   if (blocks > cap) blocks = cap;
+  if (spec) {
+    uint32_t cpr_arg = (uint32_t)cpr;
+    uint64_t total_arg = total;
+    void* args[3] = {(void*)p, (void*)&cpr_arg, (void*)&total_arg};
+    NBK_HIP(hipLaunchKernel(spec->kernel, dim3((unsigned)blocks), dim3(256), args, 0, st));
+    return NBK_OK;
+  }
   hipLaunchKernelGGL(rp_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, *p, (uint32_t)cpr,
                      total);
   return nbk_check_launch("rp_flat_kernel");

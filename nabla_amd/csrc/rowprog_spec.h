@@ -1,0 +1,18 @@
+// Lookup table of ahead-of-time specialised row kernels.  The generated sources
+// rowprog_spec_gen<N>.hip each define one table; rowprog.hip searches them by the
+// hash of the program it is asked to launch.
+#pragma once
+#include <stdint.h>
+
+struct rp_spec_entry {
+  uint64_t hash;
+  const void* kernel;  // same signature as rp_block_kernel / rp_flat_kernel
+  int block_mode;
+};
+
+#define NBK_RP_SPEC_FILES 4
+extern const rp_spec_entry rp_spec_table_0[];
+extern const rp_spec_entry rp_spec_table_1[];
+extern const rp_spec_entry rp_spec_table_2[];
+extern const rp_spec_entry rp_spec_table_3[];
+extern const int rp_spec_count_0, rp_spec_count_1, rp_spec_count_2, rp_spec_count_3;

@@ -3,9 +3,9 @@ result, program) triples.
 
 ``*_inputs`` build the seeded synthetic inputs (numpy ``default_rng(seed)``,
 generated on the host), ``*_reference`` evaluates the step with the fp64 oracle
-of ``oracle.ops``, and ``*_program`` is the same step written against the
-public API of the package under test (passed in as ``nb`` so that nothing here
-imports the product).  Sizes default to the full configuration and can be
+of ``oracle.ops``, and ``*_program`` runs the same step of the package under
+test (its ``workloads`` module; the package is passed in as ``nb`` so that
+nothing here imports the product).  Sizes default to the full configuration and can be
 reduced for parity tests.
 """
 from __future__ import annotations
@@ -41,10 +41,7 @@ def c1_reference(x, W1, b1, W2, b2, dtype=np.float64):
 
 
 def c1_program(nb, t: dict):
-    def loss_fn(W1, b1, W2, b2, x):
-        return nb.mean(nb.relu(x @ W1 + b1) @ W2 + b2)
-
-    return nb.value_and_grad(loss_fn, argnums=(0, 1, 2, 3))(t["W1"], t["b1"], t["W2"], t["b2"], t["x"])
+    return nb.workloads.c1_step(t)
 
 
 # ------------------------------------- C2: elementwise + reduction stress
@@ -64,19 +61,12 @@ def c2_reference(x, y, dtype=np.float64):
 
 
 def c2_chain(nb, X, Y):
-    p = X * Y
-    m = nb.reduce_max(p, axis=1, keepdims=True)
-    return nb.reduce_sum(nb.exp(p - m) * nb.relu(X), axis=1)
+    return nb.workloads.c2_chain(X, Y)
 
 
 def c2_program(nb, X, Y):
     """out and d(sum(out))/dx, both lazy."""
-    def total(X, Y):
-        return nb.reduce_sum(c2_chain(nb, X, Y))
-
-    out = c2_chain(nb, X, Y)
-    gx = nb.grad(total, argnums=0)(X, Y)
-    return out, gx
+    return nb.workloads.c2_step(X, Y)
 
 
 # ------------------------------------------------- C3: transformer block
@@ -113,32 +103,11 @@ def c3_reference(t: dict, num_heads=16, dtype=np.float64):
 
 
 def c3_block(nb, x, p: dict, num_heads: int):
-    F = nb.nn.functional
-    b, s, d = x.shape
-    hd = d // num_heads
-
-    def heads(t):
-        return nb.swap_axes(nb.reshape(t, (b, s, num_heads, hd)), 1, 2)
-
-    normed = F.layer_norm(x, p["ln1_w"], p["ln1_b"])
-    q = heads(F.linear(normed, p["wq"], p["bq"]))
-    k = heads(F.linear(normed, p["wk"], p["bk"]))
-    v = heads(F.linear(normed, p["wv"], p["bv"]))
-    a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
-    a = nb.reshape(nb.swap_axes(a, 1, 2), (b, s, d))
-    x = x + F.linear(a, p["wo"], p["bo"])
-    normed = F.layer_norm(x, p["ln2_w"], p["ln2_b"])
-    ff = F.linear(nb.gelu(F.linear(normed, p["w1"], p["b1"])), p["w2"], p["b2"])
-    return x + ff
+    return nb.workloads.transformer_block(x, p, num_heads)
 
 
 def c3_program(nb, t: dict, num_heads=16):
-    def loss_fn(params, x):
-        out = c3_block(nb, x, params, num_heads)
-        return nb.mean(out * out)
-
-    params = {k: t[k] for k in C3_PARAMS}
-    return nb.value_and_grad(loss_fn, argnums=0)(params, t["x"])
+    return nb.workloads.c3_step(t, num_heads)
 
 
 # -------------------------------------------------------------- C4: CNN step
@@ -172,20 +141,11 @@ def c4_reference(t: dict, dtype=np.float64):
 
 
 def c4_logits(nb, p: dict, img):
-    h = nb.relu(nb.conv2d(img, p["k1"], padding=1, bias=p["c1b"]))
-    h = nb.relu(nb.conv2d(h, p["k2"], padding=1, bias=p["c2b"]))
-    h = nb.max_pool2d(h, kernel_size=2)
-    h = nb.relu(nb.conv2d(h, p["k3"], padding=1, bias=p["c3b"]))
-    h = nb.mean(h, axis=(1, 2))
-    return nb.nn.functional.linear(h, p["wl"], p["bl"])
+    return nb.workloads.c4_logits(p, img)
 
 
 def c4_program(nb, t: dict):
-    def loss_fn(params, img, labels):
-        return nb.nn.functional.cross_entropy_loss(c4_logits(nb, params, img), labels)
-
-    params = {k: t[k] for k in C4_PARAMS}
-    return nb.value_and_grad(loss_fn, argnums=0)(params, t["img"], t["labels"])
+    return nb.workloads.c4_step(t)
 
 
 # ------------------------------------------------------ C5: LoRA decoder step
@@ -247,30 +207,7 @@ def c5_reference(t: dict, num_heads=16, alpha=16.0, dtype=np.float64):
 
 def c5_program(nb, t: dict, num_heads=16, alpha=16.0):
     """``t`` holds tensors of the package under test in the same nesting as c5_inputs."""
-    F = nb.nn.functional
-    lora_linear = nb.nn.finetune.lora_linear
-
-    def loss_fn(lora, base, ids):
-        x = F.embedding(ids, base["embed"])
-        b, s, d = x.shape
-        hd = d // num_heads
-        heads = lambda z: nb.swap_axes(nb.reshape(z, (b, s, num_heads, hd)), 1, 2)
-        for L, ad in zip(base["layers"], lora):
-            normed = F.layer_norm(x, L["ln1_w"], L["ln1_b"])
-            q = heads(lora_linear(normed, L["wq"], {"A": ad["qA"], "B": ad["qB"]}, alpha=alpha) + L["bq"])
-            k = heads(F.linear(normed, L["wk"], L["bk"]))
-            v = heads(lora_linear(normed, L["wv"], {"A": ad["vA"], "B": ad["vB"]}, alpha=alpha) + L["bv"])
-            a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
-            a = nb.reshape(nb.swap_axes(a, 1, 2), (b, s, d))
-            x = x + F.linear(a, L["wo"], L["bo"])
-            normed = F.layer_norm(x, L["ln2_w"], L["ln2_b"])
-            x = x + F.linear(nb.gelu(F.linear(normed, L["w1"], L["b1"])), L["w2"], L["b2"])
-        x = F.layer_norm(x, base["lnf_w"], base["lnf_b"])
-        logits = x @ base["head"]
-        return F.cross_entropy_loss(logits, ids)
-
-    base = {k: t[k] for k in ("embed", "head", "lnf_w", "lnf_b", "layers")}
-    return nb.value_and_grad(loss_fn, argnums=0)(t["lora"], base, t["ids"])
+    return nb.workloads.c5_step(t, num_heads, alpha)
 
 
 def upload(nb, tree, dtype=None):
