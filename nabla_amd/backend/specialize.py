@@ -89,18 +89,40 @@ def _ew_scalar(op: int, dst: int, a: int, b: int, c: int) -> str:
     return f"s{dst} = fmaf(s{a}, s{b}, s{c});"
 
 
-def generate_kernel(a: dict, name: str) -> str:
-    """HIP source of one specialised kernel for the row program ``a``."""
+MAX_RESIDENT_REGS = 16  # float4 registers a row-resident kernel may spend on inputs
+
+
+def full_inputs(a: dict) -> list[int]:
+    """Operand indices that the bodies load with LDG."""
+    return sorted({i[2] for i in a["ins"] if i[0] == isa.LDG})
+
+
+def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
+    """HIP source of one specialised kernel for the row program ``a``.
+
+    ``cpt`` = 0: generic form, chunk loops with a run-time trip count, rows that
+    are read in several phases staged in LDS.  ``cpt`` > 0 (reduction programs
+    only): every lane owns exactly ``cpt`` chunks of the row; all inputs are
+    loaded once into registers with every load in flight together, the chunk
+    loops are fully unrolled, and arithmetic repeated in a later phase is
+    removed by the compiler's common-subexpression elimination."""
     ops = a["operands"]
     ins = a["ins"]
     block_mode = bool(a["has_reduce"])
+    resident = cpt > 0
+    assert not resident or block_mode
+    inputs = full_inputs(a)
     L: list[str] = []
     w = L.append
     if block_mode:
-        w(f"__global__ __launch_bounds__(512) void {name}(const nbk_rowprog P, int64_t rows) {{")
+        # register-resident forms: cap registers so that two 512-lane workgroups (or
+        # more smaller ones) share a CU and one loads while the other computes
+        occ = "__attribute__((amdgpu_waves_per_eu(4))) " if 0 < cpt <= 4 else ""
+        w(f"__global__ __launch_bounds__(512) {occ}void {name}(const nbk_rowprog P, int64_t rows) {{")
         w("  __shared__ float red_buf[16];")
         w("  const int64_t C = P.C, c_pad = (C + 3) & ~(int64_t)3, n_chunks = c_pad >> 2;")
         w("  const bool writer = threadIdx.x == 0;")
+        w("  (void)c_pad;")
     else:
         w(f"__global__ __launch_bounds__(256) void {name}(const nbk_rowprog P, uint32_t cpr, "
           "uint64_t total_chunks) {")
@@ -137,7 +159,22 @@ def generate_kernel(a: dict, name: str) -> str:
         w("    const int valid = left >= 4 ? 4 : (int)left;")
     for k in range(len(ops)):
         w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
-    if block_mode and a["n_stage"] > 0:
+    if resident:
+        # every lane loads its chunks of every input up front
+        w(f"    int64_t colj[{cpt}]; int validj[{cpt}];")
+        w("#pragma unroll")
+        w(f"    for (int j = 0; j < {cpt}; ++j) {{")
+        w("      const int64_t ch = threadIdx.x + (int64_t)j * blockDim.x;")
+        w("      colj[j] = ch << 2;")
+        w("      const int64_t left = C - colj[j];")
+        w("      validj[j] = ch < n_chunks ? (left >= 4 ? 4 : (int)left) : 0;")
+        w("    }")
+        for k in inputs:
+            w(f"    float4 r{k}[{cpt}];")
+            w("#pragma unroll")
+            w(f"    for (int j = 0; j < {cpt}; ++j) r{k}[j] = validj[j] > 0 ? "
+              f"rp_load4(o{k}, off{k}, colj[j], validj[j]) : make_float4(0.f, 0.f, 0.f, 0.f);")
+    elif block_mode and a["n_stage"] > 0:
         for k, o in enumerate(ops):
             if o.stage_slot >= 0:
                 w(f"    rp_stage_row(o{k}, off{k}, rp_stage_lds + {o.stage_slot} * c_pad, C, n_chunks);")
@@ -154,7 +191,12 @@ def generate_kernel(a: dict, name: str) -> str:
         if op == isa.BODY:
             body = ins[pc + 1:pc + 1 + aux]
             ind = "      " if block_mode else "    "
-            if block_mode:
+            if resident:
+                w("#pragma unroll")
+                w(f"    for (int j = 0; j < {cpt}; ++j) {{")
+                w("      const int64_t col = colj[j];")
+                w("      const int valid = validj[j];")
+            elif block_mode:
                 w("    for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {")
                 w("      const int64_t col = ch << 2;")
                 w("      const int64_t left = C - col;")
@@ -169,12 +211,17 @@ def generate_kernel(a: dict, name: str) -> str:
             for bop, bd, bx, by, bz, _ in body:
                 if bop == isa.LDG:
                     o = ops[bx]
-                    if block_mode and o.stage_slot >= 0:
+                    if resident:
+                        w(ind + f"v{bd} = r{bx}[j];")
+                    elif block_mode and o.stage_slot >= 0:
                         w(ind + f"v{bd} = *(const float4*)(rp_stage_lds + {o.stage_slot} * c_pad + col);")
                     else:
                         w(ind + f"v{bd} = rp_load4(o{bx}, off{bx}, col, valid);")
                 elif bop == isa.STG:
-                    w(ind + f"rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
+                    if resident:
+                        w(ind + f"if (valid > 0) rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
+                    else:
+                        w(ind + f"rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
                 elif bop == isa.ACC:
                     w(ind + f"acc{bd} = rp_acc4(acc{bd}, {_as_vec(bx)}, {by}, valid);")
                 elif bop == isa.COLIDX:
@@ -203,6 +250,14 @@ def generate_kernel(a: dict, name: str) -> str:
     w("  }")
     w("}")
     return "\n".join(L)
+
+
+def resident_variants(a: dict) -> list[int]:
+    """Chunks-per-lane values for which a register-resident kernel is generated."""
+    if not a["has_reduce"]:
+        return []
+    n_in = max(1, len(full_inputs(a)))
+    return [c for c in (1, 2, 4, 8) if c * n_in <= MAX_RESIDENT_REGS]
 
 
 _PRELUDE = '''// GENERATED by nabla_amd/backend/specialize.py -- do not edit.
@@ -300,12 +355,17 @@ def write_sources(programs: dict[int, dict]) -> list[Path]:
         for h, a in chunk:
             src.append(f"// members: {' '.join(a.get('members', []))}")
             src.append(generate_kernel(a, f"rp_spec_{h:016x}"))
+            for c in resident_variants(a):
+                src.append(generate_kernel(a, f"rp_spec_{h:016x}_c{c}", cpt=c))
             src.append("")
         src.append(f"extern const rp_spec_entry rp_spec_table_{fi}[] = {{")
         for h, a in chunk:
-            kind = "block" if a["has_reduce"] else "flat"
-            src.append(f"  {{0x{h:016x}ULL, (const void*)rp_spec_{h:016x}, {1 if a['has_reduce'] else 0}}},  // {kind}")
-        src.append("  {0ULL, nullptr, 0}};")
+            rv = resident_variants(a)
+            ks = [f"(const void*)rp_spec_{h:016x}"]
+            for c in (1, 2, 4, 8):
+                ks.append(f"(const void*)rp_spec_{h:016x}_c{c}" if c in rv else "nullptr")
+            src.append(f"  {{0x{h:016x}ULL, {{{', '.join(ks)}}}, {1 if a['has_reduce'] else 0}}},")
+        src.append("  {0ULL, {nullptr, nullptr, nullptr, nullptr, nullptr}, 0}};")
         src.append(f"extern const int rp_spec_count_{fi} = {len(chunk)};")
         path = CSRC / f"rowprog_spec_gen{fi}.hip"
         path.write_text("\n".join(src) + "\n")

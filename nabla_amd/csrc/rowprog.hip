@@ -448,7 +448,7 @@ static uint64_t rp_program_hash(const nbk_rowprog* p) {
   return h;
 }
 
-struct RpSpec { const void* kernel; int block_mode; bool lds_attr_set; };
+struct RpSpec { const void* kernel[5]; int block_mode; bool lds_attr_set; };
 static std::mutex g_spec_mu;
 static std::unordered_map<uint64_t, RpSpec>* g_specs = nullptr;
 
@@ -462,7 +462,13 @@ static RpSpec* rp_find_spec(uint64_t h) {
                                            rp_spec_count_3};
     for (int t = 0; t < NBK_RP_SPEC_FILES; ++t)
       for (int i = 0; i < counts[t]; ++i)
-        (*g_specs)[tabs[t][i].hash] = RpSpec{tabs[t][i].kernel, tabs[t][i].block_mode, false};
+      {
+        RpSpec e;
+        for (int k = 0; k < 5; ++k) e.kernel[k] = tabs[t][i].kernel[k];
+        e.block_mode = tabs[t][i].block_mode;
+        e.lds_attr_set = false;
+        (*g_specs)[tabs[t][i].hash] = e;
+      }
   }
   auto it = g_specs->find(h);
   return it == g_specs->end() ? nullptr : &it->second;
@@ -523,14 +529,24 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     int64_t grid = (int64_t)nbk_num_cus() * per_cu;
     if (grid > rows) grid = rows;
     if (spec) {
+      int64_t rows_arg = rows;
+      void* args[2] = {(void*)p, (void*)&rows_arg};
+      // register-resident form: lanes own ceil(chunks / block) chunks each
+      const int64_t n_chunks = c_pad >> 2;
+      const int64_t need = (n_chunks + block - 1) / block;
+      int slot = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 3 : need <= 8 ? 4 : 0;
+      if (slot && spec->kernel[slot]) {
+        int64_t g2 = (int64_t)nbk_num_cus() * (block >= 512 ? 3 : (block >= 256 ? 6 : 12));
+        if (g2 > rows) g2 = rows;
+        NBK_HIP(hipLaunchKernel(spec->kernel[slot], dim3((unsigned)g2), dim3(block), args, 0, st));
+        return NBK_OK;
+      }
       if (lds > 32 * 1024 && !spec->lds_attr_set) {
-        NBK_HIP(hipFuncSetAttribute(spec->kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+        NBK_HIP(hipFuncSetAttribute(spec->kernel[0], hipFuncAttributeMaxDynamicSharedMemorySize,
                                     64 * 1024));
         spec->lds_attr_set = true;
       }
-      int64_t rows_arg = rows;
-      void* args[2] = {(void*)p, (void*)&rows_arg};
-      NBK_HIP(hipLaunchKernel(spec->kernel, dim3((unsigned)grid), dim3(block), args, lds, st));
+      NBK_HIP(hipLaunchKernel(spec->kernel[0], dim3((unsigned)grid), dim3(block), args, lds, st));
       return NBK_OK;
     }
     hipLaunchKernelGGL(rp_block_kernel, dim3((unsigned)grid), dim3(block), lds, st, *p, rows);
@@ -549,7 +565,7 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     uint32_t cpr_arg = (uint32_t)cpr;
     uint64_t total_arg = total;
     void* args[3] = {(void*)p, (void*)&cpr_arg, (void*)&total_arg};
-    NBK_HIP(hipLaunchKernel(spec->kernel, dim3((unsigned)blocks), dim3(256), args, 0, st));
+    NBK_HIP(hipLaunchKernel(spec->kernel[0], dim3((unsigned)blocks), dim3(256), args, 0, st));
     return NBK_OK;
   }
   hipLaunchKernelGGL(rp_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, *p, (uint32_t)cpr,

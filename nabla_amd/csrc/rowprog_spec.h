@@ -6,7 +6,11 @@
 
 struct rp_spec_entry {
   uint64_t hash;
-  const void* kernel;  // same signature as rp_block_kernel / rp_flat_kernel
+  // [0]: generic form (any row length).  [1..4]: register-resident forms for
+  // reduction programs whose lanes own exactly 1 / 2 / 4 / 8 chunks of a row;
+  // nullptr where that form was not generated.  All have the signature of
+  // rp_block_kernel / rp_flat_kernel.
+  const void* kernel[5];
   int block_mode;
 };
 
