@@ -40,6 +40,7 @@ struct GemmArgs {
   float alpha;
   int32_t tiles_m, tiles_n;
   int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
+  int32_t order;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -53,13 +54,15 @@ __device__ __forceinline__ float gemm_act(float v, int act) {
 // walk that run in groups of 8 tile-rows per tile-column: workgroups that share
 // an L2 also share the A and B panels they read.
 __device__ __forceinline__ void gemm_tile_coords(int bid, int tiles_m, int tiles_n, int& tm,
-                                                 int& tn) {
-  {
+                                                 int& tn, int order = 0) {
+  if (order == 1) { tm = bid / tiles_n; tn = bid % tiles_n; return; }
+  if (order != 3) {
     const int n = tiles_m * tiles_n;
     const int xcd = bid & 7, local = bid >> 3;
     const int per = n >> 3, rem = n & 7;
     bid = xcd < rem ? xcd * (per + 1) + local : rem * (per + 1) + (xcd - rem) * per + local;
   }
+  if (order == 2) { tm = bid / tiles_n; tn = bid % tiles_n; return; }
   const int group = 8;
   const int per_group = group * tiles_n;
   const int g = bid / per_group;
@@ -90,7 +93,14 @@ __device__ __forceinline__ uint4 ld8_bf16(const uint16_t* p, int64_t valid, bool
   return r;
 }
 
-template <int ROWS, bool KC>
+// FAST loaders assume 16-byte-aligned operands, K % 8 == 0 and, for an operand
+// that is contiguous along its rows, a row count that is a multiple of 8; then
+// every access is one predicated 16-byte load.  Rows past the edge are clamped
+// to the last valid row (their products are never stored); chunks past K read
+// zero.  Everything else goes through the guarded element-wise path (FAST=false),
+// which is kept out of the hot kernels because its code size alone would push
+// the main loop out of the instruction cache.
+template <int ROWS, bool KC, bool FAST>
 struct TileLoader {
   // KC : operand contiguous along K   -> ROWS*8 chunk tasks, ROWS/32 per lane
   // !KC: operand contiguous along rows -> ROWS (8x8 block) tasks, <=1 per lane
@@ -106,8 +116,14 @@ struct TileLoader {
         const int t = tid + s * 256;
         const int row = t >> 3, c = t & 7;
         const int64_t gr = row0 + row, gk = k0 + c * 8;
-        if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
-        else reg[s] = make_uint4(0, 0, 0, 0);
+        if (FAST) {
+          const int64_t r = gr < rows_total ? gr : rows_total - 1;
+          const uint4* p = (const uint4*)(base + r * rs + gk);
+          reg[s] = gk < K ? *p : make_uint4(0, 0, 0, 0);
+        } else {
+          if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
+          else reg[s] = make_uint4(0, 0, 0, 0);
+        }
       }
     } else {
       constexpr int NC = ROWS / 8;
@@ -117,8 +133,14 @@ struct TileLoader {
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           const int64_t gk = k0 + kg * 8 + r;
-          if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
-          else reg[r] = make_uint4(0, 0, 0, 0);
+          if (FAST) {
+            const int64_t rr = gr < rows_total ? gr : rows_total - 8;
+            const uint4* p = (const uint4*)(base + gk * cs + rr);
+            reg[r] = gk < K ? *p : make_uint4(0, 0, 0, 0);
+          } else {
+            if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
+            else reg[r] = make_uint4(0, 0, 0, 0);
+          }
         }
       }
     }
@@ -137,32 +159,34 @@ struct TileLoader {
       const int nc = tid % NC, kg = tid / NC;
       if (kg < 8) {
         // 8x8 transpose of 16-bit elements: out[j] holds k = 0..7 of column j
-        const uint32_t* in = (const uint32_t*)reg;  // in[r*4 + d]
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const int d = j >> 1;
           const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
           uint4 o;
-          o.x = __builtin_amdgcn_perm(in[1 * 4 + d], in[0 * 4 + d], sel);
-          o.y = __builtin_amdgcn_perm(in[3 * 4 + d], in[2 * 4 + d], sel);
-          o.z = __builtin_amdgcn_perm(in[5 * 4 + d], in[4 * 4 + d], sel);
-          o.w = __builtin_amdgcn_perm(in[7 * 4 + d], in[6 * 4 + d], sel);
+          o.x = __builtin_amdgcn_perm(comp(reg[1], j >> 1), comp(reg[0], j >> 1), sel);
+          o.y = __builtin_amdgcn_perm(comp(reg[3], j >> 1), comp(reg[2], j >> 1), sel);
+          o.z = __builtin_amdgcn_perm(comp(reg[5], j >> 1), comp(reg[4], j >> 1), sel);
+          o.w = __builtin_amdgcn_perm(comp(reg[7], j >> 1), comp(reg[6], j >> 1), sel);
           lds[swz(nc * 8 + j, kg)] = o;
         }
       }
     }
   }
+
+  static __device__ __forceinline__ uint32_t comp(const uint4& v, int d) {
+    return d == 0 ? v.x : d == 1 ? v.y : d == 2 ? v.z : v.w;
+  }
 };
 
 extern __shared__ __align__(16) uint4 gemm_lds[];
 
-template <int BM, int BN, bool A_KC, bool B_KC>
+template <int BM, int BN, bool A_KC, bool B_KC, bool FAST, bool EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int TILE_CHUNKS = (BM + BN) * 8;
   int tm_i, tn_i;
-  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i, g.order);
   const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
   const int64_t b = blockIdx.y;
   const uint16_t* A = (const uint16_t*)g.A + b * g.a_bs;
@@ -177,8 +201,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
 
-  TileLoader<BM, A_KC> la;
-  TileLoader<BN, B_KC> lb;
+  TileLoader<BM, A_KC, FAST> la;
+  TileLoader<BN, B_KC, FAST> lb;
   const int64_t nk = (g.K + 63) / 64;
   // A is rows = m; for the loader a K-contiguous operand has (rs = row stride, k unit),
   // a row-contiguous one has (cs = k stride, row unit).
@@ -187,6 +211,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   la.store(gemm_lds);
   lb.store(gemm_lds + BM * 8);
   __syncthreads();
+
+  // fragment addresses: row part is loop-invariant, only the chunk index moves
+  int a_row[TM], b_row[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a_row[i] = wm + i * 32 + li;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b_row[j] = wn + j * 32 + li;
 
   for (int64_t kt = 0; kt < nk; ++kt) {
     const uint4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
@@ -204,12 +235,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
       bf16x8 fa[TM], fb[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        uint4 u = As[swz(wm + i * 32 + li, kc)];
+        uint4 u = As[swz(a_row[i], kc)];
         fa[i] = *(bf16x8*)&u;
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        uint4 u = Bs[swz(wn + j * 32 + li, kc)];
+        uint4 u = Bs[swz(b_row[j], kc)];
         fb[j] = *(bf16x8*)&u;
       }
 #pragma unroll
@@ -225,30 +256,83 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  // epilogue: D[i][j] of a 32x32 tile lives in lane (j, (i / 4) % 2), register
-  // (i / 8) * 4 + i % 4.
-  char* Cb = (char*)g.C;
+  // Epilogue.  D[i][j] of a 32x32 MFMA tile lives in lane (j, (i / 4) % 2),
+  // register (i / 8) * 4 + i % 4.  Each wave passes its accumulators through a
+  // private LDS slab, 32 rows at a time, so that C is written as whole
+  // 16-byte (bf16) / 32-byte (fp32) pieces of a row: 8 columns per lane.
+  // The plain form (no bias / activation / residual) is a separate
+  // instantiation: the fused form carries erf() bodies, and an epilogue that does
+  // not fit the instruction cache costs more than the whole K loop of a short GEMM.
+  constexpr int SLAB_LD = WN + 4;  // floats per slab row (padding spreads the two row groups)
+  float* slab = (float*)gemm_lds + wave * (32 * SLAB_LD);
   const bool out_f32 = g.dtype_c == NBK_F32;
-  static_for<TM * TN>([&](auto t) {
-    constexpr int i = decltype(t)::value / TN, j = decltype(t)::value % TN;
-    const int64_t col = n0 + wn + j * 32 + li;
-    const bool col_ok = col < g.N;
-    float bv = 0.f;
-    if (g.bias && col_ok) bv = nbk_load_as_f32(g.bias, col, g.dtype_c);
-    const f32x16 a = acc[i][j];
-    const int64_t row_base = m0 + wm + i * 32 + kg * 4;
+  constexpr int LANES_PER_ROW = WN / 8;        // each lane writes 8 consecutive columns
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  const int sub_r = lane / LANES_PER_ROW, sub_c = (lane % LANES_PER_ROW) * 8;
+  const int64_t col = n0 + wn + sub_c;
+  const bool vec_store = FAST && (col + 8 <= g.N) && ((g.ldc & 7) == 0) && ((g.c_bs & 7) == 0);
+  float bias_v[8];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int64_t row = row_base + (r >> 2) * 8 + (r & 3);
-      if (col_ok && row < g.M) {
-        float v = a[r] * g.alpha + bv;
-        v = gemm_act(v, g.act);
+  for (int e = 0; e < 8; ++e) bias_v[e] = 0.f;
+  if (EPI && g.bias) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (col + e < g.N) bias_v[e] = nbk_load_as_f32(g.bias, col + e, g.dtype_c);
+  }
+  static_for<TM>([&](auto ti) {
+    constexpr int i = decltype(ti)::value;
+    static_for<TN>([&](auto tj) {
+      constexpr int j = decltype(tj)::value;
+      const f32x16 a = acc[i][j];
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        slab[((r >> 2) * 8 + kg * 4 + (r & 3)) * SLAB_LD + j * 32 + li] = a[r];
+    });
+    // the slab is private to the wave: no workgroup barrier, only LDS ordering
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+#pragma unroll 1
+    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+      const int lr = pass * ROWS_PER_PASS + sub_r;
+      const int64_t row = m0 + wm + i * 32 + lr;
+      float v[8];
+      const float4 p0 = *(const float4*)&slab[lr * SLAB_LD + sub_c];
+      const float4 p1 = *(const float4*)&slab[lr * SLAB_LD + sub_c + 4];
+      v[0] = p0.x; v[1] = p0.y; v[2] = p0.z; v[3] = p0.w;
+      v[4] = p1.x; v[5] = p1.y; v[6] = p1.z; v[7] = p1.w;
+      if (row < g.M && col < g.N) {
         const int64_t idx = b * g.c_bs + row * g.ldc + col;
-        if (g.residual) v += nbk_load_as_f32(g.residual, idx, g.dtype_c);
-        if (out_f32) ((float*)Cb)[idx] = v;
-        else ((uint16_t*)Cb)[idx] = nbk_f32_to_bf16(v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
+        if (EPI) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float x = gemm_act(v[e] + bias_v[e], g.act);
+            if (g.residual && col + e < g.N) x += nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
+            v[e] = x;
+          }
+        }
+        if (vec_store && !out_f32) {
+          uint4 o;
+          o.x = (uint32_t)nbk_f32_to_bf16(v[0]) | ((uint32_t)nbk_f32_to_bf16(v[1]) << 16);
+          o.y = (uint32_t)nbk_f32_to_bf16(v[2]) | ((uint32_t)nbk_f32_to_bf16(v[3]) << 16);
+          o.z = (uint32_t)nbk_f32_to_bf16(v[4]) | ((uint32_t)nbk_f32_to_bf16(v[5]) << 16);
+          o.w = (uint32_t)nbk_f32_to_bf16(v[6]) | ((uint32_t)nbk_f32_to_bf16(v[7]) << 16);
+          *(uint4*)((uint16_t*)g.C + idx) = o;
+        } else if (vec_store && out_f32) {
+          float4* dst = (float4*)((float*)g.C + idx);
+          dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+          dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < g.N) {
+              if (out_f32) ((float*)g.C)[idx + e] = v[e];
+              else ((uint16_t*)g.C)[idx + e] = nbk_f32_to_bf16(v[e]);
+            }
+        }
       }
     }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next tile row overwrites it
   });
 }
 
@@ -365,16 +449,24 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
 }
 
 // ------------------------------------------------------------------------- dispatch
-template <int BM, int BN>
+template <int BM, int BN, bool FAST>
 static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
   GemmArgs g = a;
   g.tiles_m = (int)((a.M + BM - 1) / BM);
   g.tiles_n = (int)((a.N + BN - 1) / BN);
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
-  const size_t lds = 2 * (size_t)(BM + BN) * 8 * sizeof(uint4);
+  const size_t pipe = 2 * (size_t)(BM + BN) * 8 * sizeof(uint4);
+  const size_t slabs = 4 * 32 * (size_t)(BN / 2 + 4) * sizeof(float);
+  const size_t lds = pipe > slabs ? pipe : slabs;
+  const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
 #define NBK_LAUNCH_BF16(AK, BK_)                                                              \
   do {                                                                                        \
-    auto kern = gemm_bf16_kernel<BM, BN, AK, BK_>;                                            \
+    if (epi) NBK_LAUNCH_BF16_E(AK, BK_, true);                                                \
+    else NBK_LAUNCH_BF16_E(AK, BK_, false);                                                   \
+  } while (0)
+#define NBK_LAUNCH_BF16_E(AK, BK_, EP)                                                        \
+  do {                                                                                        \
+    auto kern = gemm_bf16_kernel<BM, BN, AK, BK_, FAST, EP>;                                  \
     static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
     if (!attr_set) {                                                                          \
       NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -388,6 +480,7 @@ static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hip
   else if (!akc && bkc) NBK_LAUNCH_BF16(false, true);
   else NBK_LAUNCH_BF16(false, false);
 #undef NBK_LAUNCH_BF16
+#undef NBK_LAUNCH_BF16_E
   return nbk_check_launch("gemm_bf16_kernel");
 }
 
@@ -417,6 +510,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.a_rs = d->a_rs; a.a_cs = d->a_cs; a.b_rs = d->b_rs; a.b_cs = d->b_cs; a.ldc = d->ldc;
   a.a_bs = d->a_bs; a.b_bs = d->b_bs; a.c_bs = d->c_bs;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
+  { const char* e = getenv("NBK_GEMM_ORDER"); a.order = e ? atoi(e) : 0; }
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;
@@ -428,10 +522,13 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs);
   if (d->dtype_ab == NBK_BF16) {
+    const bool fast = a.a_vec && a.b_vec && (d->K % 8 == 0) && (akc || d->M % 8 == 0) &&
+                      (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
+    if (!fast) return launch_bf16<128, 128, false>(a, akc, bkc, d->batch, st);
     const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
     if (big_tiles >= 384 && d->M >= 256 && d->N >= 256)
-      return launch_bf16<256, 256>(a, akc, bkc, d->batch, st);
-    return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);
+      return launch_bf16<256, 256, true>(a, akc, bkc, d->batch, st);
+    return launch_bf16<128, 128, true>(a, akc, bkc, d->batch, st);
   }
   a.tiles_m = (int)((d->M + 127) / 128);
   a.tiles_n = (int)((d->N + 127) / 128);
