@@ -152,7 +152,7 @@ typedef struct nbk_rowprog {
   int32_t has_reduce;     /* 0: flat launch, 1: one workgroup per row          */
   int32_t block;          /* workgroup size for has_reduce=1 (64..512, pow2)   */
   int32_t n_stage;        /* operands pre-loaded into LDS (has_reduce=1 only)  */
-  int32_t reserved;
+  int32_t reserved;       /* 1: run on the interpreter even if a specialised kernel exists */
   float imm[NBK_RP_MAX_IMM];
   nbk_operand operand[NBK_RP_MAX_OPERANDS];
   nbk_ins ins[NBK_RP_MAX_INS];

@@ -43,6 +43,7 @@ class BoundPlan:
                     self.base[b.id] = a0 + b.offset
         self.dynamic = [b.id for b in plan.bufs if b.role in ("input", "output")]
         self.calls: list[tuple] = []  # (fn, args tuple, patch list)
+        self.has_gather = any(st.kind == "gather" for st in plan.steps)
         self._prepare()
 
     # -- address helpers -------------------------------------------------------
@@ -77,6 +78,7 @@ class BoundPlan:
                 rp.has_reduce = 1 if a["has_reduce"] else 0
                 rp.block = a["block"]
                 rp.n_stage = a["n_stage"]
+                rp.reserved = 1 if self.ex.force_interpreter else 0
                 for i, v in enumerate(a["imm"]):
                     rp.imm[i] = v
                 for i, o in enumerate(a["operands"]):
@@ -262,6 +264,8 @@ class BoundPlan:
             if after is not None:
                 after()
         del keep
+        if self.has_gather:
+            ex.status_dirty = True
         return outs
 
 
@@ -289,6 +293,8 @@ class HipExecutor:
         lib.check(self.lib.nbk_init(device))
         self.torch_device = torch.device("cuda", device)
         self.status_flag = torch.zeros(1, dtype=torch.int32, device=self.torch_device)
+        self.status_dirty = False        # a launched plan may have flagged a bad gather index
+        self.force_interpreter = False   # plans bound while set never use specialised row kernels
 
     def current_stream(self) -> int:
         return torch.cuda.current_stream(self.torch_device).cuda_stream
@@ -301,6 +307,9 @@ class HipExecutor:
 
     def check_status(self) -> None:
         """Raise if a kernel flagged a data-dependent error (out-of-range gather index)."""
+        if not self.status_dirty:
+            return
+        self.status_dirty = False
         if int(self.status_flag.item()) != 0:
             self.status_flag.zero_()
             raise IndexError("gather: index out of range")

@@ -290,6 +290,8 @@ class Tensor:
 
     def to_numpy(self) -> np.ndarray:
         buf = self.buffers
+        from ..backend.executor import get_executor
+        get_executor().check_status()
         if buf.dtype == torch.bfloat16:
             buf = buf.float()
         return buf.detach().cpu().numpy()

@@ -40,7 +40,6 @@ struct GemmArgs {
   float alpha;
   int32_t tiles_m, tiles_n;
   int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
-  int32_t order;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -54,15 +53,13 @@ __device__ __forceinline__ float gemm_act(float v, int act) {
 // walk that run in groups of 8 tile-rows per tile-column: workgroups that share
 // an L2 also share the A and B panels they read.
 __device__ __forceinline__ void gemm_tile_coords(int bid, int tiles_m, int tiles_n, int& tm,
-                                                 int& tn, int order = 0) {
-  if (order == 1) { tm = bid / tiles_n; tn = bid % tiles_n; return; }
-  if (order != 3) {
+                                                 int& tn) {
+  {
     const int n = tiles_m * tiles_n;
     const int xcd = bid & 7, local = bid >> 3;
     const int per = n >> 3, rem = n & 7;
     bid = xcd < rem ? xcd * (per + 1) + local : rem * (per + 1) + (xcd - rem) * per + local;
   }
-  if (order == 2) { tm = bid / tiles_n; tn = bid % tiles_n; return; }
   const int group = 8;
   const int per_group = group * tiles_n;
   const int g = bid / per_group;
@@ -186,7 +183,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int TILE_CHUNKS = (BM + BN) * 8;
   int tm_i, tn_i;
-  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i, g.order);
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
   const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
   const int64_t b = blockIdx.y;
   const uint16_t* A = (const uint16_t*)g.A + b * g.a_bs;
@@ -510,7 +507,6 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.a_rs = d->a_rs; a.a_cs = d->a_cs; a.b_rs = d->b_rs; a.b_cs = d->b_cs; a.ldc = d->ldc;
   a.a_bs = d->a_bs; a.b_bs = d->b_bs; a.c_bs = d->c_bs;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
-  { const char* e = getenv("NBK_GEMM_ORDER"); a.order = e ? atoi(e) : 0; }
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;

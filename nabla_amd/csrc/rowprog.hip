@@ -500,7 +500,8 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     for (int i = 0; i < norm.n_operands; ++i) norm.operand[i].lead_stride[k] = 0;
   }
   const nbk_rowprog* p = &norm;
-  RpSpec* spec = rp_specs_disabled() ? nullptr : rp_find_spec(rp_program_hash(prog));
+  RpSpec* spec = (rp_specs_disabled() || prog->reserved == 1) ? nullptr
+                                                               : rp_find_spec(rp_program_hash(prog));
   if (spec && spec->block_mode != (p->has_reduce ? 1 : 0)) spec = nullptr;
   hipStream_t st = (hipStream_t)stream;
   int64_t rows = 1;

@@ -1,0 +1,135 @@
+"""The C-ABI library: it loads, exports every symbol that include/nbk.h declares,
+and the ctypes mirrors of its structs have the layout the C compiler gives them.
+No compute calls are made here (no GPU needed)."""
+import ctypes as C
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "nbk.h"
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from nabla_amd.backend import lib
+
+    L = lib.load()
+    hdr = HEADER.read_text()
+    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(nbk_[a-z0-9_]+)\s*\(", hdr, re.M))
+    assert len(declared) >= 20
+    for name in sorted(declared):
+        assert hasattr(L, name), f"{name} is declared in nbk.h but not exported"
+        assert name in lib.EXPORTS, f"{name} has no ctypes signature in lib.py"
+    assert L.nbk_abi_version() == lib.ABI_VERSION
+    m = re.search(r"#define NBK_ABI_VERSION (\d+)", hdr)
+    assert int(m.group(1)) == lib.ABI_VERSION
+
+
+def test_isa_numbers_match_header():
+    from nabla_amd.backend import isa
+
+    hdr = HEADER.read_text()
+    enum = dict((k, int(v)) for k, v in re.findall(r"NBK_OP_([A-Z0-9]+)\s*=\s*(\d+)", hdr))
+    for name, code in isa.STRUCT_NAMES.items():
+        assert enum[name] == code, name
+    for name, code in isa.EW.items():
+        assert enum[name.upper()] == code, name
+    lim = dict((k, int(v)) for k, v in re.findall(r"#define NBK_RP_([A-Z_]+) (\d+)", hdr))
+    assert lim["MAX_OPERANDS"] == isa.MAX_OPERANDS and lim["MAX_INS"] == isa.MAX_INS
+    assert lim["MAX_IMM"] == isa.MAX_IMM and lim["MAX_LEAD"] == isa.MAX_LEAD
+    assert lim["NVEC"] == isa.NVEC and lim["NSCL"] == isa.NSCL and lim["NACC"] == isa.NACC
+
+
+def test_struct_layouts_match_the_c_compiler(tmp_path):
+    from nabla_amd.backend import lib
+
+    src = tmp_path / "sizes.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "nbk.h"\n'
+        "int main(void) {\n"
+        '  printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(nbk_rowprog), sizeof(nbk_operand),\n'
+        "         sizeof(nbk_ins), sizeof(nbk_gemm_desc), sizeof(nbk_conv_desc), sizeof(nbk_pool_desc),\n"
+        "         sizeof(nbk_tensor));\n"
+        '  printf("%zu %zu %zu %zu\\n", offsetof(nbk_rowprog, imm), offsetof(nbk_rowprog, operand),\n'
+        "         offsetof(nbk_rowprog, ins), offsetof(nbk_gemm_desc, alpha));\n"
+        "  return 0;\n}\n")
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", f"-I{ROOT / 'include'}", str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()
+    sizes = [int(x) for x in out]
+    assert sizes[:7] == [C.sizeof(lib.RowProg), C.sizeof(lib.Operand), C.sizeof(lib.Ins),
+                         C.sizeof(lib.GemmDesc), C.sizeof(lib.ConvDesc), C.sizeof(lib.PoolDesc),
+                         C.sizeof(lib.TensorDesc)]
+    assert sizes[7:] == [lib.RowProg.imm.offset, lib.RowProg.operand.offset, lib.RowProg.ins.offset,
+                         lib.GemmDesc.alpha.offset]
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    from nabla_amd.backend import lib
+
+    monkeypatch.setattr(lib, "_lib", None)
+    with pytest.raises(lib.NbkError, match="missing"):
+        lib.load(tmp_path / "libnbk.so")
+
+
+def test_no_gpu_means_no_executor():
+    """Without a GPU the package must refuse to compute rather than fall back."""
+    import torch
+    from nabla_amd.backend import executor
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    prev = executor.set_executor(None)
+    try:
+        with pytest.raises(RuntimeError, match="no CPU execution path"):
+            executor.get_executor()
+    finally:
+        executor.set_executor(prev)
+
+
+def test_specialised_program_hash_matches_between_python_and_c(emulator):
+    """The generator's hash and the library's hash must agree, or specialised
+    kernels would silently never be used."""
+    import numpy as np
+    import nabla_amd as nb
+    from nabla_amd.backend import lib, specialize
+    from nabla_amd.backend.executor import BoundPlan
+    from nabla_amd.core.engine import _PLAN_CACHE
+
+    x = nb.Tensor.constant(np.ones((64, 8192), np.float32))
+    y = nb.Tensor.constant(np.ones((64, 8192), np.float32))
+    out, gx = nb.workloads.c2_step(x, y)
+    nb.realize_all(out, gx)
+    plan = list(_PLAN_CACHE.values())[-1].plan
+    L = lib.load()
+
+    class _FakeEx:
+        lib = L
+        torch_device = None
+
+    progs = [s for s in plan.steps if s.kind == "rowprog"]
+    assert progs
+    # build the ctypes record exactly as the executor does and ask the library
+    for st in progs:
+        a = st.attrs
+        rp = lib.RowProg()
+        rp.n_lead = len(a["lead"])
+        for i, d in enumerate(a["lead"]):
+            rp.lead_dim[i] = d
+        rp.C, rp.n_operands, rp.n_ins, rp.n_imm = a["C"], len(a["operands"]), len(a["ins"]), len(a["imm"])
+        rp.has_reduce, rp.block, rp.n_stage = int(a["has_reduce"]), a["block"], a["n_stage"]
+        for i, v in enumerate(a["imm"]):
+            rp.imm[i] = v
+        for i, o in enumerate(a["operands"]):
+            od = rp.operand[i]
+            od.ptr = 4096  # any non-null, aligned address; nothing is launched
+            od.col_stride, od.dtype, od.vec_ok, od.stage_slot = o.col_stride, o.dtype.abi, int(o.vec_ok), o.stage_slot
+            for j, s_ in enumerate(o.lead_strides):
+                od.lead_stride[j] = s_
+        for i, ins in enumerate(a["ins"]):
+            d = rp.ins[i]
+            d.op, d.dst, d.a, d.b, d.c, d.aux = ins
+        assert L.nbk_rowprog_is_specialized(C.byref(rp)) == 1, \
+            f"hash {specialize.program_hash(a):016x} not found in the library's table"

@@ -1,0 +1,362 @@
+"""Host logic (no GPU): tracing, autodiff replay, lowering / fusion / view
+folding, plan cache and ``compile`` semantics, checked by running the produced
+launch records on the numpy interpreter of oracle/emulator.py and comparing with
+the CPU oracle.  The HIP path itself is covered by the ``gpu`` tests."""
+import numpy as np
+import pytest
+
+import nabla_amd as nb
+from oracle import configs as oc
+from oracle import ops as O
+
+RNG = np.random.default_rng(11)
+F = nb.nn.functional
+
+
+def T(a, dtype=None):
+    return nb.Tensor.constant(a, dtype=dtype)
+
+
+def last_plan():
+    from nabla_amd.core.engine import _PLAN_CACHE
+    return list(_PLAN_CACHE.values())[-1].plan
+
+
+def relerr(a, b):
+    return np.abs(np.asarray(a, np.float64) - b).max() / (np.abs(b).max() + 1e-30)
+
+
+# ---- ops ---------------------------------------------------------------------------
+def test_elementwise_broadcast_and_scalars(emulator):
+    x = RNG.standard_normal((3, 1, 5)).astype(np.float32)
+    y = RNG.standard_normal((4, 5)).astype(np.float32)
+    z = (T(x) + T(y)) * 2.0 - 1.0 / (nb.exp(T(y)) + 1.0)
+    ref = (x + y) * np.float32(2.0) - np.float32(1.0) / (np.exp(y) + np.float32(1.0))
+    np.testing.assert_allclose(z.numpy(), ref, rtol=1e-6, atol=1e-6)
+    assert z.shape == (3, 4, 5)
+    # the arithmetic ops are single IEEE operations: bit-exact against numpy
+    np.testing.assert_array_equal((T(x) * T(x) - T(x)).numpy(), x * x - x)
+
+
+def test_comparisons_where_cast_are_exact(emulator):
+    x = RNG.standard_normal((6, 7)).astype(np.float32)
+    y = RNG.standard_normal((6, 7)).astype(np.float32)
+    m = nb.greater(T(x), T(y))
+    assert m.dtype is nb.DType.bool
+    np.testing.assert_array_equal(m.numpy(), x > y)
+    np.testing.assert_array_equal(nb.equal(T(x), T(x)).numpy(), np.ones_like(x, bool))
+    np.testing.assert_array_equal(nb.where(m, T(x), T(y)).numpy(), np.where(x > y, x, y))
+    np.testing.assert_array_equal(nb.cast(m, nb.DType.float32).numpy(), (x > y).astype(np.float32))
+    np.testing.assert_array_equal(nb.less(T(x), 0.0).numpy(), x < 0)
+
+
+def test_reductions_all_axes_and_keepdims(emulator):
+    x = RNG.standard_normal((3, 4, 5)).astype(np.float32)
+    for axis in (None, 0, 1, -1, (0, 2), (1, 2)):
+        for keep in (False, True):
+            np.testing.assert_allclose(nb.reduce_sum(T(x), axis=axis, keepdims=keep).numpy(),
+                                       x.sum(axis=axis, keepdims=keep), rtol=1e-5, atol=1e-5)
+            np.testing.assert_array_equal(nb.reduce_max(T(x), axis=axis, keepdims=keep).numpy(),
+                                          x.max(axis=axis, keepdims=keep))
+    np.testing.assert_allclose(nb.mean(T(x), axis=(0, 1)).numpy(), x.mean(axis=(0, 1)), rtol=1e-5)
+    assert nb.argmax(T(x), axis=1).dtype is nb.DType.int64
+    np.testing.assert_array_equal(nb.argmax(T(x), axis=1).numpy(), x.argmax(1))
+    np.testing.assert_array_equal(nb.argmax(T(x), axis=-1, keepdims=True).numpy(),
+                                  x.argmax(-1)[..., None])
+
+
+def test_views_are_folded_not_copied(emulator):
+    x = RNG.standard_normal((4, 6, 8)).astype(np.float32)
+    y = nb.swap_axes(T(x), 0, 2)[1:5] * 1.0
+    np.testing.assert_array_equal(y.numpy(), x.transpose(2, 1, 0)[1:5])
+    stats = last_plan().stats
+    assert stats.get("copy", 0) == 0, stats  # permute + slice became strides of one kernel
+    z = nb.reshape(nb.permute(T(x), (1, 0, 2)), (6, 32))  # needs one materialisation
+    np.testing.assert_array_equal(z.numpy(), x.transpose(1, 0, 2).reshape(6, 32))
+    b = nb.broadcast_to(nb.unsqueeze(T(x[0, 0]), 0), (5, 8)) + 0.0
+    np.testing.assert_array_equal(b.numpy(), np.broadcast_to(x[0, 0], (5, 8)))
+    np.testing.assert_array_equal(nb.squeeze(nb.unsqueeze(T(x), 1), 1).numpy(), x)
+    np.testing.assert_array_equal(nb.flatten(T(x), 1).numpy(), x.reshape(4, 48))
+    np.testing.assert_array_equal(nb.moveaxis(T(x), 0, 2).numpy(), np.moveaxis(x, 0, 2))
+    np.testing.assert_array_equal(nb.stack([T(x), T(x)], axis=1).numpy(), np.stack([x, x], 1))
+    np.testing.assert_array_equal(
+        nb.slice_update(T(x), T(np.zeros((2, 6, 3), np.float32)), (1, 0, 2), (2, 6, 3)).numpy(),
+        np.concatenate([x[:, :, :2], np.where(np.isin(np.arange(4), [1, 2])[:, None, None],
+                                               0, x[:, :, 2:5]), x[:, :, 5:]], 2))
+
+
+def test_creation_ops(emulator):
+    np.testing.assert_array_equal(nb.zeros((2, 3)).numpy(), np.zeros((2, 3), np.float32))
+    np.testing.assert_array_equal(nb.full((4,), 2.5).numpy(), np.full(4, 2.5, np.float32))
+    np.testing.assert_array_equal(nb.arange(0, 7, dtype=nb.DType.int64).numpy(), np.arange(7))
+    np.testing.assert_array_equal(nb.arange(1, 4, 0.5).numpy(), np.arange(1, 4, 0.5, dtype=np.float32))
+    x = RNG.standard_normal((2, 5, 5)).astype(np.float32)
+    np.testing.assert_array_equal(nb.tril(T(x)).numpy(), np.tril(x))
+    np.testing.assert_array_equal(nb.triu(T(x), 1).numpy(), np.triu(x, 1))
+    np.testing.assert_array_equal(nb.ones_like(T(x)).numpy(), np.ones_like(x))
+
+
+def test_matmul_promotion_rules(emulator):
+    a = RNG.standard_normal((5, 4)).astype(np.float32)
+    b = RNG.standard_normal((4, 3)).astype(np.float32)
+    v = RNG.standard_normal((4,)).astype(np.float32)
+    np.testing.assert_allclose((T(a) @ T(b)).numpy(), a @ b, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose((T(a) @ T(v)).numpy(), a @ v, rtol=1e-5, atol=1e-6)      # 1-D rhs
+    np.testing.assert_allclose((T(v) @ T(b)).numpy(), v @ b, rtol=1e-5, atol=1e-6)      # 1-D lhs
+    batched = RNG.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    np.testing.assert_allclose((T(batched) @ T(b)).numpy(), batched @ b, rtol=1e-5, atol=1e-6)  # batch broadcast
+    with pytest.raises(ValueError):
+        T(a) @ T(a)
+
+
+# ---- autodiff -------------------------------------------------------------------------
+def test_grad_value_and_grad_vjp_agree_with_oracle(emulator):
+    x = RNG.standard_normal((4, 6)).astype(np.float32)
+    w = RNG.standard_normal((6, 3)).astype(np.float32)
+
+    def f(x, w):
+        return nb.mean(nb.tanh(x @ w) * nb.sigmoid(x @ w))
+
+    vx, vw = O.V(x.astype(np.float64)), O.V(w.astype(np.float64))
+    h = O.matmul(vx, vw)
+    ref_loss = O.mean(O.tanh(h) * (O.V(1.0) / (O.exp(O.neg(h)) + 1.0)))
+    gx_ref, gw_ref = O.grad_of(ref_loss, [vx, vw])
+    g = nb.grad(f, argnums=(0, 1))(T(x), T(w))
+    assert relerr(g[0].numpy(), gx_ref) < 1e-5 and relerr(g[1].numpy(), gw_ref) < 1e-5
+    val, g1 = nb.value_and_grad(f, argnums=1)(T(x), T(w))
+    assert abs(val.item() - float(ref_loss.a)) < 1e-6
+    assert relerr(g1.numpy(), gw_ref) < 1e-5
+    out, pullback = nb.vjp(f, T(x), T(w))
+    gx2, gw2 = pullback(nb.ones_like(out))
+    assert relerr(gx2.numpy(), gx_ref) < 1e-5 and relerr(gw2.numpy(), gw_ref) < 1e-5
+
+
+def test_grad_stays_lazy_and_unreached_inputs_get_zeros(emulator):
+    x, y = T(np.ones((3,), np.float32)), T(np.ones((3,), np.float32))
+    gx, gy = nb.grad(lambda a, b: nb.reduce_sum(a * 2.0), argnums=(0, 1))(x, y)
+    assert not gx.real  # create_graph=True keeps results lazy (grad.py:23-25)
+    np.testing.assert_array_equal(gx.numpy(), np.full(3, 2.0, np.float32))
+    np.testing.assert_array_equal(gy.numpy(), np.zeros(3, np.float32))
+
+
+def test_pytorch_style_backward_accumulates(emulator):
+    w = T(RNG.standard_normal((4, 2)).astype(np.float32)).requires_grad_(True)
+    x = T(RNG.standard_normal((3, 4)).astype(np.float32))
+    loss = nb.mean((x @ w) * (x @ w))
+    loss.backward()
+    g1 = w.grad.numpy().copy()
+    ref = 2 * x.numpy().T @ (x.numpy() @ w.numpy()) / 6
+    np.testing.assert_allclose(g1, ref, rtol=1e-5, atol=1e-6)
+    nb.mean((x @ w) * (x @ w)).backward()
+    np.testing.assert_allclose(w.grad.numpy(), 2 * g1, rtol=1e-5, atol=1e-6)
+
+
+def test_second_order_through_create_graph(emulator):
+    x = T(np.array([0.3, -1.2, 2.0], np.float32))
+    f = lambda t: nb.reduce_sum(t * t * t)
+    gg = nb.grad(lambda t: nb.reduce_sum(nb.grad(f)(t)))(x)
+    np.testing.assert_allclose(gg.numpy(), 6 * x.numpy(), rtol=1e-5)
+
+
+def test_vjp_error_is_wrapped(emulator):
+    class Broken(nb.UnaryOperation):
+        @property
+        def name(self):
+            return "broken"
+
+        def kernel(self, args, kwargs):
+            from nabla_amd.backend import ir
+            return [ir.ew("mov", args[0])]
+
+    with pytest.raises(RuntimeError, match="VJP rule failed for operation 'broken'"):
+        nb.grad(lambda t: nb.reduce_sum(Broken()([t], {})[0]))(T(np.ones(2, np.float32)))
+
+
+# ---- fusion structure ---------------------------------------------------------------------
+def test_layernorm_softmax_forward_is_one_kernel(emulator):
+    x = RNG.standard_normal((8, 64)).astype(np.float32)
+    w, b = np.ones(64, np.float32), np.zeros(64, np.float32)
+    y = nb.softmax(F.layer_norm(T(x), T(w), T(b)), axis=-1)
+    ref = O.softmax(O.layer_norm(O.V(x.astype(np.float64)), O.V(w), O.V(b))).a
+    assert relerr(y.numpy(), ref) < 1e-5
+    stats = last_plan().stats
+    assert stats["rowprog"] == 1 and stats["steps"] == 1, stats
+
+
+def test_forward_traced_twice_is_computed_once(emulator):
+    x = T(RNG.standard_normal((16, 128)).astype(np.float32))
+    y = T(RNG.standard_normal((16, 128)).astype(np.float32))
+    out, gx = nb.workloads.c2_step(x, y)
+    nb.realize_all(out, gx)
+    plan = last_plan()
+    progs = [s for s in plan.steps if s.kind == "rowprog"]
+    assert len(progs) == 1, plan.stats
+    n_exp = sum(1 for i in progs[0].attrs["members"] if i == "ew.exp")
+    assert n_exp == 1  # common-subexpression elimination merged the two traces
+
+
+def test_plan_cache_is_structural_not_by_value(emulator):
+    from nabla_amd.core.engine import clear_plan_cache, get_cache_stats
+    clear_plan_cache()
+    for k in range(3):
+        a = T(RNG.standard_normal((4, 4)).astype(np.float32))
+        (nb.relu(a) * float(k + 1)).numpy()
+    st = get_cache_stats()
+    assert st["misses"] == 1 and st["hits"] == 2, st
+    (nb.relu(T(np.ones((5, 4), np.float32))) * 2.0).numpy()  # another shape: new plan
+    assert get_cache_stats()["misses"] == 2
+    # x*x and x*y have different structure even with equal shapes
+    a = T(np.full((4, 4), 3.0, np.float32))
+    b = T(np.full((4, 4), 5.0, np.float32))
+    np.testing.assert_array_equal((a * a).numpy(), np.full((4, 4), 9.0, np.float32))
+    np.testing.assert_array_equal((a * b).numpy(), np.full((4, 4), 15.0, np.float32))
+
+
+# ---- compile (behavioural spec: reference tests/unit/test_compile.py:18-77) --------------------
+def test_compile_basic_hits_and_misses(emulator):
+    @nb.compile
+    def f(x):
+        return x * 2.0 + 1.0
+
+    x_np = np.array([1.0, 2.0, 3.0], dtype=np.float32)
+    x = nb.Tensor.constant(x_np)
+    np.testing.assert_allclose(f(x).to_numpy(), x_np * 2.0 + 1.0)
+    assert f.stats.misses == 1 and f.stats.hits == 0
+    np.testing.assert_allclose(f(x).to_numpy(), x_np * 2.0 + 1.0)
+    assert f.stats.misses == 1 and f.stats.hits == 1
+    np.testing.assert_allclose(f(T(x_np + 5)).to_numpy(), (x_np + 5) * 2.0 + 1.0)  # new values, same plan
+    assert f.stats.hits == 2
+
+
+def test_compile_dynamic_dims_reuse_signature(emulator):
+    @nb.compile(dynamic_dims={0: {0: "batch"}})
+    def f(x, w):
+        return x @ w
+
+    w_np = RNG.standard_normal((4, 3)).astype(np.float32)
+    x1 = RNG.standard_normal((2, 4)).astype(np.float32)
+    x2 = RNG.standard_normal((5, 4)).astype(np.float32)
+    w = T(w_np)
+    np.testing.assert_allclose(f(T(x1), w).to_numpy(), x1 @ w_np, atol=1e-5)
+    assert f.stats.misses == 1
+    f(T(x1), w)
+    assert f.stats.hits == 1
+    np.testing.assert_allclose(f(T(x2), w).to_numpy(), x2 @ w_np, atol=1e-5)
+    assert f.stats.hits == 2 and f.stats.misses == 1  # a new batch size is not a new signature
+
+
+def test_compile_train_step_with_pytrees_and_closures(emulator):
+    scale = T(np.float32(0.5))
+
+    @nb.compile
+    def step(params, x):
+        loss, g = nb.value_and_grad(lambda p, x: nb.mean((x @ p["w"] + p["b"]) ** 2.0) * scale)(params, x)
+        return loss, {k: params[k] - g[k] * 0.1 for k in params}
+
+    p = {"w": T(RNG.standard_normal((4, 2)).astype(np.float32)), "b": T(np.zeros((1, 2), np.float32))}
+    x = T(RNG.standard_normal((8, 4)).astype(np.float32))
+    l0, p1 = step(p, x)
+    l1, p2 = step(p1, x)
+    l2, _ = step(p2, x)
+    assert step.stats.misses == 1 and step.stats.hits == 2
+    assert l2.item() < l1.item() < l0.item()
+
+
+# ---- nn modules ----------------------------------------------------------------------------
+def test_modules_are_pytrees_and_track_parameters(emulator):
+    nn = nb.nn
+    nn.functional.manual_seed(0)
+    layer = nn.TransformerEncoderLayer(16, 4, dim_feedforward=32, dropout=0.0)
+    names = [n for n, _ in layer.named_parameters()]
+    assert "self_attn.q_proj.weight" in names and "norm2.bias" in names and len(names) == 16
+    leaves, treedef = nb.tree_flatten(layer)
+    rebuilt = nb.tree_unflatten(treedef, leaves)
+    x = T(RNG.standard_normal((2, 5, 16)).astype(np.float32))
+    np.testing.assert_allclose(rebuilt(x, is_causal=True).numpy(), layer(x, is_causal=True).numpy())
+    lin = nn.Linear(3, 2)
+    assert lin.weight.shape == (3, 2) and lin.bias.shape == (1, 2)  # (in, out) and (1, out)
+    sd = lin.state_dict()
+    lin2 = nn.Linear(3, 2)
+    lin2.load_state_dict(sd)
+    np.testing.assert_array_equal(lin2.weight.numpy(), lin.weight.numpy())
+
+
+def test_module_forward_matches_oracle_block(emulator):
+    t = oc.c3_inputs(2, 8, 16, 32, seed=3, bf16=False)
+    want, _ = oc.c3_reference(t, num_heads=4)
+    nn = nb.nn
+    layer = nn.TransformerEncoderLayer(16, 4, dim_feedforward=32, dropout=0.0)
+    sd = {"self_attn.q_proj.weight": "wq", "self_attn.q_proj.bias": "bq", "self_attn.k_proj.weight": "wk",
+          "self_attn.k_proj.bias": "bk", "self_attn.v_proj.weight": "wv", "self_attn.v_proj.bias": "bv",
+          "self_attn.out_proj.weight": "wo", "self_attn.out_proj.bias": "bo", "linear1.weight": "w1",
+          "linear1.bias": "b1", "linear2.weight": "w2", "linear2.bias": "b2", "norm1.weight": "ln1_w",
+          "norm1.bias": "ln1_b", "norm2.weight": "ln2_w", "norm2.bias": "ln2_b"}
+    layer.load_state_dict({k: T(t[v]) for k, v in sd.items()})
+    out = layer(T(t["x"]), is_causal=True)
+    assert abs(nb.mean(out * out).item() - want) < 1e-5 * abs(want)
+
+
+# ---- whole configurations at reduced size -----------------------------------------------------
+def test_configs_reduced_against_oracle(emulator):
+    t = oc.c3_inputs(2, 16, 32, 64, seed=0, bf16=False)
+    wl, wg = oc.c3_reference(t, num_heads=4)
+    loss, grads = oc.c3_program(nb, oc.upload(nb, t), num_heads=4)
+    nb.realize_all(loss, *grads.values())
+    assert abs(loss.item() - wl) < 1e-5 * abs(wl)
+    scale = max(np.abs(g).max() for g in wg.values())
+    for k in oc.C3_PARAMS:
+        assert np.abs(grads[k].numpy() - wg[k]).max() <= 2e-5 * max(np.abs(wg[k]).max(), 1e-3 * scale), k
+
+    t = oc.c4_inputs(batch=4, hw=8, c=(3, 8, 16, 32), seed=0)
+    wl, wg, wam, _ = oc.c4_reference(t)
+    T4 = oc.upload(nb, t)
+    loss, grads = oc.c4_program(nb, T4)
+    am = nb.argmax(oc.c4_logits(nb, {k: T4[k] for k in oc.C4_PARAMS}, T4["img"]), axis=-1)
+    nb.realize_all(loss, am, *grads.values())
+    assert abs(loss.item() - wl) < 1e-5 * abs(wl)
+    np.testing.assert_array_equal(am.numpy(), wam)
+    for k in oc.C4_PARAMS:
+        assert relerr(grads[k].numpy(), wg[k]) < 2e-5, k
+
+    t = oc.c5_inputs(layers=2, batch=2, seq=8, d_model=32, d_ff=64, vocab=50, rank=4, seed=0,
+                     b_zero=False, bf16=False)
+    wl, wg = oc.c5_reference(t, num_heads=4)
+    loss, grads = oc.c5_program(nb, oc.upload(nb, t), num_heads=4)
+    flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
+    nb.realize_all(loss, *flat)
+    assert abs(loss.item() - wl) < 1e-5 * abs(wl)
+    for g, w in zip(flat, wg):
+        assert relerr(g.numpy(), w) < 2e-5
+
+
+# ---- validation messages the reference tests match on --------------------------------------------
+def test_conv_and_pool_validation(emulator):
+    x = T(np.zeros((1, 4, 4, 2), np.float32))
+    w = T(np.zeros((3, 3, 2, 2), np.float32))
+    with pytest.raises(ValueError, match="stride values must be > 0"):
+        nb.conv2d(x, w, stride=(0, 1))
+    with pytest.raises(ValueError, match="dilation"):
+        nb.conv2d(x, w, dilation=(2, 2))
+    with pytest.raises(ValueError, match="grouped mode"):
+        nb.conv2d(x, w, groups=2)
+    with pytest.raises(ValueError, match="padding values must be >= 0"):
+        nb.conv2d(x, w, padding=-1)
+    with pytest.raises(ValueError, match="Input channels"):
+        nb.conv2d(x, T(np.zeros((3, 3, 3, 2), np.float32)))
+    with pytest.raises(ValueError, match="Non-positive pool2d output size"):
+        nb.max_pool2d(x, kernel_size=9)
+    with pytest.raises(ValueError, match="Cannot broadcast"):
+        T(np.zeros((2, 3), np.float32)) + T(np.zeros((4,), np.float32))
+
+
+def test_context_isolation_of_flags():
+    """Flags are ContextVars: a change inside a copied context does not leak."""
+    import contextvars
+    from nabla_amd import config
+
+    def inner():
+        config.set_flag("EAGER_MAX_GRAPH", True)
+        return config.EAGER_MAX_GRAPH
+
+    assert contextvars.copy_context().run(inner) is True
+    assert config.EAGER_MAX_GRAPH is False

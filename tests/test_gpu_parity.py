@@ -1,0 +1,355 @@
+"""GPU parity: the HIP path against the CPU oracle on the five benchmark
+configurations (reduced sizes), full-size spot checks, the specialised row
+kernels against the interpreter, data-movement / index kernels on awkward
+shapes, user kernels, and ``compile`` on the device.
+
+Tolerances: 1e-5 relative for fp32 work (2e-5 where a long fp32 accumulation
+sits between input and output), 2e-2 for bf16, exact for integer results.
+"""
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import nabla_amd as nb
+from oracle import configs as oc
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 2e-5
+BF16_TOL = 2e-2
+
+
+def T(a, dtype=None):
+    return nb.Tensor.constant(a, dtype=dtype)
+
+
+def relerr(got, want, floor=0.0):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    return np.abs(got - want).max() / max(np.abs(want).max(), floor, 1e-30)
+
+
+# ---- C1 ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,d_in,d_hidden,d_out", [(128, 784, 256, 10), (7, 33, 19, 3), (1, 8, 8, 1)])
+def test_c1_mlp_step(hip, batch, d_in, d_hidden, d_out):
+    t = oc.c1_inputs(batch, d_in, d_hidden, d_out, seed=4)
+    t["b1"] = np.random.default_rng(1).uniform(-0.05, 0.05, t["b1"].shape).astype(np.float32)
+    wl, wg = oc.c1_reference(**t)
+    loss, grads = oc.c1_program(nb, oc.upload(nb, t))
+    nb.realize_all(loss, *grads)
+    assert abs(loss.item() - wl) <= F32_TOL * abs(wl) + 1e-9
+    for g, w in zip(grads, wg):
+        assert g.shape == w.shape
+        assert relerr(g.numpy(), w) < F32_TOL
+
+
+# ---- C2 ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,cols", [(64, 512), (33, 1000), (5, 4108), (16, 8192), (3, 20000), (1, 1)])
+def test_c2_chain_reduced(hip, rows, cols):
+    t = oc.c2_inputs(rows, cols, seed=rows)
+    wo, wg = oc.c2_reference(t["x"], t["y"])
+    out, gx = oc.c2_program(nb, T(t["x"]), T(t["y"]))
+    nb.realize_all(out, gx)
+    assert relerr(out.numpy(), wo) < F32_TOL
+    assert relerr(gx.numpy(), wg) < F32_TOL
+
+
+def test_c2_full_size_rows_against_oracle(hip):
+    """8192 x 8192 on the device; the oracle recomputes a sample of rows (rows are independent)."""
+    t = oc.c2_inputs(8192, 8192, seed=0)
+    out, gx = oc.c2_program(nb, T(t["x"]), T(t["y"]))
+    nb.realize_all(out, gx)
+    o, g = out.numpy(), gx.numpy()
+    assert np.isfinite(o).all() and np.isfinite(g).all()
+    rows = np.random.default_rng(0).choice(8192, 24, replace=False)
+    rows = np.concatenate([rows, [0, 8191]])
+    wo, wg = oc.c2_reference(t["x"][rows], t["y"][rows])
+    assert relerr(o[rows], wo) < F32_TOL
+    assert relerr(g[rows], wg) < F32_TOL
+    # structure that holds for every row: the gradient vanishes exactly where relu(x) is flat
+    # and p = x*y stays below the row maximum, and out >= 0
+    assert (o >= 0).all()
+
+
+def test_specialised_kernels_match_interpreter(hip):
+    """The ahead-of-time row kernels and the interpreter run the same program:
+    same operation order per element, so results agree to the last bit for the
+    elementwise part and to reduction-order noise for sums."""
+    from nabla_amd.backend import lib
+    from nabla_amd.core import engine
+    t = oc.c2_inputs(8192, 8192, seed=1)
+    X, Y = T(t["x"]), T(t["y"])
+
+    engine.clear_plan_cache()
+    hip.force_interpreter = False
+    out_s, gx_s = oc.c2_program(nb, X, Y)
+    nb.realize_all(out_s, gx_s)
+    L = lib.load()
+    n_spec = 0
+    for bound in engine._PLAN_CACHE.values():
+        for call in bound.calls:
+            if call[0] is L.nbk_rowprog_launch:
+                n_spec += int(L.nbk_rowprog_is_specialized(C.byref(call[3])))
+    assert n_spec >= 1, "the full-size C2 program must hit a specialised kernel"
+
+    engine.clear_plan_cache()
+    hip.force_interpreter = True
+    try:
+        out_i, gx_i = oc.c2_program(nb, X, Y)
+        nb.realize_all(out_i, gx_i)
+    finally:
+        hip.force_interpreter = False
+        engine.clear_plan_cache()
+    np.testing.assert_allclose(out_s.numpy(), out_i.numpy(), rtol=2e-6, atol=0)
+    np.testing.assert_allclose(gx_s.numpy(), gx_i.numpy(), rtol=2e-6, atol=1e-30)
+
+
+# ---- C3 ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape,heads", [((2, 16, 32, 64), 4), ((2, 128, 256, 512), 4), ((1, 72, 64, 96), 2)])
+def test_c3_block_fp32(hip, shape, heads):
+    t = oc.c3_inputs(*shape, seed=0, bf16=False)
+    wl, wg = oc.c3_reference(t, num_heads=heads)
+    loss, grads = oc.c3_program(nb, oc.upload(nb, t), num_heads=heads)
+    nb.realize_all(loss, *grads.values())
+    assert abs(loss.item() - wl) < F32_TOL * abs(wl)
+    scale = max(np.abs(g).max() for g in wg.values())
+    for k in oc.C3_PARAMS:
+        # bk's true gradient is zero (softmax is shift invariant): compare on the common scale
+        assert relerr(grads[k].numpy(), wg[k], floor=1e-3 * scale) < 5e-5, k
+
+
+def test_c3_block_bf16(hip):
+    t = oc.c3_inputs(2, 128, 256, 512, seed=1, bf16=True)
+    wl, wg = oc.c3_reference(t, num_heads=4)
+    loss, grads = oc.c3_program(nb, oc.upload(nb, t, dtype=nb.DType.bfloat16), num_heads=4)
+    nb.realize_all(loss, *grads.values())
+    assert loss.dtype == nb.DType.bfloat16
+    assert abs(loss.item() - wl) < BF16_TOL * abs(wl)
+    scale = max(np.abs(g).max() for g in wg.values())
+    for k in oc.C3_PARAMS:
+        assert grads[k].dtype == nb.DType.bfloat16
+        assert relerr(grads[k].numpy(), wg[k], floor=0.05 * scale) < BF16_TOL, k
+
+
+# ---- C4 ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,hw,c", [(4, 8, (3, 8, 16, 32)), (3, 16, (3, 20, 24, 40)), (8, 32, (3, 64, 128, 256))])
+def test_c4_cnn_step(hip, batch, hw, c):
+    t = oc.c4_inputs(batch=batch, hw=hw, c=c, seed=2)
+    wl, wg, wam, wlogits = oc.c4_reference(t)
+    T4 = oc.upload(nb, t)
+    loss, grads = oc.c4_program(nb, T4)
+    logits = oc.c4_logits(nb, {k: T4[k] for k in oc.C4_PARAMS}, T4["img"])
+    am = nb.argmax(logits, axis=-1)
+    nb.realize_all(loss, am, logits, *grads.values())
+    assert abs(loss.item() - wl) < F32_TOL * abs(wl)
+    assert relerr(logits.numpy(), wlogits) < F32_TOL
+    # the arg-max is an index: exact unless the top two logits tie within fp32 noise
+    top2 = np.sort(wlogits, axis=-1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 1e-4 * np.abs(top2[:, 1])
+    np.testing.assert_array_equal(am.numpy()[clear], wam[clear])
+    for k in oc.C4_PARAMS:
+        assert relerr(grads[k].numpy(), wg[k]) < 5e-5, k
+
+
+# ---- C5 ------------------------------------------------------------------------------------------
+def test_c5_lora_fp32(hip):
+    t = oc.c5_inputs(layers=2, batch=2, seq=16, d_model=64, d_ff=128, vocab=97, rank=4, seed=0,
+                     b_zero=False, bf16=False)
+    wl, wg = oc.c5_reference(t, num_heads=4)
+    loss, grads = oc.c5_program(nb, oc.upload(nb, t), num_heads=4)
+    flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
+    nb.realize_all(loss, *flat)
+    assert abs(loss.item() - wl) < F32_TOL * abs(wl)
+    for g, w in zip(flat, wg):
+        assert relerr(g.numpy(), w) < 5e-5
+
+
+def test_c5_lora_bf16(hip):
+    t = oc.c5_inputs(layers=2, batch=2, seq=64, d_model=128, d_ff=256, vocab=300, rank=8, seed=3,
+                     b_zero=False, bf16=True)
+    wl, wg = oc.c5_reference(t, num_heads=4)
+    loss, grads = oc.c5_program(nb, oc.upload(nb, t, dtype=nb.DType.bfloat16), num_heads=4)
+    flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
+    nb.realize_all(loss, *flat)
+    assert abs(loss.item() - wl) < BF16_TOL * abs(wl)
+    scale = max(np.abs(w).max() for w in wg)
+    for g, w in zip(flat, wg):
+        assert relerr(g.numpy(), w, floor=0.05 * scale) < 2 * BF16_TOL
+
+
+# ---- movement, reductions and index kernels on awkward shapes ------------------------------------
+@pytest.mark.parametrize("shape,perm", [((5, 7), (1, 0)), ((64, 96), (1, 0)), ((3, 33, 65), (2, 0, 1)),
+                                        ((2, 4, 130, 64), (0, 2, 1, 3)), ((2, 3, 4, 5, 6), (4, 2, 0, 3, 1)),
+                                        ((1, 1000), (1, 0))])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "i32"])
+def test_permute_copy_exact(hip, shape, perm, dtype):
+    rng = np.random.default_rng(5)
+    if dtype == "i32":
+        a = rng.integers(-2 ** 31, 2 ** 31 - 1, shape).astype(np.int32)
+        x = T(a)
+    elif dtype == "bf16":
+        a = oc.to_bf16_grid(rng.standard_normal(shape).astype(np.float32))
+        x = T(a, dtype=nb.DType.bfloat16)
+    else:
+        a = rng.standard_normal(shape).astype(np.float32)
+        x = T(a)
+    # the trailing add forces a materialised copy in the permuted order
+    y = nb.reshape(nb.permute(x, perm), (-1,))
+    y.realize()
+    np.testing.assert_array_equal(y.numpy(), np.transpose(a, perm).reshape(-1))
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 5, 6), 0), ((4, 5, 6), 1), ((2, 300, 7), 1), ((1000, 3), 0),
+                                        ((8, 1, 16), 1), ((3, 4097), 1), ((70000,), 0), ((2, 3, 4, 5), 2)])
+@pytest.mark.parametrize("kind", ["sum", "max", "min", "mean"])
+def test_axis_reductions(hip, shape, axis, kind):
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal(shape).astype(np.float32)
+    fn = {"sum": nb.reduce_sum, "max": nb.reduce_max, "min": nb.reduce_min, "mean": nb.mean}[kind]
+    want = {"sum": np.sum, "max": np.max, "min": np.min, "mean": np.mean}[kind](a.astype(np.float64), axis=axis)
+    got = fn(T(a), axis=axis).numpy()
+    assert got.shape == want.shape
+    if kind in ("max", "min"):
+        np.testing.assert_array_equal(got, want.astype(np.float32))
+    else:
+        absum = np.abs(a).astype(np.float64).sum(axis=axis) / (a.shape[axis] if kind == "mean" else 1)
+        assert (np.abs(got - want) <= 1e-6 * absum + 1e-30).all()
+
+
+def test_argmax_ties_and_nan(hip):
+    a = np.zeros((6, 300), np.float32)
+    a[0, [5, 9, 250]] = 3.0          # first maximum wins
+    a[1, :] = -1.0                   # all equal -> 0
+    a[2, 299] = 1.0
+    a[3, 17] = np.inf
+    a[4, [100, 200]] = [2.0, np.nan]  # NaN counts as the maximum, as in numpy/torch
+    a[5, 0] = -np.inf
+    got = nb.argmax(T(a), axis=-1).numpy()
+    np.testing.assert_array_equal(got, torch.from_numpy(a).argmax(-1).numpy())
+    got0 = nb.argmax(T(a), axis=0).numpy()
+    np.testing.assert_array_equal(got0, torch.from_numpy(a).argmax(0).numpy())
+    assert got.dtype == np.int64
+
+
+def test_gather_rows_and_out_of_range(hip):
+    rng = np.random.default_rng(7)
+    table = rng.standard_normal((50, 24)).astype(np.float32)
+    idx = rng.integers(0, 50, (3, 11)).astype(np.int64)
+    got = nb.gather(T(table), T(idx), axis=0).numpy()
+    np.testing.assert_array_equal(got, table[idx])
+    idx32 = idx.astype(np.int32)
+    np.testing.assert_array_equal(nb.gather(T(table), T(idx32), axis=0).numpy(), table[idx32])
+    bad = idx.copy()
+    bad[1, 2] = 50
+    with pytest.raises(IndexError):
+        nb.gather(T(table), T(bad), axis=0).numpy()
+    # the flag is cleared by the failed call
+    np.testing.assert_array_equal(nb.gather(T(table), T(idx), axis=0).numpy(), table[idx])
+
+
+def test_integer_and_bool_elementwise_exact(hip):
+    rng = np.random.default_rng(8)
+    a = rng.integers(-1000, 1000, (17, 129)).astype(np.int32)
+    b = rng.integers(-1000, 1000, (17, 129)).astype(np.int32)
+    np.testing.assert_array_equal((T(a) + T(b)).numpy(), a + b)
+    np.testing.assert_array_equal((T(a) * T(b)).numpy(), a * b)
+    np.testing.assert_array_equal(nb.greater(T(a), T(b)).numpy(), a > b)
+    np.testing.assert_array_equal(nb.where(nb.greater(T(a), T(b)), T(a), T(b)).numpy(), np.maximum(a, b))
+    np.testing.assert_array_equal(nb.reduce_sum(T(a), axis=1).numpy(), a.sum(1))
+
+
+def test_slice_pad_concat_exact(hip):
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((6, 10, 12)).astype(np.float32)
+    b = rng.standard_normal((6, 3, 12)).astype(np.float32)
+    x, y = T(a), T(b)
+    np.testing.assert_array_equal(x[1:5, ::1, 2:9].numpy(), a[1:5, :, 2:9])
+    np.testing.assert_array_equal(nb.concatenate([x, y], axis=1).numpy(), np.concatenate([a, b], 1))
+    g = nb.grad(lambda x: nb.reduce_sum(x[1:5, 2:4, 3:8] * 2.0))(x)
+    want = np.zeros_like(a)
+    want[1:5, 2:4, 3:8] = 2.0
+    np.testing.assert_array_equal(g.numpy(), want)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(n=2, h=9, w=11, ci=3, co=5, k=3, stride=(1, 1), pad=(1, 1, 1, 1), dil=(1, 1)),
+    dict(n=1, h=12, w=12, ci=4, co=6, k=3, stride=(2, 2), pad=(0, 1, 2, 0), dil=(1, 1)),
+    dict(n=2, h=14, w=10, ci=2, co=4, k=3, stride=(1, 2), pad=(2, 2, 2, 2), dil=(1, 1)),
+    dict(n=3, h=8, w=8, ci=16, co=8, k=1, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1)),
+])
+def test_conv2d_forward_and_grads(hip, cfg):
+    from oracle import ops as O
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((cfg["n"], cfg["h"], cfg["w"], cfg["ci"])).astype(np.float32)
+    w = rng.standard_normal((cfg["k"], cfg["k"], cfg["ci"], cfg["co"])).astype(np.float32)
+    kw = dict(stride=cfg["stride"], padding=cfg["pad"])
+    X, W = O.V(x.astype(np.float64)), O.V(w.astype(np.float64))
+    out = O.conv2d(X, W, **kw)
+    wgx, wgw = O.grad_of(O.reduce_sum(out * out), [X, W])
+    f = lambda x, w: nb.reduce_sum(nb.conv2d(x, w, **kw) ** 2)
+    got = nb.conv2d(T(x), T(w), **kw)
+    gx, gw = nb.grad(f, argnums=(0, 1))(T(x), T(w))
+    assert relerr(got.numpy(), out.a) < F32_TOL
+    assert relerr(gx.numpy(), wgx) < 5e-5
+    assert relerr(gw.numpy(), wgw) < 5e-5
+
+
+# ---- user kernels ---------------------------------------------------------------------------------
+class AddOneCustomOp(nb.ops.UnaryOperation):
+    """Same shape as the reference's example op (tests/mojo/op.py:15-27)."""
+
+    @property
+    def name(self) -> str:
+        return "my_kernel"
+
+    def kernel(self, args, kwargs):
+        kernel_dir = Path(__file__).parent / "custom_kernels"
+        x = args[0]
+        return [nb.ops.call_custom_kernel("my_kernel", kernel_dir, x, x.type)]
+
+
+def test_custom_kernel_op(hip):
+    a = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    y = AddOneCustomOp()([T(a)], {})[0]
+    np.testing.assert_array_equal(y.numpy(), a + 1)
+    # composes with built-in ops inside one graph
+    z = nb.reduce_sum(AddOneCustomOp()([T(a) * 2.0], {})[0], axis=-1)
+    np.testing.assert_array_equal(z.numpy(), (a * 2 + 1).sum(-1))
+
+
+def test_custom_kernel_missing_library_is_an_error(hip):
+    class Broken(AddOneCustomOp):
+        def kernel(self, args, kwargs):
+            return [nb.ops.call_custom_kernel("nope", Path(__file__).parent / "golden", args[0], args[0].type)]
+
+    with pytest.raises(FileNotFoundError):
+        Broken()([T(np.zeros(4, np.float32))], {})[0].numpy()
+
+
+# ---- compile --------------------------------------------------------------------------------------
+def test_compiled_train_step_on_device(hip):
+    t = oc.c1_inputs(32, 48, 24, 5, seed=11)
+    params = {k: T(t[k]) for k in ("W1", "b1", "W2", "b2")}
+    x = T(t["x"])
+
+    def step(params, x):
+        def loss_fn(p):
+            return nb.mean(nb.relu(x @ p["W1"] + p["b1"]) @ p["W2"] + p["b2"])
+        loss, g = nb.value_and_grad(loss_fn)(params)
+        return loss, {k: params[k] - 0.1 * g[k] for k in params}
+
+    cstep = nb.compile(step)
+    ref = {k: t[k].astype(np.float64) for k in params}
+    p = params
+    for _ in range(3):
+        loss, p = cstep(p, x)
+        wl, wg = oc.c1_reference(t["x"], *[ref[k].astype(np.float32) for k in ("W1", "b1", "W2", "b2")])
+        assert abs(loss.item() - wl) <= 5e-5 * abs(wl) + 1e-8
+        for k, g in zip(("W1", "b1", "W2", "b2"), wg):
+            ref[k] = ref[k] - 0.1 * g
+    assert cstep.stats.misses == 1 and cstep.stats.hits == 2
+    for k in params:
+        assert relerr(p[k].numpy(), ref[k]) < 5e-5

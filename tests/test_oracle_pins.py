@@ -1,0 +1,329 @@
+"""Pins of the CPU oracle (oracle/ops.py): before it may judge the HIP path it is
+itself checked against torch-CPU autograd in fp64, brute-force loops on tiny
+inputs, and closed forms / invariants, chosen so that a dropped term, a wrong
+sign or a transposed operand fails one of them."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as TF
+
+from oracle import configs as oc
+from oracle import ops as O
+
+RNG = np.random.default_rng(7)
+
+
+def _t(a):
+    return torch.tensor(a, dtype=torch.float64, requires_grad=True)
+
+
+def _close(a, b, tol=1e-10):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    assert a.shape == b.shape
+    assert np.abs(a - b).max() <= tol * (1 + np.abs(b).max()), np.abs(a - b).max()
+
+
+# ---- primitives vs torch autograd -----------------------------------------------
+@pytest.mark.parametrize("name,ofn,tfn", [
+    ("relu", O.relu, torch.relu), ("exp", O.exp, torch.exp), ("neg", O.neg, torch.neg),
+    ("tanh", O.tanh, torch.tanh), ("erf", O.erf, torch.erf),
+    ("gelu", O.gelu, lambda t: TF.gelu(t, approximate="none")),
+    ("rsqrt", lambda v: O.rsqrt(v * v + 1.0), lambda t: torch.rsqrt(t * t + 1.0)),
+    ("sqrt", lambda v: O.sqrt(v * v + 1.0), lambda t: torch.sqrt(t * t + 1.0)),
+    ("log", lambda v: O.log(v * v + 1.0), lambda t: torch.log(t * t + 1.0)),
+])
+def test_unary_value_and_vjp(name, ofn, tfn):
+    x = RNG.standard_normal((5, 7))
+    v = O.V(x)
+    out = ofn(v)
+    w = RNG.standard_normal(out.a.shape)
+    (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+    t = _t(x)
+    to = tfn(t)
+    (to * torch.tensor(w)).sum().backward()
+    _close(out.a, to.detach().numpy())
+    _close(g, t.grad.numpy())
+
+
+def test_binary_broadcast_vjps():
+    a, b = RNG.standard_normal((4, 1, 6)), RNG.standard_normal((3, 1)) + 3.0
+    for ofn, tfn in ((O.add, torch.add), (O.sub, torch.sub), (O.mul, torch.mul), (O.div, torch.div)):
+        va, vb = O.V(a), O.V(b)
+        out = ofn(va, vb)
+        w = RNG.standard_normal(out.a.shape)
+        ga, gb = O.grad_of(O.reduce_sum(out * w), [va, vb])
+        ta, tb = _t(a), _t(b)
+        (tfn(ta, tb) * torch.tensor(w)).sum().backward()
+        _close(out.a, tfn(ta, tb).detach().numpy())
+        _close(ga, ta.grad.numpy())
+        _close(gb, tb.grad.numpy())
+
+
+def test_matmul_brute_force_and_vjp():
+    a, b = RNG.standard_normal((2, 3, 4)), RNG.standard_normal((4, 5))
+    brute = np.zeros((2, 3, 5))
+    for n in range(2):
+        for i in range(3):
+            for j in range(5):
+                for k in range(4):
+                    brute[n, i, j] += a[n, i, k] * b[k, j]
+    va, vb = O.V(a), O.V(b)
+    out = O.matmul(va, vb)
+    _close(out.a, brute)
+    w = RNG.standard_normal(out.a.shape)
+    ga, gb = O.grad_of(O.reduce_sum(out * w), [va, vb])
+    ta, tb = _t(a), _t(b)
+    ((ta @ tb) * torch.tensor(w)).sum().backward()
+    _close(ga, ta.grad.numpy())
+    _close(gb, tb.grad.numpy())  # includes the sum over the broadcast batch axis
+    # a transposed operand must fail: the product is not symmetric
+    assert np.abs(out.a - np.matmul(a, b[:, ::-1])).max() > 1e-3
+
+
+def test_reductions_and_tie_rule():
+    x = RNG.standard_normal((3, 4, 5))
+    v = O.V(x)
+    _close(O.reduce_sum(v, axis=(0, 2)).a, x.sum(axis=(0, 2)))
+    _close(O.mean(v, axis=1, keepdims=True).a, x.mean(axis=1, keepdims=True))
+    _close(O.reduce_max(v, axis=-1).a, x.max(axis=-1))
+    (g,) = O.grad_of(O.reduce_sum(O.mean(v, axis=(1, 2))), [v])
+    _close(g, np.full_like(x, 1.0 / 20))
+    # ties: EVERY maximal element receives the full cotangent (reduction.py:219-230)
+    t = np.array([[1.0, 3.0, 3.0, 2.0], [5.0, 5.0, 5.0, 0.0]])
+    vt = O.V(t)
+    (gt,) = O.grad_of(O.reduce_sum(O.reduce_max(vt, axis=1) * np.array([2.0, 7.0])), [vt])
+    _close(gt, np.array([[0, 2, 2, 0], [7, 7, 7, 0]], dtype=float))
+    assert np.array_equal(O.argmax(vt, axis=1), np.array([1, 0]))  # lowest index wins
+
+
+def test_softmax_logsoftmax():
+    x = RNG.standard_normal((4, 9)) * 3
+    v = O.V(x)
+    s = O.softmax(v, axis=-1)
+    _close(s.a.sum(-1), np.ones(4))
+    _close(O.logsoftmax(v).a, np.log(s.a))
+    w = RNG.standard_normal((4, 9))
+    for ofn, tfn in ((O.softmax, torch.softmax), (O.logsoftmax, torch.log_softmax)):
+        (g,) = O.grad_of(O.reduce_sum(ofn(v, -1) * w), [v])
+        t = _t(x)
+        (tfn(t, -1) * torch.tensor(w)).sum().backward()
+        _close(g, t.grad.numpy())
+    # shift invariance of softmax
+    _close(O.softmax(O.V(x + 100.0)).a, s.a)
+
+
+def test_layer_norm_invariants_and_grads():
+    x, w, b = RNG.standard_normal((6, 16)), RNG.standard_normal(16), RNG.standard_normal(16)
+    y0 = O.layer_norm(O.V(x)).a
+    _close(y0.mean(-1), np.zeros(6), 1e-12)
+    assert np.abs(y0.var(-1) - 1.0).max() < 1e-4  # biased variance, eps 1e-5
+    vx, vw, vb = O.V(x), O.V(w), O.V(b)
+    out = O.layer_norm(vx, vw, vb)
+    c = RNG.standard_normal(out.a.shape)
+    gs = O.grad_of(O.reduce_sum(out * c), [vx, vw, vb])
+    tx, tw, tb = _t(x), _t(w), _t(b)
+    to = TF.layer_norm(tx, (16,), tw, tb, eps=1e-5)
+    (to * torch.tensor(c)).sum().backward()
+    _close(out.a, to.detach().numpy())
+    for g, t in zip(gs, (tx, tw, tb)):
+        _close(g, t.grad.numpy(), 1e-9)
+
+
+def test_attention_matches_manual_torch_causal_and_not():
+    q, k, v = (RNG.standard_normal((2, 3, 6, 4)) for _ in range(3))
+    for causal in (False, True):
+        vq, vk, vv = O.V(q), O.V(k), O.V(v)
+        out = O.scaled_dot_product_attention(vq, vk, vv, is_causal=causal)
+        tq, tk, tv = _t(q), _t(k), _t(v)
+        sc = tq @ tk.transpose(-1, -2) / math.sqrt(4)
+        if causal:
+            sc = sc.masked_fill(~torch.tril(torch.ones(6, 6, dtype=torch.bool)), float("-inf"))
+        to = torch.softmax(sc, -1) @ tv
+        _close(out.a, to.detach().numpy())
+        c = RNG.standard_normal(out.a.shape)
+        gs = O.grad_of(O.reduce_sum(out * c), [vq, vk, vv])
+        (to * torch.tensor(c)).sum().backward()
+        for g, t in zip(gs, (tq, tk, tv)):
+            _close(g, t.grad.numpy(), 1e-9)
+
+
+def test_conv2d_brute_force_and_torch():
+    x = RNG.standard_normal((2, 5, 6, 3))
+    w = RNG.standard_normal((3, 2, 3, 4))
+    bias = RNG.standard_normal(4)
+    stride, pad = (2, 1), (1, 0, 2, 1)
+    out = O.conv2d(O.V(x), O.V(w), O.V(bias), stride=stride, padding=pad)
+    xp = np.pad(x, ((0, 0), (1, 0), (2, 1), (0, 0)))
+    ho, wo = out.a.shape[1], out.a.shape[2]
+    brute = np.zeros_like(out.a)
+    for n in range(2):
+        for i in range(ho):
+            for j in range(wo):
+                for co in range(4):
+                    acc = bias[co]
+                    for r in range(3):
+                        for s in range(2):
+                            for c in range(3):
+                                acc += xp[n, i * 2 + r, j * 1 + s, c] * w[r, s, c, co]
+                    brute[n, i, j, co] = acc
+    _close(out.a, brute)
+    vx, vw, vb = O.V(x), O.V(w), O.V(bias)
+    o2 = O.conv2d(vx, vw, vb, stride=stride, padding=pad)
+    c = RNG.standard_normal(o2.a.shape)
+    gs = O.grad_of(O.reduce_sum(o2 * c), [vx, vw, vb])
+    tx, tw, tb = _t(x), _t(w), _t(bias)
+    to = TF.conv2d(TF.pad(tx.permute(0, 3, 1, 2), (2, 1, 1, 0)), tw.permute(3, 2, 0, 1), tb, stride=stride)
+    (to.permute(0, 2, 3, 1) * torch.tensor(c)).sum().backward()
+    for g, t in zip(gs, (tx, tw, tb)):
+        _close(g, t.grad.numpy(), 1e-9)
+
+
+def test_max_pool_window_clipping_and_ties():
+    x = RNG.standard_normal((2, 5, 5, 3))
+    out = O.max_pool2d(O.V(x), (3, 3), (2, 2), (1, 1, 1, 1))
+    to = TF.max_pool2d(torch.tensor(x).permute(0, 3, 1, 2), 3, 2, 1).permute(0, 2, 3, 1)
+    _close(out.a, to.numpy())
+    t = np.zeros((1, 2, 2, 1))
+    t[0, :, :, 0] = [[1.0, 1.0], [0.0, 1.0]]
+    vt = O.V(t)
+    (g,) = O.grad_of(O.reduce_sum(O.max_pool2d(vt, (2, 2)) * 5.0), [vt])
+    _close(g[0, :, :, 0], np.array([[5.0, 5.0], [0.0, 5.0]]))  # all three tied maxima
+
+
+def test_cross_entropy_divides_by_first_dim_only():
+    logits = RNG.standard_normal((2, 3, 5))
+    labels = RNG.integers(0, 5, (2, 3))
+    v = O.V(logits)
+    loss = O.cross_entropy_loss(v, labels)
+    t = _t(logits)
+    ref = TF.cross_entropy(t.reshape(-1, 5), torch.tensor(labels).reshape(-1), reduction="sum") / 2
+    _close(loss.a, ref.detach().numpy())
+    (g,) = O.grad_of(loss, [v])
+    ref.backward()
+    _close(g, t.grad.numpy())
+
+
+def test_lora_linear_and_gather():
+    x, w = RNG.standard_normal((3, 8)), RNG.standard_normal((8, 6))
+    A, B = RNG.standard_normal((8, 2)), RNG.standard_normal((2, 6))
+    vA, vB = O.V(A), O.V(B)
+    out = O.lora_linear(O.V(x), O.V(w), vA, vB, alpha=4.0)
+    _close(out.a, x @ w + x @ (A @ B) * 2.0)
+    c = RNG.standard_normal(out.a.shape)
+    gA, gB = O.grad_of(O.reduce_sum(out * c), [vA, vB])
+    tA, tB = _t(A), _t(B)
+    ((torch.tensor(x) @ torch.tensor(w) + torch.tensor(x) @ ((tA @ tB) * 2.0)) * torch.tensor(c)).sum().backward()
+    _close(gA, tA.grad.numpy())
+    _close(gB, tB.grad.numpy())
+    table = RNG.standard_normal((7, 3))
+    idx = np.array([[6, 0], [3, 3]])
+    assert np.array_equal(O.gather(O.V(table), O.V(idx)).a, table[idx])
+
+
+# ---- whole configurations vs torch autograd --------------------------------------
+def test_config_c1_against_torch():
+    inp = oc.c1_inputs(16, 24, 12, 5, seed=1)
+    loss, grads = oc.c1_reference(**inp)
+    ts = {k: _t(v) for k, v in inp.items()}
+    tl = (torch.relu(ts["x"] @ ts["W1"] + ts["b1"]) @ ts["W2"] + ts["b2"]).mean()
+    tl.backward()
+    _close(loss, tl.item())
+    for g, k in zip(grads, ("W1", "b1", "W2", "b2")):
+        _close(g, ts[k].grad.numpy())
+
+
+def test_config_c2_closed_form_gradient():
+    inp = oc.c2_inputs(6, 40, seed=2)
+    out, gx = oc.c2_reference(**inp)
+    x, y = inp["x"].astype(np.float64), inp["y"].astype(np.float64)
+    p = x * y
+    m = p.max(1, keepdims=True)
+    e = np.exp(p - m)
+    r = np.maximum(x, 0)
+    _close(out, (e * r).sum(1))
+    # d/dx sum_j e_j r_j with the max treated through the tie rule
+    closed = e * (x > 0) + y * (e * r - (p == m) * (e * r).sum(1, keepdims=True))
+    _close(gx, closed)
+    tx = _t(x)
+    tp = tx * torch.tensor(y)
+    (torch.exp(tp - tp.max(1, keepdim=True).values) * torch.relu(tx)).sum().backward()
+    _close(gx, tx.grad.numpy())
+
+
+def test_config_c3_against_torch_module_formulas():
+    t = oc.c3_inputs(2, 8, 16, 32, seed=3, bf16=False)
+    t = {k: v.astype(np.float64) + (0.1 * RNG.standard_normal(v.shape) if k.startswith("b") or k.startswith("ln") else 0)
+         for k, v in t.items()}
+    loss, grads = oc.c3_reference(t, num_heads=4)
+    ts = {k: _t(v) for k, v in t.items()}
+
+    def heads(z):
+        return z.reshape(2, 8, 4, 4).transpose(1, 2)
+
+    x = ts["x"]
+    n1 = TF.layer_norm(x, (16,), ts["ln1_w"], ts["ln1_b"])
+    q, k, v = (heads(n1 @ ts[w] + ts[b]) for w, b in (("wq", "bq"), ("wk", "bk"), ("wv", "bv")))
+    a = TF.scaled_dot_product_attention(q, k, v, is_causal=True)
+    x = x + a.transpose(1, 2).reshape(2, 8, 16) @ ts["wo"] + ts["bo"]
+    n2 = TF.layer_norm(x, (16,), ts["ln2_w"], ts["ln2_b"])
+    out = x + TF.gelu(n2 @ ts["w1"] + ts["b1"]) @ ts["w2"] + ts["b2"]
+    tl = (out * out).mean()
+    tl.backward()
+    _close(loss, tl.item(), 1e-9)
+    for k in oc.C3_PARAMS:
+        _close(grads[k], ts[k].grad.numpy(), 1e-8)
+
+
+def test_config_c4_against_torch():
+    t = oc.c4_inputs(batch=3, hw=8, c=(3, 4, 6, 8), classes=5, seed=4)
+    loss, grads, am, logits = oc.c4_reference(t)
+    ts = {k: _t(v) for k, v in t.items() if k != "labels"}
+
+    def conv(h, k, b):
+        return TF.conv2d(h, ts[k].permute(3, 2, 0, 1), ts[b], padding=1)
+
+    h = torch.relu(conv(ts["img"].permute(0, 3, 1, 2), "k1", "c1b"))
+    h = TF.max_pool2d(torch.relu(conv(h, "k2", "c2b")), 2)
+    h = torch.relu(conv(h, "k3", "c3b")).mean(dim=(2, 3))
+    lg = h @ ts["wl"] + ts["bl"]
+    tl = TF.cross_entropy(lg, torch.tensor(t["labels"]))
+    tl.backward()
+    _close(loss, tl.item(), 1e-9)
+    _close(logits, lg.detach().numpy(), 1e-9)
+    assert np.array_equal(am, lg.argmax(-1).numpy())
+    for k in oc.C4_PARAMS:
+        _close(grads[k], ts[k].grad.numpy(), 1e-8)
+
+
+def test_config_c5_lora_grads_against_torch_and_zero_at_init():
+    t = oc.c5_inputs(layers=2, batch=2, seq=6, d_model=16, d_ff=32, vocab=20, rank=2, seed=5,
+                     b_zero=False, bf16=False)
+    loss, grads = oc.c5_reference(t, num_heads=4, alpha=4.0)
+    lora = [{k: _t(v) for k, v in ad.items()} for ad in t["lora"]]
+    c = lambda a: torch.tensor(a, dtype=torch.float64)
+    x = c(t["embed"])[torch.tensor(t["ids"])]
+    heads = lambda z: z.reshape(2, 6, 4, 4).transpose(1, 2)
+    for L, ad in zip(t["layers"], lora):
+        n1 = TF.layer_norm(x, (16,), c(L["ln1_w"]), c(L["ln1_b"]))
+        q = heads(n1 @ c(L["wq"]) + n1 @ ((ad["qA"] @ ad["qB"]) * 2.0) + c(L["bq"]))
+        k = heads(n1 @ c(L["wk"]) + c(L["bk"]))
+        v = heads(n1 @ c(L["wv"]) + n1 @ ((ad["vA"] @ ad["vB"]) * 2.0) + c(L["bv"]))
+        a = TF.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + a.transpose(1, 2).reshape(2, 6, 16) @ c(L["wo"]) + c(L["bo"])
+        n2 = TF.layer_norm(x, (16,), c(L["ln2_w"]), c(L["ln2_b"]))
+        x = x + TF.gelu(n2 @ c(L["w1"]) + c(L["b1"])) @ c(L["w2"]) + c(L["b2"])
+    x = TF.layer_norm(x, (16,), c(t["lnf_w"]), c(t["lnf_b"]))
+    lg = x @ c(t["head"])
+    tl = TF.cross_entropy(lg.reshape(-1, 20), torch.tensor(t["ids"]).reshape(-1), reduction="sum") / 2
+    tl.backward()
+    _close(loss, tl.item(), 1e-9)
+    flat = [ad[k] for ad in lora for k in ("qA", "qB", "vA", "vB")]
+    for g, tt in zip(grads, flat):
+        _close(g, tt.grad.numpy(), 1e-8)
+    # with B = 0 (the initialisation of the configuration) dA is exactly zero
+    t0 = oc.c5_inputs(layers=1, batch=1, seq=4, d_model=8, d_ff=16, vocab=10, rank=2, seed=6,
+                      b_zero=True, bf16=False)
+    _, g0 = oc.c5_reference(t0, num_heads=2)
+    assert np.all(g0[0] == 0) and np.all(g0[2] == 0) and np.abs(g0[1]).max() > 0
