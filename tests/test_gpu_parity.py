@@ -325,7 +325,7 @@ def test_custom_kernel_missing_library_is_an_error(hip):
         def kernel(self, args, kwargs):
             return [nb.ops.call_custom_kernel("nope", Path(__file__).parent / "golden", args[0], args[0].type)]
 
-    with pytest.raises(FileNotFoundError):
+    with pytest.raises(RuntimeError, match="no built kernel library"):
         Broken()([T(np.zeros(4, np.float32))], {})[0].numpy()
 
 
