@@ -1183,8 +1183,14 @@ class _RowCodegen:
                     operands[idx].stage_slot = n_stage
                     n_stage += 1
         chunks = (C + 3) // 4
+        # chunks a lane may own: long rows of few inputs keep up to 8 float4 per input in
+        # registers (16 in all), which halves the workgroup and its barrier cost
+        cpt_max = 8
+        n_in = max(1, len({i[2] for i in ins if i[0] == isa.LDG}))
+        while cpt_max > 2 and cpt_max * n_in > 16:
+            cpt_max //= 2
         block = 64
-        while block < isa.MAX_BLOCK and block * 2 < chunks:
+        while block < isa.MAX_BLOCK and block * cpt_max < chunks:
             block *= 2
         reads = sorted({o.buf for o in operands if not o.is_output})
         writes = sorted({o.buf for o in operands if o.is_output})

@@ -90,6 +90,7 @@ def _ew_scalar(op: int, dst: int, a: int, b: int, c: int) -> str:
 
 
 MAX_RESIDENT_REGS = 16  # float4 registers a row-resident kernel may spend on inputs
+PREFETCH_MAX_REGS = 8   # ... and on the next row's inputs when rows are software-pipelined
 
 
 def full_inputs(a: dict) -> list[int]:
@@ -117,9 +118,14 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
     if block_mode:
         # register-resident forms: cap registers so that two 512-lane workgroups (or
         # more smaller ones) share a CU and one loads while the other computes
-        occ = "__attribute__((amdgpu_waves_per_eu(4))) " if 0 < cpt <= 4 else ""
+        occ = ""
+        if resident:
+            # FULL: the row is exactly cpt chunks per lane, no lane or element is masked
+            # STREAM: fp32 unit-stride operands are read and written with the non-temporal hint
+            w("template <bool FULL, bool STREAM>")
         w(f"__global__ __launch_bounds__(512) {occ}void {name}(const nbk_rowprog P, int64_t rows) {{")
-        w("  __shared__ float red_buf[16];")
+        w("  __shared__ float red_buf[64];")
+        w("  int red_phase = 0; (void)red_phase;")
         w("  const int64_t C = P.C, c_pad = (C + 3) & ~(int64_t)3, n_chunks = c_pad >> 2;")
         w("  const bool writer = threadIdx.x == 0;")
         w("  (void)c_pad;")
@@ -135,12 +141,82 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
           + (f" o{k}.col_stride = {o.col_stride};" if o.col_stride in (0, 1) else ""))
     w("  const int64_t ld1 = P.lead_dim[1], ld2 = P.lead_dim[2], ld3 = P.lead_dim[3];")
     used_s = sorted({r for i in ins for r in (i[1], i[2], i[3], i[4]) if isa.NVEC <= r < 32})
-    if block_mode:
+    written = {i[1] for i in ins if i[0] in (isa.STR, isa.STG)}
+    hoisted: dict[int, str] = {}
+    for i in ins:
+        # scalar operand reads do not depend on anything the row computes: issue them with
+        # the row's first loads instead of between the phases, where their latency is exposed
+        if i[0] == isa.LDR and i[2] not in written and i[2] not in hoisted:
+            hoisted[i[2]] = f"ldr{i[2]}"
+    decomp = ("rp_decompose_row((uint32_t)(ROW), P.n_lead, (uint32_t)ld1, (uint32_t)ld2, "
+              "(uint32_t)ld3, LI);")
+    if resident:
+        # Software pipeline over the rows of a persistent workgroup: the loads of the next
+        # row are issued before the current row is computed and stored, so a row's load
+        # latency overlaps the previous row's arithmetic and never queues behind its stores.
+        w(f"  int64_t colj[{cpt}]; int validj[{cpt}];")
+        w("#pragma unroll")
+        w(f"  for (int j = 0; j < {cpt}; ++j) {{")
+        w("    const int64_t ch = threadIdx.x + (int64_t)j * blockDim.x;")
+        w("    colj[j] = ch << 2;")
+        w("    const int64_t left = C - colj[j];")
+        w("    validj[j] = FULL ? 4 : (ch < n_chunks ? (left >= 4 ? 4 : (int)left) : 0);")
+        w("  }")
+        w("  uint32_t nlead[4];")
+        w("  int64_t " + ", ".join(f"noff{k} = 0" for k in range(len(ops))) + ";")
+        for k in hoisted:
+            w(f"  float nldr{k} = 0.f;")
+        for k in inputs:
+            w(f"  float4 n{k}[{cpt}];")
+
+        def fetch(row_expr: str, ind: str) -> None:
+            w(ind + decomp.replace("ROW", row_expr).replace("LI", "nlead"))
+            w(ind + "if (P.n_lead <= 1) {")
+            for k in range(len(ops)):
+                w(ind + f"  noff{k} = (int64_t)nlead[0] * o{k}.lead_stride[0];")
+            w(ind + "} else {")
+            for k in range(len(ops)):
+                w(ind + f"  noff{k} = rp_row_offset(o{k}, nlead, 4);")
+            w(ind + "}")
+            for k in hoisted:
+                w(ind + f"nldr{k} = nbk_load_as_f32(o{k}.ptr, noff{k}, o{k}.dtype);")
+            for k in inputs:
+                full_load = f"rp_load4(o{k}, noff{k}, colj[j], 4)"
+                if ops[k].dtype.abi == 0 and ops[k].vec_ok and ops[k].col_stride == 1:
+                    full_load = (f"(STREAM ? rp_load4_stream((const float*)o{k}.ptr + noff{k} + colj[j]) : "
+                                 f"{full_load})")
+                w("#pragma unroll")
+                w(ind + f"for (int j = 0; j < {cpt}; ++j) n{k}[j] = FULL ? {full_load} : "
+                  f"(validj[j] > 0 ? rp_load4(o{k}, noff{k}, colj[j], validj[j]) : "
+                  "make_float4(0.f, 0.f, 0.f, 0.f));")
+
+        # the pipeline doubles the registers that hold inputs; past 8 float4 per lane that
+        # costs more occupancy than the overlap returns
+        prefetch = cpt * max(1, len(inputs)) <= PREFETCH_MAX_REGS
+        if prefetch:
+            fetch("blockIdx.x", "  ")
         w("  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {")
-        w("    int64_t lead_idx[4];")
-        w("    { int64_t rem = row, q; q = rem / ld3; lead_idx[3] = rem - q * ld3; rem = q;"
-          " q = rem / ld2; lead_idx[2] = rem - q * ld2; rem = q;"
-          " q = rem / ld1; lead_idx[1] = rem - q * ld1; rem = q; lead_idx[0] = rem; }")
+        if not prefetch:
+            fetch("row", "    ")
+        w("    uint32_t lead_idx[4] = {nlead[0], nlead[1], nlead[2], nlead[3]};")
+        w("    (void)lead_idx;")
+        for k in range(len(ops)):
+            w(f"    const int64_t off{k} = noff{k};")
+        for k in hoisted:
+            w(f"    const float ldr{k} = nldr{k};")
+        for k in inputs:
+            w(f"    float4 r{k}[{cpt}];")
+            w("#pragma unroll")
+            w(f"    for (int j = 0; j < {cpt}; ++j) r{k}[j] = n{k}[j];")
+        if prefetch:
+            w("    if (row + gridDim.x < rows) {")
+            fetch("row + gridDim.x", "      ")
+            w("    }")
+    elif block_mode:
+        w("  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {")
+        # the host rejects launches of 2^31 rows or more, so 32-bit division is exact
+        w("    uint32_t lead_idx[4];")
+        w("    " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
     else:
         w("  const uint64_t stride = (uint64_t)gridDim.x * 256u;")
         w("  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {")
@@ -149,35 +225,20 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         w("    else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }")
         w("    else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }")
         w("    uint32_t lead_idx[4] = {0, 0, 0, 0};")
-        w("    if (P.n_lead > 0) { uint32_t rem = row, q; const uint32_t d1 = (uint32_t)ld1, "
-          "d2 = (uint32_t)ld2, d3 = (uint32_t)ld3;"
-          " q = rem / d3; lead_idx[3] = rem - q * d3; rem = q; q = rem / d2; lead_idx[2] = rem - q * d2; rem = q;"
-          " q = rem / d1; lead_idx[1] = rem - q * d1; rem = q; lead_idx[0] = rem; }")
+        w("    if (P.n_lead > 0) " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
         w("    const bool writer = cc == 0;")
         w("    const int64_t col = (int64_t)cc << 2;")
         w("    const int64_t left = C - col;")
         w("    const int valid = left >= 4 ? 4 : (int)left;")
-    for k in range(len(ops)):
-        w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
-    if resident:
-        # every lane loads its chunks of every input up front
-        w(f"    int64_t colj[{cpt}]; int validj[{cpt}];")
-        w("#pragma unroll")
-        w(f"    for (int j = 0; j < {cpt}; ++j) {{")
-        w("      const int64_t ch = threadIdx.x + (int64_t)j * blockDim.x;")
-        w("      colj[j] = ch << 2;")
-        w("      const int64_t left = C - colj[j];")
-        w("      validj[j] = ch < n_chunks ? (left >= 4 ? 4 : (int)left) : 0;")
-        w("    }")
-        for k in inputs:
-            w(f"    float4 r{k}[{cpt}];")
-            w("#pragma unroll")
-            w(f"    for (int j = 0; j < {cpt}; ++j) r{k}[j] = validj[j] > 0 ? "
-              f"rp_load4(o{k}, off{k}, colj[j], validj[j]) : make_float4(0.f, 0.f, 0.f, 0.f);")
-    elif block_mode and a["n_stage"] > 0:
-        for k, o in enumerate(ops):
-            if o.stage_slot >= 0:
-                w(f"    rp_stage_row(o{k}, off{k}, rp_stage_lds + {o.stage_slot} * c_pad, C, n_chunks);")
+    if not resident:
+        for k in range(len(ops)):
+            w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
+        for k in hoisted:
+            w(f"    const float ldr{k} = nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
+        if block_mode and a["n_stage"] > 0:
+            for k, o in enumerate(ops):
+                if o.stage_slot >= 0:
+                    w(f"    rp_stage_row(o{k}, off{k}, rp_stage_lds + {o.stage_slot} * c_pad, C, n_chunks);")
     if used_s:
         w("    float " + ", ".join(f"s{r} = 0.f" for r in used_s) + ";")
     w("    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;")
@@ -195,7 +256,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                 w("#pragma unroll")
                 w(f"    for (int j = 0; j < {cpt}; ++j) {{")
                 w("      const int64_t col = colj[j];")
-                w("      const int valid = validj[j];")
+                w("      const int valid = FULL ? 4 : validj[j];")
             elif block_mode:
                 w("    for (int64_t ch = threadIdx.x; ch < n_chunks; ch += blockDim.x) {")
                 w("      const int64_t col = ch << 2;")
@@ -219,7 +280,11 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                         w(ind + f"v{bd} = rp_load4(o{bx}, off{bx}, col, valid);")
                 elif bop == isa.STG:
                     if resident:
-                        w(ind + f"if (valid > 0) rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
+                        od = ops[bd]
+                        if od.dtype.abi == 0 and od.vec_ok and od.col_stride == 1:
+                            w(ind + f"if (FULL && STREAM) rp_store4_stream((float*)o{bd}.ptr + off{bd} + col, "
+                              f"{_as_vec(bx)}); else")
+                        w(ind + f"if (FULL || valid > 0) rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
                     else:
                         w(ind + f"rp_store4(o{bd}, off{bd}, col, valid, {_as_vec(bx)});")
                 elif bop == isa.ACC:
@@ -235,7 +300,10 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         if op == isa.IMM:
             w(f"    s{dst} = P.imm[{x}];")
         elif op == isa.LDR:
-            w(f"    s{dst} = nbk_load_as_f32(o{x}.ptr, off{x}, o{x}.dtype);")
+            if x in hoisted:
+                w(f"    s{dst} = {hoisted[x]};")
+            else:
+                w(f"    s{dst} = nbk_load_as_f32(o{x}.ptr, off{x}, o{x}.dtype);")
         elif op == isa.STR:
             w(f"    if (writer) nbk_store_from_f32(o{dst}.ptr, off{dst}, o{dst}.dtype, s{x});")
         elif op == isa.LEADIDX:
@@ -243,7 +311,19 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         elif op == isa.ACCINIT:
             w(f"    acc{dst} = rp_identity({x});")
         elif op == isa.RED:
-            w(f"    s{dst} = rp_block_reduce(acc{x}, {y}, red_buf);")
+            # consecutive reductions share one barrier
+            group = [(dst, x, y)]
+            while (len(group) < 4 and pc + len(group) < len(ins)
+                   and ins[pc + len(group)][0] == isa.RED):
+                g = ins[pc + len(group)]
+                group.append((g[1], g[2], g[3]))
+            n = len(group)
+            w(f"    {{ float rv[{n}] = {{{', '.join(f'acc{g[1]}' for g in group)}}}; "
+              f"const int rk[{n}] = {{{', '.join(str(g[2]) for g in group)}}}; "
+              f"rp_block_reduce_n(rv, rk, {n}, red_buf, red_phase); "
+              + " ".join(f"s{g[0]} = rv[{q}];" for q, g in enumerate(group)) + " }")
+            pc += n
+            continue
         else:
             w("    " + _ew_scalar(op, dst, x, y, z))
         pc += 1
@@ -362,10 +442,17 @@ def write_sources(programs: dict[int, dict]) -> list[Path]:
         for h, a in chunk:
             rv = resident_variants(a)
             ks = [f"(const void*)rp_spec_{h:016x}"]
+            kf = ["nullptr"]
+            kst = ["nullptr"]
             for c in (1, 2, 4, 8):
-                ks.append(f"(const void*)rp_spec_{h:016x}_c{c}" if c in rv else "nullptr")
-            src.append(f"  {{0x{h:016x}ULL, {{{', '.join(ks)}}}, {1 if a['has_reduce'] else 0}}},")
-        src.append("  {0ULL, {nullptr, nullptr, nullptr, nullptr, nullptr}, 0}};")
+                ks.append(f"(const void*)rp_spec_{h:016x}_c{c}<false, false>" if c in rv else "nullptr")
+                kf.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, false>" if c in rv else "nullptr")
+                kst.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, true>" if c in rv else "nullptr")
+            src.append(f"  {{0x{h:016x}ULL, {{{', '.join(ks)}}}, {{{', '.join(kf)}}}, "
+                       f"{{{', '.join(kst)}}}, {1 if a['has_reduce'] else 0}}},")
+        src.append("  {0ULL, {nullptr, nullptr, nullptr, nullptr, nullptr}, "
+                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, "
+                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, 0}};")
         src.append(f"extern const int rp_spec_count_{fi} = {len(chunk)};")
         path = CSRC / f"rowprog_spec_gen{fi}.hip"
         path.write_text("\n".join(src) + "\n")

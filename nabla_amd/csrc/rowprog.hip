@@ -448,7 +448,13 @@ static uint64_t rp_program_hash(const nbk_rowprog* p) {
   return h;
 }
 
-struct RpSpec { const void* kernel[5]; int block_mode; bool lds_attr_set; };
+struct RpSpec {
+  const void* kernel[5];
+  const void* kernel_full[5];
+  const void* kernel_stream[5];
+  int block_mode;
+  bool lds_attr_set;
+};
 static std::mutex g_spec_mu;
 static std::unordered_map<uint64_t, RpSpec>* g_specs = nullptr;
 
@@ -464,7 +470,11 @@ static RpSpec* rp_find_spec(uint64_t h) {
       for (int i = 0; i < counts[t]; ++i)
       {
         RpSpec e;
-        for (int k = 0; k < 5; ++k) e.kernel[k] = tabs[t][i].kernel[k];
+        for (int k = 0; k < 5; ++k) {
+          e.kernel[k] = tabs[t][i].kernel[k];
+          e.kernel_full[k] = tabs[t][i].kernel_full[k];
+          e.kernel_stream[k] = tabs[t][i].kernel_stream[k];
+        }
         e.block_mode = tabs[t][i].block_mode;
         e.lds_attr_set = false;
         (*g_specs)[tabs[t][i].hash] = e;
@@ -472,6 +482,24 @@ static RpSpec* rp_find_spec(uint64_t h) {
   }
   auto it = g_specs->find(h);
   return it == g_specs->end() ? nullptr : &it->second;
+}
+
+// Resident workgroups per CU of a kernel at a block size (no dynamic LDS); cached.
+static int rp_occupancy(const void* fn, int block, int* out) {
+  static std::mutex mu;
+  static std::unordered_map<uint64_t, int>* cache = nullptr;
+  const uint64_t key = (uint64_t)(uintptr_t)fn ^ ((uint64_t)block << 48);
+  std::lock_guard<std::mutex> lk(mu);
+  if (!cache) cache = new std::unordered_map<uint64_t, int>();
+  auto it = cache->find(key);
+  if (it == cache->end()) {
+    int n = 0;
+    NBK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, block, 0));
+    if (n < 1) n = 1;
+    it = cache->emplace(key, n).first;
+  }
+  *out = it->second;
+  return NBK_OK;
 }
 
 // 1: interpreter only (debug / comparison); read once.
@@ -537,9 +565,27 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
       const int64_t need = (n_chunks + block - 1) / block;
       int slot = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 3 : need <= 8 ? 4 : 0;
       if (slot && spec->kernel[slot]) {
-        int64_t g2 = (int64_t)nbk_num_cus() * (block >= 512 ? 3 : (block >= 256 ? 6 : 12));
+        static const int cpt_of[5] = {0, 1, 2, 4, 8};
+        const bool full = p->C == (int64_t)4 * cpt_of[slot] * block && spec->kernel_full[slot];
+        const void* fn = spec->kernel[slot];
+        if (full) {
+          // bytes of the row-shaped operands; beyond the 256 MiB last-level cache nothing
+          // written here survives until a consumer runs, so stream it
+          int64_t bytes = 0;
+          for (int i = 0; i < p->n_operands; ++i)
+            if (p->operand[i].col_stride != 0)
+              bytes += rows * p->C * (int64_t)nbk_dtype_size(p->operand[i].dtype);
+          fn = (bytes > (256ll << 20) && spec->kernel_stream[slot]) ? spec->kernel_stream[slot]
+                                                                    : spec->kernel_full[slot];
+        }
+        // persistent workgroups, exactly as many as are resident at once: the program
+        // descriptor is read from kernel-argument memory once per workgroup, not once per
+        // row, and no second partial wave of workgroups trails behind the first
+        int per_cu = 0;
+        { const int orc = rp_occupancy(fn, block, &per_cu); if (orc != NBK_OK) return orc; }
+        int64_t g2 = (int64_t)nbk_num_cus() * per_cu;
         if (g2 > rows) g2 = rows;
-        NBK_HIP(hipLaunchKernel(spec->kernel[slot], dim3((unsigned)g2), dim3(block), args, 0, st));
+        NBK_HIP(hipLaunchKernel(fn, dim3((unsigned)g2), dim3(block), args, 0, st));
         return NBK_OK;
       }
       if (lds > 32 * 1024 && !spec->lds_attr_set) {

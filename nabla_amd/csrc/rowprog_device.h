@@ -16,6 +16,18 @@ __device__ __forceinline__ float rp_identity(int kind) {
 }
 
 // ---- chunk load / store ----------------------------------------------------
+// Streaming forms for launches whose operands exceed the last-level cache: the
+// non-temporal hint keeps lines that are touched once from displacing others.
+typedef float rp_vf4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 rp_load4_stream(const float* p) {
+  rp_vf4 v = __builtin_nontemporal_load((const rp_vf4*)p);
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void rp_store4_stream(float* p, float4 r) {
+  rp_vf4 v = {r.x, r.y, r.z, r.w};
+  __builtin_nontemporal_store(v, (rp_vf4*)p);
+}
+
 __device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, int64_t col,
                                            int valid) {
   const int dt = o.dtype;
@@ -157,19 +169,93 @@ __device__ __forceinline__ int64_t rp_row_offset(const nbk_operand& o, const IDX
          (int64_t)lead_idx[2] * o.lead_stride[2] + (int64_t)lead_idx[3] * o.lead_stride[3];
 }
 
-// Block-wide reduction of one float: wavefront shuffles, then an LDS tree.
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the
+// wave's outstanding global loads and stores; the reductions below exchange data
+// through LDS alone, and the pipelined row kernels want their next row's loads to
+// stay in flight across them.
+__device__ __forceinline__ void rp_lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Cross-lane step: combine every lane's value with the value the DPP control word
+// selects; lanes the row mask excludes (or that select an invalid lane) take part
+// with the identity.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float rp_dpp_step(float v, int kind) {
+  const int ident = __float_as_int(rp_identity(kind));
+  const int t = __builtin_amdgcn_update_dpp(ident, __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
+  return rp_combine(v, __int_as_float(t), kind);
+}
+
+// Reduction over the 64 lanes of a wavefront on the VALU's data-parallel-primitive
+// path (no LDS round trips).  Every lane must be active.  Returns the wave's total,
+// uniform across the wave.
+__device__ __forceinline__ float rp_wave_reduce(float v, int kind) {
+  v = rp_dpp_step<0xB1, 0xf>(v, kind);   // quad_perm [1,0,3,2]: lane ^ 1
+  v = rp_dpp_step<0x4E, 0xf>(v, kind);   // quad_perm [2,3,0,1]: lane ^ 2
+  v = rp_dpp_step<0x141, 0xf>(v, kind);  // row_half_mirror: the other quad of each 8
+  v = rp_dpp_step<0x140, 0xf>(v, kind);  // row_mirror: the other half of each row of 16
+  v = rp_dpp_step<0x142, 0xa>(v, kind);  // row_bcast15 into rows 1 and 3
+  v = rp_dpp_step<0x143, 0xc>(v, kind);  // row_bcast31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// Total over the first eight lanes (one partial per wave of the workgroup), uniform.
+__device__ __forceinline__ float rp_reduce8(float v, int kind) {
+  v = rp_dpp_step<0xB1, 0xf>(v, kind);
+  v = rp_dpp_step<0x4E, 0xf>(v, kind);
+  v = rp_dpp_step<0x141, 0xf>(v, kind);
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+
+// Block-wide reduction of one float: DPP within each wave, then one partial per
+// wave through LDS.  Two barriers: safe to call back to back on the same buffer.
 __device__ __forceinline__ float rp_block_reduce(float v, int kind, float* red_buf) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = rp_combine(v, __shfl_xor(v, off, 64), kind);
+  v = rp_wave_reduce(v, kind);
   const int nw = blockDim.x >> 6;
   if (nw == 1) return v;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   if (lane == 0) red_buf[w] = v;
-  __syncthreads();
-  float r = red_buf[0];
-  for (int i = 1; i < nw; ++i) r = rp_combine(r, red_buf[i], kind);
-  __syncthreads();
+  rp_lds_barrier();
+  float r = rp_reduce8(lane < nw ? red_buf[lane] : rp_identity(kind), kind);
+  rp_lds_barrier();
   return r;
+}
+
+// The same with ONE barrier per call.  ``red2`` holds two banks of 32 floats and
+// ``phase`` counts the calls of the workgroup: consecutive calls use different banks,
+// and a bank is rewritten only after the barrier of the call in between, which every
+// wave reaches after it has read that bank.  Up to four values (slot k of a bank
+// holds the partials of value k) share the barrier.
+__device__ __forceinline__ void rp_block_reduce_n(float* v, const int* kind, int n, float* red2,
+                                                  int& phase) {
+  for (int k = 0; k < n; ++k) v[k] = rp_wave_reduce(v[k], kind[k]);
+  const int nw = blockDim.x >> 6;
+  if (nw == 1) return;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  float* bank = red2 + ((phase & 1) << 5);
+  ++phase;
+  if (lane == 0)
+    for (int k = 0; k < n; ++k) bank[k * 8 + w] = v[k];
+  rp_lds_barrier();
+  for (int k = 0; k < n; ++k)
+    v[k] = rp_reduce8(lane < nw ? bank[k * 8 + lane] : rp_identity(kind[k]), kind[k]);
+}
+
+// Row index -> indices of the (up to four) leading dimensions; rows < 2^31.
+__device__ __forceinline__ void rp_decompose_row(uint32_t row, int n_lead, uint32_t d1, uint32_t d2,
+                                                 uint32_t d3, uint32_t* li) {
+  if (n_lead <= 1) {
+    li[0] = row; li[1] = 0; li[2] = 0; li[3] = 0;
+    return;
+  }
+  uint32_t rem = row, q;
+  q = rem / d3; li[3] = rem - q * d3; rem = q;
+  q = rem / d2; li[2] = rem - q * d2; rem = q;
+  q = rem / d1; li[1] = rem - q * d1; rem = q;
+  li[0] = rem;
 }
 
 

@@ -11,6 +11,12 @@ struct rp_spec_entry {
   // nullptr where that form was not generated.  All have the signature of
   // rp_block_kernel / rp_flat_kernel.
   const void* kernel[5];
+  // [1..4]: the same register-resident forms compiled for rows of exactly
+  // 1 / 2 / 4 / 8 chunks per lane (no masked lanes or elements); [0] unused.
+  const void* kernel_full[5];
+  // [1..4]: kernel_full with non-temporal loads and stores, for launches that move
+  // more bytes than the last-level cache holds.
+  const void* kernel_stream[5];
   int block_mode;
 };
 
