@@ -19,6 +19,10 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+// 16-byte register / LDS unit.  A native vector (an SSA value), not the uint4 struct:
+// arrays of structs that are filled by loads and drained by stores are turned into
+// memcpy through a stack slot, which puts the staging registers in scratch.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // Compile-time loop: accumulator tiles must be indexed with constants or they
 // leave the register file.
@@ -76,9 +80,9 @@ __device__ __forceinline__ int swz(int row, int chunk) {
 }
 
 // 16-byte guarded load of 8 consecutive bf16 along the unit-stride axis.
-__device__ __forceinline__ uint4 ld8_bf16(const uint16_t* p, int64_t valid, bool vec) {
-  uint4 r = make_uint4(0, 0, 0, 0);
-  if (valid >= 8 && vec) return *(const uint4*)p;
+__device__ __forceinline__ u32x4 ld8_bf16(const uint16_t* p, int64_t valid, bool vec) {
+  u32x4 r = {0u, 0u, 0u, 0u};
+  if (valid >= 8 && vec) return *(const u32x4*)p;
   if (valid <= 0) return r;
   uint16_t t[8];
 #pragma unroll
@@ -90,19 +94,23 @@ __device__ __forceinline__ uint4 ld8_bf16(const uint16_t* p, int64_t valid, bool
   return r;
 }
 
-// FAST loaders assume 16-byte-aligned operands, K % 8 == 0 and, for an operand
+// FAST loaders assume 16-byte-aligned operands, K % 64 == 0 and, for an operand
 // that is contiguous along its rows, a row count that is a multiple of 8; then
-// every access is one predicated 16-byte load.  Rows past the edge are clamped
-// to the last valid row (their products are never stored); chunks past K read
-// zero.  Everything else goes through the guarded element-wise path (FAST=false),
+// every access is one unconditional 16-byte load and the K loop has no branches.
+// Rows past the edge are clamped to the last valid row (their products are never
+// stored).  Everything else goes through the guarded element-wise path (FAST=false),
 // which is kept out of the hot kernels because its code size alone would push
 // the main loop out of the instruction cache.
 template <int ROWS, bool KC, bool FAST>
 struct TileLoader {
-  // KC : operand contiguous along K   -> ROWS*8 chunk tasks, ROWS/32 per lane
-  // !KC: operand contiguous along rows -> ROWS (8x8 block) tasks, <=1 per lane
-  static constexpr int NREG = KC ? ROWS / 32 : 8;
-  uint4 reg[NREG];
+  // KC : operand contiguous along K    -> ROWS*8 chunk tasks, ROWS/32 per lane.
+  // !KC: operand contiguous along rows -> every lane transposes a KPT(k) x 8(rows) block:
+  //      one 8x8 block per lane for 256 rows, half a block (4 k-values) for 128 rows,
+  //      so that all 256 lanes take part and the K loop has no divergent branch.
+  static constexpr int KPT = ROWS >= 256 ? 8 : 4;
+  static constexpr int NREG = KC ? ROWS / 32 : KPT;
+  static_assert(ROWS == 256 || ROWS == 128, "tile rows");
+  u32x4 reg[NREG];
 
   __device__ __forceinline__ void load(const uint16_t* base, int64_t rs, int64_t cs, int64_t row0,
                                        int64_t rows_total, int64_t k0, int64_t K, bool vec) {
@@ -115,67 +123,66 @@ struct TileLoader {
         const int64_t gr = row0 + row, gk = k0 + c * 8;
         if (FAST) {
           const int64_t r = gr < rows_total ? gr : rows_total - 1;
-          const uint4* p = (const uint4*)(base + r * rs + gk);
-          reg[s] = gk < K ? *p : make_uint4(0, 0, 0, 0);
+          reg[s] = *(const u32x4*)(base + r * rs + gk);
         } else {
           if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
-          else reg[s] = make_uint4(0, 0, 0, 0);
+          else reg[s] = (u32x4){0u, 0u, 0u, 0u};
         }
       }
     } else {
       constexpr int NC = ROWS / 8;
-      const int nc = tid % NC, kg = tid / NC;
-      if (kg < 8) {
-        const int64_t gr = row0 + nc * 8;
+      const int nc = tid % NC, kq = tid / NC;  // kq: which KPT-row slice of the 64 k
+      const int64_t gr = row0 + nc * 8;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const int64_t gk = k0 + kg * 8 + r;
-          if (FAST) {
-            const int64_t rr = gr < rows_total ? gr : rows_total - 8;
-            const uint4* p = (const uint4*)(base + gk * cs + rr);
-            reg[r] = gk < K ? *p : make_uint4(0, 0, 0, 0);
-          } else {
-            if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
-            else reg[r] = make_uint4(0, 0, 0, 0);
-          }
+      for (int r = 0; r < KPT; ++r) {
+        const int64_t gk = k0 + kq * KPT + r;
+        if (FAST) {
+          const int64_t rr = gr < rows_total ? gr : rows_total - 8;
+          reg[r] = *(const u32x4*)(base + gk * cs + rr);
+        } else {
+          if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
+          else reg[r] = (u32x4){0u, 0u, 0u, 0u};
         }
       }
     }
   }
 
-  __device__ __forceinline__ void store(uint4* lds) {
+  // The tile goes to LDS in NPIECE independent pieces so that the K loop can place
+  // them between its matrix instructions.
+  static constexpr int NPIECE = KC ? NREG : 8;
+  template <int P>
+  __device__ __forceinline__ void store_piece(u32x4* lds) {
     const int tid = threadIdx.x;
     if (KC) {
-#pragma unroll
-      for (int s = 0; s < NREG; ++s) {
-        const int t = tid + s * 256;
-        lds[swz(t >> 3, t & 7)] = reg[s];
-      }
+      const int t = tid + P * 256;
+      lds[swz(t >> 3, t & 7)] = reg[P];
     } else {
       constexpr int NC = ROWS / 8;
-      const int nc = tid % NC, kg = tid / NC;
-      if (kg < 8) {
-        // 8x8 transpose of 16-bit elements: out[j] holds k = 0..7 of column j
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-          uint4 o;
-          o.x = __builtin_amdgcn_perm(comp(reg[1], j >> 1), comp(reg[0], j >> 1), sel);
-          o.y = __builtin_amdgcn_perm(comp(reg[3], j >> 1), comp(reg[2], j >> 1), sel);
-          o.z = __builtin_amdgcn_perm(comp(reg[5], j >> 1), comp(reg[4], j >> 1), sel);
-          o.w = __builtin_amdgcn_perm(comp(reg[7], j >> 1), comp(reg[6], j >> 1), sel);
-          lds[swz(nc * 8 + j, kg)] = o;
-        }
+      const int nc = tid % NC, kq = tid / NC;
+      // row P of the transpose of 16-bit elements: the lane's k-values of column P
+      constexpr uint32_t sel = (P & 1) ? 0x07060302u : 0x05040100u;
+      if (KPT == 8) {
+        u32x4 o;
+        o.x = __builtin_amdgcn_perm(reg[1][P >> 1], reg[0][P >> 1], sel);
+        o.y = __builtin_amdgcn_perm(reg[3][P >> 1], reg[2][P >> 1], sel);
+        o.z = __builtin_amdgcn_perm(reg[5 % NREG][P >> 1], reg[4 % NREG][P >> 1], sel);
+        o.w = __builtin_amdgcn_perm(reg[7 % NREG][P >> 1], reg[6 % NREG][P >> 1], sel);
+        lds[swz(nc * 8 + P, kq)] = o;
+      } else {
+        uint2 o;
+        o.x = __builtin_amdgcn_perm(reg[1][P >> 1], reg[0][P >> 1], sel);
+        o.y = __builtin_amdgcn_perm(reg[3][P >> 1], reg[2][P >> 1], sel);
+        uint2* dst = (uint2*)(lds + swz(nc * 8 + P, kq >> 1)) + (kq & 1);
+        *dst = o;
       }
     }
   }
-
-  static __device__ __forceinline__ uint32_t comp(const uint4& v, int d) {
-    return d == 0 ? v.x : d == 1 ? v.y : d == 2 ? v.z : v.w;
+  __device__ __forceinline__ void store(u32x4* lds) {
+    static_for<NPIECE>([&](auto pc) { store_piece<decltype(pc)::value>(lds); });
   }
 };
 
-extern __shared__ __align__(16) uint4 gemm_lds[];
+extern __shared__ __align__(16) u32x4 gemm_lds[];
 
 template <int BM, int BN, bool A_KC, bool B_KC, bool FAST, bool EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
@@ -209,49 +216,149 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   lb.store(gemm_lds + BM * 8);
   __syncthreads();
 
-  // fragment addresses: row part is loop-invariant, only the chunk index moves
-  int a_row[TM], b_row[TN];
+  // Fragment addresses.  swz(row, ks * 2 + kg) = (row * 8 | t) ^ (ks * 2) with
+  // t = kg ^ (row % 8) ^ (row / 8 % 8): only a constant XOR moves with ks.
+  int a_addr[TM], b_addr[TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) a_row[i] = wm + i * 32 + li;
-#pragma unroll
-  for (int j = 0; j < TN; ++j) b_row[j] = wn + j * 32 + li;
-
-  for (int64_t kt = 0; kt < nk; ++kt) {
-    const uint4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
-    uint4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      la.load(A, g.a_rs, g.a_cs, m0, g.M, (kt + 1) * 64, g.K, g.a_vec);
-      lb.load(B, g.b_cs, g.b_rs, n0, g.N, (kt + 1) * 64, g.K, g.b_vec);
-    }
-    const uint4* As = cur;
-    const uint4* Bs = cur + BM * 8;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int kc = ks * 2 + kg;
-      bf16x8 fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        uint4 u = As[swz(a_row[i], kc)];
-        fa[i] = *(bf16x8*)&u;
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        uint4 u = Bs[swz(b_row[j], kc)];
-        fb[j] = *(bf16x8*)&u;
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) {
-      la.store(nxt);
-      lb.store(nxt + BM * 8);
-    }
-    __syncthreads();
+  for (int i = 0; i < TM; ++i) {
+    const int row = wm + i * 32 + li;
+    a_addr[i] = row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
   }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int row = wn + j * 32 + li;
+    b_addr[j] = BM * 8 + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
+  }
+
+  // Software pipeline.  One wave per SIMD owns the matrix pipe, so nothing hides a
+  // stall but the wave's own instruction stream; every load is therefore issued one
+  // stage before its use and sits between matrix instructions:
+  //   * fragments of k-step ks + 1 are read from LDS while the MFMAs of ks run
+  //     (two fragment sets, frag[0] / frag[1]);
+  //   * the tile of iteration kt + 1, fetched from global memory during iteration
+  //     kt - 1, is written to the other LDS buffer during k-step 2;
+  //   * the global loads of tile kt + 2 are issued behind those writes;
+  //   * the workgroup barrier falls in the middle of k-step 3, whose remaining
+  //     MFMAs cover the first fragment reads of the next tile.
+  bf16x8 fa[2][TM], fb[2][TN];
+  constexpr int NFRAG = TM + TN, NMFMA = TM * TN;
+  // read fragment r (A tiles first, then B) of k-step ks from `tile` into set SET
+  auto read_frag = [&](auto set, auto r, const u32x4* tile, int ks) {
+    // order of use by the MFMAs (row-major over the wave's tiles): A0, every B, A1, A2 ...
+    constexpr int SET = decltype(set)::value, R0 = decltype(r)::value;
+    constexpr int R = R0 == 0 ? 0 : (R0 <= TN ? TM + R0 - 1 : R0 - TN);
+    // The XOR is recomputed at every read: hoisted out of the K loop, the 4 x (TM + TN)
+    // x 2 variants of these addresses would spill the accumulating kernel.
+    int sel = ks * 2;
+    asm volatile("" : "+s"(sel));
+    if constexpr (R < TM) {
+      const u32x4 u = tile[a_addr[R] ^ sel];
+      fa[SET][R] = *(const bf16x8*)&u;
+    } else {
+      const u32x4 u = tile[b_addr[R - TM] ^ sel];
+      fb[SET][R - TM] = *(const bf16x8*)&u;
+    }
+  };
+  auto mfma = [&](auto set, auto q) {
+    constexpr int SET = decltype(set)::value, Q = decltype(q)::value;
+    constexpr int i = Q / TN, j = Q % TN;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][i], fb[SET][j], acc[i][j], 0, 0, 0);
+  };
+  // k-step on fragment set SET while set 1 - SET is filled for k-step `ks_next` of `tile`
+  auto stage = [&](auto set, const u32x4* tile, int ks_next) {
+    constexpr int SET = decltype(set)::value;
+    static_for<NFRAG>([&](auto r) {
+      read_frag(std::integral_constant<int, 1 - SET>{}, r, tile, ks_next);
+    });
+    static_for<NMFMA>([&](auto q) { mfma(set, q); });
+    // interleave: one fragment read, then its share of the MFMAs
+#pragma unroll
+    for (int r = 0; r < NFRAG; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
+      __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / NFRAG, 0);  // MFMAs
+    }
+    __builtin_amdgcn_sched_barrier(0);  // later stages' work (and its waits) stays behind
+  };
+
+  static_for<NFRAG>([&](auto r) { read_frag(std::integral_constant<int, 0>{}, r, gemm_lds, 0); });
+  {
+    const int64_t k1 = nk > 1 ? 64 : 0;  // a single-tile problem re-reads tile 0 (never stored)
+    la.load(A, g.a_rs, g.a_cs, m0, g.M, k1, g.K, g.a_vec);
+    lb.load(B, g.b_cs, g.b_rs, n0, g.N, k1, g.K, g.b_vec);
+  }
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  for (int64_t kt = 0; kt + 1 < nk; ++kt) {
+    const u32x4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
+    u32x4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
+    stage(S0{}, cur, 1);
+    stage(S1{}, cur, 2);
+    // k-step 2, with tile kt + 1 going from registers to LDS
+    // (LDS reads and writes keep their program order, so they alternate in the source)
+    {
+      using LA = TileLoader<BM, A_KC, FAST>;
+      using LB = TileLoader<BN, B_KC, FAST>;
+      constexpr int NPA = LA::NPIECE, NP = LA::NPIECE + LB::NPIECE;
+      constexpr int PER = (NP + NFRAG - 1) / NFRAG;
+      static_for<NFRAG>([&](auto r) {
+        read_frag(S1{}, r, cur, 3);
+        static_for<PER>([&](auto e) {
+          constexpr int P = decltype(r)::value * PER + decltype(e)::value;
+          if constexpr (P < NPA) la.template store_piece<P>(nxt);
+          else if constexpr (P < NP) lb.template store_piece<P - NPA>(nxt + BM * 8);
+        });
+      });
+      static_for<NMFMA>([&](auto q) { mfma(S0{}, q); });
+#pragma unroll
+      for (int r = 0; r < NFRAG; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                  // DS read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x200, PER, 0);                // DS writes
+        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / NFRAG - 1, 0);  // MFMA
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 3: fetch tile kt + 2 (the last iteration re-fetches tile nk - 1, unused),
+    // half of the MFMAs, barrier, first fragments of the next tile, the other half
+    {
+      const int64_t k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * 64;
+      la.load(A, g.a_rs, g.a_cs, m0, g.M, k2, g.K, g.a_vec);
+      lb.load(B, g.b_cs, g.b_rs, n0, g.N, k2, g.K, g.b_vec);
+    }
+    static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
+    {
+      constexpr int NL = TileLoader<BM, A_KC, FAST>::NREG + TileLoader<BN, B_KC, FAST>::NREG;
+#pragma unroll
+      for (int q = 0; q < NMFMA / 2; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x020, (NL + NMFMA / 2 - 1) / (NMFMA / 2), 0);  // VMEM reads
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NFRAG>([&](auto r) { read_frag(S0{}, r, nxt, 0); });
+    static_for<NMFMA / 2>([&](auto q) {
+      mfma(S1{}, std::integral_constant<int, decltype(q)::value + NMFMA / 2>{});
+    });
+#pragma unroll
+    for (int r = 0; r < NFRAG; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, (NMFMA / 2 + NFRAG - 1) / NFRAG, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    // last tile: nothing left to stage
+    const u32x4* cur = gemm_lds + ((nk - 1) & 1) * TILE_CHUNKS;
+    stage(S0{}, cur, 1);
+    stage(S1{}, cur, 2);
+    stage(S0{}, cur, 3);
+    static_for<NMFMA>([&](auto q) { mfma(S1{}, q); });
+  }
+  __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
 
   // Epilogue.  D[i][j] of a 32x32 MFMA tile lives in lane (j, (i / 4) % 2),
   // register (i / 8) * 4 + i % 4.  Each wave passes its accumulators through a
@@ -518,7 +625,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs);
   if (d->dtype_ab == NBK_BF16) {
-    const bool fast = a.a_vec && a.b_vec && (d->K % 8 == 0) && (akc || d->M % 8 == 0) &&
+    const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
     if (!fast) return launch_bf16<128, 128, false>(a, akc, bkc, d->batch, st);
     const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
