@@ -52,7 +52,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 3
+#define NBK_ABI_VERSION 4
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -238,8 +238,14 @@ int nbk_conv2d_fwd(const nbk_conv_desc* d, const void* x, const void* w,
                    const void* bias, void* y, void* stream);
 int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const void* w,
                      void* dx, void* stream);
+/* The filter gradient contracts over every output pixel of the batch, so it is
+ * computed in K slices whose partial sums go to `workspace` (device memory,
+ * 16-byte aligned, nbk_conv2d_wgrad_workspace(d) bytes; contents undefined on
+ * return) and are then added in a fixed order.  With workspace == NULL or too
+ * small the product runs unsplit: same result up to summation order, slower. */
+int64_t nbk_conv2d_wgrad_workspace(const nbk_conv_desc* d);
 int nbk_conv2d_wgrad(const nbk_conv_desc* d, const void* x, const void* dy,
-                     void* dw, void* stream);
+                     void* dw, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* max_pool2d forward/backward; replaces the per-window slice + reduce_max +
  * stack graph of nabla/ops/pooling.py:53-137.  Backward follows the

@@ -154,6 +154,12 @@ class BoundPlan:
                 if k == "conv2d" and not a["has_bias"]:
                     refs.append(None)
                 refs.append(a["dst"])
+                extra = []
+                if k == "conv2d_wgrad":
+                    ws = a.get("workspace")
+                    refs.append(ws)
+                    extra = [C.c_int64(a.get("workspace_bytes", 0) if ws is not None else 0)]
+                    n_ptr = 4
                 names = []
                 for i, r in enumerate(refs):
                     nm = f"p{i}"
@@ -164,7 +170,7 @@ class BoundPlan:
                         ptr_field(holder, nm, r.buf, r.offset * r.dtype.size_in_bytes)
                 fn = {"conv2d": L.nbk_conv2d_fwd, "conv2d_dgrad": L.nbk_conv2d_dgrad,
                       "conv2d_wgrad": L.nbk_conv2d_wgrad}[k]
-                self.calls.append((fn, [C.byref(d), holder, tuple(names[:n_ptr])], patches, d))
+                self.calls.append((fn, [C.byref(d), holder, tuple(names[:n_ptr]), *extra], patches, d))
             elif k in ("maxpool2d", "maxpool2d_bwd"):
                 d = lib.PoolDesc()
                 xs, ys = a["x_shape"], a["y_shape"]

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 MAX_RANK = 8
 
@@ -114,8 +114,9 @@ _SIGNATURES = {
                         C.c_void_p], C.c_int),
     "nbk_conv2d_dgrad": ([C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p],
                          C.c_int),
-    "nbk_conv2d_wgrad": ([C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p],
-                         C.c_int),
+    "nbk_conv2d_wgrad_workspace": ([C.POINTER(ConvDesc)], C.c_int64),
+    "nbk_conv2d_wgrad": ([C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                          C.c_int64, C.c_void_p], C.c_int),
     "nbk_maxpool2d_fwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_maxpool2d_bwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                            C.c_void_p], C.c_int),

@@ -32,6 +32,19 @@ FUSABLE = ("ew", "reduce", "tril", "iota")
 VIEW_KINDS = ("reshape", "broadcast", "permute", "slice")
 
 
+def _wgrad_workspace_bytes(xs, ws, ys, n_cus: int = 256) -> int:
+    """Scratch for the K-split partial sums of the filter gradient; the same rule as
+    nbk_conv2d_wgrad_workspace() for a 256-CU device (the kernel falls back to an
+    unsplit product if it is handed less than it wants)."""
+    r, s_, cin, cout = ws
+    m, k = r * s_ * cin, ys[0] * ys[1] * ys[2]
+    tiles = ((m + 127) // 128) * ((cout + 127) // 128)
+    want = max(1, min((2 * n_cus + tiles - 1) // tiles, max(k // 64, 1)))
+    kps = ((k + want - 1) // want + 15) // 16 * 16
+    splits = (k + kps - 1) // kps
+    return 0 if splits <= 1 else splits * m * cout * 4
+
+
 class FusionLimit(Exception):
     """A fused group does not fit the row-program limits; planning retries smaller."""
 
@@ -688,9 +701,18 @@ class Planner:
                 xs, ws, ys = out.shape, n.inputs[1].shape, n.inputs[0].shape
             else:
                 xs, ws, ys = n.inputs[0].shape, out.shape, n.inputs[1].shape
-            self._emit(Step(k, [i.buf for i in ins], [dst.buf], dict(
-                ins=ins, dst=dst, x_shape=xs, w_shape=ws, y_shape=ys, stride=n.attrs["stride"],
-                padding=n.attrs["padding"], has_bias=n.attrs.get("has_bias", False))))
+            attrs = dict(ins=ins, dst=dst, x_shape=xs, w_shape=ws, y_shape=ys,
+                         stride=n.attrs["stride"], padding=n.attrs["padding"],
+                         has_bias=n.attrs.get("has_bias", False))
+            writes = [dst.buf]
+            if k == "conv2d_wgrad":
+                nbytes = _wgrad_workspace_bytes(xs, ws, ys)
+                if nbytes:
+                    wbuf = self._new_buf((nbytes // 4,), DType.float32, "temp", -1)
+                    attrs["workspace"] = ViewRef(wbuf.id, 0, (nbytes // 4,), (1,), DType.float32)
+                    attrs["workspace_bytes"] = nbytes
+                    writes.append(wbuf.id)
+            self._emit(Step(k, [i.buf for i in ins], writes, attrs))
         elif k in ("maxpool2d", "maxpool2d_bwd"):
             ins = [self._contig(i) for i in n.inputs]
             dst = self._alloc_value(out)

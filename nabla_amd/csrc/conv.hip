@@ -1,14 +1,24 @@
 // conv2d (NHWC x RSCK) forward, input gradient and filter gradient as implicit
-// GEMMs on v_mfma_f32_32x32x2f32.  No im2col buffer is materialised: the A / B
-// tile loaders compute the gather addresses of each 128 x 16 / 16 x 128 tile.
+// GEMMs on v_mfma_f32_32x32x2f32.  No im2col buffer is materialised: the tile
+// loaders gather straight from the image.
 //
-//   forward : M = N*Ho*Wo   Ng = Cout   K = R*S*Cin
+//   forward : M = N*Ho*Wo   Ng = Cout   K = R*S*Cin   (k = (r, s, c), c fastest)
 //             A[m,k] = x[n, ho*sh-pt+r, wo*sw-pl+s, c]      B[k,j] = w[r,s,c,j]
-//   dgrad   : M = N*H*W     Ng = Cin    K = R*S*Cout
+//   dgrad   : M = N*H*W     Ng = Cin    K = R*S*Cout  (k = (r, s, co))
 //             A[m,k] = dy[n, (h+pt-r)/sh, (w+pl-s)/sw, co]  B[k,j] = w[r,s,j,co]
-//   wgrad   : M = R*S*Cin   Ng = Cout   K = N*Ho*Wo
+//   wgrad   : M = R*S*Cin   Ng = Cout   K = N*Ho*Wo   (k = output pixel)
 //             A[m,k] = x[n, ho*sh-pt+r, wo*sw-pl+s, c]      B[k,j] = dy[n,ho,wo,j]
 // Out-of-image taps read zero, which is the zero padding of the reference op.
+//
+// Address arithmetic is kept out of the K loop: a lane owns one output pixel
+// (forward, dgrad) or one run of 8 filter rows (wgrad) for the whole tile and
+// decomposes it once; with channel counts that are multiples of 16 (8 for wgrad)
+// a 16-wide K step lies inside one filter tap, the tap is uniform across the
+// workgroup, and every lane fetches 8 consecutive channels as two 16-byte loads
+// (FAST).  Other channel counts take the element-wise gather.
+// wgrad contracts over every output pixel of the batch while its result is tiny,
+// so it is split along K over blockIdx.z into a workspace and summed by a second
+// kernel in a fixed order (no atomics: results do not depend on scheduling).
 #include "nbk_common.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -20,15 +30,17 @@ struct ConvArgs {
   const float* a;     // x (fwd, wgrad) or dy (dgrad)
   const float* b;     // w (fwd, dgrad) or dy (wgrad)
   const float* bias;  // fwd only
-  float* out;
+  float* out;         // result, or the [splits, M, Ng] workspace when splits > 1
   int64_t M, Ng, K;
-  int32_t tiles_m, tiles_n;
+  int64_t k_per_split;  // multiple of 16
+  int32_t tiles_m, tiles_n, splits;
 };
 
+// ---- element-wise gather (any channel count) ----------------------------------------------
 template <int MODE>
-__device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m, int64_t k) {
+__device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m, int64_t k, int64_t k_end) {
   const nbk_conv_desc& d = g.d;
-  if (m >= g.M || k >= g.K) return 0.f;
+  if (m >= g.M || k >= k_end) return 0.f;
   if (MODE == CONV_FWD) {
     const int64_t c = k % d.Cin;
     const int64_t rs = k / d.Cin;
@@ -65,9 +77,9 @@ __device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m, int64
 }
 
 template <int MODE>
-__device__ __forceinline__ float conv_load_b(const ConvArgs& g, int64_t k, int64_t j) {
+__device__ __forceinline__ float conv_load_b(const ConvArgs& g, int64_t k, int64_t j, int64_t k_end) {
   const nbk_conv_desc& d = g.d;
-  if (k >= g.K || j >= g.Ng) return 0.f;
+  if (k >= k_end || j >= g.Ng) return 0.f;
   if (MODE == CONV_FWD) return g.b[k * d.Cout + j];  // w viewed as [R*S*Cin, Cout]
   if (MODE == CONV_DGRAD) {
     const int64_t co = k % d.Cout, rs = k / d.Cout;
@@ -76,13 +88,27 @@ __device__ __forceinline__ float conv_load_b(const ConvArgs& g, int64_t k, int64
   return g.b[k * d.Cout + j];  // dy viewed as [N*Ho*Wo, Cout]
 }
 
-template <int MODE>
+__device__ __forceinline__ void conv_ld8(const float* p, bool ok, float* r) {
+  float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+  if (ok) {
+    v0 = *(const float4*)p;
+    v1 = *(const float4*)(p + 4);
+  }
+  r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+  r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+}
+
+template <int MODE, bool FAST>
 __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
   constexpr int BK = 16, LD = 128 + 4;
   __shared__ float As[2][BK][LD];
   __shared__ float Bs[2][BK][LD];
+  const nbk_conv_desc& d = g.d;
   const int tm_i = blockIdx.x % g.tiles_m, tn_i = blockIdx.x / g.tiles_m;
   const int64_t m0 = (int64_t)tm_i * 128, n0 = (int64_t)tn_i * 128;
+  const int64_t k_begin = (int64_t)blockIdx.z * g.k_per_split;
+  const int64_t k_end = min(g.K, k_begin + g.k_per_split);
+  float* out = g.out + (g.splits > 1 ? (int64_t)blockIdx.z * g.M * g.Ng : 0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
   const int li = lane & 31, kg = lane >> 5;
@@ -93,45 +119,123 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = (f32x16)(0.f);
 
-  // A staging: forward / dgrad walk k fastest (channels are contiguous in
-  // memory), wgrad walks m fastest.  B is always contiguous along j.
+  // ---- per-lane constants of the A gather ----
+  // forward / dgrad: the lane's pixel; wgrad: the lane's first filter row and, as running
+  // state, the pixel of its K column.
+  const int a_row = tid >> 1, a_kk = (tid & 1) * 8;  // fwd / dgrad: pixel row, 8 k
+  const int w_kk = tid >> 4, w_rr = (tid & 15) * 8;  // wgrad: pixel column, 8 filter rows
+  int p_n = 0, p_y = 0, p_x = 0;
+  bool p_ok = false;
+  int f_r = 0, f_s = 0, f_c = 0;
+  bool f_ok = false;
+  if (MODE == CONV_WGRAD) {
+    const int64_t m = m0 + w_rr;
+    f_ok = m < g.M;
+    const int mm = f_ok ? (int)m : 0;
+    f_c = mm % (int)d.Cin;
+    const int rs = mm / (int)d.Cin;
+    f_s = rs % (int)d.S;
+    f_r = rs / (int)d.S;
+    const int64_t px = k_begin + w_kk;  // < 2^31 (checked on the host)
+    p_x = (int)(px % d.Wo);
+    const int t = (int)(px / d.Wo);
+    p_y = t % (int)d.Ho;
+    p_n = t / (int)d.Ho;
+  } else {
+    const int64_t m = m0 + a_row;
+    p_ok = m < g.M;
+    const int mm = p_ok ? (int)m : 0;
+    const int wd = MODE == CONV_FWD ? (int)d.Wo : (int)d.W;
+    const int hd = MODE == CONV_FWD ? (int)d.Ho : (int)d.H;
+    p_x = mm % wd;
+    const int t = mm / wd;
+    p_y = t % hd;
+    p_n = t / hd;
+  }
+
   float ra[8], rb[8];
   auto load_a = [&](int64_t k0) {
     if (MODE == CONV_WGRAD) {
-      const int kk = tid >> 4, rr = (tid & 15) * 8;
+      // pixel (p_n, p_y, p_x) is column k0 + w_kk; taps of rows m0 + w_rr .. + 7
+      const bool k_ok = k0 + w_kk < k_end;
+      if (FAST) {
+        const int h = p_y * d.stride_h - d.pad_t + f_r, w = p_x * d.stride_w - d.pad_l + f_s;
+        const bool ok = f_ok && k_ok && h >= 0 && h < d.H && w >= 0 && w < d.W;
+        conv_ld8(g.a + (((int64_t)p_n * d.H + h) * d.W + w) * d.Cin + f_c, ok, ra);
+      } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ra[e] = conv_load_a<MODE>(g, m0 + rr + e, k0 + kk);
+        for (int e = 0; e < 8; ++e) ra[e] = conv_load_a<MODE>(g, m0 + w_rr + e, k0 + w_kk, k_end);
+      }
+      // advance the pixel by one K step
+      p_x += BK;
+      while (p_x >= d.Wo) {
+        p_x -= (int)d.Wo;
+        if (++p_y >= d.Ho) { p_y = 0; ++p_n; }
+      }
+    } else if (FAST) {
+      const int ck = MODE == CONV_FWD ? (int)d.Cin : (int)d.Cout;
+      const int tap = (int)(k0 / ck), c0 = (int)(k0 - (int64_t)tap * ck) + a_kk;
+      const int r = tap / (int)d.S, s = tap - r * (int)d.S;
+      if (MODE == CONV_FWD) {
+        const int h = p_y * d.stride_h - d.pad_t + r, w = p_x * d.stride_w - d.pad_l + s;
+        const bool ok = p_ok && h >= 0 && h < d.H && w >= 0 && w < d.W;
+        conv_ld8(g.a + (((int64_t)p_n * d.H + h) * d.W + w) * d.Cin + c0, ok, ra);
+      } else {
+        const int hn = p_y + d.pad_t - r, wn = p_x + d.pad_l - s;
+        const int ho = hn / d.stride_h, wo = wn / d.stride_w;
+        const bool ok = p_ok && hn >= 0 && wn >= 0 && ho * d.stride_h == hn &&
+                        wo * d.stride_w == wn && ho < d.Ho && wo < d.Wo;
+        conv_ld8(g.a + (((int64_t)p_n * d.Ho + ho) * d.Wo + wo) * d.Cout + c0, ok, ra);
+      }
     } else {
-      const int row = tid >> 1, kk = (tid & 1) * 8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ra[e] = conv_load_a<MODE>(g, m0 + row, k0 + kk + e);
+      for (int e = 0; e < 8; ++e) ra[e] = conv_load_a<MODE>(g, m0 + a_row, k0 + a_kk + e, k_end);
     }
   };
   auto store_a = [&](float (*S)[LD]) {
     if (MODE == CONV_WGRAD) {
-      const int kk = tid >> 4, rr = (tid & 15) * 8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[kk][rr + e] = ra[e];
+      for (int e = 0; e < 8; ++e) S[w_kk][w_rr + e] = ra[e];
     } else {
-      const int row = tid >> 1, kk = (tid & 1) * 8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[kk + e][row] = ra[e];
+      for (int e = 0; e < 8; ++e) S[a_kk + e][a_row] = ra[e];
     }
   };
   auto load_b = [&](int64_t k0) {
-    const int kk = tid >> 4, jj = (tid & 15) * 8;
+    if (MODE == CONV_DGRAD) {
+      // w[r, s, j, co]: contiguous along k = co for a fixed input channel j
+      const int64_t j = n0 + a_row;
+      if (FAST) {
+        const int tap = (int)(k0 / d.Cout), co = (int)(k0 - (int64_t)tap * d.Cout) + a_kk;
+        conv_ld8(g.b + ((int64_t)tap * d.Cin + j) * d.Cout + co, j < g.Ng, rb);
+      } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) rb[e] = conv_load_b<MODE>(g, k0 + kk, n0 + jj + e);
+        for (int e = 0; e < 8; ++e) rb[e] = conv_load_b<MODE>(g, k0 + a_kk + e, j, k_end);
+      }
+    } else {
+      // [K, Cout] row-major: w for the forward product, dy for wgrad
+      const int64_t k = k0 + w_kk, j = n0 + w_rr;
+      if (FAST) {
+        conv_ld8(g.b + k * d.Cout + j, k < k_end && j < g.Ng, rb);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rb[e] = conv_load_b<MODE>(g, k, j + e, k_end);
+      }
+    }
   };
   auto store_b = [&](float (*S)[LD]) {
-    const int kk = tid >> 4, jj = (tid & 15) * 8;
+    if (MODE == CONV_DGRAD) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) S[kk][jj + e] = rb[e];
+      for (int e = 0; e < 8; ++e) S[a_kk + e][a_row] = rb[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) S[w_kk][w_rr + e] = rb[e];
+    }
   };
 
-  const int64_t nk = (g.K + BK - 1) / BK;
-  load_a(0);
-  load_b(0);
+  const int64_t nk = (k_end - k_begin + BK - 1) / BK;
+  load_a(k_begin);
+  load_b(k_begin);
   store_a(As[0]);
   store_b(Bs[0]);
   __syncthreads();
@@ -139,8 +243,8 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
     const int cur = kt & 1;
     const bool more = kt + 1 < nk;
     if (more) {
-      load_a((kt + 1) * BK);
-      load_b((kt + 1) * BK);
+      load_a(k_begin + (kt + 1) * BK);
+      load_b(k_begin + (kt + 1) * BK);
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 2; ++ks) {
@@ -172,9 +276,19 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t row = m0 + wm + i * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
-        if (col_ok && row < g.M) g.out[row * g.Ng + col] = acc[i][j][r] + bv;
+        if (col_ok && row < g.M) out[row * g.Ng + col] = acc[i][j][r] + bv;
       }
     }
+}
+
+// out[i] = sum over z of partial[z][i], z ascending.
+__global__ __launch_bounds__(256) void conv_sum_partials(const float* partial, float* out,
+                                                         int64_t n, int splits) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += partial[(int64_t)z * n + i];
+    out[i] = s;
+  }
 }
 
 static int conv_check(const nbk_conv_desc* d) {
@@ -190,16 +304,23 @@ static int conv_check(const nbk_conv_desc* d) {
   const int64_t wo = (d->W + d->pad_l + d->pad_r - d->S) / d->stride_w + 1;
   NBK_REQUIRE(ho == d->Ho && wo == d->Wo, "conv2d: output size %lld x %lld does not match %lld x %lld",
               (long long)d->Ho, (long long)d->Wo, (long long)ho, (long long)wo);
+  NBK_REQUIRE(d->N * d->H * d->W < 0x7fffffffLL && d->N * d->Ho * d->Wo < 0x7fffffffLL &&
+                  d->R * d->S * d->Cin < 0x7fffffffLL && d->R * d->S * d->Cout < 0x7fffffffLL,
+              "conv2d: extent beyond 2^31 elements");
   return NBK_OK;
 }
 
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
 template <int MODE>
-static int conv_launch(ConvArgs& a, hipStream_t st) {
+static int conv_launch(ConvArgs& a, bool fast, hipStream_t st) {
   a.tiles_m = (int)((a.M + 127) / 128);
   a.tiles_n = (int)((a.Ng + 127) / 128);
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   NBK_REQUIRE(blocks <= 0x7fffffffLL, "conv2d: launch too large");
-  hipLaunchKernelGGL(conv_kernel<MODE>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  const dim3 grid((unsigned)blocks, 1, (unsigned)a.splits);
+  if (fast) hipLaunchKernelGGL((conv_kernel<MODE, true>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((conv_kernel<MODE, false>), grid, dim3(256), 0, st, a);
   return nbk_check_launch("conv_kernel");
 }
 
@@ -212,7 +333,9 @@ extern "C" int nbk_conv2d_fwd(const nbk_conv_desc* d, const void* x, const void*
   a.d = *d;
   a.a = (const float*)x; a.b = (const float*)w; a.bias = (const float*)bias; a.out = (float*)y;
   a.M = d->N * d->Ho * d->Wo; a.Ng = d->Cout; a.K = d->R * d->S * d->Cin;
-  return conv_launch<CONV_FWD>(a, (hipStream_t)stream);
+  a.splits = 1; a.k_per_split = (a.K + 15) / 16 * 16;
+  const bool fast = d->Cin % 16 == 0 && d->Cout % 8 == 0 && aligned16(x) && aligned16(w);
+  return conv_launch<CONV_FWD>(a, fast, (hipStream_t)stream);
 }
 
 extern "C" int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const void* w, void* dx,
@@ -224,11 +347,37 @@ extern "C" int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const vo
   a.d = *d;
   a.a = (const float*)dy; a.b = (const float*)w; a.bias = nullptr; a.out = (float*)dx;
   a.M = d->N * d->H * d->W; a.Ng = d->Cin; a.K = d->R * d->S * d->Cout;
-  return conv_launch<CONV_DGRAD>(a, (hipStream_t)stream);
+  a.splits = 1; a.k_per_split = (a.K + 15) / 16 * 16;
+  const bool fast = d->Cout % 16 == 0 && aligned16(dy) && aligned16(w);
+  return conv_launch<CONV_DGRAD>(a, fast, (hipStream_t)stream);
+}
+
+// K split of the filter-gradient product: enough workgroups to fill the GPU twice over,
+// at least four K steps each.
+static void wgrad_split(const nbk_conv_desc* d, int* splits, int64_t* k_per_split) {
+  const int64_t M = d->R * d->S * d->Cin, K = d->N * d->Ho * d->Wo;
+  const int64_t tiles = ((M + 127) / 128) * ((d->Cout + 127) / 128);
+  int64_t want = (2 * (int64_t)nbk_num_cus() + tiles - 1) / tiles;
+  const int64_t most = K / 64 > 0 ? K / 64 : 1;
+  if (want > most) want = most;
+  if (want < 1) want = 1;
+  int64_t kps = (K + want - 1) / want;
+  kps = (kps + 15) / 16 * 16;
+  *k_per_split = kps;
+  *splits = (int)((K + kps - 1) / kps);
+}
+
+extern "C" int64_t nbk_conv2d_wgrad_workspace(const nbk_conv_desc* d) {
+  if (conv_check(d) != NBK_OK) return -1;
+  int splits;
+  int64_t kps;
+  wgrad_split(d, &splits, &kps);
+  if (splits <= 1) return 0;
+  return (int64_t)splits * d->R * d->S * d->Cin * d->Cout * (int64_t)sizeof(float);
 }
 
 extern "C" int nbk_conv2d_wgrad(const nbk_conv_desc* d, const void* x, const void* dy, void* dw,
-                                void* stream) {
+                                void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = conv_check(d);
   if (rc) return rc;
   NBK_REQUIRE(x && dy && dw, "conv2d: null pointer");
@@ -236,5 +385,24 @@ extern "C" int nbk_conv2d_wgrad(const nbk_conv_desc* d, const void* x, const voi
   a.d = *d;
   a.a = (const float*)x; a.b = (const float*)dy; a.bias = nullptr; a.out = (float*)dw;
   a.M = d->R * d->S * d->Cin; a.Ng = d->Cout; a.K = d->N * d->Ho * d->Wo;
-  return conv_launch<CONV_WGRAD>(a, (hipStream_t)stream);
+  int splits;
+  int64_t kps;
+  wgrad_split(d, &splits, &kps);
+  const int64_t need = (int64_t)splits * a.M * a.Ng * (int64_t)sizeof(float);
+  if (splits > 1 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))) {
+    splits = 1;  // no room for partial sums: one pass over all of K
+    kps = (a.K + 15) / 16 * 16;
+  }
+  a.splits = splits;
+  a.k_per_split = kps;
+  if (splits > 1) a.out = (float*)workspace;
+  const bool fast = d->Cin % 8 == 0 && d->Cout % 8 == 0 && aligned16(x) && aligned16(dy);
+  rc = conv_launch<CONV_WGRAD>(a, fast, (hipStream_t)stream);
+  if (rc || splits == 1) return rc;
+  const int64_t n = a.M * a.Ng;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(conv_sum_partials, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const float*)workspace, (float*)dw, n, splits);
+  return nbk_check_launch("conv_sum_partials");
 }
