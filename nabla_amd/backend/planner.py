@@ -444,7 +444,12 @@ class Planner:
                             cands.append(g)
                 # groups that read one of the same external tensors over the same domain
                 sib: list[Unit] = []
+                dom_numel = _numel(dom_shape)
                 for i in node.inputs:
+                    # sharing a tensor pays only if it is read at full size: a broadcast scalar
+                    # or bias in common would chain unrelated work into one oversized group
+                    if self._base(i).numel() < dom_numel:
+                        continue
                     for g in by_root.get(self._base(i).id, ()):
                         g = self._find(g)
                         if g.fused and g not in cands and g not in sib:

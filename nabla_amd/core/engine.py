@@ -67,12 +67,23 @@ class ComputeGraph:
         order = []
         leaves: list[TensorImpl] = []
         leaf_ids: dict[int, int] = {}
+        scalar_bufs: dict[int, int] = {}
         seen: set[int] = set()
 
         def visit_leaf(impl: TensorImpl) -> None:
-            if id(impl) not in leaf_ids:
-                leaf_ids[id(impl)] = len(leaves)
-                leaves.append(impl)
+            if id(impl) in leaf_ids:
+                return
+            if not impl.shape:
+                # 0-d constants come from a by-value cache and share their buffer: one graph
+                # input per buffer (engine.py:185-258 dedups inputs by buffer identity), so
+                # that ``x > 0.0`` written in twelve layers is one value, not twelve
+                idx = scalar_bufs.get(id(impl._buffer))
+                if idx is not None:
+                    leaf_ids[id(impl)] = idx
+                    return
+                scalar_bufs[id(impl._buffer)] = len(leaves)
+            leaf_ids[id(impl)] = len(leaves)
+            leaves.append(impl)
 
         for t in targets:
             if t._buffer is not None:
@@ -140,12 +151,13 @@ class ComputeGraph:
 
     # ------------------------------------------------------------------ lower
     @staticmethod
-    def _lower(order, leaves, targets):
+    def _lower(order, leaves, targets, leaf_ids):
         builder = ir.Builder()
         vals: dict[int, ir.Value] = {}
         with ir.building(builder):
-            for impl in leaves:
-                vals[id(impl)] = ir.input(impl.shape, impl.dtype)
+            leaf_vals = [ir.input(impl.shape, impl.dtype) for impl in leaves]
+            for key, idx in leaf_ids.items():
+                vals[key] = leaf_vals[idx]
             for node in order:
                 args = [vals[id(a)] if isinstance(a, TensorImpl) else a for a in node.op_args]
                 try:
@@ -199,7 +211,7 @@ class ComputeGraph:
         if bound is None:
             _STATS["misses"] += 1
             t1 = time.perf_counter()
-            plan = self._lower(order, leaves, targets)
+            plan = self._lower(order, leaves, targets, leaf_ids)
             bound = ex.bind(plan)
             _STATS["lower_ms"] += (time.perf_counter() - t1) * 1e3
             _PLAN_CACHE[key] = bound
