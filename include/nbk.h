@@ -211,6 +211,11 @@ typedef struct nbk_gemm_desc {
   int64_t M, N, K;
   int64_t a_rs, a_cs, b_rs, b_cs, ldc;
   int64_t batch, a_bs, b_bs, c_bs;
+  /* Second batch level: batch index z = zo * batch_inner + zi; operand offsets are
+   * zo * x_bs + zi * x_bs2 (batch_inner <= 1: one level, the *_bs2 are ignored).
+   * This is how [B, S, H, hd] heads are read and written as [B, H] batches of
+   * S x hd matrices without a transposing copy. */
+  int64_t batch_inner, a_bs2, b_bs2, c_bs2;
   int32_t dtype_ab, dtype_c;
   int32_t act;
   int32_t batch_reduce;

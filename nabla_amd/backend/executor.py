@@ -131,6 +131,8 @@ class BoundPlan:
                 d.a_rs, d.a_cs, d.b_rs, d.b_cs = a["a_rs"], a["a_cs"], a["b_rs"], a["b_cs"]
                 d.ldc = a["ldc"]
                 d.batch, d.a_bs, d.b_bs, d.c_bs = a["batch"], a["a_bs"], a["b_bs"], a["c_bs"]
+                d.batch_inner = a.get("batch_inner", 1)
+                d.a_bs2, d.b_bs2, d.c_bs2 = a.get("a_bs2", 0), a.get("b_bs2", 0), a.get("c_bs2", 0)
                 if ra.dtype is not rb.dtype:
                     raise TypeError(f"matmul operands differ in dtype: {ra.dtype} vs {rb.dtype}")
                 d.dtype_ab = ra.dtype.abi

@@ -63,6 +63,7 @@ class GemmDesc(C.Structure):
         ("a_rs", C.c_int64), ("a_cs", C.c_int64), ("b_rs", C.c_int64), ("b_cs", C.c_int64),
         ("ldc", C.c_int64),
         ("batch", C.c_int64), ("a_bs", C.c_int64), ("b_bs", C.c_int64), ("c_bs", C.c_int64),
+        ("batch_inner", C.c_int64), ("a_bs2", C.c_int64), ("b_bs2", C.c_int64), ("c_bs2", C.c_int64),
         ("dtype_ab", C.c_int32), ("dtype_c", C.c_int32),
         ("act", C.c_int32), ("batch_reduce", C.c_int32),
         ("alpha", C.c_float), ("reserved", C.c_int32),

@@ -595,6 +595,11 @@ class Planner:
         for i, v in enumerate(self.b.inputs):
             b = self._new_buf(v.shape, v.dtype, "input", i)
             self.loc[v.id] = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
+        self.skip_nodes: set[int] = set()  # reductions folded into an earlier one
+        self.users: dict[int, list[ir.Node]] = {}
+        for n in nodes:
+            for i in n.inputs:
+                self.users.setdefault(i.id, []).append(n)
         units = self._group(nodes)
         order = self._order(units)
 
@@ -632,6 +637,17 @@ class Planner:
                 outs.append((self._out_done[oi], v.shape, v.dtype))
                 continue
             src = self._resolve(v)
+            if (isinstance(src, ViewRef) and src.offset == 0 and
+                    tuple(src.strides) == tuple(contiguous_strides(v.shape)) and
+                    self.bufs[src.buf].role == "temp" and
+                    self.bufs[src.buf].numel == _numel(v.shape) and
+                    self.bufs[src.buf].dtype is v.dtype):
+                # the output is a reshape of a whole intermediate: that buffer becomes the
+                # output allocation instead of being copied into one
+                tb = self.bufs[src.buf]
+                tb.role, tb.index = "output", oi
+                outs.append((tb.id, v.shape, v.dtype))
+                continue
             b = self._new_buf(v.shape, v.dtype, "output", oi)
             if isinstance(src, Const):
                 self._emit(Step("fill", [], [b.id], dict(buf=b.id, numel=_numel(v.shape),
@@ -764,12 +780,58 @@ class Planner:
         self._emit(Step("copy", [src.buf], [dst.buf], dict(src=src, dst=window)))
 
     def _lower_reduce_mid(self, n: ir.Node) -> None:
+        if n.pos in self.skip_nodes:
+            return
         x = n.inputs[0]
         axis = n.attrs["axis"]
         out = n.outputs[0]
-        src = self._contig(x)
-        outer, red, inner = _numel(x.shape[:axis]), x.shape[axis], _numel(x.shape[axis + 1:])
         kind = n.fn
+        # A chain of keep-dims reductions over neighbouring axes (the un-broadcast of a bias
+        # or norm-weight gradient walks the axes one at a time) is one reduction over the
+        # merged axis: one pass over the input, fp32 accumulation throughout.
+        lo = hi = axis
+        # axis_of[i]: axis of x behind axis i of the value the chain has reached (None for a
+        # size-1 axis that a reshape inserted)
+        axis_of: list = list(range(x.rank))
+        while True:
+            users = self.users.get(out.id, ())
+            if len(users) != 1 or out.id in self._out_pending:
+                break
+            m = users[0]
+            via = None
+            if m.kind == "reshape":
+                # only size-1 axes may come and go
+                keep = [(axis_of[i], d) for i, d in enumerate(out.shape) if d != 1]
+                new_dims = [d for d in m.outputs[0].shape if d != 1]
+                mu = self.users.get(m.outputs[0].id, ())
+                if ([d for _, d in keep] != new_dims or len(mu) != 1 or
+                        m.outputs[0].id in self._out_pending):
+                    break
+                via, m = m, mu[0]
+            if (m.kind != "reduce" or m.fn != kind or m.pos in self.skip_nodes or
+                    m.attrs["axis"] == m.inputs[0].rank - 1 or self._unit(m.pos) is None or
+                    self._unit(m.pos).fused or m.outputs[0].dtype is not out.dtype):
+                break
+            cur_axes = axis_of
+            if via is not None:
+                it = iter(a for a, _ in keep)
+                cur_axes = [next(it) if d != 1 else None for d in via.outputs[0].shape]
+            a2 = cur_axes[m.attrs["axis"]]
+            if a2 is None:
+                break
+            if a2 < lo and all(d == 1 for d in x.shape[a2 + 1:lo]):
+                lo = a2
+            elif a2 > hi and all(d == 1 for d in x.shape[hi + 1:a2]):
+                hi = a2
+            else:
+                break
+            self.skip_nodes.add(m.pos)
+            if via is not None:
+                self.skip_nodes.add(via.pos)
+            axis_of = cur_axes
+            out = m.outputs[0]
+        src = self._contig(x)
+        outer, red, inner = _numel(x.shape[:lo]), _numel(x.shape[lo:hi + 1]), _numel(x.shape[hi + 1:])
         # few output columns and a long axis: split the axis so the launch has
         # enough workgroups, then reduce the partials
         blocks = outer * ((inner + 63) // 64)
@@ -796,9 +858,23 @@ class Planner:
 
     # ................................................................ matmul
     @staticmethod
-    def _mat_operand(ref: ViewRef):
-        """(batch_stride, row_stride, col_stride) if the view is a strided batch
-        of matrices the GEMM can read directly, else None."""
+    def _batch_groups(dims, strides):
+        """Batch dims merged into as few (extent, stride) levels as their strides allow."""
+        groups: list[tuple[int, int]] = []
+        for d, s in zip(dims, strides):
+            if d == 1:
+                continue
+            if groups and (groups[-1][1] == s * d or (groups[-1][1] == 0 and s == 0)):
+                groups[-1] = (groups[-1][0] * d, s)
+            else:
+                groups.append((d, s))
+        return groups
+
+    @classmethod
+    def _mat_operand(cls, ref: ViewRef):
+        """(batch levels, row_stride, col_stride) if the view is a strided batch of
+        matrices the GEMM can read directly (one unit stride, at most two batch
+        levels), else None."""
         shape, st = ref.shape, ref.strides
         rs, cs = st[-2], st[-1]
         r, c = shape[-2], shape[-1]
@@ -808,17 +884,33 @@ class Planner:
             cs = 1 if rs != 1 else (r * rs)
         if rs != 1 and cs != 1:
             return None
-        if rs < 0 or cs < 0:
+        if rs < 0 or cs < 0 or any(s < 0 for s in st[:-2]):
             return None
-        bdims = [(d, s) for d, s in zip(shape[:-2], st[:-2]) if d != 1]
-        if not bdims:
-            return (0, rs, cs)
-        if all(s == 0 for _, s in bdims):
-            return (0, rs, cs)
-        for (d0, s0), (d1, s1) in zip(bdims[:-1], bdims[1:]):
-            if s0 != s1 * d1:
-                return None
-        return (bdims[-1][1], rs, cs)
+        groups = cls._batch_groups(shape[:-2], st[:-2])
+        if len(groups) > 2:
+            return None
+        return (groups, rs, cs)
+
+    def _matmul_out_layout(self, out: ir.Value):
+        """Strides the product should be written with.  When its only reader is a permute
+        that keeps the last axis (heads [B,H,S,hd] going back to [B,S,H,hd]), the GEMM
+        writes that layout directly and the permute becomes a contiguous view."""
+        strides = contiguous_strides(out.shape)
+        if out.id in self._out_pending or out.rank < 3:
+            return strides
+        users = self.users.get(out.id, ())
+        if len(users) != 1 or users[0].kind != "permute":
+            return strides
+        perm = users[0].attrs["perm"]
+        if perm[-1] != out.rank - 1:
+            return strides
+        pst = contiguous_strides(tuple(out.shape[p] for p in perm))
+        cand = [0] * out.rank
+        for i, p in enumerate(perm):
+            cand[p] = pst[i]
+        if len(self._batch_groups(out.shape[:-2], cand[:-2])) > 2 or cand[-2] < out.shape[-1]:
+            return strides
+        return tuple(cand)
 
     def _lower_matmul(self, n: ir.Node) -> None:
         a, b = n.inputs
@@ -838,11 +930,48 @@ class Planner:
             pb = self._mat_operand(rb)
         M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
         batch = _numel(out.shape[:-2])
-        dst = self._alloc_value(out)
+        c_strides = self._matmul_out_layout(out)
+        gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
+        # one (outer, inner) split of the batch index has to serve A, B and C
+        split = None
+        for grp in (gc, pa[0], pb[0]):
+            if len(grp) == 2:
+                split = (grp[0][0], grp[1][0])
+                break
+        if split is not None:
+            if len(pa[0]) == 2 and (pa[0][0][0], pa[0][1][0]) != split:
+                ra = self._materialize(ra)
+                pa = self._mat_operand(ra)
+            if len(pb[0]) == 2 and (pb[0][0][0], pb[0][1][0]) != split:
+                rb = self._materialize(rb)
+                pb = self._mat_operand(rb)
+            if len(gc) == 2 and (gc[0][0], gc[1][0]) != split:
+                c_strides = contiguous_strides(out.shape)
+                gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
+        inner = split[1] if split is not None else 1
+
+        def levels(groups):
+            if not groups:
+                return 0, 0
+            if len(groups) == 2:
+                return groups[0][1], groups[1][1]
+            s = groups[0][1]
+            return (s * inner, s) if inner > 1 else (s, 0)
+
+        a_bs, a_bs2 = levels(pa[0])
+        b_bs, b_bs2 = levels(pb[0])
+        c_bs, c_bs2 = levels(gc)
+        if c_strides == contiguous_strides(out.shape):
+            dst = self._alloc_value(out)
+        else:
+            buf = self._new_buf(out.shape, out.dtype, "temp", -1)
+            dst = ViewRef(buf.id, 0, out.shape, c_strides, out.dtype)
+            self.loc[out.id] = dst
         self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
-            a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch,
-            a_bs=pa[0], a_rs=pa[1], a_cs=pa[2], b_bs=pb[0], b_rs=pb[1], b_cs=pb[2],
-            ldc=N, c_bs=M * N, alpha=1.0)))
+            a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
+            a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
+            a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
+            ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs, alpha=1.0)))
 
     # ................................................................ groups
     def _lower_group(self, g: Unit) -> None:

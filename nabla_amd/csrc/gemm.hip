@@ -40,6 +40,7 @@ struct GemmArgs {
   int64_t M, N, K;
   int64_t a_rs, a_cs, b_rs, b_cs, ldc;
   int64_t a_bs, b_bs, c_bs;
+  int64_t batch_inner, a_bs2, b_bs2, c_bs2;  // batch_inner >= 1
   int32_t dtype_c, act;
   float alpha;
   int32_t tiles_m, tiles_n;
@@ -192,9 +193,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   int tm_i, tn_i;
   gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
   const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
-  const int64_t b = blockIdx.y;
-  const uint16_t* A = (const uint16_t*)g.A + b * g.a_bs;
-  const uint16_t* B = (const uint16_t*)g.B + b * g.b_bs;
+  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
+  const uint16_t* A = (const uint16_t*)g.A + bo * g.a_bs + bi * g.a_bs2;
+  const uint16_t* B = (const uint16_t*)g.B + bo * g.b_bs + bi * g.b_bs2;
+  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
   const int li = lane & 31, kg = lane >> 5;
@@ -374,7 +376,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
   const int sub_r = lane / LANES_PER_ROW, sub_c = (lane % LANES_PER_ROW) * 8;
   const int64_t col = n0 + wn + sub_c;
-  const bool vec_store = FAST && (col + 8 <= g.N) && ((g.ldc & 7) == 0) && ((g.c_bs & 7) == 0);
+  const bool vec_store = FAST && (col + 8 <= g.N) && ((g.ldc & 7) == 0) && ((g.c_bs & 7) == 0) &&
+                         ((g.c_bs2 & 7) == 0);
   float bias_v[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) bias_v[e] = 0.f;
@@ -404,7 +407,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
       v[0] = p0.x; v[1] = p0.y; v[2] = p0.z; v[3] = p0.w;
       v[4] = p1.x; v[5] = p1.y; v[6] = p1.z; v[7] = p1.w;
       if (row < g.M && col < g.N) {
-        const int64_t idx = b * g.c_bs + row * g.ldc + col;
+        const int64_t idx = c_off + row * g.ldc + col;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
         if (EPI) {
@@ -450,9 +453,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
   int tm_i, tn_i;
   gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
   const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
-  const int64_t b = blockIdx.y;
-  const float* A = (const float*)g.A + b * g.a_bs;
-  const float* B = (const float*)g.B + b * g.b_bs;
+  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
+  const float* A = (const float*)g.A + bo * g.a_bs + bi * g.a_bs2;
+  const float* B = (const float*)g.B + bo * g.b_bs + bi * g.b_bs2;
+  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
   const int li = lane & 31, kg = lane >> 5;
@@ -545,7 +549,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
         const int64_t row = m0 + wm + i * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
         if (row >= g.M) continue;
         float v = gemm_act(acc[i][j][r] * g.alpha + bv, g.act);
-        const int64_t idx = b * g.c_bs + row * g.ldc + col;
+        const int64_t idx = c_off + row * g.ldc + col;
         if (g.residual) v += ((const float*)g.residual)[idx];
         C[idx] = v;
       }
@@ -613,17 +617,23 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.M = d->M; a.N = d->N; a.K = d->K;
   a.a_rs = d->a_rs; a.a_cs = d->a_cs; a.b_rs = d->b_rs; a.b_cs = d->b_cs; a.ldc = d->ldc;
   a.a_bs = d->a_bs; a.b_bs = d->b_bs; a.c_bs = d->c_bs;
+  a.batch_inner = d->batch_inner > 1 ? d->batch_inner : 1;
+  NBK_REQUIRE(d->batch % a.batch_inner == 0, "gemm: batch %lld is not a multiple of batch_inner %lld",
+              (long long)d->batch, (long long)a.batch_inner);
+  a.a_bs2 = a.batch_inner > 1 ? d->a_bs2 : 0;
+  a.b_bs2 = a.batch_inner > 1 ? d->b_bs2 : 0;
+  a.c_bs2 = a.batch_inner > 1 ? d->c_bs2 : 0;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;
   const int esz = d->dtype_ab == NBK_F32 ? 4 : 2;
-  auto vec_ok = [&](const void* p, int64_t other_stride, int64_t bs) {
+  auto vec_ok = [&](const void* p, int64_t other_stride, int64_t bs, int64_t bs2) {
     const int64_t q = 16 / esz;
-    return ((uintptr_t)p % 16 == 0) && (other_stride % q == 0) && (bs % q == 0);
+    return ((uintptr_t)p % 16 == 0) && (other_stride % q == 0) && (bs % q == 0) && (bs2 % q == 0);
   };
-  a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs);
-  a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs);
+  a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs, a.a_bs2);
+  a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs, a.b_bs2);
   if (d->dtype_ab == NBK_BF16) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;

@@ -185,14 +185,17 @@ def _view(mem, ref: ViewRef) -> torch.Tensor:
 
 
 def _gemm(a, mem):
-    def mat(ref, bs, rs, cs, rows, cols):
+    bi = max(1, a.get("batch_inner", 1))
+    bo = a["batch"] // bi
+
+    def mat(ref, bs, bs2, rs, cs, rows, cols):
         base = mem[ref.buf]
-        return torch.as_strided(base, (a["batch"], rows, cols), (bs, rs, cs), ref.offset).float()
-    A = mat(a["a"], a["a_bs"], a["a_rs"], a["a_cs"], a["M"], a["K"])
-    B = mat(a["b"], a["b_bs"], a["b_rs"], a["b_cs"], a["K"], a["N"])
+        return torch.as_strided(base, (bo, bi, rows, cols), (bs, bs2 if bi > 1 else 0, rs, cs), ref.offset)
+    A = mat(a["a"], a["a_bs"], a.get("a_bs2", 0), a["a_rs"], a["a_cs"], a["M"], a["K"]).float()
+    B = mat(a["b"], a["b_bs"], a.get("b_bs2", 0), a["b_rs"], a["b_cs"], a["K"], a["N"]).float()
     C = torch.matmul(A.double(), B.double()).float() * a.get("alpha", 1.0)
     dst = a["dst"]
-    out = torch.as_strided(mem[dst.buf], (a["batch"], a["M"], a["N"]), (a["c_bs"], a["ldc"], 1), dst.offset)
+    out = mat(dst, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"])
     out.copy_(C.to(out.dtype))
 
 
