@@ -556,6 +556,102 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     }
 }
 
+// --------------------------------------------------------------- fp32, small problems
+// A product with only a handful of 128 x 128 tiles (the layers of a small MLP, a
+// classifier head) leaves most of the GPU idle and is bound by the latency of one
+// workgroup's K loop.  Here a workgroup owns a 32 x 32 tile of C, its four waves
+// split K between them (wave w takes k-steps w, w + 4, ...), operands go from global
+// memory straight to the MFMA registers in chunks of 8 k-steps that are all in
+// flight together while the previous chunk is multiplied, and the four partial
+// tiles meet in LDS.
+// Lane l of a v_mfma_f32_32x32x2f32 supplies A[row l % 32][k = l / 32] and
+// B[k = l / 32][col l % 32]; which two k values share an instruction is free as
+// long as A and B agree, so the lane with half h = l / 32 owns k = kb + 4h .. 4h + 3
+// of every 8-wide step and issues four instructions per step.
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_f32_small_kernel(const GemmArgs g) {
+  constexpr int U = 8;  // k-steps (of 8) per chunk
+  __shared__ float part[4][32][33];
+  const int tn_i = blockIdx.x % g.tiles_n, tm_i = blockIdx.x / g.tiles_n;
+  const int64_t m0 = (int64_t)tm_i * 32, n0 = (int64_t)tn_i * 32;
+  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
+  const float* A = (const float*)g.A + bo * g.a_bs + bi * g.a_bs2;
+  const float* B = (const float*)g.B + bo * g.b_bs + bi * g.b_bs2;
+  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 31, h = lane >> 5;
+  const int64_t m = m0 + li, n = n0 + li;
+  const bool m_ok = m < g.M, n_ok = n < g.N;
+  const float* a_base = A_KC ? A + (m_ok ? m : 0) * g.a_rs : A + (m_ok ? m : 0);
+  const float* b_base = B_KC ? B + (n_ok ? n : 0) * g.b_cs : B + (n_ok ? n : 0);
+  const int64_t K = g.K;
+  // k-steps of this wave: s = wave + 4 * i, covering k in [8 s, 8 s + 8)
+  const int64_t n_steps = (K + 7) / 8;
+  const int64_t my_steps = n_steps > wave ? (n_steps - wave + 3) / 4 : 0;
+
+  auto fetch = [&](int64_t i, float* a, float* b) {
+    const int64_t kb = (wave + 4 * i) * 8 + 4 * h;
+    const bool in = i < my_steps;
+    if (A_KC) {
+      if (in && m_ok && g.a_vec && kb + 3 < K) {
+        const float4 v = *(const float4*)(a_base + kb);
+        a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = (in && m_ok && kb + j < K) ? a_base[kb + j] : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[j] = (in && m_ok && kb + j < K) ? a_base[(kb + j) * g.a_cs] : 0.f;
+    }
+    if (B_KC) {
+      if (in && n_ok && g.b_vec && kb + 3 < K) {
+        const float4 v = *(const float4*)(b_base + kb);
+        b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = (in && n_ok && kb + j < K) ? b_base[kb + j] : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = (in && n_ok && kb + j < K) ? b_base[(kb + j) * g.b_rs] : 0.f;
+    }
+  };
+
+  f32x16 acc = (f32x16)(0.f);
+  float ca[U][4], cb[U][4], na[U][4], nb[U][4];
+#pragma unroll
+  for (int u = 0; u < U; ++u) fetch(u, ca[u], cb[u]);
+  for (int64_t c0 = 0; c0 < my_steps; c0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) fetch(c0 + U + u, na[u], nb[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[u][j], cb[u][j], acc, 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { ca[u][j] = na[u][j]; cb[u][j] = nb[u][j]; }
+  }
+  // D register r of lane (col li, half h) is row (r / 4) * 8 + h * 4 + r % 4
+#pragma unroll
+  for (int r = 0; r < 16; ++r) part[wave][(r >> 2) * 8 + h * 4 + (r & 3)][li] = acc[r];
+  __syncthreads();
+  float* C = (float*)g.C;
+  for (int e = threadIdx.x; e < 32 * 32; e += 256) {
+    const int r = e >> 5, c = e & 31;
+    const int64_t row = m0 + r, col = n0 + c;
+    if (row >= g.M || col >= g.N) continue;
+    float v = (part[0][r][c] + part[1][r][c]) + (part[2][r][c] + part[3][r][c]);
+    v = gemm_act(v * g.alpha + (g.bias ? ((const float*)g.bias)[col] : 0.f), g.act);
+    const int64_t idx = c_off + row * g.ldc + col;
+    if (g.residual) v += ((const float*)g.residual)[idx];
+    C[idx] = v;
+  }
+}
+
 // ------------------------------------------------------------------------- dispatch
 template <int BM, int BN, bool FAST>
 static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
@@ -645,6 +741,17 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   }
   a.tiles_m = (int)((d->M + 127) / 128);
   a.tiles_n = (int)((d->N + 127) / 128);
+  if ((int64_t)a.tiles_m * a.tiles_n * d->batch <= 32) {
+    // too few big tiles to occupy the GPU: 32 x 32 tiles with K split inside the workgroup
+    a.tiles_m = (int)((d->M + 31) / 32);
+    a.tiles_n = (int)((d->N + 31) / 32);
+    dim3 sgrid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)d->batch);
+    if (akc && bkc) hipLaunchKernelGGL((gemm_f32_small_kernel<true, true>), sgrid, dim3(256), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((gemm_f32_small_kernel<true, false>), sgrid, dim3(256), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((gemm_f32_small_kernel<false, true>), sgrid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_f32_small_kernel<false, false>), sgrid, dim3(256), 0, st, a);
+    return nbk_check_launch("gemm_f32_small_kernel");
+  }
   dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)d->batch);
   if (akc && bkc) hipLaunchKernelGGL((gemm_f32_kernel<true, true>), grid, dim3(256), 0, st, a);
   else if (akc) hipLaunchKernelGGL((gemm_f32_kernel<true, false>), grid, dim3(256), 0, st, a);
