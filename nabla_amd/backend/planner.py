@@ -833,13 +833,15 @@ class Planner:
         src = self._contig(x)
         outer, red, inner = _numel(x.shape[:lo]), _numel(x.shape[lo:hi + 1]), _numel(x.shape[hi + 1:])
         # few output columns and a long axis: split the axis so the launch has
-        # enough workgroups, then reduce the partials
-        blocks = outer * ((inner + 63) // 64)
+        # enough workgroups, then reduce the partials.  A workgroup covers 64 lanes x
+        # one 16-byte vector of columns and wants about 64 rows (16 per wave).
+        vec = 16 // x.dtype.size_in_bytes if inner % (16 // x.dtype.size_in_bytes) == 0 else 1
+        blocks = outer * ((inner + 64 * vec - 1) // (64 * vec))
         split = 1
         if blocks < 256 and red >= 256:
-            want = min(64, max(1, 1024 // max(blocks, 1)))
+            want = min(256, red // 64, max(1, 1024 // max(blocks, 1)))
             for s in range(want, 1, -1):
-                if red % s == 0 and red // s >= 16 and outer * s <= 65535:
+                if red % s == 0 and outer * s <= 65535:
                     split = s
                     break
         if split > 1:

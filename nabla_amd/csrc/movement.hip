@@ -189,6 +189,65 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict_
   }
 }
 
+// Vector form: a lane owns VEC consecutive columns (16 bytes of input per row), a
+// workgroup 64 * VEC columns; its four waves take every fourth row and keep eight
+// row loads in flight each.  T is the input element (uint16_t = bf16, float).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
+                                                             void* __restrict__ out, int dto,
+                                                             int64_t red, int64_t inner, int kind) {
+  __shared__ float part[4][64][VEC + 1];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t o = blockIdx.y;
+  const int64_t col = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const float ident = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = ident;
+  if (col < inner) {
+    const T* base = in + o * red * inner + col;
+    auto load = [&](int64_t r, float* v) {
+      const uint4 u = *(const uint4*)(base + r * inner);
+      if (sizeof(T) == 2) {
+        v[0] = __uint_as_float(u.x << 16); v[1] = __uint_as_float(u.x & 0xffff0000u);
+        v[2] = __uint_as_float(u.y << 16); v[3] = __uint_as_float(u.y & 0xffff0000u);
+        v[4 % VEC] = __uint_as_float(u.z << 16); v[5 % VEC] = __uint_as_float(u.z & 0xffff0000u);
+        v[6 % VEC] = __uint_as_float(u.w << 16); v[7 % VEC] = __uint_as_float(u.w & 0xffff0000u);
+      } else {
+        v[0] = __uint_as_float(u.x); v[1] = __uint_as_float(u.y);
+        v[2] = __uint_as_float(u.z); v[3] = __uint_as_float(u.w);
+      }
+    };
+    int64_t r = w;
+    for (; r + 28 < red; r += 32) {
+      float v[8][VEC];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) load(r + 4 * q, v[q]);
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = red_comb(acc[e], v[q][e], kind);
+    }
+    for (; r < red; r += 4) {
+      float v[VEC];
+      load(r, v);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = red_comb(acc[e], v[e], kind);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) part[w][lane][e] = acc[e];
+  __syncthreads();
+  if (w == 0 && col < inner) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float v = red_comb(red_comb(part[0][lane][e], part[1][lane][e], kind),
+                               red_comb(part[2][lane][e], part[3][lane][e], kind), kind);
+      nbk_store_from_f32(out, o * inner + col + e, dto, v);
+    }
+  }
+}
+
 extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
                               int64_t red, int64_t inner, int32_t kind, void* stream) {
   NBK_REQUIRE(in && out, "reduce_mid: null pointer");
@@ -196,6 +255,19 @@ extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dt
   NBK_REQUIRE(kind >= NBK_RED_SUM && kind <= NBK_RED_MIN, "reduce_mid: kind %d", kind);
   NBK_REQUIRE(nbk_dtype_size(dti) > 0 && nbk_dtype_size(dto) > 0, "reduce_mid: bad dtype");
   NBK_REQUIRE(outer <= 65535, "reduce_mid: outer %lld exceeds the grid limit", (long long)outer);
+  const bool aligned = ((uintptr_t)in & 15) == 0;
+  if (dti == NBK_BF16 && inner % 8 == 0 && aligned) {
+    dim3 grid((unsigned)((inner / 8 + 63) / 64), (unsigned)outer);
+    hipLaunchKernelGGL((reduce_mid_vec_kernel<uint16_t, 8>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)in, out, dto, red, inner, kind);
+    return nbk_check_launch("reduce_mid_vec_kernel");
+  }
+  if (dti == NBK_F32 && inner % 4 == 0 && aligned) {
+    dim3 grid((unsigned)((inner / 4 + 63) / 64), (unsigned)outer);
+    hipLaunchKernelGGL((reduce_mid_vec_kernel<float, 4>), grid, dim3(256), 0, (hipStream_t)stream,
+                       (const float*)in, out, dto, red, inner, kind);
+    return nbk_check_launch("reduce_mid_vec_kernel");
+  }
   dim3 grid((unsigned)((inner + 63) / 64), (unsigned)outer);
   hipLaunchKernelGGL(reduce_mid_kernel, grid, dim3(256), 0, (hipStream_t)stream, in, out, dti, dto,
                      red, inner, kind);
