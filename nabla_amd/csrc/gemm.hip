@@ -35,6 +35,11 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// Part i of `total` items dealt as evenly as possible into `parts` consecutive shares.
+constexpr int share(int total, int parts, int i) {
+  return total * (i + 1) / parts - total * i / parts;
+}
+
 struct GemmArgs {
   const void* A; const void* B; void* C; const void* bias; const void* residual;
   int64_t M, N, K;
@@ -274,11 +279,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
     });
     static_for<NMFMA>([&](auto q) { mfma(set, q); });
     // interleave: one fragment read, then its share of the MFMAs
-#pragma unroll
-    for (int r = 0; r < NFRAG; ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
-      __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / NFRAG, 0);  // MFMAs
-    }
+    static_for<NFRAG>([&](auto r) {
+      constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);  // MFMAs
+    });
     __builtin_amdgcn_sched_barrier(0);  // later stages' work (and its waits) stays behind
   };
 
@@ -311,13 +316,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
         });
       });
       static_for<NMFMA>([&](auto q) { mfma(S0{}, q); });
-#pragma unroll
-      for (int r = 0; r < NFRAG; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                  // DS read
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x200, PER, 0);                // DS writes
-        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / NFRAG - 1, 0);  // MFMA
-      }
+      static_for<NFRAG>([&](auto r) {
+        constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x200, PER, 0);  // DS writes
+        if constexpr (n > 1) __builtin_amdgcn_sched_group_barrier(0x008, n - 1, 0);  // MFMA
+      });
     }
     __builtin_amdgcn_sched_barrier(0);
     // k-step 3: fetch tile kt + 2 (the last iteration re-fetches tile nk - 1, unused),
@@ -330,11 +335,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
     static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
     {
       constexpr int NL = TileLoader<BM, A_KC, FAST>::NREG + TileLoader<BN, B_KC, FAST>::NREG;
-#pragma unroll
-      for (int q = 0; q < NMFMA / 2; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x020, (NL + NMFMA / 2 - 1) / (NMFMA / 2), 0);  // VMEM reads
+      static_for<NMFMA / 2>([&](auto q) {
+        constexpr int n = share(NL, NMFMA / 2, decltype(q)::value);
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);  // VMEM reads
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
+      });
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -345,11 +350,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const GemmArgs g) {
     static_for<NMFMA / 2>([&](auto q) {
       mfma(S1{}, std::integral_constant<int, decltype(q)::value + NMFMA / 2>{});
     });
-#pragma unroll
-    for (int r = 0; r < NFRAG; ++r) {
+    static_for<NFRAG>([&](auto r) {
+      constexpr int n = share(NMFMA / 2, NFRAG, decltype(r)::value);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, (NMFMA / 2 + NFRAG - 1) / NFRAG, 0);
-    }
+      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);
+    });
     __builtin_amdgcn_sched_barrier(0);
   }
   {
@@ -737,6 +742,9 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
     if (big_tiles >= 384 && d->M >= 256 && d->N >= 256)
       return launch_bf16<256, 256, true>(a, akc, bkc, d->batch, st);
+    // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
+    // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
+    // 128 x 128 workgroups hide it better)
     return launch_bf16<128, 128, true>(a, akc, bkc, d->batch, st);
   }
   a.tiles_m = (int)((d->M + 127) / 128);
