@@ -739,8 +739,13 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
     if (!fast) return launch_bf16<128, 128, false>(a, akc, bkc, d->batch, st);
+    // 256 x 256 tiles run at about twice the rate of 128 x 128 ones per CU, one workgroup
+    // per CU at a time: take them when the rounds of workgroups they need are at least
+    // 60 % full (256 tiles on 256 CUs is the ideal case, 128 or 300 tiles are not).
     const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
-    if (big_tiles >= 384 && d->M >= 256 && d->N >= 256)
+    const int64_t cus = nbk_num_cus();
+    const int64_t rounds = (big_tiles + cus - 1) / cus;
+    if (big_tiles * 10 >= rounds * cus * 6 && d->M >= 256 && d->N >= 256)
       return launch_bf16<256, 256, true>(a, akc, bkc, d->batch, st);
     // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
     // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
