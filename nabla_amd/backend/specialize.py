@@ -67,23 +67,25 @@ def _as_vec(r: int) -> str:
     return f"v{r}" if r < isa.NVEC else f"rp_splat(s{r})"
 
 
-def _ew_vec(op: int, dst: int, a: int, b: int, c: int) -> str:
+def _ew_vec(op: int, dst: int, a: int, b: int, c: int, lowp: bool = False) -> str:
     name = isa.EW_NAME[op]
+    lp = ", true" if lowp else ""
     if name in isa.UNARY:
-        return f"v{dst} = rp_un4<{op}>({_as_vec(a)});"
+        return f"v{dst} = rp_un4<{op}{lp}>({_as_vec(a)});"
     if name in isa.BINARY:
-        return f"v{dst} = rp_bin4<{op}>({_as_vec(a)}, {_as_vec(b)});"
+        return f"v{dst} = rp_bin4<{op}{lp}>({_as_vec(a)}, {_as_vec(b)});"
     if name == "where":
         return f"v{dst} = rp_where4({_as_vec(a)}, {_as_vec(b)}, {_as_vec(c)});"
     return f"v{dst} = rp_fma4({_as_vec(a)}, {_as_vec(b)}, {_as_vec(c)});"
 
 
-def _ew_scalar(op: int, dst: int, a: int, b: int, c: int) -> str:
+def _ew_scalar(op: int, dst: int, a: int, b: int, c: int, lowp: bool = False) -> str:
     name = isa.EW_NAME[op]
+    lp = "_lowp" if lowp else ""
     if name in isa.UNARY:
-        return f"s{dst} = rp_unary({op}, s{a});"
+        return f"s{dst} = rp_unary{lp}({op}, s{a});"
     if name in isa.BINARY:
-        return f"s{dst} = rp_binary({op}, s{a}, s{b});"
+        return f"s{dst} = rp_binary{lp}({op}, s{a}, s{b});"
     if name == "where":
         return f"s{dst} = s{a} != 0.f ? s{b} : s{c};"
     return f"s{dst} = fmaf(s{a}, s{b}, s{c});"
@@ -113,6 +115,9 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
     resident = cpt > 0
     assert not resident or block_mode
     inputs = full_inputs(a)
+    # every stored tensor a 16-bit float: hardware transcendentals are accurate enough
+    stored = {i[1] for i in ins if i[0] in (isa.STR, isa.STG)}
+    lowp = bool(stored) and all(ops[k].dtype.abi in (1, 2) for k in stored)
     L: list[str] = []
     w = L.append
     if block_mode:
@@ -218,11 +223,19 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         w("    uint32_t lead_idx[4];")
         w("    " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
     else:
+        # scalar operands that do not move with the row (constants such as 0.5 or 1/sqrt(2)) are
+        # read once, not once per chunk
+        for k in hoisted:
+            w(f"  const bool uni{k} = (o{k}.lead_stride[0] | o{k}.lead_stride[1] | o{k}.lead_stride[2] | "
+              f"o{k}.lead_stride[3]) == 0;")
+            w(f"  const float pre{k} = uni{k} ? nbk_load_as_f32(o{k}.ptr, 0, o{k}.dtype) : 0.f;")
         w("  const uint64_t stride = (uint64_t)gridDim.x * 256u;")
+        w("  const bool small = total_chunks <= 0xffffffffull;  // 32-bit row arithmetic suffices")
         w("  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {")
         w("    uint32_t row, cc;")
         w("    if (cpr == 1) { row = (uint32_t)g; cc = 0; }")
         w("    else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }")
+        w("    else if (small) { row = (uint32_t)g / cpr; cc = (uint32_t)g - row * cpr; }")
         w("    else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }")
         w("    uint32_t lead_idx[4] = {0, 0, 0, 0};")
         w("    if (P.n_lead > 0) " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
@@ -231,10 +244,23 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         w("    const int64_t left = C - col;")
         w("    const int valid = left >= 4 ? 4 : (int)left;")
     if not resident:
-        for k in range(len(ops)):
-            w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
-        for k in hoisted:
-            w(f"    const float ldr{k} = nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
+        if block_mode:
+            for k in range(len(ops)):
+                w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
+            for k in hoisted:
+                w(f"    const float ldr{k} = nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
+        else:
+            # per-lane rows: with at most one leading dim an offset is one multiply-add
+            w("    int64_t " + ", ".join(f"off{k}" for k in range(len(ops))) + ";")
+            w("    if (P.n_lead <= 1) {")
+            for k in range(len(ops)):
+                w(f"      off{k} = (int64_t)lead_idx[0] * o{k}.lead_stride[0];")
+            w("    } else {")
+            for k in range(len(ops)):
+                w(f"      off{k} = rp_row_offset(o{k}, lead_idx, 4);")
+            w("    }")
+            for k in hoisted:
+                w(f"    const float ldr{k} = uni{k} ? pre{k} : nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
         if block_mode and a["n_stage"] > 0:
             for k, o in enumerate(ops):
                 if o.stage_slot >= 0:
@@ -293,7 +319,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                     w(ind + f"v{bd} = make_float4((float)col, (float)col + 1.f, (float)col + 2.f, "
                       "(float)col + 3.f);")
                 else:
-                    w(ind + _ew_vec(bop, bd, bx, by, bz))
+                    w(ind + _ew_vec(bop, bd, bx, by, bz, lowp))
             w("    }")
             pc += 1 + aux
             continue
@@ -325,7 +351,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
             pc += n
             continue
         else:
-            w("    " + _ew_scalar(op, dst, x, y, z))
+            w("    " + _ew_scalar(op, dst, x, y, z, lowp))
         pc += 1
     w("  }")
     w("}")

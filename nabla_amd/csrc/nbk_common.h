@@ -57,12 +57,10 @@ static inline int nbk_dtype_size(int dt) {
 __device__ __forceinline__ float nbk_bf16_to_f32(uint16_t h) {
   return __uint_as_float(((uint32_t)h) << 16);
 }
-// round-to-nearest-even, NaN kept quiet; branch-free so that unrolled epilogues stay small
+// round-to-nearest-even, NaN kept quiet: one hardware conversion (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t nbk_f32_to_bf16(float f) {
-  const uint32_t u = __float_as_uint(f);
-  const uint32_t rounded = u + 0x7fffu + ((u >> 16) & 1u);
-  const uint32_t quiet = u | 0x00400000u;
-  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded) >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, b);
 }
 __device__ __forceinline__ float nbk_load_as_f32(const void* p, int64_t i, int dt) {
   switch (dt) {

@@ -158,6 +158,39 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
   }
 }
 
+// Reduced-precision forms for programs whose every stored tensor is a 16-bit float:
+// hardware exp2 / log2 / rcp / rsq (about 1e-6 relative) and a five-term erf (1.5e-7
+// absolute, Abramowitz & Stegun 7.1.26) are far inside the 4e-3 of a bf16 result, and
+// they take a fifth of the instructions of the correctly rounded library routines,
+// which is what bounds these kernels once their traffic is halved by the 16-bit I/O.
+__device__ __forceinline__ float rp_fast_erf(float x) {
+  const float ax = fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, ax, 1.0f));
+  float p = fmaf(1.061405429f, t, -1.453152027f);
+  p = fmaf(p, t, 1.421413741f);
+  p = fmaf(p, t, -0.284496736f);
+  p = fmaf(p, t, 0.254829592f);
+  const float e = __expf(-ax * ax);
+  const float r = fmaf(-p * t, e, 1.0f);
+  return copysignf(r, x);
+}
+__device__ __forceinline__ float rp_unary_lowp(int op, float a) {
+  switch (op) {
+    case NBK_OP_EXP: return __expf(a);
+    case NBK_OP_LOG: return __logf(a);
+    case NBK_OP_SQRT: return __builtin_amdgcn_sqrtf(a);
+    case NBK_OP_RSQRT: return __builtin_amdgcn_rsqf(a);
+    case NBK_OP_ERF: return rp_fast_erf(a);
+    case NBK_OP_GELU: return 0.5f * a * (1.0f + rp_fast_erf(a * 0.70710678118654752440f));
+    case NBK_OP_SIGMOID: return __builtin_amdgcn_rcpf(1.0f + __expf(-a));
+    default: return rp_unary(op, a);
+  }
+}
+__device__ __forceinline__ float rp_binary_lowp(int op, float a, float b) {
+  if (op == NBK_OP_DIV) return a * __builtin_amdgcn_rcpf(b);
+  return rp_binary(op, a, b);
+}
+
 // Offset of the current row inside one operand.  Strides and indices beyond
 // n_lead are zero, so all four terms can be added unconditionally (constant
 // indices keep both arrays in registers).
@@ -262,12 +295,18 @@ __device__ __forceinline__ void rp_decompose_row(uint32_t row, int n_lead, uint3
 // ---- helpers of the specialised (straight-line) row kernels ---------------------
 __device__ __forceinline__ float4 rp_splat(float s) { return make_float4(s, s, s, s); }
 
-template <int OP>
+template <int OP, bool LOWP = false>
 __device__ __forceinline__ float4 rp_un4(float4 a) {
+  if (LOWP)
+    return make_float4(rp_unary_lowp(OP, a.x), rp_unary_lowp(OP, a.y), rp_unary_lowp(OP, a.z),
+                       rp_unary_lowp(OP, a.w));
   return make_float4(rp_unary(OP, a.x), rp_unary(OP, a.y), rp_unary(OP, a.z), rp_unary(OP, a.w));
 }
-template <int OP>
+template <int OP, bool LOWP = false>
 __device__ __forceinline__ float4 rp_bin4(float4 a, float4 b) {
+  if (LOWP)
+    return make_float4(rp_binary_lowp(OP, a.x, b.x), rp_binary_lowp(OP, a.y, b.y),
+                       rp_binary_lowp(OP, a.z, b.z), rp_binary_lowp(OP, a.w, b.w));
   return make_float4(rp_binary(OP, a.x, b.x), rp_binary(OP, a.y, b.y), rp_binary(OP, a.z, b.z),
                      rp_binary(OP, a.w, b.w));
 }
