@@ -963,6 +963,13 @@ class Planner:
         a_bs, a_bs2 = levels(pa[0])
         b_bs, b_bs2 = levels(pb[0])
         c_bs, c_bs2 = levels(gc)
+        # x[b, M, K] @ W[K, N] with contiguous x and result is one product with b * M rows:
+        # the tiles of all batches then share W's panels in the order the GEMM walks them
+        if (batch > 1 and inner == 1 and len(pa[0]) == 1 and all(st == 0 for _, st in pb[0]) and
+                pa[2] == 1 and
+                pa[0][0][1] == M * pa[1] and c_strides == contiguous_strides(out.shape)):
+            M, batch = M * batch, 1
+            a_bs = c_bs = 0
         if c_strides == contiguous_strides(out.shape):
             dst = self._alloc_value(out)
         else:
@@ -973,7 +980,7 @@ class Planner:
             a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
-            ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs, alpha=1.0)))
+            ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
 
     # ................................................................ groups
     def _lower_group(self, g: Unit) -> None:

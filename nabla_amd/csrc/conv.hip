@@ -281,12 +281,20 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
     }
 }
 
-// out[i] = sum over z of partial[z][i], z ascending.
+// out[i] = sum over z of partial[z][i]; eight slices are in flight per lane and the order
+// of the additions is fixed, so the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void conv_sum_partials(const float* partial, float* out,
                                                          int64_t n, int splits) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
     float s = 0.f;
-    for (int z = 0; z < splits; ++z) s += partial[(int64_t)z * n + i];
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = partial[(int64_t)(z + q) * n + i];
+      s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    }
+    for (; z < splits; ++z) s += partial[(int64_t)z * n + i];
     out[i] = s;
   }
 }
