@@ -596,6 +596,7 @@ class Planner:
             b = self._new_buf(v.shape, v.dtype, "input", i)
             self.loc[v.id] = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
         self.skip_nodes: set[int] = set()  # reductions folded into an earlier one
+        self.n_split = 0                   # fusion groups cut in two at lowering time
         self.users: dict[int, list[ir.Node]] = {}
         for n in nodes:
             for i in n.inputs:
@@ -661,6 +662,8 @@ class Planner:
                  "fused_groups": sum(1 for u in units if u.fused)}
         for s in self.steps:
             stats[s.kind] = stats.get(s.kind, 0) + 1
+        if self.n_split:
+            stats["split_groups"] = self.n_split
         return Plan(self.bufs, self.steps, len(self.b.inputs), outs, arena, stats)
 
     def _assign_arena(self) -> int:
@@ -984,8 +987,49 @@ class Planner:
 
     # ................................................................ groups
     def _lower_group(self, g: Unit) -> None:
-        gen = _RowCodegen(self, g)
-        step = gen.generate()
+        """One row program for the group; a group that exceeds a limit of the row-program
+        format (operands, registers, instructions) is cut in two in program order, the values
+        that cross the cut go through memory, and each half is lowered on its own."""
+        snap = (len(self.bufs), dict(self.loc), dict(self._out_pending), dict(self._out_done))
+        try:
+            step = _RowCodegen(self, g).generate()
+        except FusionLimit:
+            if len(g.nodes) < 2:
+                raise
+            del self.bufs[snap[0]:]
+            self.loc, self._out_pending, self._out_done = snap[1], snap[2], snap[3]
+            self.n_split += 1
+            nodes = sorted(g.nodes, key=lambda n: n.pos)
+            cut = len(nodes) // 2
+            first = {n.pos for n in nodes[:cut]}
+            halves = []
+            for part in (nodes[:cut], nodes[cut:]):
+                keep = []
+                for n in part:
+                    if n.pos in self.alias_nodes and n.inputs[0].node.pos in first and n.pos not in first:
+                        # a broadcast whose source stays on the other side: an ordinary view again
+                        self.alias_nodes.discard(n.pos)
+                        self.unit_of.pop(n.pos, None)
+                        self.need_store.add(n.inputs[0].id)
+                        continue
+                    keep.append(n)
+                if not keep:
+                    continue
+                u = Unit(-1, keep[0], True)
+                for n in keep[1:]:
+                    u.add(n)
+                u.lead, u.C = g.lead, g.C
+                u.n_reduce = sum(1 for n in keep if n.kind == "reduce")
+                for n in keep:
+                    self.unit_of[n.pos] = u
+                halves.append(u)
+            for n in nodes[cut:]:
+                for i in n.inputs:
+                    if i.node.pos in first:
+                        self.need_store.add(i.id)
+            for u in halves:
+                self._lower_group(u)
+            return
         self._emit(step)
 
 

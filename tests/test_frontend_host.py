@@ -360,3 +360,23 @@ def test_context_isolation_of_flags():
 
     assert contextvars.copy_context().run(inner) is True
     assert config.EAGER_MAX_GRAPH is False
+
+
+def test_oversized_group_is_split_locally(emulator):
+    """22 results of one shared input exceed the 20 operands of a row program: the planner
+    cuts that group alone and everything else keeps its fusion."""
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((6, 40)).astype(np.float32)
+    X = T(x)
+    ys = [X * float(i + 1) for i in range(22)]
+    z = nb.reduce_sum(nb.relu(X) * 2.0, axis=1)       # an unrelated group in the same graph
+    engine.clear_plan_cache()
+    nb.realize_all(z, *ys)
+    plans = list(engine._PLAN_CACHE.values())
+    assert len(plans) == 1
+    stats = plans[0].plan.stats
+    assert stats.get("split_groups", 0) >= 1 and 2 <= stats["rowprog"] <= 4, stats
+    for i, y in enumerate(ys):
+        np.testing.assert_array_equal(y.numpy(), x * np.float32(i + 1))
+    np.testing.assert_allclose(z.numpy(), (np.maximum(x, 0) * 2).sum(1), rtol=1e-6)

@@ -176,3 +176,112 @@ def test_gather_argmax_views(hip):
     np.testing.assert_array_equal(z.numpy(), np.pad(x, [(1, 0), (0, 2), (1, 1)], constant_values=-1))
     c = nb.concatenate([T(x), T(x) + 1.0], axis=1)
     np.testing.assert_array_equal(c.numpy(), np.concatenate([x, x + 1], 1))
+
+
+def test_gemm_two_batch_levels(hip):
+    """Heads stay in place: A is [B,S,H,hd] read as a [B,H] batch of S x hd matrices and C is
+    written in [B,S,H,hd] order, as the attention products of the transformer block do."""
+    from nabla_amd.backend import lib
+    Bn, S, H, hd = 2, 96, 3, 64
+    rng = np.random.default_rng(11)
+    q = torch.tensor(rng.standard_normal((Bn, S, H, hd)), dtype=torch.bfloat16)
+    k = torch.tensor(rng.standard_normal((Bn, S, H, hd)), dtype=torch.bfloat16)
+    p = torch.tensor(rng.standard_normal((Bn, H, S, S)), dtype=torch.bfloat16)
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    qd, kd, pd = q.cuda(), k.cuda(), p.cuda()
+    # scores[b,h] = q[b,:,h,:] @ k[b,:,h,:]^T
+    sc = torch.empty((Bn, H, S, S), dtype=torch.bfloat16, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = qd.data_ptr(), kd.data_ptr(), sc.data_ptr()
+    d.M, d.N, d.K = S, S, hd
+    d.a_rs, d.a_cs, d.b_rs, d.b_cs = H * hd, 1, 1, H * hd
+    d.ldc = S
+    d.batch, d.batch_inner = Bn * H, H
+    d.a_bs, d.a_bs2 = S * H * hd, hd
+    d.b_bs, d.b_bs2 = S * H * hd, hd
+    d.c_bs, d.c_bs2 = H * S * S, S * S
+    d.dtype_ab = d.dtype_c = 1
+    d.alpha = 1.0
+    lib.check(L.nbk_gemm(C.byref(d), st))
+    # out[b,:,h,:] = p[b,h] @ k[b,:,h,:]  written with head stride hd, row stride H*hd
+    out = torch.zeros((Bn, S, H, hd), dtype=torch.bfloat16, device="cuda")
+    d2 = lib.GemmDesc()
+    d2.A, d2.B, d2.C = pd.data_ptr(), kd.data_ptr(), out.data_ptr()
+    d2.M, d2.N, d2.K = S, hd, S
+    d2.a_rs, d2.a_cs, d2.b_rs, d2.b_cs = S, 1, H * hd, 1
+    d2.ldc = H * hd
+    d2.batch, d2.batch_inner = Bn * H, H
+    d2.a_bs, d2.a_bs2 = H * S * S, S * S
+    d2.b_bs, d2.b_bs2 = S * H * hd, hd
+    d2.c_bs, d2.c_bs2 = S * H * hd, hd
+    d2.dtype_ab = d2.dtype_c = 1
+    d2.alpha = 1.0
+    lib.check(L.nbk_gemm(C.byref(d2), st))
+    torch.cuda.synchronize()
+    ref_sc = torch.einsum("bshd,bthd->bhst", q.double(), k.double())
+    ref_out = torch.einsum("bhst,bthd->bshd", p.double(), k.double())
+    for got, ref in ((sc, ref_sc), (out, ref_out)):
+        err = (got.double().cpu() - ref).abs() - 2.0 ** -8 * ref.abs()
+        assert err.max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("outer,red,inner", [(1, 8192, 1024), (3, 100, 40), (2, 77, 8), (1, 5, 1048576),
+                                             (4, 300, 1), (1, 4096, 24)])
+def test_reduce_mid_direct(hip, dtype, outer, red, inner):
+    from nabla_amd.backend import lib
+    rng = np.random.default_rng(12)
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    x = torch.tensor(rng.standard_normal((outer, red, inner)), dtype=tdt)
+    xd = x.cuda()
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    code = 0 if dtype == "f32" else 1
+    for kind, fn in ((0, lambda t: t.sum(1)), (1, lambda t: t.max(1).values), (2, lambda t: t.min(1).values)):
+        out = torch.empty((outer, inner), dtype=torch.float32, device="cuda")
+        lib.check(L.nbk_reduce_mid(C.c_void_p(xd.data_ptr()), C.c_void_p(out.data_ptr()), code, 0,
+                                   outer, red, inner, kind, st))
+        torch.cuda.synchronize()
+        ref = fn(x.double())
+        if kind == 0:
+            tol = 1e-6 * x.double().abs().sum(1) + 1e-30
+            assert ((out.cpu().double() - ref).abs() <= tol).all()
+        else:
+            assert torch.equal(out.cpu().double(), ref)
+
+
+def test_conv_wgrad_workspace_and_fallback(hip):
+    """The K-split filter gradient (with workspace) and the unsplit one (workspace NULL)
+    agree to summation-order noise, and both match a float64 reference."""
+    import torch.nn.functional as F
+    from nabla_amd.backend import lib
+    rng = np.random.default_rng(13)
+    N, H, W, Cin, Cout = 8, 16, 16, 16, 24
+    x = torch.tensor(rng.standard_normal((N, H, W, Cin)), dtype=torch.float32)
+    dy = torch.tensor(rng.standard_normal((N, H, W, Cout)), dtype=torch.float32)
+    d = lib.ConvDesc()
+    d.N, d.H, d.W, d.Cin, d.R, d.S, d.Cout, d.Ho, d.Wo = N, H, W, Cin, 3, 3, Cout, H, W
+    d.stride_h = d.stride_w = 1
+    d.pad_t = d.pad_b = d.pad_l = d.pad_r = 1
+    d.dtype = 0
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    need = L.nbk_conv2d_wgrad_workspace(C.byref(d))
+    assert need > 0
+    xd, dyd = x.cuda(), dy.cuda()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    dw1 = torch.empty((3, 3, Cin, Cout), dtype=torch.float32, device="cuda")
+    dw2 = torch.empty_like(dw1)
+    lib.check(L.nbk_conv2d_wgrad(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(dyd.data_ptr()),
+                                 C.c_void_p(dw1.data_ptr()), C.c_void_p(ws.data_ptr()), need, st))
+    lib.check(L.nbk_conv2d_wgrad(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(dyd.data_ptr()),
+                                 C.c_void_p(dw2.data_ptr()), None, 0, st))
+    torch.cuda.synchronize()
+    wt = torch.zeros((Cout, Cin, 3, 3), dtype=torch.float64, requires_grad=True)
+    y = F.conv2d(x.double().permute(0, 3, 1, 2), wt, padding=1)
+    (g,) = torch.autograd.grad(y, wt, dy.double().permute(0, 3, 1, 2))
+    ref = g.permute(2, 3, 1, 0)
+    scale = ref.abs().max().item()
+    assert (dw1.cpu().double() - ref).abs().max().item() <= 1e-5 * scale
+    assert (dw2.cpu().double() - ref).abs().max().item() <= 1e-5 * scale
