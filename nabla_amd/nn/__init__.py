@@ -1,3 +1,3 @@
-from . import finetune, functional
+from . import finetune, functional, optim
 from .modules import (GELU, Dropout, Embedding, LayerNorm, Linear, Module, MultiHeadAttention,
                       ReLU, Sequential, TransformerEncoderLayer)

@@ -353,3 +353,41 @@ def test_compiled_train_step_on_device(hip):
     assert cstep.stats.misses == 1 and cstep.stats.hits == 2
     for k in params:
         assert relerr(p[k].numpy(), ref[k]) < 5e-5
+
+
+# ---- optimizer step (next row after the hot path: nn/optim) ---------------------------------------
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-5), ("bf16", 2e-2)])
+def test_adamw_and_sgd_steps_on_device(hip, dtype, tol):
+    from nabla_amd.nn import optim
+    rng = np.random.default_rng(21)
+    shapes = {"w1": (256, 384), "b1": (1, 384), "w2": (384, 10)}
+    p0 = {k: rng.standard_normal(s).astype(np.float32) * 0.1 for k, s in shapes.items()}
+    dt = None if dtype == "f32" else nb.DType.bfloat16
+    if dtype == "bf16":
+        p0 = {k: oc.to_bf16_grid(v) for k, v in p0.items()}
+    up = lambda tree: {k: T(v, dtype=dt) for k, v in tree.items()}
+    tp = {k: torch.tensor(v, dtype=torch.float64, requires_grad=True) for k, v in p0.items()}
+    t_adam = torch.optim.AdamW(list(tp.values()), lr=1e-2, betas=(0.9, 0.99), weight_decay=0.02)
+    adam = optim.AdamW(up(p0), lr=1e-2, betas=(0.9, 0.99), weight_decay=0.02)
+    sp = {k: torch.tensor(v, dtype=torch.float64, requires_grad=True) for k, v in p0.items()}
+    t_sgd = torch.optim.SGD(list(sp.values()), lr=0.05, momentum=0.9, weight_decay=0.01)
+    sgd = optim.SGD(up(p0), lr=0.05, momentum=0.9, weight_decay=0.01)
+    for _ in range(3):
+        g = {k: rng.standard_normal(s).astype(np.float32) for k, s in shapes.items()}
+        if dtype == "bf16":
+            g = {k: oc.to_bf16_grid(v) for k, v in g.items()}
+        for k in shapes:
+            tp[k].grad = torch.tensor(g[k], dtype=torch.float64)
+            sp[k].grad = torch.tensor(g[k], dtype=torch.float64)
+        t_adam.step()
+        t_sgd.step()
+        a_new = adam.step(up(g))
+        s_new = sgd.step(up(g))
+        if dtype == "f32":
+            for k in shapes:
+                assert relerr(a_new[k].numpy(), tp[k].detach().numpy()) < tol, k
+                assert relerr(s_new[k].numpy(), sp[k].detach().numpy()) < tol, k
+    # bf16 parameters accumulate one rounding per step: compare after the last step only
+    for k in shapes:
+        assert relerr(a_new[k].numpy(), tp[k].detach().numpy()) < tol * 3, k
+        assert relerr(s_new[k].numpy(), sp[k].detach().numpy()) < tol * 3, k
