@@ -249,11 +249,26 @@ def main() -> int:
     dominant_kinds = {"rowprog": ["rowprog"], "gemm": ["gemm"],
                       "conv": ["conv2d", "conv2d_dgrad", "conv2d_wgrad"]}[w["dominant"]]
     timer = KernelTimer(L, dominant_kinds)
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        spec.bound.run(inputs, timer=timer)
-    sync()
-    wall = time.perf_counter() - t0
+    if len(plan.steps) == 1:
+        # one launch per step: the HIP events sit inside the timed region
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            spec.bound.run(inputs, timer=timer)
+        sync()
+        wall = time.perf_counter() - t0
+    else:
+        # several launches per step: the product path replays the repeated step as one HIP
+        # graph, inside which no event can be recorded; the step rate is timed on that path
+        # and the kernel durations for the roofline come from a second pass of plain launches
+        # with events on the launch stream
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            spec.bound.run(inputs)
+        sync()
+        wall = time.perf_counter() - t0
+        for _ in range(min(a.steps, 20)):
+            spec.bound.run(inputs, timer=timer)
+        sync()
     ms_per_step = wall / a.steps * 1e3
     dur = timer.durations_ms()
     per_step_total = {}
@@ -280,7 +295,7 @@ def main() -> int:
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": w["name"], "step": "compiled replay of forward + gradients",
-                   "plan": plan.stats},
+                   "plan": plan.stats, "graph_replays": ex.graph_replays},
         "roofline": roofline, "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -52,7 +52,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 4
+#define NBK_ABI_VERSION 5
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -313,6 +313,26 @@ int nbk_event_record(void* ev, void* stream);
 int nbk_event_elapsed_ms(void* start, void* stop, float* ms); /* syncs stop */
 int nbk_event_destroy(void* ev);
 int nbk_stream_sync(void* stream);
+
+/* ===================================================================== */
+/*  Plan replay as a HIP graph                                            */
+/* ===================================================================== */
+/* The reference replays a compiled model once per step
+ * (CompiledFunction._execute_cached_impl, nabla/transforms/compile.py:508-555);
+ * here a cached plan is a fixed sequence of launches, and when a step runs again
+ * on the same buffers the sequence is recorded once and replayed with a single
+ * call.  Capture needs a stream of its own (the default stream cannot record):
+ *   nbk_stream_create(&s); nbk_graph_begin_capture(s);
+ *   ... every nbk_* launch of the plan with stream = s (nothing executes) ...
+ *   nbk_graph_end_capture(s, &g);      then per step: nbk_graph_launch(g, any stream)
+ * The recording holds the pointers it was made with; the caller replays only while
+ * they are unchanged.  No memset nodes are ever recorded (nbk_fill is a kernel). */
+int nbk_stream_create(void** stream);            /* non-blocking, default priority */
+int nbk_stream_destroy(void* stream);
+int nbk_graph_begin_capture(void* stream);
+int nbk_graph_end_capture(void* stream, void** graph_exec);
+int nbk_graph_launch(void* graph_exec, void* stream);
+int nbk_graph_destroy(void* graph_exec);
 
 #ifdef __cplusplus
 }

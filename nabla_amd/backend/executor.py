@@ -12,6 +12,7 @@ same launch records.
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import Any, Sequence
 
 import torch
@@ -44,6 +45,9 @@ class BoundPlan:
         self.dynamic = [b.id for b in plan.bufs if b.role in ("input", "output")]
         self.calls: list[tuple] = []  # (fn, args tuple, patch list)
         self.has_gather = any(st.kind == "gather" for st in plan.steps)
+        self._graphs: dict = {}  # pointer tuple -> recorded launch sequence (at most four)
+        self._seen: set = set()  # pointer tuples that have run once already
+        self._graph_off = any(st.kind == "custom" for st in plan.steps)  # user kernels may not be capturable
         self._prepare()
 
     # -- address helpers -------------------------------------------------------
@@ -256,6 +260,55 @@ class BoundPlan:
         stream = C.c_void_p(ex.current_stream())
         base = self.base
         check = lib.check
+        # Replay as a HIP graph: a step that runs again on the very buffers of an earlier
+        # run (inputs unchanged, the allocator handed the same output blocks back) is
+        # recorded once and from then on costs one launch call instead of one per kernel.
+        if ex.use_graphs and timer is None and not keep and len(self.calls) > 1 and not self._graph_off:
+            key = tuple(base[b] for b in self.dynamic)
+            g = self._graphs.get(key)
+            if g is None and key in self._seen and len(self._graphs) < 4:
+                g = self._record(key)
+            if g is not None:
+                check(ex.lib.nbk_graph_launch(g, stream))
+                ex.graph_replays += 1
+                if self.has_gather:
+                    ex.status_dirty = True
+                return outs
+            if len(self._seen) < 64:
+                self._seen.add(key)
+        self._issue(stream, timer)
+        del keep
+        if self.has_gather:
+            ex.status_dirty = True
+        return outs
+
+    def _record(self, key):
+        """Capture the launch sequence (with the pointers now patched in) on the executor's
+        side stream and return the executable graph, or None.  Any failure switches graphs off
+        for this plan; nothing has executed either way."""
+        ex = self.ex
+        L = ex.lib
+        side = ex.capture_stream()
+        if side is None or L.nbk_graph_begin_capture(side) != 0:
+            self._graph_off = True
+            return None
+        ok = True
+        try:
+            self._issue(side, None)
+        except Exception:
+            ok = False
+        g = C.c_void_p()
+        rc = L.nbk_graph_end_capture(side, C.byref(g))
+        if not ok or rc != 0 or not g.value:
+            self._graph_off = True
+            return None
+        self._graphs[key] = g
+        return g
+
+    def _issue(self, stream, timer) -> None:
+        plan = self.plan
+        base = self.base
+        check = lib.check
         for si, (fn, args, patches, _keep) in enumerate(self.calls):
             after = timer(si, plan.steps[si].kind, stream) if timer is not None else None
             for obj, fieldname, buf, off in patches:
@@ -271,10 +324,6 @@ class BoundPlan:
             check(fn(*call_args, stream))
             if after is not None:
                 after()
-        del keep
-        if self.has_gather:
-            ex.status_dirty = True
-        return outs
 
 
 class _Ptrs:
@@ -301,6 +350,9 @@ class HipExecutor:
         lib.check(self.lib.nbk_init(device))
         self.torch_device = torch.device("cuda", device)
         self.status_flag = torch.zeros(1, dtype=torch.int32, device=self.torch_device)
+        self.use_graphs = os.environ.get("NBK_GRAPHS", "1") != "0"  # replay repeated steps as HIP graphs
+        self._capture_stream = None
+        self.graph_replays = 0
         self.status_dirty = False        # a launched plan may have flagged a bad gather index
         self.force_interpreter = False   # plans bound while set never use specialised row kernels
 
@@ -309,6 +361,15 @@ class HipExecutor:
 
     def bind(self, plan: Plan) -> BoundPlan:
         return BoundPlan(plan, self)
+
+    def capture_stream(self):
+        """Side stream that graph recordings are made on (the default stream cannot record)."""
+        if self._capture_stream is None:
+            s = C.c_void_p()
+            if self.lib.nbk_stream_create(C.byref(s)) != 0 or not s.value:
+                return None
+            self._capture_stream = s
+        return self._capture_stream
 
     def synchronize(self) -> None:
         torch.cuda.current_stream(self.torch_device).synchronize()

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 MAX_RANK = 8
 
@@ -102,6 +102,12 @@ _SIGNATURES = {
     "nbk_init": ([C.c_int], C.c_int),
     "nbk_last_error": ([], C.c_char_p),
     "nbk_abi_version": ([], C.c_int),
+    "nbk_stream_create": ([C.POINTER(C.c_void_p)], C.c_int),
+    "nbk_stream_destroy": ([C.c_void_p], C.c_int),
+    "nbk_graph_begin_capture": ([C.c_void_p], C.c_int),
+    "nbk_graph_end_capture": ([C.c_void_p, C.POINTER(C.c_void_p)], C.c_int),
+    "nbk_graph_launch": ([C.c_void_p, C.c_void_p], C.c_int),
+    "nbk_graph_destroy": ([C.c_void_p], C.c_int),
     "nbk_rowprog_launch": ([C.POINTER(RowProg), C.c_void_p], C.c_int),
     "nbk_rowprog_is_specialized": ([C.POINTER(RowProg)], C.c_int),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,

@@ -73,6 +73,49 @@ extern "C" int nbk_stream_sync(void* stream) {
   return NBK_OK;
 }
 
+// ---- plan replay as a HIP graph -------------------------------------------------
+extern "C" int nbk_stream_create(void** stream) {
+  NBK_REQUIRE(stream != nullptr, "nbk_stream_create: null out pointer");
+  hipStream_t s;
+  NBK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = (void*)s;
+  return NBK_OK;
+}
+extern "C" int nbk_stream_destroy(void* stream) {
+  NBK_HIP(hipStreamDestroy((hipStream_t)stream));
+  return NBK_OK;
+}
+extern "C" int nbk_graph_begin_capture(void* stream) {
+  NBK_REQUIRE(stream != nullptr, "nbk_graph_begin_capture: the default stream cannot record");
+  NBK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return NBK_OK;
+}
+extern "C" int nbk_graph_end_capture(void* stream, void** graph_exec) {
+  NBK_REQUIRE(graph_exec != nullptr, "nbk_graph_end_capture: null out pointer");
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  NBK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+  NBK_REQUIRE(graph != nullptr, "nbk_graph_end_capture: the capture was invalidated");
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    nbk_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    return NBK_ERR_LAUNCH;
+  }
+  *graph_exec = (void*)exec;
+  return NBK_OK;
+}
+extern "C" int nbk_graph_launch(void* graph_exec, void* stream) {
+  NBK_REQUIRE(graph_exec != nullptr, "nbk_graph_launch: null graph");
+  NBK_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return NBK_OK;
+}
+extern "C" int nbk_graph_destroy(void* graph_exec) {
+  if (graph_exec) NBK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  return NBK_OK;
+}
+
 // ---- custom kernels -----------------------------------------------------------
 // Libraries stay loaded for the life of the process; the handle table is the
 // only mutable global and is guarded by a mutex.

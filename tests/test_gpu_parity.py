@@ -391,3 +391,34 @@ def test_adamw_and_sgd_steps_on_device(hip, dtype, tol):
     for k in shapes:
         assert relerr(a_new[k].numpy(), tp[k].detach().numpy()) < tol * 3, k
         assert relerr(s_new[k].numpy(), sp[k].detach().numpy()) < tol * 3, k
+
+
+# ---- replay of a repeated step as a HIP graph -----------------------------------------------------
+def test_graph_replay_matches_eager_every_time(hip):
+    """A compiled step called again on the same buffers is recorded once and replayed; every
+    replay is checked against the oracle, with unrelated eager work and synchronisation between
+    the replays, and a call on new buffers falls back to plain launches."""
+    t = oc.c1_inputs(64, 96, 48, 10, seed=31)
+    t["b1"] = np.random.default_rng(2).uniform(-0.05, 0.05, t["b1"].shape).astype(np.float32)
+    wl, wg = oc.c1_reference(**t)
+    dev = oc.upload(nb, t)
+    step = nb.compile(lambda d: nb.workloads.c1_step(d))
+    before = hip.graph_replays
+    other = T(np.arange(12, dtype=np.float32))
+    for it in range(7):
+        loss, grads = step(dev)
+        got = [loss.numpy()] + [g.numpy() for g in grads]
+        assert abs(got[0] - wl) <= F32_TOL * abs(wl) + 1e-9, it
+        for g, w in zip(got[1:], wg):
+            assert relerr(g, w) < F32_TOL, it
+        del loss, grads
+        # unrelated work between replays
+        np.testing.assert_array_equal((other * 2.0 + float(it)).numpy(), np.arange(12) * 2.0 + it)
+    assert hip.graph_replays > before, "the repeated step was never replayed as a graph"
+    # new input buffers: pointers differ, the recording must not be used
+    t2 = oc.c1_inputs(64, 96, 48, 10, seed=32)
+    wl2, wg2 = oc.c1_reference(**t2)
+    loss, grads = step(oc.upload(nb, t2))
+    assert abs(loss.item() - wl2) <= F32_TOL * abs(wl2) + 1e-9
+    for g, w in zip(grads, wg2):
+        assert relerr(g.numpy(), w) < F32_TOL
