@@ -745,7 +745,9 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     const int64_t big_tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256) * d->batch;
     const int64_t cus = nbk_num_cus();
     const int64_t rounds = (big_tiles + cus - 1) / cus;
-    if (big_tiles * 10 >= rounds * cus * 6 && d->M >= 256 && d->N >= 256)
+    // (a K loop of one or two iterations is all prologue and epilogue: there two co-resident
+    // 128 x 128 workgroups per CU overlap better than one 256 x 256)
+    if (big_tiles * 10 >= rounds * cus * 6 && d->M >= 256 && d->N >= 256 && d->K > 128)
       return launch_bf16<256, 256, true>(a, akc, bkc, d->batch, st);
     // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
     // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
