@@ -241,10 +241,27 @@ class BoundPlan:
             raise ValueError(f"plan expects {plan.n_inputs} inputs, got {len(inputs)}")
         keep = []
         outs: list[torch.Tensor] = [None] * len(plan.outputs)  # type: ignore
+        # every output of the step is a view into one allocation.  It is at least 2 MiB so that
+        # it comes from the allocator's pool for large blocks: a loop that drops its results
+        # before the next step then gets the same block back whatever small allocations happen
+        # in between, which is what lets the step be replayed as a recorded graph
         out_by_buf = {}
+        offs, total = {}, 0
+        for bid, shape, dtype in plan.outputs:
+            if bid not in offs:
+                offs[bid] = total
+                n = 1
+                for d in shape:
+                    n *= d
+                total += (max(n, 1) * dtype.size_in_bytes + 255) & ~255
+        slab = torch.empty(max(total, 1 << 21), dtype=torch.uint8, device=ex.torch_device)
         for oi, (bid, shape, dtype) in enumerate(plan.outputs):
             if bid not in out_by_buf:
-                out_by_buf[bid] = torch.empty(shape, dtype=dtype.to_torch(), device=ex.torch_device)
+                n = 1
+                for d in shape:
+                    n *= d
+                piece = slab[offs[bid]:offs[bid] + n * dtype.size_in_bytes]
+                out_by_buf[bid] = piece.view(dtype.to_torch()).reshape(shape)
             outs[oi] = out_by_buf[bid]
         for b in plan.bufs:
             if b.role == "input":

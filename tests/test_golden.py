@@ -125,7 +125,10 @@ def run_package(tol):
     py = nb.max_pool2d(p, kernel_size=(2, 2))
     gp = nb.grad(lambda a: nb.reduce_sum(nb.max_pool2d(a, kernel_size=(2, 2)) ** 2))(p)
     np.testing.assert_array_equal(py.numpy(), z["pool_y"])
-    np.testing.assert_array_equal(gp.numpy(), z["pool_gx"])
+    # the routing is exact (which element of each window receives the gradient); the value
+    # 2 * y goes through the device's pow, which is not correctly rounded
+    np.testing.assert_array_equal(gp.numpy() != 0, z["pool_gx"] != 0)
+    assert rel(gp.numpy(), z["pool_gx"]) < tol
     np.testing.assert_array_equal(nb.argmax(T(z["argmax_x"]), axis=-1).numpy(), z["argmax_y"])
     np.testing.assert_array_equal(nb.gather(T(z["gather_table"]), T(z["gather_idx"]), axis=0).numpy(),
                                   z["gather_y"])
