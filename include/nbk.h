@@ -16,7 +16,9 @@
  *   - kernels never allocate: the caller owns inputs, outputs and workspace
  *   - return value: 0 on success, negative nbk_status otherwise;
  *     nbk_last_error() returns a thread-local message for the last failure
- *   - the library keeps no mutable global state besides that message
+ *   - mutable global state is limited to that message (thread-local) and to
+ *     mutex-guarded caches that are filled on first use: the table of
+ *     specialised row kernels, per-kernel occupancy, loaded user libraries
  */
 #ifndef NBK_H_
 #define NBK_H_
