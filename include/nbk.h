@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 5
+#define NBK_ABI_VERSION 6
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -268,6 +268,43 @@ typedef struct nbk_pool_desc {
 int nbk_maxpool2d_fwd(const nbk_pool_desc* d, const void* x, void* y, void* stream);
 int nbk_maxpool2d_bwd(const nbk_pool_desc* d, const void* x, const void* y,
                       const void* dy, void* dx, void* stream);
+
+/* ===================================================================== */
+/*  Fused attention                                                       */
+/* ===================================================================== */
+/* O = softmax(mask(Q K^T * scale)) V in one kernel, and its gradients in three;
+ * replaces the matmul / mul / where / softmax / matmul graph that
+ * scaled_dot_product_attention builds (nabla/nn/functional/layers.py:106-153) and
+ * the VJP graphs of those ops, for the case without an explicit mask or dropout.
+ * The S x S scores and probabilities are never stored: the forward keeps one
+ * log-sum-exp per score row (lse, fp32 [B, H, S]) and the backward recomputes.
+ * Tensors are [B, S, H, hd] addressed through element strides (sb, ss, sh) with
+ * hd contiguous, so heads are read and written in place of a transpose.
+ * dtype NBK_BF16, hd 64 or 128, S a multiple of 128; pointers 16-byte aligned,
+ * strides multiples of 8.  causal != 0 masks key > query. */
+typedef struct nbk_attn_desc {
+  int64_t B, H, S, hd;
+  float scale;
+  int32_t causal;
+  int32_t dtype;
+  int32_t reserved;
+} nbk_attn_desc;
+typedef struct nbk_attn_tensor {
+  void* ptr;
+  int64_t sb, ss, sh;
+} nbk_attn_tensor;
+int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
+                      const nbk_attn_tensor* k, const nbk_attn_tensor* v,
+                      const nbk_attn_tensor* o, void* lse, void* stream);
+/* Backward needs nbk_attention_bwd_workspace(d) bytes of caller scratch (one
+ * fp32 per score row: rowsum(dO * O)). */
+int64_t nbk_attention_bwd_workspace(const nbk_attn_desc* d);
+int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
+                      const nbk_attn_tensor* k, const nbk_attn_tensor* v,
+                      const nbk_attn_tensor* o, const void* lse,
+                      const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                      const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
+                      void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ===================================================================== */
 /*  Index ops (bit-exact)                                                 */

@@ -195,6 +195,38 @@ class BoundPlan:
                     ptr_field(holder, nm, r.buf, r.offset * r.dtype.size_in_bytes)
                 fn = L.nbk_maxpool2d_fwd if k == "maxpool2d" else L.nbk_maxpool2d_bwd
                 self.calls.append((fn, [C.byref(d), holder, tuple(names)], patches, d))
+            elif k in ("attention", "attention_bwd"):
+                d = lib.AttnDesc()
+                d.B, d.H, d.S, d.hd = a["B"], a["H"], a["S"], a["hd"]
+                d.scale = a["scale"]
+                d.causal = 1 if a["causal"] else 0
+                d.dtype = a["q"].dtype.abi
+                keep_alive = [d]
+
+                def heads(ref):
+                    """[B, H, S, hd] view -> (batch, sequence, head) strides."""
+                    t = lib.AttnTensor()
+                    sb, sh, ss, _ = ref.strides
+                    t.sb, t.ss, t.sh = sb, ss, (sh if ref.shape[1] > 1 else a["hd"])
+                    if ref.shape[0] == 1:
+                        t.sb = 0
+                    ptr_field(t, "ptr", ref.buf, ref.offset * ref.dtype.size_in_bytes)
+                    keep_alive.append(t)
+                    return C.byref(t)
+
+                holder = _Ptrs(2)
+                ptr_field(holder, "p0", a["lse"].buf, a["lse"].offset * 4)
+                if k == "attention":
+                    args = [_LATE, C.byref(d), heads(a["q"]), heads(a["k"]), heads(a["v"]), heads(a["o"]),
+                            _Late(holder, "p0")]
+                    self.calls.append((L.nbk_attention_fwd, args, patches, keep_alive))
+                else:
+                    ws = a["workspace"]
+                    ptr_field(holder, "p1", ws.buf, ws.offset * 4)
+                    args = [_LATE, C.byref(d), heads(a["q"]), heads(a["k"]), heads(a["v"]), heads(a["o"]),
+                            _Late(holder, "p0"), heads(a["dout"]), heads(a["dq"]), heads(a["dk"]),
+                            heads(a["dv"]), _Late(holder, "p1"), C.c_int64(a["workspace_bytes"])]
+                    self.calls.append((L.nbk_attention_bwd, args, patches, keep_alive))
             elif k == "gather":
                 t, ix, dst = a["table"], a["idx"], a["dst"]
                 holder = _Ptrs(3)
@@ -330,7 +362,9 @@ class BoundPlan:
             after = timer(si, plan.steps[si].kind, stream) if timer is not None else None
             for obj, fieldname, buf, off in patches:
                 setattr(obj, fieldname, base[buf] + off)
-            if len(args) >= 2 and isinstance(args[0], _Ptrs):
+            if args[0] is _LATE:
+                call_args = [C.c_void_p(getattr(x.h, x.n)) if type(x) is _Late else x for x in args[1:]]
+            elif len(args) >= 2 and isinstance(args[0], _Ptrs):
                 h = args[0]
                 call_args = [C.c_void_p(getattr(h, n)) for n in args[1]] + list(args[2:])
             elif len(args) >= 3 and isinstance(args[1], _Ptrs):
@@ -350,6 +384,18 @@ class _Ptrs:
 
     def __init__(self, n: int):
         self.p0 = self.p1 = self.p2 = self.p3 = None
+
+
+class _Late:
+    """An address argument read from its holder when the call is made."""
+
+    __slots__ = ("h", "n")
+
+    def __init__(self, holder: _Ptrs, name: str):
+        self.h, self.n = holder, name
+
+
+_LATE = "late"  # first element of an argument list that contains _Late entries
 
 
 class HipExecutor:

@@ -378,3 +378,20 @@ def slice_update(x: Value, update: Value, starts) -> Value:
 def custom(name: str, library: str, inputs: Sequence[Value], out_types: Sequence[tuple]) -> list[Value]:
     return current().add("custom", list(inputs), [(tuple(s), d) for s, d in out_types], name=name,
                          library=str(library))
+
+
+# ---- fused attention ----------------------------------------------------------------------
+def attention(q: Value, k: Value, v: Value, scale: float, causal: bool) -> list[Value]:
+    """[B, H, S, hd] heads -> (output [B, H, S, hd], log-sum-exp of the score rows [B, H, S])."""
+    if not (q.shape == k.shape == v.shape) or q.rank != 4:
+        raise ValueError(f"attention: q, k, v must share one [B, H, S, hd] shape, got "
+                         f"{q.shape}, {k.shape}, {v.shape}")
+    return current().add("attention", [q, k, v], [(q.shape, q.dtype), (q.shape[:-1], DType.float32)],
+                         scale=float(scale), causal=bool(causal))
+
+
+def attention_bwd(q: Value, k: Value, v: Value, o: Value, lse: Value, dout: Value, scale: float,
+                  causal: bool) -> list[Value]:
+    """Gradients (dq, dk, dv) of ``attention`` from its inputs, both outputs and d(output)."""
+    return current().add("attention_bwd", [q, k, v, o, lse, dout], [(q.shape, q.dtype)] * 3,
+                         scale=float(scale), causal=bool(causal))

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 MAX_RANK = 8
 
@@ -91,6 +91,17 @@ class PoolDesc(C.Structure):
     ]
 
 
+class AttnDesc(C.Structure):
+    _fields_ = [
+        ("B", C.c_int64), ("H", C.c_int64), ("S", C.c_int64), ("hd", C.c_int64),
+        ("scale", C.c_float), ("causal", C.c_int32), ("dtype", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class AttnTensor(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("sb", C.c_int64), ("ss", C.c_int64), ("sh", C.c_int64)]
+
+
 class TensorDesc(C.Structure):
     _fields_ = [
         ("ptr", C.c_void_p), ("dtype", C.c_int32), ("rank", C.c_int32),
@@ -127,6 +138,11 @@ _SIGNATURES = {
     "nbk_maxpool2d_fwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_maxpool2d_bwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                            C.c_void_p], C.c_int),
+    "nbk_attention_fwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_void_p],
+                          C.c_int),
+    "nbk_attention_bwd_workspace": ([C.POINTER(AttnDesc)], C.c_int64),
+    "nbk_attention_bwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p] +
+                          [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_int64, C.c_void_p], C.c_int),
     "nbk_gather": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64,
                     C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_argmax_rows": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32,

@@ -737,6 +737,8 @@ class Planner:
                     attrs["workspace_bytes"] = nbytes
                     writes.append(wbuf.id)
             self._emit(Step(k, [i.buf for i in ins], writes, attrs))
+        elif k in ("attention", "attention_bwd"):
+            self._lower_attention(n)
         elif k in ("maxpool2d", "maxpool2d_bwd"):
             ins = [self._contig(i) for i in n.inputs]
             dst = self._alloc_value(out)
@@ -984,6 +986,66 @@ class Planner:
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
             ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
+
+    # ................................................................ attention
+    def _heads_operand(self, v: ir.Value) -> ViewRef:
+        """A [B, H, S, hd] value where the attention kernels can read it: unit stride along hd
+        and every other stride a non-negative multiple of 8 elements (16-byte rows); anything
+        else is copied first."""
+        ref = self._resolve(v)
+        if isinstance(ref, Const):
+            return self._materialize(ref)
+        ok = ref.strides[-1] == 1 and ref.offset % 8 == 0
+        for d, s in zip(ref.shape[:-1], ref.strides[:-1]):
+            if d > 1 and (s <= 0 or s % 8):
+                ok = False
+        return ref if ok else self._materialize(ref)
+
+    def _heads_result(self, out: ir.Value) -> ViewRef:
+        """Storage for a [B, H, S, hd] result.  When it is read through one permute that keeps
+        hd last (the transpose back to [B, S, H, hd]) it is written in that order, and the
+        permute becomes a contiguous view."""
+        strides = contiguous_strides(out.shape)
+        users = self.users.get(out.id, ())
+        perms = [u for u in users if u.kind == "permute"]
+        # the attention kernels themselves read any layout, so the backward kernel reading the
+        # forward result does not stand in the way
+        if (out.id not in self._out_pending and len(perms) == 1 and
+                perms[0].attrs["perm"][-1] == out.rank - 1 and
+                all(u.kind in ("permute", "attention", "attention_bwd") for u in users)):
+            perm = perms[0].attrs["perm"]
+            pst = contiguous_strides(tuple(out.shape[p] for p in perm))
+            cand = [0] * out.rank
+            for i, p in enumerate(perm):
+                cand[p] = pst[i]
+            strides = tuple(cand)
+        if strides == contiguous_strides(out.shape) or any(s % 8 for s in strides[:-1]):
+            return self._alloc_value(out)
+        buf = self._new_buf(out.shape, out.dtype, "temp", -1)
+        dst = ViewRef(buf.id, 0, out.shape, strides, out.dtype)
+        self.loc[out.id] = dst
+        return dst
+
+    def _lower_attention(self, n: ir.Node) -> None:
+        B, H, S, hd = n.inputs[0].shape
+        common = dict(B=B, H=H, S=S, hd=hd, scale=n.attrs["scale"], causal=n.attrs["causal"])
+        if n.kind == "attention":
+            q, k, v = (self._heads_operand(i) for i in n.inputs)
+            o = self._heads_result(n.outputs[0])
+            lse = self._alloc_value(n.outputs[1])
+            self._emit(Step("attention", [q.buf, k.buf, v.buf], [o.buf, lse.buf],
+                            dict(common, q=q, k=k, v=v, o=o, lse=lse)))
+            return
+        q, k, v, o = (self._heads_operand(i) for i in n.inputs[:4])
+        lse = self._contig(n.inputs[4])
+        dout = self._heads_operand(n.inputs[5])
+        dq, dk, dv = (self._heads_result(t) for t in n.outputs)
+        wbuf = self._new_buf((B * H * S,), DType.float32, "temp", -1)
+        ws = ViewRef(wbuf.id, 0, (B * H * S,), (1,), DType.float32)
+        self._emit(Step("attention_bwd", [q.buf, k.buf, v.buf, o.buf, lse.buf, dout.buf],
+                        [dq.buf, dk.buf, dv.buf, wbuf.id],
+                        dict(common, q=q, k=k, v=v, o=o, lse=lse, dout=dout, dq=dq, dk=dk, dv=dv,
+                             workspace=ws, workspace_bytes=B * H * S * 4)))
 
     # ................................................................ groups
     def _lower_group(self, g: Unit) -> None:

@@ -21,11 +21,16 @@ _VERIFY_EAGER_SHAPES: ContextVar[bool] = ContextVar(
     "VERIFY_EAGER_SHAPES", default=_env_flag("VERIFY_EAGER_SHAPES")
 )
 _TRACING: ContextVar[bool] = ContextVar("TRACING", default=False)
+# scaled_dot_product_attention as one fused op where its kernels apply (bf16, head size 64 or
+# 128, no explicit mask or dropout); off: always the reference's composition of primitive ops
+_FUSED_ATTENTION: ContextVar[bool] = ContextVar("FUSED_ATTENTION",
+                                                default=_env_flag("NBK_FUSED_ATTENTION", True))
 
 _FLAGS = {
     "EAGER_MAX_GRAPH": _EAGER_MAX_GRAPH,
     "VERIFY_EAGER_SHAPES": _VERIFY_EAGER_SHAPES,
     "TRACING": _TRACING,
+    "FUSED_ATTENTION": _FUSED_ATTENTION,
 }
 
 

@@ -1,0 +1,660 @@
+// Fused scaled-dot-product attention for gfx950, bf16 in / fp32 accumulate.
+//
+//   forward : O = softmax(mask(Q K^T * scale)) V,  LSE = log-sum-exp of every score row
+//   backward: dQ, dK, dV from (Q, K, V, O, LSE, dO) with the probabilities recomputed
+//
+// The S x S score matrix never reaches memory.  Tensors are [B, S, H, hd] in any
+// strides with a unit stride along hd (heads are read in place), hd = 64 or 128,
+// S a multiple of 128.
+//
+// Register layouts of v_mfma_f32_32x32x16_bf16 (lane l, li = l % 32, h = l / 32):
+//   A: lane holds A[row li][k = 8h .. 8h+7]      B: lane holds B[k = 8h .. 8h+7][col li]
+//   D: register r holds D[row (r/4)*8 + 4h + r%4][col li]
+// All three kernels compute the scores TRANSPOSED with respect to the tensor the wave
+// owns in registers: the owned rows (queries in the forward and dQ kernels, keys in
+// the dK/dV kernel) sit on the MFMA's column side, one per lane, so that
+//   * a softmax row lives in one lane pair (li, li + 32): row max and sum are
+//     register reductions plus one exchange between the two halves;
+//   * the probabilities (or dS) leave the first MFMA in exactly the layout the second
+//     MFMA wants for its B operand: registers 8t .. 8t+7 of a 32-row tile are k-slots
+//     8h .. 8h+7 of the t-th 16-wide k-step, if slot 8h + i stands for row
+//     16t + 4h + i (i < 4) and 16t + 8 + 4h + (i - 4) (i >= 4).  The A operand of that
+//     second MFMA is read from a transposed LDS tile with the same permutation: two
+//     8-byte reads at columns 16t + 4h and 16t + 8 + 4h.
+// LDS tiles:
+//   row-major  [64 rows][hd]      16-byte chunks XOR-swizzled by row % 8 (conflict-free
+//                                  16-byte fragment reads of 32 consecutive rows)
+//   transposed [hd rows][64 cols]  row pitch 68 elements: the 8-byte reads of 32
+//                                  consecutive rows fall on distinct banks per half
+#include "nbk_common.h"
+
+#include <utility>
+
+typedef __bf16 at_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float at_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t at_u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename F, int... I>
+__device__ __forceinline__ void at_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void at_static_for(F&& f) {
+  at_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+struct AttnTensor {
+  const uint16_t* p;
+  int64_t sb, ss, sh;  // element strides of batch, sequence, head; hd is contiguous
+};
+
+struct AttnArgs {
+  AttnTensor q, k, v, o, dout, dq, dk, dv;
+  float* lse;    // [B, H, S]
+  float* delta;  // [B, H, S]: rowsum(dO * O), backward only
+  int32_t B, H, S;
+  int32_t causal;
+  float scale;
+};
+
+constexpr int AT_TP = 68;  // pitch (elements) of a transposed tile row
+
+__device__ __forceinline__ float at_neg_big() { return -1.0e30f; }
+
+__device__ __forceinline__ uint32_t at_pack2(float a, float b) {
+  return (uint32_t)nbk_f32_to_bf16(a) | ((uint32_t)nbk_f32_to_bf16(b) << 16);
+}
+
+// 64 x HD tile -> LDS, row-major swizzled.  256 lanes, 16 bytes each per pass.
+template <int HD>
+struct AtRowTile {
+  static constexpr int NCH = HD / 8;             // 16-byte chunks per row
+  static constexpr int NREG = 64 * NCH / 256;    // passes (2 for hd 64, 4 for hd 128)
+  at_u32x4 reg[NREG];
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0) {
+#pragma unroll
+    for (int s = 0; s < NREG; ++s) {
+      const int t = threadIdx.x + s * 256;
+      const int row = t / NCH, c = t % NCH;
+      reg[s] = *(const at_u32x4*)(base + (int64_t)(row0 + row) * row_stride + c * 8);
+    }
+  }
+  __device__ __forceinline__ void store(at_u32x4* lds) const {
+#pragma unroll
+    for (int s = 0; s < NREG; ++s) {
+      const int t = threadIdx.x + s * 256;
+      const int row = t / NCH, c = t % NCH;
+      lds[row * NCH + (c ^ (row & 7))] = reg[s];
+    }
+  }
+  // fragment: 8 consecutive k (chunk) of `row`
+  static __device__ __forceinline__ at_bf16x8 frag(const at_u32x4* lds, int row, int chunk) {
+    const at_u32x4 u = lds[row * NCH + (chunk ^ (row & 7))];
+    return __builtin_bit_cast(at_bf16x8, u);
+  }
+};
+
+// 64 x HD tile -> LDS transposed ([HD][64], pitch AT_TP).  A lane transposes one 8 x 8
+// block: 8 rows of 16 bytes in, 8 columns of 16 bytes (two 8-byte stores) out.
+template <int HD>
+struct AtTransTile {
+  static constexpr int NBLK = 8 * (HD / 8);  // 64 (hd 64) or 128 (hd 128) blocks
+  at_u32x4 reg[8];
+  __device__ __forceinline__ bool active() const { return threadIdx.x < NBLK; }
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0) {
+    if (!active()) return;
+    const int rb = threadIdx.x % 8, db = threadIdx.x / 8;  // row block, d block
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      reg[r] = *(const at_u32x4*)(base + (int64_t)(row0 + rb * 8 + r) * row_stride + db * 8);
+  }
+  __device__ __forceinline__ void store(uint16_t* lds) const {
+    if (!active()) return;
+    const int rb = threadIdx.x % 8, db = threadIdx.x / 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // column j of the block: element j of each of the 8 rows
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      at_u32x2 lo, hi;
+      lo.x = __builtin_amdgcn_perm(reg[1][j >> 1], reg[0][j >> 1], sel);
+      lo.y = __builtin_amdgcn_perm(reg[3][j >> 1], reg[2][j >> 1], sel);
+      hi.x = __builtin_amdgcn_perm(reg[5][j >> 1], reg[4][j >> 1], sel);
+      hi.y = __builtin_amdgcn_perm(reg[7][j >> 1], reg[6][j >> 1], sel);
+      uint16_t* dst = lds + (db * 8 + j) * AT_TP + rb * 8;
+      *(at_u32x2*)dst = lo;
+      *(at_u32x2*)(dst + 4) = hi;
+    }
+  }
+  // A fragment of the second MFMA: row d, k-slots of the t-th 16-wide step of 32-row tile kt2
+  static __device__ __forceinline__ at_bf16x8 frag(const uint16_t* lds, int d, int kt2, int t, int h) {
+    const uint16_t* p = lds + d * AT_TP + kt2 * 32 + t * 16 + 4 * h;
+    const at_u32x2 a = *(const at_u32x2*)p;
+    const at_u32x2 b = *(const at_u32x2*)(p + 8);
+    const at_u32x4 u = {a.x, a.y, b.x, b.y};
+    return __builtin_bit_cast(at_bf16x8, u);
+  }
+};
+
+// B fragment of the second MFMA from the registers of a transposed score tile
+__device__ __forceinline__ at_bf16x8 at_regs_frag(const at_f32x16& s, int t) {
+  at_u32x4 u;
+  if (t == 0) {
+    u.x = at_pack2(s[0], s[1]); u.y = at_pack2(s[2], s[3]);
+    u.z = at_pack2(s[4], s[5]); u.w = at_pack2(s[6], s[7]);
+  } else {
+    u.x = at_pack2(s[8], s[9]); u.y = at_pack2(s[10], s[11]);
+    u.z = at_pack2(s[12], s[13]); u.w = at_pack2(s[14], s[15]);
+  }
+  return __builtin_bit_cast(at_bf16x8, u);
+}
+
+__device__ __forceinline__ float at_xhalf(float v) { return __shfl_xor(v, 32, 64); }
+
+// ------------------------------------------------------------------------------ forward
+// Grid: (S / 128, B * H).  Wave w owns queries q0 + 32w .. + 31 (one per lane pair).
+template <int HD>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
+  using RowT = AtRowTile<HD>;
+  using TrT = AtTransTile<HD>;
+  constexpr int KSTEPS = HD / 16, DT = HD / 32;
+  constexpr int ROW_BYTES = 64 * HD * 2, TR_BYTES = HD * AT_TP * 2;
+  extern __shared__ __align__(16) unsigned char at_lds[];
+  auto k_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * (ROW_BYTES + TR_BYTES)); };
+  auto v_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * (ROW_BYTES + TR_BYTES) + ROW_BYTES); };
+
+  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
+  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;  // long causal rows first
+  const int q0 = qt * 128;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
+  const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
+  const uint16_t* K = g.k.p + (int64_t)b * g.k.sb + (int64_t)hh * g.k.sh;
+  const uint16_t* V = g.v.p + (int64_t)b * g.v.sb + (int64_t)hh * g.v.sh;
+  const int my_q = q0 + wave * 32 + li;
+
+  // the wave's queries as B fragments of the score MFMA
+  at_bf16x8 qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const at_u32x4 u = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
+    qf[s] = __builtin_bit_cast(at_bf16x8, u);
+  }
+
+  at_f32x16 o_acc[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o_acc[d] = (at_f32x16)(0.f);
+  float m_i = at_neg_big(), l_i = 0.f;
+
+  const int n_tiles = g.causal ? (q0 + 128) / 64 : g.S / 64;
+  RowT kl;
+  TrT vl;
+  kl.load(K, g.k.ss, 0);
+  vl.load(V, g.v.ss, 0);
+  kl.store(k_tile(0));
+  vl.store(v_tile(0));
+  __syncthreads();
+  for (int kt = 0; kt < n_tiles; ++kt) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < n_tiles;
+    if (more) {
+      kl.load(K, g.k.ss, (kt + 1) * 64);
+      vl.load(V, g.v.ss, (kt + 1) * 64);
+    }
+    const at_u32x4* Ks = k_tile(cur);
+    const uint16_t* Vs = v_tile(cur);
+    const int k0 = kt * 64;
+    // transposed scores: rows = keys (two 32-row tiles), columns = the wave's queries
+    at_f32x16 st[2];
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2) {
+      at_f32x16 acc = (at_f32x16)(0.f);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
+                                                      acc, 0, 0, 0);
+      st[kt2] = acc;
+    }
+    // scale, mask, running max
+    float mx = at_neg_big();
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
+        float v = st[kt2][r] * g.scale;
+        if (g.causal && key > my_q) v = at_neg_big();
+        st[kt2][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, at_xhalf(mx));
+    const float m_new = fmaxf(m_i, mx);
+    const float alpha = __expf(m_i - m_new);
+    float sum = 0.f;
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __expf(st[kt2][r] - m_new);
+        st[kt2][r] = p;
+        sum += p;
+      }
+    sum += at_xhalf(sum);
+    l_i = l_i * alpha + sum;
+    m_i = m_new;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o_acc[d] *= alpha;
+    // O^T[d, q] += V^T[d, key] P^T[key, q]
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const at_bf16x8 pf = at_regs_frag(st[kt2], t);
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+          o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
+                                                             o_acc[d], 0, 0, 0);
+      }
+    if (more) {
+      kl.store(k_tile(cur ^ 1));
+      vl.store(v_tile(cur ^ 1));
+    }
+    __syncthreads();
+  }
+  // normalise and write: register r of tile d is O[my_q][32 d + (r/4)*8 + 4h + r%4]
+  const float inv = 1.0f / l_i;
+  uint16_t* O = (uint16_t*)g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)my_q * g.o.ss;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      at_u32x2 w;
+      w.x = at_pack2(o_acc[d][gq * 4 + 0] * inv, o_acc[d][gq * 4 + 1] * inv);
+      w.y = at_pack2(o_acc[d][gq * 4 + 2] * inv, o_acc[d][gq * 4 + 3] * inv);
+      *(at_u32x2*)(O + d * 32 + gq * 8 + 4 * h) = w;
+    }
+  if (h == 0) g.lse[((int64_t)b * g.H + hh) * g.S + my_q] = m_i + __logf(l_i);
+}
+
+// ------------------------------------------------------------------------------ backward
+// delta[b, h, q] = sum_d dO[q, d] * O[q, d]: one lane per (row, 8-wide slice), reduced
+// over the HD / 8 lanes of a row.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs g) {
+  constexpr int LPR = HD / 8;  // lanes per row
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = idx / LPR;
+  const int c = (int)(idx % LPR);
+  const int64_t rows = (int64_t)g.B * g.H * g.S;
+  float s = 0.f;
+  if (row < rows) {
+    const int q = (int)(row % g.S);
+    const int64_t bh = row / g.S;
+    const int hh = (int)(bh % g.H), b = (int)(bh / g.H);
+    const uint16_t* o = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)q * g.o.ss + c * 8;
+    const uint16_t* d = g.dout.p + (int64_t)b * g.dout.sb + (int64_t)hh * g.dout.sh +
+                        (int64_t)q * g.dout.ss + c * 8;
+    const at_u32x4 uo = *(const at_u32x4*)o, ud = *(const at_u32x4*)d;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s += __uint_as_float(uo[e] << 16) * __uint_as_float(ud[e] << 16);
+      s += __uint_as_float(uo[e] & 0xffff0000u) * __uint_as_float(ud[e] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (row < rows && c == 0) g.delta[row] = s;
+}
+
+// dK, dV.  Grid: (S / 128, B * H).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
+// and walks the query tiles that can see them.
+//   S[q, key]  = Q K^T          (A: Q tile rows, B: the wave's K fragments)
+//   P          = exp(S * scale - LSE[q])
+//   dV^T[d,key] += dO^T[d, q] P[q, key]        (A: transposed dO tile, B: P registers)
+//   dP[q, key] = dO V^T         (A: dO tile rows, B: the wave's V fragments)
+//   dS         = P * (dP - delta[q])
+//   dK^T[d,key] += Q^T[d, q] dS[q, key] * scale (A: transposed Q tile, B: dS registers)
+template <int HD>
+__global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
+  using RowT = AtRowTile<HD>;
+  using TrT = AtTransTile<HD>;
+  constexpr int KSTEPS = HD / 16, DT = HD / 32;
+  constexpr int ROW_BYTES = 64 * HD * 2, TR_BYTES = HD * AT_TP * 2;
+  constexpr int STAGE = 2 * ROW_BYTES + 2 * TR_BYTES + 2 * 64 * 4;
+  extern __shared__ __align__(16) unsigned char at_lds[];
+  auto q_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE); };
+  auto do_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE + ROW_BYTES); };
+  auto qt_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * STAGE + 2 * ROW_BYTES); };
+  auto dot_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * STAGE + 2 * ROW_BYTES + TR_BYTES); };
+  auto lse_tile = [&](int buf) { return (float*)(at_lds + buf * STAGE + 2 * ROW_BYTES + 2 * TR_BYTES); };
+
+  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
+  const int k0 = blockIdx.x * 128;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
+  const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
+  const uint16_t* K = g.k.p + (int64_t)b * g.k.sb + (int64_t)hh * g.k.sh;
+  const uint16_t* V = g.v.p + (int64_t)b * g.v.sb + (int64_t)hh * g.v.sh;
+  const uint16_t* DO = g.dout.p + (int64_t)b * g.dout.sb + (int64_t)hh * g.dout.sh;
+  const float* LSE = g.lse + ((int64_t)b * g.H + hh) * g.S;
+  const float* DEL = g.delta + ((int64_t)b * g.H + hh) * g.S;
+  const int my_k = k0 + wave * 32 + li;
+
+  at_bf16x8 kf[KSTEPS], vf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const at_u32x4 uk = *(const at_u32x4*)(K + (int64_t)my_k * g.k.ss + s * 16 + h * 8);
+    const at_u32x4 uv = *(const at_u32x4*)(V + (int64_t)my_k * g.v.ss + s * 16 + h * 8);
+    kf[s] = __builtin_bit_cast(at_bf16x8, uk);
+    vf[s] = __builtin_bit_cast(at_bf16x8, uv);
+  }
+  at_f32x16 dk_acc[DT], dv_acc[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) {
+    dk_acc[d] = (at_f32x16)(0.f);
+    dv_acc[d] = (at_f32x16)(0.f);
+  }
+
+  const int first = g.causal ? k0 / 64 : 0;  // first query tile that sees key k0
+  const int n_tiles = g.S / 64;
+  RowT ql, dol;
+  TrT qtl, dotl;
+  float lreg = 0.f;  // lanes 0..63: LSE, 64..127: delta of the tile's queries
+  auto load_all = [&](int qt) {
+    ql.load(Q, g.q.ss, qt * 64);
+    dol.load(DO, g.dout.ss, qt * 64);
+    qtl.load(Q, g.q.ss, qt * 64);
+    dotl.load(DO, g.dout.ss, qt * 64);
+    if (threadIdx.x < 64) lreg = LSE[qt * 64 + threadIdx.x];
+    else if (threadIdx.x < 128) lreg = DEL[qt * 64 + threadIdx.x - 64];
+  };
+  auto store_all = [&](int buf) {
+    ql.store(q_tile(buf));
+    dol.store(do_tile(buf));
+    qtl.store(qt_tile(buf));
+    dotl.store(dot_tile(buf));
+    if (threadIdx.x < 128) lse_tile(buf)[threadIdx.x] = lreg;
+  };
+  load_all(first);
+  store_all(0);
+  __syncthreads();
+  for (int qt = first; qt < n_tiles; ++qt) {
+    const int cur = (qt - first) & 1;
+    const bool more = qt + 1 < n_tiles;
+    if (more) load_all(qt + 1);
+    const at_u32x4* Qs = q_tile(cur);
+    const at_u32x4* DOs = do_tile(cur);
+    const uint16_t* QTs = qt_tile(cur);
+    const uint16_t* DOTs = dot_tile(cur);
+    const float* Ls = lse_tile(cur);
+    const int q0 = qt * 64;
+#pragma unroll
+    for (int qt2 = 0; qt2 < 2; ++qt2) {
+      at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Qs, qt2 * 32 + li, 2 * s + h), kf[s],
+                                                        s_acc, 0, 0, 0);
+        dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(DOs, qt2 * 32 + li, 2 * s + h), vf[s],
+                                                         dp_acc, 0, 0, 0);
+      }
+      // rows of these tiles are queries: register r is query q0 + 32 qt2 + (r/4)*8 + 4h + r%4
+      at_f32x16 p, ds;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ql_ = qt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
+        const int q = q0 + ql_;
+        float pv = __expf(s_acc[r] * g.scale - Ls[ql_]);
+        if (g.causal && my_k > q) pv = 0.f;
+        p[r] = pv;
+        ds[r] = pv * (dp_acc[r] - Ls[64 + ql_]) * g.scale;
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const at_bf16x8 pf = at_regs_frag(p, t), dsf = at_regs_frag(ds, t);
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+          dv_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(DOTs, d * 32 + li, qt2, t, h), pf,
+                                                              dv_acc[d], 0, 0, 0);
+          dk_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(QTs, d * 32 + li, qt2, t, h), dsf,
+                                                              dk_acc[d], 0, 0, 0);
+        }
+      }
+    }
+    if (more) store_all(cur ^ 1);
+    __syncthreads();
+  }
+  uint16_t* DK = (uint16_t*)g.dk.p + (int64_t)b * g.dk.sb + (int64_t)hh * g.dk.sh + (int64_t)my_k * g.dk.ss;
+  uint16_t* DV = (uint16_t*)g.dv.p + (int64_t)b * g.dv.sb + (int64_t)hh * g.dv.sh + (int64_t)my_k * g.dv.ss;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      at_u32x2 wk, wv;
+      wk.x = at_pack2(dk_acc[d][gq * 4 + 0], dk_acc[d][gq * 4 + 1]);
+      wk.y = at_pack2(dk_acc[d][gq * 4 + 2], dk_acc[d][gq * 4 + 3]);
+      wv.x = at_pack2(dv_acc[d][gq * 4 + 0], dv_acc[d][gq * 4 + 1]);
+      wv.y = at_pack2(dv_acc[d][gq * 4 + 2], dv_acc[d][gq * 4 + 3]);
+      *(at_u32x2*)(DK + d * 32 + gq * 8 + 4 * h) = wk;
+      *(at_u32x2*)(DV + d * 32 + gq * 8 + 4 * h) = wv;
+    }
+}
+
+// dQ.  Grid: (S / 128, B * H).  Wave w owns queries q0 + 32w .. + 31 and walks the key tiles.
+//   S^T[key, q]  = K Q^T                (A: K tile rows, B: the wave's Q fragments)
+//   P^T          = exp(S^T * scale - LSE[q])
+//   dP^T[key, q] = V dO^T               (A: V tile rows, B: the wave's dO fragments)
+//   dS^T         = P^T * (dP^T - delta[q])
+//   dQ^T[d, q]  += K^T[d, key] dS^T[key, q] * scale   (A: transposed K tile, B: dS^T registers)
+template <int HD>
+__global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
+  using RowT = AtRowTile<HD>;
+  using TrT = AtTransTile<HD>;
+  constexpr int KSTEPS = HD / 16, DT = HD / 32;
+  constexpr int ROW_BYTES = 64 * HD * 2, TR_BYTES = HD * AT_TP * 2;
+  constexpr int STAGE = 2 * ROW_BYTES + TR_BYTES;
+  extern __shared__ __align__(16) unsigned char at_lds[];
+  auto k_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE); };
+  auto v_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE + ROW_BYTES); };
+  auto kt_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * STAGE + 2 * ROW_BYTES); };
+
+  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
+  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int q0 = qt * 128;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
+  const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
+  const uint16_t* K = g.k.p + (int64_t)b * g.k.sb + (int64_t)hh * g.k.sh;
+  const uint16_t* V = g.v.p + (int64_t)b * g.v.sb + (int64_t)hh * g.v.sh;
+  const uint16_t* DO = g.dout.p + (int64_t)b * g.dout.sb + (int64_t)hh * g.dout.sh;
+  const int my_q = q0 + wave * 32 + li;
+  const float my_lse = g.lse[((int64_t)b * g.H + hh) * g.S + my_q];
+  const float my_delta = g.delta[((int64_t)b * g.H + hh) * g.S + my_q];
+
+  at_bf16x8 qf[KSTEPS], dof[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const at_u32x4 uq = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
+    const at_u32x4 ud = *(const at_u32x4*)(DO + (int64_t)my_q * g.dout.ss + s * 16 + h * 8);
+    qf[s] = __builtin_bit_cast(at_bf16x8, uq);
+    dof[s] = __builtin_bit_cast(at_bf16x8, ud);
+  }
+  at_f32x16 dq_acc[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) dq_acc[d] = (at_f32x16)(0.f);
+
+  const int n_tiles = g.causal ? (q0 + 128) / 64 : g.S / 64;
+  RowT kl, vl;
+  TrT ktl;
+  kl.load(K, g.k.ss, 0);
+  vl.load(V, g.v.ss, 0);
+  ktl.load(K, g.k.ss, 0);
+  kl.store(k_tile(0));
+  vl.store(v_tile(0));
+  ktl.store(kt_tile(0));
+  __syncthreads();
+  for (int kt = 0; kt < n_tiles; ++kt) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < n_tiles;
+    if (more) {
+      kl.load(K, g.k.ss, (kt + 1) * 64);
+      vl.load(V, g.v.ss, (kt + 1) * 64);
+      ktl.load(K, g.k.ss, (kt + 1) * 64);
+    }
+    const at_u32x4* Ks = k_tile(cur);
+    const at_u32x4* Vs = v_tile(cur);
+    const uint16_t* KTs = kt_tile(cur);
+    const int k0 = kt * 64;
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2) {
+      at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
+                                                        s_acc, 0, 0, 0);
+        dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Vs, kt2 * 32 + li, 2 * s + h), dof[s],
+                                                         dp_acc, 0, 0, 0);
+      }
+      at_f32x16 ds;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
+        float pv = __expf(s_acc[r] * g.scale - my_lse);
+        if (g.causal && key > my_q) pv = 0.f;
+        ds[r] = pv * (dp_acc[r] - my_delta) * g.scale;
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const at_bf16x8 dsf = at_regs_frag(ds, t);
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+          dq_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(KTs, d * 32 + li, kt2, t, h), dsf,
+                                                              dq_acc[d], 0, 0, 0);
+      }
+    }
+    if (more) {
+      kl.store(k_tile(cur ^ 1));
+      vl.store(v_tile(cur ^ 1));
+      ktl.store(kt_tile(cur ^ 1));
+    }
+    __syncthreads();
+  }
+  uint16_t* DQ = (uint16_t*)g.dq.p + (int64_t)b * g.dq.sb + (int64_t)hh * g.dq.sh + (int64_t)my_q * g.dq.ss;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      at_u32x2 w;
+      w.x = at_pack2(dq_acc[d][gq * 4 + 0], dq_acc[d][gq * 4 + 1]);
+      w.y = at_pack2(dq_acc[d][gq * 4 + 2], dq_acc[d][gq * 4 + 3]);
+      *(at_u32x2*)(DQ + d * 32 + gq * 8 + 4 * h) = w;
+    }
+}
+
+// ------------------------------------------------------------------------------ host
+static int attn_tensor(const nbk_attn_tensor* t, const char* what, AttnTensor* out, bool need) {
+  if (!need && (t == nullptr || t->ptr == nullptr)) {
+    out->p = nullptr;
+    out->sb = out->ss = out->sh = 0;
+    return NBK_OK;
+  }
+  NBK_REQUIRE(t != nullptr && t->ptr != nullptr, "attention: null tensor %s", what);
+  NBK_REQUIRE(((uintptr_t)t->ptr & 15) == 0, "attention: %s is not 16-byte aligned", what);
+  NBK_REQUIRE(t->sb >= 0 && t->ss > 0 && t->sh > 0 && t->sb % 8 == 0 && t->ss % 8 == 0 && t->sh % 8 == 0,
+              "attention: strides of %s (%lld, %lld, %lld) must be positive multiples of 8 elements",
+              what, (long long)t->sb, (long long)t->ss, (long long)t->sh);
+  out->p = (const uint16_t*)t->ptr;
+  out->sb = t->sb; out->ss = t->ss; out->sh = t->sh;
+  return NBK_OK;
+}
+
+static int attn_common(const nbk_attn_desc* d, AttnArgs* a) {
+  NBK_REQUIRE(d != nullptr, "attention: null descriptor");
+  NBK_REQUIRE(d->dtype == NBK_BF16, "attention: only bf16 is implemented (dtype %d)", d->dtype);
+  NBK_REQUIRE(d->hd == 64 || d->hd == 128, "attention: head size %lld must be 64 or 128", (long long)d->hd);
+  NBK_REQUIRE(d->B > 0 && d->H > 0 && d->S > 0 && d->S % 128 == 0,
+              "attention: B %lld, H %lld, S %lld (S must be a positive multiple of 128)",
+              (long long)d->B, (long long)d->H, (long long)d->S);
+  NBK_REQUIRE(d->B * d->H <= 65535 && d->S <= (1 << 24), "attention: extent beyond the grid limits");
+  a->B = (int32_t)d->B; a->H = (int32_t)d->H; a->S = (int32_t)d->S;
+  a->causal = d->causal ? 1 : 0;
+  a->scale = d->scale;
+  return NBK_OK;
+}
+
+template <typename Kern>
+static int attn_set_lds(Kern kern, size_t bytes) {
+  if (bytes > 64 * 1024)
+    NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  return NBK_OK;
+}
+
+extern "C" int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
+                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, void* lse,
+                                 void* stream) {
+  AttnArgs a = {};
+  int rc = attn_common(d, &a);
+  if (rc) return rc;
+  if ((rc = attn_tensor(q, "q", &a.q, true)) || (rc = attn_tensor(k, "k", &a.k, true)) ||
+      (rc = attn_tensor(v, "v", &a.v, true)) || (rc = attn_tensor(o, "o", &a.o, true)))
+    return rc;
+  NBK_REQUIRE(lse != nullptr, "attention: null lse");
+  a.lse = (float*)lse;
+  const dim3 grid((unsigned)(d->S / 128), (unsigned)(d->B * d->H));
+  hipStream_t st = (hipStream_t)stream;
+  if (d->hd == 64) {
+    const size_t lds = 2 * (64 * 64 * 2 + 64 * AT_TP * 2);
+    if ((rc = attn_set_lds(attn_fwd_kernel<64>, lds))) return rc;
+    hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, dim3(256), lds, st, a);
+  } else {
+    const size_t lds = 2 * (64 * 128 * 2 + 128 * AT_TP * 2);
+    if ((rc = attn_set_lds(attn_fwd_kernel<128>, lds))) return rc;
+    hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, dim3(256), lds, st, a);
+  }
+  return nbk_check_launch("attn_fwd_kernel");
+}
+
+extern "C" int64_t nbk_attention_bwd_workspace(const nbk_attn_desc* d) {
+  if (d == nullptr || d->B <= 0 || d->H <= 0 || d->S <= 0) return -1;
+  return d->B * d->H * d->S * (int64_t)sizeof(float);
+}
+
+extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
+                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
+                                 const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                                 const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, void* workspace,
+                                 int64_t workspace_bytes, void* stream) {
+  AttnArgs a = {};
+  int rc = attn_common(d, &a);
+  if (rc) return rc;
+  if ((rc = attn_tensor(q, "q", &a.q, true)) || (rc = attn_tensor(k, "k", &a.k, true)) ||
+      (rc = attn_tensor(v, "v", &a.v, true)) || (rc = attn_tensor(o, "o", &a.o, true)) ||
+      (rc = attn_tensor(dout, "dout", &a.dout, true)) || (rc = attn_tensor(dq, "dq", &a.dq, true)) ||
+      (rc = attn_tensor(dk, "dk", &a.dk, true)) || (rc = attn_tensor(dv, "dv", &a.dv, true)))
+    return rc;
+  NBK_REQUIRE(lse != nullptr, "attention: null lse");
+  NBK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 15) == 0 &&
+                  workspace_bytes >= nbk_attention_bwd_workspace(d),
+              "attention: backward needs %lld bytes of 16-byte aligned workspace",
+              (long long)nbk_attention_bwd_workspace(d));
+  a.lse = (float*)lse;
+  a.delta = (float*)workspace;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t rows = d->B * d->H * d->S;
+  const dim3 grid((unsigned)(d->S / 128), (unsigned)(d->B * d->H));
+  if (d->hd == 64) {
+    hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)((rows * 8 + 255) / 256)), dim3(256), 0, st, a);
+    const size_t lds_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * AT_TP * 2 + 2 * 64 * 4);
+    const size_t lds_q = 2 * (2 * 64 * 64 * 2 + 64 * AT_TP * 2);
+    if ((rc = attn_set_lds(attn_bwd_kv_kernel<64>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<64>, lds_q)))
+      return rc;
+    hipLaunchKernelGGL(attn_bwd_kv_kernel<64>, grid, dim3(256), lds_kv, st, a);
+    hipLaunchKernelGGL(attn_bwd_q_kernel<64>, grid, dim3(256), lds_q, st, a);
+  } else {
+    hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st, a);
+    const size_t lds_kv = 2 * (2 * 64 * 128 * 2 + 2 * 128 * AT_TP * 2 + 2 * 64 * 4);
+    const size_t lds_q = 2 * (2 * 64 * 128 * 2 + 128 * AT_TP * 2);
+    if ((rc = attn_set_lds(attn_bwd_kv_kernel<128>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<128>, lds_q)))
+      return rc;
+    hipLaunchKernelGGL(attn_bwd_kv_kernel<128>, grid, dim3(256), lds_kv, st, a);
+    hipLaunchKernelGGL(attn_bwd_q_kernel<128>, grid, dim3(256), lds_q, st, a);
+  }
+  return nbk_check_launch("attn_bwd kernels");
+}

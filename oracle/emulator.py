@@ -256,6 +256,33 @@ def _pool(kind, a, mem):
     dst.copy_(torch.from_numpy(dx).to(dst.dtype))
 
 
+def _attention(kind, a, mem):
+    """Plain softmax attention in float64 on [B, H, S, hd] views; the backward through
+    autograd of that same expression."""
+    q, k, v = (_view(mem, a[n]).double() for n in ("q", "k", "v"))
+    S = a["S"]
+
+    def forward(q, k, v):
+        s = (q @ k.transpose(-1, -2)) * a["scale"]
+        if a["causal"]:
+            keep = torch.ones(S, S, dtype=torch.bool).tril()
+            s = s.masked_fill(~keep, float("-inf"))
+        return torch.softmax(s, dim=-1) @ v, torch.logsumexp(s, dim=-1)
+
+    if kind == "attention":
+        o, lse = forward(q, k, v)
+        dst = _view(mem, a["o"])
+        dst.copy_(o.float().to(dst.dtype))
+        _view(mem, a["lse"]).copy_(lse.float())
+        return
+    q, k, v = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o, _ = forward(q, k, v)
+    grads = torch.autograd.grad(o, (q, k, v), _view(mem, a["dout"]).double())
+    for name, g in zip(("dq", "dk", "dv"), grads):
+        dst = _view(mem, a[name])
+        dst.copy_(g.float().to(dst.dtype))
+
+
 class EmulatedPlan:
     def __init__(self, plan: Plan):
         self.plan = plan
@@ -299,6 +326,8 @@ class EmulatedPlan:
                 _conv(k, a, mem)
             elif k in ("maxpool2d", "maxpool2d_bwd"):
                 _pool(k, a, mem)
+            elif k in ("attention", "attention_bwd"):
+                _attention(k, a, mem)
             elif k == "gather":
                 t = _view(mem, a["table"]).reshape(a["outer"], a["axis_len"], a["inner"])
                 ix = _view(mem, a["idx"]).reshape(-1).long()

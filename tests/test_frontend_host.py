@@ -380,3 +380,91 @@ def test_oversized_group_is_split_locally(emulator):
     for i, y in enumerate(ys):
         np.testing.assert_array_equal(y.numpy(), x * np.float32(i + 1))
     np.testing.assert_allclose(z.numpy(), (np.maximum(x, 0) * 2).sum(1), rtol=1e-6)
+
+
+# ---- fused attention -------------------------------------------------------------------------------
+def _attn_inputs(b, h, s, hd, seed):
+    rng = np.random.default_rng(seed)
+    return [rng.standard_normal((b, h, s, hd)).astype(np.float32) for _ in range(4)]
+
+
+def _bf16_round(a):
+    import torch
+    return torch.from_numpy(a).to(torch.bfloat16).float().numpy()
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_fused_attention_op_matches_oracle_composition(emulator, causal):
+    """bf16 heads of size 64 take the fused op; its value and its three gradients agree with the
+    oracle's composition of primitive ops (float64 on the bf16-rounded inputs)."""
+    q, k, v, g = (_bf16_round(a) for a in _attn_inputs(1, 2, 128, 64, seed=5))
+    tq, tk, tv, tg = (T(a, dtype=nb.DType.bfloat16) for a in (q, k, v, g))
+
+    def loss(tq, tk, tv):
+        o = F.scaled_dot_product_attention(tq, tk, tv, is_causal=causal)
+        return nb.reduce_sum(nb.cast(o * tg, nb.DType.float32))
+
+    val, grads = nb.value_and_grad(loss, argnums=(0, 1, 2))(tq, tk, tv)
+    nb.realize_all(val, *grads)
+    kinds = last_plan().stats
+    assert kinds.get("attention") == 1 and kinds.get("attention_bwd") == 1 and "gemm" not in kinds
+    vq, vk, vv = (O.V(a.astype(np.float64)) for a in (q, k, v))
+    want = O.scaled_dot_product_attention(vq, vk, vv, is_causal=causal)
+    wl = O.reduce_sum(want * O.V(g.astype(np.float64)))
+    wg = O.grad_of(wl, [vq, vk, vv])
+    assert abs(val.item() - float(wl.a)) < 2e-2 * np.abs(want.a * g).sum()
+    for got, w in zip(grads, wg):
+        assert relerr(got.numpy().astype(np.float64), w) < 2e-2
+
+
+def test_fused_attention_reads_and_writes_heads_in_place(emulator):
+    """Inside multi-head attention the fused op reads q, k, v as strided views of the projections
+    and writes the context in [B, S, H, hd] order: no head transpose is materialised."""
+    t = oc.c3_inputs(1, 128, 128, 256, seed=2, bf16=True)
+    wl, wg = oc.c3_reference(t, num_heads=2)
+    loss, grads = oc.c3_program(nb, oc.upload(nb, t, nb.DType.bfloat16), num_heads=2)
+    nb.realize_all(loss, *grads.values())
+    st = last_plan().stats
+    assert st.get("attention") == 1 and st.get("attention_bwd") == 1
+    assert st.get("copy", 0) == 0, st
+    assert abs(loss.item() - wl) < 2e-2 * abs(wl)
+    scale = max(np.abs(g).max() for g in wg.values())
+    for k in oc.C3_PARAMS:
+        got = grads[k].numpy().astype(np.float64)
+        assert np.abs(got - wg[k]).max() <= 3e-2 * max(np.abs(wg[k]).max(), 1e-2 * scale), k
+
+
+def test_attention_falls_back_to_primitive_ops(emulator):
+    """fp32, odd head sizes, explicit masks and second-order derivatives keep the composition."""
+    q, k, v, _ = _attn_inputs(1, 2, 128, 64, seed=6)
+    o = F.scaled_dot_product_attention(T(q), T(k), T(v), is_causal=True)
+    o.realize()
+    assert "attention" not in last_plan().stats
+    with nb.config.flag("FUSED_ATTENTION", False):
+        o = F.scaled_dot_product_attention(*(T(a, dtype=nb.DType.bfloat16) for a in (q, k, v)))
+        o.realize()
+        assert "attention" not in last_plan().stats
+    with pytest.raises(ValueError, match="fused_attention covers"):
+        nb.ops.attention.fused_attention(T(q), T(k), T(v))
+
+
+def test_fused_attention_second_order_matches_primitive_ops(emulator):
+    q, k, v, g = (_bf16_round(a) for a in _attn_inputs(1, 1, 128, 64, seed=8))
+    w = _bf16_round(np.random.default_rng(9).standard_normal(q.shape).astype(np.float32))
+
+    def second(fused):
+        with nb.config.flag("FUSED_ATTENTION", fused):
+            tq, tk, tv, tg, tw = (T(a, dtype=nb.DType.bfloat16) for a in (q, k, v, g, w))
+
+            def inner(tq):
+                return nb.reduce_sum(nb.cast(F.scaled_dot_product_attention(tq, tk, tv, is_causal=True) * tg,
+                                             nb.DType.float32))
+
+            def outer(tq):
+                return nb.reduce_sum(nb.cast(nb.grad(inner)(tq) * tw, nb.DType.float32))
+
+            return nb.grad(outer)(tq).numpy().astype(np.float64)
+
+    a, b = second(True), second(False)
+    assert np.isfinite(a).all() and np.abs(b).max() > 0
+    assert relerr(a, b) < 5e-2
