@@ -937,6 +937,24 @@ class Planner:
             pb = self._mat_operand(rb)
         M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
         batch = _numel(out.shape[:-2])
+        # sum_b A[b] @ B[b] (the weight gradient x^T dy of a layer applied to a batch) is one
+        # product over the contraction index (b, k) when both operands step through it with
+        # one stride: no per-batch products to store and add up, fp32 accumulation throughout
+        users = self.users.get(out.id, ())
+        if (out.rank == 3 and batch > 1 and len(users) == 1 and out.id not in self._out_pending and
+                users[0].kind == "reduce" and users[0].fn == "sum" and users[0].attrs["axis"] == 0 and
+                users[0].pos not in self.skip_nodes and self._unit(users[0].pos) is not None and
+                not self._unit(users[0].pos).fused and
+                len(pa[0]) == 1 and len(pb[0]) == 1 and
+                pa[0][0] == (batch, K * pa[2]) and pb[0][0] == (batch, K * pb[1])):
+            red = users[0]
+            self.skip_nodes.add(red.pos)
+            dst = self._alloc_value(red.outputs[0])
+            self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
+                a=ra, b=rb, dst=dst, M=M, N=N, K=K * batch, batch=1, batch_inner=1,
+                a_bs=0, a_rs=pa[1], a_cs=pa[2], b_bs=0, b_rs=pb[1], b_cs=pb[2],
+                a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)))
+            return
         c_strides = self._matmul_out_layout(out)
         gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
         # one (outer, inner) split of the batch index has to serve A, B and C

@@ -62,8 +62,12 @@ constexpr int AT_TP = 68;  // pitch (elements) of a transposed tile row
 
 __device__ __forceinline__ float at_neg_big() { return -1.0e30f; }
 
+typedef float at_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 at_bf16x2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ uint32_t at_pack2(float a, float b) {
-  return (uint32_t)nbk_f32_to_bf16(a) | ((uint32_t)nbk_f32_to_bf16(b) << 16);
+  const at_f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, at_bf16x2));
 }
 
 // 64 x HD tile -> LDS, row-major swizzled.  256 lanes, 16 bytes each per pass.
@@ -95,35 +99,43 @@ struct AtRowTile {
   }
 };
 
-// 64 x HD tile -> LDS transposed ([HD][64], pitch AT_TP).  A lane transposes one 8 x 8
-// block: 8 rows of 16 bytes in, 8 columns of 16 bytes (two 8-byte stores) out.
+// 64 x HD tile -> LDS transposed ([HD][64], pitch AT_TP).  Every lane transposes one block of
+// KPB rows x 8 columns (KPB = 2 for hd 64, 4 for hd 128, so that 256 lanes cover the tile):
+// KPB loads of 16 bytes in, 8 stores of KPB elements out.  Lane -> block: four neighbouring
+// lanes read 64 contiguous bytes of one row, and the stores of a wave spread over all banks.
 template <int HD>
 struct AtTransTile {
-  static constexpr int NBLK = 8 * (HD / 8);  // 64 (hd 64) or 128 (hd 128) blocks
-  at_u32x4 reg[8];
-  __device__ __forceinline__ bool active() const { return threadIdx.x < NBLK; }
+  static constexpr int KPB = HD / 32;
+  static constexpr int NKB = 64 / KPB;  // row blocks
+  at_u32x4 reg[KPB];
+  static __device__ __forceinline__ void block_of(int& kb, int& db) {
+    const int t = threadIdx.x;
+    kb = (t >> 2) % NKB;
+    db = (t & 3) + 4 * (t / (4 * NKB));
+  }
   __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0) {
-    if (!active()) return;
-    const int rb = threadIdx.x % 8, db = threadIdx.x / 8;  // row block, d block
+    int kb, db;
+    block_of(kb, db);
 #pragma unroll
-    for (int r = 0; r < 8; ++r)
-      reg[r] = *(const at_u32x4*)(base + (int64_t)(row0 + rb * 8 + r) * row_stride + db * 8);
+    for (int r = 0; r < KPB; ++r)
+      reg[r] = *(const at_u32x4*)(base + (int64_t)(row0 + kb * KPB + r) * row_stride + db * 8);
   }
   __device__ __forceinline__ void store(uint16_t* lds) const {
-    if (!active()) return;
-    const int rb = threadIdx.x % 8, db = threadIdx.x / 8;
+    int kb, db;
+    block_of(kb, db);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      // column j of the block: element j of each of the 8 rows
+      // column j of the block: element j of each of the KPB rows
       const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-      at_u32x2 lo, hi;
-      lo.x = __builtin_amdgcn_perm(reg[1][j >> 1], reg[0][j >> 1], sel);
-      lo.y = __builtin_amdgcn_perm(reg[3][j >> 1], reg[2][j >> 1], sel);
-      hi.x = __builtin_amdgcn_perm(reg[5][j >> 1], reg[4][j >> 1], sel);
-      hi.y = __builtin_amdgcn_perm(reg[7][j >> 1], reg[6][j >> 1], sel);
-      uint16_t* dst = lds + (db * 8 + j) * AT_TP + rb * 8;
-      *(at_u32x2*)dst = lo;
-      *(at_u32x2*)(dst + 4) = hi;
+      uint16_t* dst = lds + (db * 8 + j) * AT_TP + kb * KPB;
+      if constexpr (KPB == 2) {
+        *(uint32_t*)dst = __builtin_amdgcn_perm(reg[1][j >> 1], reg[0][j >> 1], sel);
+      } else {
+        at_u32x2 w;
+        w.x = __builtin_amdgcn_perm(reg[1][j >> 1], reg[0][j >> 1], sel);
+        w.y = __builtin_amdgcn_perm(reg[3][j >> 1], reg[2][j >> 1], sel);
+        *(at_u32x2*)dst = w;
+      }
     }
   }
   // A fragment of the second MFMA: row d, k-slots of the t-th 16-wide step of 32-row tile kt2
@@ -153,6 +165,15 @@ __device__ __forceinline__ float at_xhalf(float v) { return __shfl_xor(v, 32, 64
 
 // ------------------------------------------------------------------------------ forward
 // Grid: (S / 128, B * H).  Wave w owns queries q0 + 32w .. + 31 (one per lane pair).
+//
+// The softmax runs in base 2 on t = score * scale * log2(e).  The running maximum m of a
+// row is only raised when some row of the wave has outgrown it by more than AT_SLACK (a
+// wave-uniform decision): until then exp2(t - m) <= 2^AT_SLACK, which fp32 sums and bf16
+// probabilities hold without loss, and the accumulators need no rescaling.
+constexpr float AT_SLACK = 8.0f;
+constexpr float AT_LOG2E = 1.4426950408889634f;
+constexpr float AT_LN2 = 0.6931471805599453f;
+
 template <int HD>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
   using RowT = AtRowTile<HD>;
@@ -170,7 +191,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
   const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
   const uint16_t* K = g.k.p + (int64_t)b * g.k.sb + (int64_t)hh * g.k.sh;
   const uint16_t* V = g.v.p + (int64_t)b * g.v.sb + (int64_t)hh * g.v.sh;
-  const int my_q = q0 + wave * 32 + li;
+  const int wq0 = q0 + wave * 32;  // first query of the wave
+  const int my_q = wq0 + li;
+  const float c = g.scale * AT_LOG2E;
 
   // the wave's queries as B fragments of the score MFMA
   at_bf16x8 qf[KSTEPS];
@@ -203,57 +226,64 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
     const at_u32x4* Ks = k_tile(cur);
     const uint16_t* Vs = v_tile(cur);
     const int k0 = kt * 64;
-    // transposed scores: rows = keys (two 32-row tiles), columns = the wave's queries
-    at_f32x16 st[2];
+    auto tile = [&](auto masked) {
+      constexpr bool MASK = decltype(masked)::value;
+      // transposed scores: rows = keys (two 32-row tiles), columns = the wave's queries
+      at_f32x16 st[2];
 #pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2) {
-      at_f32x16 acc = (at_f32x16)(0.f);
+      for (int kt2 = 0; kt2 < 2; ++kt2) {
+        at_f32x16 acc = (at_f32x16)(0.f);
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
-                                                      acc, 0, 0, 0);
-      st[kt2] = acc;
-    }
-    // scale, mask, running max
-    float mx = at_neg_big();
-#pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
-        float v = st[kt2][r] * g.scale;
-        if (g.causal && key > my_q) v = at_neg_big();
-        st[kt2][r] = v;
-        mx = fmaxf(mx, v);
+        for (int s = 0; s < KSTEPS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
+                                                        acc, 0, 0, 0);
+        st[kt2] = acc;
       }
-    mx = fmaxf(mx, at_xhalf(mx));
-    const float m_new = fmaxf(m_i, mx);
-    const float alpha = __expf(m_i - m_new);
-    float sum = 0.f;
+      float mx = at_neg_big();
 #pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2)
+      for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __expf(st[kt2][r] - m_new);
-        st[kt2][r] = p;
-        sum += p;
+        for (int r = 0; r < 16; ++r) {
+          if (MASK) {
+            const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
+            if (key > my_q) st[kt2][r] = at_neg_big();
+          }
+          mx = fmaxf(mx, st[kt2][r]);
+        }
+      mx = fmaxf(mx, at_xhalf(mx)) * c;
+      if (__any(mx - m_i > AT_SLACK)) {
+        const float m_new = fmaxf(m_i, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+        l_i *= alpha;
+        m_i = m_new;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) o_acc[d] *= alpha;
       }
-    sum += at_xhalf(sum);
-    l_i = l_i * alpha + sum;
-    m_i = m_new;
+      float sum = 0.f;
 #pragma unroll
-    for (int d = 0; d < DT; ++d) o_acc[d] *= alpha;
-    // O^T[d, q] += V^T[d, key] P^T[key, q]
+      for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2)
+        for (int r = 0; r < 16; ++r) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kt2][r], c, -m_i));
+          st[kt2][r] = p;
+          sum += p;
+        }
+      l_i += sum;  // each half of the lane pair keeps the sum of its own keys
+      // O^T[d, q] += V^T[d, key] P^T[key, q]
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const at_bf16x8 pf = at_regs_frag(st[kt2], t);
+      for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-        for (int d = 0; d < DT; ++d)
-          o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
-                                                             o_acc[d], 0, 0, 0);
-      }
+        for (int t = 0; t < 2; ++t) {
+          const at_bf16x8 pf = at_regs_frag(st[kt2], t);
+#pragma unroll
+          for (int d = 0; d < DT; ++d)
+            o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
+                                                               o_acc[d], 0, 0, 0);
+        }
+    };
+    // keys of this tile against the wave's queries: all visible, some, or none
+    if (!g.causal || k0 + 63 <= wq0) tile(std::false_type{});
+    else if (k0 <= wq0 + 31) tile(std::true_type{});
     if (more) {
       kl.store(k_tile(cur ^ 1));
       vl.store(v_tile(cur ^ 1));
@@ -261,6 +291,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
     __syncthreads();
   }
   // normalise and write: register r of tile d is O[my_q][32 d + (r/4)*8 + 4h + r%4]
+  l_i += at_xhalf(l_i);
   const float inv = 1.0f / l_i;
   uint16_t* O = (uint16_t*)g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)my_q * g.o.ss;
 #pragma unroll
@@ -272,7 +303,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
       w.y = at_pack2(o_acc[d][gq * 4 + 2] * inv, o_acc[d][gq * 4 + 3] * inv);
       *(at_u32x2*)(O + d * 32 + gq * 8 + 4 * h) = w;
     }
-  if (h == 0) g.lse[((int64_t)b * g.H + hh) * g.S + my_q] = m_i + __logf(l_i);
+  if (h == 0) g.lse[((int64_t)b * g.H + hh) * g.S + my_q] = m_i * AT_LN2 + __logf(l_i);
 }
 
 // ------------------------------------------------------------------------------ backward
@@ -308,11 +339,11 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs g) {
 // dK, dV.  Grid: (S / 128, B * H).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
 // and walks the query tiles that can see them.
 //   S[q, key]  = Q K^T          (A: Q tile rows, B: the wave's K fragments)
-//   P          = exp(S * scale - LSE[q])
+//   P          = exp(S * scale - LSE[q])   (as exp2, with LSE staged in base-2 units)
 //   dV^T[d,key] += dO^T[d, q] P[q, key]        (A: transposed dO tile, B: P registers)
 //   dP[q, key] = dO V^T         (A: dO tile rows, B: the wave's V fragments)
 //   dS         = P * (dP - delta[q])
-//   dK^T[d,key] += Q^T[d, q] dS[q, key] * scale (A: transposed Q tile, B: dS registers)
+//   dK^T[d,key] += Q^T[d, q] dS[q, key]         (A: transposed Q tile, B: dS registers; * scale at the end)
 template <int HD>
 __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
   using RowT = AtRowTile<HD>;
@@ -363,7 +394,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
     dol.load(DO, g.dout.ss, qt * 64);
     qtl.load(Q, g.q.ss, qt * 64);
     dotl.load(DO, g.dout.ss, qt * 64);
-    if (threadIdx.x < 64) lreg = LSE[qt * 64 + threadIdx.x];
+    if (threadIdx.x < 64) lreg = LSE[qt * 64 + threadIdx.x] * AT_LOG2E;
     else if (threadIdx.x < 128) lreg = DEL[qt * 64 + threadIdx.x - 64];
   };
   auto store_all = [&](int buf) {
@@ -373,6 +404,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
     dotl.store(dot_tile(buf));
     if (threadIdx.x < 128) lse_tile(buf)[threadIdx.x] = lreg;
   };
+  const int wk0 = k0 + wave * 32;  // first key of the wave
+  const float c = g.scale * AT_LOG2E;
   load_all(first);
   store_all(0);
   __syncthreads();
@@ -386,8 +419,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
     const uint16_t* DOTs = dot_tile(cur);
     const float* Ls = lse_tile(cur);
     const int q0 = qt * 64;
-#pragma unroll
-    for (int qt2 = 0; qt2 < 2; ++qt2) {
+    auto subtile = [&](auto masked, int qt2) {
+      constexpr bool MASK = decltype(masked)::value;
       at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
@@ -399,13 +432,19 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
       // rows of these tiles are queries: register r is query q0 + 32 qt2 + (r/4)*8 + 4h + r%4
       at_f32x16 p, ds;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int ql_ = qt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
-        const int q = q0 + ql_;
-        float pv = __expf(s_acc[r] * g.scale - Ls[ql_]);
-        if (g.causal && my_k > q) pv = 0.f;
-        p[r] = pv;
-        ds[r] = pv * (dp_acc[r] - Ls[64 + ql_]) * g.scale;
+      for (int gq = 0; gq < 4; ++gq) {
+        const int qb = qt2 * 32 + gq * 8 + 4 * h;
+        const float4 l4 = *(const float4*)(Ls + qb);
+        const float4 d4 = *(const float4*)(Ls + 64 + qb);
+        const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dv[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = gq * 4 + e;
+          float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[r], c, -lv[e]));
+          if (MASK && my_k > q0 + qb + e) pv = 0.f;
+          p[r] = pv;
+          ds[r] = pv * (dp_acc[r] - dv[e]);
+        }
       }
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -418,6 +457,12 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
                                                               dk_acc[d], 0, 0, 0);
         }
       }
+    };
+#pragma unroll
+    for (int qt2 = 0; qt2 < 2; ++qt2) {
+      const int sq0 = q0 + qt2 * 32;  // queries sq0 .. sq0 + 31 against keys wk0 .. wk0 + 31
+      if (!g.causal || wk0 + 31 <= sq0) subtile(std::false_type{}, qt2);
+      else if (wk0 <= sq0 + 31) subtile(std::true_type{}, qt2);
     }
     if (more) store_all(cur ^ 1);
     __syncthreads();
@@ -429,8 +474,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       at_u32x2 wk, wv;
-      wk.x = at_pack2(dk_acc[d][gq * 4 + 0], dk_acc[d][gq * 4 + 1]);
-      wk.y = at_pack2(dk_acc[d][gq * 4 + 2], dk_acc[d][gq * 4 + 3]);
+      wk.x = at_pack2(dk_acc[d][gq * 4 + 0] * g.scale, dk_acc[d][gq * 4 + 1] * g.scale);
+      wk.y = at_pack2(dk_acc[d][gq * 4 + 2] * g.scale, dk_acc[d][gq * 4 + 3] * g.scale);
       wv.x = at_pack2(dv_acc[d][gq * 4 + 0], dv_acc[d][gq * 4 + 1]);
       wv.y = at_pack2(dv_acc[d][gq * 4 + 2], dv_acc[d][gq * 4 + 3]);
       *(at_u32x2*)(DK + d * 32 + gq * 8 + 4 * h) = wk;
@@ -443,7 +488,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
 //   P^T          = exp(S^T * scale - LSE[q])
 //   dP^T[key, q] = V dO^T               (A: V tile rows, B: the wave's dO fragments)
 //   dS^T         = P^T * (dP^T - delta[q])
-//   dQ^T[d, q]  += K^T[d, key] dS^T[key, q] * scale   (A: transposed K tile, B: dS^T registers)
+//   dQ^T[d, q]  += K^T[d, key] dS^T[key, q]   (A: transposed K tile, B: dS^T registers; * scale at the end)
 template <int HD>
 __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
   using RowT = AtRowTile<HD>;
@@ -465,7 +510,9 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
   const uint16_t* V = g.v.p + (int64_t)b * g.v.sb + (int64_t)hh * g.v.sh;
   const uint16_t* DO = g.dout.p + (int64_t)b * g.dout.sb + (int64_t)hh * g.dout.sh;
   const int my_q = q0 + wave * 32 + li;
-  const float my_lse = g.lse[((int64_t)b * g.H + hh) * g.S + my_q];
+  const float my_lse = g.lse[((int64_t)b * g.H + hh) * g.S + my_q] * AT_LOG2E;
+  const int wq0 = q0 + wave * 32;  // first query of the wave
+  const float c = g.scale * AT_LOG2E;
   const float my_delta = g.delta[((int64_t)b * g.H + hh) * g.S + my_q];
 
   at_bf16x8 qf[KSTEPS], dof[KSTEPS];
@@ -502,8 +549,8 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
     const at_u32x4* Vs = v_tile(cur);
     const uint16_t* KTs = kt_tile(cur);
     const int k0 = kt * 64;
-#pragma unroll
-    for (int kt2 = 0; kt2 < 2; ++kt2) {
+    auto subtile = [&](auto masked, int kt2) {
+      constexpr bool MASK = decltype(masked)::value;
       at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
@@ -515,10 +562,12 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
       at_f32x16 ds;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
-        float pv = __expf(s_acc[r] * g.scale - my_lse);
-        if (g.causal && key > my_q) pv = 0.f;
-        ds[r] = pv * (dp_acc[r] - my_delta) * g.scale;
+        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[r], c, -my_lse));
+        if (MASK) {
+          const int key = k0 + kt2 * 32 + (r >> 2) * 8 + 4 * h + (r & 3);
+          if (key > my_q) pv = 0.f;
+        }
+        ds[r] = pv * (dp_acc[r] - my_delta);
       }
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -528,6 +577,12 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
           dq_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(KTs, d * 32 + li, kt2, t, h), dsf,
                                                               dq_acc[d], 0, 0, 0);
       }
+    };
+#pragma unroll
+    for (int kt2 = 0; kt2 < 2; ++kt2) {
+      const int sk0 = k0 + kt2 * 32;  // keys sk0 .. sk0 + 31 against queries wq0 .. wq0 + 31
+      if (!g.causal || sk0 + 31 <= wq0) subtile(std::false_type{}, kt2);
+      else if (sk0 <= wq0 + 31) subtile(std::true_type{}, kt2);
     }
     if (more) {
       kl.store(k_tile(cur ^ 1));
@@ -542,8 +597,8 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       at_u32x2 w;
-      w.x = at_pack2(dq_acc[d][gq * 4 + 0], dq_acc[d][gq * 4 + 1]);
-      w.y = at_pack2(dq_acc[d][gq * 4 + 2], dq_acc[d][gq * 4 + 3]);
+      w.x = at_pack2(dq_acc[d][gq * 4 + 0] * g.scale, dq_acc[d][gq * 4 + 1] * g.scale);
+      w.y = at_pack2(dq_acc[d][gq * 4 + 2] * g.scale, dq_acc[d][gq * 4 + 3] * g.scale);
       *(at_u32x2*)(DQ + d * 32 + gq * 8 + 4 * h) = w;
     }
 }

@@ -468,3 +468,16 @@ def test_fused_attention_second_order_matches_primitive_ops(emulator):
     a, b = second(True), second(False)
     assert np.isfinite(a).all() and np.abs(b).max() > 0
     assert relerr(a, b) < 5e-2
+
+
+def test_weight_gradient_over_a_batch_is_one_product(emulator):
+    """sum_b x[b]^T dy[b] contracts over (b, s) in a single GEMM: no per-batch products, no
+    reduction afterwards."""
+    x = RNG.standard_normal((3, 16, 8)).astype(np.float32)
+    w = RNG.standard_normal((8, 5)).astype(np.float32)
+    g = RNG.standard_normal((3, 16, 5)).astype(np.float32)
+    gw = nb.grad(lambda w: nb.reduce_sum(nb.matmul(T(x), w) * T(g)), create_graph=False)(T(w))
+    gw.realize()
+    st = last_plan().stats
+    assert "reduce_mid" not in st and st["gemm"] == 1, st
+    np.testing.assert_allclose(gw.numpy(), np.einsum("bsd,bsn->dn", x, g), rtol=1e-5, atol=1e-5)
