@@ -949,11 +949,7 @@ class Planner:
                 pa[0][0] == (batch, K * pa[2]) and pb[0][0] == (batch, K * pb[1])):
             red = users[0]
             self.skip_nodes.add(red.pos)
-            dst = self._alloc_value(red.outputs[0])
-            self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
-                a=ra, b=rb, dst=dst, M=M, N=N, K=K * batch, batch=1, batch_inner=1,
-                a_bs=0, a_rs=pa[1], a_cs=pa[2], b_bs=0, b_rs=pb[1], b_cs=pb[2],
-                a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)))
+            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K * batch, red.outputs[0])
             return
         c_strides = self._matmul_out_layout(out)
         gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
@@ -993,6 +989,9 @@ class Planner:
                 pa[0][0][1] == M * pa[1] and c_strides == contiguous_strides(out.shape)):
             M, batch = M * batch, 1
             a_bs = c_bs = 0
+        if batch == 1 and c_strides == contiguous_strides(out.shape):
+            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K, out)
+            return
         if c_strides == contiguous_strides(out.shape):
             dst = self._alloc_value(out)
         else:
@@ -1004,6 +1003,38 @@ class Planner:
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
             ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
+
+    @staticmethod
+    def _split_k(M: int, N: int, K: int, dtype: DType) -> int:
+        """Slices of the contraction axis for a product whose output has too few 128 x 128
+        tiles to occupy the GPU while K is long (weight gradients: K = batch x sequence)."""
+        if dtype is not DType.bfloat16:
+            return 1
+        tiles = ((M + 127) // 128) * ((N + 127) // 128)
+        ks = 1
+        while tiles * ks < 512 and tiles < 128 and K % (ks * 2 * 64) == 0 and K // (ks * 2) >= 512:
+            ks *= 2
+        return ks
+
+    def _emit_plain_gemm(self, ra: ViewRef, rb: ViewRef, pa, pb, M: int, N: int, K: int,
+                         out: ir.Value) -> None:
+        """One unbatched product into contiguous storage for ``out``; split along K into fp32
+        partial products plus their sum when the output alone gives too few workgroups."""
+        ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32)
+        dst = self._alloc_value(out)
+        common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
+                      batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
+        if ks == 1:
+            self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
+                common, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
+            return
+        kc = K // ks
+        tmp = self._new_buf((ks, M, N), DType.float32)
+        tref = ViewRef(tmp.id, 0, (ks, M, N), contiguous_strides((ks, M, N)), DType.float32)
+        self._emit(Step("gemm", [ra.buf, rb.buf], [tmp.id], dict(
+            common, dst=tref, K=kc, batch=ks, a_bs=kc * pa[2], b_bs=kc * pb[1])))
+        self._emit(Step("reduce_mid", [tmp.id], [dst.buf], dict(
+            src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum")))
 
     # ................................................................ attention
     def _heads_operand(self, v: ir.Value) -> ViewRef:
