@@ -379,6 +379,7 @@ extern __shared__ __align__(16) float rp_stage_lds[];
 def collect_programs() -> dict[int, dict]:
     """Plan the five benchmark steps at full size and return {hash: rowprog attrs}."""
     import nabla_amd as nb
+    from nabla_amd import config
     from nabla_amd import workloads as W
     from nabla_amd.backend import executor
     from nabla_amd.core.engine import _PLAN_CACHE, clear_plan_cache
@@ -436,6 +437,20 @@ def collect_programs() -> dict[int, dict]:
         t5 = leaves({k: v for k, v in s5.items() if k != "ids"}, bf16)
         t5["ids"] = nb.Tensor._from_torch(torch.zeros(s5["ids"], dtype=i64))
         jobs.append(lambda: W.c5_step(t5))
+
+        def with_flags(job, **flags):
+            """The same step under other evaluation orders (attention out of primitive ops,
+            lora_linear as the reference writes it), so that those keep compiled kernels too."""
+            def run():
+                import contextlib
+                with contextlib.ExitStack() as es:
+                    for name, value in flags.items():
+                        es.enter_context(config.flag(name, value))
+                    return job()
+            return run
+
+        jobs.append(with_flags(jobs[2], FUSED_ATTENTION=False))
+        jobs.append(with_flags(jobs[4], FUSED_ATTENTION=False, LORA_LOW_RANK_ORDER=False))
         for job in jobs:
             clear_plan_cache()
             res = job()

@@ -26,11 +26,17 @@ _TRACING: ContextVar[bool] = ContextVar("TRACING", default=False)
 _FUSED_ATTENTION: ContextVar[bool] = ContextVar("FUSED_ATTENTION",
                                                 default=_env_flag("NBK_FUSED_ATTENTION", True))
 
+# lora_linear as x@W + ((x@A)@B)*s instead of the reference's x@W + x@((A@B)*s): the same
+# function without the full-size delta and its two extra full GEMMs (three with the backward)
+_LORA_LOW_RANK_ORDER: ContextVar[bool] = ContextVar("LORA_LOW_RANK_ORDER",
+                                                    default=_env_flag("NBK_LORA_LOW_RANK_ORDER", True))
+
 _FLAGS = {
     "EAGER_MAX_GRAPH": _EAGER_MAX_GRAPH,
     "VERIFY_EAGER_SHAPES": _VERIFY_EAGER_SHAPES,
     "TRACING": _TRACING,
     "FUSED_ATTENTION": _FUSED_ATTENTION,
+    "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
 }
 
 

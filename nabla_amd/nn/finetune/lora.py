@@ -1,8 +1,15 @@
 """LoRA helpers (nabla/nn/finetune/lora.py): init_lora_adapter 16-52,
-lora_delta 55-69 = ``(A @ B) * (alpha / rank)``, lora_linear 72-79 =
-``x @ W + x @ delta`` exactly as written there, merge / unmerge."""
+lora_delta 55-69 = ``(A @ B) * (alpha / rank)``, lora_linear 72-79, merge / unmerge.
+
+The reference writes ``lora_linear`` as ``x @ W + x @ delta``: a full ``[D, D]`` delta and
+a second full GEMM forward, and two more full GEMMs in the backward pass (``x^T dy`` and
+``dy delta^T``).  With ``config.LORA_LOW_RANK_ORDER`` (the default) the same function is
+evaluated as ``x @ W + ((x @ A) @ B) * (alpha / rank)``: every adapter product is rank-sized
+in both directions.  The two orders differ by rounding only; switch the flag off for the
+order as written."""
 from __future__ import annotations
 
+from ... import config
 from ...core.dtype import DType
 from ...core.tensor import Tensor
 from ...ops.creation import zeros
@@ -30,6 +37,9 @@ def lora_delta(adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
 
 def lora_linear(x: Tensor, frozen_weight: Tensor, adapter: dict[str, Tensor],
                 alpha: float = 1.0) -> Tensor:
+    if config.LORA_LOW_RANK_ORDER:
+        A, B = adapter["A"], adapter["B"]
+        return (x @ frozen_weight) + ((x @ A) @ B) * (alpha / float(int(A.shape[1])))
     return (x @ frozen_weight) + (x @ lora_delta(adapter, alpha=alpha))
 
 
