@@ -175,7 +175,7 @@ constexpr float AT_LOG2E = 1.4426950408889634f;
 constexpr float AT_LN2 = 0.6931471805599453f;
 
 template <int HD>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs g) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   using RowT = AtRowTile<HD>;
   using TrT = AtTransTile<HD>;
   constexpr int KSTEPS = HD / 16, DT = HD / 32;
@@ -489,8 +489,11 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
 //   dP^T[key, q] = V dO^T               (A: V tile rows, B: the wave's dO fragments)
 //   dS^T         = P^T * (dP^T - delta[q])
 //   dQ^T[d, q]  += K^T[d, key] dS^T[key, q]   (A: transposed K tile, B: dS^T registers; * scale at the end)
-template <int HD>
-__global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
+// NSTAGE: LDS stages.  With head size 128 one stage is 50 KB: a single stage lets two workgroups
+// share a CU (two waves per SIMD that cover each other's waits), which is worth more than
+// overlapping the tile copy inside one workgroup.
+template <int HD, int NSTAGE>
+__global__ __launch_bounds__(256, 2) void attn_bwd_q_kernel(const AttnArgs g) {
   using RowT = AtRowTile<HD>;
   using TrT = AtTransTile<HD>;
   constexpr int KSTEPS = HD / 16, DT = HD / 32;
@@ -538,7 +541,8 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
   ktl.store(kt_tile(0));
   __syncthreads();
   for (int kt = 0; kt < n_tiles; ++kt) {
-    const int cur = kt & 1;
+    const int cur = NSTAGE == 2 ? (kt & 1) : 0;
+    const int nxt = NSTAGE == 2 ? (cur ^ 1) : 0;
     const bool more = kt + 1 < n_tiles;
     if (more) {
       kl.load(K, g.k.ss, (kt + 1) * 64);
@@ -585,9 +589,10 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const AttnArgs g) {
       else if (sk0 <= wq0 + 31) subtile(std::true_type{}, kt2);
     }
     if (more) {
-      kl.store(k_tile(cur ^ 1));
-      vl.store(v_tile(cur ^ 1));
-      ktl.store(kt_tile(cur ^ 1));
+      if (NSTAGE == 1) __syncthreads();  // everyone is done reading the only stage
+      kl.store(k_tile(nxt));
+      vl.store(v_tile(nxt));
+      ktl.store(kt_tile(nxt));
     }
     __syncthreads();
   }
@@ -698,18 +703,18 @@ extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* 
     hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)((rows * 8 + 255) / 256)), dim3(256), 0, st, a);
     const size_t lds_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * AT_TP * 2 + 2 * 64 * 4);
     const size_t lds_q = 2 * (2 * 64 * 64 * 2 + 64 * AT_TP * 2);
-    if ((rc = attn_set_lds(attn_bwd_kv_kernel<64>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<64>, lds_q)))
+    if ((rc = attn_set_lds(attn_bwd_kv_kernel<64>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<64, 2>, lds_q)))
       return rc;
     hipLaunchKernelGGL(attn_bwd_kv_kernel<64>, grid, dim3(256), lds_kv, st, a);
-    hipLaunchKernelGGL(attn_bwd_q_kernel<64>, grid, dim3(256), lds_q, st, a);
+    hipLaunchKernelGGL((attn_bwd_q_kernel<64, 2>), grid, dim3(256), lds_q, st, a);
   } else {
     hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st, a);
     const size_t lds_kv = 2 * (2 * 64 * 128 * 2 + 2 * 128 * AT_TP * 2 + 2 * 64 * 4);
-    const size_t lds_q = 2 * (2 * 64 * 128 * 2 + 128 * AT_TP * 2);
-    if ((rc = attn_set_lds(attn_bwd_kv_kernel<128>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<128>, lds_q)))
+    const size_t lds_q = 2 * 64 * 128 * 2 + 128 * AT_TP * 2;
+    if ((rc = attn_set_lds(attn_bwd_kv_kernel<128>, lds_kv)) || (rc = attn_set_lds(attn_bwd_q_kernel<128, 1>, lds_q)))
       return rc;
     hipLaunchKernelGGL(attn_bwd_kv_kernel<128>, grid, dim3(256), lds_kv, st, a);
-    hipLaunchKernelGGL(attn_bwd_q_kernel<128>, grid, dim3(256), lds_q, st, a);
+    hipLaunchKernelGGL((attn_bwd_q_kernel<128, 1>), grid, dim3(256), lds_q, st, a);
   }
   return nbk_check_launch("attn_bwd kernels");
 }
