@@ -52,7 +52,8 @@ def test_row_reduce_and_grad(hip):
 @pytest.mark.parametrize("shape", [(128, 128, 64), (200, 136, 72), (512, 384, 256), (64, 10, 256),
                                    (1024, 1024, 512),
                                    (5000, 4104, 192),    # 128 x 128 tiles, many, ragged edges
-                                   (5000, 5128, 128)])   # 256 x 256 tiles with ragged edges
+                                   (5000, 5128, 128),
+                                   (4000, 2600, 192)])   # 256 x 256 tiles with ragged edges
 def test_gemm(hip, dtype, layout, shape):
     from nabla_amd.backend import lib
     M, N, K = shape
