@@ -287,7 +287,8 @@ def main() -> int:
         peak, unit = MFMA_PEAK_TFLOPS[w["dtype"]], "TFLOP/s"
     roofline = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
                 "frac": round(achieved / peak, 4), "traffic": measured_traffic(a.workload),
-                "kernel": "+".join(dominant_kinds), "kernel_ms_per_step": round(dom_ms, 4),
+                "kernel": "+".join(k for k in dominant_kinds if k in plan.stats),
+                "kernel_ms_per_step": round(dom_ms, 4),
                 "launches_per_step": len(per_step_total)}
     cpu = None if a.no_cpu else w["cpu"]()
     line = {
