@@ -151,8 +151,8 @@ extern "C" int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void*
 // ---- reduction over a middle axis ---------------------------------------------
 // in [outer, red, inner] -> out [outer, inner].  Lanes run along `inner`
 // (coalesced); each workgroup owns a 64-column strip and splits `red` over its
-// four waves, then combines the four partials through LDS.  Two-level split of
-// `red` across workgroups goes through fp32 atomics only for sums of long axes.
+// four waves, then combines the four partials through LDS.  (A long axis over few
+// columns is cut into slices by the caller: two launches, fp32 partials in between.)
 __device__ __forceinline__ float red_comb(float a, float b, int kind) {
   return kind == NBK_RED_SUM ? a + b : (kind == NBK_RED_MAX ? fmaxf(a, b) : fminf(a, b));
 }
