@@ -17,6 +17,7 @@ from .ops import (BinaryOperation, CreationOperation, Operation, ReduceOperation
 from .ops.reduction import reduce_max as max, reduce_min as min, reduce_sum as sum  # noqa: A001
 from .transforms import (CompilationStats, CompiledFunction, compile, grad, value_and_grad, vjp)
 from . import nn  # noqa: E402
+from . import testing  # noqa: E402
 from . import workloads  # noqa: E402
 
 __version__ = "0.1.0"

@@ -91,6 +91,13 @@ class Builder:
                     return hit.outputs
             except TypeError:
                 key = None
+        if kind in ("ew", "reduce", "argreduce", "matmul", "fill"):
+            for _, dtype in outs:
+                if dtype is DType.uint8:
+                    # the kernels store one-byte results as 0 / 1 (bool); uint8 is for data that
+                    # comes in from the host (quantised weights) and is cast before arithmetic
+                    raise TypeError(f"'{fn or kind}' would produce uint8: cast uint8 data to "
+                                    "int32 or a float type first")
         node = Node(kind, fn, inputs, attrs, len(self.nodes))
         for i, (shape, dtype) in enumerate(outs):
             node.outputs.append(Value(shape, dtype, node, i, self._n_values))

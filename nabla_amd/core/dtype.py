@@ -19,6 +19,7 @@ class DType(enum.Enum):
     float16 = "float16"
     int32 = "int32"
     int64 = "int64"
+    uint8 = "uint8"
     bool = "bool"
 
     # -- classification ---------------------------------------------------
@@ -26,7 +27,7 @@ class DType(enum.Enum):
         return self in (DType.float32, DType.bfloat16, DType.float16)
 
     def is_integral(self) -> bool:
-        return self in (DType.int32, DType.int64)
+        return self in (DType.int32, DType.int64, DType.uint8)
 
     @property
     def size_in_bytes(self) -> int:
@@ -67,23 +68,23 @@ class DType(enum.Enum):
 
 _SIZE = {
     DType.float32: 4, DType.bfloat16: 2, DType.float16: 2,
-    DType.int32: 4, DType.int64: 8, DType.bool: 1,
+    DType.int32: 4, DType.int64: 8, DType.uint8: 1, DType.bool: 1,
 }
 _TO_TORCH = {
     DType.float32: torch.float32, DType.bfloat16: torch.bfloat16, DType.float16: torch.float16,
-    DType.int32: torch.int32, DType.int64: torch.int64, DType.bool: torch.bool,
+    DType.int32: torch.int32, DType.int64: torch.int64, DType.uint8: torch.uint8,
+    DType.bool: torch.bool,
 }
 _FROM_TORCH = {v: k for k, v in _TO_TORCH.items()}
-_FROM_TORCH[torch.uint8] = DType.bool
 _TO_NUMPY = {
     DType.float32: np.float32, DType.float16: np.float16,
-    DType.int32: np.int32, DType.int64: np.int64, DType.bool: np.bool_,
+    DType.int32: np.int32, DType.int64: np.int64, DType.uint8: np.uint8, DType.bool: np.bool_,
 }
 _FROM_NUMPY = {np.dtype(v): k for k, v in _TO_NUMPY.items()}
 _FROM_NUMPY[np.dtype(np.float64)] = DType.float32  # host doubles narrow to the default float
 _ABI = {
     DType.float32: 0, DType.bfloat16: 1, DType.float16: 2,
-    DType.int32: 3, DType.int64: 4, DType.bool: 5,
+    DType.int32: 3, DType.int64: 4, DType.uint8: 5, DType.bool: 5,  # one byte either way
 }
 
 
@@ -91,7 +92,8 @@ def promote(a: DType, b: DType) -> DType:
     """Result type of a binary arithmetic op on ``a`` and ``b``."""
     if a is b:
         return a
-    order = [DType.bool, DType.int32, DType.int64, DType.float16, DType.bfloat16, DType.float32]
+    order = [DType.bool, DType.uint8, DType.int32, DType.int64, DType.float16, DType.bfloat16,
+             DType.float32]
     if {a, b} == {DType.float16, DType.bfloat16}:
         return DType.float32
     return order[max(order.index(a), order.index(b))]

@@ -387,6 +387,13 @@ class Tensor:
 
     astype = cast
 
+    def to(self, target):
+        """``to(dtype)`` casts; ``to(device)`` is the identity on this single-device backend
+        (api.py ``Tensor.to``)."""
+        if isinstance(target, DType):
+            return self if target is self.dtype else self.cast(target)
+        return self
+
     def type_as(self, other: "Tensor"):
         return self.cast(other.dtype)
 

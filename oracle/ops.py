@@ -528,3 +528,34 @@ def lora_linear(x, w, A, B, alpha: float) -> V:
     A = _v(A)
     scale = alpha / float(A.a.shape[1])
     return matmul(x, w) + matmul(x, matmul(A, B) * scale)
+
+
+# ---- NF4 (nn/finetune/qlora.py) -------------------------------------------------------------
+#: qlora.py:18-38
+NF4_LEVELS = np.array([-1.0, -0.6962, -0.5251, -0.3949, -0.2844, -0.1848, -0.0911, 0.0,
+                       0.0796, 0.1609, 0.2461, 0.3379, 0.4407, 0.5626, 0.7230, 1.0], dtype=np.float32)
+
+
+def nf4_quantize(w: np.ndarray, block_size: int = 64) -> dict:
+    """qlora.py:41-75 in fp32: flatten, zero-pad to whole blocks, scale every block by its
+    absolute maximum (1 for an all-zero block), index of the nearest level (first on a tie)."""
+    flat = np.asarray(w, dtype=np.float32).reshape(-1)
+    numel = flat.size
+    pad = (block_size - numel % block_size) % block_size
+    flat = np.pad(flat, (0, pad))
+    blocks = flat.reshape(-1, block_size)
+    scales = np.max(np.abs(blocks), axis=-1, keepdims=True)
+    scales[scales == 0] = 1.0
+    normalized = blocks / scales
+    indices = np.empty(normalized.size, dtype=np.uint8)
+    for i, x in enumerate(normalized.reshape(-1)):
+        indices[i] = int(np.argmin(np.abs(x - NF4_LEVELS)))
+    return dict(indices=indices, scales=scales.reshape(-1).astype(np.float32), shape=tuple(np.shape(w)),
+                numel=numel, padded=flat.size, block=block_size)
+
+
+def nf4_dequantize(q: dict) -> np.ndarray:
+    """qlora.py:77-98: level[index] * block scale, trimmed to the original element count."""
+    levels = NF4_LEVELS[q["indices"].astype(np.int64)].reshape(-1, q["block"])
+    flat = (levels * q["scales"][:, None]).reshape(-1)
+    return flat[:q["numel"]].reshape(q["shape"])

@@ -327,3 +327,39 @@ def test_config_c5_lora_grads_against_torch_and_zero_at_init():
                       b_zero=True, bf16=False)
     _, g0 = oc.c5_reference(t0, num_heads=2)
     assert np.all(g0[0] == 0) and np.all(g0[2] == 0) and np.abs(g0[1]).max() > 0
+
+
+def test_nf4_quantisation_pins():
+    """The NF4 restatement against what fixes it: nearest level by decision thresholds (the
+    midpoints between levels -- a different formulation of the same rule), exact round trips
+    for values that are level x scale, the all-zero block, padding, idempotence."""
+    rng = np.random.default_rng(21)
+    lv = O.NF4_LEVELS
+    assert lv.size == 16 and np.all(np.diff(lv) > 0) and lv[0] == -1 and lv[-1] == 1 and lv[7] == 0
+    w = rng.standard_normal((13, 10)).astype(np.float32)
+    q = O.nf4_quantize(w, block_size=8)
+    assert q["padded"] == 136 and q["numel"] == 130 and q["indices"].size == 136 and q["scales"].size == 17
+    flat = np.pad(w.reshape(-1), (0, 6)).reshape(-1, 8)
+    np.testing.assert_array_equal(q["scales"], np.abs(flat).max(1))
+    mid = ((lv[1:].astype(np.float64) + lv[:-1]) / 2)
+    normed = (flat / q["scales"][:, None]).reshape(-1)
+    by_threshold = np.searchsorted(mid, normed.astype(np.float64), side="left")
+    ties = np.isin(normed.astype(np.float64), mid)
+    np.testing.assert_array_equal(q["indices"][~ties], by_threshold[~ties])
+    # the block maximum is +-1 after scaling: first or last level
+    peak = np.abs(flat).argmax(1)
+    assert set(q["indices"].reshape(-1, 8)[np.arange(17), peak]) <= {0, 15}
+    # values that are exactly level x scale come back exactly; requantising is a fixed point
+    d = O.nf4_dequantize(q)
+    assert d.shape == w.shape and d.dtype == np.float32
+    q2 = O.nf4_quantize(d, block_size=8)
+    np.testing.assert_array_equal(q2["indices"][:130], q["indices"][:130])
+    np.testing.assert_array_equal(O.nf4_dequantize(q2), d)
+    # all-zero block: scale 1, level 7 (0.0)
+    z = O.nf4_quantize(np.zeros((2, 8), np.float32), block_size=8)
+    assert np.all(z["scales"] == 1) and np.all(z["indices"] == 7) and np.all(O.nf4_dequantize(z) == 0)
+    # lossy but bounded: the largest gap between neighbouring levels is 0.3038, so the error
+    # is at most half of that times the block scale
+    err = np.abs(d - w).reshape(-1)
+    bound = 0.5 * np.diff(lv).max() * np.repeat(q["scales"], 8)[:130]
+    assert np.all(err <= bound + 1e-6)
