@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 6
+#define NBK_ABI_VERSION 7
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -268,6 +268,10 @@ typedef struct nbk_pool_desc {
 int nbk_maxpool2d_fwd(const nbk_pool_desc* d, const void* x, void* y, void* stream);
 int nbk_maxpool2d_bwd(const nbk_pool_desc* d, const void* x, const void* y,
                       const void* dy, void* dx, void* stream);
+/* avg_pool2d forward/backward (nabla/ops/pooling.py:77-110, 140-173): the input is
+ * zero-padded first and every window sum is divided by kh * kw, padding included. */
+int nbk_avgpool2d_fwd(const nbk_pool_desc* d, const void* x, void* y, void* stream);
+int nbk_avgpool2d_bwd(const nbk_pool_desc* d, const void* dy, void* dx, void* stream);
 
 /* ===================================================================== */
 /*  Fused attention                                                       */

@@ -177,7 +177,7 @@ class BoundPlan:
                 fn = {"conv2d": L.nbk_conv2d_fwd, "conv2d_dgrad": L.nbk_conv2d_dgrad,
                       "conv2d_wgrad": L.nbk_conv2d_wgrad}[k]
                 self.calls.append((fn, [C.byref(d), holder, tuple(names[:n_ptr]), *extra], patches, d))
-            elif k in ("maxpool2d", "maxpool2d_bwd"):
+            elif k in ("maxpool2d", "maxpool2d_bwd", "avgpool2d", "avgpool2d_bwd"):
                 d = lib.PoolDesc()
                 xs, ys = a["x_shape"], a["y_shape"]
                 d.N, d.H, d.W, d.C = xs
@@ -193,7 +193,8 @@ class BoundPlan:
                     nm = f"p{i}"
                     names.append(nm)
                     ptr_field(holder, nm, r.buf, r.offset * r.dtype.size_in_bytes)
-                fn = L.nbk_maxpool2d_fwd if k == "maxpool2d" else L.nbk_maxpool2d_bwd
+                fn = {"maxpool2d": L.nbk_maxpool2d_fwd, "maxpool2d_bwd": L.nbk_maxpool2d_bwd,
+                      "avgpool2d": L.nbk_avgpool2d_fwd, "avgpool2d_bwd": L.nbk_avgpool2d_bwd}[k]
                 self.calls.append((fn, [C.byref(d), holder, tuple(names)], patches, d))
             elif k in ("attention", "attention_bwd"):
                 d = lib.AttnDesc()

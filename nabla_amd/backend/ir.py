@@ -343,6 +343,19 @@ def maxpool2d_bwd(x: Value, y: Value, dy: Value, kernel, stride, padding) -> Val
                          stride=tuple(stride), padding=tuple(padding))[0]
 
 
+def avgpool2d(x: Value, kernel, stride, padding) -> Value:
+    n, h, w, c = x.shape
+    ho = (h + padding[0] + padding[1] - kernel[0]) // stride[0] + 1
+    wo = (w + padding[2] + padding[3] - kernel[1]) // stride[1] + 1
+    return current().add("avgpool2d", [x], [((n, ho, wo, c), x.dtype)], kernel=tuple(kernel),
+                         stride=tuple(stride), padding=tuple(padding))[0]
+
+
+def avgpool2d_bwd(dy: Value, x_shape, kernel, stride, padding) -> Value:
+    return current().add("avgpool2d_bwd", [dy], [(tuple(x_shape), dy.dtype)], kernel=tuple(kernel),
+                         stride=tuple(stride), padding=tuple(padding), x_shape=tuple(x_shape))[0]
+
+
 # ---- indexing / movement ------------------------------------------------------------------
 def gather(table: Value, idx: Value, axis: int) -> Value:
     if axis < 0:

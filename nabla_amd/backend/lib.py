@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 MAX_RANK = 8
 
@@ -138,6 +138,8 @@ _SIGNATURES = {
     "nbk_maxpool2d_fwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_maxpool2d_bwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                            C.c_void_p], C.c_int),
+    "nbk_avgpool2d_fwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
+    "nbk_avgpool2d_bwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_attention_fwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_void_p],
                           C.c_int),
     "nbk_attention_bwd_workspace": ([C.POINTER(AttnDesc)], C.c_int64),

@@ -739,11 +739,14 @@ class Planner:
             self._emit(Step(k, [i.buf for i in ins], writes, attrs))
         elif k in ("attention", "attention_bwd"):
             self._lower_attention(n)
-        elif k in ("maxpool2d", "maxpool2d_bwd"):
+        elif k in ("maxpool2d", "maxpool2d_bwd", "avgpool2d", "avgpool2d_bwd"):
             ins = [self._contig(i) for i in n.inputs]
             dst = self._alloc_value(out)
-            xs = n.inputs[0].shape
-            ys = out.shape if k == "maxpool2d" else n.inputs[1].shape
+            if k == "avgpool2d_bwd":
+                xs, ys = out.shape, n.inputs[0].shape
+            else:
+                xs = n.inputs[0].shape
+                ys = out.shape if k in ("maxpool2d", "avgpool2d") else n.inputs[1].shape
             self._emit(Step(k, [i.buf for i in ins], [dst.buf], dict(
                 ins=ins, dst=dst, x_shape=xs, y_shape=ys, kernel=n.attrs["kernel"],
                 stride=n.attrs["stride"], padding=n.attrs["padding"])))

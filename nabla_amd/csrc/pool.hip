@@ -1,6 +1,7 @@
-// max_pool2d forward / backward over NHWC.  Lanes run along C (coalesced).
-// Windows are clipped at the padded border; the backward pass gives the full
+// max_pool2d and avg_pool2d forward / backward over NHWC.  Lanes run along C (coalesced).
+// max: windows are clipped at the padded border; the backward pass gives the full
 // cotangent of a window to every element equal to that window's maximum.
+// avg: the padding counts as zeros and every window is divided by kh * kw.
 #include "nbk_common.h"
 
 __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const void* __restrict__ x,
@@ -58,6 +59,56 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const void* __restrict
   }
 }
 
+__global__ __launch_bounds__(256) void avgpool_fwd_kernel(const void* __restrict__ x,
+                                                          void* __restrict__ y, nbk_pool_desc d) {
+  const int64_t total = d.N * d.Ho * d.Wo * d.C;
+  const float inv = 1.0f / (float)(d.kh * d.kw);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    const int64_t c = i % d.C;
+    int64_t t = i / d.C;
+    const int64_t wo = t % d.Wo; t /= d.Wo;
+    const int64_t ho = t % d.Ho;
+    const int64_t n = t / d.Ho;
+    const int64_t h0 = max((int64_t)0, ho * d.stride_h - d.pad_t);
+    const int64_t h1 = min(d.H, ho * d.stride_h - d.pad_t + d.kh);
+    const int64_t w0 = max((int64_t)0, wo * d.stride_w - d.pad_l);
+    const int64_t w1 = min(d.W, wo * d.stride_w - d.pad_l + d.kw);
+    float s = 0.f;
+    for (int64_t h = h0; h < h1; ++h)
+      for (int64_t w = w0; w < w1; ++w)
+        s += nbk_load_as_f32(x, ((n * d.H + h) * d.W + w) * d.C + c, d.dtype);
+    nbk_store_from_f32(y, i, d.dtype, s * inv);
+  }
+}
+
+__global__ __launch_bounds__(256) void avgpool_bwd_kernel(const void* __restrict__ dy,
+                                                          void* __restrict__ dx, nbk_pool_desc d) {
+  // gather form: each input element sums the cotangents of the windows that contain it
+  const int64_t total = d.N * d.H * d.W * d.C;
+  const float inv = 1.0f / (float)(d.kh * d.kw);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    const int64_t c = i % d.C;
+    int64_t t = i / d.C;
+    const int64_t w = t % d.W; t /= d.W;
+    const int64_t h = t % d.H;
+    const int64_t n = t / d.H;
+    const int64_t hp = h + d.pad_t, wp = w + d.pad_l;
+    int64_t ho_lo = hp - d.kh + 1;
+    ho_lo = ho_lo <= 0 ? 0 : (ho_lo + d.stride_h - 1) / d.stride_h;
+    const int64_t ho_hi = min(d.Ho - 1, hp / d.stride_h);
+    int64_t wo_lo = wp - d.kw + 1;
+    wo_lo = wo_lo <= 0 ? 0 : (wo_lo + d.stride_w - 1) / d.stride_w;
+    const int64_t wo_hi = min(d.Wo - 1, wp / d.stride_w);
+    float g = 0.f;
+    for (int64_t ho = ho_lo; ho <= ho_hi; ++ho)
+      for (int64_t wo = wo_lo; wo <= wo_hi; ++wo)
+        g += nbk_load_as_f32(dy, ((n * d.Ho + ho) * d.Wo + wo) * d.C + c, d.dtype);
+    nbk_store_from_f32(dx, i, d.dtype, g * inv);
+  }
+}
+
 static int pool_check(const nbk_pool_desc* d) {
   NBK_REQUIRE(d != nullptr, "pool: null descriptor");
   NBK_REQUIRE(d->N > 0 && d->H > 0 && d->W > 0 && d->C > 0 && d->Ho > 0 && d->Wo > 0,
@@ -91,4 +142,28 @@ extern "C" int nbk_maxpool2d_bwd(const nbk_pool_desc* d, const void* x, const vo
   hipLaunchKernelGGL(maxpool_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                      x, y, dy, dx, *d);
   return nbk_check_launch("maxpool_bwd_kernel");
+}
+
+extern "C" int nbk_avgpool2d_fwd(const nbk_pool_desc* d, const void* x, void* y, void* stream) {
+  int rc = pool_check(d);
+  if (rc) return rc;
+  NBK_REQUIRE(x && y, "pool: null pointer");
+  int64_t total = d->N * d->Ho * d->Wo * d->C;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 1 << 20) blocks = 1 << 20;
+  hipLaunchKernelGGL(avgpool_fwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     x, y, *d);
+  return nbk_check_launch("avgpool_fwd_kernel");
+}
+
+extern "C" int nbk_avgpool2d_bwd(const nbk_pool_desc* d, const void* dy, void* dx, void* stream) {
+  int rc = pool_check(d);
+  if (rc) return rc;
+  NBK_REQUIRE(dy && dx, "pool: null pointer");
+  int64_t total = d->N * d->H * d->W * d->C;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 1 << 20) blocks = 1 << 20;
+  hipLaunchKernelGGL(avgpool_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     dy, dx, *d);
+  return nbk_check_launch("avgpool_bwd_kernel");
 }

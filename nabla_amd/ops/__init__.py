@@ -7,10 +7,10 @@ from .control_flow import where
 from .convolution import conv2d
 from .creation import (arange, constant, full, full_like, ones, ones_like, tril, triu, zeros,
                        zeros_like)
-from .pooling import max_pool2d
+from .pooling import avg_pool2d, max_pool2d
 from .reduction import (argmax, argmin, mean, reduce_max, reduce_min, reduce_sum)
 from .unary import (abs, cast, erf, exp, gelu, log, logsoftmax, neg, relu, rsqrt, sigmoid,
-                    softmax, sqrt, tanh)
+                    silu, softmax, sqrt, tanh)
 from .utils import call_custom_kernel
 from .view import (broadcast_to, concatenate, flatten, gather, moveaxis, pad, permute, reshape,
                    slice_tensor, slice_update, squeeze, stack, swap_axes, take, transpose,

@@ -1,11 +1,12 @@
-"""max_pool2d over NHWC (nabla/ops/pooling.py:53-137, 177-211).
+"""max_pool2d and avg_pool2d over NHWC (nabla/ops/pooling.py:53-137, 140-211).
 
 The reference unrolls pooling in Python -- one slice + reduce_max per output
 pixel, then stack -- which makes a 32x32 feature map cost hundreds of graph
 nodes.  Here it is one op with one kernel each way.  Semantics kept: windows
 are clipped at the padded border (111-130), and the gradient follows the
 reduce_max tie rule (reduction.py:219-230): every element equal to its
-window's maximum receives that window's full cotangent.
+window's maximum receives that window's full cotangent.  avg_pool2d pads with
+zeros first and divides every window by kh * kw, padding included (77-110).
 """
 from __future__ import annotations
 
@@ -60,8 +61,68 @@ class MaxPool2DGradOp(Operation):
                                  kwargs["padding"])]
 
 
+class AvgPool2DOp(Operation):
+    @property
+    def name(self) -> str:
+        return "avg_pool2d"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x = args[0]
+        return ([MaxPool2DOp._out_shape(x.shape, kwargs["kernel_size"], kwargs["stride"],
+                                        kwargs["padding"])], [x.dtype], [x.device])
+
+    def kernel(self, args, kwargs):
+        return [ir.avgpool2d(args[0], kwargs["kernel_size"], kwargs["stride"], kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        return [_avg_pool2d_grad_op([cotangents[0]], dict(kwargs, x_shape=tuple(primals[0].shape)))[0]]
+
+
+class AvgPool2DGradOp(Operation):
+    """The transpose of avg_pool2d: cotangent [N,Ho,Wo,C] -> [N,H,W,C]."""
+
+    @property
+    def name(self) -> str:
+        return "avg_pool2d_grad"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        return [tuple(kwargs["x_shape"])], [args[0].dtype], [args[0].device]
+
+    def kernel(self, args, kwargs):
+        return [ir.avgpool2d_bwd(args[0], kwargs["x_shape"], kwargs["kernel_size"], kwargs["stride"],
+                                 kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        # linear: the transpose of the transpose is the pooling itself
+        kw = {k: kwargs[k] for k in ("kernel_size", "stride", "padding")}
+        return [_avg_pool2d_op([cotangents[0]], kw)[0]]
+
+
 _max_pool2d_op = MaxPool2DOp()
 _max_pool2d_grad_op = MaxPool2DGradOp()
+_avg_pool2d_op = AvgPool2DOp()
+_avg_pool2d_grad_op = AvgPool2DGradOp()
+
+
+def _pool_args(x, kernel_size, stride, padding, dilation, what: str):
+    x = ensure_tensor(x)
+    if len(x.shape) != 4:
+        raise ValueError(f"{what} expects an NHWC rank-4 tensor, got shape {tuple(x.shape)}")
+    kernel = _normalize_2tuple(kernel_size, "kernel_size")
+    stride_n = _normalize_2tuple(stride if stride is not None else kernel, "stride")
+    padding_n = _normalize_4padding(padding)
+    dil = _normalize_2tuple(dilation, "dilation")
+    _require_all_positive_2tuple(kernel, "kernel_size")
+    _require_all_positive_2tuple(stride_n, "stride")
+    _require_all_nonnegative(padding_n, "padding")
+    if dil != (1, 1):
+        raise ValueError("pool2d currently supports only dilation=(1, 1)")
+    return x, {"kernel_size": kernel, "stride": stride_n, "padding": padding_n}
+
+
+def avg_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Tensor:
+    x, kw = _pool_args(x, kernel_size, stride, padding, dilation, "avg_pool2d")
+    return _avg_pool2d_op([x], kw)[0]
 
 
 def max_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Tensor:

@@ -155,6 +155,24 @@ class SigmoidOp(UnaryOperation):
         return mul(output, sub(1.0, output))
 
 
+class SiluOp(UnaryOperation):
+    """``x * sigmoid(x)`` (unary.py:504-520); emitted as those two primitive ops, which the
+    lowering fuses with their neighbours."""
+
+    @property
+    def name(self) -> str:
+        return "silu"
+
+    def kernel(self, args, kwargs):
+        return [ir.ew("mul", args[0], ir.ew("sigmoid", args[0]))]
+
+    def _derivative(self, primal, output):
+        # sigmoid(x) + silu(x) * (1 - sigmoid(x))
+        from .binary import add, mul, sub
+        s = sigmoid(primal)
+        return add(s, mul(output, sub(1.0, s)))
+
+
 class GeluOp(UnaryOperation):
     """Exact GELU ``x * Phi(x)``; ``approximate="tanh"`` selects the tanh form."""
 
@@ -287,6 +305,7 @@ class CastOp(UnaryOperation):
 _relu_op, _exp_op, _neg_op, _abs_op = ReluOp(), ExpOp(), NegOp(), AbsOp()
 _log_op, _sqrt_op, _rsqrt_op, _erf_op = LogOp(), SqrtOp(), RsqrtOp(), ErfOp()
 _tanh_op, _sigmoid_op, _gelu_op, _cast_op = TanhOp(), SigmoidOp(), GeluOp(), CastOp()
+_silu_op = SiluOp()
 _softmax_native, _logsoftmax_native = _SoftmaxNativeOp(), _LogSoftmaxNativeOp()
 
 
@@ -328,6 +347,10 @@ def tanh(x) -> Tensor:
 
 def sigmoid(x) -> Tensor:
     return _sigmoid_op([ensure_tensor(x)], {})[0]
+
+
+def silu(x) -> Tensor:
+    return _silu_op([ensure_tensor(x)], {})[0]
 
 
 def gelu(x, approximate: str = "none") -> Tensor:

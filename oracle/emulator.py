@@ -283,6 +283,29 @@ def _attention(kind, a, mem):
         dst.copy_(g.float().to(dst.dtype))
 
 
+def _avgpool(kind, a, mem):
+    """Zero padding, window sums divided by kh * kw; the backward is its transpose."""
+    kh, kw = a["kernel"]
+    sh, sw = a["stride"]
+    pt, _, pl, _ = a["padding"]
+    N, H, W, C = a["x_shape"]
+    _, Ho, Wo, _ = a["y_shape"]
+    src = _view(mem, a["ins"][0]).double().numpy()
+    dst = _view(mem, a["dst"])
+    res = np.zeros((N, Ho, Wo, C) if kind == "avgpool2d" else (N, H, W, C))
+    for i in range(Ho):
+        for j in range(Wo):
+            h0, h1 = max(0, i * sh - pt), min(H, i * sh - pt + kh)
+            w0, w1 = max(0, j * sw - pl), min(W, j * sw - pl + kw)
+            if h0 >= h1 or w0 >= w1:
+                continue
+            if kind == "avgpool2d":
+                res[:, i, j, :] = src[:, h0:h1, w0:w1, :].sum(axis=(1, 2)) / (kh * kw)
+            else:
+                res[:, h0:h1, w0:w1, :] += src[:, i:i + 1, j:j + 1, :] / (kh * kw)
+    dst.copy_(torch.from_numpy(res).float().to(dst.dtype))
+
+
 class EmulatedPlan:
     def __init__(self, plan: Plan):
         self.plan = plan
@@ -326,6 +349,8 @@ class EmulatedPlan:
                 _conv(k, a, mem)
             elif k in ("maxpool2d", "maxpool2d_bwd"):
                 _pool(k, a, mem)
+            elif k in ("avgpool2d", "avgpool2d_bwd"):
+                _avgpool(k, a, mem)
             elif k in ("attention", "attention_bwd"):
                 _attention(k, a, mem)
             elif k == "gather":

@@ -453,6 +453,38 @@ def max_pool2d(x, kernel, stride=None, padding=(0, 0, 0, 0)) -> V:
 
 
 # ------------------------------------------------------------ nn composites
+def avg_pool2d(x, kernel, stride=None, padding=(0, 0, 0, 0)) -> V:
+    """pooling.py:77-110, 140-173: the input is zero-padded first, then every window is summed
+    and divided by kh * kw (the padding counts); the VJP of slice + sum + pad spreads
+    g / (kh * kw) back over the window and drops what falls on the padding."""
+    x = _v(x)
+    kh, kw = kernel
+    sh, sw = stride if stride is not None else kernel
+    pt, pb, pl, pr = padding
+    xp = np.pad(x.a, ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+    n, h, w, c = xp.shape
+    ho, wo = (h - kh) // sh + 1, (w - kw) // sw + 1
+    y = np.empty((n, ho, wo, c), dtype=x.a.dtype)
+    for i in range(ho):
+        for j in range(wo):
+            y[:, i, j, :] = xp[:, i * sh:i * sh + kh, j * sw:j * sw + kw, :].sum(axis=(1, 2)) / (kh * kw)
+
+    def vjp(g):
+        gp = np.zeros(xp.shape, dtype=g.dtype)
+        for i in range(ho):
+            for j in range(wo):
+                gp[:, i * sh:i * sh + kh, j * sw:j * sw + kw, :] += g[:, i:i + 1, j:j + 1, :] / (kh * kw)
+        return (gp[:, pt:h - pb, pl:w - pr, :],)
+
+    return V(y, (x,), vjp)
+
+
+def silu(x) -> V:  # unary.py:504-520: x * sigmoid(x)
+    x = _v(x)
+    s = 1.0 / (1.0 + np.exp(-x.a))
+    return V(x.a * s, (x,), lambda g: (g * (s + x.a * s * (1.0 - s)),))
+
+
 def linear(x, w, b=None) -> V:  # nn/functional/layers.py:30-35
     out = matmul(x, w)
     return out + b if b is not None else out

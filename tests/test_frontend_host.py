@@ -481,3 +481,39 @@ def test_weight_gradient_over_a_batch_is_one_product(emulator):
     st = last_plan().stats
     assert "reduce_mid" not in st and st["gemm"] == 1, st
     np.testing.assert_allclose(gw.numpy(), np.einsum("bsd,bsn->dn", x, g), rtol=1e-5, atol=1e-5)
+
+
+# ---- avg_pool2d, silu ------------------------------------------------------------------------------
+@pytest.mark.parametrize("kernel,stride,padding", [((2, 2), None, 0), ((3, 3), (2, 1), 1), ((3, 2), (1, 2), (1, 0, 2, 1))])
+def test_avg_pool2d_value_grad_and_second_order(emulator, kernel, stride, padding):
+    x = RNG.standard_normal((2, 9, 8, 3)).astype(np.float32)
+    pad4 = (padding,) * 4 if isinstance(padding, int) else padding
+    y = nb.avg_pool2d(T(x), kernel_size=kernel, stride=stride, padding=padding)
+    want = O.avg_pool2d(O.V(x.astype(np.float64)), kernel, stride, pad4)
+    np.testing.assert_allclose(y.numpy(), want.a, rtol=1e-6, atol=1e-6)
+    assert "avgpool2d" in last_plan().stats
+    g = RNG.standard_normal(want.a.shape).astype(np.float32)
+    vx = O.V(x.astype(np.float64))
+    (wg,) = O.grad_of(O.reduce_sum(O.avg_pool2d(vx, kernel, stride, pad4) * O.V(g.astype(np.float64))), [vx])
+    f = lambda t: nb.reduce_sum(nb.avg_pool2d(t, kernel_size=kernel, stride=stride, padding=padding) * T(g))
+    np.testing.assert_allclose(nb.grad(f)(T(x)).numpy(), wg, rtol=1e-5, atol=1e-6)
+    # the gradient does not depend on x (the op is linear): differentiating it again gives zeros
+    gg = nb.grad(lambda t: nb.reduce_sum(nb.grad(f)(t) * nb.grad(f)(t)))(T(x))
+    np.testing.assert_array_equal(gg.numpy(), np.zeros_like(x))
+
+
+def test_avg_pool2d_validation(emulator):
+    with pytest.raises(ValueError, match="rank-4"):
+        nb.avg_pool2d(T(np.zeros((4, 4), np.float32)), kernel_size=2)
+    with pytest.raises(ValueError, match="dilation"):
+        nb.avg_pool2d(T(np.zeros((1, 4, 4, 1), np.float32)), kernel_size=2, dilation=2)
+    with pytest.raises(ValueError, match="Non-positive"):
+        nb.avg_pool2d(T(np.zeros((1, 2, 2, 1), np.float32)), kernel_size=3)
+
+
+def test_silu_value_and_grad(emulator):
+    x = RNG.standard_normal((5, 33)).astype(np.float32)
+    vx = O.V(x.astype(np.float64))
+    np.testing.assert_allclose(nb.silu(T(x)).numpy(), O.silu(vx).a, rtol=1e-6, atol=1e-6)
+    (wg,) = O.grad_of(O.reduce_sum(O.silu(vx)), [vx])
+    np.testing.assert_allclose(nb.grad(lambda t: nb.reduce_sum(nb.silu(t)))(T(x)).numpy(), wg, rtol=1e-5, atol=1e-6)

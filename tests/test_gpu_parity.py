@@ -422,3 +422,34 @@ def test_graph_replay_matches_eager_every_time(hip):
     assert abs(loss.item() - wl2) <= F32_TOL * abs(wl2) + 1e-9
     for g, w in zip(grads, wg2):
         assert relerr(g.numpy(), w) < F32_TOL
+
+
+# ---- avg_pool2d, silu -------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("kernel,stride,padding", [((2, 2), None, 0), ((3, 3), (2, 1), 1),
+                                                   ((3, 2), (1, 2), (1, 0, 2, 1))])
+def test_avg_pool2d_and_silu_on_device(hip, dtype, kernel, stride, padding):
+    from oracle import ops as O
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((4, 17, 12, 24)).astype(np.float32)
+    dt = nb.DType.float32 if dtype == "f32" else nb.DType.bfloat16
+    if dtype == "bf16":
+        import torch
+        x = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    tol = 2e-5 if dtype == "f32" else 2e-2
+    pad4 = (padding,) * 4 if isinstance(padding, int) else padding
+    X = nb.Tensor.constant(x, dtype=dt)
+    vx = O.V(x.astype(np.float64))
+    want = O.avg_pool2d(O.silu(vx), kernel, stride, pad4)
+    g = rng.standard_normal(want.a.shape).astype(np.float32)
+    (wg,) = O.grad_of(O.reduce_sum(want * O.V(g.astype(np.float64))), [vx])
+
+    def f(t):
+        y = nb.avg_pool2d(nb.silu(t), kernel_size=kernel, stride=stride, padding=padding)
+        return nb.reduce_sum(nb.cast(y, nb.DType.float32) * nb.Tensor.constant(g))
+
+    y = nb.avg_pool2d(nb.silu(X), kernel_size=kernel, stride=stride, padding=padding)
+    got = nb.cast(y, nb.DType.float32).numpy()
+    assert np.abs(got - want.a).max() <= tol * max(np.abs(want.a).max(), 1.0)
+    gx = nb.cast(nb.grad(f)(X), nb.DType.float32).numpy()
+    assert np.abs(gx - wg).max() <= tol * max(np.abs(wg).max(), 1.0)

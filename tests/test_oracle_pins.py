@@ -363,3 +363,30 @@ def test_nf4_quantisation_pins():
     err = np.abs(d - w).reshape(-1)
     bound = 0.5 * np.diff(lv).max() * np.repeat(q["scales"], 8)[:130]
     assert np.all(err <= bound + 1e-6)
+
+
+def test_avg_pool_and_silu_against_torch():
+    """avg_pool2d is torch's with count_include_pad=True (symmetric padding), checked with
+    overlapping windows, strides and padding; silu and both gradients against autograd."""
+    import torch.nn.functional as F
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((2, 9, 8, 3))
+    for kernel, stride, pad in (((2, 2), (2, 2), (0, 0)), ((3, 3), (2, 1), (1, 1)), ((3, 2), (1, 2), (1, 0))):
+        xt = torch.tensor(x, requires_grad=True)
+        yt = F.avg_pool2d(xt.permute(0, 3, 1, 2), kernel, stride, pad, count_include_pad=True).permute(0, 2, 3, 1)
+        g = rng.standard_normal(tuple(yt.shape))
+        yt.backward(torch.tensor(g))
+        vx = O.V(x)
+        y = O.avg_pool2d(vx, kernel, stride, (pad[0], pad[0], pad[1], pad[1]))
+        np.testing.assert_allclose(y.a, yt.detach().numpy(), rtol=1e-12, atol=1e-12)
+        (gx,) = O.grad_of(O.reduce_sum(y * O.V(g)), [vx])
+        np.testing.assert_allclose(gx, xt.grad.numpy(), rtol=1e-12, atol=1e-12)
+    # asymmetric padding (top 2, bottom 0): a window that lies wholly in the padding is 0
+    y = O.avg_pool2d(O.V(np.ones((1, 2, 2, 1))), (2, 2), (2, 2), (2, 0, 0, 0))
+    np.testing.assert_array_equal(y.a.reshape(-1), [0.0, 1.0])
+    xt = torch.tensor(x, requires_grad=True)
+    F.silu(xt).backward(torch.ones_like(xt))
+    vx = O.V(x)
+    s = O.silu(vx)
+    np.testing.assert_allclose(s.a, F.silu(torch.tensor(x)).numpy(), rtol=1e-12)
+    np.testing.assert_allclose(O.grad_of(O.reduce_sum(s), [vx])[0], xt.grad.numpy(), rtol=1e-12)
