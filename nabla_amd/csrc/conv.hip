@@ -98,26 +98,28 @@ __device__ __forceinline__ void conv_ld8(const float* p, bool ok, float* r) {
   r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
 }
 
-template <int MODE, bool FAST>
+// NJ: 32-column MFMA tiles per wave along the output's channel axis: 2 for a 128 x 128
+// workgroup tile, 1 for 128 x 64 (channel counts up to 64 would waste half of the wider tile).
+template <int MODE, bool FAST, int NJ>
 __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
-  constexpr int BK = 16, LD = 128 + 4;
+  constexpr int BK = 16, LD = 128 + 4, BN = 64 * NJ;
   __shared__ float As[2][BK][LD];
   __shared__ float Bs[2][BK][LD];
   const nbk_conv_desc& d = g.d;
   const int tm_i = blockIdx.x % g.tiles_m, tn_i = blockIdx.x / g.tiles_m;
-  const int64_t m0 = (int64_t)tm_i * 128, n0 = (int64_t)tn_i * 128;
+  const int64_t m0 = (int64_t)tm_i * 128, n0 = (int64_t)tn_i * BN;
   const int64_t k_begin = (int64_t)blockIdx.z * g.k_per_split;
   const int64_t k_end = min(g.K, k_begin + g.k_per_split);
   float* out = g.out + (g.splits > 1 ? (int64_t)blockIdx.z * g.M * g.Ng : 0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 32 * NJ;
   const int li = lane & 31, kg = lane >> 5;
 
-  f32x16 acc[2][2];
+  f32x16 acc[2][NJ];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = (f32x16)(0.f);
+    for (int j = 0; j < NJ; ++j) acc[i][j] = (f32x16)(0.f);
 
   // ---- per-lane constants of the A gather ----
   // forward / dgrad: the lane's pixel; wgrad: the lane's first filter row and, as running
@@ -249,15 +251,15 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
 #pragma unroll
     for (int ks = 0; ks < BK / 2; ++ks) {
       const int k = ks * 2 + kg;
-      float fa[2], fb[2];
+      float fa[2], fb[NJ];
 #pragma unroll
       for (int i = 0; i < 2; ++i) fa[i] = As[cur][k][wm + i * 32 + li];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = Bs[cur][k][wn + j * 32 + li];
+      for (int j = 0; j < NJ; ++j) fb[j] = Bs[cur][k][wn + j * 32 + li];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
     if (more) {
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const int64_t col = n0 + wn + j * 32 + li;
       const bool col_ok = col < g.Ng;
       const float bv = (g.bias && col_ok) ? g.bias[col] : 0.f;
@@ -322,13 +324,20 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 template <int MODE>
 static int conv_launch(ConvArgs& a, bool fast, hipStream_t st) {
+  // the narrow workgroup tile when the last 128-wide column tile would be at most half full,
+  // or when the wide tiling gives fewer workgroups than the GPU has CUs
+  const int64_t wide = ((a.M + 127) / 128) * ((a.Ng + 127) / 128) * a.splits;
+  const bool narrow = (a.Ng - 1) % 128 < 64 || wide < nbk_num_cus();
+  const int bn = narrow ? 64 : 128;
   a.tiles_m = (int)((a.M + 127) / 128);
-  a.tiles_n = (int)((a.Ng + 127) / 128);
+  a.tiles_n = (int)((a.Ng + bn - 1) / bn);
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   NBK_REQUIRE(blocks <= 0x7fffffffLL, "conv2d: launch too large");
   const dim3 grid((unsigned)blocks, 1, (unsigned)a.splits);
-  if (fast) hipLaunchKernelGGL((conv_kernel<MODE, true>), grid, dim3(256), 0, st, a);
-  else hipLaunchKernelGGL((conv_kernel<MODE, false>), grid, dim3(256), 0, st, a);
+  if (fast && narrow) hipLaunchKernelGGL((conv_kernel<MODE, true, 1>), grid, dim3(256), 0, st, a);
+  else if (fast) hipLaunchKernelGGL((conv_kernel<MODE, true, 2>), grid, dim3(256), 0, st, a);
+  else if (narrow) hipLaunchKernelGGL((conv_kernel<MODE, false, 1>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((conv_kernel<MODE, false, 2>), grid, dim3(256), 0, st, a);
   return nbk_check_launch("conv_kernel");
 }
 
