@@ -581,9 +581,16 @@ class Planner:
             return ViewRef(b.id, 0, src.shape, contiguous_strides(src.shape), src.dtype)
         if src.is_contiguous():
             return src
+        # one copy per distinct view: a broadcast cotangent that feeds two products and a
+        # reduction is materialised once (values are written once, so the copy stays valid)
+        key = (src.buf, src.offset, tuple(src.shape), tuple(src.strides), src.dtype)
+        hit = self._materialized.get(key)
+        if hit is not None:
+            return hit
         b = self._new_buf(src.shape, src.dtype)
         dst = ViewRef(b.id, 0, src.shape, contiguous_strides(src.shape), src.dtype)
         self._emit(Step("copy", [src.buf], [b.id], dict(src=src, dst=dst)))
+        self._materialized[key] = dst
         return dst
 
     def _contig(self, v: ir.Value) -> ViewRef:
@@ -597,6 +604,7 @@ class Planner:
             self.loc[v.id] = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
         self.skip_nodes: set[int] = set()  # reductions folded into an earlier one
         self.n_split = 0                   # fusion groups cut in two at lowering time
+        self._materialized: dict = {}
         self.users: dict[int, list[ir.Node]] = {}
         for n in nodes:
             for i in n.inputs:
@@ -1104,14 +1112,17 @@ class Planner:
         """One row program for the group; a group that exceeds a limit of the row-program
         format (operands, registers, instructions) is cut in two in program order, the values
         that cross the cut go through memory, and each half is lowered on its own."""
-        snap = (len(self.bufs), dict(self.loc), dict(self._out_pending), dict(self._out_done))
+        snap = (len(self.bufs), dict(self.loc), dict(self._out_pending), dict(self._out_done),
+                len(self.steps), dict(self._materialized))
         try:
             step = _RowCodegen(self, g).generate()
         except FusionLimit:
             if len(g.nodes) < 2:
                 raise
             del self.bufs[snap[0]:]
+            del self.steps[snap[4]:]
             self.loc, self._out_pending, self._out_done = snap[1], snap[2], snap[3]
+            self._materialized = snap[5]
             self.n_split += 1
             nodes = sorted(g.nodes, key=lambda n: n.pos)
             cut = len(nodes) // 2

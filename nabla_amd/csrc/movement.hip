@@ -166,9 +166,20 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict_
   float acc = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
   if (col < inner) {
     const int64_t base = o * red * inner + col;
-    // four accumulators keep four loads in flight
+    // four accumulators; sixteen loads in flight while the axis is long enough (a short axis
+    // over few columns is pure latency: every round trip saved shows), then four
     float a0 = acc, a1 = acc, a2 = acc, a3 = acc;
     int64_t r = w;
+    for (; r + 60 < red; r += 64) {
+      float v[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) v[q] = nbk_load_as_f32(in, base + (r + 4 * q) * inner, dti);
+#pragma unroll
+      for (int q = 0; q < 16; q += 4) {
+        a0 = red_comb(a0, v[q], kind); a1 = red_comb(a1, v[q + 1], kind);
+        a2 = red_comb(a2, v[q + 2], kind); a3 = red_comb(a3, v[q + 3], kind);
+      }
+    }
     for (; r + 12 < red; r += 16) {
       float v0 = nbk_load_as_f32(in, base + r * inner, dti);
       float v1 = nbk_load_as_f32(in, base + (r + 4) * inner, dti);
@@ -190,8 +201,8 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict_
 }
 
 // Vector form: a lane owns VEC consecutive columns (16 bytes of input per row), a
-// workgroup 64 * VEC columns; its four waves take every fourth row and keep eight
-// row loads in flight each.  T is the input element (uint16_t = bf16, float).
+// workgroup 64 * VEC columns; its four waves take every fourth row and keep up to
+// sixteen row loads in flight each.  T is the input element (uint16_t = bf16, float).
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
                                                              void* __restrict__ out, int dto,
@@ -206,8 +217,7 @@ __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict
   for (int e = 0; e < VEC; ++e) acc[e] = ident;
   if (col < inner) {
     const T* base = in + o * red * inner + col;
-    auto load = [&](int64_t r, float* v) {
-      const uint4 u = *(const uint4*)(base + r * inner);
+    auto unpack = [&](const uint4 u, float* v) {
       if (sizeof(T) == 2) {
         v[0] = __uint_as_float(u.x << 16); v[1] = __uint_as_float(u.x & 0xffff0000u);
         v[2] = __uint_as_float(u.y << 16); v[3] = __uint_as_float(u.y & 0xffff0000u);
@@ -218,7 +228,20 @@ __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict
         v[2] = __uint_as_float(u.z); v[3] = __uint_as_float(u.w);
       }
     };
+    auto load = [&](int64_t r, float* v) { unpack(*(const uint4*)(base + r * inner), v); };
     int64_t r = w;
+    for (; r + 60 < red; r += 64) {  // sixteen rows in flight, kept packed until they are added
+      uint4 raw[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) raw[q] = *(const uint4*)(base + (r + 4 * q) * inner);
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        float v[VEC];
+        unpack(raw[q], v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = red_comb(acc[e], v[e], kind);
+      }
+    }
     for (; r + 28 < red; r += 32) {
       float v[8][VEC];
 #pragma unroll
