@@ -45,6 +45,9 @@ class MaxPool2DOp(Operation):
     def vjp_rule(self, primals, cotangents, outputs, kwargs):
         return [_max_pool2d_grad_op([primals[0], outputs[0], cotangents[0]], dict(kwargs))[0]]
 
+    def jvp_rule(self, primals, tangents, outputs, kwargs):
+        return [_window_sum_at_maxima(primals[0], outputs[0], tangents[0], kwargs)]
+
 
 class MaxPool2DGradOp(Operation):
     @property
@@ -59,6 +62,35 @@ class MaxPool2DGradOp(Operation):
         x, y, dy = args
         return [ir.maxpool2d_bwd(x, y, dy, kwargs["kernel_size"], kwargs["stride"],
                                  kwargs["padding"])]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        # linear in dy, piecewise constant in x and y
+        x, y, _ = primals
+        return [None, None, _window_sum_at_maxima(x, y, cotangents[0], kwargs)]
+
+
+def _window_sum_at_maxima(x: Tensor, y: Tensor, t: Tensor, kwargs) -> Tensor:
+    """sum over each window of ``t`` where ``x`` equals the window maximum ``y``: the transpose
+    of the max-pool gradient under its tie rule (and so the pool's JVP).  Written with
+    reshapes for windows that tile the image (stride == kernel, no padding, extents divisible);
+    other windows overlap or are clipped and have no such form here."""
+    from .comparison import equal
+    from .control_flow import where
+    from .creation import zeros_like
+    from .reduction import reduce_sum
+    from .view import broadcast_to, reshape
+    kh, kw = kwargs["kernel_size"]
+    n, h, w, c = (int(d) for d in x.shape)
+    if tuple(kwargs["stride"]) != (kh, kw) or any(kwargs["padding"]) or h % kh or w % kw:
+        raise NotImplementedError(
+            "forward mode / second order through max_pool2d needs windows that tile the image "
+            "(stride == kernel_size, no padding, extents divisible by the kernel)")
+    ho, wo = h // kh, w // kw
+    six = (n, ho, kh, wo, kw, c)
+    xr, tr = reshape(x, six), reshape(t, six)
+    yr = broadcast_to(reshape(y, (n, ho, 1, wo, 1, c)), six)
+    picked = where(equal(xr, yr), tr, zeros_like(tr))
+    return reshape(reduce_sum(picked, axis=[2, 4], keepdims=True), (n, ho, wo, c))
 
 
 class AvgPool2DOp(Operation):

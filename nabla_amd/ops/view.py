@@ -390,6 +390,10 @@ class GatherOp(AxisOp):
         x, idx = primals
         return [_scatter_op([zeros_like(x), idx, cotangents[0]], dict(kwargs))[0], None]
 
+    def jvp_rule(self, primals, tangents, outputs, kwargs):
+        # linear in the table: the same rows of the tangent (indexing.py:183-190)
+        return [_gather_op([tangents[0], primals[1]], dict(kwargs))[0]]
+
 
 class ScatterOp(AxisOp):
     """``x`` with the rows selected by ``indices`` along ``axis`` replaced by

@@ -453,3 +453,37 @@ def test_avg_pool2d_and_silu_on_device(hip, dtype, kernel, stride, padding):
     assert np.abs(got - want.a).max() <= tol * max(np.abs(want.a).max(), 1.0)
     gx = nb.cast(nb.grad(f)(X), nb.DType.float32).numpy()
     assert np.abs(gx - wg).max() <= tol * max(np.abs(wg).max(), 1.0)
+
+
+# ---- forward mode -----------------------------------------------------------------------------------
+def test_jvp_on_device_against_oracle_central_differences(hip):
+    """jvp of a small CNN + MLP head on the device: the tangent equals the float64 oracle's
+    central difference along the same direction, and <J v, u> = <v, J^T u> against vjp."""
+    from oracle import ops as O
+    rng = np.random.default_rng(43)
+    shapes = [(2, 8, 8, 3), (3, 3, 3, 8), (8,), (8, 5)]
+    xs = [rng.standard_normal(s) for s in shapes]
+    vs = [rng.standard_normal(s) for s in shapes]
+
+    def fn(x, w, b, wl):
+        h = nb.max_pool2d(nb.relu(nb.conv2d(x, w, padding=1, bias=b)), kernel_size=2)
+        return nb.softmax(nb.mean(h, axis=(1, 2)) @ wl, axis=-1)
+
+    def ofn(x, w, b, wl):
+        h = O.max_pool2d(O.relu(O.conv2d(x, w, b, (1, 1), (1, 1, 1, 1))), (2, 2))
+        return O.softmax(O.matmul(O.mean(h, axis=(1, 2)), wl), axis=-1)
+
+    T = lambda a: nb.Tensor.constant(a.astype(np.float32))
+    out, tan = nb.jvp(fn, tuple(T(x) for x in xs), tuple(T(v) for v in vs))
+    eps = 1e-6
+    p = ofn(*[O.V(x + eps * v) for x, v in zip(xs, vs)]).a
+    m = ofn(*[O.V(x - eps * v) for x, v in zip(xs, vs)]).a
+    want = (p - m) / (2 * eps)
+    np.testing.assert_allclose(out.numpy(), ofn(*[O.V(x) for x in xs]).a, rtol=2e-5, atol=2e-6)
+    assert np.abs(tan.numpy() - want).max() <= 2e-4 * max(np.abs(want).max(), 1e-3)
+    u = rng.standard_normal(out.shape)
+    _, pull = nb.vjp(fn, *[T(x) for x in xs])
+    gs = pull(T(u))
+    lhs = float((tan.numpy().astype(np.float64) * u).sum())
+    rhs = sum(float((g.numpy().astype(np.float64) * v).sum()) for g, v in zip(gs, vs))
+    assert abs(lhs - rhs) <= 2e-4 * max(abs(lhs), abs(rhs), 1e-3)
