@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 7
+#define NBK_ABI_VERSION 8
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -320,6 +320,14 @@ int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
 int nbk_gather(const void* table, const void* idx, void* out, int32_t dtype,
                int32_t idx_dtype, int64_t outer, int64_t axis_len, int64_t n_idx,
                int64_t inner, int32_t* status, void* stream);
+/* out[o, idx[j], i] = upd[o, j, i] on top of what `out` already holds (the caller copies x
+ * there first); replaces ops.scatter at nabla/ops/view/indexing.py:185-447, which the VJP of
+ * gather uses (173-182).  A row named more than once takes the update at the largest j
+ * (numpy's assignment rule; the reference leaves that order to its backend).  `winner` is
+ * axis_len int32 of caller scratch.  Index wrapping and range errors as in nbk_gather. */
+int nbk_scatter(const void* idx, const void* upd, void* out, int32_t dtype, int32_t idx_dtype,
+                int64_t outer, int64_t axis_len, int64_t n_idx, int64_t inner,
+                int32_t* winner, int32_t* status, void* stream);
 /* out[r] = index of the first maximum of in[r, 0..C) as int64; replaces
  * ops.argmax at nabla/ops/reduction.py:745-765. */
 int nbk_argmax_rows(const void* in, int64_t* out, int32_t dtype, int64_t rows,

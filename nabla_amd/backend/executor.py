@@ -44,7 +44,7 @@ class BoundPlan:
                     self.base[b.id] = a0 + b.offset
         self.dynamic = [b.id for b in plan.bufs if b.role in ("input", "output")]
         self.calls: list[tuple] = []  # (fn, args tuple, patch list)
-        self.has_gather = any(st.kind == "gather" for st in plan.steps)
+        self.has_gather = any(st.kind in ("gather", "scatter") for st in plan.steps)
         self._graphs: dict = {}  # pointer tuple -> recorded launch sequence (at most four)
         self._seen: set = set()  # pointer tuples that have run once already
         self._graph_off = any(st.kind == "custom" for st in plan.steps)  # user kernels may not be capturable
@@ -237,6 +237,18 @@ class BoundPlan:
                 self.calls.append((L.nbk_gather,
                                    [holder, ("p0", "p1", "p2"), t.dtype.abi, ix.dtype.abi, a["outer"],
                                     a["axis_len"], a["n_idx"], a["inner"],
+                                    C.c_void_p(self.ex.status_flag.data_ptr())], patches, None))
+            elif k == "scatter":
+                ix, up, dst, wn = a["idx"], a["upd"], a["dst"], a["winner"]
+                holder = _Ptrs(4)
+                ptr_field(holder, "p0", ix.buf, ix.offset * ix.dtype.size_in_bytes)
+                ptr_field(holder, "p1", up.buf, up.offset * up.dtype.size_in_bytes)
+                ptr_field(holder, "p2", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                ptr_field(holder, "p3", wn.buf, wn.offset * 4)
+                self.calls.append((L.nbk_scatter,
+                                   [_LATE, _Late(holder, "p0"), _Late(holder, "p1"), _Late(holder, "p2"),
+                                    dst.dtype.abi, ix.dtype.abi, a["outer"], a["axis_len"], a["n_idx"],
+                                    a["inner"], _Late(holder, "p3"),
                                     C.c_void_p(self.ex.status_flag.data_ptr())], patches, None))
             elif k == "argreduce":
                 src, dst = a["src"], a["dst"]

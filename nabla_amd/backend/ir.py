@@ -364,6 +364,16 @@ def gather(table: Value, idx: Value, axis: int) -> Value:
     return current().add("gather", [table, idx], [(shape, table.dtype)], axis=axis)[0]
 
 
+def scatter(x: Value, idx: Value, updates: Value, axis: int) -> Value:
+    """Copy of ``x`` whose rows ``idx`` along ``axis`` are replaced by ``updates``."""
+    if axis < 0:
+        axis += x.rank
+    want = x.shape[:axis] + idx.shape + x.shape[axis + 1:]
+    if tuple(updates.shape) != tuple(want):
+        raise ValueError(f"scatter: updates of shape {updates.shape}, expected {want}")
+    return current().add("scatter", [x, idx, updates], [(x.shape, x.dtype)], axis=axis)[0]
+
+
 def pad(x: Value, lo, hi, value: float = 0.0) -> Value:
     shape = tuple(d + a + b for d, a, b in zip(x.shape, lo, hi))
     if shape == x.shape:

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 MAX_RANK = 8
 
@@ -147,6 +147,8 @@ _SIGNATURES = {
                           [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_int64, C.c_void_p], C.c_int),
     "nbk_gather": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64,
                     C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p], C.c_int),
+    "nbk_scatter": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
+                     C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_argmax_rows": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32,
                          C.c_void_p], C.c_int),
     "nbk_custom": ([C.c_char_p, C.c_char_p, C.POINTER(TensorDesc), C.c_int,

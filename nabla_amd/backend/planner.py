@@ -723,6 +723,23 @@ class Planner:
                 table=t, idx=ix, dst=dst, outer=_numel(table.shape[:axis]),
                 axis_len=table.shape[axis], n_idx=idx.numel(),
                 inner=_numel(table.shape[axis + 1:]))))
+        elif k == "scatter":
+            x, idx, upd = n.inputs
+            axis = n.attrs["axis"]
+            src = self._resolve(x)
+            ix = self._contig(idx)
+            up = self._contig(upd)
+            dst = self._alloc_value(out)
+            if isinstance(src, Const):
+                self._emit(Step("fill", [], [dst.buf], dict(buf=dst.buf, numel=out.numel(),
+                                                             value=src.value, dtype=out.dtype)))
+            else:
+                self._copy_into(src, dst, [0] * out.rank, out.shape)
+            wbuf = self._new_buf((x.shape[axis],), DType.int32, "temp", -1)
+            self._emit(Step("scatter", [ix.buf, up.buf, dst.buf], [dst.buf, wbuf.id], dict(
+                idx=ix, upd=up, dst=dst, winner=ViewRef(wbuf.id, 0, (x.shape[axis],), (1,), DType.int32),
+                outer=_numel(x.shape[:axis]), axis_len=x.shape[axis], n_idx=idx.numel(),
+                inner=_numel(x.shape[axis + 1:]))))
         elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
             ins = [self._contig(i) for i in n.inputs]
             dst = self._alloc_value(out)

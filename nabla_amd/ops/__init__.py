@@ -13,5 +13,5 @@ from .unary import (abs, cast, erf, exp, gelu, log, logsoftmax, neg, relu, rsqrt
                     silu, softmax, sqrt, tanh)
 from .utils import call_custom_kernel
 from .view import (broadcast_to, concatenate, flatten, gather, moveaxis, pad, permute, reshape,
-                   slice_tensor, slice_update, squeeze, stack, swap_axes, take, transpose,
+                   scatter, slice_tensor, slice_update, squeeze, stack, swap_axes, take, transpose,
                    unsqueeze)

@@ -396,9 +396,10 @@ class GatherOp(AxisOp):
 
 
 class ScatterOp(AxisOp):
-    """``x`` with the rows selected by ``indices`` along ``axis`` replaced by
-    ``updates`` (indexing.py:185-447).  Recorded so that gather stays
-    differentiable in the trace; it has no kernel in this backend."""
+    """``x`` with the rows selected by ``indices`` along ``axis`` replaced by ``updates``
+    (indexing.py:185-447); the VJP of gather scatters the cotangent into zeros with it
+    (173-182).  A row named more than once takes the LAST update (numpy's assignment rule);
+    the reference leaves that order to its backend."""
 
     @property
     def name(self) -> str:
@@ -409,10 +410,24 @@ class ScatterOp(AxisOp):
         return [tuple(x.shape)], [x.dtype], [x.device]
 
     def kernel(self, args, kwargs):
-        raise NotImplementedError(
-            "scatter (the gradient of gather w.r.t. its table) is outside the op set of "
-            "this backend; treat the table as a constant"
-        )
+        x, idx, upd = args
+        if not idx.dtype.is_integral():
+            raise TypeError(f"scatter: indices must be integers, got {idx.dtype}")
+        if upd.dtype is not x.dtype:
+            upd = ir.cast(upd, x.dtype)
+        return [ir.scatter(x, idx, upd, self._norm_axis(kwargs.get("axis", 0), x.rank))]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        # the replaced rows of x receive nothing; every update receives the row it was written
+        # to (for a row named twice that is exact for the update that won)
+        from .creation import zeros_like
+        x, idx, upd = primals
+        g = cotangents[0]
+        gx = _scatter_op([g, idx, zeros_like(upd)], dict(kwargs))[0]
+        return [gx, None, _gather_op([g, idx], dict(kwargs))[0]]
+
+    def jvp_rule(self, primals, tangents, outputs, kwargs):
+        return [_scatter_op([tangents[0], primals[1], tangents[2]], dict(kwargs))[0]]
 
 
 _gather_op = GatherOp()
@@ -427,6 +442,13 @@ def gather(x: Tensor, indices: Tensor | None = None, axis: int = 0) -> Tensor:
 
 
 take = gather
+
+
+def scatter(x: Tensor, indices: Tensor, updates: Tensor, axis: int = 0) -> Tensor:
+    """Out-of-place ``out = x.copy(); out[indices] = updates`` along ``axis``
+    (indexing.py:483-504)."""
+    x, indices, updates = ensure_tensor(x), ensure_tensor(indices), ensure_tensor(updates)
+    return _scatter_op([x, indices, updates], {"axis": axis})[0]
 
 
 # ------------------------------------------------------------------ __getitem__

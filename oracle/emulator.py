@@ -360,6 +360,15 @@ class EmulatedPlan:
                     raise IndexError("gather: index out of range")
                 ix = torch.where(ix < 0, ix + a["axis_len"], ix)
                 _view(mem, a["dst"]).copy_(t.index_select(1, ix).reshape(a["dst"].shape))
+            elif k == "scatter":
+                dst = _view(mem, a["dst"]).reshape(a["outer"], a["axis_len"], a["inner"])
+                up = _view(mem, a["upd"]).reshape(a["outer"], a["n_idx"], a["inner"])
+                ix = _view(mem, a["idx"]).reshape(-1).long()
+                if bool(((ix < -a["axis_len"]) | (ix >= a["axis_len"])).any()):
+                    raise IndexError("scatter: index out of range")
+                ix = torch.where(ix < 0, ix + a["axis_len"], ix)
+                for j in range(a["n_idx"]):  # in order: the last write to a row wins
+                    dst[:, int(ix[j]), :] = up[:, j, :]
             elif k == "argreduce":
                 x = _as_f32(_view(mem, a["src"])).reshape(a["rows"], a["C"])
                 r = np.argmin(x, axis=1) if a["fn"] == "min" else np.argmax(x, axis=1)

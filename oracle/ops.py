@@ -356,9 +356,41 @@ def concatenate(xs, axis: int = 0) -> V:  # view/shape.py:821-980
     return V(np.concatenate([x.a for x in xs], axis=axis), xs, vjp)
 
 
-def gather(table, idx, axis: int = 0) -> V:  # view/indexing.py:100-171 (no table gradient here)
-    table, idx = _v(table), _v(idx)
-    return V(np.take(table.a, idx.a.astype(np.int64), axis=axis))
+def scatter(x, idx, updates, axis: int = 0) -> V:
+    """view/indexing.py:185-447, 483-504: ``out = x.copy(); out[idx] = updates`` along ``axis``.
+    Duplicate indices: the reference leaves the order to its backend; here (and in the kernels)
+    the last update wins, which is what numpy's assignment does.  Parity unpinned for
+    duplicates: none of the reference's fixtures fixes that order."""
+    x, updates = _v(x), _v(updates)
+    idx = (idx.a if isinstance(idx, V) else np.asarray(idx)).astype(np.int64)
+    out = x.a.copy()
+    sel = (slice(None),) * axis
+    flat_idx = idx.reshape(-1)
+    up = updates.a.reshape(x.a.shape[:axis] + (flat_idx.size,) + x.a.shape[axis + 1:])
+    for j, i in enumerate(flat_idx):
+        out[sel + (int(i),)] = up[sel + (j,)]
+
+    def vjp(g):
+        gx = g.copy()
+        for i in flat_idx:
+            gx[sel + (int(i),)] = 0
+        gu = np.stack([g[sel + (int(i),)] for i in flat_idx], axis=axis).reshape(updates.a.shape)
+        return (gx, gu)
+
+    return V(out, (x, updates), vjp)
+
+
+def gather(table, idx, axis: int = 0) -> V:  # view/indexing.py:100-182
+    """take along ``axis``; the VJP scatters the cotangent into zeros (173-182), i.e. a row
+    gathered several times receives the cotangent of its LAST occurrence, not their sum."""
+    table = _v(table)
+    idx = (idx.a if isinstance(idx, V) else np.asarray(idx)).astype(np.int64)
+    y = np.take(table.a, idx, axis=axis)
+
+    def vjp(g):
+        return (scatter(V(np.zeros_like(table.a, dtype=g.dtype)), idx, V(g), axis).a,)
+
+    return V(y, (table,), vjp)
 
 
 def tril(x, k: int = 0) -> V:  # creation.py:225-274

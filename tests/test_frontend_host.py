@@ -517,3 +517,35 @@ def test_silu_value_and_grad(emulator):
     np.testing.assert_allclose(nb.silu(T(x)).numpy(), O.silu(vx).a, rtol=1e-6, atol=1e-6)
     (wg,) = O.grad_of(O.reduce_sum(O.silu(vx)), [vx])
     np.testing.assert_allclose(nb.grad(lambda t: nb.reduce_sum(nb.silu(t)))(T(x)).numpy(), wg, rtol=1e-5, atol=1e-6)
+
+
+# ---- scatter / embedding-table gradient ----------------------------------------------------------------
+def test_scatter_value_rules_and_embedding_table_gradient(emulator):
+    x, upd = RNG.standard_normal((7, 5)).astype(np.float32), RNG.standard_normal((4, 5)).astype(np.float32)
+    idx = np.array([5, 0, 3, 5], dtype=np.int64)  # row 5 twice: the later update wins
+    I = nb.Tensor.constant(idx)
+    got = nb.scatter(T(x), I, T(upd))
+    np.testing.assert_array_equal(got.numpy(), O.scatter(O.V(x), idx, O.V(upd)).a)
+    assert last_plan().stats.get("scatter") == 1
+    x3 = RNG.standard_normal((2, 6, 3)).astype(np.float32)
+    u3 = RNG.standard_normal((2, 2, 3)).astype(np.float32)
+    i3 = np.array([-1, 2], dtype=np.int32)
+    np.testing.assert_array_equal(nb.scatter(T(x3), nb.Tensor.constant(i3), T(u3), axis=1).numpy(),
+                                  O.scatter(O.V(x3), i3 % 6, O.V(u3), axis=1).a)
+    # gradients of scatter
+    g = RNG.standard_normal((7, 5)).astype(np.float32)
+    gx, gu = nb.grad(lambda a, b: nb.reduce_sum(nb.scatter(a, I, b) * T(g)), argnums=(0, 1))(T(x), T(upd))
+    vx, vu = O.V(x.astype(np.float64)), O.V(upd.astype(np.float64))
+    wx, wu = O.grad_of(O.reduce_sum(O.scatter(vx, idx, vu) * O.V(g.astype(np.float64))), [vx, vu])
+    np.testing.assert_allclose(gx.numpy(), wx, rtol=1e-6)
+    np.testing.assert_allclose(gu.numpy(), wu, rtol=1e-6)
+    # the gradient of an embedding table: the cotangent scattered into zeros
+    table = RNG.standard_normal((9, 4)).astype(np.float32)
+    ids = np.array([[1, 7, 2], [0, 8, 3]], dtype=np.int64)
+    w = RNG.standard_normal((2, 3, 4)).astype(np.float32)
+    gt = nb.grad(lambda t: nb.reduce_sum(F.embedding(nb.Tensor.constant(ids), t) * T(w)))(T(table))
+    vt = O.V(table.astype(np.float64))
+    (wt,) = O.grad_of(O.reduce_sum(O.gather(vt, ids) * O.V(w.astype(np.float64))), [vt])
+    np.testing.assert_allclose(gt.numpy(), wt, rtol=1e-6)
+    with pytest.raises(Exception, match="updates of shape"):
+        nb.scatter(T(x), I, T(upd[:2])).realize()

@@ -487,3 +487,34 @@ def test_jvp_on_device_against_oracle_central_differences(hip):
     lhs = float((tan.numpy().astype(np.float64) * u).sum())
     rhs = sum(float((g.numpy().astype(np.float64) * v).sum()) for g, v in zip(gs, vs))
     assert abs(lhs - rhs) <= 2e-4 * max(abs(lhs), abs(rhs), 1e-3)
+
+
+# ---- scatter ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_scatter_on_device_is_exact_and_deterministic(hip, dtype):
+    """Bit-exact against the oracle (numpy assignment), including rows named several times
+    (the last update wins, whatever order the workgroups run in), negative indices, another
+    axis, and the embedding-table gradient that is built on it."""
+    from oracle import ops as O
+    rng = np.random.default_rng(47)
+    dt = nb.DType.float32 if dtype == "f32" else nb.DType.bfloat16
+    rnd = lambda *s: torch.from_numpy(rng.standard_normal(s).astype(np.float32)).to(dt.to_torch()).float().numpy()
+    x, upd = rnd(1000, 72), rnd(4096, 72)
+    idx = rng.integers(-1000, 1000, size=4096).astype(np.int64)   # many duplicates, half negative
+    T = lambda a: nb.Tensor.constant(a, dtype=dt)
+    want = O.scatter(O.V(x), idx % 1000, O.V(upd)).a
+    for _ in range(3):
+        got = nb.scatter(T(x), nb.Tensor.constant(idx), T(upd))
+        np.testing.assert_array_equal(nb.cast(got, nb.DType.float32).numpy(), want)
+    x3, u3 = rnd(3, 17, 5), rnd(3, 2, 2, 5)
+    i3 = np.array([[16, 0], [3, 16]], dtype=np.int32)
+    got = nb.scatter(T(x3), nb.Tensor.constant(i3), T(u3), axis=1)
+    np.testing.assert_array_equal(nb.cast(got, nb.DType.float32).numpy(), O.scatter(O.V(x3), i3, O.V(u3), axis=1).a)
+    with pytest.raises(IndexError):
+        nb.scatter(T(x), nb.Tensor.constant(np.array([1000], dtype=np.int64)), T(upd[:1])).numpy()
+    if dtype == "f32":
+        table, ids, w = rnd(500, 64), rng.integers(0, 500, size=(4, 33)).astype(np.int64), rnd(4, 33, 64)
+        gt = nb.grad(lambda t: nb.reduce_sum(nb.nn.functional.embedding(nb.Tensor.constant(ids), t) * T(w)))(T(table))
+        vt = O.V(table.astype(np.float64))
+        (wt,) = O.grad_of(O.reduce_sum(O.gather(vt, ids) * O.V(w.astype(np.float64))), [vt])
+        np.testing.assert_array_equal(gt.numpy(), wt.astype(np.float32))

@@ -390,3 +390,38 @@ def test_avg_pool_and_silu_against_torch():
     s = O.silu(vx)
     np.testing.assert_allclose(s.a, F.silu(torch.tensor(x)).numpy(), rtol=1e-12)
     np.testing.assert_allclose(O.grad_of(O.reduce_sum(s), [vx])[0], xt.grad.numpy(), rtol=1e-12)
+
+
+def test_scatter_and_gather_gradient_pins():
+    """scatter is numpy's ``out[idx] = updates`` (last write wins on duplicates) and torch's
+    index_copy for distinct indices; its VJP and the scatter-into-zeros VJP of gather are
+    checked against the definitions."""
+    rng = np.random.default_rng(25)
+    x, upd = rng.standard_normal((6, 4)), rng.standard_normal((3, 4))
+    idx = np.array([4, 0, 2])
+    got = O.scatter(O.V(x), idx, O.V(upd), axis=0)
+    want = x.copy(); want[idx] = upd
+    np.testing.assert_array_equal(got.a, want)
+    np.testing.assert_array_equal(got.a, torch.tensor(x).index_copy(0, torch.tensor(idx), torch.tensor(upd)).numpy())
+    # along another axis, with a 2-d index
+    x3, idx2 = rng.standard_normal((2, 5, 3)), np.array([[3, 1], [0, 4]])
+    upd3 = rng.standard_normal((2, 2, 2, 3))
+    want3 = x3.copy(); want3[:, idx2.reshape(-1), :] = upd3.reshape(2, 4, 3)
+    np.testing.assert_array_equal(O.scatter(O.V(x3), idx2, O.V(upd3), axis=1).a, want3)
+    # duplicates: the last update of a row wins
+    dup = O.scatter(O.V(np.zeros((3, 2))), np.array([1, 1, 2, 1]), O.V(np.arange(8.0).reshape(4, 2)))
+    np.testing.assert_array_equal(dup.a, [[0, 0], [6, 7], [4, 5]])
+    # VJP: replaced rows of x get nothing, updates get the rows they were written to
+    vx, vu = O.V(x), O.V(upd)
+    g = rng.standard_normal((6, 4))
+    gx, gu = O.grad_of(O.reduce_sum(O.scatter(vx, idx, vu) * O.V(g)), [vx, vu])
+    wx = g.copy(); wx[idx] = 0
+    np.testing.assert_array_equal(gx, wx)
+    np.testing.assert_array_equal(gu, g[idx])
+    # gather VJP = cotangent scattered into zeros (distinct indices: torch's index_select grad)
+    tt = torch.tensor(x, requires_grad=True)
+    gg = rng.standard_normal((3, 4))
+    tt.index_select(0, torch.tensor(idx)).backward(torch.tensor(gg))
+    vt = O.V(x)
+    (gt,) = O.grad_of(O.reduce_sum(O.gather(vt, idx) * O.V(gg)), [vt])
+    np.testing.assert_array_equal(gt, tt.grad.numpy())
