@@ -10,8 +10,11 @@ against torch-CPU autograd in fp64, against brute-force loops on tiny inputs
 (matmul, conv2d, max_pool2d), and against closed forms (softmax rows sum to
 one, layer_norm output has zero mean / unit variance, tie rule of reduce_max).
 What those checks cannot see -- the bit-level rounding and accumulation order
-of the MAX kernels the reference calls, and its argmax tie-break -- is parity
-unpinned; argmax adopts the lowest index (numpy / torch / jax agree).
+of the MAX kernels the reference calls, its argmax tie-break, and the order in
+which its backend applies scatter updates that name one row several times --
+is parity unpinned; argmax adopts the lowest index (numpy / torch / jax agree)
+and scatter the last update (numpy assignment).  The NF4 functions are pinned by
+the decision thresholds between levels, exact round trips and the zero block.
 
 The oracle is eager: a ``V`` carries a numpy value and, when gradients are
 wanted, the closure that maps its cotangent to its parents' cotangents.
@@ -359,8 +362,8 @@ def concatenate(xs, axis: int = 0) -> V:  # view/shape.py:821-980
 def scatter(x, idx, updates, axis: int = 0) -> V:
     """view/indexing.py:185-447, 483-504: ``out = x.copy(); out[idx] = updates`` along ``axis``.
     Duplicate indices: the reference leaves the order to its backend; here (and in the kernels)
-    the last update wins, which is what numpy's assignment does.  Parity unpinned for
-    duplicates: none of the reference's fixtures fixes that order."""
+    the last update wins, which is what numpy's assignment does (parity unpinned for
+    duplicates: none of the reference's fixtures fixes that order)."""
     x, updates = _v(x), _v(updates)
     idx = (idx.a if isinstance(idx, V) else np.asarray(idx)).astype(np.int64)
     out = x.a.copy()
