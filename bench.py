@@ -75,22 +75,20 @@ def compiled_plan(nb, fn, args):
 
 
 # ------------------------------------------------------------------ workloads
-def workload_c2(nb, oc, rows=8192, cols=8192):
-    inp = oc.c2_inputs(rows, cols, seed=0)
-    X, Y = nb.Tensor.constant(inp["x"]), nb.Tensor.constant(inp["y"])
-
-    def step(X, Y):
-        return oc.c2_program(nb, X, Y)
-
+# The timed path uses the product only (nabla_amd.workloads: step programs and synthetic
+# inputs).  The CPU oracle is imported inside the cpu_baseline closures and nowhere else.
+def workload_c2(nb, rows=8192, cols=8192):
+    t = nb.workloads.synthetic_inputs("c2", rows=rows, cols=cols)
     algo_bytes = 3 * rows * cols * 4 + 2 * rows * 4
-    return dict(name=f"c2 elementwise+reduction fwd+grad, x,y[{rows},{cols}] fp32", fn=step,
-                args=(X, Y), dtype="f32", bound="hbm", algo=algo_bytes, dominant="rowprog",
-                cpu=lambda: cpu_c2(oc, rows, cols))
+    return dict(name=f"c2 elementwise+reduction fwd+grad, x,y[{rows},{cols}] fp32",
+                fn=nb.workloads.c2_step, args=(t["x"], t["y"]), dtype="f32", bound="hbm",
+                algo=algo_bytes, dominant="rowprog", cpu=lambda: cpu_c2(rows, cols))
 
 
-def cpu_c2(oc, rows, cols):
+def cpu_c2(rows, cols):
     # rows are independent, so a slice of them times like the whole step; the slice is sized
     # for a run of about ten seconds (one untimed pass first: page faults, numpy warm-up)
+    from oracle import configs as oc
     sample_rows = max(64, rows // 4)
     inp = oc.c2_inputs(sample_rows, cols, seed=0)
     oc.c2_reference(inp["x"][:64], inp["y"][:64], dtype=np.float32)
@@ -103,14 +101,12 @@ def cpu_c2(oc, rows, cols):
                 sample=f"{sample_rows} of {rows} rows x {reps} passes, numpy fp32 oracle, scaled by rows")
 
 
-def workload_c1(nb, oc):
-    inp = oc.c1_inputs()
-    t = {k: nb.Tensor.constant(v) for k, v in inp.items()}
-
-    def step(t):
-        return oc.c1_program(nb, t)
+def workload_c1(nb):
+    t = nb.workloads.synthetic_inputs("c1")
 
     def cpu():
+        from oracle import configs as oc
+        inp = oc.c1_inputs()
         t0 = time.perf_counter()
         n = 20
         for _ in range(n):
@@ -118,17 +114,12 @@ def workload_c1(nb, oc):
         return dict(value=n / (time.perf_counter() - t0), unit="steps/s", cores=os.cpu_count(),
                     kind="port", sample=f"{n} full steps, numpy fp32 oracle")
 
-    return dict(name="c1 2-layer MLP fwd+grad fp32, x[128,784]", fn=step, args=(t,), dtype="f32",
-                bound="mfma", algo=104.7e6, dominant="gemm", cpu=cpu)
+    return dict(name="c1 2-layer MLP fwd+grad fp32, x[128,784]", fn=nb.workloads.c1_step, args=(t,),
+                dtype="f32", bound="mfma", algo=104.7e6, dominant="gemm", cpu=cpu)
 
 
-def workload_c3(nb, oc, batch=8, seq=1024, d=1024, ff=4096):
-    inp = oc.c3_inputs(batch, seq, d, ff, seed=0, bf16=True)
-    t = oc.upload(nb, inp, dtype=nb.DType.bfloat16)
-
-    def step(t):
-        return oc.c3_program(nb, t, num_heads=16)
-
+def workload_c3(nb, batch=8, seq=1024, d=1024, ff=4096):
+    t = nb.workloads.synthetic_inputs("c3", batch=batch, seq=seq, d=d, ff=ff)
     T = batch * seq
     hd = d // 16
     qkvo = 4 * 2 * T * d * d
@@ -137,6 +128,7 @@ def workload_c3(nb, oc, batch=8, seq=1024, d=1024, ff=4096):
     flops = 3 * (qkvo + mlp + attn_causal)
 
     def cpu():
+        from oracle import configs as oc
         small = oc.c3_inputs(1, 128, d, ff, seed=0, bf16=True)
         t0 = time.perf_counter()
         oc.c3_reference(small, num_heads=16, dtype=np.float32)
@@ -147,17 +139,15 @@ def workload_c3(nb, oc, batch=8, seq=1024, d=1024, ff=4096):
                            "(attention cost per token is under-counted)")
 
     return dict(name=f"c3 pre-LN transformer block fwd+bwd bf16, B{batch} S{seq} D{d} FF{ff}",
-                fn=step, args=(t,), dtype="bf16", bound="mfma", algo=flops, dominant="gemm", cpu=cpu)
+                fn=lambda t: nb.workloads.c3_step(t, 16), args=(t,), dtype="bf16", bound="mfma",
+                algo=flops, dominant="gemm", cpu=cpu)
 
 
-def workload_c4(nb, oc):
-    inp = oc.c4_inputs()
-    t = oc.upload(nb, inp)
-
-    def step(t):
-        return oc.c4_program(nb, t)
+def workload_c4(nb):
+    t = nb.workloads.synthetic_inputs("c4")
 
     def cpu():
+        from oracle import configs as oc
         small = oc.c4_inputs(batch=4)
         t0 = time.perf_counter()
         oc.c4_reference(small, dtype=np.float32)
@@ -165,23 +155,20 @@ def workload_c4(nb, oc):
         return dict(value=1.0 / (dt * 16), unit="steps/s", cores=os.cpu_count(), kind="port",
                     sample="4 of 64 images, numpy fp32 oracle, scaled by batch")
 
-    return dict(name="c4 CNN step fp32, img[64,32,32,3]", fn=step, args=(t,), dtype="f32",
-                bound="mfma", algo=58.4e9, dominant="conv", cpu=cpu)
+    return dict(name="c4 CNN step fp32, img[64,32,32,3]", fn=nb.workloads.c4_step, args=(t,),
+                dtype="f32", bound="mfma", algo=58.4e9, dominant="conv", cpu=cpu)
 
 
-def workload_c5(nb, oc, layers=12):
-    inp = oc.c5_inputs(layers=layers, seed=0, b_zero=True, bf16=True)
-    t = oc.upload(nb, inp, dtype=nb.DType.bfloat16)
-
-    def step(t):
-        return oc.c5_program(nb, t, num_heads=16)
+def workload_c5(nb, layers=12):
+    t = nb.workloads.synthetic_inputs("c5", layers=layers)
 
     def cpu():
         return dict(value=None, unit="steps/s", cores=os.cpu_count(), kind="port",
                     sample="not run: one step is ~27 TFLOP on the host")
 
-    return dict(name=f"c5 LoRA step bf16, {layers} layers D2048 S2048 B4", fn=step, args=(t,),
-                dtype="bf16", bound="mfma", algo=24.5e12 * layers / 12, dominant="gemm", cpu=cpu)
+    return dict(name=f"c5 LoRA step bf16, {layers} layers D2048 S2048 B4 (lora_linear in low-rank order)",
+                fn=lambda t: nb.workloads.c5_step(t, 16), args=(t,), dtype="bf16", bound="mfma",
+                algo=24.5e12 * layers / 12, dominant="gemm", cpu=cpu)
 
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4,
@@ -221,11 +208,10 @@ def main() -> int:
     import nabla_amd as nb
     from nabla_amd.backend import lib as nbk_lib
     from nabla_amd.backend.executor import get_executor
-    from oracle import configs as oc
 
     ex = get_executor()  # raises without libnbk.so or without a gfx950 GPU
     L = nbk_lib.load()
-    w = WORKLOADS[a.workload](nb, oc)
+    w = WORKLOADS[a.workload](nb)
     cf, spec, bufs, first = compiled_plan(nb, w["fn"], w["args"])
     plan = spec.bound.plan
     inputs = bufs()

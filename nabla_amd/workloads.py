@@ -135,3 +135,49 @@ def c5_shapes(layers=12, batch=4, seq=2048, d=2048, ff=8192, vocab=32000, rank=1
             "layers": [_block_shapes(d, ff) for _ in range(layers)],
             "lora": [{"qA": (d, rank), "qB": (rank, d), "vA": (d, rank), "vB": (rank, d)}
                      for _ in range(layers)]}
+
+
+# ---- synthetic inputs of the five configurations ---------------------------------------------
+def synthetic_inputs(config: str, seed: int = 0, **size):
+    """Seeded random leaf tensors for ``c1`` .. ``c5`` (sizes default to the full configuration;
+    keyword arguments go to the matching ``*_shapes``).  Weights are small normals (uniform for
+    the MLP, fan-in scaled for the CNN), biases zero, layer-norm weights one, LoRA ``B`` factors
+    zero as at the start of fine-tuning; the transformer and LoRA configurations are bfloat16."""
+    import math
+
+    import numpy as np
+
+    from .core.dtype import DType
+
+    rng = np.random.default_rng(seed)
+    shapes = {"c1": c1_shapes, "c2": c2_shapes, "c3": c3_shapes, "c4": c4_shapes, "c5": c5_shapes}[config](**size)
+    float_dtype = DType.bfloat16 if config in ("c3", "c5") else DType.float32
+
+    def leaf(name: str, shape):
+        if name in ("ids", "labels"):
+            hi = size.get("vocab", 32000) if name == "ids" else size.get("classes", 10)
+            return nb.Tensor.constant(rng.integers(0, hi, shape).astype(np.int64))
+        if name.startswith("b") or (name.endswith("b") and name[0] in "cl") or name in ("qB", "vB"):
+            a = np.zeros(shape, np.float32)                      # biases, ln*_b, c*b, LoRA B
+        elif name.startswith("ln") or name == "lnf_w":
+            a = np.ones(shape, np.float32)                       # layer-norm weights
+        elif config == "c1":
+            a = rng.uniform(-0.05, 0.05, shape).astype(np.float32)
+        elif name == "img":
+            a = rng.uniform(0.0, 1.0, shape).astype(np.float32)
+        elif config == "c4":
+            a = (rng.standard_normal(shape) * math.sqrt(2.0 / math.prod(shape[:-1]))).astype(np.float32)
+        elif name in ("x", "y"):
+            a = rng.standard_normal(shape, dtype=np.float32)
+        else:
+            a = rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)
+        return nb.Tensor.constant(a, dtype=float_dtype)
+
+    def build(tree, name=""):
+        if isinstance(tree, dict):
+            return {k: build(v, k) for k, v in tree.items()}
+        if isinstance(tree, list):
+            return [build(v, name) for v in tree]
+        return leaf(name, tree)
+
+    return build(shapes)
