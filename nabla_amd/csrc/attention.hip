@@ -164,7 +164,7 @@ __device__ __forceinline__ at_bf16x8 at_regs_frag(const at_f32x16& s, int t) {
 __device__ __forceinline__ float at_xhalf(float v) { return __shfl_xor(v, 32, 64); }
 
 // ------------------------------------------------------------------------------ forward
-// Grid: (S / 128, B * H).  Wave w owns queries q0 + 32w .. + 31 (one per lane pair).
+// Grid: (B * H, S / 128).  Wave w owns queries q0 + 32w .. + 31 (one per lane pair).
 //
 // The softmax runs in base 2 on t = score * scale * log2(e).  The running maximum m of a
 // row is only raised when some row of the wave has outgrown it by more than AT_SLACK (a
@@ -184,8 +184,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   auto k_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * (ROW_BYTES + TR_BYTES)); };
   auto v_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * (ROW_BYTES + TR_BYTES) + ROW_BYTES); };
 
-  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
-  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;  // long causal rows first
+  // Grid (B * H, tiles): workgroups are handed out along x first, so every (batch, head) runs
+  // its longest causal rows before any runs a shorter one, and the tail of the launch consists
+  // of the shortest workgroups.
+  const int bh = blockIdx.x, b = bh / g.H, hh = bh % g.H;
+  const int qt = (int)gridDim.y - 1 - (int)blockIdx.y;
   const int q0 = qt * 128;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
   const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs g) {
   if (row < rows && c == 0) g.delta[row] = s;
 }
 
-// dK, dV.  Grid: (S / 128, B * H).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
+// dK, dV.  Grid: (B * H, S / 128).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
 // and walks the query tiles that can see them.
 //   S[q, key]  = Q K^T          (A: Q tile rows, B: the wave's K fragments)
 //   P          = exp(S * scale - LSE[q])   (as exp2, with LSE staged in base-2 units)
@@ -358,8 +361,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
   auto dot_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * STAGE + 2 * ROW_BYTES + TR_BYTES); };
   auto lse_tile = [&](int buf) { return (float*)(at_lds + buf * STAGE + 2 * ROW_BYTES + 2 * TR_BYTES); };
 
-  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
-  const int k0 = blockIdx.x * 128;
+  const int bh = blockIdx.x, b = bh / g.H, hh = bh % g.H;
+  const int k0 = blockIdx.y * 128;  // the first key tiles see the most queries
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
   const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
   const uint16_t* K = g.k.p + (int64_t)b * g.k.sb + (int64_t)hh * g.k.sh;
@@ -483,7 +486,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
     }
 }
 
-// dQ.  Grid: (S / 128, B * H).  Wave w owns queries q0 + 32w .. + 31 and walks the key tiles.
+// dQ.  Grid: (B * H, S / 128).  Wave w owns queries q0 + 32w .. + 31 and walks the key tiles.
 //   S^T[key, q]  = K Q^T                (A: K tile rows, B: the wave's Q fragments)
 //   P^T          = exp(S^T * scale - LSE[q])
 //   dP^T[key, q] = V dO^T               (A: V tile rows, B: the wave's dO fragments)
@@ -504,8 +507,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_kernel(const AttnArgs g) {
   auto v_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE + ROW_BYTES); };
   auto kt_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * STAGE + 2 * ROW_BYTES); };
 
-  const int bh = blockIdx.y, b = bh / g.H, hh = bh % g.H;
-  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int bh = blockIdx.x, b = bh / g.H, hh = bh % g.H;
+  const int qt = (int)gridDim.y - 1 - (int)blockIdx.y;
   const int q0 = qt * 128;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 31, h = lane >> 5;
   const uint16_t* Q = g.q.p + (int64_t)b * g.q.sb + (int64_t)hh * g.q.sh;
@@ -632,7 +635,7 @@ static int attn_common(const nbk_attn_desc* d, AttnArgs* a) {
   NBK_REQUIRE(d->B > 0 && d->H > 0 && d->S > 0 && d->S % 128 == 0,
               "attention: B %lld, H %lld, S %lld (S must be a positive multiple of 128)",
               (long long)d->B, (long long)d->H, (long long)d->S);
-  NBK_REQUIRE(d->B * d->H <= 65535 && d->S <= (1 << 24), "attention: extent beyond the grid limits");
+  NBK_REQUIRE(d->B * d->H <= 0x7fffffffLL && d->S / 128 <= 65535, "attention: extent beyond the grid limits");
   a->B = (int32_t)d->B; a->H = (int32_t)d->H; a->S = (int32_t)d->S;
   a->causal = d->causal ? 1 : 0;
   a->scale = d->scale;
@@ -657,7 +660,7 @@ extern "C" int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* 
     return rc;
   NBK_REQUIRE(lse != nullptr, "attention: null lse");
   a.lse = (float*)lse;
-  const dim3 grid((unsigned)(d->S / 128), (unsigned)(d->B * d->H));
+  const dim3 grid((unsigned)(d->B * d->H), (unsigned)(d->S / 128));
   hipStream_t st = (hipStream_t)stream;
   if (d->hd == 64) {
     const size_t lds = 2 * (64 * 64 * 2 + 64 * AT_TP * 2);
@@ -698,7 +701,7 @@ extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* 
   a.delta = (float*)workspace;
   hipStream_t st = (hipStream_t)stream;
   const int64_t rows = d->B * d->H * d->S;
-  const dim3 grid((unsigned)(d->S / 128), (unsigned)(d->B * d->H));
+  const dim3 grid((unsigned)(d->B * d->H), (unsigned)(d->S / 128));
   if (d->hd == 64) {
     hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)((rows * 8 + 255) / 256)), dim3(256), 0, st, a);
     const size_t lds_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * AT_TP * 2 + 2 * 64 * 4);
