@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 8
+#define NBK_ABI_VERSION 9
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -176,6 +176,17 @@ int nbk_rowprog_is_specialized(const nbk_rowprog* prog);
 int nbk_reduce_mid(const void* in, void* out, int32_t dtype_in, int32_t dtype_out,
                    int64_t outer, int64_t red, int64_t inner, int32_t kind,
                    void* stream);
+/* Several independent reductions of that form in one launch (the un-broadcast sums of a
+ * backward pass -- one per bias and norm parameter -- are many, small and ready together).
+ * `tasks` is a host array; results are those of nbk_reduce_mid task by task. */
+#define NBK_REDUCE_BATCH_MAX 24   /* tasks per launch; longer lists take several */
+typedef struct nbk_reduce_task {
+  const void* in;
+  void* out;
+  int64_t outer, red, inner;
+  int32_t dtype_in, dtype_out, kind, reserved;
+} nbk_reduce_task;
+int nbk_reduce_mid_batch(const nbk_reduce_task* tasks, int32_t n, void* stream);
 
 /* ===================================================================== */
 /*  Strided copy (materialise a view)                                     */

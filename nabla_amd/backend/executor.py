@@ -123,6 +123,15 @@ class BoundPlan:
                 self.calls.append((L.nbk_reduce_mid,
                                    [holder, ("p0", "p1"), src.dtype.abi, dst.dtype.abi, a["outer"],
                                     a["red"], a["inner"], _RED[a["fn"]]], patches, None))
+            elif k == "reduce_batch":
+                tasks = (lib.ReduceTask * len(a["tasks"]))()
+                for t, ta in zip(tasks, a["tasks"]):
+                    src, dst = ta["src"], ta["dst"]
+                    ptr_field(t, "in_", src.buf, src.offset * src.dtype.size_in_bytes)
+                    ptr_field(t, "out", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                    t.outer, t.red, t.inner = ta["outer"], ta["red"], ta["inner"]
+                    t.dtype_in, t.dtype_out, t.kind = src.dtype.abi, dst.dtype.abi, _RED[ta["fn"]]
+                self.calls.append((L.nbk_reduce_mid_batch, [tasks, len(a["tasks"])], patches, tasks))
             elif k == "gemm":
                 d = lib.GemmDesc()
                 ra, rb, rc = a["a"], a["b"], a["dst"]

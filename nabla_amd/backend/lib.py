@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 MAX_RANK = 8
 
@@ -102,6 +102,14 @@ class AttnTensor(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("sb", C.c_int64), ("ss", C.c_int64), ("sh", C.c_int64)]
 
 
+class ReduceTask(C.Structure):
+    _fields_ = [
+        ("in_", C.c_void_p), ("out", C.c_void_p),
+        ("outer", C.c_int64), ("red", C.c_int64), ("inner", C.c_int64),
+        ("dtype_in", C.c_int32), ("dtype_out", C.c_int32), ("kind", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
 class TensorDesc(C.Structure):
     _fields_ = [
         ("ptr", C.c_void_p), ("dtype", C.c_int32), ("rank", C.c_int32),
@@ -123,6 +131,7 @@ _SIGNATURES = {
     "nbk_rowprog_is_specialized": ([C.POINTER(RowProg)], C.c_int),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
                         C.c_int64, C.c_int32, C.c_void_p], C.c_int),
+    "nbk_reduce_mid_batch": ([C.POINTER(ReduceTask), C.c_int32, C.c_void_p], C.c_int),
     "nbk_copy_strided": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
                           C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64),
                           C.c_void_p], C.c_int),

@@ -605,6 +605,7 @@ class Planner:
         self.skip_nodes: set[int] = set()  # reductions folded into an earlier one
         self.n_split = 0                   # fusion groups cut in two at lowering time
         self._materialized: dict = {}
+        self._deferred_reduces: list[list[Step]] = [[], []]  # first-stage / second-stage tasks
         self.users: dict[int, list[ir.Node]] = {}
         for n in nodes:
             for i in n.inputs:
@@ -640,6 +641,7 @@ class Planner:
             else:
                 self._lower_single(u.nodes[0])
 
+        self._flush_reduces()
         outs = []
         for oi, v in enumerate(self.outputs):
             if oi in self._out_done:
@@ -812,6 +814,31 @@ class Planner:
             src = self._materialize(src)
         self._emit(Step("copy", [src.buf], [dst.buf], dict(src=src, dst=window)))
 
+    def _terminal(self, v: ir.Value) -> bool:
+        """Nothing computes on ``v``: it only leaves the plan, possibly through views."""
+        for u in self.users.get(v.id, ()):
+            if u.kind not in VIEW_KINDS or not self._terminal(u.outputs[0]):
+                return False
+        return True
+
+    def _emit_reduce(self, step: Step, stage: int, terminal: bool) -> None:
+        """A reduction whose result only leaves the plan waits for the end of the plan, where all
+        such reductions go out together (one launch per stage instead of one each)."""
+        if terminal:
+            self._deferred_reduces[stage].append(step)
+        else:
+            self._emit(step)
+
+    def _flush_reduces(self) -> None:
+        for tasks in self._deferred_reduces:
+            if len(tasks) == 1:
+                self._emit(tasks[0])
+            elif tasks:
+                self._emit(Step("reduce_batch", [r for t in tasks for r in t.reads],
+                                [w for t in tasks for w in t.writes],
+                                dict(tasks=[t.attrs for t in tasks])))
+        self._deferred_reduces = [[], []]
+
     def _lower_reduce_mid(self, n: ir.Node) -> None:
         if n.pos in self.skip_nodes:
             return
@@ -877,19 +904,20 @@ class Planner:
                 if red % s == 0 and outer * s <= 65535:
                     split = s
                     break
+        terminal = self._terminal(out)
         if split > 1:
             tmp = self._new_buf((outer, split, inner), DType.float32)
             tref = ViewRef(tmp.id, 0, (outer, split, inner),
                            contiguous_strides((outer, split, inner)), DType.float32)
-            self._emit(Step("reduce_mid", [src.buf], [tmp.id], dict(
-                src=src, dst=tref, outer=outer * split, red=red // split, inner=inner, fn=kind)))
+            self._emit_reduce(Step("reduce_mid", [src.buf], [tmp.id], dict(
+                src=src, dst=tref, outer=outer * split, red=red // split, inner=inner, fn=kind)), 0, terminal)
             dst = self._alloc_value(out)
-            self._emit(Step("reduce_mid", [tmp.id], [dst.buf], dict(
-                src=tref, dst=dst, outer=outer, red=split, inner=inner, fn=kind)))
+            self._emit_reduce(Step("reduce_mid", [tmp.id], [dst.buf], dict(
+                src=tref, dst=dst, outer=outer, red=split, inner=inner, fn=kind)), 1, terminal)
             return
         dst = self._alloc_value(out)
-        self._emit(Step("reduce_mid", [src.buf], [dst.buf], dict(
-            src=src, dst=dst, outer=outer, red=red, inner=inner, fn=kind)))
+        self._emit_reduce(Step("reduce_mid", [src.buf], [dst.buf], dict(
+            src=src, dst=dst, outer=outer, red=red, inner=inner, fn=kind)), 0, terminal)
 
     # ................................................................ matmul
     @staticmethod
@@ -1061,8 +1089,8 @@ class Planner:
         tref = ViewRef(tmp.id, 0, (ks, M, N), contiguous_strides((ks, M, N)), DType.float32)
         self._emit(Step("gemm", [ra.buf, rb.buf], [tmp.id], dict(
             common, dst=tref, K=kc, batch=ks, a_bs=kc * pa[2], b_bs=kc * pb[1])))
-        self._emit(Step("reduce_mid", [tmp.id], [dst.buf], dict(
-            src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum")))
+        self._emit_reduce(Step("reduce_mid", [tmp.id], [dst.buf], dict(
+            src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum")), 1, self._terminal(out))
 
     # ................................................................ attention
     def _heads_operand(self, v: ir.Value) -> ViewRef:

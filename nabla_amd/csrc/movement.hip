@@ -156,13 +156,12 @@ extern "C" int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void*
 __device__ __forceinline__ float red_comb(float a, float b, int kind) {
   return kind == NBK_RED_SUM ? a + b : (kind == NBK_RED_MAX ? fmaxf(a, b) : fminf(a, b));
 }
-__global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict__ in,
-                                                         void* __restrict__ out, int dti, int dto,
-                                                         int64_t red, int64_t inner, int kind) {
+__device__ __forceinline__ void reduce_mid_body(const void* __restrict__ in, void* __restrict__ out,
+                                                int dti, int dto, int64_t red, int64_t inner,
+                                                int kind, int64_t bx, int64_t o) {
   __shared__ float part[4][64];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int64_t o = blockIdx.y;
-  const int64_t col = (int64_t)blockIdx.x * 64 + lane;
+  const int64_t col = bx * 64 + lane;
   float acc = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
   if (col < inner) {
     const int64_t base = o * red * inner + col;
@@ -199,18 +198,22 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict_
     nbk_store_from_f32(out, o * inner + col, dto, v);
   }
 }
+__global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict__ in,
+                                                         void* __restrict__ out, int dti, int dto,
+                                                         int64_t red, int64_t inner, int kind) {
+  reduce_mid_body(in, out, dti, dto, red, inner, kind, blockIdx.x, blockIdx.y);
+}
 
 // Vector form: a lane owns VEC consecutive columns (16 bytes of input per row), a
 // workgroup 64 * VEC columns; its four waves take every fourth row and keep up to
 // sixteen row loads in flight each.  T is the input element (uint16_t = bf16, float).
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
-                                                             void* __restrict__ out, int dto,
-                                                             int64_t red, int64_t inner, int kind) {
+__device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, void* __restrict__ out,
+                                                    int dto, int64_t red, int64_t inner, int kind,
+                                                    int64_t bx, int64_t o) {
   __shared__ float part[4][64][VEC + 1];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int64_t o = blockIdx.y;
-  const int64_t col = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const int64_t col = (bx * 64 + lane) * VEC;
   const float ident = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
   float acc[VEC];
 #pragma unroll
@@ -270,6 +273,37 @@ __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict
     }
   }
 }
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
+                                                             void* __restrict__ out, int dto,
+                                                             int64_t red, int64_t inner, int kind) {
+  reduce_mid_vec_body<T, VEC>(in, out, dto, red, inner, kind, blockIdx.x, blockIdx.y);
+}
+
+// Several independent reductions in one launch (the column sums behind the bias and norm
+// gradients of a step are many, small and ready at the same time: one launch instead of one
+// each).  A workgroup finds its task from the running block counts and runs the same body.
+struct ReduceBatchArgs {
+  int32_t n;
+  int32_t first_block[NBK_REDUCE_BATCH_MAX + 1];
+  int32_t blocks_x[NBK_REDUCE_BATCH_MAX];
+  int32_t mode[NBK_REDUCE_BATCH_MAX];  // 0: element-wise, 1: bf16 x 8, 2: fp32 x 4
+  nbk_reduce_task t[NBK_REDUCE_BATCH_MAX];
+};
+
+__global__ __launch_bounds__(256) void reduce_batch_kernel(const ReduceBatchArgs B) {
+  int i = 0;
+  while (i + 1 < B.n && (int)blockIdx.x >= B.first_block[i + 1]) ++i;
+  const nbk_reduce_task& t = B.t[i];
+  const int lb = (int)blockIdx.x - B.first_block[i];
+  const int64_t bx = lb % B.blocks_x[i], o = lb / B.blocks_x[i];
+  if (B.mode[i] == 1)
+    reduce_mid_vec_body<uint16_t, 8>((const uint16_t*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o);
+  else if (B.mode[i] == 2)
+    reduce_mid_vec_body<float, 4>((const float*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o);
+  else
+    reduce_mid_body(t.in, t.out, t.dtype_in, t.dtype_out, t.red, t.inner, t.kind, bx, o);
+}
 
 extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
                               int64_t red, int64_t inner, int32_t kind, void* stream) {
@@ -295,4 +329,35 @@ extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dt
   hipLaunchKernelGGL(reduce_mid_kernel, grid, dim3(256), 0, (hipStream_t)stream, in, out, dti, dto,
                      red, inner, kind);
   return nbk_check_launch("reduce_mid_kernel");
+}
+
+extern "C" int nbk_reduce_mid_batch(const nbk_reduce_task* tasks, int32_t n, void* stream) {
+  NBK_REQUIRE(tasks != nullptr && n > 0, "reduce_mid_batch: no tasks");
+  for (int32_t base = 0; base < n; base += NBK_REDUCE_BATCH_MAX) {
+    ReduceBatchArgs B;
+    B.n = n - base < NBK_REDUCE_BATCH_MAX ? n - base : NBK_REDUCE_BATCH_MAX;
+    int64_t blocks = 0;
+    for (int i = 0; i < B.n; ++i) {
+      const nbk_reduce_task& t = tasks[base + i];
+      NBK_REQUIRE(t.in && t.out, "reduce_mid_batch: task %d: null pointer", base + i);
+      NBK_REQUIRE(t.outer > 0 && t.red > 0 && t.inner > 0, "reduce_mid_batch: task %d: empty extent", base + i);
+      NBK_REQUIRE(t.kind >= NBK_RED_SUM && t.kind <= NBK_RED_MIN, "reduce_mid_batch: task %d: kind %d", base + i, t.kind);
+      NBK_REQUIRE(nbk_dtype_size(t.dtype_in) > 0 && nbk_dtype_size(t.dtype_out) > 0,
+                  "reduce_mid_batch: task %d: bad dtype", base + i);
+      const bool aligned = ((uintptr_t)t.in & 15) == 0;
+      int vec = 1;
+      B.mode[i] = 0;
+      if (t.dtype_in == NBK_BF16 && t.inner % 8 == 0 && aligned) { B.mode[i] = 1; vec = 8; }
+      else if (t.dtype_in == NBK_F32 && t.inner % 4 == 0 && aligned) { B.mode[i] = 2; vec = 4; }
+      const int64_t bx = (t.inner / vec + 63) / 64;
+      B.blocks_x[i] = (int32_t)bx;
+      B.first_block[i] = (int32_t)blocks;
+      blocks += bx * t.outer;
+      NBK_REQUIRE(blocks <= 0x7fffffffLL, "reduce_mid_batch: launch too large");
+      B.t[i] = t;
+    }
+    B.first_block[B.n] = (int32_t)blocks;
+    hipLaunchKernelGGL(reduce_batch_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, B);
+  }
+  return nbk_check_launch("reduce_batch_kernel");
 }

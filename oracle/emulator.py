@@ -337,12 +337,13 @@ class EmulatedPlan:
                 v = a["value"]
                 t = mem[a["buf"]]
                 t.fill_(bool(v) if t.dtype == torch.bool else (int(v) if not t.dtype.is_floating_point else v))
-            elif k == "reduce_mid":
-                src = mem[a["src"].buf][a["src"].offset:a["src"].offset + a["outer"] * a["red"] * a["inner"]]
-                x = _as_f32(src).reshape(a["outer"], a["red"], a["inner"])
-                r = {"sum": x.sum(axis=1, dtype=np.float64), "max": x.max(axis=1), "min": x.min(axis=1)}[a["fn"]]
-                d = a["dst"]
-                _store(mem[d.buf], d.offset + np.arange(a["outer"] * a["inner"]), np.asarray(r, dtype=_F32))
+            elif k in ("reduce_mid", "reduce_batch"):
+                for t in ([a] if k == "reduce_mid" else a["tasks"]):
+                    src = mem[t["src"].buf][t["src"].offset:t["src"].offset + t["outer"] * t["red"] * t["inner"]]
+                    x = _as_f32(src).reshape(t["outer"], t["red"], t["inner"])
+                    r = {"sum": x.sum(axis=1, dtype=np.float64), "max": x.max(axis=1), "min": x.min(axis=1)}[t["fn"]]
+                    d = t["dst"]
+                    _store(mem[d.buf], d.offset + np.arange(t["outer"] * t["inner"]), np.asarray(r, dtype=_F32))
             elif k == "gemm":
                 _gemm(a, mem)
             elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):

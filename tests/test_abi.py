@@ -54,6 +54,8 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
         "         sizeof(nbk_tensor));\n"
         '  printf("%zu %zu %zu %zu\\n", offsetof(nbk_rowprog, imm), offsetof(nbk_rowprog, operand),\n'
         "         offsetof(nbk_rowprog, ins), offsetof(nbk_gemm_desc, alpha));\n"
+        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(nbk_attn_desc), sizeof(nbk_attn_tensor),\n'
+        "         sizeof(nbk_reduce_task), offsetof(nbk_attn_desc, scale), offsetof(nbk_reduce_task, dtype_in));\n"
         "  return 0;\n}\n")
     exe = tmp_path / "sizes"
     subprocess.run(["gcc", f"-I{ROOT / 'include'}", str(src), "-o", str(exe)], check=True)
@@ -62,8 +64,10 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
     assert sizes[:7] == [C.sizeof(lib.RowProg), C.sizeof(lib.Operand), C.sizeof(lib.Ins),
                          C.sizeof(lib.GemmDesc), C.sizeof(lib.ConvDesc), C.sizeof(lib.PoolDesc),
                          C.sizeof(lib.TensorDesc)]
-    assert sizes[7:] == [lib.RowProg.imm.offset, lib.RowProg.operand.offset, lib.RowProg.ins.offset,
-                         lib.GemmDesc.alpha.offset]
+    assert sizes[7:11] == [lib.RowProg.imm.offset, lib.RowProg.operand.offset, lib.RowProg.ins.offset,
+                           lib.GemmDesc.alpha.offset]
+    assert sizes[11:] == [C.sizeof(lib.AttnDesc), C.sizeof(lib.AttnTensor), C.sizeof(lib.ReduceTask),
+                          lib.AttnDesc.scale.offset, lib.ReduceTask.dtype_in.offset]
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):

@@ -252,6 +252,38 @@ def test_reduce_mid_direct(hip, dtype, outer, red, inner):
             assert torch.equal(out.cpu().double(), ref)
 
 
+def test_reduce_mid_batch_matches_single_launches(hip):
+    """One launch for many reductions: mixed dtypes, kinds, vector and element-wise shapes, more
+    tasks than one launch holds; every result equals the single-task entry point's bit for bit."""
+    from nabla_amd.backend import lib
+    rng = np.random.default_rng(15)
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    specs = [(1, 128, 1024, "bf16", 0), (3, 64, 40, "f32", 1), (2, 77, 8, "bf16", 2), (1, 8, 4096, "f32", 0),
+             (4, 300, 1, "f32", 0), (1, 515, 24, "bf16", 0)] * 5          # 30 tasks > 24 per launch
+    tasks = (lib.ReduceTask * len(specs))()
+    keep, want = [], []
+    for t, (outer, red, inner, dt, kind) in zip(tasks, specs):
+        tdt = torch.float32 if dt == "f32" else torch.bfloat16
+        x = torch.tensor(rng.standard_normal((outer, red, inner)), dtype=tdt, device="cuda")
+        out = torch.full((outer, inner), float("nan"), dtype=torch.float32, device="cuda")
+        ref = torch.empty_like(out)
+        code = 0 if dt == "f32" else 1
+        lib.check(L.nbk_reduce_mid(C.c_void_p(x.data_ptr()), C.c_void_p(ref.data_ptr()), code, 0, outer, red,
+                                   inner, kind, st))
+        t.in_, t.out = x.data_ptr(), out.data_ptr()
+        t.outer, t.red, t.inner = outer, red, inner
+        t.dtype_in, t.dtype_out, t.kind = code, 0, kind
+        keep.append((x, out))
+        want.append(ref)
+    lib.check(L.nbk_reduce_mid_batch(tasks, len(specs), st))
+    torch.cuda.synchronize()
+    for (x, out), ref in zip(keep, want):
+        assert torch.equal(out, ref)
+    with pytest.raises(ValueError, match="no tasks"):
+        lib.check(L.nbk_reduce_mid_batch(tasks, 0, st))
+
+
 def test_conv_wgrad_workspace_and_fallback(hip):
     """The K-split filter gradient (with workspace) and the unsplit one (workspace NULL)
     agree to summation-order noise, and both match a float64 reference."""
