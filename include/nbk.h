@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 9
+#define NBK_ABI_VERSION 10
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -139,7 +139,9 @@ enum nbk_rp_op {
   NBK_OP_POW = 44, NBK_OP_AND = 45, NBK_OP_OR = 46,
   /* ternary */
   NBK_OP_WHERE = 48,   /* dst <- a != 0 ? b : c                                */
-  NBK_OP_FMA = 49      /* dst <- a * b + c                                     */
+  NBK_OP_FMA = 49,     /* dst <- a * b + c                                     */
+  /* more unary ops (the block 16..31 is full) */
+  NBK_OP_DGELU = 50    /* derivative of the exact GELU: Phi(a) + a * phi(a)    */
 };
 
 enum nbk_red_kind { NBK_RED_SUM = 0, NBK_RED_MAX = 1, NBK_RED_MIN = 2 };

@@ -50,6 +50,10 @@ __device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
 
 __device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead);
 
+__host__ __device__ __forceinline__ bool rp_is_unary(int op) {
+  return (op >= NBK_OP_MOV && op < NBK_OP_ADD) || op == NBK_OP_DGELU;
+}
+
 // One body instruction on one chunk.
 template <typename IDX>
 __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins in, RpRegs& R,
@@ -67,7 +71,7 @@ __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins
                         rp_binary(op, a.z, b.z), rp_binary(op, a.w, b.w));
     }
     rp_write(R, in.dst, r);
-  } else if (op >= NBK_OP_MOV && op < NBK_OP_ADD) {
+  } else if (rp_is_unary(op)) {
     float4 a = rp_read(R, in.a);
     float4 r = make_float4(rp_unary(op, a.x), rp_unary(op, a.y), rp_unary(op, a.z),
                            rp_unary(op, a.w));
@@ -134,7 +138,7 @@ __device__ __forceinline__ void rp_exec_scalar(const nbk_rowprog& P, const nbk_i
     R.s[d] = rp_block_reduce(R.acc[in.a], in.b, red_buf);
   } else if (op >= NBK_OP_ADD && op < NBK_OP_WHERE) {
     R.s[d] = rp_binary(op, R.s[in.a - NBK_RP_NVEC], R.s[in.b - NBK_RP_NVEC]);
-  } else if (op >= NBK_OP_MOV && op < NBK_OP_ADD) {
+  } else if (rp_is_unary(op)) {
     R.s[d] = rp_unary(op, R.s[in.a - NBK_RP_NVEC]);
   } else if (op == NBK_OP_WHERE) {
     R.s[d] = R.s[in.a - NBK_RP_NVEC] != 0.f ? R.s[in.b - NBK_RP_NVEC] : R.s[in.c - NBK_RP_NVEC];
@@ -374,7 +378,7 @@ static int rp_validate(const nbk_rowprog* p) {
                       "rowprog: bad ACC at %d", q);
         } else if (op == NBK_OP_COLIDX) {
           NBK_REQUIRE(b.dst < NBK_RP_NVEC, "rowprog: bad COLIDX at %d", q);
-        } else if (op >= NBK_OP_MOV && op <= NBK_OP_FMA) {
+        } else if ((op >= NBK_OP_MOV && op <= NBK_OP_FMA) || rp_is_unary(op)) {
           NBK_REQUIRE(b.dst < NBK_RP_NVEC && b.a < 32 && b.b < 32 && b.c < 32,
                       "rowprog: bad register at %d", q);
         } else {
@@ -400,12 +404,12 @@ static int rp_validate(const nbk_rowprog* p) {
     } else if (op == NBK_OP_RED) {
       NBK_REQUIRE(p->has_reduce && sreg_dst && in.a < NBK_RP_NACC && in.b <= NBK_RED_MIN,
                   "rowprog: bad RED at %d", pc);
-    } else if (op >= NBK_OP_MOV && op <= NBK_OP_FMA) {
+    } else if ((op >= NBK_OP_MOV && op <= NBK_OP_FMA) || rp_is_unary(op)) {
       NBK_REQUIRE(sreg_dst && in.a >= NBK_RP_NVEC && in.a < 32, "rowprog: bad scalar op at %d",
                   pc);
-      if (op >= NBK_OP_ADD)
+      if (op >= NBK_OP_ADD && !rp_is_unary(op))
         NBK_REQUIRE(in.b >= NBK_RP_NVEC && in.b < 32, "rowprog: bad scalar op at %d", pc);
-      if (op >= NBK_OP_WHERE)
+      if (op >= NBK_OP_WHERE && !rp_is_unary(op))
         NBK_REQUIRE(in.c >= NBK_RP_NVEC && in.c < 32, "rowprog: bad scalar op at %d", pc);
     } else {
       NBK_REQUIRE(false, "rowprog: opcode %d not allowed in a prologue (at %d)", op, pc);

@@ -127,6 +127,9 @@ __device__ __forceinline__ float rp_unary(int op, float a) {
     case NBK_OP_RSQRT: return 1.0f / sqrtf(a);
     case NBK_OP_ERF: return erff(a);
     case NBK_OP_GELU: return 0.5f * a * (1.0f + erff(a * 0.70710678118654752440f));
+    case NBK_OP_DGELU:  // Phi(a) + a * phi(a)
+      return 0.5f * (1.0f + erff(a * 0.70710678118654752440f)) +
+             a * 0.39894228040143267794f * expf(-0.5f * a * a);
     case NBK_OP_TANH: return tanhf(a);
     case NBK_OP_SIGMOID: return 1.0f / (1.0f + expf(-a));
     case NBK_OP_ABS: return fabsf(a);
@@ -163,17 +166,18 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
 // absolute, Abramowitz & Stegun 7.1.26) are far inside the 4e-3 of a bf16 result, and
 // they take a fifth of the instructions of the correctly rounded library routines,
 // which is what bounds these kernels once their traffic is halved by the 16-bit I/O.
-__device__ __forceinline__ float rp_fast_erf(float x) {
+// e = exp(-x^2), passed in so that a caller that needs it anyway computes it once
+__device__ __forceinline__ float rp_fast_erf_with(float x, float e) {
   const float ax = fabsf(x);
   const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, ax, 1.0f));
   float p = fmaf(1.061405429f, t, -1.453152027f);
   p = fmaf(p, t, 1.421413741f);
   p = fmaf(p, t, -0.284496736f);
   p = fmaf(p, t, 0.254829592f);
-  const float e = __expf(-ax * ax);
   const float r = fmaf(-p * t, e, 1.0f);
   return copysignf(r, x);
 }
+__device__ __forceinline__ float rp_fast_erf(float x) { return rp_fast_erf_with(x, __expf(-x * x)); }
 __device__ __forceinline__ float rp_unary_lowp(int op, float a) {
   switch (op) {
     case NBK_OP_EXP: return __expf(a);
@@ -182,6 +186,13 @@ __device__ __forceinline__ float rp_unary_lowp(int op, float a) {
     case NBK_OP_RSQRT: return __builtin_amdgcn_rsqf(a);
     case NBK_OP_ERF: return rp_fast_erf(a);
     case NBK_OP_GELU: return 0.5f * a * (1.0f + rp_fast_erf(a * 0.70710678118654752440f));
+    case NBK_OP_DGELU: {
+      // the same exp(-a^2 / 2) serves the erf approximation and the density, and a GELU of
+      // the same value in the same kernel shares all of it after common-subexpression removal
+      const float z = a * 0.70710678118654752440f;
+      const float e = __expf(-z * z);
+      return 0.5f * (1.0f + rp_fast_erf_with(z, e)) + a * 0.39894228040143267794f * e;
+    }
     case NBK_OP_SIGMOID: return __builtin_amdgcn_rcpf(1.0f + __expf(-a));
     default: return rp_unary(op, a);
   }

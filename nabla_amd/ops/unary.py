@@ -197,14 +197,27 @@ class GeluOp(UnaryOperation):
         return [ir.ew("mul", ir.ew("mul", x, 0.5), ir.ew("add", ir.ew("tanh", inner), 1.0))]
 
     def _derivative(self, primal, output):
-        # GELU'(x) = cdf(x) + x * pdf(x)  (unary.py:583-595)
-        from .binary import add, div, mul
+        # GELU'(x) = cdf(x) + x * pdf(x)  (unary.py:583-595) as ONE elementwise function of x:
+        # its erf and its density share one exponential, and a GELU of the same x in the same
+        # kernel shares them too
+        return _gelu_grad_op([primal], {})[0]
+
+
+class GeluGradOp(UnaryOperation):
+    """``Phi(x) + x * phi(x)``, the derivative of the exact GELU."""
+
+    @property
+    def name(self) -> str:
+        return "gelu_grad"
+
+    kernel = _ew1("dgelu")
+
+    def _derivative(self, primal, output):
+        # d/dx [Phi + x phi] = phi * (2 - x^2)
+        from .binary import div, mul, sub
         x = primal
-        sqrt2 = math.sqrt(2.0)
-        sqrt2pi = math.sqrt(2.0 * math.pi)
-        cdf = mul(0.5, add(1.0, erf(div(x, sqrt2))))
-        pdf = div(exp(neg(div(mul(x, x), 2.0))), sqrt2pi)
-        return add(cdf, mul(x, pdf))
+        pdf = div(exp(neg(div(mul(x, x), 2.0))), math.sqrt(2.0 * math.pi))
+        return mul(pdf, sub(2.0, mul(x, x)))
 
 
 def _softmax_ir(x, axis: int, log: bool):
@@ -306,6 +319,7 @@ _relu_op, _exp_op, _neg_op, _abs_op = ReluOp(), ExpOp(), NegOp(), AbsOp()
 _log_op, _sqrt_op, _rsqrt_op, _erf_op = LogOp(), SqrtOp(), RsqrtOp(), ErfOp()
 _tanh_op, _sigmoid_op, _gelu_op, _cast_op = TanhOp(), SigmoidOp(), GeluOp(), CastOp()
 _silu_op = SiluOp()
+_gelu_grad_op = GeluGradOp()
 _softmax_native, _logsoftmax_native = _SoftmaxNativeOp(), _LogSoftmaxNativeOp()
 
 

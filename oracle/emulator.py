@@ -36,6 +36,8 @@ _UNARY = {
     "rsqrt": lambda a: (_F32(1) / np.sqrt(a)).astype(_F32),
     "erf": lambda a: _sp.erf(a.astype(np.float64)).astype(_F32),
     "gelu": lambda a: (0.5 * a.astype(np.float64) * (1.0 + _sp.erf(a.astype(np.float64) / np.sqrt(2.0)))).astype(_F32),
+    "dgelu": lambda a: (0.5 * (1.0 + _sp.erf(a.astype(np.float64) / np.sqrt(2.0))) +
+                        a.astype(np.float64) * np.exp(-0.5 * a.astype(np.float64) ** 2) / np.sqrt(2.0 * np.pi)).astype(_F32),
     "tanh": lambda a: np.tanh(a),
     "sigmoid": lambda a: (_F32(1) / (_F32(1) + np.exp(-a))).astype(_F32),
     "abs": lambda a: np.abs(a),
