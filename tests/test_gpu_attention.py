@@ -125,3 +125,99 @@ def test_attention_inside_the_transformer_block(hip):
     for k in oc.C3_PARAMS:
         got = grads[k].numpy().astype(np.float64)
         assert np.abs(got - wg[k]).max() <= 3e-2 * max(np.abs(wg[k]).max(), 1e-2 * scale), k
+
+
+def _run_fwd(lib, L, st, q, k, v, causal):
+    """q, k, v: device bf16 [B, S, H, hd] (any strides with hd contiguous) -> o, lse."""
+    B, S, H, hd = q.shape
+    o = torch.empty((B, S, H, hd), dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+    d = lib.AttnDesc()
+    d.B, d.H, d.S, d.hd, d.scale, d.causal, d.dtype = B, H, S, hd, 1.0 / math.sqrt(hd), int(causal), 1
+
+    def desc(t):
+        a = lib.AttnTensor()
+        a.ptr = t.data_ptr()
+        a.sb, a.ss, a.sh = t.stride(0), t.stride(1), t.stride(2)
+        return a
+
+    ts = [desc(t) for t in (q, k, v, o)]
+    lib.check(L.nbk_attention_fwd(C.byref(d), *[C.byref(t) for t in ts], C.c_void_p(lse.data_ptr()), st))
+    return o, lse, d, ts
+
+
+@pytest.mark.parametrize("shape", [(8, 1024, 16, 64), (4, 2048, 16, 128)])
+def test_attention_properties_at_full_size(hip, shape):
+    """Size-independent facts at the benchmark shapes, where a float64 reference is too slow:
+    probability rows sum to one (V = 1 gives O = 1 and dV = column sums of dO-weighted P),
+    causality (later keys and values do not reach earlier queries), linearity in V, and the
+    gradient identity sum(dQ * Q) = sum(dK * K) (scores are bilinear in Q and K)."""
+    from nabla_amd.backend import lib
+    B, S, H, hd = shape
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    rnd = lambda: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    q, k, v, v2, g = rnd(), rnd(), rnd(), rnd(), rnd()
+    print(f"attention properties {shape}", flush=True)
+    ones = torch.ones_like(v)
+    o1, lse, d, ts = _run_fwd(lib, L, st, q, k, ones, True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(lse).all()
+    assert (o1.float() - 1.0).abs().max().item() <= 2 ** -7          # rows of P sum to one
+    o, _, _, _ = _run_fwd(lib, L, st, q, k, v, True)
+    # causality: scramble the second half of K and V; the first half of the output must not move
+    k_mod, v_mod = k.clone(), v.clone()
+    k_mod[:, S // 2:] = rnd()[:, S // 2:]
+    v_mod[:, S // 2:] = rnd()[:, S // 2:]
+    o_mod, _, _, _ = _run_fwd(lib, L, st, q, k_mod, v_mod, True)
+    torch.cuda.synchronize()
+    assert torch.equal(o[:, :S // 2], o_mod[:, :S // 2])
+    assert not torch.equal(o[:, S // 2:], o_mod[:, S // 2:])
+    # linearity in V (same probabilities): O(v + v2) = O(v) + O(v2) up to bf16 rounding
+    o2, _, _, _ = _run_fwd(lib, L, st, q, k, v2, True)
+    o12, _, _, _ = _run_fwd(lib, L, st, q, k, (v.float() + v2.float()).to(torch.bfloat16), True)
+    torch.cuda.synchronize()
+    assert (o12.float() - (o.float() + o2.float())).abs().max().item() <= 0.06
+    # backward: sum(dQ * Q) = sum(dK * K) per (batch, head); both equal sum(dS * S)
+    dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+
+    def desc(t):
+        a = lib.AttnTensor()
+        a.ptr = t.data_ptr()
+        a.sb, a.ss, a.sh = t.stride(0), t.stride(1), t.stride(2)
+        return a
+
+    o, lse, d, ts = _run_fwd(lib, L, st, q, k, v, True)
+    ws = torch.empty(L.nbk_attention_bwd_workspace(C.byref(d)), dtype=torch.uint8, device="cuda")
+    extra = [desc(t) for t in (g, dq, dk, dv)]
+    lib.check(L.nbk_attention_bwd(C.byref(d), *[C.byref(t) for t in ts], C.c_void_p(lse.data_ptr()),
+                                  *[C.byref(t) for t in extra], C.c_void_p(ws.data_ptr()), ws.numel(), st))
+    torch.cuda.synchronize()
+    a = (dq.float() * q.float()).sum(dim=(1, 3))
+    b = (dk.float() * k.float()).sum(dim=(1, 3))
+    scale = (dq.float().abs() * q.float().abs()).sum(dim=(1, 3))
+    assert ((a - b).abs() <= 2e-2 * scale).all()
+    # dV = P^T dO: with dO = 1 its sum over keys is the number of queries (rows of P sum to one)
+    lib.check(L.nbk_attention_bwd(C.byref(d), *[C.byref(t) for t in ts], C.c_void_p(lse.data_ptr()),
+                                  C.byref(desc(torch.ones_like(g))), *[C.byref(t) for t in extra[1:]],
+                                  C.c_void_p(ws.data_ptr()), ws.numel(), st))
+    torch.cuda.synchronize()
+    total = dv.float().sum(dim=1)                                     # [B, H, hd]
+    assert (total - S).abs().max().item() <= 2e-2 * S
+
+
+def test_attention_strided_operands_from_different_buffers(hip):
+    """q, k, v as slices of one packed [B, S, 3, H, hd] projection, the output written into a
+    wider buffer: the strides the planner hands over inside multi-head attention."""
+    from nabla_amd.backend import lib
+    B, S, H, hd = 2, 256, 5, 64            # B * H = 10: not a multiple of the 8 XCDs
+    rng = np.random.default_rng(9)
+    packed = torch.tensor(rng.standard_normal((B, S, 3, H, hd)), dtype=torch.bfloat16)
+    want = _reference(*(packed[:, :, i].double() for i in range(3)), torch.zeros(B, S, H, hd).double(), True)[0]
+    pd = packed.cuda()
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    o, lse, _, _ = _run_fwd(lib, L, st, pd[:, :, 0], pd[:, :, 1], pd[:, :, 2], True)
+    torch.cuda.synchronize()
+    _close(o, want, "o from packed qkv")
