@@ -196,6 +196,29 @@ def fixture_c5():
 
 
 # ---------------------------------------------------------------- single kernels, awkward cases
+def fixture_attention_bf16():
+    """Causal attention on bfloat16 inputs (stored as their 16-bit patterns) with float64
+    results (stored as float16: the comparison tolerance for bf16 kernels is 2e-2): output,
+    log-sum-exp of the score rows and the three gradients for a given d(output).  This is the
+    shape class the fused attention kernels take (head size 64, S a multiple of 128)."""
+    rng = np.random.default_rng(6)
+    shape = (1, 1, 128, 64)                                    # [B, H, S, hd]
+    bits = {}
+    vals = {}
+    for name in ("q", "k", "v", "g"):
+        t = torch.tensor(rng.standard_normal(shape), dtype=torch.float32).to(torch.bfloat16)
+        bits[name] = t.view(torch.int16).numpy().view(np.uint16)
+        vals[name] = t.to(f64)
+    q, k, v = (vals[n].clone().requires_grad_(True) for n in ("q", "k", "v"))
+    o = attention(q, k, v, causal=True)
+    s = (q @ k.transpose(-2, -1)) / math.sqrt(shape[-1])
+    s = s.masked_fill(~(torch.tril(torch.ones(shape[-2], shape[-2])) > 0), float("-inf"))
+    dq, dk, dv = torch.autograd.grad(o, (q, k, v), vals["g"])
+    h = lambda t: t.detach().numpy().astype(np.float16)
+    save("attention_bf16", **{"in_" + n + "_bf16_bits": b for n, b in bits.items()},
+         o=h(o), lse=torch.logsumexp(s, -1).detach().numpy().astype(np.float32), dq=h(dq), dk=h(dk), dv=h(dv))
+
+
 def fixture_kernels():
     rng = np.random.default_rng(106)
     # conv2d with stride (2, 1) and asymmetric padding (tests/unit test_convolution.py:51-195 shapes)
@@ -238,3 +261,4 @@ if __name__ == "__main__":
     fixture_c4()
     fixture_c5()
     fixture_kernels()
+    fixture_attention_bf16()

@@ -153,3 +153,51 @@ def test_frontend_on_emulator_matches_golden(emulator):
 @pytest.mark.gpu
 def test_hip_matches_golden(hip):
     run_package(2e-5)
+
+
+# ---- bf16 causal attention (the fused kernels' shape class) -------------------------------------------
+def _attention_fixture():
+    import torch
+    z = load("attention_bf16")
+    ins = {n: torch.from_numpy(z[f"in_{n}_bf16_bits"].view(np.int16)).view(torch.bfloat16) for n in "qkvg"}
+    return z, ins
+
+
+def test_oracle_attention_matches_golden():
+    z, ins = _attention_fixture()
+    q, k, v = (O.V(ins[n].double().numpy()) for n in "qkv")
+    o = O.scaled_dot_product_attention(q, k, v, is_causal=True)
+    dq, dk, dv = O.grad_of(O.reduce_sum(o * O.V(ins["g"].double().numpy())), [q, k, v])
+    # the vectors are stored as float16: 2^-11 relative
+    for got, name in ((o.a, "o"), (dq, "dq"), (dk, "dk"), (dv, "dv")):
+        assert rel(got, z[name]) < 1e-3, name
+
+
+def _package_attention(tol):
+    z, ins = _attention_fixture()
+    bf = nb.DType.bfloat16
+    q, k, v, g = (nb.Tensor.from_dlpack(ins[n]) for n in "qkvg")
+    assert q.dtype is bf
+
+    def loss(q, k, v):
+        o = nb.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+        return nb.reduce_sum(nb.cast(o * g, nb.DType.float32))
+
+    o = nb.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+    grads = nb.grad(loss, argnums=(0, 1, 2))(q, k, v)
+    from nabla_amd.core.engine import _PLAN_CACHE
+    nb.realize_all(o, *grads)
+    assert any("attention_bwd" in b.plan.stats for b in _PLAN_CACHE.values())
+    f32 = lambda t: nb.cast(t, nb.DType.float32).numpy()
+    assert rel(f32(o), z["o"]) < tol
+    for got, name in zip(grads, ("dq", "dk", "dv")):
+        assert rel(f32(got), z[name]) < tol, name
+
+
+def test_frontend_attention_on_emulator_matches_golden(emulator):
+    _package_attention(2e-2)
+
+
+@pytest.mark.gpu
+def test_hip_attention_matches_golden(hip):
+    _package_attention(2e-2)
