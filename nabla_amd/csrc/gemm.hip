@@ -1,16 +1,18 @@
 // GEMM for gfx950: C[b] = alpha * A[b] @ B[b] (+bias) (act) (+residual).
 //
-// bf16 path (fp32 accumulate): v_mfma_f32_32x32x16_bf16.  A workgroup of four
-// waves (2 x 2; 128 x 128 tile) or eight (2 x 4; 256 x 256 tile) owns a BM x BN tile of C;
-// K advances in steps of 64 through two LDS buffers.  Both operands sit in LDS as [row][64 k] with 128-byte rows whose
-// eight 16-byte chunks are XOR-swizzled by (row % 8) ^ (row / 8 % 8), which makes
-// the 16-byte fragment reads of the MFMA (32 consecutive rows, one chunk) and
-// both kinds of tile writes below conflict-free without padding.
-//   * an operand that is contiguous along K is copied 16 bytes at a time;
-//   * an operand that is contiguous along its row index (the transposed operand
-//     of the two backward products, and B of the forward product) is read as
-//     8 x 8 blocks and transposed in registers before it is written, so the
-//     swap_axes of the backward GEMMs never touches memory.
+// bf16 path (fp32 accumulate): v_mfma_f32_32x32x16_bf16.  A workgroup of four waves (2 x 2;
+// 128 x 128 tile) or eight (2 x 4; 256 x 256 tile) owns a BM x BN tile of C; K advances in
+// steps of 64 through two LDS buffers.
+//   * an operand that is contiguous along K sits in LDS as [row][64 k], 128-byte rows whose
+//     eight 16-byte chunks are XOR-swizzled, so that the 16-byte fragment reads of the MFMA
+//     (32 consecutive rows, one chunk) are conflict-free without padding;
+//   * an operand that is contiguous along its row index (the transposed operand of the two
+//     backward products, and B of the forward product) sits in LDS k-major, [64 k][rows], and
+//     its MFMA fragments come out through the transposing read (ds_read_b64_tr_b16): the
+//     swap_axes of the backward GEMMs never touches memory or the vector ALU.
+// Two kernels share this layout idea: gemm_bf16_dl_kernel (aligned operands, K % 64 == 0) copies
+// global memory straight into LDS (global_load_lds_dwordx4); gemm_bf16_kernel takes every other
+// shape through guarded element-wise loads and registers.
 // fp32 path: v_mfma_f32_32x32x2f32 with a 128 x 128 x 16 tile, operands kept
 // k-major in LDS.
 #include "nbk_common.h"
@@ -100,24 +102,30 @@ __device__ __forceinline__ u32x4 ld8_bf16(const uint16_t* p, int64_t valid, bool
   return r;
 }
 
-// FAST loaders assume 16-byte-aligned operands, K % 64 == 0 and, for an operand
-// that is contiguous along its rows, a row count that is a multiple of 8; then
-// every access is one unconditional 16-byte load and the K loop has no branches.
-// Rows past the edge are clamped to the last valid row (their products are never
-// stored).  Everything else goes through the guarded element-wise path (FAST=false),
-// which is kept out of the hot kernels because its code size alone would push
-// the main loop out of the instruction cache.
-template <int ROWS, bool KC, bool FAST, int NT>
+// ------------------------------------------------------- bf16, guarded register-staged loads
+// The general form: any alignment, any K, ragged edges.  Every access is guarded element by
+// element; it is kept out of the hot kernel because its code size alone would push the main
+// loop out of the instruction cache.
+// LDS geometry of one operand tile, in 16-byte chunks.  K-contiguous: [row][8 chunks],
+// swizzled.  Row-contiguous: [64 k][ROWS / 8 + 4 chunks]; the pitch is 64 bytes past a
+// multiple of 256, so the eight 32-byte row segments that half a wave touches in one
+// transposing read (4 k-rows x 2 groups of 16 rows) fall on eight different bank groups.
+template <int ROWS, bool KC>
+struct TileGeom {
+  static constexpr int PITCH = ROWS / 8 + 4;
+  static constexpr int CHUNKS = KC ? ROWS * 8 : 64 * PITCH;
+};
+
+template <int ROWS, bool KC, int NT>
 struct TileLoader {
-  // NT lanes (256 or 512) share the tile.
-  // KC : operand contiguous along K    -> ROWS*8 chunk tasks, ROWS*8/NT per lane.
-  // !KC: operand contiguous along rows -> every lane transposes a KPT(k) x 8(rows) block:
-  //      one 8x8 block per lane for 256 rows on 256 lanes, half a block (4 k-values) when
-  //      there are twice as many lanes as blocks, so that all lanes take part and the K loop
-  //      has no divergent branch.
-  static constexpr int KPT = 8 * ROWS / NT;
-  static constexpr int NREG = KC ? ROWS * 8 / NT : KPT;
-  static_assert((ROWS == 256 || ROWS == 128) && (KPT == 8 || KPT == 4), "tile rows / lanes");
+  // NT lanes (256 or 512) share the tile: ROWS * 8 chunk tasks, ROWS * 8 / NT per lane.
+  // KC : operand contiguous along K    -> task t is chunk t % 8 of row t / 8.
+  // !KC: operand contiguous along rows -> task t is rows 8 * (t % (ROWS / 8)) .. + 8 of
+  //      k-row t / (ROWS / 8): consecutive lanes read consecutive 16 bytes of one k-row.
+  static constexpr int NREG = ROWS * 8 / NT;
+  static constexpr int NC = ROWS / 8;
+  static constexpr int PITCH = TileGeom<ROWS, KC>::PITCH;
+  static_assert(ROWS == 256 || ROWS == 128, "tile rows");
   u32x4 reg[NREG];
 
   __device__ __forceinline__ void load(const uint16_t* base, int64_t rs, int64_t cs, int64_t row0,
@@ -129,249 +137,89 @@ struct TileLoader {
         const int t = tid + s * NT;
         const int row = t >> 3, c = t & 7;
         const int64_t gr = row0 + row, gk = k0 + c * 8;
-        if (FAST) {
-          const int64_t r = gr < rows_total ? gr : rows_total - 1;
-          reg[s] = *(const u32x4*)(base + r * rs + gk);
-        } else {
-          if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
-          else reg[s] = (u32x4){0u, 0u, 0u, 0u};
-        }
+        if (gr < rows_total) reg[s] = ld8_bf16(base + gr * rs + gk, K - gk, vec);
+        else reg[s] = (u32x4){0u, 0u, 0u, 0u};
       }
     } else {
-      constexpr int NC = ROWS / 8;
-      const int nc = tid % NC, kq = tid / NC;  // kq: which KPT-row slice of the 64 k
-      const int64_t gr = row0 + nc * 8;
 #pragma unroll
-      for (int r = 0; r < KPT; ++r) {
-        const int64_t gk = k0 + kq * KPT + r;
-        if (FAST) {
-          const int64_t rr = gr < rows_total ? gr : rows_total - 8;
-          reg[r] = *(const u32x4*)(base + gk * cs + rr);
-        } else {
-          if (gk < K) reg[r] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
-          else reg[r] = (u32x4){0u, 0u, 0u, 0u};
-        }
+      for (int s = 0; s < NREG; ++s) {
+        const int t = tid + s * NT;
+        const int k = t / NC, c = t % NC;
+        const int64_t gr = row0 + c * 8, gk = k0 + k;
+        if (gk < K) reg[s] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
+        else reg[s] = (u32x4){0u, 0u, 0u, 0u};
       }
     }
   }
 
   // The tile goes to LDS in NPIECE independent pieces so that the K loop can place
   // them between its matrix instructions.
-  static constexpr int NPIECE = KC ? NREG : 8;
+  static constexpr int NPIECE = NREG;
   template <int P>
   __device__ __forceinline__ void store_piece(u32x4* lds) {
-    const int tid = threadIdx.x;
-    if (KC) {
-      const int t = tid + P * NT;
-      lds[swz(t >> 3, t & 7)] = reg[P];
-    } else {
-      constexpr int NC = ROWS / 8;
-      const int nc = tid % NC, kq = tid / NC;
-      // row P of the transpose of 16-bit elements: the lane's k-values of column P
-      constexpr uint32_t sel = (P & 1) ? 0x07060302u : 0x05040100u;
-      if (KPT == 8) {
-        u32x4 o;
-        o.x = __builtin_amdgcn_perm(reg[1][P >> 1], reg[0][P >> 1], sel);
-        o.y = __builtin_amdgcn_perm(reg[3][P >> 1], reg[2][P >> 1], sel);
-        o.z = __builtin_amdgcn_perm(reg[5 % NREG][P >> 1], reg[4 % NREG][P >> 1], sel);
-        o.w = __builtin_amdgcn_perm(reg[7 % NREG][P >> 1], reg[6 % NREG][P >> 1], sel);
-        lds[swz(nc * 8 + P, kq)] = o;
-      } else {
-        uint2 o;
-        o.x = __builtin_amdgcn_perm(reg[1][P >> 1], reg[0][P >> 1], sel);
-        o.y = __builtin_amdgcn_perm(reg[3][P >> 1], reg[2][P >> 1], sel);
-        uint2* dst = (uint2*)(lds + swz(nc * 8 + P, kq >> 1)) + (kq & 1);
-        *dst = o;
-      }
-    }
+    const int t = threadIdx.x + P * NT;
+    if (KC) lds[swz(t >> 3, t & 7)] = reg[P];
+    else lds[(t / NC) * PITCH + t % NC] = reg[P];
   }
   __device__ __forceinline__ void store(u32x4* lds) {
     static_for<NPIECE>([&](auto pc) { store_piece<decltype(pc)::value>(lds); });
   }
 };
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// Transposing LDS read: the 16 lanes of a group hand in 16 addresses of 4 consecutive
+// 16-bit values, In[p][e]; lane i of the group receives In[4 j + i / 4][i % 4], j = 0..3.
+// With lane p pointing at (k-row p / 4, rows 4 * (p % 4) .. + 4) of a k-major tile, lane i
+// ends up with 4 consecutive k of row i: half an MFMA operand fragment.
+__device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+}
+
+// The same read as inline assembly, for kernels that fill LDS with global_load_lds: the
+// compiler puts a wait for every such copy in flight in front of the intrinsic form (it cannot
+// tell that the two never touch the same buffer between two barriers).  It knows nothing about
+// the result being asynchronous either: lds_wait_for() has to stand between these reads and
+// the first use of their results.
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+__device__ __forceinline__ bf16x8 lds_read_tr_pair(uint32_t addr, int off_lo, int off_hi) {
+  s16x4 lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr), "n"(off_lo) : "memory");
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(off_hi) : "memory");
+  const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return *(const bf16x8*)&u;
+}
+__device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
+  u32x4 u;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(u) : "v"(addr) : "memory");
+  return *(const bf16x8*)&u;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_for(bf16x8 (&f)[N]) {
+  static_assert(N == 2 || N == 4 || N == 8, "fragments per set");
+  if constexpr (N == 2)
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1])::"memory");
+  else if constexpr (N == 4)
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3])::"memory");
+  else
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]),
+                   "+v"(f[7])::"memory");
+}
+
 extern __shared__ __align__(16) u32x4 gemm_lds[];
 
-// NW waves: 4 as 2 x 2, or 8 as 2 x 4 (two waves per SIMD, each with half the accumulators:
-// they cover each other's waits at the price of 1.5 x the LDS fragment traffic).
-template <int BM, int BN, bool A_KC, bool B_KC, bool FAST, bool EPI, int NW>
-__global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
-  constexpr int NT = NW * 64, WGN = NW / 2;
-  constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
-  constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int TILE_CHUNKS = (BM + BN) * 8;
-  int tm_i, tn_i;
-  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
-  const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
-  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
-  const uint16_t* A = (const uint16_t*)g.A + bo * g.a_bs + bi * g.a_bs2;
-  const uint16_t* B = (const uint16_t*)g.B + bo * g.b_bs + bi * g.b_bs2;
-  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
+// Epilogue shared by the bf16 kernels (the caller has passed a workgroup barrier: the tile
+// buffers are free).
+template <int TM, int TN, int WN, bool FAST, bool EPI>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
+                                              int64_t n0, int wm, int wn, int64_t c_off, int wave,
+                                              int lane) {
   const int li = lane & 31, kg = lane >> 5;
-
-  f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
-
-  TileLoader<BM, A_KC, FAST, NT> la;
-  TileLoader<BN, B_KC, FAST, NT> lb;
-  const int64_t nk = (g.K + 63) / 64;
-  // A is rows = m; for the loader a K-contiguous operand has (rs = row stride, k unit),
-  // a row-contiguous one has (cs = k stride, row unit).
-  la.load(A, g.a_rs, g.a_cs, m0, g.M, 0, g.K, g.a_vec);
-  lb.load(B, g.b_cs, g.b_rs, n0, g.N, 0, g.K, g.b_vec);
-  la.store(gemm_lds);
-  lb.store(gemm_lds + BM * 8);
-  __syncthreads();
-
-  // Fragment addresses.  swz(row, ks * 2 + kg) = (row * 8 | t) ^ (ks * 2) with
-  // t = kg ^ (row % 8) ^ (row / 8 % 8): only a constant XOR moves with ks.
-  int a_addr[TM], b_addr[TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int row = wm + i * 32 + li;
-    a_addr[i] = row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
-  }
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int row = wn + j * 32 + li;
-    b_addr[j] = BM * 8 + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
-  }
-
-  // Software pipeline.  A SIMD holds one or two waves of the tile, so little hides a
-  // stall but the wave's own instruction stream; every load is therefore issued one
-  // stage before its use and sits between matrix instructions:
-  //   * fragments of k-step ks + 1 are read from LDS while the MFMAs of ks run
-  //     (two fragment sets, frag[0] / frag[1]);
-  //   * the tile of iteration kt + 1, fetched from global memory during iteration
-  //     kt - 1, is written to the other LDS buffer during k-step 2;
-  //   * the global loads of tile kt + 2 are issued behind those writes;
-  //   * the workgroup barrier falls in the middle of k-step 3, whose remaining
-  //     MFMAs cover the first fragment reads of the next tile.
-  bf16x8 fa[2][TM], fb[2][TN];
-  constexpr int NFRAG = TM + TN, NMFMA = TM * TN;
-  // read fragment r (A tiles first, then B) of k-step ks from `tile` into set SET
-  auto read_frag = [&](auto set, auto r, const u32x4* tile, int ks) {
-    // order of use by the MFMAs (row-major over the wave's tiles): A0, every B, A1, A2 ...
-    constexpr int SET = decltype(set)::value, R0 = decltype(r)::value;
-    constexpr int R = R0 == 0 ? 0 : (R0 <= TN ? TM + R0 - 1 : R0 - TN);
-    // The XOR is recomputed at every read: hoisted out of the K loop, the 4 x (TM + TN)
-    // x 2 variants of these addresses would spill the accumulating kernel.
-    int sel = ks * 2;
-    asm volatile("" : "+s"(sel));
-    if constexpr (R < TM) {
-      const u32x4 u = tile[a_addr[R] ^ sel];
-      fa[SET][R] = *(const bf16x8*)&u;
-    } else {
-      const u32x4 u = tile[b_addr[R - TM] ^ sel];
-      fb[SET][R - TM] = *(const bf16x8*)&u;
-    }
-  };
-  auto mfma = [&](auto set, auto q) {
-    constexpr int SET = decltype(set)::value, Q = decltype(q)::value;
-    constexpr int i = Q / TN, j = Q % TN;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][i], fb[SET][j], acc[i][j], 0, 0, 0);
-  };
-  // k-step on fragment set SET while set 1 - SET is filled for k-step `ks_next` of `tile`
-  auto stage = [&](auto set, const u32x4* tile, int ks_next) {
-    constexpr int SET = decltype(set)::value;
-    static_for<NFRAG>([&](auto r) {
-      read_frag(std::integral_constant<int, 1 - SET>{}, r, tile, ks_next);
-    });
-    static_for<NMFMA>([&](auto q) { mfma(set, q); });
-    // interleave: one fragment read, then its share of the MFMAs
-    static_for<NFRAG>([&](auto r) {
-      constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);  // MFMAs
-    });
-    __builtin_amdgcn_sched_barrier(0);  // later stages' work (and its waits) stays behind
-  };
-
-  static_for<NFRAG>([&](auto r) { read_frag(std::integral_constant<int, 0>{}, r, gemm_lds, 0); });
-  {
-    const int64_t k1 = nk > 1 ? 64 : 0;  // a single-tile problem re-reads tile 0 (never stored)
-    la.load(A, g.a_rs, g.a_cs, m0, g.M, k1, g.K, g.a_vec);
-    lb.load(B, g.b_cs, g.b_rs, n0, g.N, k1, g.K, g.b_vec);
-  }
-  using S0 = std::integral_constant<int, 0>;
-  using S1 = std::integral_constant<int, 1>;
-  for (int64_t kt = 0; kt + 1 < nk; ++kt) {
-    const u32x4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
-    u32x4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
-    stage(S0{}, cur, 1);
-    stage(S1{}, cur, 2);
-    // k-step 2, with tile kt + 1 going from registers to LDS
-    // (LDS reads and writes keep their program order, so they alternate in the source)
-    {
-      using LA = TileLoader<BM, A_KC, FAST, NT>;
-      using LB = TileLoader<BN, B_KC, FAST, NT>;
-      constexpr int NPA = LA::NPIECE, NP = LA::NPIECE + LB::NPIECE;
-      constexpr int PER = (NP + NFRAG - 1) / NFRAG;
-      static_for<NFRAG>([&](auto r) {
-        read_frag(S1{}, r, cur, 3);
-        static_for<PER>([&](auto e) {
-          constexpr int P = decltype(r)::value * PER + decltype(e)::value;
-          if constexpr (P < NPA) la.template store_piece<P>(nxt);
-          else if constexpr (P < NP) lb.template store_piece<P - NPA>(nxt + BM * 8);
-        });
-      });
-      static_for<NMFMA>([&](auto q) { mfma(S0{}, q); });
-      static_for<NFRAG>([&](auto r) {
-        constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x200, PER, 0);  // DS writes
-        if constexpr (n > 1) __builtin_amdgcn_sched_group_barrier(0x008, n - 1, 0);  // MFMA
-      });
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // k-step 3: fetch tile kt + 2 (the last iteration re-fetches tile nk - 1, unused),
-    // half of the MFMAs, barrier, first fragments of the next tile, the other half
-    {
-      const int64_t k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * 64;
-      la.load(A, g.a_rs, g.a_cs, m0, g.M, k2, g.K, g.a_vec);
-      lb.load(B, g.b_cs, g.b_rs, n0, g.N, k2, g.K, g.b_vec);
-    }
-    static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
-    {
-      constexpr int NL = TileLoader<BM, A_KC, FAST, NT>::NREG + TileLoader<BN, B_KC, FAST, NT>::NREG;
-      static_for<NMFMA / 2>([&](auto q) {
-        constexpr int n = share(NL, NMFMA / 2, decltype(q)::value);
-        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);  // VMEM reads
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      });
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<NFRAG>([&](auto r) { read_frag(S0{}, r, nxt, 0); });
-    static_for<NMFMA / 2>([&](auto q) {
-      mfma(S1{}, std::integral_constant<int, decltype(q)::value + NMFMA / 2>{});
-    });
-    static_for<NFRAG>([&](auto r) {
-      constexpr int n = share(NMFMA / 2, NFRAG, decltype(r)::value);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);
-    });
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  {
-    // last tile: nothing left to stage
-    const u32x4* cur = gemm_lds + ((nk - 1) & 1) * TILE_CHUNKS;
-    stage(S0{}, cur, 1);
-    stage(S1{}, cur, 2);
-    stage(S0{}, cur, 3);
-    static_for<NMFMA>([&](auto q) { mfma(S1{}, q); });
-  }
-  __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
-
   // Epilogue.  D[i][j] of a 32x32 MFMA tile lives in lane (j, (i / 4) % 2),
   // register (i / 8) * 4 + i % 4.  Each wave passes its accumulators through a
   // private LDS slab, 32 rows at a time, so that C is written as whole
@@ -451,6 +299,484 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next tile row overwrites it
   });
+}
+
+// NW waves: 4 as 2 x 2, or 8 as 2 x 4 (two waves per SIMD, each with half the accumulators:
+// they cover each other's waits at the price of 1.5 x the LDS fragment traffic).
+template <int BM, int BN, bool A_KC, bool B_KC, bool EPI, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
+  constexpr int NT = NW * 64, WGN = NW / 2;
+  constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int CA = TileGeom<BM, A_KC>::CHUNKS, CB = TileGeom<BN, B_KC>::CHUNKS;
+  constexpr int TILE_CHUNKS = CA + CB;
+  constexpr int PA = TileGeom<BM, A_KC>::PITCH * 16, PB = TileGeom<BN, B_KC>::PITCH * 16;  // bytes
+  int tm_i, tn_i;
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
+  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
+  const uint16_t* A = (const uint16_t*)g.A + bo * g.a_bs + bi * g.a_bs2;
+  const uint16_t* B = (const uint16_t*)g.B + bo * g.b_bs + bi * g.b_bs2;
+  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
+  const int li = lane & 31, kg = lane >> 5;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
+
+  TileLoader<BM, A_KC, NT> la;
+  TileLoader<BN, B_KC, NT> lb;
+  const int64_t nk = (g.K + 63) / 64;
+  // A is rows = m; for the loader a K-contiguous operand has (rs = row stride, k unit),
+  // a row-contiguous one has (cs = k stride, row unit).
+  la.load(A, g.a_rs, g.a_cs, m0, g.M, 0, g.K, g.a_vec);
+  lb.load(B, g.b_cs, g.b_rs, n0, g.N, 0, g.K, g.b_vec);
+  la.store(gemm_lds);
+  lb.store(gemm_lds + CA);
+  __syncthreads();
+
+  // Fragment addresses.  swz(row, ks * 2 + kg) = (row * 8 | t) ^ (ks * 2) with
+  // t = kg ^ (row % 8) ^ (row / 8 % 8): only a constant XOR moves with ks.
+  // A k-major operand needs one byte offset per wave: lane p of group q = lane / 16 points at
+  // k-row 8 * (q / 2) + p / 4, rows 16 * (q % 2) + 4 * (p % 4) of the wave's first tile; the
+  // tile row, the k-step and the second half of the fragment are constant offsets.
+  int a_addr[TM], b_addr[TN];
+  const int tr_k = 8 * (lane >> 5) + ((lane & 15) >> 2), tr_r = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int a_tr = tr_k * PA + (wm + tr_r) * 2, b_tr = CA * 16 + tr_k * PB + (wn + tr_r) * 2;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int row = wm + i * 32 + li;
+    a_addr[i] = row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int row = wn + j * 32 + li;
+    b_addr[j] = CA + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 7));
+  }
+
+  // Software pipeline.  A SIMD holds one or two waves of the tile, so little hides a
+  // stall but the wave's own instruction stream; every load is therefore issued one
+  // stage before its use and sits between matrix instructions:
+  //   * fragments of k-step ks + 1 are read from LDS while the MFMAs of ks run
+  //     (two fragment sets, frag[0] / frag[1]);
+  //   * the tile of iteration kt + 1, fetched from global memory during iteration
+  //     kt - 1, is written to the other LDS buffer during k-step 2;
+  //   * the global loads of tile kt + 2 are issued behind those writes;
+  //   * the workgroup barrier falls in the middle of k-step 3, whose remaining
+  //     MFMAs cover the first fragment reads of the next tile.
+  bf16x8 fa[2][TM], fb[2][TN];
+  constexpr int NFRAG = TM + TN, NMFMA = TM * TN;
+  // read fragment r (A tiles first, then B) of k-step ks from `tile` into set SET
+  auto read_frag = [&](auto set, auto r, const u32x4* tile, int ks) {
+    // order of use by the MFMAs (row-major over the wave's tiles): A0, every B, A1, A2 ...
+    constexpr int SET = decltype(set)::value, R0 = decltype(r)::value;
+    constexpr int R = R0 == 0 ? 0 : (R0 <= TN ? TM + R0 - 1 : R0 - TN);
+    // The XOR is recomputed at every read: hoisted out of the K loop, the 4 x (TM + TN)
+    // x 2 variants of these addresses would spill the accumulating kernel.
+    int sel = ks * 2;
+    asm volatile("" : "+s"(sel));
+    if constexpr (R < TM) {
+      if constexpr (A_KC) {
+        const u32x4 u = tile[a_addr[R] ^ sel];
+        fa[SET][R] = *(const bf16x8*)&u;
+      } else {
+        const char* p = (const char*)tile + a_tr + (R * 64 + ks * 16 * PA);
+        const s16x4 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * PA);
+        const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        fa[SET][R] = *(const bf16x8*)&u;
+      }
+    } else {
+      if constexpr (B_KC) {
+        const u32x4 u = tile[b_addr[R - TM] ^ sel];
+        fb[SET][R - TM] = *(const bf16x8*)&u;
+      } else {
+        const char* p = (const char*)tile + b_tr + ((R - TM) * 64 + ks * 16 * PB);
+        const s16x4 lo = lds_read_tr(p), hi = lds_read_tr(p + 4 * PB);
+        const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        fb[SET][R - TM] = *(const bf16x8*)&u;
+      }
+    }
+  };
+  // LDS read instructions of fragment r in the order above: a k-major operand takes two
+  auto frag_reads = [](int r0) constexpr {
+    const int r = r0 == 0 ? 0 : (r0 <= TN ? TM + r0 - 1 : r0 - TN);
+    return r < TM ? (A_KC ? 1 : 2) : (B_KC ? 1 : 2);
+  };
+  auto mfma = [&](auto set, auto q) {
+    constexpr int SET = decltype(set)::value, Q = decltype(q)::value;
+    constexpr int i = Q / TN, j = Q % TN;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][i], fb[SET][j], acc[i][j], 0, 0, 0);
+  };
+  // k-step on fragment set SET while set 1 - SET is filled for k-step `ks_next` of `tile`
+  auto stage = [&](auto set, const u32x4* tile, int ks_next) {
+    constexpr int SET = decltype(set)::value;
+    static_for<NFRAG>([&](auto r) {
+      read_frag(std::integral_constant<int, 1 - SET>{}, r, tile, ks_next);
+    });
+    static_for<NMFMA>([&](auto q) { mfma(set, q); });
+    // interleave: one fragment read, then its share of the MFMAs
+    static_for<NFRAG>([&](auto r) {
+      constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
+      __builtin_amdgcn_sched_group_barrier(0x100, frag_reads(decltype(r)::value), 0);  // DS read
+      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);  // MFMAs
+    });
+    __builtin_amdgcn_sched_barrier(0);  // later stages' work (and its waits) stays behind
+  };
+
+  static_for<NFRAG>([&](auto r) { read_frag(std::integral_constant<int, 0>{}, r, gemm_lds, 0); });
+  {
+    const int64_t k1 = nk > 1 ? 64 : 0;  // a single-tile problem re-reads tile 0 (never stored)
+    la.load(A, g.a_rs, g.a_cs, m0, g.M, k1, g.K, g.a_vec);
+    lb.load(B, g.b_cs, g.b_rs, n0, g.N, k1, g.K, g.b_vec);
+  }
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  for (int64_t kt = 0; kt + 1 < nk; ++kt) {
+    const u32x4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
+    u32x4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
+    stage(S0{}, cur, 1);
+    stage(S1{}, cur, 2);
+    // k-step 2, with tile kt + 1 going from registers to LDS
+    // (LDS reads and writes keep their program order, so they alternate in the source)
+    {
+      using LA = TileLoader<BM, A_KC, NT>;
+      using LB = TileLoader<BN, B_KC, NT>;
+      constexpr int NPA = LA::NPIECE, NP = LA::NPIECE + LB::NPIECE;
+      constexpr int PER = (NP + NFRAG - 1) / NFRAG;
+      static_for<NFRAG>([&](auto r) {
+        read_frag(S1{}, r, cur, 3);
+        static_for<PER>([&](auto e) {
+          constexpr int P = decltype(r)::value * PER + decltype(e)::value;
+          if constexpr (P < NPA) la.template store_piece<P>(nxt);
+          else if constexpr (P < NP) lb.template store_piece<P - NPA>(nxt + CA);
+        });
+      });
+      static_for<NMFMA>([&](auto q) { mfma(S0{}, q); });
+      static_for<NFRAG>([&](auto r) {
+        constexpr int n = share(NMFMA, NFRAG, decltype(r)::value);
+        __builtin_amdgcn_sched_group_barrier(0x100, frag_reads(decltype(r)::value), 0);  // DS read
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x200, PER, 0);  // DS writes
+        if constexpr (n > 1) __builtin_amdgcn_sched_group_barrier(0x008, n - 1, 0);  // MFMA
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 3: fetch tile kt + 2 (the last iteration re-fetches tile nk - 1, unused),
+    // half of the MFMAs, barrier, first fragments of the next tile, the other half
+    {
+      const int64_t k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * 64;
+      la.load(A, g.a_rs, g.a_cs, m0, g.M, k2, g.K, g.a_vec);
+      lb.load(B, g.b_cs, g.b_rs, n0, g.N, k2, g.K, g.b_vec);
+    }
+    static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
+    {
+      constexpr int NL = TileLoader<BM, A_KC, NT>::NREG + TileLoader<BN, B_KC, NT>::NREG;
+      static_for<NMFMA / 2>([&](auto q) {
+        constexpr int n = share(NL, NMFMA / 2, decltype(q)::value);
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);  // VMEM reads
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NFRAG>([&](auto r) { read_frag(S0{}, r, nxt, 0); });
+    static_for<NMFMA / 2>([&](auto q) {
+      mfma(S1{}, std::integral_constant<int, decltype(q)::value + NMFMA / 2>{});
+    });
+    static_for<NFRAG>([&](auto r) {
+      constexpr int n = share(NMFMA / 2, NFRAG, decltype(r)::value);
+      __builtin_amdgcn_sched_group_barrier(0x100, frag_reads(decltype(r)::value), 0);
+      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x008, n, 0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    // last tile: nothing left to stage
+    const u32x4* cur = gemm_lds + ((nk - 1) & 1) * TILE_CHUNKS;
+    stage(S0{}, cur, 1);
+    stage(S1{}, cur, 2);
+    stage(S0{}, cur, 3);
+    static_for<NMFMA>([&](auto q) { mfma(S1{}, q); });
+  }
+  __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
+
+  gemm_epilogue<TM, TN, WN, false, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
+}
+
+// ------------------------------------------------------------- bf16, direct-to-LDS loads
+// The hot form (16-byte-aligned operands, K % 64 == 0): tiles go from global memory into LDS
+// without passing through registers (global_load_lds_dwordx4: lane l of a wave deposits its
+// 16 bytes at a wave-uniform LDS base + 16 l), so that the fragment reads are the only LDS
+// instructions of the K loop and the lanes hold no staging registers.  Because the LDS side
+// of such a load is linear in the lane, both layouts are unpadded and XOR-swizzled, and the
+// swizzle is applied to the global address each lane fetches from:
+//   K-contiguous operand   [row][8 chunks]: chunk c of row r sits at c ^ (r % 8) ^ (r / 8 % 2);
+//   row-contiguous operand [64 k][ROWS / 8 chunks]: chunk c of k-row k sits at
+//     c ^ 2 * T[k % 4], T = {0, 3, 6, 5}, which sends the eight 32-byte segments that half a
+//     wave touches in one transposing read to eight different bank groups.
+__device__ __forceinline__ int dl_swz_kc(int row, int c) {
+  return row * 8 + (c ^ (row & 7) ^ ((row >> 3) & 1));
+}
+__device__ __forceinline__ int dl_seg_xor(int k) { return (k & 3) ^ (((k & 3) << 1) & 7); }
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glb_void_t;
+
+template <int ROWS, bool KC, int NW>
+struct DirectLoader {
+  // ROWS * 8 chunks, 64 per wave instruction, dealt to the waves in consecutive runs
+  static constexpr int N = ROWS / (8 * NW);
+  static constexpr int NC = ROWS / 8;
+  static_assert(N >= 1 && N % 2 == 0, "instructions per wave");
+  int voff[N];         // byte offset of this lane's chunk from the tile's first element
+  const char* base;    // operand + tile row offset (wave-uniform)
+  int64_t kstep;       // bytes between consecutive K tiles (wave-uniform)
+  int first;           // first instruction of this wave
+
+  __device__ __forceinline__ void init(const uint16_t* op, int64_t rs, int64_t cs, int64_t row0,
+                                       int64_t rows_total, int wave, int lane) {
+    first = wave * N;
+    if (KC) {
+      base = (const char*)(op + row0 * rs);
+      kstep = 128;
+      const int64_t last = rows_total - 1 - row0;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const int row = (first + j) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ (row & 7) ^ ((row >> 3) & 1);
+        const int64_t r = row < last ? row : last;
+        voff[j] = (int)(r * rs * 2 + c * 16);
+      }
+    } else {
+      base = (const char*)(op + row0);
+      kstep = 128 * cs;
+      const int64_t last = rows_total - 8 - row0;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const int l = (first + j) * 64 + lane;
+        const int k = l / NC, c = (l % NC) ^ (dl_seg_xor(k) << 1);
+        const int64_t r = c * 8 < last ? c * 8 : last;
+        voff[j] = (int)(k * cs * 2 + r * 2);
+      }
+    }
+  }
+  // start the copy of K tile `kt` into `region` (this operand's part of a tile buffer)
+  __device__ __forceinline__ const char* tile_src(int64_t kt) const { return base + kt * kstep; }
+  template <int J>
+  __device__ __forceinline__ void issue_one(u32x4* region, const char* src) const {
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(src + voff[J]),
+                                     (lds_void_t*)(region + (first + J) * 64), 16, 0, 0);
+  }
+  __device__ __forceinline__ void issue(u32x4* region, int64_t kt) const {
+    const char* src = tile_src(kt);
+    static_for<N>([&](auto j) { issue_one<decltype(j)::value>(region, src); });
+  }
+};
+
+// KSS: k-steps (of 16) per fragment set.  A step of KSS k-steps is multiplied out of one
+// set while the other is filled for the next step; small wave tiles take 2, so that a read has
+// more than a handful of MFMAs to land.
+template <int BM, int BN, bool A_KC, bool B_KC, bool EPI, int NW, int KSS>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g) {
+  constexpr int WGN = NW / 2;
+  constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int CA = BM * 8, TILE_CHUNKS = (BM + BN) * 8;
+  int tm_i, tn_i;
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
+  const int64_t bo = (int64_t)blockIdx.y / g.batch_inner, bi = (int64_t)blockIdx.y % g.batch_inner;
+  const uint16_t* A = (const uint16_t*)g.A + bo * g.a_bs + bi * g.a_bs2;
+  const uint16_t* B = (const uint16_t*)g.B + bo * g.b_bs + bi * g.b_bs2;
+  const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
+  const int li = lane & 31, kg = lane >> 5;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
+
+  DirectLoader<BM, A_KC, NW> la;
+  DirectLoader<BN, B_KC, NW> lb;
+  la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
+  lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
+  const int64_t nk = g.K / 64;
+  la.issue(gemm_lds, 0);
+  lb.issue(gemm_lds + CA, 0);
+
+  // Fragment addresses, one per 32-row block of the wave tile.
+  //   K-contiguous: byte address 16 ((row * 8 | t) ^ (2 ks)), t = kg ^ (row % 8) ^ (row / 8 % 2);
+  //   row-contiguous: byte address of this lane's 8 bytes in the transposing read of k-step 0,
+  //     first half; the k-step and the half are constant offsets.  Lane p of group q = lane / 16
+  //     points at k-row 8 (q / 2) + p / 4, rows 16 (q % 2) + 4 (p % 4) .. + 4 of the block.
+  int a_addr[TM], b_addr[TN];
+  {
+    const int p = lane & 15, q = lane >> 4;
+    const int kl = 8 * (q >> 1) + (p >> 2), sx = dl_seg_xor(p >> 2);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm + i * 32 + li;
+      if (A_KC) a_addr[i] = (row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
+      else a_addr[i] = kl * (BM * 2) + ((((wm >> 4) + 2 * i + (q & 1)) ^ sx) * 32) + 8 * (p & 3);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn + j * 32 + li;
+      if (B_KC) b_addr[j] = (CA + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
+      else b_addr[j] = CA * 16 + kl * (BN * 2) + ((((wn >> 4) + 2 * j + (q & 1)) ^ sx) * 32) + 8 * (p & 3);
+    }
+  }
+
+  bf16x8 fa[2][KSS * TM], fb[2][KSS * TN];
+  constexpr int NSTEP = 4 / KSS;
+  constexpr int NFRAG = KSS * (TM + TN), NMFMA = KSS * TM * TN;  // per step
+  // read fragment r of step `step` from `tile` into set SET; order of use by the MFMAs
+  // (k-step by k-step, row-major over the wave's blocks): A0, every B, A1, A2 ...
+  auto read_frag = [&](auto set, auto r, const u32x4* tile, int step) {
+    constexpr int SET = decltype(set)::value;
+    constexpr int KL = decltype(r)::value / (TM + TN), R0 = decltype(r)::value % (TM + TN);
+    constexpr int R = R0 == 0 ? 0 : (R0 <= TN ? TM + R0 - 1 : R0 - TN);
+    const int ks = step * KSS + KL;
+    if constexpr (R < TM) {
+      if constexpr (A_KC) {
+        int sel = ks * 32;
+        asm volatile("" : "+s"(sel));  // recomputed at every read: hoisted variants would spill
+        fa[SET][KL * TM + R] = lds_read_b128(lds_addr(tile) + (a_addr[R] ^ sel));
+      } else {
+        const uint32_t p = lds_addr(tile) + a_addr[R];
+        fa[SET][KL * TM + R] = lds_read_tr_pair(p, ks * 16 * (BM * 2), (ks * 16 + 4) * (BM * 2));
+      }
+    } else {
+      if constexpr (B_KC) {
+        int sel = ks * 32;
+        asm volatile("" : "+s"(sel));
+        fb[SET][KL * TN + R - TM] = lds_read_b128(lds_addr(tile) + (b_addr[R - TM] ^ sel));
+      } else {
+        const uint32_t p = lds_addr(tile) + b_addr[R - TM];
+        fb[SET][KL * TN + R - TM] = lds_read_tr_pair(p, ks * 16 * (BN * 2), (ks * 16 + 4) * (BN * 2));
+      }
+    }
+  };
+  // The compiler does not see the fragment reads (inline assembly): before the MFMAs of a
+  // k-step may touch a fragment set, wait for LDS by hand, with the set's registers as
+  // operands of the wait so that no MFMA can be moved in front of it.
+  auto frags_ready = [&](auto set) {
+    constexpr int SET = decltype(set)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    lds_wait_for(fa[SET]);
+    lds_wait_for(fb[SET]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto mfma = [&](auto set, auto q) {
+    constexpr int SET = decltype(set)::value, Q = decltype(q)::value;
+    constexpr int kl = Q / (TM * TN), i = Q % (TM * TN) / TN, j = Q % TN;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kl * TM + i], fb[SET][kl * TN + j],
+                                                        acc[i][j], 0, 0, 0);
+  };
+  // step on fragment set SET while set 1 - SET is filled for step `step_next` of `tile`
+  auto stage = [&](auto set, const u32x4* tile, int step_next) {
+    constexpr int SET = decltype(set)::value;
+    frags_ready(set);
+    // the reads go out between the MFMAs of the first half (pinned: the scheduler would batch
+    // them), so that they have the second half to land
+    constexpr int SPREAD = NMFMA / 2;
+    static_for<NMFMA>([&](auto q) {
+      constexpr int Q = decltype(q)::value;
+      static_for<NFRAG>([&](auto r) {
+        if constexpr (decltype(r)::value * SPREAD / NFRAG == Q)
+          read_frag(std::integral_constant<int, 1 - SET>{}, r, tile, step_next);
+      });
+      mfma(set, q);
+      if constexpr (Q < SPREAD) __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  // a workgroup barrier behind which every wave's copies have landed
+  auto tile_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's copies are in LDS
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // Two tile buffers.  Tile kt + 1 is on its way while tile kt is multiplied; the barrier that
+  // ends tile kt (in the middle of its last step, whose fragments are in registers by then)
+  // frees its buffer for tile kt + 2, whose copies are started right behind that barrier and
+  // have the whole of tile kt + 1 to land.
+  tile_barrier();
+  static_for<NFRAG>([&](auto r) { read_frag(S0{}, r, gemm_lds, 0); });
+  if (nk > 1) {
+    la.issue(gemm_lds + TILE_CHUNKS, 1);
+    lb.issue(gemm_lds + TILE_CHUNKS + CA, 1);
+  }
+  for (int64_t kt = 0; kt + 1 < nk; ++kt) {
+    u32x4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
+    const u32x4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
+    static_for<NSTEP - 1>([&](auto st) {
+      constexpr int ST = decltype(st)::value;
+      stage(std::integral_constant<int, ST & 1>{}, cur, ST + 1);
+    });
+    frags_ready(S1{});  // the last step (NSTEP is even) is on set 1
+    static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
+    tile_barrier();
+    {
+      // Behind the barrier: the first fragments of tile kt + 1, the copies of tile kt + 2 and
+      // the second half of the MFMAs, dealt out evenly and pinned in this order (the copies
+      // and the reads both touch LDS, so the scheduler would otherwise leave the MFMAs last).
+      // (the last pass has no tile kt + 2: it fetches tile nk - 1 again, into a buffer that
+      // is not read any more, which keeps this block free of branches)
+      using LA = DirectLoader<BM, A_KC, NW>;
+      using LB = DirectLoader<BN, B_KC, NW>;
+      constexpr int NL = LA::N + LB::N, H = NMFMA / 2;
+      const int64_t k2 = kt + 2 < nk ? kt + 2 : nk - 1;
+      const char* src_a = la.tile_src(k2);
+      const char* src_b = lb.tile_src(k2);
+      static_for<H>([&](auto q) {
+        constexpr int Q = decltype(q)::value;
+        static_for<NFRAG>([&](auto r) {
+          constexpr int R = decltype(r)::value;
+          if constexpr (R >= NFRAG * Q / H && R < NFRAG * (Q + 1) / H) read_frag(S0{}, r, nxt, 0);
+        });
+        static_for<NL>([&](auto l) {
+          constexpr int L = decltype(l)::value;
+          if constexpr (L >= NL * Q / H && L < NL * (Q + 1) / H) {
+            if constexpr (L < LA::N) la.template issue_one<L>(cur, src_a);
+            else lb.template issue_one<L - LA::N>(cur + CA, src_b);
+          }
+        });
+        mfma(S1{}, std::integral_constant<int, Q + H>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    const u32x4* cur = gemm_lds + ((nk - 1) & 1) * TILE_CHUNKS;
+    static_for<NSTEP - 1>([&](auto st) {
+      constexpr int ST = decltype(st)::value;
+      stage(std::integral_constant<int, ST & 1>{}, cur, ST + 1);
+    });
+    frags_ready(S1{});
+    static_for<NMFMA>([&](auto q) { mfma(S1{}, q); });
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no copy may land in a slab
+  __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
+  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
 }
 
 // ---------------------------------------------------------------------------- fp32
@@ -663,13 +989,18 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const GemmArgs g) {
 }
 
 // ------------------------------------------------------------------------- dispatch
-template <int BM, int BN, bool FAST, int NW = 4>
+template <int BM, int BN, int NW = 4>
 static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
   GemmArgs g = a;
   g.tiles_m = (int)((a.M + BM - 1) / BM);
   g.tiles_n = (int)((a.N + BN - 1) / BN);
   dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
-  const size_t pipe = 2 * (size_t)(BM + BN) * 8 * sizeof(uint4);
+  const size_t pipe_of[2][2] = {
+      {2 * (size_t)(TileGeom<BM, false>::CHUNKS + TileGeom<BN, false>::CHUNKS) * 16,
+       2 * (size_t)(TileGeom<BM, false>::CHUNKS + TileGeom<BN, true>::CHUNKS) * 16},
+      {2 * (size_t)(TileGeom<BM, true>::CHUNKS + TileGeom<BN, false>::CHUNKS) * 16,
+       2 * (size_t)(TileGeom<BM, true>::CHUNKS + TileGeom<BN, true>::CHUNKS) * 16}};
+  const size_t pipe = pipe_of[akc][bkc];
   const size_t slabs = NW * 32 * (size_t)(BN / (NW / 2) + 4) * sizeof(float);
   const size_t lds = pipe > slabs ? pipe : slabs;
   const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
@@ -680,7 +1011,7 @@ static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hip
   } while (0)
 #define NBK_LAUNCH_BF16_E(AK, BK_, EP)                                                        \
   do {                                                                                        \
-    auto kern = gemm_bf16_kernel<BM, BN, AK, BK_, FAST, EP, NW>;                              \
+    auto kern = gemm_bf16_kernel<BM, BN, AK, BK_, EP, NW>;                              \
     static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
     if (!attr_set) {                                                                          \
       NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -696,6 +1027,41 @@ static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hip
 #undef NBK_LAUNCH_BF16
 #undef NBK_LAUNCH_BF16_E
   return nbk_check_launch("gemm_bf16_kernel");
+}
+
+template <int BM, int BN, int NW, int KSS>
+static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
+  GemmArgs g = a;
+  g.tiles_m = (int)((a.M + BM - 1) / BM);
+  g.tiles_n = (int)((a.N + BN - 1) / BN);
+  dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
+  const size_t pipe = 2 * (size_t)(BM + BN) * 8 * 16;
+  const size_t slabs = NW * 32 * (size_t)(BN / (NW / 2) + 4) * sizeof(float);
+  const size_t lds = pipe > slabs ? pipe : slabs;
+  const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
+#define NBK_LAUNCH_DL(AK, BK_, EP)                                                            \
+  do {                                                                                        \
+    auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS>;                                 \
+    static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
+    if (!attr_set) {                                                                          \
+      NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                  (int)lds));                                                 \
+      attr_set = true;                                                                        \
+    }                                                                                         \
+    hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, st, g);                                \
+  } while (0)
+#define NBK_LAUNCH_DL2(AK, BK_)                                                               \
+  do {                                                                                        \
+    if (epi) NBK_LAUNCH_DL(AK, BK_, true);                                                    \
+    else NBK_LAUNCH_DL(AK, BK_, false);                                                       \
+  } while (0)
+  if (akc && bkc) NBK_LAUNCH_DL2(true, true);
+  else if (akc && !bkc) NBK_LAUNCH_DL2(true, false);
+  else if (!akc && bkc) NBK_LAUNCH_DL2(false, true);
+  else NBK_LAUNCH_DL2(false, false);
+#undef NBK_LAUNCH_DL
+#undef NBK_LAUNCH_DL2
+  return nbk_check_launch("gemm_bf16_dl_kernel");
 }
 
 extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
@@ -743,7 +1109,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   if (d->dtype_ab == NBK_BF16) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
-    if (!fast) return launch_bf16<128, 128, false>(a, akc, bkc, d->batch, st);
+    if (!fast) return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);
     // 256 x 256 tiles run at about twice the rate of 128 x 128 ones per CU, one workgroup
     // per CU at a time: take them when the rounds of workgroups they need are at least
     // 60 % full (256 tiles on 256 CUs is the ideal case, 128 or 300 tiles are not).
@@ -754,11 +1120,11 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     // 128 x 128 workgroups per CU overlap better than one 256 x 256)
     // (eight waves on the big tile: 8-16 % faster than four on every shape measured)
     if (big_tiles * 10 >= rounds * cus * 6 && d->M >= 256 && d->N >= 256 && d->K > 128)
-      return launch_bf16<256, 256, true, 8>(a, akc, bkc, d->batch, st);
+      return launch_bf16_dl<256, 256, 8, 2>(a, akc, bkc, d->batch, st);
     // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
     // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
     // 128 x 128 workgroups hide it better)
-    return launch_bf16<128, 128, true>(a, akc, bkc, d->batch, st);
+    return launch_bf16_dl<128, 128, 4, 1>(a, akc, bkc, d->batch, st);
   }
   a.tiles_m = (int)((d->M + 127) / 128);
   a.tiles_n = (int)((d->N + 127) / 128);

@@ -210,10 +210,14 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* __restrict_
 template <typename T, int VEC>
 __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, void* __restrict__ out,
                                                     int dto, int64_t red, int64_t inner, int kind,
-                                                    int64_t bx, int64_t o) {
+                                                    int64_t bx, int64_t o, int wc) {
+  // The four waves stand wc (1, 2 or 4) side by side along the row and 4 / wc deep along the
+  // reduced axis: a wide row is read in long contiguous runs, and a short reduced axis (the
+  // partial sums of a split product) still keeps every wave busy.
   __shared__ float part[4][64][VEC + 1];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int64_t col = (bx * 64 + lane) * VEC;
+  const int wcid = w % wc, wr = w / wc, WR = 4 / wc;
+  const int64_t col = ((bx * wc + wcid) * 64 + lane) * VEC;
   const float ident = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
   float acc[VEC];
 #pragma unroll
@@ -232,11 +236,11 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
       }
     };
     auto load = [&](int64_t r, float* v) { unpack(*(const uint4*)(base + r * inner), v); };
-    int64_t r = w;
-    for (; r + 60 < red; r += 64) {  // sixteen rows in flight, kept packed until they are added
+    int64_t r = wr;
+    for (; r + 15 * WR < red; r += 16 * WR) {  // sixteen rows in flight, kept packed until added
       uint4 raw[16];
 #pragma unroll
-      for (int q = 0; q < 16; ++q) raw[q] = *(const uint4*)(base + (r + 4 * q) * inner);
+      for (int q = 0; q < 16; ++q) raw[q] = *(const uint4*)(base + (r + WR * q) * inner);
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         float v[VEC];
@@ -245,16 +249,16 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
         for (int e = 0; e < VEC; ++e) acc[e] = red_comb(acc[e], v[e], kind);
       }
     }
-    for (; r + 28 < red; r += 32) {
+    for (; r + 7 * WR < red; r += 8 * WR) {
       float v[8][VEC];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) load(r + 4 * q, v[q]);
+      for (int q = 0; q < 8; ++q) load(r + WR * q, v[q]);
 #pragma unroll
       for (int q = 0; q < 8; ++q)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = red_comb(acc[e], v[q][e], kind);
     }
-    for (; r < red; r += 4) {
+    for (; r < red; r += WR) {
       float v[VEC];
       load(r, v);
 #pragma unroll
@@ -264,11 +268,11 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
 #pragma unroll
   for (int e = 0; e < VEC; ++e) part[w][lane][e] = acc[e];
   __syncthreads();
-  if (w == 0 && col < inner) {
+  if (wr == 0 && col < inner) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      const float v = red_comb(red_comb(part[0][lane][e], part[1][lane][e], kind),
-                               red_comb(part[2][lane][e], part[3][lane][e], kind), kind);
+      float v = part[wcid][lane][e];
+      for (int k = 1; k < WR; ++k) v = red_comb(v, part[k * wc + wcid][lane][e], kind);
       nbk_store_from_f32(out, o * inner + col + e, dto, v);
     }
   }
@@ -276,8 +280,9 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
                                                              void* __restrict__ out, int dto,
-                                                             int64_t red, int64_t inner, int kind) {
-  reduce_mid_vec_body<T, VEC>(in, out, dto, red, inner, kind, blockIdx.x, blockIdx.y);
+                                                             int64_t red, int64_t inner, int kind,
+                                                             int wc) {
+  reduce_mid_vec_body<T, VEC>(in, out, dto, red, inner, kind, blockIdx.x, blockIdx.y, wc);
 }
 
 // Several independent reductions in one launch (the column sums behind the bias and norm
@@ -288,6 +293,7 @@ struct ReduceBatchArgs {
   int32_t first_block[NBK_REDUCE_BATCH_MAX + 1];
   int32_t blocks_x[NBK_REDUCE_BATCH_MAX];
   int32_t mode[NBK_REDUCE_BATCH_MAX];  // 0: element-wise, 1: bf16 x 8, 2: fp32 x 4
+  int32_t wc[NBK_REDUCE_BATCH_MAX];    // waves side by side along the row (vector modes)
   nbk_reduce_task t[NBK_REDUCE_BATCH_MAX];
 };
 
@@ -298,12 +304,17 @@ __global__ __launch_bounds__(256) void reduce_batch_kernel(const ReduceBatchArgs
   const int lb = (int)blockIdx.x - B.first_block[i];
   const int64_t bx = lb % B.blocks_x[i], o = lb / B.blocks_x[i];
   if (B.mode[i] == 1)
-    reduce_mid_vec_body<uint16_t, 8>((const uint16_t*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o);
+    reduce_mid_vec_body<uint16_t, 8>((const uint16_t*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o, B.wc[i]);
   else if (B.mode[i] == 2)
-    reduce_mid_vec_body<float, 4>((const float*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o);
+    reduce_mid_vec_body<float, 4>((const float*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o, B.wc[i]);
   else
     reduce_mid_body(t.in, t.out, t.dtype_in, t.dtype_out, t.red, t.inner, t.kind, bx, o);
 }
+
+// Waves side by side for a row of `chunks` 16-byte pieces: as many as the row fills.  (A
+// function of the row alone: the order of summation, and so the result, does not depend on
+// how reductions are grouped into launches.)
+static int reduce_waves_across(int64_t chunks) { return chunks >= 256 ? 4 : (chunks >= 128 ? 2 : 1); }
 
 extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
                               int64_t red, int64_t inner, int32_t kind, void* stream) {
@@ -314,15 +325,17 @@ extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dt
   NBK_REQUIRE(outer <= 65535, "reduce_mid: outer %lld exceeds the grid limit", (long long)outer);
   const bool aligned = ((uintptr_t)in & 15) == 0;
   if (dti == NBK_BF16 && inner % 8 == 0 && aligned) {
-    dim3 grid((unsigned)((inner / 8 + 63) / 64), (unsigned)outer);
+    const int wc = reduce_waves_across(inner / 8);
+    dim3 grid((unsigned)((inner / 8 + 64 * wc - 1) / (64 * wc)), (unsigned)outer);
     hipLaunchKernelGGL((reduce_mid_vec_kernel<uint16_t, 8>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const uint16_t*)in, out, dto, red, inner, kind);
+                       (const uint16_t*)in, out, dto, red, inner, kind, wc);
     return nbk_check_launch("reduce_mid_vec_kernel");
   }
   if (dti == NBK_F32 && inner % 4 == 0 && aligned) {
-    dim3 grid((unsigned)((inner / 4 + 63) / 64), (unsigned)outer);
+    const int wc = reduce_waves_across(inner / 4);
+    dim3 grid((unsigned)((inner / 4 + 64 * wc - 1) / (64 * wc)), (unsigned)outer);
     hipLaunchKernelGGL((reduce_mid_vec_kernel<float, 4>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const float*)in, out, dto, red, inner, kind);
+                       (const float*)in, out, dto, red, inner, kind, wc);
     return nbk_check_launch("reduce_mid_vec_kernel");
   }
   dim3 grid((unsigned)((inner + 63) / 64), (unsigned)outer);
@@ -349,7 +362,8 @@ extern "C" int nbk_reduce_mid_batch(const nbk_reduce_task* tasks, int32_t n, voi
       B.mode[i] = 0;
       if (t.dtype_in == NBK_BF16 && t.inner % 8 == 0 && aligned) { B.mode[i] = 1; vec = 8; }
       else if (t.dtype_in == NBK_F32 && t.inner % 4 == 0 && aligned) { B.mode[i] = 2; vec = 4; }
-      const int64_t bx = (t.inner / vec + 63) / 64;
+      B.wc[i] = vec > 1 ? reduce_waves_across(t.inner / vec) : 1;
+      const int64_t bx = (t.inner / vec + 64 * B.wc[i] - 1) / (64 * B.wc[i]);
       B.blocks_x[i] = (int32_t)bx;
       B.first_block[i] = (int32_t)blocks;
       blocks += bx * t.outer;
