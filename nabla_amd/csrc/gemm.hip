@@ -244,8 +244,22 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
     for (int e = 0; e < 8; ++e)
       if (col + e < g.N) bias_v[e] = nbk_load_as_f32(g.bias, col + e, g.dtype_c);
   }
+  constexpr int NP = 32 / ROWS_PER_PASS;
+  const bool res_vec = EPI && g.residual && vec_store && !out_f32;
   static_for<TM>([&](auto ti) {
     constexpr int i = decltype(ti)::value;
+    // the residual of the whole tile row is requested before the slab round trip, so that
+    // its latency is paid once and not pass by pass
+    uint4 rpre[NP];
+    if constexpr (EPI) {
+#pragma unroll
+      for (int pass = 0; pass < NP; ++pass) {
+        const int64_t row = m0 + wm + i * 32 + pass * ROWS_PER_PASS + sub_r;
+        rpre[pass] = make_uint4(0u, 0u, 0u, 0u);
+        if (res_vec && row < g.M)
+          rpre[pass] = *(const uint4*)((const uint16_t*)g.residual + c_off + row * g.ldc + col);
+      }
+    }
     static_for<TN>([&](auto tj) {
       constexpr int j = decltype(tj)::value;
       const f32x16 a = acc[i][j];
@@ -255,8 +269,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
     });
     // the slab is private to the wave: no workgroup barrier, only LDS ordering
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-#pragma unroll 1
-    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+    auto one_pass = [&](int pass, const uint4 u) {
       const int lr = pass * ROWS_PER_PASS + sub_r;
       const int64_t row = m0 + wm + i * 32 + lr;
       float v[8];
@@ -269,12 +282,21 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
         if (EPI) {
+          float res[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float x = gemm_act(v[e] + bias_v[e], g.act);
-            if (g.residual && col + e < g.N) x += nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
-            v[e] = x;
+          for (int e = 0; e < 8; ++e) res[e] = 0.f;
+          if (res_vec) {
+            res[0] = __uint_as_float(u.x << 16); res[1] = __uint_as_float(u.x & 0xffff0000u);
+            res[2] = __uint_as_float(u.y << 16); res[3] = __uint_as_float(u.y & 0xffff0000u);
+            res[4] = __uint_as_float(u.z << 16); res[5] = __uint_as_float(u.z & 0xffff0000u);
+            res[6] = __uint_as_float(u.w << 16); res[7] = __uint_as_float(u.w & 0xffff0000u);
+          } else if (g.residual) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < g.N) res[e] = nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
           }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = gemm_act(v[e] + bias_v[e], g.act) + res[e];
         }
         if (vec_store && !out_f32) {
           uint4 o;
@@ -296,6 +318,13 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
             }
         }
       }
+    };
+    if constexpr (EPI) {
+#pragma unroll
+      for (int pass = 0; pass < NP; ++pass) one_pass(pass, rpre[pass]);
+    } else {
+#pragma unroll 1
+      for (int pass = 0; pass < NP; ++pass) one_pass(pass, make_uint4(0u, 0u, 0u, 0u));
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next tile row overwrites it
   });
@@ -836,6 +865,60 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
   }
 }
 
+// ------------------------------------------------------------------- bf16, K <= 16
+// C = alpha * A @ B (+ residual) with a contraction of at most 16 (the "up" product of a
+// low-rank adapter): one MFMA deep, all memory traffic.  No K loop and no operand tiles in
+// LDS: every lane reads its 8 k-values of an A row / a B column straight from global memory
+// into the MFMA fragment, and the tile leaves through the shared epilogue.
+template <bool B_KC, bool EPI>
+__global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
+  constexpr int TM = 2, TN = 2, WN = 64;
+  int tm_i, tn_i;
+  gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
+  const int64_t m0 = (int64_t)tm_i * 128, n0 = (int64_t)tn_i * 128;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int li = lane & 31, kg = lane >> 5;
+  const uint16_t* A = (const uint16_t*)g.A;
+  const uint16_t* B = (const uint16_t*)g.B;
+  // 8 k-values from k0 = 8 kg on, zero past K; rows / columns past the edge are clamped
+  // (their products are never stored)
+  auto frag8 = [&](const uint16_t* p, int64_t stride, bool vec) {
+    const int k0 = 8 * kg;
+    u32x4 u = {0u, 0u, 0u, 0u};
+    if (vec && k0 + 8 <= g.K) {
+      u = *(const u32x4*)(p + k0);
+    } else {
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) h[e] = k0 + e < g.K ? p[(k0 + e) * stride] : 0u;
+      u.x = h[0] | (h[1] << 16); u.y = h[2] | (h[3] << 16);
+      u.z = h[4] | (h[5] << 16); u.w = h[6] | (h[7] << 16);
+    }
+    return *(const bf16x8*)&u;
+  };
+  bf16x8 fa[TM], fb[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int64_t row = m0 + wm + i * 32 + li;
+    row = row < g.M ? row : g.M - 1;
+    fa[i] = frag8(A + row * g.a_rs, 1, g.a_vec);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int64_t col = n0 + wn + j * 32 + li;
+    col = col < g.N ? col : g.N - 1;
+    fb[j] = B_KC ? frag8(B + col * g.b_cs, 1, g.b_vec) : frag8(B + col, g.b_rs, false);
+  }
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], (f32x16)(0.f), 0, 0, 0);
+  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane);
+}
+
 // ---------------------------------------------------------------------------- fp32
 // 128 x 128 x 16 tile, LDS k-major ([k][rows], rows padded by 4 floats).
 template <bool A_KC, bool B_KC>
@@ -1163,6 +1246,23 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   };
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs, a.a_bs2);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs, a.b_bs2);
+  if (d->dtype_ab == NBK_BF16 && d->K <= 16 && akc && d->batch == 1 && d->N % 8 == 0 &&
+      d->ldc % 8 == 0 && ((uintptr_t)d->C & 15) == 0 && ((uintptr_t)d->residual & 15) == 0 &&
+      (d->K == 16 ? a.a_vec : d->K == 8 && (d->a_rs % 8 == 0) && ((uintptr_t)d->A & 15) == 0)) {
+    // (the vector path reads whole 16-byte pieces of A rows: K = 16 or 8)
+    a.a_vec = 1;
+    a.b_vec = bkc && (d->K == 16 ? a.b_vec : (d->b_cs % 8 == 0) && ((uintptr_t)d->B & 15) == 0);
+    a.tiles_m = (int)((d->M + 127) / 128);
+    a.tiles_n = (int)((d->N + 127) / 128);
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
+    const size_t lds = 4 * 32 * (size_t)(64 + 4) * sizeof(float);
+    const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
+    if (bkc && epi) hipLaunchKernelGGL((gemm_skinny_k_kernel<true, true>), grid, dim3(256), lds, st, a);
+    else if (bkc) hipLaunchKernelGGL((gemm_skinny_k_kernel<true, false>), grid, dim3(256), lds, st, a);
+    else if (epi) hipLaunchKernelGGL((gemm_skinny_k_kernel<false, true>), grid, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_k_kernel<false, false>), grid, dim3(256), lds, st, a);
+    return nbk_check_launch("gemm_skinny_k_kernel");
+  }
   if (d->dtype_ab == NBK_BF16) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
