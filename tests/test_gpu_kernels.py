@@ -84,6 +84,78 @@ def test_gemm(hip, dtype, layout, shape):
     assert err.max() <= atol, err.max()
 
 
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape", [(384, 256, 2048), (1000, 520, 4096)])
+def test_gemm_long_k_small_output(hip, layout, shape):
+    """bf16 products whose 128 x 128 tiles split every K tile between two groups of waves
+    (K >= 2048): the partial sums meet in LDS before the result is rounded."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(5)
+    A = torch.tensor(rng.standard_normal((M, K)), dtype=torch.bfloat16)
+    B = torch.tensor(rng.standard_normal((K, N)), dtype=torch.bfloat16)
+    ref = (A.double() @ B.double()).numpy()
+    a_dev = (A if layout[0] == "n" else A.t().contiguous()).cuda()
+    b_dev = (B if layout[1] == "n" else B.t().contiguous()).cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs = (K, 1) if layout[0] == "n" else (1, M)
+    d.b_rs, d.b_cs = (N, 1) if layout[1] == "n" else (1, K)
+    d.ldc = N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
+    d.dtype_ab = d.dtype_c = 1
+    d.alpha = 1.0
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    err = np.abs(got - ref) - 2.0 ** -8 * np.abs(ref)
+    assert err.max() <= 2e-2, err.max()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("act", [0, 1, 2])
+@pytest.mark.parametrize("shape", [(256, 384, 128),      # 128 x 128 tiles
+                                   (300, 200, 72),       # guarded kernel (K % 64 != 0)
+                                   (640, 520, 2048),     # 128 x 128 tiles, two k-groups
+                                   (4096, 2560, 192)])   # 256 x 256 tiles
+def test_gemm_epilogue(hip, dtype, act, shape):
+    """act(alpha * A @ B + bias) + residual, the fused way out of nbk_gemm."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(6)
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    A = torch.tensor(rng.standard_normal((M, K)) / np.sqrt(K), dtype=tdt)
+    B = torch.tensor(rng.standard_normal((N, K)), dtype=tdt)            # "nt": both K-contiguous
+    bias = torch.tensor(rng.standard_normal((N,)), dtype=tdt)
+    R = torch.tensor(rng.standard_normal((M, N)), dtype=tdt)
+    alpha = 1.5
+    z = alpha * (A.double() @ B.double().t()) + bias.double()
+    z = z if act == 0 else (torch.relu(z) if act == 1 else torch.nn.functional.gelu(z))
+    ref = (z + R.double()).numpy()
+    a_dev, b_dev, bias_dev, r_dev = A.cuda(), B.cuda(), bias.cuda(), R.cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr()
+    d.bias, d.residual = bias_dev.data_ptr(), r_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs, d.b_rs, d.b_cs = K, 1, 1, K
+    d.ldc = N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, M * N
+    d.dtype_ab = d.dtype_c = 0 if dtype == "f32" else 1
+    d.act = act
+    d.alpha = alpha
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    rtol, atol = (1e-5, 2e-5) if dtype == "f32" else (2.0 ** -8, 2e-2)
+    err = np.abs(got - ref) - rtol * np.abs(ref)
+    assert err.max() <= atol, err.max()
+
+
 @pytest.mark.parametrize("b_layout", ["n", "t"])
 @pytest.mark.parametrize("out", ["bf16", "f32"])
 @pytest.mark.parametrize("shape", [(4096, 512, 16), (3001, 1032, 16), (2048, 1024, 8), (1100, 2048, 13)])
