@@ -140,6 +140,11 @@ class BoundPlan:
                 ptr_field(d, "C", rc.buf, rc.offset * rc.dtype.size_in_bytes)
                 d.bias = None
                 d.residual = None
+                if a.get("bias") is not None:
+                    rbias = a["bias"]
+                    if rbias.dtype is not rc.dtype:
+                        raise TypeError(f"matmul bias is {rbias.dtype}, the result {rc.dtype}")
+                    ptr_field(d, "bias", rbias.buf, rbias.offset * rbias.dtype.size_in_bytes)
                 d.M, d.N, d.K = a["M"], a["N"], a["K"]
                 d.a_rs, d.a_cs, d.b_rs, d.b_cs = a["a_rs"], a["a_cs"], a["b_rs"], a["b_cs"]
                 d.ldc = a["ldc"]

@@ -597,6 +597,55 @@ class Planner:
         return self._materialize(self._resolve(v))
 
     # ................................................................ build
+    def _fold_bias_into_matmul(self) -> None:
+        """``x @ W + b`` with ``b`` a row vector broadcast over the leading axes: the bias
+        becomes a third input of the matmul (added in the kernel's epilogue, before the result
+        is rounded) and the add disappears.  Only where the product is the add's alone and is
+        not split along K."""
+        nodes = self._live_nodes()
+        n_users: dict[int, int] = {}
+        for n in nodes:
+            for i in n.inputs:
+                n_users[i.id] = n_users.get(i.id, 0) + 1
+        out_ids = {v.id for v in self.outputs}
+        replace: dict[int, ir.Value] = {}
+        for n in nodes:
+            if not (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2):
+                continue
+            for m, bb in ((n.inputs[0], n.inputs[1]), (n.inputs[1], n.inputs[0])):
+                mm = m.node
+                if not (mm.kind == "matmul" and len(mm.inputs) == 2 and n_users.get(m.id) == 1 and
+                        m.id not in out_ids and bb.node.kind == "broadcast"):
+                    continue
+                src = bb.node.inputs[0]
+                N = m.shape[-1]
+                out = n.outputs[0]
+                if not (src.rank >= 1 and src.shape[-1] == N and _numel(src.shape) == N and
+                        src.dtype is m.dtype and out.dtype is m.dtype and out.shape == m.shape and
+                        m.dtype in (DType.float32, DType.bfloat16) and
+                        src.node.pos < mm.pos):
+                    continue
+                a, b = mm.inputs
+                K = a.shape[-1]
+                # (a product that would be split along K keeps its add: the partial products
+                # cannot carry the bias; batched x @ W is one product with all the rows)
+                dt = a.dtype if a.dtype is b.dtype else DType.float32
+                if self._split_k(_numel(m.shape[:-1]), N, K, dt) != 1:
+                    continue
+                mm.inputs.append(src)
+                mm.attrs = dict(mm.attrs or {}, has_bias=True)
+                replace[out.id] = m
+                break
+        if not replace:
+            return
+        for n in self.b.nodes:
+            n.inputs = [replace.get(i.id, i) for i in n.inputs]
+            if n.attrs and "operands" in n.attrs:  # element-wise nodes list their operands again
+                n.attrs = dict(n.attrs, operands=tuple(
+                    replace.get(o.id, o) if isinstance(o, ir.Value) else o
+                    for o in n.attrs["operands"]))
+        self.outputs = [replace.get(v.id, v) for v in self.outputs]
+
     def build(self) -> Plan:
         nodes = self._live_nodes()
         for i, v in enumerate(self.b.inputs):
@@ -976,8 +1025,11 @@ class Planner:
         return tuple(cand)
 
     def _lower_matmul(self, n: ir.Node) -> None:
-        a, b = n.inputs
+        a, b = n.inputs[:2]
         out = n.outputs[0]
+        bias = None
+        if (n.attrs or {}).get("has_bias"):
+            bias = self._contig(n.inputs[2])
         ra, rb = self._resolve(a), self._resolve(b)
         if isinstance(ra, Const):
             ra = self._materialize(ra)
@@ -1046,7 +1098,7 @@ class Planner:
             M, batch = M * batch, 1
             a_bs = c_bs = 0
         if batch == 1 and c_strides == contiguous_strides(out.shape):
-            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K, out)
+            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K, out, bias)
             return
         if c_strides == contiguous_strides(out.shape):
             dst = self._alloc_value(out)
@@ -1054,8 +1106,10 @@ class Planner:
             buf = self._new_buf(out.shape, out.dtype, "temp", -1)
             dst = ViewRef(buf.id, 0, out.shape, c_strides, out.dtype)
             self.loc[out.id] = dst
-        self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
-            a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
+        extra = dict(bias=bias) if bias is not None else {}
+        self._emit(Step("gemm", [ra.buf, rb.buf] + ([bias.buf] if bias is not None else []),
+                        [dst.buf], dict(
+            extra, a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
             ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
@@ -1073,16 +1127,17 @@ class Planner:
         return ks
 
     def _emit_plain_gemm(self, ra: ViewRef, rb: ViewRef, pa, pb, M: int, N: int, K: int,
-                         out: ir.Value) -> None:
+                         out: ir.Value, bias: ViewRef | None = None) -> None:
         """One unbatched product into contiguous storage for ``out``; split along K into fp32
         partial products plus their sum when the output alone gives too few workgroups."""
         ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32)
         dst = self._alloc_value(out)
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
-        if ks == 1:
-            self._emit(Step("gemm", [ra.buf, rb.buf], [dst.buf], dict(
-                common, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
+        if ks == 1 or bias is not None:  # (a product with a folded bias is never split)
+            extra = dict(bias=bias) if bias is not None else {}
+            self._emit(Step("gemm", [ra.buf, rb.buf] + ([bias.buf] if bias is not None else []),
+                            [dst.buf], dict(common, **extra, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
             return
         kc = K // ks
         tmp = self._new_buf((ks, M, N), DType.float32)
@@ -1697,6 +1752,10 @@ class _RowCodegen:
 def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     """Plan with shrinking fusion limits until every group fits a row program."""
     last = None
+    # graph rewrites happen once, before the attempts below share the builder
+    pre = Planner(builder, outputs)
+    pre._fold_bias_into_matmul()
+    outputs = pre.outputs
     for limit in (28, 16, 8, 4, 1):
         try:
             return Planner(builder, outputs, max_members=limit).build()

@@ -215,7 +215,8 @@ extern __shared__ __align__(16) u32x4 gemm_lds[];
 
 // Epilogue shared by the bf16 kernels (the caller has passed a workgroup barrier: the tile
 // buffers are free).
-template <int TM, int TN, int WN, bool FAST, bool EPI>
+// EPI: 0 plain, 1 bias only (as lean as the plain form), 2 bias / activation / residual.
+template <int TM, int TN, int WN, bool FAST, int EPI>
 __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
                                               int64_t n0, int wm, int wn, int64_t c_off, int wave,
                                               int lane) {
@@ -239,19 +240,19 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
   float bias_v[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) bias_v[e] = 0.f;
-  if (EPI && g.bias) {
+  if (EPI != 0 && g.bias) {
 #pragma unroll
     for (int e = 0; e < 8; ++e)
       if (col + e < g.N) bias_v[e] = nbk_load_as_f32(g.bias, col + e, g.dtype_c);
   }
   constexpr int NP = 32 / ROWS_PER_PASS;
-  const bool res_vec = EPI && g.residual && vec_store && !out_f32;
+  const bool res_vec = EPI == 2 && g.residual && vec_store && !out_f32;
   static_for<TM>([&](auto ti) {
     constexpr int i = decltype(ti)::value;
     // the residual of the whole tile row is requested before the slab round trip, so that
     // its latency is paid once and not pass by pass
     uint4 rpre[NP];
-    if constexpr (EPI) {
+    if constexpr (EPI == 2) {
 #pragma unroll
       for (int pass = 0; pass < NP; ++pass) {
         const int64_t row = m0 + wm + i * 32 + pass * ROWS_PER_PASS + sub_r;
@@ -281,7 +282,11 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
         const int64_t idx = c_off + row * g.ldc + col;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
-        if (EPI) {
+        if (EPI == 1) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
+        }
+        if (EPI == 2) {
           float res[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) res[e] = 0.f;
@@ -319,7 +324,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
         }
       }
     };
-    if constexpr (EPI) {
+    if constexpr (EPI == 2) {
 #pragma unroll
       for (int pass = 0; pass < NP; ++pass) one_pass(pass, rpre[pass]);
     } else {
@@ -536,7 +541,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
   }
   __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
 
-  gemm_epilogue<TM, TN, WN, false, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
+  gemm_epilogue<TM, TN, WN, false, EPI ? 2 : 0>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
 }
 
 // ------------------------------------------------------------- bf16, direct-to-LDS loads
@@ -616,7 +621,7 @@ struct DirectLoader {
 // even and the odd k-steps of every tile, each group covering the whole tile with two
 // 128 x 64 wave tiles (6 fragment reads per 8 MFMAs instead of 4 per 4: the small tile is
 // bound by LDS reads), and the two partial sums are added through LDS before the epilogue.
-template <int BM, int BN, bool A_KC, bool B_KC, bool EPI, int NW, int KSS, int KSPLIT>
+template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS, int KSPLIT>
 __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const GemmArgs g) {
   static_assert(KSPLIT == 1 || (KSPLIT == 2 && NW == 4 && BM == 128 && BN == 128), "k split");
   constexpr int GW = NW / KSPLIT;                         // waves per k-group
@@ -916,7 +921,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], (f32x16)(0.f), 0, 0, 0);
-  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane);
+  gemm_epilogue<TM, TN, WN, true, EPI ? 2 : 0>(acc, g, m0, n0, wm, wn, 0, wave, lane);
 }
 
 // ---------------------------------------------------------------------------- fp32
@@ -1178,7 +1183,7 @@ static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, 
   const size_t pipe = 2 * (size_t)(BM + BN) * 8 * 16;
   const size_t slabs = NW * 32 * (size_t)(BN / (NW / 2) + 4) * sizeof(float);
   const size_t lds = pipe > slabs ? pipe : slabs;
-  const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
+  const int epi = (a.residual != nullptr || a.act != NBK_ACT_NONE) ? 2 : (a.bias != nullptr ? 1 : 0);
 #define NBK_LAUNCH_DL(AK, BK_, EP)                                                            \
   do {                                                                                        \
     auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS, KSPLIT>;                                 \
@@ -1192,8 +1197,9 @@ static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, 
   } while (0)
 #define NBK_LAUNCH_DL2(AK, BK_)                                                               \
   do {                                                                                        \
-    if (epi) NBK_LAUNCH_DL(AK, BK_, true);                                                    \
-    else NBK_LAUNCH_DL(AK, BK_, false);                                                       \
+    if (epi == 2) NBK_LAUNCH_DL(AK, BK_, 2);                                                  \
+    else if (epi == 1) NBK_LAUNCH_DL(AK, BK_, 1);                                             \
+    else NBK_LAUNCH_DL(AK, BK_, 0);                                                           \
   } while (0)
   if (akc && bkc) NBK_LAUNCH_DL2(true, true);
   else if (akc && !bkc) NBK_LAUNCH_DL2(true, false);

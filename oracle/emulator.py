@@ -196,6 +196,8 @@ def _gemm(a, mem):
     A = mat(a["a"], a["a_bs"], a.get("a_bs2", 0), a["a_rs"], a["a_cs"], a["M"], a["K"]).float()
     B = mat(a["b"], a["b_bs"], a.get("b_bs2", 0), a["b_rs"], a["b_cs"], a["K"], a["N"]).float()
     C = torch.matmul(A.double(), B.double()).float() * a.get("alpha", 1.0)
+    if a.get("bias") is not None:  # added before the result is rounded, as in the kernel's epilogue
+        C = C + _view(mem, a["bias"]).reshape(-1).float()
     dst = a["dst"]
     out = mat(dst, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"])
     out.copy_(C.to(out.dtype))

@@ -183,6 +183,36 @@ def test_layernorm_softmax_forward_is_one_kernel(emulator):
     assert stats["rowprog"] == 1 and stats["steps"] == 1, stats
 
 
+def test_bias_add_rides_in_the_matmul(emulator):
+    """x @ W + b with a row-vector b: the add is folded into the product's epilogue; a product
+    with a second reader keeps its add (the plain product is needed too)."""
+    x = RNG.standard_normal((3, 16, 32)).astype(np.float32)
+    W = RNG.standard_normal((32, 24)).astype(np.float32)
+    b = RNG.standard_normal((1, 24)).astype(np.float32)
+    y = T(x) @ T(W) + T(b)
+    ref = x.astype(np.float64) @ W + b
+    assert relerr(y.numpy(), ref) < 1e-5
+    plan = last_plan()
+    assert plan.stats == {"steps": 1, "units": 1, "fused_groups": 0, "gemm": 1}, plan.stats
+    assert plan.steps[0].attrs.get("bias") is not None
+    # two readers of the product
+    X, Wt, bt = T(x), T(W), T(b)
+    p = X @ Wt
+    y2, z2 = p + bt, nb.relu(p)
+    nb.realize_all(y2, z2)
+    assert relerr(y2.numpy(), ref) < 1e-5
+    assert relerr(z2.numpy(), np.maximum(x.astype(np.float64) @ W, 0)) < 1e-5
+    plan = last_plan()
+    assert all(s.attrs.get("bias") is None for s in plan.steps if s.kind == "gemm")
+    # gradients flow through the folded form as before
+    def loss(Wt, bt):
+        return nb.reduce_sum(nb.relu(X @ Wt + bt))
+    gW, gb = nb.grad(loss, argnums=(0, 1), realize=True)(Wt, bt)
+    mask = ((x.astype(np.float64) @ W + b) > 0).astype(np.float64)
+    assert relerr(gW.numpy(), np.einsum("bmk,bmn->kn", x.astype(np.float64), mask)) < 1e-5
+    assert relerr(gb.numpy(), mask.sum(axis=(0, 1))[None, :]) < 1e-5
+
+
 def test_forward_traced_twice_is_computed_once(emulator):
     x = T(RNG.standard_normal((16, 128)).astype(np.float32))
     y = T(RNG.standard_normal((16, 128)).astype(np.float32))
