@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 10
+#define NBK_ABI_VERSION 11
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -208,8 +208,7 @@ int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void* stream);
 /* ===================================================================== */
 /*  GEMM                                                                  */
 /* ===================================================================== */
-/* C[b] = alpha * op(A[b]) @ op(B[b]) (+ bias) (+ residual) with optional
- * activation; replaces ops.matmul at nabla/ops/binary.py:198 for the forward
+/* C[b] = act(alpha * op(A[b]) @ op(B[b]) + bias) (+ or x) residual; replaces ops.matmul at nabla/ops/binary.py:198 for the forward
  * product and for both backward products of MatmulOp.vjp_rule
  * (binary.py:303-314), whose swap_axes are folded into the strides here.
  * A is M x K with element strides (a_rs, a_cs), B is K x N with (b_rs, b_cs);
@@ -219,10 +218,13 @@ int nbk_fill(void* dst, int32_t dtype, int64_t n, double value, void* stream);
  * (dW of a 3-D activation against a 2-D weight: backward.py:36-41).
  * dtype_ab: NBK_F32 or NBK_BF16; accumulation is always fp32. */
 enum nbk_gemm_act { NBK_ACT_NONE = 0, NBK_ACT_RELU = 1, NBK_ACT_GELU = 2 };
+/* what the residual does to the result: added (x + r: a skip connection, an accumulated
+ * gradient) or multiplied in (x * r: the saved derivative of an activation, a mask) */
+enum nbk_gemm_residual_op { NBK_RES_ADD = 0, NBK_RES_MUL = 1 };
 typedef struct nbk_gemm_desc {
   const void* A; const void* B; void* C;
   const void* bias;      /* NULL or [N] (dtype_c), added to every row        */
-  const void* residual;  /* NULL or same layout as C, added after activation */
+  const void* residual;  /* NULL or same layout as C, applied after activation */
   int64_t M, N, K;
   int64_t a_rs, a_cs, b_rs, b_cs, ldc;
   int64_t batch, a_bs, b_bs, c_bs;
@@ -235,7 +237,7 @@ typedef struct nbk_gemm_desc {
   int32_t act;
   int32_t batch_reduce;
   float alpha;
-  int32_t reserved;
+  int32_t residual_op;   /* enum nbk_gemm_residual_op */
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
 

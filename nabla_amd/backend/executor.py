@@ -145,6 +145,13 @@ class BoundPlan:
                     if rbias.dtype is not rc.dtype:
                         raise TypeError(f"matmul bias is {rbias.dtype}, the result {rc.dtype}")
                     ptr_field(d, "bias", rbias.buf, rbias.offset * rbias.dtype.size_in_bytes)
+                d.residual_op = 0
+                if a.get("residual") is not None:
+                    rres = a["residual"]
+                    if rres.dtype is not rc.dtype:
+                        raise TypeError(f"matmul residual is {rres.dtype}, the result {rc.dtype}")
+                    ptr_field(d, "residual", rres.buf, rres.offset * rres.dtype.size_in_bytes)
+                    d.residual_op = 1 if a["res_op"] == "mul" else 0
                 d.M, d.N, d.K = a["M"], a["N"], a["K"]
                 d.a_rs, d.a_cs, d.b_rs, d.b_cs = a["a_rs"], a["a_cs"], a["b_rs"], a["b_cs"]
                 d.ldc = a["ldc"]

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 MAX_RANK = 8
 
@@ -66,7 +66,7 @@ class GemmDesc(C.Structure):
         ("batch_inner", C.c_int64), ("a_bs2", C.c_int64), ("b_bs2", C.c_int64), ("c_bs2", C.c_int64),
         ("dtype_ab", C.c_int32), ("dtype_c", C.c_int32),
         ("act", C.c_int32), ("batch_reduce", C.c_int32),
-        ("alpha", C.c_float), ("reserved", C.c_int32),
+        ("alpha", C.c_float), ("residual_op", C.c_int32),
     ]
 
 

@@ -598,53 +598,49 @@ class Planner:
 
     # ................................................................ build
     def _fold_bias_into_matmul(self) -> None:
-        """``x @ W + b`` with ``b`` a row vector broadcast over the leading axes: the bias
-        becomes a third input of the matmul (added in the kernel's epilogue, before the result
-        is rounded) and the add disappears.  Only where the product is the add's alone and is
-        not split along K."""
+        """``x @ W + b`` with ``b`` a row vector broadcast over the leading axes: the add node
+        itself turns into the matmul node with the bias as a third input
+        (``attrs["bias_in"]``; it comes after everything the product reads, so program order
+        stays a valid order) and the original product, now without readers, is dropped by the
+        liveness pass.  The bias is added in the kernel's epilogue, before the result is
+        rounded.  Only where the product has no other reader and is not split along K
+        (partial products cannot carry an epilogue)."""
         nodes = self._live_nodes()
         n_users: dict[int, int] = {}
         for n in nodes:
             for i in n.inputs:
                 n_users[i.id] = n_users.get(i.id, 0) + 1
         out_ids = {v.id for v in self.outputs}
-        replace: dict[int, ir.Value] = {}
         for n in nodes:
             if not (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2):
                 continue
+            out = n.outputs[0]
             for m, bb in ((n.inputs[0], n.inputs[1]), (n.inputs[1], n.inputs[0])):
                 mm = m.node
-                if not (mm.kind == "matmul" and len(mm.inputs) == 2 and n_users.get(m.id) == 1 and
-                        m.id not in out_ids and bb.node.kind == "broadcast"):
+                if not (bb.node.kind == "broadcast" and mm.kind == "matmul" and
+                        len(mm.inputs) == 2 and n_users.get(m.id) == 1 and m.id not in out_ids and
+                        self._epilogue_ok(mm, out)):
                     continue
                 src = bb.node.inputs[0]
                 N = m.shape[-1]
-                out = n.outputs[0]
                 if not (src.rank >= 1 and src.shape[-1] == N and _numel(src.shape) == N and
-                        src.dtype is m.dtype and out.dtype is m.dtype and out.shape == m.shape and
-                        m.dtype in (DType.float32, DType.bfloat16) and
-                        src.node.pos < mm.pos):
+                        src.dtype is m.dtype):
                     continue
-                a, b = mm.inputs
-                K = a.shape[-1]
-                # (a product that would be split along K keeps its add: the partial products
-                # cannot carry the bias; batched x @ W is one product with all the rows)
-                dt = a.dtype if a.dtype is b.dtype else DType.float32
-                if self._split_k(_numel(m.shape[:-1]), N, K, dt) != 1:
-                    continue
-                mm.inputs.append(src)
-                mm.attrs = dict(mm.attrs or {}, has_bias=True)
-                replace[out.id] = m
+                n.kind, n.fn = "matmul", None
+                n.inputs = list(mm.inputs) + [src]
+                n.attrs = dict(mm.attrs or {}, bias_in=2)
                 break
-        if not replace:
-            return
-        for n in self.b.nodes:
-            n.inputs = [replace.get(i.id, i) for i in n.inputs]
-            if n.attrs and "operands" in n.attrs:  # element-wise nodes list their operands again
-                n.attrs = dict(n.attrs, operands=tuple(
-                    replace.get(o.id, o) if isinstance(o, ir.Value) else o
-                    for o in n.attrs["operands"]))
-        self.outputs = [replace.get(v.id, v) for v in self.outputs]
+
+    def _epilogue_ok(self, mm: ir.Node, out: ir.Value) -> bool:
+        """The product ``mm`` may write ``out`` through its epilogue."""
+        m = mm.outputs[0]
+        if not (out.dtype is m.dtype and out.shape == m.shape and
+                m.dtype in (DType.float32, DType.bfloat16)):
+            return False
+        a, b = mm.inputs[:2]
+        dt = a.dtype if a.dtype is b.dtype else DType.float32
+        # (batched x @ W is one product with all the rows)
+        return self._split_k(_numel(m.shape[:-1]), m.shape[-1], a.shape[-1], dt) == 1
 
     def build(self) -> Plan:
         nodes = self._live_nodes()
@@ -1027,9 +1023,10 @@ class Planner:
     def _lower_matmul(self, n: ir.Node) -> None:
         a, b = n.inputs[:2]
         out = n.outputs[0]
-        bias = None
-        if (n.attrs or {}).get("has_bias"):
-            bias = self._contig(n.inputs[2])
+        epi: dict = {}
+        at = n.attrs or {}
+        if "bias_in" in at:
+            epi["bias"] = self._contig(n.inputs[at["bias_in"]])
         ra, rb = self._resolve(a), self._resolve(b)
         if isinstance(ra, Const):
             ra = self._materialize(ra)
@@ -1098,7 +1095,7 @@ class Planner:
             M, batch = M * batch, 1
             a_bs = c_bs = 0
         if batch == 1 and c_strides == contiguous_strides(out.shape):
-            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K, out, bias)
+            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K, out, epi)
             return
         if c_strides == contiguous_strides(out.shape):
             dst = self._alloc_value(out)
@@ -1106,10 +1103,8 @@ class Planner:
             buf = self._new_buf(out.shape, out.dtype, "temp", -1)
             dst = ViewRef(buf.id, 0, out.shape, c_strides, out.dtype)
             self.loc[out.id] = dst
-        extra = dict(bias=bias) if bias is not None else {}
-        self._emit(Step("gemm", [ra.buf, rb.buf] + ([bias.buf] if bias is not None else []),
-                        [dst.buf], dict(
-            extra, a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
+        self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), [dst.buf], dict(
+            epi, a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
             ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
@@ -1127,17 +1122,17 @@ class Planner:
         return ks
 
     def _emit_plain_gemm(self, ra: ViewRef, rb: ViewRef, pa, pb, M: int, N: int, K: int,
-                         out: ir.Value, bias: ViewRef | None = None) -> None:
+                         out: ir.Value, epi: dict | None = None) -> None:
         """One unbatched product into contiguous storage for ``out``; split along K into fp32
         partial products plus their sum when the output alone gives too few workgroups."""
         ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32)
         dst = self._alloc_value(out)
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
-        if ks == 1 or bias is not None:  # (a product with a folded bias is never split)
-            extra = dict(bias=bias) if bias is not None else {}
-            self._emit(Step("gemm", [ra.buf, rb.buf] + ([bias.buf] if bias is not None else []),
-                            [dst.buf], dict(common, **extra, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
+        epi = epi or {}
+        if ks == 1 or epi:  # (a product with a folded epilogue is never split)
+            self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), [dst.buf],
+                            dict(common, **epi, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
             return
         kc = K // ks
         tmp = self._new_buf((ks, M, N), DType.float32)
@@ -1146,6 +1141,10 @@ class Planner:
             common, dst=tref, K=kc, batch=ks, a_bs=kc * pa[2], b_bs=kc * pb[1])))
         self._emit_reduce(Step("reduce_mid", [tmp.id], [dst.buf], dict(
             src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum")), 1, self._terminal(out))
+
+    @staticmethod
+    def _epi_bufs(epi: dict) -> list[int]:
+        return [epi[k].buf for k in ("bias", "residual") if k in epi]
 
     # ................................................................ attention
     def _heads_operand(self, v: ir.Value) -> ViewRef:

@@ -49,6 +49,7 @@ struct GemmArgs {
   int64_t a_bs, b_bs, c_bs;
   int64_t batch_inner, a_bs2, b_bs2, c_bs2;  // batch_inner >= 1
   int32_t dtype_c, act;
+  int32_t res_mul;  // the residual multiplies instead of adding
   float alpha;
   int32_t tiles_m, tiles_n;
   int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
@@ -247,20 +248,22 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
   }
   constexpr int NP = 32 / ROWS_PER_PASS;
   const bool res_vec = EPI == 2 && g.residual && vec_store && !out_f32;
-  static_for<TM>([&](auto ti) {
-    constexpr int i = decltype(ti)::value;
-    // the residual of the whole tile row is requested before the slab round trip, so that
-    // its latency is paid once and not pass by pass
-    uint4 rpre[NP];
-    if constexpr (EPI == 2) {
+  // the residual of the whole wave tile is requested before the first slab round trip, so that
+  // its latency is paid once and not pass by pass (the K loop's registers are free by now)
+  uint4 rpre[EPI == 2 ? TM : 1][NP];
+  if constexpr (EPI == 2) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int pass = 0; pass < NP; ++pass) {
         const int64_t row = m0 + wm + i * 32 + pass * ROWS_PER_PASS + sub_r;
-        rpre[pass] = make_uint4(0u, 0u, 0u, 0u);
+        rpre[i][pass] = make_uint4(0u, 0u, 0u, 0u);
         if (res_vec && row < g.M)
-          rpre[pass] = *(const uint4*)((const uint16_t*)g.residual + c_off + row * g.ldc + col);
+          rpre[i][pass] = *(const uint4*)((const uint16_t*)g.residual + c_off + row * g.ldc + col);
       }
-    }
+  }
+  static_for<TM>([&](auto ti) {
+    constexpr int i = decltype(ti)::value;
     static_for<TN>([&](auto tj) {
       constexpr int j = decltype(tj)::value;
       const f32x16 a = acc[i][j];
@@ -301,7 +304,10 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
               if (col + e < g.N) res[e] = nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
           }
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = gemm_act(v[e] + bias_v[e], g.act) + res[e];
+          for (int e = 0; e < 8; ++e) {
+            const float x = gemm_act(v[e] + bias_v[e], g.act);
+            v[e] = !g.residual ? x : (g.res_mul ? x * res[e] : x + res[e]);
+          }
         }
         if (vec_store && !out_f32) {
           uint4 o;
@@ -326,7 +332,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
     };
     if constexpr (EPI == 2) {
 #pragma unroll
-      for (int pass = 0; pass < NP; ++pass) one_pass(pass, rpre[pass]);
+      for (int pass = 0; pass < NP; ++pass) one_pass(pass, rpre[i][pass]);
     } else {
 #pragma unroll 1
       for (int pass = 0; pass < NP; ++pass) one_pass(pass, make_uint4(0u, 0u, 0u, 0u));
@@ -1031,7 +1037,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
         if (row >= g.M) continue;
         float v = gemm_act(acc[i][j][r] * g.alpha + bv, g.act);
         const int64_t idx = c_off + row * g.ldc + col;
-        if (g.residual) v += ((const float*)g.residual)[idx];
+        if (g.residual) v = g.res_mul ? v * ((const float*)g.residual)[idx] : v + ((const float*)g.residual)[idx];
         C[idx] = v;
       }
     }
@@ -1128,7 +1134,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const GemmArgs g) {
     float v = (part[0][r][c] + part[1][r][c]) + (part[2][r][c] + part[3][r][c]);
     v = gemm_act(v * g.alpha + (g.bias ? ((const float*)g.bias)[col] : 0.f), g.act);
     const int64_t idx = c_off + row * g.ldc + col;
-    if (g.residual) v += ((const float*)g.residual)[idx];
+    if (g.residual) v = g.res_mul ? v * ((const float*)g.residual)[idx] : v + ((const float*)g.residual)[idx];
     C[idx] = v;
   }
 }
@@ -1242,6 +1248,9 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.b_bs2 = a.batch_inner > 1 ? d->b_bs2 : 0;
   a.c_bs2 = a.batch_inner > 1 ? d->c_bs2 : 0;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
+  NBK_REQUIRE(d->residual_op == NBK_RES_ADD || d->residual_op == NBK_RES_MUL,
+              "gemm: residual_op %d", d->residual_op);
+  a.res_mul = d->residual_op == NBK_RES_MUL;
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;

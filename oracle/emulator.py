@@ -198,6 +198,10 @@ def _gemm(a, mem):
     C = torch.matmul(A.double(), B.double()).float() * a.get("alpha", 1.0)
     if a.get("bias") is not None:  # added before the result is rounded, as in the kernel's epilogue
         C = C + _view(mem, a["bias"]).reshape(-1).float()
+    if a.get("residual") is not None:
+        res = a["residual"]
+        R = mat(res, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"]).float()
+        C = C * R if a["res_op"] == "mul" else C + R
     dst = a["dst"]
     out = mat(dst, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"])
     out.copy_(C.to(out.dtype))

@@ -121,8 +121,9 @@ def test_gemm_long_k_small_output(hip, layout, shape):
                                    (300, 200, 72),       # guarded kernel (K % 64 != 0)
                                    (640, 520, 2048),     # 128 x 128 tiles, two k-groups
                                    (4096, 2560, 192)])   # 256 x 256 tiles
-def test_gemm_epilogue(hip, dtype, act, shape):
-    """act(alpha * A @ B + bias) + residual, the fused way out of nbk_gemm."""
+@pytest.mark.parametrize("res_op", [0, 1])
+def test_gemm_epilogue(hip, dtype, act, shape, res_op):
+    """act(alpha * A @ B + bias) (+ or x) residual, the fused way out of nbk_gemm."""
     from nabla_amd.backend import lib
     M, N, K = shape
     rng = np.random.default_rng(6)
@@ -134,7 +135,7 @@ def test_gemm_epilogue(hip, dtype, act, shape):
     alpha = 1.5
     z = alpha * (A.double() @ B.double().t()) + bias.double()
     z = z if act == 0 else (torch.relu(z) if act == 1 else torch.nn.functional.gelu(z))
-    ref = (z + R.double()).numpy()
+    ref = (z * R.double() if res_op else z + R.double()).numpy()
     a_dev, b_dev, bias_dev, r_dev = A.cuda(), B.cuda(), bias.cuda(), R.cuda()
     c_dev = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
     d = lib.GemmDesc()
@@ -146,6 +147,7 @@ def test_gemm_epilogue(hip, dtype, act, shape):
     d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, M * N
     d.dtype_ab = d.dtype_c = 0 if dtype == "f32" else 1
     d.act = act
+    d.residual_op = res_op
     d.alpha = alpha
     L = lib.load()
     lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
