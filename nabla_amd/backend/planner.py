@@ -1110,11 +1110,13 @@ class Planner:
             ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
 
     @staticmethod
-    def _split_k(M: int, N: int, K: int, dtype: DType) -> int:
+    def _split_k(M: int, N: int, K: int, dtype: DType, a_k_contiguous: bool = False) -> int:
         """Slices of the contraction axis for a product whose output has too few 128 x 128
         tiles to occupy the GPU while K is long (weight gradients: K = batch x sequence)."""
         if dtype is not DType.bfloat16:
             return 1
+        if a_k_contiguous and N <= 32 and M >= 1024 and K % 64 == 0:
+            return 1  # tall products with a few columns have a kernel that splits K by itself
         tiles = ((M + 127) // 128) * ((N + 127) // 128)
         ks = 1
         while tiles * ks < 512 and tiles < 128 and K % (ks * 2 * 64) == 0 and K // (ks * 2) >= 512:
@@ -1125,7 +1127,8 @@ class Planner:
                          out: ir.Value, epi: dict | None = None) -> None:
         """One unbatched product into contiguous storage for ``out``; split along K into fp32
         partial products plus their sum when the output alone gives too few workgroups."""
-        ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32)
+        ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32,
+                           a_k_contiguous=pa[2] == 1)
         dst = self._alloc_value(out)
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)

@@ -930,6 +930,111 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
   gemm_epilogue<TM, TN, WN, true, EPI ? 2 : 0>(acc, g, m0, n0, wm, wn, 0, wave, lane);
 }
 
+// ------------------------------------------------------------------- bf16, N <= 32
+// C[M x N] = alpha * A[M x K] @ B[K x N] with at most 32 columns (the "down" product of a
+// low-rank adapter and its transpose in the backward pass): A is read once and that is all the
+// traffic there is.  One workgroup per 32 rows of A; its eight waves split K, each reads its
+// part of the rows straight from global memory into MFMA fragments (one 32 x 32 accumulator
+// tile; columns past N hold whatever the clamped or padded reads give and are never stored:
+// a column of B only reaches the same column of C), and the eight partial tiles are added
+// through LDS.
+//   B_KC:  B given as [N][K] (K contiguous): fragments come straight from global memory too.
+//   !B_KC: B given as [K][N] (N contiguous, N % 8 == 0): every wave stages its K range in LDS
+//          k-major and reads fragments through the transposing read.
+extern __shared__ __align__(16) u32x4 skinny_lds[];
+
+constexpr int SKN_WAVES = 8;
+
+template <bool B_KC>
+__global__ __launch_bounds__(SKN_WAVES * 64) void gemm_skinny_n_kernel(const GemmArgs g,
+                                                                        int pitch_chunks) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 31, kg = lane >> 5;
+  const uint16_t* A = (const uint16_t*)g.A;
+  const uint16_t* B = (const uint16_t*)g.B;
+  const int64_t row0 = (int64_t)blockIdx.x * 32;
+  const int64_t arow = row0 + li < g.M ? row0 + li : g.M - 1;
+  const uint16_t* ap = A + arow * g.a_rs + 8 * kg;
+  // this wave's 64-wide K chunks
+  const int chunks = (int)(g.K >> 6);
+  const int per = (chunks + SKN_WAVES - 1) / SKN_WAVES;
+  const int c_begin = wave * per;
+  const int c_end = c_begin + per < chunks ? c_begin + per : chunks;
+  float* red = (float*)skinny_lds;                                   // [waves][16 regs][64 lanes]
+  char* stage = (char*)(skinny_lds + SKN_WAVES * 16 * 64 / 4);        // behind the reduction area
+  const int pitch = pitch_chunks * 16;                                // bytes per staged k-row
+  const char* tr_ptr = nullptr;
+  const uint16_t* bp = nullptr;
+  if (B_KC) {
+    const int64_t col = li < g.N ? li : g.N - 1;
+    bp = B + col * g.b_cs + 8 * kg;
+  } else {
+    // stage rows [64 c_begin, 64 c_end) of B; a k-row holds N / 8 chunks (pitch_chunks >= that)
+    const int nch = (int)(g.N >> 3);
+    const int rows = (c_end - c_begin) * 64;
+    for (int t = lane; t < rows * nch; t += 64) {
+      const int k = t / nch, c = t - k * nch;
+      const int64_t gk = (int64_t)c_begin * 64 + k;
+      *(u32x4*)(stage + (size_t)gk * pitch + c * 16) = *(const u32x4*)(B + gk * g.b_rs + c * 8);
+    }
+    // lane p of group q = lane / 16: k-row 8 (q / 2) + p / 4, columns 16 (q % 2) + 4 (p % 4) .. + 4
+    // (every lane of a group takes part in the exchange, also those that point at padding)
+    const int p = lane & 15, q = lane >> 4;
+    const int col0 = 16 * (q & 1) + 4 * (p & 3);
+    tr_ptr = stage + (8 * (q >> 1) + (p >> 2)) * pitch + col0 * 2;
+  }
+  f32x16 acc = (f32x16)(0.f);
+  // the rows of the next chunk are requested before the MFMAs of this one
+  u32x4 an[4], bn[4];
+  auto fetch = [&](int c) {
+    const int64_t k0 = (int64_t)c * 64;
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) an[s4] = *(const u32x4*)(ap + k0 + 16 * s4);
+    if (B_KC) {
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) bn[s4] = *(const u32x4*)(bp + k0 + 16 * s4);
+    }
+  };
+  if (c_begin < c_end) fetch(c_begin);
+  for (int c = c_begin; c < c_end; ++c) {
+    const int64_t k0 = (int64_t)c * 64;
+    bf16x8 fa[4], fb[4];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *(const bf16x8*)&an[s4];
+    if (B_KC) {
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) fb[s4] = *(const bf16x8*)&bn[s4];
+    } else {
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const char* a0 = tr_ptr + (k0 + 16 * s4) * pitch;
+        const s16x4 lo = lds_read_tr(a0), hi = lds_read_tr(a0 + 4 * pitch);
+        const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        fb[s4] = *(const bf16x8*)&u;
+      }
+    }
+    if (c + 1 < c_end) fetch(c + 1);
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s4], fb[s4], acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
+  __syncthreads();
+  if (wave != 0) return;
+  const int64_t col = li;
+  if (col >= g.N) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < SKN_WAVES; ++w) v += red[(w * 16 + r) * 64 + lane];
+    const int64_t row = row0 + 8 * (r >> 2) + 4 * kg + (r & 3);
+    if (row < g.M) nbk_store_from_f32(g.C, row * g.ldc + col, g.dtype_c, v * g.alpha);
+  }
+}
+
 // ---------------------------------------------------------------------------- fp32
 // 128 x 128 x 16 tile, LDS k-major ([k][rows], rows padded by 4 floats).
 template <bool A_KC, bool B_KC>
@@ -1261,6 +1366,31 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   };
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs, a.a_bs2);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs, a.b_bs2);
+  if (d->dtype_ab == NBK_BF16 && d->N <= 32 && d->M >= 1024 && d->K >= 256 && d->K % 64 == 0 &&
+      akc && a.a_vec && d->batch == 1 && d->bias == nullptr && d->residual == nullptr &&
+      d->act == NBK_ACT_NONE && (bkc ? (bool)a.b_vec : (d->b_cs == 1 && d->N % 8 == 0 && a.b_vec))) {
+    // 32 rows per workgroup, K split over its eight waves
+    const int pitch_chunks = d->N <= 16 ? 2 : 4;
+    const size_t red = SKN_WAVES * 16 * 64 * sizeof(float);
+    const size_t stage = bkc ? 0 : (size_t)d->K * pitch_chunks * 16 + 64;
+    if (red + stage <= 160 * 1024 - 512 && (d->M + 31) / 32 <= 0x7fffffff) {
+      dim3 grid((unsigned)((d->M + 31) / 32));
+      if (bkc) {
+        hipLaunchKernelGGL((gemm_skinny_n_kernel<true>), grid, dim3(SKN_WAVES * 64), red, st, a,
+                           pitch_chunks);
+      } else {
+        static bool attr_set = false; /* idempotent, so a race only repeats the call */
+        if (!attr_set) {
+          NBK_HIP(hipFuncSetAttribute((const void*)gemm_skinny_n_kernel<false>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+          attr_set = true;
+        }
+        hipLaunchKernelGGL((gemm_skinny_n_kernel<false>), grid, dim3(SKN_WAVES * 64), red + stage, st, a,
+                           pitch_chunks);
+      }
+      return nbk_check_launch("gemm_skinny_n_kernel");
+    }
+  }
   if (d->dtype_ab == NBK_BF16 && d->K <= 16 && akc && d->batch == 1 && d->N % 8 == 0 &&
       d->ldc % 8 == 0 && ((uintptr_t)d->C & 15) == 0 && ((uintptr_t)d->residual & 15) == 0 &&
       (d->K == 16 ? a.a_vec : d->K == 8 && (d->a_rs % 8 == 0) && ((uintptr_t)d->A & 15) == 0)) {

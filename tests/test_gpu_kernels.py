@@ -160,6 +160,42 @@ def test_gemm_epilogue(hip, dtype, act, shape, res_op):
 
 @pytest.mark.parametrize("b_layout", ["n", "t"])
 @pytest.mark.parametrize("out", ["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(2048, 16, 2048), (1500, 8, 320), (1024, 32, 1024), (4100, 24, 256),
+                                   (3000, 5, 192)])
+def test_gemm_few_columns(hip, b_layout, out, shape):
+    """bf16 products with at most 32 columns (the down-projection of a low-rank adapter and its
+    transpose): rows of A straight into MFMA fragments, K split over the waves of a workgroup."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(13)
+    A = torch.tensor(rng.standard_normal((M, K)) / np.sqrt(K), dtype=torch.bfloat16)
+    B = torch.tensor(rng.standard_normal((K, N)), dtype=torch.bfloat16)
+    odt = torch.bfloat16 if out == "bf16" else torch.float32
+    alpha = 0.75
+    ref = (alpha * (A.double() @ B.double())).numpy()
+    a_dev = A.cuda()
+    b_dev = (B if b_layout == "n" else B.t().contiguous()).cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=odt, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs = K, 1
+    d.b_rs, d.b_cs = (N, 1) if b_layout == "n" else (1, K)
+    d.ldc = N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
+    d.dtype_ab, d.dtype_c = 1, (1 if out == "bf16" else 0)
+    d.alpha = alpha
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    rtol, atol = (2.0 ** -8, 1e-4) if out == "bf16" else (1e-5, 1e-5)
+    err = np.abs(got - ref) - rtol * np.abs(ref)
+    assert err.max() <= atol, err.max()
+
+
+@pytest.mark.parametrize("b_layout", ["n", "t"])
+@pytest.mark.parametrize("out", ["bf16", "f32"])
 @pytest.mark.parametrize("shape", [(4096, 512, 16), (3001, 1032, 16), (2048, 1024, 8), (1100, 2048, 13)])
 def test_gemm_low_rank_product(hip, b_layout, out, shape):
     """bf16 products with a contraction of at most 16 (the up-projection of a low-rank
