@@ -623,16 +623,10 @@ struct DirectLoader {
 // KSS: k-steps (of 16) per fragment set.  A step of KSS k-steps is multiplied out of one
 // set while the other is filled for the next step; small wave tiles take 2, so that a read has
 // more than a handful of MFMAs to land.
-// KSPLIT: 1, or 2 for the 128 x 128 tile: its four waves then form two groups that take the
-// even and the odd k-steps of every tile, each group covering the whole tile with two
-// 128 x 64 wave tiles (6 fragment reads per 8 MFMAs instead of 4 per 4: the small tile is
-// bound by LDS reads), and the two partial sums are added through LDS before the epilogue.
-template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS, int KSPLIT>
-__global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const GemmArgs g) {
-  static_assert(KSPLIT == 1 || (KSPLIT == 2 && NW == 4 && BM == 128 && BN == 128), "k split");
-  constexpr int GW = NW / KSPLIT;                         // waves per k-group
-  constexpr int WGM = KSPLIT == 1 ? 2 : 1, WGN = GW / WGM;
-  constexpr int WM = BM / WGM, WN = BN / WGN;  // wave tile
+template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g) {
+  constexpr int WGN = NW / 2;
+  constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int CA = BM * 8, TILE_CHUNKS = (BM + BN) * 8;
   int tm_i, tn_i;
@@ -644,8 +638,7 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
   const int64_t c_off = bo * g.c_bs + bi * g.c_bs2;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kpar = wave / GW;  // k-group of this wave
-  const int wm = (wave % GW / WGN) * WM, wn = (wave % WGN) * WN;
+  const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
   const int li = lane & 31, kg = lane >> 5;
 
   f32x16 acc[TM][TN];
@@ -667,7 +660,6 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
   //   row-contiguous: byte address of this lane's 8 bytes in the transposing read of k-step 0,
   //     first half; the k-step and the half are constant offsets.  Lane p of group q = lane / 16
   //     points at k-row 8 (q / 2) + p / 4, rows 16 (q % 2) + 4 (p % 4) .. + 4 of the block.
-  //   (with two k-groups, group 1 starts one k-step further: folded into the addresses)
   int a_addr[TM], b_addr[TN];
   {
     const int p = lane & 15, q = lane >> 4;
@@ -675,24 +667,21 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int row = wm + i * 32 + li;
-      if (A_KC) a_addr[i] = ((row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16) ^ (kpar * 32);
-      else
-        a_addr[i] = (kl + 16 * kpar) * (BM * 2) + ((((wm >> 4) + 2 * i + (q & 1)) ^ sx) * 32) +
-                    8 * (p & 3);
+      if (A_KC) a_addr[i] = (row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
+      else a_addr[i] = kl * (BM * 2) + ((((wm >> 4) + 2 * i + (q & 1)) ^ sx) * 32) + 8 * (p & 3);
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int row = wn + j * 32 + li;
-      if (B_KC)
-        b_addr[j] = ((CA + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16) ^ (kpar * 32);
+      if (B_KC) b_addr[j] = (CA + row * 8 + (kg ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
       else
-        b_addr[j] = CA * 16 + (kl + 16 * kpar) * (BN * 2) +
-                    ((((wn >> 4) + 2 * j + (q & 1)) ^ sx) * 32) + 8 * (p & 3);
+        b_addr[j] = CA * 16 + kl * (BN * 2) + ((((wn >> 4) + 2 * j + (q & 1)) ^ sx) * 32) +
+                    8 * (p & 3);
     }
   }
 
   bf16x8 fa[2][KSS * TM], fb[2][KSS * TN];
-  constexpr int NSTEP = 4 / (KSS * KSPLIT);
+  constexpr int NSTEP = 4 / KSS;
   static_assert(NSTEP >= 2 && NSTEP % 2 == 0, "steps per tile");
   constexpr int NFRAG = KSS * (TM + TN), NMFMA = KSS * TM * TN;  // per step
   // read fragment r of step `step` from `tile` into set SET; order of use by the MFMAs
@@ -701,7 +690,7 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
     constexpr int SET = decltype(set)::value;
     constexpr int KL = decltype(r)::value / (TM + TN), R0 = decltype(r)::value % (TM + TN);
     constexpr int R = R0 == 0 ? 0 : (R0 <= TN ? TM + R0 - 1 : R0 - TN);
-    const int ks = KSPLIT * (step * KSS + KL);  // relative to the group's first k-step
+    const int ks = step * KSS + KL;
     if constexpr (R < TM) {
       if constexpr (A_KC) {
         int sel = ks * 32;
@@ -830,50 +819,7 @@ __global__ __launch_bounds__(NW * 64, KSPLIT) void gemm_bf16_dl_kernel(const Gem
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no copy may land in a slab
   __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
-  if constexpr (KSPLIT == 1) {
-    gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
-  } else {
-    // The two waves that hold partial sums of the same 128 x 64 half swap halves of it: group
-    // 0 keeps row blocks 0-1 and hands over 2-3, group 1 the reverse.  Each wave ends up
-    // with a finished 64 x 64 tile.  float4 units, [wave][block][r / 4][lane]: conflict-free.
-    float4* ex = (float4*)gemm_lds + wave * (4 * 4 * 64) + lane;
-    const float4* px = (const float4*)gemm_lds + (wave ^ GW) * (4 * 4 * 64) + lane;
-    f32x16 fin[2][TN];
-    auto give = [&](auto first) {
-      constexpr int F = decltype(first)::value;
-      static_for<2>([&](auto ii) {
-        static_for<TN>([&](auto j) {
-          const f32x16 a = acc[F + decltype(ii)::value][decltype(j)::value];
-          constexpr int blk = decltype(ii)::value * TN + decltype(j)::value;
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4)
-            ex[(blk * 4 + r4) * 64] = make_float4(a[r4 * 4], a[r4 * 4 + 1], a[r4 * 4 + 2], a[r4 * 4 + 3]);
-        });
-      });
-    };
-    auto take = [&](auto first) {
-      constexpr int F = decltype(first)::value;
-      static_for<2>([&](auto ii) {
-        static_for<TN>([&](auto j) {
-          f32x16 a = acc[F + decltype(ii)::value][decltype(j)::value];
-          constexpr int blk = decltype(ii)::value * TN + decltype(j)::value;
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const float4 v = px[(blk * 4 + r4) * 64];
-            a[r4 * 4] += v.x; a[r4 * 4 + 1] += v.y; a[r4 * 4 + 2] += v.z; a[r4 * 4 + 3] += v.w;
-          }
-          fin[decltype(ii)::value][decltype(j)::value] = a;
-        });
-      });
-    };
-    if (kpar == 0) give(std::integral_constant<int, 2>{});
-    else give(std::integral_constant<int, 0>{});
-    __syncthreads();
-    if (kpar == 0) take(std::integral_constant<int, 0>{});
-    else take(std::integral_constant<int, 2>{});
-    __syncthreads();  // the slabs below overlap the exchange area
-    gemm_epilogue<2, TN, WN, true, EPI>(fin, g, m0, n0, kpar * 64, wn, c_off, wave, lane);
-  }
+  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
 }
 
 // ------------------------------------------------------------------- bf16, K <= 16
@@ -1285,7 +1231,7 @@ static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hip
   return nbk_check_launch("gemm_bf16_kernel");
 }
 
-template <int BM, int BN, int NW, int KSS, int KSPLIT = 1>
+template <int BM, int BN, int NW, int KSS>
 static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
   GemmArgs g = a;
   g.tiles_m = (int)((a.M + BM - 1) / BM);
@@ -1297,7 +1243,7 @@ static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, 
   const int epi = (a.residual != nullptr || a.act != NBK_ACT_NONE) ? 2 : (a.bias != nullptr ? 1 : 0);
 #define NBK_LAUNCH_DL(AK, BK_, EP)                                                            \
   do {                                                                                        \
-    auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS, KSPLIT>;                                 \
+    auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS>;                                 \
     static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
     if (!attr_set) {                                                                          \
       NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -1426,9 +1372,6 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
     // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
     // 128 x 128 workgroups hide it better)
-    // (two k-groups per workgroup: 3-13 % faster from K = 2048 on, 2-4 % slower at K = 1024,
-    // where the exchange of the partial sums is a larger part of the whole)
-    if (d->K >= 2048) return launch_bf16_dl<128, 128, 4, 1, 2>(a, akc, bkc, d->batch, st);
     return launch_bf16_dl<128, 128, 4, 1>(a, akc, bkc, d->batch, st);
   }
   a.tiles_m = (int)((d->M + 127) / 128);

@@ -87,8 +87,8 @@ def test_gemm(hip, dtype, layout, shape):
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
 @pytest.mark.parametrize("shape", [(384, 256, 2048), (1000, 520, 4096)])
 def test_gemm_long_k_small_output(hip, layout, shape):
-    """bf16 products whose 128 x 128 tiles split every K tile between two groups of waves
-    (K >= 2048): the partial sums meet in LDS before the result is rounded."""
+    """bf16 products with a long contraction and few 128 x 128 tiles (the shapes the planner
+    would otherwise split along K), through the C ABI in one piece."""
     from nabla_amd.backend import lib
     M, N, K = shape
     rng = np.random.default_rng(5)
@@ -119,7 +119,7 @@ def test_gemm_long_k_small_output(hip, layout, shape):
 @pytest.mark.parametrize("act", [0, 1, 2])
 @pytest.mark.parametrize("shape", [(256, 384, 128),      # 128 x 128 tiles
                                    (300, 200, 72),       # guarded kernel (K % 64 != 0)
-                                   (640, 520, 2048),     # 128 x 128 tiles, two k-groups
+                                   (640, 520, 2048),     # 128 x 128 tiles, long K
                                    (4096, 2560, 192)])   # 256 x 256 tiles
 @pytest.mark.parametrize("res_op", [0, 1])
 def test_gemm_epilogue(hip, dtype, act, shape, res_op):
