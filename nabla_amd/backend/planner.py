@@ -597,6 +597,88 @@ class Planner:
         return self._materialize(self._resolve(v))
 
     # ................................................................ build
+    _REMAT_FNS = ("eq", "ne", "gt", "ge", "lt", "le", "mov", "not", "and", "or")
+
+    def _rematerialize_masks(self) -> None:
+        """A large tensor that is a cheap function of small ones (a one-hot: labels compared
+        with an iota, cast to the compute type; a causal or padding mask) and has readers in
+        several places is not worth a trip through memory: every reader after the first gets
+        its own copy of the few nodes that make it, which then fuse into that reader's kernel.
+        Cheap means: comparisons, logic and casts only, over broadcasts of values at least 64
+        times smaller than the result."""
+        nodes = self._live_nodes()
+        users: dict[int, list[ir.Node]] = {}
+        for n in nodes:
+            for i in n.inputs:
+                if not users.get(i.id) or users[i.id][-1] is not n:
+                    users.setdefault(i.id, []).append(n)
+        out_ids = {v.id for v in self.outputs}
+        clones_before: dict[int, list[ir.Node]] = {}  # pos of a reader -> nodes to put before it
+        for n in nodes:
+            if not (n.kind == "ew" and n.fn in self._REMAT_FNS):
+                continue
+            v = n.outputs[0]
+            readers = users.get(v.id, [])
+            big = _numel(v.shape)
+            if len(readers) < 2 or v.id in out_ids or big < (1 << 22):
+                continue
+            chain: list[ir.Node] = []
+            ok, stack, seen = True, [n], set()
+            while stack and ok:
+                m = stack.pop()
+                if m.pos in seen:
+                    continue
+                seen.add(m.pos)
+                chain.append(m)
+                if len(chain) > 8:
+                    ok = False
+                    break
+                for i in m.inputs:
+                    if _numel(i.shape) * 64 <= big:
+                        continue  # a small leaf: read again by the copy
+                    pn = i.node
+                    if pn.kind in ("broadcast", "reshape") or (pn.kind == "ew" and pn.fn in self._REMAT_FNS):
+                        stack.append(pn)
+                    else:
+                        ok = False
+                        break
+            if not ok:
+                continue
+            chain.sort(key=lambda m: m.pos)
+            for reader in readers[1:]:
+                if reader.pos in seen:
+                    continue
+                vmap: dict[int, ir.Value] = {}
+                made = []
+                for m in chain:
+                    attrs = dict(m.attrs or {})
+                    ins = [vmap.get(i.id, i) for i in m.inputs]
+                    if "operands" in attrs:
+                        attrs["operands"] = tuple(vmap.get(o.id, o) if isinstance(o, ir.Value) else o
+                                                  for o in attrs["operands"])
+                    c = ir.Node(m.kind, m.fn, ins, attrs, -1)
+                    for k, o in enumerate(m.outputs):
+                        nv = ir.Value(o.shape, o.dtype, c, k, self.b._n_values)
+                        self.b._n_values += 1
+                        c.outputs.append(nv)
+                        vmap[o.id] = nv
+                    made.append(c)
+                reader.inputs = [vmap.get(i.id, i) if i.id == v.id else i for i in reader.inputs]
+                if reader.attrs and "operands" in reader.attrs:
+                    reader.attrs = dict(reader.attrs, operands=tuple(
+                        vmap[v.id] if isinstance(o, ir.Value) and o.id == v.id else o
+                        for o in reader.attrs["operands"]))
+                clones_before.setdefault(id(reader), []).extend(made)
+        if not clones_before:
+            return
+        out: list[ir.Node] = []
+        for n in self.b.nodes:
+            out.extend(clones_before.get(id(n), ()))
+            out.append(n)
+        for k, n in enumerate(out):
+            n.pos = k
+        self.b.nodes[:] = out
+
     def _fold_bias_into_matmul(self) -> None:
         """``x @ W + b`` with ``b`` a row vector broadcast over the leading axes: the add node
         itself turns into the matmul node with the bias as a third input
@@ -1623,7 +1705,7 @@ class _RowCodegen:
         # registers (16 in all), which halves the workgroup and its barrier cost
         cpt_max = 8
         n_in = max(1, len({i[2] for i in ins if i[0] == isa.LDG}))
-        while cpt_max > 2 and cpt_max * n_in > 16:
+        while cpt_max > 1 and cpt_max * n_in > 16:
             cpt_max //= 2
         block = 64
         while block < isa.MAX_BLOCK and block * cpt_max < chunks:
@@ -1756,6 +1838,7 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     last = None
     # graph rewrites happen once, before the attempts below share the builder
     pre = Planner(builder, outputs)
+    pre._rematerialize_masks()
     pre._fold_bias_into_matmul()
     outputs = pre.outputs
     for limit in (28, 16, 8, 4, 1):
