@@ -1355,8 +1355,12 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     return nbk_check_launch("gemm_skinny_k_kernel");
   }
   if (d->dtype_ab == NBK_BF16) {
+    // (the direct kernel keeps per-lane byte offsets within a tile in 32 bits: 256 rows or
+    // 64 k-rows times the stride)
+    const int64_t a_stride = akc ? d->a_rs : d->a_cs, b_stride = bkc ? d->b_cs : d->b_rs;
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
-                      (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8;
+                      (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8 &&
+                      a_stride >= 0 && b_stride >= 0 && a_stride < (1 << 22) && b_stride < (1 << 22);
     if (!fast) return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);
     // 256 x 256 tiles run at about twice the rate of 128 x 128 ones per CU, one workgroup
     // per CU at a time: take them when the rounds of workgroups they need are at least
