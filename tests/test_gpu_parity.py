@@ -398,6 +398,12 @@ def test_graph_replay_matches_eager_every_time(hip):
     """A compiled step called again on the same buffers is recorded once and replayed; every
     replay is checked against the oracle, with unrelated eager work and synchronisation between
     the replays, and a call on new buffers falls back to plain launches."""
+    import gc
+    import torch
+    # (a replay needs the allocator to hand the step the same output block again: start from
+    # an empty cache so that blocks left behind by earlier tests do not take turns)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
     t = oc.c1_inputs(64, 96, 48, 10, seed=31)
     t["b1"] = np.random.default_rng(2).uniform(-0.05, 0.05, t["b1"].shape).astype(np.float32)
     wl, wg = oc.c1_reference(**t)
@@ -411,7 +417,8 @@ def test_graph_replay_matches_eager_every_time(hip):
         assert abs(got[0] - wl) <= F32_TOL * abs(wl) + 1e-9, it
         for g, w in zip(got[1:], wg):
             assert relerr(g, w) < F32_TOL, it
-        del loss, grads
+        del loss, grads, got
+        gc.collect()  # (graph nodes of the step form cycles: drop them now, not when the collector likes)
         # unrelated work between replays
         np.testing.assert_array_equal((other * 2.0 + float(it)).numpy(), np.arange(12) * 2.0 + it)
     assert hip.graph_replays > before, "the repeated step was never replayed as a graph"
