@@ -81,7 +81,12 @@ def tree_flatten(tree: Any, is_leaf: Callable[[Any], bool] | None = None):
         leaves.append(node)
         return _LEAF_DEF
 
-    treedef = go(tree)
+    try:
+        treedef = go(tree)
+    finally:
+        # the closure refers to itself: unless that is undone it lives, and `leaves` with it,
+        # until the cycle collector runs (device memory of dropped tensors would wait for that)
+        go = None
     return leaves, treedef
 
 
