@@ -134,7 +134,8 @@ class Tensor:
             arr = array
             if arr.dtype == np.float64:
                 arr = arr.astype(np.float32)
-            t = torch.from_numpy(np.ascontiguousarray(arr))
+            # ascontiguousarray promotes a 0-d array to one dimension; keep the caller's shape
+            t = torch.from_numpy(np.ascontiguousarray(arr).reshape(arr.shape))
         elif hasattr(array, "__dlpack__"):
             t = torch.from_dlpack(array)
         else:
@@ -160,7 +161,8 @@ class Tensor:
             arr = np.asarray(value)
             if arr.dtype == np.float64:
                 arr = arr.astype(np.float32)
-            t = torch.from_numpy(np.ascontiguousarray(arr))
+            # ascontiguousarray promotes a 0-d array to one dimension; keep the caller's shape
+            t = torch.from_numpy(np.ascontiguousarray(arr).reshape(arr.shape))
         if dtype is not None and t.dtype != dtype.to_torch():
             t = t.to(dtype.to_torch())
         return cls._from_torch(t, device)

@@ -4,7 +4,7 @@ from .binary import add, div, matmul, mul, pow, sub
 from .comparison import (equal, greater, greater_equal, less, less_equal, logical_and,
                          logical_not, logical_or, not_equal)
 from .control_flow import where
-from .convolution import conv2d
+from .convolution import conv2d, conv2d_transpose
 from .creation import (arange, constant, full, full_like, ones, ones_like, tril, triu, zeros,
                        zeros_like)
 from .pooling import avg_pool2d, max_pool2d

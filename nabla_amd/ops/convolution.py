@@ -57,6 +57,17 @@ def _out_hw(x_shape, w_shape, stride, padding) -> tuple[int, int]:
     return ho, wo
 
 
+def _transpose_out_hw(x_shape, w_shape, stride, padding) -> tuple[int, int]:
+    """Output size of the transposed convolution with dilation 1 and no output padding
+    (convolution.py:140-160)."""
+    pt, pb, pl, pr = padding
+    ho = (x_shape[1] - 1) * stride[0] - pt - pb + w_shape[0]
+    wo = (x_shape[2] - 1) * stride[1] - pl - pr + w_shape[1]
+    if ho <= 0 or wo <= 0:
+        raise ValueError(f"Non-positive conv2d_transpose output size H={ho}, W={wo}.")
+    return ho, wo
+
+
 class Conv2DOp(Operation):
     @property
     def name(self) -> str:
@@ -132,7 +143,31 @@ class Conv2DFilterGradOp(Operation):
         return [g_x, g_dy]
 
 
+
+class Conv2DTransposeOp(Conv2DInputGradOp):
+    """``conv2d_transpose`` (nabla/ops/convolution.py:424-566): ``x`` [N,H,W,Cin] and a filter
+    [R,S,Cout,Cin] -> [N,Ho,Wo,Cout].  It is the input gradient of ``conv2d`` with the same
+    filter read as HWIO, so it runs on the dgrad kernel and inherits its derivative rules
+    (dX: a forward convolution of the cotangent; dW: a filter gradient)."""
+
+    @property
+    def name(self) -> str:
+        return "conv2d_transpose"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x, w = args[0], args[1]
+        ho, wo = _transpose_out_hw(x.shape, w.shape, kwargs["stride"], kwargs["padding"])
+        return [(x.shape[0], ho, wo, w.shape[2])], [x.dtype], [x.device]
+
+    def kernel(self, args, kwargs):
+        x, w = args[0], args[1]
+        ho, wo = _transpose_out_hw(x.shape, w.shape, kwargs["stride"], kwargs["padding"])
+        return [ir.conv2d_dgrad(x, w, (x.shape[0], ho, wo, w.shape[2]), kwargs["stride"],
+                                kwargs["padding"])]
+
+
 _conv2d_op = Conv2DOp()
+_conv2d_transpose_op = Conv2DTransposeOp()
 _conv2d_dgrad_op = Conv2DInputGradOp()
 _conv2d_wgrad_op = Conv2DFilterGradOp()
 
@@ -176,3 +211,45 @@ def conv2d(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0, 0, 0), g
     kwargs = {"stride": norm_stride, "padding": norm_padding}
     args = [x, filter] if bias_t is None else [x, filter, bias_t]
     return _conv2d_op(args, kwargs)[0]
+
+
+def conv2d_transpose(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0, 0, 0),  # noqa: A002
+                     output_paddings=(0, 0), bias=None, input_layout: Any = None,
+                     filter_layout: Any = None) -> Tensor:
+    """Transposed 2-D convolution (convolution.py:699-787): ``x`` [N,H,W,Cin], ``filter``
+    [R,S,Cout,Cin] (channels the other way round than ``conv2d``), optional ``bias`` [Cout].
+    The same argument checks and messages as the reference; dilation and output padding other
+    than the defaults are rejected, as there (762-763 for the output padding)."""
+    x = ensure_tensor(x)
+    filter = ensure_tensor(filter)
+    bias_t = ensure_tensor(bias) if bias is not None else None
+    if len(x.shape) != 4 or len(filter.shape) != 4:
+        raise ValueError(
+            f"conv2d_transpose expects rank-4 tensors, got x={tuple(x.shape)}, filter={tuple(filter.shape)}"
+        )
+    if input_layout is not None or filter_layout is not None:
+        raise ValueError("conv2d_transpose currently supports only the default NHWC layouts")
+    norm_stride = _normalize_2tuple(stride, "stride")
+    norm_dilation = _normalize_2tuple(dilation, "dilation")
+    norm_padding = _normalize_4padding(padding)
+    norm_out_pad = _normalize_2tuple(output_paddings, "output_paddings")
+    _require_all_positive_2tuple(norm_stride, "stride")
+    _require_all_positive_2tuple(norm_dilation, "dilation")
+    _require_all_nonnegative(norm_padding, "padding")
+    _require_all_nonnegative(norm_out_pad, "output_paddings")
+    if norm_out_pad != (0, 0):
+        raise ValueError("conv2d_transpose currently supports only output_paddings=(0, 0)")
+    if norm_dilation != (1, 1):
+        raise ValueError("conv2d_transpose currently supports only dilation=(1, 1)")
+    c_in, c_out, c_in_w = x.shape[-1], filter.shape[2], filter.shape[3]
+    if c_in != c_in_w:
+        raise ValueError(f"Input channels ({c_in}) must match filter input channels ({c_in_w})")
+    if bias_t is not None:
+        if len(bias_t.shape) != 1:
+            raise ValueError(
+                f"conv2d_transpose bias must be rank-1 [C_out], got shape={tuple(bias_t.shape)}")
+        if bias_t.shape[0] != c_out:
+            raise ValueError(
+                f"conv2d_transpose bias size ({bias_t.shape[0]}) must match filter C_out ({c_out})")
+    y = _conv2d_transpose_op([x, filter], {"stride": norm_stride, "padding": norm_padding})[0]
+    return y if bias_t is None else y + bias_t

@@ -1,0 +1,174 @@
+"""``jacrev`` and ``jacfwd`` (nabla/transforms/jacrev.py:27-115, jacfwd.py:32-119).
+
+Both walk the standard basis one direction at a time, as the reference does (jacrev.py:78-82
+calls the pullback once per output element, jacfwd.py:81-104 calls ``jvp`` once per input
+element), and stack the results.  Here the forward trace is captured once for ``jacrev``
+(one ``vjp``) and every pullback is a replay over it; all rows are realised together, so
+the backward programs of all directions land in one plan.
+
+The Jacobian of a function with one output tensor has shape ``(*out_shape, *in_shape)``;
+several differentiated arguments give a tuple of Jacobians.  Several output tensors raise
+``NotImplementedError`` with the reference's message (jacrev.py:191-194, jacfwd.py:189-192).
+"""
+from __future__ import annotations
+
+from typing import Any, Callable
+
+import numpy as np
+
+from ..core import pytree
+from ..core.tensor import Tensor
+from .jvp import jvp
+from .vjp import vjp
+
+
+def resolve_argnums(argnums, n_args: int) -> tuple[int, ...]:
+    """``None`` → every argument; negative indices count from the end
+    (nabla/transforms/utils.py:52-67)."""
+    if argnums is None:
+        sel = tuple(range(n_args))
+    elif isinstance(argnums, int):
+        sel = (argnums,)
+    else:
+        sel = tuple(argnums)
+    norm = tuple(a if a >= 0 else n_args + a for a in sel)
+    for a in norm:
+        if not 0 <= a < n_args:
+            raise ValueError(f"argnum {a} out of bounds for {n_args} arguments")
+    return norm
+
+
+def _partial(fn: Callable, argnums, args: tuple):
+    """The differentiated arguments and ``fn`` with the others held fixed
+    (nabla/transforms/utils.py:112-127)."""
+    norm = resolve_argnums(argnums, len(args))
+    diff_args = tuple(args[i] for i in norm)
+
+    def partial_func(*inner):
+        full = list(args)
+        for idx, a in zip(norm, inner):
+            full[idx] = a
+        return fn(*full)
+
+    return diff_args, partial_func
+
+
+def _tensor_leaves(tree: Any):
+    return pytree.tree_flatten(tree, is_leaf=lambda x: isinstance(x, Tensor))
+
+
+def _numel(t: Tensor) -> int:
+    n = 1
+    for d in t.shape:
+        n *= int(d)
+    return max(n, 1)
+
+
+def _one_hot_like(t: Tensor, j: int | None) -> Tensor:
+    """A tensor of ``t``'s shape and dtype that is one at flat position ``j`` (row-major) and
+    zero elsewhere; all zeros for ``j = None`` (nabla/transforms/utils.py:130-156 builds the
+    same vectors as rows of one host array)."""
+    sh = tuple(int(d) for d in t.shape)
+    a = np.zeros(max(int(np.prod(sh, dtype=np.int64)), 1), dtype=np.float32)
+    if j is not None:
+        a[j] = 1.0
+    return Tensor.constant(a.reshape(sh), dtype=t.dtype)
+
+
+def _basis(flat: list[Tensor]):
+    """For every element of every tensor in ``flat``, the list of per-tensor directions that
+    selects it."""
+    sizes = [_numel(t) for t in flat]
+    for k, n in enumerate(sizes):
+        for j in range(n):
+            yield [_one_hot_like(t, j if i == k else None) for i, t in enumerate(flat)]
+
+
+_MULTI_OUT = ("{} with multiple output tensors is not yet supported. "
+              "Wrap your function to return a single tensor.")
+
+
+def jacrev(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
+    """Jacobian by reverse mode: one pullback per output element."""
+    from ..ops.view import reshape, stack
+
+    def jacrev_fn(*args: Any) -> Any:
+        diff_args, partial_func = _partial(fn, argnums, args)
+        if has_aux:
+            output, pullback, aux = vjp(partial_func, *diff_args, has_aux=True)
+        else:
+            output, pullback = vjp(partial_func, *diff_args)
+            aux = None
+        flat_out, out_td = _tensor_leaves(output)
+        if len(flat_out) != 1:
+            raise NotImplementedError(_MULTI_OUT.format("jacrev"))
+        flat_in, _ = _tensor_leaves(diff_args)
+        if len(flat_in) != len(diff_args):
+            raise NotImplementedError("jacrev: every differentiated argument must be one tensor")
+        out_shape = tuple(int(d) for d in flat_out[0].shape)
+
+        rows: list[list[Tensor]] = [[] for _ in flat_in]
+        for direction in _basis(flat_out):
+            grads = pullback(pytree.tree_unflatten(out_td, direction))
+            g_flat, _ = _tensor_leaves(grads)
+            for k, g in enumerate(g_flat):
+                rows[k].append(g)
+
+        jacs = []
+        for r, x in zip(rows, flat_in):
+            in_shape = tuple(int(d) for d in x.shape)
+            j = r[0] if len(r) == 1 else stack(r, axis=0)
+            jacs.append(reshape(j, out_shape + in_shape))
+        jac = jacs[0] if len(jacs) == 1 else tuple(jacs)
+        return (jac, aux) if has_aux else jac
+
+    return jacrev_fn
+
+
+def jacfwd(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
+    """Jacobian by forward mode: one ``jvp`` per input element."""
+    from ..ops.view import permute, reshape, stack
+
+    def jacfwd_fn(*args: Any) -> Any:
+        diff_args, partial_func = _partial(fn, argnums, args)
+        flat_in, in_td = _tensor_leaves(diff_args)
+        if len(flat_in) != len(diff_args):
+            raise NotImplementedError("jacfwd: every differentiated argument must be one tensor")
+        sizes = [_numel(t) for t in flat_in]
+
+        cols: list[Tensor] = []
+        aux = None
+        out_shape: tuple[int, ...] = ()
+        for direction in _basis(flat_in):
+            tangents = pytree.tree_unflatten(in_td, direction)
+            if not isinstance(tangents, tuple):
+                tangents = (tangents,)
+            if has_aux:
+                out, tan, aux = jvp(partial_func, tuple(diff_args), tangents, has_aux=True)
+            else:
+                out, tan = jvp(partial_func, tuple(diff_args), tangents)
+            t_flat, _ = _tensor_leaves(tan)
+            if len(t_flat) != 1:
+                raise NotImplementedError(_MULTI_OUT.format("jacfwd"))
+            out_shape = tuple(int(d) for d in t_flat[0].shape)
+            cols.append(t_flat[0])
+
+        jacs = []
+        off = 0
+        for x, n in zip(flat_in, sizes):
+            in_shape = tuple(int(d) for d in x.shape)
+            chunk = cols[off:off + n]
+            off += n
+            j = chunk[0] if n == 1 else stack(chunk, axis=0)
+            j = reshape(j, in_shape + out_shape)
+            if in_shape and out_shape:
+                ni, no = len(in_shape), len(out_shape)
+                j = permute(j, tuple(range(ni, ni + no)) + tuple(range(ni)))
+            jacs.append(j)
+        jac = jacs[0] if len(jacs) == 1 else tuple(jacs)
+        return (jac, aux) if has_aux else jac
+
+    return jacfwd_fn
+
+
+__all__ = ["jacrev", "jacfwd"]

@@ -456,6 +456,53 @@ def conv2d(x, w, bias=None, stride=(1, 1), padding=(0, 0, 0, 0)) -> V:
     return V(y, parents, vjp)
 
 
+def conv2d_transpose(x, w, bias=None, stride=(1, 1), padding=(0, 0, 0, 0)) -> V:
+    """convolution.py:424-566, 699-787: transposed convolution of NHWC ``x`` [N,H,W,Cin] with
+    a filter [R,S,Cout,Cin].  Every input pixel scatters ``x[n,i,j,:] @ w[r,s].T`` to output
+    position (i*sh - pt + r, j*sw - pl + s); the output has (H-1)*sh - pt - pb + R rows
+    (convolution.py:140-160 with dilation 1 and no output padding).  Gradients as in 522-566:
+    dX is the forward convolution of the cotangent with the same filter, dW correlates the
+    padded cotangent with x, db sums the cotangent over N, H, W."""
+    x, w = _v(x), _v(w)
+    pt, pb, pl, pr = padding
+    sh, sw = stride
+    n, h, wd, cin = x.a.shape
+    r, s, cout, _ = w.a.shape
+    hf, wf = (h - 1) * sh + r, (wd - 1) * sw + s          # size before the padding is cut off
+    ho, wo = hf - pt - pb, wf - pl - pr
+    if ho <= 0 or wo <= 0:
+        raise ValueError(f"Non-positive conv2d_transpose output size H={ho}, W={wo}.")
+
+    def taps():
+        for i in range(r):
+            for j in range(s):
+                yield i, j, slice(i, i + (h - 1) * sh + 1, sh), slice(j, j + (wd - 1) * sw + 1, sw)
+
+    full = np.zeros((n, hf, wf, cout), dtype=np.result_type(x.a, w.a))
+    for i, j, hs, ws in taps():
+        full[:, hs, ws, :] += x.a @ w.a[i, j].T
+    y = full[:, pt:pt + ho, pl:pl + wo, :]
+    parents = [x, w]
+    if bias is not None:
+        bias = _v(bias)
+        y = y + bias.a
+        parents.append(bias)
+
+    def vjp(g):
+        gp = np.pad(g, ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+        gx = np.zeros_like(x.a, dtype=g.dtype)
+        gw = np.zeros_like(w.a, dtype=g.dtype)
+        for i, j, hs, ws in taps():
+            gx += gp[:, hs, ws, :] @ w.a[i, j]
+            gw[i, j] = np.tensordot(gp[:, hs, ws, :], x.a, axes=([0, 1, 2], [0, 1, 2]))
+        out = [gx, gw]
+        if bias is not None:
+            out.append(g.sum(axis=(0, 1, 2)))
+        return tuple(out)
+
+    return V(y, parents, vjp)
+
+
 def max_pool2d(x, kernel, stride=None, padding=(0, 0, 0, 0)) -> V:
     """pooling.py:53-137: per output pixel, reduce_max over the window clipped to
     the image; the gradient follows reduce_max's tie rule per window."""

@@ -297,6 +297,31 @@ def test_conv2d_forward_and_grads(hip, cfg):
     assert relerr(gw.numpy(), wgw) < 5e-5
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(xs=(1, 4, 5, 2), ws=(3, 2, 6, 2), stride=(2, 1), pad=(1, 0, 1, 0)),     # the reference's vjp case
+    dict(xs=(1, 4, 4, 2), ws=(3, 3, 5, 2), stride=(1, 1), pad=(1, 1, 1, 1)),     # ... and its jvp case
+    dict(xs=(4, 16, 16, 64), ws=(4, 4, 32, 64), stride=(2, 2), pad=(1, 1, 1, 1)),  # a decoder upsampling layer
+])
+def test_conv2d_transpose_forward_and_grads(hip, cfg):
+    """conv2d_transpose (the dgrad kernel behind a public op), its bias and all three gradients
+    against the float64 oracle."""
+    from oracle import ops as O
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal(cfg["xs"]).astype(np.float32)
+    w = (rng.standard_normal(cfg["ws"]) / np.sqrt(cfg["ws"][0] * cfg["ws"][1] * cfg["ws"][3])).astype(np.float32)
+    b = rng.standard_normal(cfg["ws"][2]).astype(np.float32)
+    kw = dict(stride=cfg["stride"], padding=cfg["pad"])
+    X, W, B = (O.V(a.astype(np.float64)) for a in (x, w, b))
+    out = O.conv2d_transpose(X, W, B, **kw)
+    want = O.grad_of(O.reduce_sum(out * out), [X, W, B])
+    f = lambda x, w, b: nb.reduce_sum(nb.conv2d_transpose(x, w, bias=b, **kw) ** 2)
+    got = nb.conv2d_transpose(T(x), T(w), bias=T(b), **kw)
+    assert tuple(got.shape) == out.a.shape
+    assert relerr(got.numpy(), out.a) < F32_TOL
+    for g, wg in zip(nb.grad(f, argnums=(0, 1, 2))(T(x), T(w), T(b)), want):
+        assert relerr(g.numpy(), wg) < 5e-5
+
+
 # ---- user kernels ---------------------------------------------------------------------------------
 class AddOneCustomOp(nb.ops.UnaryOperation):
     """Same shape as the reference's example op (tests/mojo/op.py:15-27)."""
@@ -494,6 +519,26 @@ def test_jvp_on_device_against_oracle_central_differences(hip):
     lhs = float((tan.numpy().astype(np.float64) * u).sum())
     rhs = sum(float((g.numpy().astype(np.float64) * v).sum()) for g, v in zip(gs, vs))
     assert abs(lhs - rhs) <= 2e-4 * max(abs(lhs), abs(rhs), 1e-3)
+
+
+@pytest.mark.parametrize("jac", ["rev", "fwd"])
+def test_jacobians_on_device_against_torch_cpu(hip, jac):
+    """jacrev / jacfwd of softmax(gelu(x @ w)) on the device against torch's CPU Jacobian in
+    float64, and the Hessian of sum(x^3) (forward over reverse) against diag(6x)."""
+    rng = np.random.default_rng(47)
+    x, w = rng.standard_normal((3, 5)), rng.standard_normal((5, 4))
+    J = nb.jacrev if jac == "rev" else nb.jacfwd
+    got = J(lambda a, b: nb.softmax(nb.gelu(nb.matmul(a, b)) * 0.7, axis=-1), argnums=(0, 1))(
+        T(x.astype(np.float32)), T(w.astype(np.float32)))
+    want = torch.autograd.functional.jacobian(
+        lambda a, b: torch.softmax(torch.nn.functional.gelu(a @ b) * 0.7, dim=-1),
+        (torch.tensor(x), torch.tensor(w)))
+    for g, wnt in zip(got, want):
+        assert g.numpy().shape == tuple(wnt.shape)
+        assert relerr(g.numpy(), wnt.numpy()) <= 1e-5
+    v = rng.standard_normal(6).astype(np.float32)
+    h = J(nb.grad(lambda t: nb.reduce_sum(t * t * t)))(T(v)).numpy()
+    assert relerr(h, np.diag(6.0 * v.astype(np.float64))) <= F32_TOL
 
 
 # ---- scatter ----------------------------------------------------------------------------------------

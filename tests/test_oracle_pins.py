@@ -180,6 +180,43 @@ def test_conv2d_brute_force_and_torch():
         _close(g, t.grad.numpy(), 1e-9)
 
 
+def test_conv2d_transpose_brute_force_torch_and_adjoint():
+    x = RNG.standard_normal((2, 4, 3, 5))
+    w = RNG.standard_normal((3, 2, 4, 5))          # [R, S, Cout, Cin]
+    bias = RNG.standard_normal(4)
+    stride, pad = (2, 3), (1, 0, 2, 1)
+    out = O.conv2d_transpose(O.V(x), O.V(w), O.V(bias), stride=stride, padding=pad)
+    hf, wf = (4 - 1) * 2 + 3, (3 - 1) * 3 + 2
+    assert out.a.shape == (2, hf - 1, wf - 3, 4)
+    full = np.zeros((2, hf, wf, 4))
+    for n in range(2):
+        for i in range(4):
+            for j in range(3):
+                for r in range(3):
+                    for s in range(2):
+                        for co in range(4):
+                            for ci in range(5):
+                                full[n, i * 2 + r, j * 3 + s, co] += x[n, i, j, ci] * w[r, s, co, ci]
+    _close(out.a, full[:, 1:hf, 2:wf - 1, :] + bias)
+    # torch: weight [Cin, Cout, R, S]; no padding there, the crop is applied afterwards
+    vx, vw, vb = O.V(x), O.V(w), O.V(bias)
+    o2 = O.conv2d_transpose(vx, vw, vb, stride=stride, padding=pad)
+    c = RNG.standard_normal(o2.a.shape)
+    gs = O.grad_of(O.reduce_sum(o2 * c), [vx, vw, vb])
+    tx, tw, tb = _t(x), _t(w), _t(bias)
+    to = TF.conv_transpose2d(tx.permute(0, 3, 1, 2), tw.permute(3, 2, 0, 1), tb, stride=stride)
+    to = to.permute(0, 2, 3, 1)[:, 1:hf, 2:wf - 1, :]
+    _close(o2.a, to.detach().numpy(), 1e-12)
+    (to * torch.tensor(c)).sum().backward()
+    for g, t in zip(gs, (tx, tw, tb)):
+        _close(g, t.grad.numpy(), 1e-9)
+    # it is the adjoint of conv2d with the same filter read as HWIO: <convT(x), y> = <x, conv(y)>
+    y = RNG.standard_normal(o2.a.shape)
+    lhs = (O.conv2d_transpose(O.V(x), O.V(w), None, stride, pad).a * y).sum()
+    rhs = (x * O.conv2d(O.V(y), O.V(w), None, stride, pad).a).sum()
+    assert abs(lhs - rhs) <= 1e-10 * max(abs(lhs), 1.0)
+
+
 def test_max_pool_window_clipping_and_ties():
     x = RNG.standard_normal((2, 5, 5, 3))
     out = O.max_pool2d(O.V(x), (3, 3), (2, 2), (1, 1, 1, 1))
