@@ -22,8 +22,8 @@
 //     second MFMA is read from a transposed LDS tile with the same permutation: two
 //     8-byte reads at columns 16t + 4h and 16t + 8 + 4h.
 // LDS tiles:
-//   row-major  [64 rows][hd]      16-byte chunks XOR-swizzled by row % 8 (conflict-free
-//                                  16-byte fragment reads of 32 consecutive rows)
+//   row-major  [64 rows][hd]      16-byte chunks XOR-swizzled by the row so that the 16-byte
+//                                  fragment reads of 16 consecutive rows hit distinct banks
 //   transposed [hd rows][64 cols]  row pitch 68 elements: the 8-byte reads of 32
 //                                  consecutive rows fall on distinct banks per half
 #include "nbk_common.h"
@@ -76,6 +76,12 @@ struct AtRowTile {
   static constexpr int NCH = HD / 8;             // 16-byte chunks per row
   static constexpr int NREG = 64 * NCH / 256;    // passes (2 for hd 64, 4 for hd 128)
   at_u32x4 reg[NREG];
+  // Chunk swizzle of a row: the LDS has 64 banks, so one ds_read_b128 serves 16 lanes per
+  // cycle; the 16 rows they read must land on 16 distinct 16-byte slots of the 256-byte window.
+  static __device__ __forceinline__ int sw(int row) {
+    if constexpr (NCH == 8) return (row & 7) ^ ((row >> 3) & 1);  // 128-byte rows: two per window
+    else return row & 15;
+  }
   __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0) {
 #pragma unroll
     for (int s = 0; s < NREG; ++s) {
@@ -89,12 +95,12 @@ struct AtRowTile {
     for (int s = 0; s < NREG; ++s) {
       const int t = threadIdx.x + s * 256;
       const int row = t / NCH, c = t % NCH;
-      lds[row * NCH + (c ^ (row & 7))] = reg[s];
+      lds[row * NCH + (c ^ sw(row))] = reg[s];
     }
   }
   // fragment: 8 consecutive k (chunk) of `row`
   static __device__ __forceinline__ at_bf16x8 frag(const at_u32x4* lds, int row, int chunk) {
-    const at_u32x4 u = lds[row * NCH + (chunk ^ (row & 7))];
+    const at_u32x4 u = lds[row * NCH + (chunk ^ sw(row))];
     return __builtin_bit_cast(at_bf16x8, u);
   }
 };
