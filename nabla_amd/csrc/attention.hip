@@ -241,11 +241,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
       at_f32x16 st[2];
 #pragma unroll
       for (int kt2 = 0; kt2 < 2; ++kt2) {
+        // all fragments of the 32 keys are requested before the first MFMA waits for one
+        at_bf16x8 kfr[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) kfr[s] = RowT::frag(Ks, kt2 * 32 + li, 2 * s + h);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the scheduler from sinking each read to its MFMA
         at_f32x16 acc = (at_f32x16)(0.f);
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s)
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
-                                                        acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[s], qf[s], acc, 0, 0, 0);
         st[kt2] = acc;
       }
       float mx = at_neg_big();
@@ -432,11 +436,20 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const AttnArgs g) {
       constexpr bool MASK = decltype(masked)::value;
       at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Qs, qt2 * 32 + li, 2 * s + h), kf[s],
-                                                        s_acc, 0, 0, 0);
-        dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(DOs, qt2 * 32 + li, 2 * s + h), vf[s],
-                                                         dp_acc, 0, 0, 0);
+      for (int s = 0; s < KSTEPS; s += 4) {
+        // fragments of four k-steps are requested before the first MFMA waits for one
+        at_bf16x8 qfr[4], dfr[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          qfr[u] = RowT::frag(Qs, qt2 * 32 + li, 2 * (s + u) + h);
+          dfr[u] = RowT::frag(DOs, qt2 * 32 + li, 2 * (s + u) + h);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keeps the scheduler from sinking each read to its MFMA
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[u], kf[s + u], s_acc, 0, 0, 0);
+          dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dfr[u], vf[s + u], dp_acc, 0, 0, 0);
+        }
       }
       // rows of these tiles are queries: register r is query q0 + 32 qt2 + (r/4)*8 + 4h + r%4
       at_f32x16 p, ds;
@@ -565,12 +578,23 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_kernel(const AttnArgs g) {
     auto subtile = [&](auto masked, int kt2) {
       constexpr bool MASK = decltype(masked)::value;
       at_f32x16 s_acc = (at_f32x16)(0.f), dp_acc = (at_f32x16)(0.f);
+      constexpr int PF = HD == 128 ? 1 : 4;  // head size 128 has no registers to spare: read, then use
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Ks, kt2 * 32 + li, 2 * s + h), qf[s],
-                                                        s_acc, 0, 0, 0);
-        dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(RowT::frag(Vs, kt2 * 32 + li, 2 * s + h), dof[s],
-                                                         dp_acc, 0, 0, 0);
+      for (int s = 0; s < KSTEPS; s += PF) {
+        // fragments of PF k-steps are requested before the first MFMA waits for one
+        at_bf16x8 kfr[PF], vfr[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+          kfr[u] = RowT::frag(Ks, kt2 * 32 + li, 2 * (s + u) + h);
+          vfr[u] = RowT::frag(Vs, kt2 * 32 + li, 2 * (s + u) + h);
+        }
+        // keeps the scheduler from sinking each read to its MFMA
+        if constexpr (PF > 1) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+          s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u], qf[s + u], s_acc, 0, 0, 0);
+          dp_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[u], dof[s + u], dp_acc, 0, 0, 0);
+        }
       }
       at_f32x16 ds;
 #pragma unroll
