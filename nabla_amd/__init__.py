@@ -16,7 +16,7 @@ from .ops import (BinaryOperation, CreationOperation, Operation, ReduceOperation
                   UnaryOperation, call_custom_kernel)
 from .ops.reduction import reduce_max as max, reduce_min as min, reduce_sum as sum  # noqa: A001
 from .transforms import (CompilationStats, CompiledFunction, compile, grad, jacfwd, jacrev, jvp,
-                         value_and_grad, vjp)
+                         value_and_grad, vjp, vmap)
 from . import nn  # noqa: E402
 from . import testing  # noqa: E402
 from . import workloads  # noqa: E402

@@ -541,6 +541,22 @@ def test_jacobians_on_device_against_torch_cpu(hip, jac):
     assert relerr(h, np.diag(6.0 * v.astype(np.float64))) <= F32_TOL
 
 
+def test_vmap_per_example_gradients_on_device(hip):
+    """vmap(grad(loss)) over 16 examples of a small MLP loss on the device against the float64
+    closed form, and grad(sum(vmap(loss))) against the sum of the per-example gradients."""
+    rng = np.random.default_rng(49)
+    W, X = rng.standard_normal((24, 8)), rng.standard_normal((16, 24))
+    loss = lambda w, x: nb.reduce_sum(nb.tanh(x @ w) ** 2)
+    got = nb.vmap(nb.grad(loss), in_axes=(None, 0))(T(W.astype(np.float32)), T(X.astype(np.float32)))
+    th = np.tanh(X @ W)
+    want = np.einsum("bi,bj->bij", X, 2 * th * (1 - th ** 2))
+    assert got.numpy().shape == want.shape
+    assert relerr(got.numpy(), want) <= F32_TOL
+    total = nb.grad(lambda w: nb.reduce_sum(nb.vmap(loss, in_axes=(None, 0))(w, T(X.astype(np.float32)))))(
+        T(W.astype(np.float32)))
+    assert relerr(total.numpy(), want.sum(axis=0)) <= F32_TOL
+
+
 # ---- scatter ----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_scatter_on_device_is_exact_and_deterministic(hip, dtype):
