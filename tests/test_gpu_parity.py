@@ -557,6 +557,25 @@ def test_vmap_per_example_gradients_on_device(hip):
     assert relerr(total.numpy(), want.sum(axis=0)) <= F32_TOL
 
 
+def test_small_composite_ops_on_device(hip):
+    """trunc / floor / is_nan / is_inf / flip exactly and log1p to fp32 rounding on the device
+    (NaN and infinity must survive the kernels' compare instructions)."""
+    x = np.array([-2.5, -2.0, -0.3, -0.0, 0.0, 0.7, 1.0, 1.5, 1e6 + 0.5, np.nan, np.inf, -np.inf] * 50, np.float32)
+    fin = np.isfinite(x)
+    np.testing.assert_array_equal(nb.trunc(T(x)).numpy()[fin], np.trunc(x)[fin])
+    np.testing.assert_array_equal(nb.floor(T(x)).numpy()[fin], np.floor(x)[fin])
+    np.testing.assert_array_equal(nb.is_nan(T(x)).numpy(), np.isnan(x))
+    np.testing.assert_array_equal(nb.is_inf(T(x)).numpy(), np.isinf(x))
+    y = np.array([0.0, 1e-12, -1e-12, 3e-8, -3e-8, 1e-4, -1e-4, 0.5, -0.5, 3.0, 100.0, -0.999] * 40, np.float32)
+    got = nb.log1p(T(y)).numpy().astype(np.float64)
+    np.testing.assert_allclose(got, np.log1p(y.astype(np.float64)), rtol=1e-6, atol=0)
+    z = np.random.default_rng(5).standard_normal((7, 33, 5)).astype(np.float32)
+    for ax in (0, 1, 2):
+        np.testing.assert_array_equal(nb.flip(T(z), ax).numpy(), np.flip(z, ax))
+    parts = nb.chunk(T(z), 4, axis=1)
+    np.testing.assert_array_equal(parts[3].numpy(), z[:, 27:])
+
+
 # ---- scatter ----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_scatter_on_device_is_exact_and_deterministic(hip, dtype):
