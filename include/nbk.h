@@ -141,7 +141,8 @@ enum nbk_rp_op {
   NBK_OP_WHERE = 48,   /* dst <- a != 0 ? b : c                                */
   NBK_OP_FMA = 49,     /* dst <- a * b + c                                     */
   /* more unary ops (the block 16..31 is full) */
-  NBK_OP_DGELU = 50    /* derivative of the exact GELU: Phi(a) + a * phi(a)    */
+  NBK_OP_DGELU = 50,   /* derivative of the exact GELU: Phi(a) + a * phi(a)    */
+  NBK_OP_SIN = 51, NBK_OP_COS = 52 /* unary; the block 16..31 is full              */
 };
 
 enum nbk_red_kind { NBK_RED_SUM = 0, NBK_RED_MAX = 1, NBK_RED_MIN = 2 };

@@ -156,7 +156,7 @@ def input(shape, dtype: DType) -> Value:  # noqa: A001 - mirrors graph "input"
 
 
 # ---- elementwise ------------------------------------------------------------------
-UNARY_FNS = {"mov", "neg", "relu", "exp", "log", "sqrt", "rsqrt", "erf", "gelu", "dgelu", "tanh", "sigmoid",
+UNARY_FNS = {"mov", "neg", "relu", "exp", "log", "sqrt", "rsqrt", "erf", "gelu", "dgelu", "tanh", "sigmoid", "sin", "cos",
              "abs", "not", "trunc", "nez"}
 BINARY_FNS = {"add", "sub", "mul", "div", "max", "min", "gt", "ge", "eq", "ne", "lt", "le", "pow",
               "and", "or"}

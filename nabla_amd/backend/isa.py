@@ -10,7 +10,7 @@ UNARY = {
     "mov": 16, "neg": 17, "relu": 18, "exp": 19, "log": 20, "sqrt": 21, "rsqrt": 22, "erf": 23,
     "gelu": 24, "tanh": 25, "sigmoid": 26, "abs": 27, "rbf16": 28, "not": 29, "trunc": 30,
     "nez": 31,
-    "dgelu": 50,  # the block 16..31 is full
+    "dgelu": 50, "sin": 51, "cos": 52,  # the block 16..31 is full
 }
 BINARY = {
     "add": 32, "sub": 33, "mul": 34, "div": 35, "max": 36, "min": 37, "gt": 38, "ge": 39,

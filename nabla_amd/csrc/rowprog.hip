@@ -51,7 +51,8 @@ __device__ __forceinline__ uint64_t rp_sgpr64(uint2 v) {
 __device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, int n_lead);
 
 __host__ __device__ __forceinline__ bool rp_is_unary(int op) {
-  return (op >= NBK_OP_MOV && op < NBK_OP_ADD) || op == NBK_OP_DGELU;
+  return (op >= NBK_OP_MOV && op < NBK_OP_ADD) || op == NBK_OP_DGELU || op == NBK_OP_SIN ||
+         op == NBK_OP_COS;
 }
 
 // One body instruction on one chunk.

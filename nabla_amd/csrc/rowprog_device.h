@@ -131,6 +131,8 @@ __device__ __forceinline__ float rp_unary(int op, float a) {
       return 0.5f * (1.0f + erff(a * 0.70710678118654752440f)) +
              a * 0.39894228040143267794f * expf(-0.5f * a * a);
     case NBK_OP_TANH: return tanhf(a);
+    case NBK_OP_SIN: return sinf(a);
+    case NBK_OP_COS: return cosf(a);
     case NBK_OP_SIGMOID: return 1.0f / (1.0f + expf(-a));
     case NBK_OP_ABS: return fabsf(a);
     case NBK_OP_RBF16: return nbk_bf16_to_f32(nbk_f32_to_bf16(a));

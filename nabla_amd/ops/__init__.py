@@ -11,8 +11,8 @@ from .extra import (chunk, flip, floor, is_inf, is_nan, log1p, logical_xor, minm
                     trunc, unbind)
 from .pooling import avg_pool2d, max_pool2d
 from .reduction import (argmax, argmin, mean, reduce_max, reduce_min, reduce_sum)
-from .unary import (abs, cast, erf, exp, gelu, log, logsoftmax, neg, relu, rsqrt, sigmoid,
-                    silu, softmax, sqrt, tanh)
+from .unary import (abs, cast, cos, erf, exp, gelu, log, logsoftmax, neg, relu, rsqrt, sigmoid,
+                    silu, sin, softmax, sqrt, tanh)
 from .utils import call_custom_kernel
 from .view import (broadcast_to, concatenate, flatten, gather, moveaxis, pad, permute, reshape,
                    scatter, slice_tensor, slice_update, squeeze, stack, swap_axes, take, transpose,

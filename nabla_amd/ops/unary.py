@@ -143,6 +143,32 @@ class TanhOp(UnaryOperation):
         return sub(1.0, mul(output, output))
 
 
+class SinOp(UnaryOperation):
+    """unary.py (SinOp): derivative cos(x)."""
+
+    @property
+    def name(self) -> str:
+        return "sin"
+
+    kernel = _ew1("sin")
+
+    def _derivative(self, primal, output):
+        return cos(primal)
+
+
+class CosOp(UnaryOperation):
+    """unary.py (CosOp): derivative -sin(x)."""
+
+    @property
+    def name(self) -> str:
+        return "cos"
+
+    kernel = _ew1("cos")
+
+    def _derivative(self, primal, output):
+        return neg(sin(primal))
+
+
 class SigmoidOp(UnaryOperation):
     @property
     def name(self) -> str:
@@ -353,6 +379,18 @@ def rsqrt(x) -> Tensor:
 
 def erf(x) -> Tensor:
     return _erf_op([ensure_tensor(x)], {})[0]
+
+
+_sin_op = SinOp()
+_cos_op = CosOp()
+
+
+def sin(x) -> Tensor:
+    return _sin_op([ensure_tensor(x)], {})[0]
+
+
+def cos(x) -> Tensor:
+    return _cos_op([ensure_tensor(x)], {})[0]
 
 
 def tanh(x) -> Tensor:

@@ -39,6 +39,8 @@ _UNARY = {
     "dgelu": lambda a: (0.5 * (1.0 + _sp.erf(a.astype(np.float64) / np.sqrt(2.0))) +
                         a.astype(np.float64) * np.exp(-0.5 * a.astype(np.float64) ** 2) / np.sqrt(2.0 * np.pi)).astype(_F32),
     "tanh": lambda a: np.tanh(a),
+    "sin": lambda a: np.sin(a),
+    "cos": lambda a: np.cos(a),
     "sigmoid": lambda a: (_F32(1) / (_F32(1) + np.exp(-a))).astype(_F32),
     "abs": lambda a: np.abs(a),
     "rbf16": _round_bf16,

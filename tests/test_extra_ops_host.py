@@ -72,3 +72,19 @@ def test_split_chunk_unbind_minmax(emulator):
     g = nb.grad(lambda t: nb.reduce_sum(nb.chunk(t, 2, axis=1)[1] * 2.0) + nb.reduce_sum(nb.unbind(t, 0)[2]))(T(x))
     want = np.zeros_like(x); want[:, 3:] += 2.0; want[2] += 1.0
     np.testing.assert_array_equal(g.numpy(), want)
+
+
+def test_sin_cos_values_and_derivatives(emulator):
+    x = RNG.uniform(-8, 8, (4, 37)).astype(np.float32)
+    np.testing.assert_allclose(nb.sin(T(x)).numpy(), np.sin(x.astype(np.float64)), rtol=0, atol=2e-7)
+    np.testing.assert_allclose(nb.cos(T(x)).numpy(), np.cos(x.astype(np.float64)), rtol=0, atol=2e-7)
+    g = nb.grad(lambda t: nb.reduce_sum(nb.sin(t) * nb.cos(t)))(T(x))          # d/dx sin cos = cos 2x
+    np.testing.assert_allclose(g.numpy(), np.cos(2 * x.astype(np.float64)), rtol=0, atol=1e-6)
+    _, tan = nb.jvp(nb.cos, (T(x),), (T(np.ones_like(x)),))
+    np.testing.assert_allclose(tan.numpy(), -np.sin(x.astype(np.float64)), rtol=0, atol=2e-7)
+    # sinusoidal position table of the transformer examples: sin on even, cos on odd columns
+    pos, d = np.arange(16)[:, None], np.arange(8)[None, :]
+    ang = (pos / 10000 ** (2 * (d // 2) / 8)).astype(np.float32)
+    table = nb.where(T((d % 2 == 0) * np.ones_like(ang), bool), nb.sin(T(ang)), nb.cos(T(ang)))
+    want = np.where(d % 2 == 0, np.sin(ang.astype(np.float64)), np.cos(ang.astype(np.float64)))
+    np.testing.assert_allclose(table.numpy(), want, rtol=0, atol=2e-7)

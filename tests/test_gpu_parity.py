@@ -574,6 +574,12 @@ def test_small_composite_ops_on_device(hip):
         np.testing.assert_array_equal(nb.flip(T(z), ax).numpy(), np.flip(z, ax))
     parts = nb.chunk(T(z), 4, axis=1)
     np.testing.assert_array_equal(parts[3].numpy(), z[:, 27:])
+    # sin / cos: library routines in the row-program kernels, derivative through the trace
+    a = np.random.default_rng(6).uniform(-8, 8, (33, 257)).astype(np.float32)
+    np.testing.assert_allclose(nb.sin(T(a)).numpy(), np.sin(a.astype(np.float64)), rtol=0, atol=3e-7)
+    np.testing.assert_allclose(nb.cos(T(a)).numpy(), np.cos(a.astype(np.float64)), rtol=0, atol=3e-7)
+    g = nb.grad(lambda t: nb.reduce_sum(nb.sin(t) * nb.cos(t)))(T(a))
+    np.testing.assert_allclose(g.numpy(), np.cos(2 * a.astype(np.float64)), rtol=0, atol=2e-6)
 
 
 # ---- scatter ----------------------------------------------------------------------------------------
