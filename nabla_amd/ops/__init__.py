@@ -7,7 +7,7 @@ from .control_flow import where
 from .convolution import conv2d, conv2d_transpose
 from .creation import (arange, constant, full, full_like, ones, ones_like, tril, triu, zeros,
                        zeros_like)
-from .extra import (chunk, flip, floor, is_inf, is_nan, log1p, logical_xor, minmax, outer, split,
+from .extra import (atanh, chunk, flip, floor, is_inf, is_nan, log1p, logical_xor, minmax, outer, split,
                     trunc, unbind)
 from .pooling import avg_pool2d, max_pool2d
 from .reduction import (argmax, argmin, mean, reduce_max, reduce_min, reduce_sum)

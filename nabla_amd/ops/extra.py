@@ -1,6 +1,6 @@
 """Small ops next to the hot path, each built from primitives the kernels already have:
 ``trunc`` / ``floor`` (nabla/ops/unary.py:405-432, 540-566: zero derivative), ``is_nan`` /
-``is_inf`` (455-470), ``log1p`` (471-486), ``logical_xor`` (comparison.py:258-262), ``outer``
+``is_inf`` (455-470), ``log1p`` (471-486), ``atanh``, ``logical_xor`` (comparison.py:258-262), ``outer``
 (binary.py:575-600), ``flip`` (view/axes.py:844-854), ``split`` / ``chunk`` / ``unbind`` /
 ``minmax`` (multi_output.py:481-538).  They lower to the same row programs, views and index
 kernels as their parts, so they add no kernels."""
@@ -76,6 +76,15 @@ def log1p(x) -> Tensor:
     one = equal(d, 0.0)
     safe = where(one, add(mul(x, 0.0), 1.0), d)      # a divisor of 1 where u == 1
     return where(one, x, mul(log(u), div(x, safe)))
+
+
+def atanh(x) -> Tensor:
+    """Inverse hyperbolic tangent as (log1p(x) - log1p(-x)) / 2, which keeps small arguments exact;
+    the derivative of the parts is 1 / (1 - x^2), the reference's rule (unary.py, AtanhOp)."""
+    from .binary import mul, sub
+    from .unary import neg
+    x = ensure_tensor(x)
+    return mul(sub(log1p(x), log1p(neg(x))), 0.5)
 
 
 def logical_xor(x, y) -> Tensor:
@@ -165,5 +174,5 @@ def minmax(x) -> dict:
     return {"min": reduce_min(x, axis=axes), "max": reduce_max(x, axis=axes)}
 
 
-__all__ = ["trunc", "floor", "is_nan", "is_inf", "log1p", "logical_xor", "outer", "flip", "split",
+__all__ = ["atanh", "trunc", "floor", "is_nan", "is_inf", "log1p", "logical_xor", "outer", "flip", "split",
            "chunk", "unbind", "minmax"]

@@ -88,3 +88,11 @@ def test_sin_cos_values_and_derivatives(emulator):
     table = nb.where(T((d % 2 == 0) * np.ones_like(ang), bool), nb.sin(T(ang)), nb.cos(T(ang)))
     want = np.where(d % 2 == 0, np.sin(ang.astype(np.float64)), np.cos(ang.astype(np.float64)))
     np.testing.assert_allclose(table.numpy(), want, rtol=0, atol=2e-7)
+
+
+def test_atanh(emulator):
+    x = np.array([0.0, 1e-10, -1e-10, 1e-4, -0.3, 0.5, 0.9, -0.99, 0.999], np.float32)
+    got = nb.atanh(T(x)).numpy().astype(np.float64)
+    np.testing.assert_allclose(got, np.arctanh(x.astype(np.float64)), rtol=1e-6, atol=0)
+    g = nb.grad(lambda t: nb.reduce_sum(nb.atanh(t)))(T(x[3:])).numpy()
+    np.testing.assert_allclose(g, 1.0 / (1.0 - x[3:].astype(np.float64) ** 2), rtol=3e-4)
