@@ -95,9 +95,12 @@ def run_package(tol):
     t = {k[3:]: T(v) for k, v in z.items() if k.startswith("in_")}
     loss, grads = nb.workloads.c3_step(t, int(z["heads"]))
     assert abs(loss.item() - z["loss"]) < tol * abs(z["loss"])
-    scale = max(np.abs(z["g_" + k]).max() for k in oc.C3_PARAMS)
     for k in oc.C3_PARAMS:
-        assert rel(grads[k].numpy(), z["g_" + k], floor=1e-3 * scale) < 3 * tol, k
+        # the key bias has no gradient (softmax ignores a shift of all its scores: the true value
+        # is zero and what comes back is the rounding of sums that cancel), so it is measured on
+        # the scale of the query bias's gradient, which is the same sum without the cancellation
+        floor = np.abs(z["g_bq"]).max() if k == "bk" else 0.0
+        assert rel(grads[k].numpy(), z["g_" + k], floor=floor) < tol, k
     z = load("c4_cnn")
     t = {k[3:]: T(v) for k, v in z.items() if k.startswith("in_")}
     loss, grads = nb.workloads.c4_step(t)
@@ -106,21 +109,21 @@ def run_package(tol):
     assert rel(logits.numpy(), z["logits"]) < tol
     np.testing.assert_array_equal(nb.argmax(logits, axis=-1).numpy(), z["argmax"])
     for k in oc.C4_PARAMS:
-        assert rel(grads[k].numpy(), z["g_" + k]) < 3 * tol, k
+        assert rel(grads[k].numpy(), z["g_" + k]) < tol, k
     z = load("c5_lora")
     tree, want = c5_tree(z)
     loss, grads = nb.workloads.c5_step(oc.upload(nb, tree), int(z["heads"]), float(z["alpha"]))
     flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
     assert abs(loss.item() - z["loss"]) < tol * abs(z["loss"])
     for g, w in zip(flat, want):
-        assert rel(g.numpy(), w) < 3 * tol
+        assert rel(g.numpy(), w) < tol
     z = load("kernels")
     x, w = T(z["conv_x"]), T(z["conv_w"])
     kw = dict(stride=(2, 1), padding=(1, 0, 2, 1))
     y = nb.conv2d(x, w, **kw)
     gx, gw = nb.grad(lambda a, b: nb.reduce_sum(nb.conv2d(a, b, **kw) ** 2), argnums=(0, 1))(x, w)
-    assert rel(y.numpy(), z["conv_y"]) < tol and rel(gx.numpy(), z["conv_gx"]) < 3 * tol
-    assert rel(gw.numpy(), z["conv_gw"]) < 3 * tol
+    assert rel(y.numpy(), z["conv_y"]) < tol and rel(gx.numpy(), z["conv_gx"]) < tol
+    assert rel(gw.numpy(), z["conv_gw"]) < tol
     p = T(z["pool_x"])
     py = nb.max_pool2d(p, kernel_size=(2, 2))
     gp = nb.grad(lambda a: nb.reduce_sum(nb.max_pool2d(a, kernel_size=(2, 2)) ** 2))(p)
@@ -137,22 +140,22 @@ def run_package(tol):
     assert rel(nb.logsoftmax(s, axis=-1).numpy(), z["lsm_y"]) < tol
     ramp = T(np.arange(10, dtype=np.float32))
     gs = nb.grad(lambda a: nb.reduce_sum(nb.softmax(a, axis=-1) * ramp))(s)
-    assert rel(gs.numpy(), z["sm_gx"]) < 3 * tol
+    assert rel(gs.numpy(), z["sm_gx"]) < tol
     lw, lb, r10 = T(z["ln_w"]), T(z["ln_b"]), T((np.arange(10) / 10.0).astype(np.float32))
     F = nb.nn.functional
     assert rel(F.layer_norm(s, lw, lb).numpy(), z["ln_y"]) < tol
     g3 = nb.grad(lambda a, b, c: nb.reduce_sum(F.layer_norm(a, b, c) ** 2 * r10), argnums=(0, 1, 2))(s, lw, lb)
     for g, k in zip(g3, ("ln_gx", "ln_gw", "ln_gb")):
-        assert rel(g.numpy(), z[k]) < 3 * tol, k
+        assert rel(g.numpy(), z[k]) < tol, k
 
 
 def test_frontend_on_emulator_matches_golden(emulator):
-    run_package(2e-5)
+    run_package(1e-5)
 
 
 @pytest.mark.gpu
 def test_hip_matches_golden(hip):
-    run_package(2e-5)
+    run_package(1e-5)
 
 
 # ---- bf16 causal attention (the fused kernels' shape class) -------------------------------------------

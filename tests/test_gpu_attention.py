@@ -121,10 +121,11 @@ def test_attention_inside_the_transformer_block(hip):
     st = list(_PLAN_CACHE.values())[-1].plan.stats
     assert st.get("attention") == 1 and st.get("attention_bwd") == 1 and st.get("copy", 0) == 0
     assert abs(loss.item() - wl) < 2e-2 * abs(wl)
-    scale = max(np.abs(g).max() for g in wg.values())
     for k in oc.C3_PARAMS:
         got = grads[k].numpy().astype(np.float64)
-        assert np.abs(got - wg[k]).max() <= 3e-2 * max(np.abs(wg[k]).max(), 1e-2 * scale), k
+        # (the key bias has a zero true gradient: measured on the scale of the query bias's)
+        floor = np.abs(wg["bq"]).max() if k == "bk" else 0.0
+        assert np.abs(got - wg[k]).max() <= 2e-2 * max(np.abs(wg[k]).max(), floor), k
 
 
 def _run_fwd(lib, L, st, q, k, v, causal):

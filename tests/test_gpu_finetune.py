@@ -44,7 +44,7 @@ def test_qlora_linear_and_training(hip, low_rank):
         A, B = adapter["A"].to_numpy().astype(np.float64), adapter["B"].to_numpy().astype(np.float64)
         want = x @ wd + x @ ((A @ B) * (8.0 / 3))
         got = ft.qlora_linear(T(x), qw, adapter, alpha=8.0)
-        np.testing.assert_allclose(got.to_numpy(), want, rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(got.to_numpy(), want, rtol=1e-5, atol=1e-5)
         opt = nb.nn.optim.adamw_init(adapter)
 
         def loss_fn(p):

@@ -43,8 +43,8 @@ def test_row_reduce_and_grad(hip):
         pt = xt * yt
         ot = (torch.exp(pt - pt.max(1, keepdim=True).values) * torch.relu(xt)).sum(1)
         ot.sum().backward()
-        np.testing.assert_allclose(out.numpy(), ot.detach().numpy(), rtol=2e-5, atol=1e-6)
-        np.testing.assert_allclose(g.numpy(), xt.grad.numpy(), rtol=2e-5, atol=2e-6)
+        np.testing.assert_allclose(out.numpy(), ot.detach().numpy(), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(g.numpy(), xt.grad.numpy(), rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
@@ -153,7 +153,7 @@ def test_gemm_epilogue(hip, dtype, act, shape, res_op):
     lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     torch.cuda.synchronize()
     got = c_dev.double().cpu().numpy()
-    rtol, atol = (1e-5, 2e-5) if dtype == "f32" else (2.0 ** -8, 2e-2)
+    rtol, atol = (1e-5, 1e-5) if dtype == "f32" else (2.0 ** -8, 2e-2)
     err = np.abs(got - ref) - rtol * np.abs(ref)
     assert err.max() <= atol, err.max()
 
@@ -277,7 +277,7 @@ def test_layernorm_softmax_grads(hip):
     assert abs(l.item() - tl.item()) < 1e-5
     for g, t in zip(gs, (tx, tw, tb)):
         ref = t.grad.numpy()
-        assert np.abs(g.numpy() - ref).max() <= 2e-5 * np.abs(ref).max() + 1e-8
+        assert np.abs(g.numpy() - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-8
 
 
 def test_conv_pool_grads(hip):
@@ -306,7 +306,7 @@ def test_conv_pool_grads(hip):
     assert abs(l.item() - tl.item()) <= 1e-5 * abs(tl.item())
     for g, t in zip(gs, (tw1, tb1, tw2, tx)):
         ref = t.grad.numpy()
-        assert np.abs(g.numpy() - ref).max() <= 2e-5 * np.abs(ref).max() + 1e-8
+        assert np.abs(g.numpy() - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-8
 
 
 def test_gather_argmax_views(hip):

@@ -3,8 +3,8 @@ configurations (reduced sizes), full-size spot checks, the specialised row
 kernels against the interpreter, data-movement / index kernels on awkward
 shapes, user kernels, and ``compile`` on the device.
 
-Tolerances: 1e-5 relative for fp32 work (2e-5 where a long fp32 accumulation
-sits between input and output), 2e-2 for bf16, exact for integer results.
+Tolerances: 1e-5 relative for fp32 work, 2e-2 for bf16, exact for integer results.  The
+error of a tensor is max |got - want| over max |want| (one scale per tensor).
 """
 import ctypes as C
 from pathlib import Path
@@ -18,7 +18,7 @@ from oracle import configs as oc
 
 pytestmark = pytest.mark.gpu
 
-F32_TOL = 2e-5
+F32_TOL = 1e-5
 BF16_TOL = 2e-2
 
 
@@ -115,10 +115,11 @@ def test_c3_block_fp32(hip, shape, heads):
     loss, grads = oc.c3_program(nb, oc.upload(nb, t), num_heads=heads)
     nb.realize_all(loss, *grads.values())
     assert abs(loss.item() - wl) < F32_TOL * abs(wl)
-    scale = max(np.abs(g).max() for g in wg.values())
     for k in oc.C3_PARAMS:
-        # bk's true gradient is zero (softmax is shift invariant): compare on the common scale
-        assert relerr(grads[k].numpy(), wg[k], floor=1e-3 * scale) < 5e-5, k
+        # bk's true gradient is zero (softmax is shift invariant): what comes back is the rounding
+        # of sums that cancel, measured on the scale of bq's gradient (the same sums, uncancelled)
+        floor = np.abs(wg["bq"]).max() if k == "bk" else 0.0
+        assert relerr(grads[k].numpy(), wg[k], floor=floor) < F32_TOL, k
 
 
 def test_c3_block_bf16(hip):
@@ -128,10 +129,10 @@ def test_c3_block_bf16(hip):
     nb.realize_all(loss, *grads.values())
     assert loss.dtype == nb.DType.bfloat16
     assert abs(loss.item() - wl) < BF16_TOL * abs(wl)
-    scale = max(np.abs(g).max() for g in wg.values())
     for k in oc.C3_PARAMS:
         assert grads[k].dtype == nb.DType.bfloat16
-        assert relerr(grads[k].numpy(), wg[k], floor=0.05 * scale) < BF16_TOL, k
+        floor = np.abs(wg["bq"]).max() if k == "bk" else 0.0  # (zero true gradient, see above)
+        assert relerr(grads[k].numpy(), wg[k], floor=floor) < BF16_TOL, k
 
 
 # ---- C4 ------------------------------------------------------------------------------------------
@@ -146,12 +147,14 @@ def test_c4_cnn_step(hip, batch, hw, c):
     nb.realize_all(loss, am, logits, *grads.values())
     assert abs(loss.item() - wl) < F32_TOL * abs(wl)
     assert relerr(logits.numpy(), wlogits) < F32_TOL
-    # the arg-max is an index: exact unless the top two logits tie within fp32 noise
+    # the arg-max is an index and must be exact; the seeded inputs leave no two top logits
+    # within fp32 noise of each other, so the oracle's index is the only right answer
     top2 = np.sort(wlogits, axis=-1)[:, -2:]
-    clear = (top2[:, 1] - top2[:, 0]) > 1e-4 * np.abs(top2[:, 1])
-    np.testing.assert_array_equal(am.numpy()[clear], wam[clear])
+    assert ((top2[:, 1] - top2[:, 0]) > 1e-4 * np.abs(top2[:, 1])).all()
+    np.testing.assert_array_equal(am.numpy(), wam)
+    np.testing.assert_array_equal(am.numpy(), np.argmax(logits.numpy(), axis=-1))
     for k in oc.C4_PARAMS:
-        assert relerr(grads[k].numpy(), wg[k]) < 5e-5, k
+        assert relerr(grads[k].numpy(), wg[k]) < F32_TOL, k
 
 
 # ---- C5 ------------------------------------------------------------------------------------------
@@ -164,20 +167,21 @@ def test_c5_lora_fp32(hip):
     nb.realize_all(loss, *flat)
     assert abs(loss.item() - wl) < F32_TOL * abs(wl)
     for g, w in zip(flat, wg):
-        assert relerr(g.numpy(), w) < 5e-5
+        assert relerr(g.numpy(), w) < F32_TOL
 
 
-def test_c5_lora_bf16(hip):
-    t = oc.c5_inputs(layers=2, batch=2, seq=64, d_model=128, d_ff=256, vocab=300, rank=8, seed=3,
+@pytest.mark.parametrize("seq,d_model,heads", [(64, 128, 4), (128, 256, 2), (256, 128, 2)])
+def test_c5_lora_bf16(hip, seq, d_model, heads):
+    """Head sizes 32 (attention as GEMM + softmax + GEMM), 128 and 64 (the fused kernels)."""
+    t = oc.c5_inputs(layers=2, batch=2, seq=seq, d_model=d_model, d_ff=256, vocab=300, rank=8, seed=3,
                      b_zero=False, bf16=True)
-    wl, wg = oc.c5_reference(t, num_heads=4)
-    loss, grads = oc.c5_program(nb, oc.upload(nb, t, dtype=nb.DType.bfloat16), num_heads=4)
+    wl, wg = oc.c5_reference(t, num_heads=heads)
+    loss, grads = oc.c5_program(nb, oc.upload(nb, t, dtype=nb.DType.bfloat16), num_heads=heads)
     flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
     nb.realize_all(loss, *flat)
     assert abs(loss.item() - wl) < BF16_TOL * abs(wl)
-    scale = max(np.abs(w).max() for w in wg)
     for g, w in zip(flat, wg):
-        assert relerr(g.numpy(), w, floor=0.05 * scale) < 2 * BF16_TOL
+        assert relerr(g.numpy(), w) < BF16_TOL
 
 
 # ---- movement, reductions and index kernels on awkward shapes ------------------------------------
@@ -293,8 +297,8 @@ def test_conv2d_forward_and_grads(hip, cfg):
     got = nb.conv2d(T(x), T(w), **kw)
     gx, gw = nb.grad(f, argnums=(0, 1))(T(x), T(w))
     assert relerr(got.numpy(), out.a) < F32_TOL
-    assert relerr(gx.numpy(), wgx) < 5e-5
-    assert relerr(gw.numpy(), wgw) < 5e-5
+    assert relerr(gx.numpy(), wgx) < F32_TOL
+    assert relerr(gw.numpy(), wgw) < F32_TOL
 
 
 @pytest.mark.parametrize("cfg", [
@@ -319,7 +323,7 @@ def test_conv2d_transpose_forward_and_grads(hip, cfg):
     assert tuple(got.shape) == out.a.shape
     assert relerr(got.numpy(), out.a) < F32_TOL
     for g, wg in zip(nb.grad(f, argnums=(0, 1, 2))(T(x), T(w), T(b)), want):
-        assert relerr(g.numpy(), wg) < 5e-5
+        assert relerr(g.numpy(), wg) < F32_TOL
 
 
 # ---- user kernels ---------------------------------------------------------------------------------
@@ -372,12 +376,12 @@ def test_compiled_train_step_on_device(hip):
     for _ in range(3):
         loss, p = cstep(p, x)
         wl, wg = oc.c1_reference(t["x"], *[ref[k].astype(np.float32) for k in ("W1", "b1", "W2", "b2")])
-        assert abs(loss.item() - wl) <= 5e-5 * abs(wl) + 1e-8
+        assert abs(loss.item() - wl) <= F32_TOL * abs(wl) + 1e-8
         for k, g in zip(("W1", "b1", "W2", "b2"), wg):
             ref[k] = ref[k] - 0.1 * g
     assert cstep.stats.misses == 1 and cstep.stats.hits == 2
     for k in params:
-        assert relerr(p[k].numpy(), ref[k]) < 5e-5
+        assert relerr(p[k].numpy(), ref[k]) < F32_TOL
 
 
 # ---- optimizer step (next row after the hot path: nn/optim) ---------------------------------------

@@ -462,3 +462,141 @@ def test_scatter_and_gather_gradient_pins():
     vt = O.V(x)
     (gt,) = O.grad_of(O.reduce_sum(O.gather(vt, idx) * O.V(gg)), [vt])
     np.testing.assert_array_equal(gt, tt.grad.numpy())
+
+
+# ---- casts, comparisons and the remaining view helpers ---------------------------------
+def test_cast_values_truncation_and_vjp():
+    """cast: float -> int truncates toward zero (numpy and torch agree), float -> narrower float
+    rounds to nearest even, the VJP casts the cotangent back to the input type and an integer
+    input receives no gradient."""
+    x = np.array([-2.7, -0.5, 0.49, 1.5, 2.5, 1e6 + 0.75])
+    got = O.cast(O.V(x), np.int64).a
+    assert got.dtype == np.int64
+    assert got.tolist() == [-2, 0, 0, 1, 2, 1000000]
+    assert got.tolist() == torch.tensor(x).to(torch.int64).tolist()
+    assert O.cast(O.V(x), np.int32).a.tolist() == torch.tensor(x).to(torch.int32).tolist()
+    # fp64 -> fp32: nearest even; 1 + 2^-24 is a tie and goes to 1.0, 1 + 3 * 2^-24 to 1 + 2^-22
+    ties = np.array([1.0 + 2.0 ** -24, 1.0 + 3.0 * 2.0 ** -24])
+    assert O.cast(O.V(ties), np.float32).a.tolist() == [1.0, 1.0 + 2.0 ** -22]
+    # bool -> float gives exact 0 / 1
+    assert O.cast(O.V(np.array([True, False])), np.float64).a.tolist() == [1.0, 0.0]
+    # gradient: a cast in the middle of a chain is the identity to the cotangent
+    a = RNG.standard_normal((3, 4))
+    v = O.V(a)
+    w = RNG.standard_normal((3, 4))
+    (g,) = O.grad_of(O.reduce_sum(O.cast(v * 3.0, np.float32) * w), [v])
+    assert g.dtype == np.float64
+    t = _t(a)
+    ((t * 3.0).to(torch.float32) * torch.tensor(w, dtype=torch.float32)).sum().backward()
+    _close(g, t.grad.numpy(), 1e-6)
+    vi = O.V(np.arange(4))
+    assert O.backward(O.reduce_sum(O.cast(vi, np.float64) * 2.0)).get(id(vi)) is None
+
+
+def test_equal_is_exact_and_broadcasts():
+    """equal: elementwise ==, bool result, numpy broadcasting, no gradient; the one-hot it
+    builds in cross_entropy (labels against an iota) is the identity matrix's rows."""
+    a = np.array([[0.0, -0.0, 1.0, np.nan]])
+    b = np.array([[0.0], [1.0], [np.nan]])
+    got = O.equal(O.V(a), O.V(b))
+    assert got.a.dtype == np.bool_ and got.a.shape == (3, 4)
+    assert got.a.tolist() == [[True, True, False, False], [False, False, True, False],
+                              [False, False, False, False]]  # -0 == 0, NaN != NaN
+    assert got.a.tolist() == torch.eq(torch.tensor(a), torch.tensor(b)).tolist()
+    assert got.vjp is None and got.parents == ()
+    labels = np.array([2, 0, 3, 3])
+    onehot = O.equal(O.unsqueeze(O.V(labels), -1), O.V(np.arange(4))).a
+    assert (onehot == np.eye(4, dtype=bool)[labels]).all()
+
+
+def test_permute_against_element_loops_and_torch():
+    """permute: out[i0, i1, i2] = x[...] with axis k of the result being axis order[k] of the
+    input (an index loop on a tiny tensor), and the VJP is the inverse permutation -- a
+    non-involutive order, so that using `order` where its inverse belongs fails."""
+    x = RNG.standard_normal((2, 3, 4))
+    order = (2, 0, 1)  # inverse is (1, 2, 0): not the same permutation
+    v = O.V(x)
+    out = O.permute(v, order)
+    assert out.a.shape == (4, 2, 3)
+    for i in range(4):
+        for j in range(2):
+            for k in range(3):
+                assert out.a[i, j, k] == x[j, k, i]
+    w = RNG.standard_normal(out.a.shape)
+    (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+    t = _t(x)
+    (t.permute(*order) * torch.tensor(w)).sum().backward()
+    _close(g, t.grad.numpy())
+    assert np.array_equal(g, np.transpose(w, (1, 2, 0)))
+    # swap_axes is the two-axis case of the same thing
+    _close(O.swap_axes(v, 0, 2).a, np.transpose(x, (2, 1, 0)))
+
+
+def test_unsqueeze_shapes_and_vjp():
+    x = RNG.standard_normal((3, 4))
+    v = O.V(x)
+    for axis, shape in ((0, (1, 3, 4)), (1, (3, 1, 4)), (-1, (3, 4, 1)), (2, (3, 4, 1))):
+        out = O.unsqueeze(v, axis)
+        assert out.a.shape == shape == tuple(torch.tensor(x).unsqueeze(axis).shape)
+        assert np.array_equal(out.a.reshape(3, 4), x)
+        w = RNG.standard_normal(shape)
+        (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+        assert np.array_equal(g, w.reshape(3, 4))
+    # a broadcast along the inserted axis sums back over it
+    out = O.mul(O.unsqueeze(v, 1), O.V(np.ones((3, 5, 4))))
+    (g,) = O.grad_of(O.reduce_sum(out), [v])
+    _close(g, np.full((3, 4), 5.0))
+
+
+def test_slice_tensor_window_and_zero_padded_vjp():
+    """slice_tensor(x, start, size) is x[start : start + size] per axis (size, not stop), and
+    its VJP puts the cotangent back into a zero tensor of the input's shape."""
+    x = RNG.standard_normal((5, 6, 3))
+    start, size = (1, 2, 0), (3, 2, 3)
+    v = O.V(x)
+    out = O.slice_tensor(v, start, size)
+    assert out.a.shape == size
+    for i in range(3):
+        for j in range(2):
+            for k in range(3):
+                assert out.a[i, j, k] == x[1 + i, 2 + j, k]
+    w = RNG.standard_normal(size)
+    (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+    t = _t(x)
+    (t[1:4, 2:4, :] * torch.tensor(w)).sum().backward()
+    _close(g, t.grad.numpy())
+    assert g[0].max() == 0.0 and g[4].min() == 0.0 and np.count_nonzero(g) == w.size
+    # two overlapping windows of one tensor accumulate
+    o2 = O.reduce_sum(O.slice_tensor(v, (0, 0, 0), (2, 6, 3))) + O.reduce_sum(O.slice_tensor(v, (1, 0, 0), (2, 6, 3)))
+    (g2,) = O.grad_of(o2, [v])
+    assert g2[0, 0, 0] == 1.0 and g2[1, 0, 0] == 2.0 and g2[2, 0, 0] == 1.0 and g2[3, 0, 0] == 0.0
+
+
+def test_torch_steps_agree_with_the_numpy_oracle():
+    """oracle/torch_steps.py (the full-size checker of the transformer and decoder steps) against
+    oracle/configs.py in float64: loss and every gradient, non-trivial biases, norm weights and
+    LoRA B factors so that no term is multiplied by zero or one."""
+    from oracle import torch_steps as ts
+    rng = np.random.default_rng(11)
+    t = oc.c3_inputs(2, 12, 16, 40, seed=5, bf16=False)
+    for k in oc.C3_PARAMS:
+        if k[0] == "b" or k.startswith("ln"):
+            t[k] = (t[k] + 0.3 * rng.standard_normal(t[k].shape)).astype(np.float32)
+    wl, wg = oc.c3_reference(t, num_heads=4)
+    gl, gg = ts.c3_step(t, num_heads=4)
+    assert abs(gl - wl) <= 1e-12 * abs(wl)
+    for k in oc.C3_PARAMS:
+        _close(gg[k], wg[k], 1e-9)
+    t5 = oc.c5_inputs(layers=2, batch=3, seq=10, d_model=24, d_ff=32, vocab=53, rank=4, seed=6,
+                      b_zero=False, bf16=False)
+    for L in t5["layers"]:
+        for k in L:
+            if k[0] == "b" or k.startswith("ln"):
+                L[k] = (L[k] + 0.3 * rng.standard_normal(L[k].shape)).astype(np.float32)
+    wl, wg = oc.c5_reference(t5, num_heads=4, alpha=8.0)
+    gl, gg = ts.c5_step(t5, num_heads=4, alpha=8.0)
+    assert abs(gl - wl) <= 1e-12 * abs(wl)
+    assert len(gg) == len(wg) == 8
+    for a, b in zip(gg, wg):
+        assert np.abs(b).max() > 0
+        _close(a, b, 1e-9)
