@@ -1,16 +1,29 @@
 """Benchmark of the hot path on one MI355X.
 
-Default workload: the elementwise + reduction stress configuration
-(x, y [8192, 8192] fp32; out = sum(exp(x*y - max(x*y)) * relu(x), axis=1) and
-the gradient of sum(out) w.r.t. x), one compiled step per iteration with the
-inputs already resident in HBM.  Prints ONE JSON line.
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5]
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5]
+Prints ONE JSON line.  With the default ``--workload all`` the line's headline (``value``,
+``ms_per_step``, ``roofline``, ``cpu_baseline``) is the largest configuration, the 12-layer LoRA
+fine-tuning step (c5: bf16, D2048, S2048, B4, V32000), and ``configs`` carries the same figures
+for each of the five configurations, so that one line holds every clause of the metric: steps/s
+per configuration, the MFMA fraction of the GEMM + attention kernels (c3, c5; convolutions for
+c4) and the HBM fraction of the fused elementwise + reduction kernel (c2).
+
+A step is one call of the public compiled function (``nb.compile(step)(*args)``: signature
+hashing, pytree flattening, plan replay, result wrapping) with its inputs resident in HBM; K
+calls are timed between device synchronisations after W warm-up calls.  The same plan called
+one layer lower (``BoundPlan.run`` on prepared buffers) is timed beside it
+(``plan_ms_per_step``).  Kernel durations for ``roofline`` come from HIP events recorded on the
+launch stream around every launch of the dominant kind: inside the timed region when a step is
+a single launch (c2), else from a second pass of plain launches, because the timed region
+replays the step as one HIP graph, inside which events cannot be recorded (``kernel_timing``
+says which).
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
+import gc
 import json
 import os
 import sys
@@ -21,8 +34,10 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+METRIC = "train steps/sec fwd+bwd at 1 MI355X; GEMM % MFMA peak; fused-op % HBM BW"
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+MFMA_KINDS = ("gemm", "attention", "attention_bwd", "conv2d", "conv2d_dgrad", "conv2d_wgrad")
 
 
 class KernelTimer:
@@ -44,15 +59,16 @@ class KernelTimer:
         return lambda: self.lib.nbk_event_record(b, stream)
 
     def durations_ms(self):
-        out = {}
+        """{(step index, kind): mean duration in ms}"""
+        acc = {}
         ms = C.c_float()
         for si, kind, a, b in self.pairs:
             self.lib.nbk_event_elapsed_ms(a, b, C.byref(ms))
-            out.setdefault((si, kind), []).append(ms.value)
+            acc.setdefault((si, kind), []).append(ms.value)
             self.lib.nbk_event_destroy(a)
             self.lib.nbk_event_destroy(b)
         self.pairs = []
-        return out
+        return {k: sum(v) / len(v) for k, v in acc.items()}
 
 
 def sync():
@@ -60,62 +76,130 @@ def sync():
     torch.cuda.synchronize()
 
 
-def compiled_plan(nb, fn, args):
-    """Trace + lower ``fn`` once; returns (bound plan, input buffers, call that
-    replays it).  The replay is what a cached ``@compile`` call executes."""
-    cf = nb.compile(fn)
-    out = cf(*args)
-    spec = next(iter(next(iter(cf._cache.values())).specializations.values()))
-    flat, _ = nb.tree_flatten((args, {}))
+# ------------------------------------------------------------------ host description
+def host_info() -> dict:
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    blas = None
+    try:
+        from threadpoolctl import threadpool_info
+        blas = max((p.get("num_threads", 1) for p in threadpool_info()
+                    if p.get("user_api") == "blas"), default=None)
+    except Exception:
+        pass
+    import torch
+    return {"cpu_model": model, "os_cpu_count": os.cpu_count(), "numpy_blas_threads": blas,
+            "torch_threads": torch.get_num_threads()}
 
-    def bufs():
-        return [flat[v]._impl._buffer if kind == "arg" else v for kind, v in spec.input_plan]
 
-    return cf, spec, bufs, out
+def _cpu_entry(value, cores, sample, host):
+    return dict(value=round(value, 5), unit="steps/s", cores=cores, kind="port", sample=sample,
+                cpu_model=host["cpu_model"], blas_threads=host["numpy_blas_threads"],
+                torch_threads=host["torch_threads"])
 
 
 # ------------------------------------------------------------------ workloads
 # The timed path uses the product only (nabla_amd.workloads: step programs and synthetic
-# inputs).  The CPU oracle is imported inside the cpu_baseline closures and nowhere else.
+# inputs).  The CPU oracle is imported inside the cpu_* functions and nowhere else.
+def cpu_c1(host):
+    from oracle import configs as oc
+    inp = oc.c1_inputs()
+    oc.c1_reference(**inp, dtype=np.float32)
+    n, t0 = 0, time.perf_counter()
+    while n < 20 or time.perf_counter() - t0 < 2.0:
+        oc.c1_reference(**inp, dtype=np.float32)
+        n += 1
+    return _cpu_entry(n / (time.perf_counter() - t0), host["numpy_blas_threads"] or 1,
+                      f"{n} full steps, numpy fp32 oracle (BLAS products, one core for the rest)", host)
+
+
+def cpu_c2(host, rows=8192, cols=8192):
+    # rows are independent, so a slice of them times like the whole step
+    from oracle import configs as oc
+    sample_rows = max(64, rows // 8)
+    inp = oc.c2_inputs(sample_rows, cols, seed=0)
+    oc.c2_reference(inp["x"][:64], inp["y"][:64], dtype=np.float32)
+    reps, t0 = 0, time.perf_counter()
+    while reps < 2 or (time.perf_counter() - t0 < 5.0 and reps < 40):
+        oc.c2_reference(inp["x"], inp["y"], dtype=np.float32)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return _cpu_entry(1.0 / (dt * rows / sample_rows), 1,
+                      f"{sample_rows} of {rows} rows x {reps} passes, numpy fp32 oracle "
+                      "(elementwise numpy: one core), scaled by rows", host)
+
+
+def cpu_c3(host, batch=8):
+    # batch elements are independent but for the mean and the parameter-gradient sums
+    import torch
+    from oracle import configs as oc
+    from oracle import torch_steps as ts
+    sample = 2
+    t = oc.c3_inputs(sample, 1024, 1024, 4096, seed=0, bf16=True)
+    ts.c3_step(oc.c3_inputs(1, 128, 1024, 4096, seed=0), 16, dtype=torch.float32)
+    t0 = time.perf_counter()
+    ts.c3_step(t, 16, dtype=torch.float32)
+    dt = time.perf_counter() - t0
+    return _cpu_entry(1.0 / (dt * batch / sample), host["torch_threads"],
+                      f"{sample} of {batch} sequences, one full step, torch-CPU fp32 oracle "
+                      "(oracle/torch_steps.py), scaled by batch", host)
+
+
+def cpu_c4(host, batch=64):
+    from oracle import configs as oc
+    sample = 16
+    small = oc.c4_inputs(batch=sample)
+    oc.c4_reference(oc.c4_inputs(batch=1), dtype=np.float32)
+    t0 = time.perf_counter()
+    oc.c4_reference(small, dtype=np.float32)
+    dt = time.perf_counter() - t0
+    return _cpu_entry(1.0 / (dt * batch / sample), host["numpy_blas_threads"] or 1,
+                      f"{sample} of {batch} images, one full step, numpy fp32 oracle "
+                      "(BLAS products, one core for the rest), scaled by batch", host)
+
+
+def cpu_c5(host, layers=12, batch=4):
+    # one sequence (of four) through one and through two layers: the difference is a layer's
+    # cost, the remainder the embedding, the final norm, the 32000-column head and the loss
+    import torch
+    from oracle import configs as oc
+    from oracle import torch_steps as ts
+    t = oc.c5_inputs(layers=2, batch=1, b_zero=False)
+    one = dict(t, layers=t["layers"][:1], lora=t["lora"][:1])
+    t0 = time.perf_counter()
+    ts.c5_step(one, 16, dtype=torch.float32)
+    t1 = time.perf_counter()
+    ts.c5_step(t, 16, dtype=torch.float32)
+    t2 = time.perf_counter()
+    per_layer = max((t2 - t1) - (t1 - t0), 1e-9)
+    rest = max((t1 - t0) - per_layer, 0.0)
+    full = batch * (layers * per_layer + rest)
+    return _cpu_entry(1.0 / full, host["torch_threads"],
+                      f"1 of {batch} sequences through 1 and through 2 of {layers} layers, torch-CPU "
+                      f"fp32 oracle (oracle/torch_steps.py; frozen-weight gradients skipped): "
+                      f"{per_layer:.2f} s per layer, {rest:.2f} s embedding + head + loss, "
+                      f"extrapolated to {layers} layers x {batch} sequences", host)
+
+
+def workload_c1(nb):
+    t = nb.workloads.synthetic_inputs("c1")
+    return dict(name="c1 2-layer MLP fwd+grad fp32, x[128,784]", fn=nb.workloads.c1_step, args=(t,),
+                dtype="f32", bound="mfma", algo=104.7e6, kinds=("gemm",), cpu=cpu_c1)
+
+
 def workload_c2(nb, rows=8192, cols=8192):
     t = nb.workloads.synthetic_inputs("c2", rows=rows, cols=cols)
     algo_bytes = 3 * rows * cols * 4 + 2 * rows * 4
     return dict(name=f"c2 elementwise+reduction fwd+grad, x,y[{rows},{cols}] fp32",
                 fn=nb.workloads.c2_step, args=(t["x"], t["y"]), dtype="f32", bound="hbm",
-                algo=algo_bytes, dominant="rowprog", cpu=lambda: cpu_c2(rows, cols))
-
-
-def cpu_c2(rows, cols):
-    # rows are independent, so a slice of them times like the whole step; the slice is sized
-    # for a run of about ten seconds (one untimed pass first: page faults, numpy warm-up)
-    from oracle import configs as oc
-    sample_rows = max(64, rows // 4)
-    inp = oc.c2_inputs(sample_rows, cols, seed=0)
-    oc.c2_reference(inp["x"][:64], inp["y"][:64], dtype=np.float32)
-    reps, t0 = 0, time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t0 < 8.0 and reps < 40):
-        oc.c2_reference(inp["x"], inp["y"], dtype=np.float32)
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    return dict(value=round(1.0 / (dt * rows / sample_rows), 4), unit="steps/s", cores=1, kind="port",
-                sample=f"{sample_rows} of {rows} rows x {reps} passes, numpy fp32 oracle, scaled by rows")
-
-
-def workload_c1(nb):
-    t = nb.workloads.synthetic_inputs("c1")
-
-    def cpu():
-        from oracle import configs as oc
-        inp = oc.c1_inputs()
-        t0 = time.perf_counter()
-        n = 20
-        for _ in range(n):
-            oc.c1_reference(**inp, dtype=np.float32)
-        return dict(value=n / (time.perf_counter() - t0), unit="steps/s", cores=os.cpu_count(),
-                    kind="port", sample=f"{n} full steps, numpy fp32 oracle")
-
-    return dict(name="c1 2-layer MLP fwd+grad fp32, x[128,784]", fn=nb.workloads.c1_step, args=(t,),
-                dtype="f32", bound="mfma", algo=104.7e6, dominant="gemm", cpu=cpu)
+                algo=algo_bytes, kinds=("rowprog",), cpu=cpu_c2)
 
 
 def workload_c3(nb, batch=8, seq=1024, d=1024, ff=4096):
@@ -126,67 +210,183 @@ def workload_c3(nb, batch=8, seq=1024, d=1024, ff=4096):
     mlp = 2 * 2 * T * d * ff
     attn_causal = 2 * 2 * batch * 16 * seq * seq * hd / 2
     flops = 3 * (qkvo + mlp + attn_causal)
-
-    def cpu():
-        from oracle import configs as oc
-        small = oc.c3_inputs(1, 128, d, ff, seed=0, bf16=True)
-        t0 = time.perf_counter()
-        oc.c3_reference(small, num_heads=16, dtype=np.float32)
-        dt = time.perf_counter() - t0
-        scale = T / 128.0
-        return dict(value=1.0 / (dt * scale), unit="steps/s", cores=os.cpu_count(), kind="port",
-                    sample="1 x 128 tokens of 8 x 1024, numpy fp32 oracle, scaled by tokens "
-                           "(attention cost per token is under-counted)")
-
     return dict(name=f"c3 pre-LN transformer block fwd+bwd bf16, B{batch} S{seq} D{d} FF{ff}",
                 fn=lambda t: nb.workloads.c3_step(t, 16), args=(t,), dtype="bf16", bound="mfma",
-                algo=flops, dominant="gemm", cpu=cpu)
+                algo=flops, kinds=("gemm", "attention", "attention_bwd"), cpu=cpu_c3)
 
 
 def workload_c4(nb):
     t = nb.workloads.synthetic_inputs("c4")
-
-    def cpu():
-        from oracle import configs as oc
-        small = oc.c4_inputs(batch=4)
-        t0 = time.perf_counter()
-        oc.c4_reference(small, dtype=np.float32)
-        dt = time.perf_counter() - t0
-        return dict(value=1.0 / (dt * 16), unit="steps/s", cores=os.cpu_count(), kind="port",
-                    sample="4 of 64 images, numpy fp32 oracle, scaled by batch")
-
     return dict(name="c4 CNN step fp32, img[64,32,32,3]", fn=nb.workloads.c4_step, args=(t,),
-                dtype="f32", bound="mfma", algo=58.4e9, dominant="conv", cpu=cpu)
+                dtype="f32", bound="mfma", algo=58.4e9,
+                kinds=("conv2d", "conv2d_dgrad", "conv2d_wgrad"), cpu=cpu_c4)
 
 
 def workload_c5(nb, layers=12):
     t = nb.workloads.synthetic_inputs("c5", layers=layers)
-
-    def cpu():
-        return dict(value=None, unit="steps/s", cores=os.cpu_count(), kind="port",
-                    sample="not run: one step is ~27 TFLOP on the host")
-
-    return dict(name=f"c5 LoRA step bf16, {layers} layers D2048 S2048 B4 (lora_linear in low-rank order)",
+    return dict(name=f"c5 LoRA step bf16, {layers} layers D2048 S2048 B4 V32000 r16 "
+                     "(lora_linear in low-rank order)",
                 fn=lambda t: nb.workloads.c5_step(t, 16), args=(t,), dtype="bf16", bound="mfma",
-                algo=24.5e12 * layers / 12, dominant="gemm", cpu=cpu)
+                algo=24.5e12 * layers / 12, kinds=("gemm", "attention", "attention_bwd"), cpu=cpu_c5)
 
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4,
              "c5": workload_c5}
 
 
-def measured_traffic(workload: str):
+def committed_traffic(workload: str, kernel_hashes: set):
     """HBM bytes per launch of the dominant kernel as the hardware counters saw them
-    (FETCH_SIZE + WRITE_SIZE from two counter runs, scaled by the same counters' reading for
-    a plain copy of known size).  Counters cannot be read from inside this process; the
-    figure comes from the committed summary of those runs, None when there is none."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
-                        f"hbm_traffic_{workload}.json")
+    (FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs of this command, each scaled by the
+    same counter's reading for a plain copy of known size).  A process cannot read those
+    counters for itself, so the figure comes from the committed summary of those runs, and
+    only while the kernel timed here is still the kernel they profiled (its program hash is
+    part of its name)."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}.json")
     try:
         with open(path) as f:
-            return json.load(f).get("traffic_bytes_per_launch")
+            z = json.load(f)
     except (OSError, ValueError):
-        return None
+        return None, None
+    if not any(h in z.get("kernel", "") for h in kernel_hashes):
+        return None, f"profiles/hbm_traffic_{workload}.json is for {z.get('kernel')}, not the kernel timed here"
+    return z.get("traffic_bytes_per_launch"), f"profiles/hbm_traffic_{workload}.json (rocprofv3 --pmc, kernel {z.get('kernel')})"
+
+
+def launch_flops(step) -> float:
+    """Algorithmic flops of one MFMA launch of the plan (attention counted causal-aware)."""
+    a, k = step.attrs, step.kind
+    if k == "gemm":
+        return 2.0 * a["M"] * a["N"] * a["K"] * max(a.get("batch", 1), 1)
+    if k in ("attention", "attention_bwd"):
+        f = 4.0 * a["B"] * a["H"] * a["S"] * a["S"] * a["hd"] * (0.5 if a["causal"] else 1.0)
+        return f if k == "attention" else 2.5 * f
+    if k.startswith("conv2d"):
+        n, ho, wo, co = a["y_shape"]
+        r, s, ci, _ = a["w_shape"]
+        return 2.0 * n * ho * wo * co * r * s * ci
+    return 0.0
+
+
+def launch_label(step) -> str:
+    a, k = step.attrs, step.kind
+    if k == "gemm":
+        lay = ("n" if a["a_cs"] == 1 else "t") + ("n" if a["b_cs"] == 1 else "t")
+        b = f" x{a['batch']}" if a.get("batch", 1) > 1 else ""
+        return f"gemm {lay} {a['M']}x{a['N']}x{a['K']}{b}"
+    if k in ("attention", "attention_bwd"):
+        return f"{k} B{a['B']} H{a['H']} S{a['S']} hd{a['hd']}"
+    if k.startswith("conv2d"):
+        return f"{k} x{tuple(a['x_shape'])} w{tuple(a['w_shape'])}"
+    return k
+
+
+def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
+    import torch
+    from nabla_amd.backend import lib as nbk_lib
+    cf = nb.compile(w["fn"])
+    args = w["args"]
+    out = cf(*args)  # miss: trace, lower, bind
+    spec = next(iter(next(iter(cf._cache.values())).specializations.values()))
+    plan = spec.bound.plan
+    flat, _ = nb.tree_flatten((args, {}))
+    inputs = [flat[v]._impl._buffer if kind == "arg" else v for kind, v in spec.input_plan]
+    single = len(plan.steps) == 1
+
+    if calibrate_copy:
+        n = 64 * 1024 * 1024  # fp32 elements: 256 MiB read, 256 MiB written per launch
+        src = torch.zeros(n, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        shape, st1 = (C.c_int64 * 1)(n), (C.c_int64 * 1)(1)
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(3):
+            nbk_lib.check(L.nbk_copy_strided(C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), 0, 0,
+                                             1, shape, st1, st1, stream))
+        sync()
+        del src, dst
+
+    for _ in range(warmup):
+        out = cf(*args)
+    sync()
+    timer = KernelTimer(L, w["kinds"])
+    replays0 = ex.graph_replays
+    if single:
+        ex.launch_timer = timer  # one launch per step: the events sit inside the timed region
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = cf(*args)
+    sync()
+    wall = time.perf_counter() - t0
+    ex.launch_timer = None
+    replays = ex.graph_replays - replays0
+    if single:
+        kernel_timing = "HIP events around the launch, inside the timed region"
+        dur = timer.durations_ms()
+    del out
+    # the same plan one layer below the public call
+    for _ in range(min(warmup, 3)):
+        spec.bound.run(inputs)
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        spec.bound.run(inputs)
+    sync()
+    wall_plan = time.perf_counter() - t0
+    if not single:
+        n2 = min(steps, 20)
+        for _ in range(n2):
+            spec.bound.run(inputs, timer=timer)
+        sync()
+        dur = timer.durations_ms()
+        kernel_timing = (f"second pass of {n2} steps, plain launches bracketed by HIP events on the "
+                         "launch stream (the timed region replays the step as one HIP graph, inside "
+                         "which events cannot be recorded)")
+    dom_ms = sum(dur.values())
+
+    if w["bound"] == "hbm":
+        achieved = w["algo"] / (dom_ms * 1e-3) / 1e9 if dom_ms else 0.0
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = w["algo"] / (dom_ms * 1e-3) / 1e12 if dom_ms else 0.0
+        peak, unit = MFMA_PEAK_TFLOPS[w["dtype"]], "TFLOP/s"
+    traffic, traffic_source = None, None
+    if w["bound"] == "hbm":
+        hashes = set()
+        for call in spec.bound.calls:
+            if call[0] is L.nbk_rowprog_launch:
+                hashes.add(f"{L.nbk_rowprog_hash(C.byref(call[3])):016x}")
+        traffic, traffic_source = committed_traffic(w["key"], hashes)
+    roofline = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                "frac": round(achieved / peak, 4), "traffic": traffic,
+                "kernel": "+".join(k for k in w["kinds"] if k in plan.stats),
+                "kernel_ms_per_step": round(dom_ms, 4), "launches_per_step": len(dur),
+                "algorithmic_per_step": w["algo"], "kernel_timing": kernel_timing}
+    if traffic_source:
+        roofline["traffic_source"] = traffic_source
+    if w["bound"] == "mfma":
+        # per product shape: launches per step, mean duration, achieved rate from that shape's own
+        # flop count (2 M N K; attention causal-aware)
+        groups: dict = {}
+        for (si, kind), ms in dur.items():
+            st = plan.steps[si]
+            g = groups.setdefault(launch_label(st), [0, 0.0, 0.0])
+            g[0] += 1
+            g[1] += ms
+            g[2] += launch_flops(st)
+        by = []
+        for label, (n, ms, fl) in sorted(groups.items(), key=lambda kv: -kv[1][1]):
+            tf = fl / (ms * 1e-3) / 1e12 if ms else 0.0
+            by.append({"kernel": label, "launches": n, "avg_us": round(ms / n * 1e3, 2),
+                       "tflops": round(tf, 1), "frac": round(tf / peak, 4)})
+        roofline["by_kernel"] = by[:12]
+        roofline["counted_flops_per_step"] = sum(g[2] for g in groups.values())
+    res = {"workload": w["name"], "value": round(steps / wall, 3), "unit": "steps/s",
+           "ms_per_step": round(wall / steps * 1e3, 4),
+           "plan_ms_per_step": round(wall_plan / steps * 1e3, 4),
+           "dtype": w["dtype"], "graph_replays_in_timed_region": replays,
+           "plan": plan.stats, "roofline": roofline}
+    if with_cpu:
+        res["cpu_baseline"] = w["cpu"](host)
+    return res
 
 
 def main() -> int:
@@ -194,8 +394,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB copy (nbk_copy_strided) three times before the "
                          "steps: the known-size kernel that hardware byte counters are scaled by")
@@ -205,87 +405,44 @@ def main() -> int:
               "(run with --gpus 1)", file=sys.stderr)
         return 2
 
+    import torch
+
     import nabla_amd as nb
     from nabla_amd.backend import lib as nbk_lib
     from nabla_amd.backend.executor import get_executor
+    from nabla_amd.core import engine
 
     ex = get_executor()  # raises without libnbk.so or without a gfx950 GPU
     L = nbk_lib.load()
-    w = WORKLOADS[a.workload](nb)
-    cf, spec, bufs, first = compiled_plan(nb, w["fn"], w["args"])
-    plan = spec.bound.plan
-    inputs = bufs()
-
-    if a.calibrate_copy:
-        import ctypes as C
-        import torch
-        n = 64 * 1024 * 1024  # fp32 elements: 256 MiB read, 256 MiB written per launch
-        src = torch.zeros(n, dtype=torch.float32, device="cuda")
-        dst = torch.empty_like(src)
-        shape = (C.c_int64 * 1)(n)
-        st1 = (C.c_int64 * 1)(1)
-        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-        for _ in range(3):
-            nbk_lib.check(L.nbk_copy_strided(C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), 0, 0,
-                                             1, shape, st1, st1, stream))
-        sync()
-    for _ in range(a.warmup):
-        spec.bound.run(inputs)
-    sync()
-    # (the fused attention kernels are MFMA work counted in the same algorithmic flops)
-    dominant_kinds = {"rowprog": ["rowprog"], "gemm": ["gemm", "attention", "attention_bwd"],
-                      "conv": ["conv2d", "conv2d_dgrad", "conv2d_wgrad"]}[w["dominant"]]
-    timer = KernelTimer(L, dominant_kinds)
-    if len(plan.steps) == 1:
-        # one launch per step: the HIP events sit inside the timed region
-        t0 = time.perf_counter()
-        for _ in range(a.steps):
-            spec.bound.run(inputs, timer=timer)
-        sync()
-        wall = time.perf_counter() - t0
-    else:
-        # several launches per step: the product path replays the repeated step as one HIP
-        # graph, inside which no event can be recorded; the step rate is timed on that path
-        # and the kernel durations for the roofline come from a second pass of plain launches
-        # with events on the launch stream
-        t0 = time.perf_counter()
-        for _ in range(a.steps):
-            spec.bound.run(inputs)
-        sync()
-        wall = time.perf_counter() - t0
-        for _ in range(min(a.steps, 20)):
-            spec.bound.run(inputs, timer=timer)
-        sync()
-    ms_per_step = wall / a.steps * 1e3
-    dur = timer.durations_ms()
-    per_step_total = {}
-    for (si, kind), v in dur.items():
-        per_step_total[(si, kind)] = sum(v) / len(v)
-    dom_ms = sum(per_step_total.values())
-    # the single longest launch of the dominant kind
-    top = max(per_step_total.items(), key=lambda kv: kv[1]) if per_step_total else None
-
-    if w["bound"] == "hbm":
-        achieved = w["algo"] / (dom_ms * 1e-3) / 1e9 if dom_ms else 0.0
-        peak, unit = HBM_PEAK_GBS, "GB/s"
-    else:
-        achieved = w["algo"] / (dom_ms * 1e-3) / 1e12 if dom_ms else 0.0
-        peak, unit = MFMA_PEAK_TFLOPS[w["dtype"]], "TFLOP/s"
-    roofline = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                "frac": round(achieved / peak, 4), "traffic": measured_traffic(a.workload),
-                "kernel": "+".join(k for k in dominant_kinds if k in plan.stats),
-                "kernel_ms_per_step": round(dom_ms, 4),
-                "launches_per_step": len(per_step_total)}
-    cpu = None if a.no_cpu else w["cpu"]()
+    host = host_info()
+    names = sorted(WORKLOADS) if a.workload == "all" else [a.workload]
+    results = {}
+    for name in names:
+        w = WORKLOADS[name](nb)
+        w["key"] = name
+        results[name] = measure(nb, L, ex, w, a.steps, a.warmup, not a.no_cpu, host,
+                                calibrate_copy=a.calibrate_copy)
+        del w
+        engine.clear_plan_cache()
+        gc.collect()
+        torch.cuda.empty_cache()
+    head = results[names[-1]]  # c5 (the largest configuration) when all five run
     line = {
-        "metric": "train steps/sec fwd+bwd at 1 MI355X; GEMM % MFMA peak; fused-op % HBM BW",
-        "value": round(a.steps / wall, 3), "unit": "steps/s", "n_gpus": 1, "steps": a.steps,
-        "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": w["name"], "step": "compiled replay of forward + gradients",
-                   "plan": plan.stats, "graph_replays": ex.graph_replays},
-        "roofline": roofline, "cpu_baseline": cpu,
+        "metric": METRIC, "value": head["value"], "unit": "steps/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": head["workload"],
+                   "step": "public compiled call: forward + gradients, inputs resident in HBM",
+                   "plan_ms_per_step": head["plan_ms_per_step"], "plan": head["plan"],
+                   "graph_replays_in_timed_region": head["graph_replays_in_timed_region"]},
+        "roofline": head["roofline"], "cpu_baseline": head.get("cpu_baseline"),
     }
+    if len(names) > 1:
+        line["configs"] = {k: {kk: v[kk] for kk in ("workload", "value", "unit", "ms_per_step",
+                                                    "plan_ms_per_step", "dtype", "roofline",
+                                                    "cpu_baseline") if kk in v}
+                           for k, v in results.items()}
+        line["host"] = host
     print(json.dumps(line))
     return 0
 

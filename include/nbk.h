@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 11
+#define NBK_ABI_VERSION 12
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -168,6 +168,11 @@ int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream);
  * for this program, 0 if the interpreter will run it.  Results are the same
  * either way; setting NBK_ROWPROG_INTERPRET=1 forces the interpreter. */
 int nbk_rowprog_is_specialized(const nbk_rowprog* prog);
+/* The 64-bit hash (FNV-1a over header, operand classes, instructions, immediates; pointers,
+ * strides and extents excluded) by which a program finds its specialised kernel.  That
+ * kernel's name ends in the hash in hex, so a profile can be matched to the program it is
+ * for.  0 for an invalid program. */
+uint64_t nbk_rowprog_hash(const nbk_rowprog* prog);
 
 /* ===================================================================== */
 /*  Reductions over a middle / leading axis                               */

@@ -45,9 +45,10 @@ class BoundPlan:
         self.dynamic = [b.id for b in plan.bufs if b.role in ("input", "output")]
         self.calls: list[tuple] = []  # (fn, args tuple, patch list)
         self.has_gather = any(st.kind in ("gather", "scatter") for st in plan.steps)
-        self._graphs: dict = {}  # pointer tuple -> recorded launch sequence (at most four)
+        self._graphs: dict = {}  # pointer tuple -> recorded launch sequence (at most eight)
         self._seen: set = set()  # pointer tuples that have run once already
         self._graph_off = any(st.kind == "custom" for st in plan.steps)  # user kernels may not be capturable
+        self._layout_outputs()
         self._prepare()
 
     # -- address helpers -------------------------------------------------------
@@ -305,30 +306,15 @@ class BoundPlan:
         ex = self.ex
         if len(inputs) != plan.n_inputs:
             raise ValueError(f"plan expects {plan.n_inputs} inputs, got {len(inputs)}")
+        if timer is None:
+            timer = ex.launch_timer
         keep = []
-        outs: list[torch.Tensor] = [None] * len(plan.outputs)  # type: ignore
-        # every output of the step is a view into one allocation.  It is at least 2 MiB so that
-        # it comes from the allocator's pool for large blocks: a loop that drops its results
-        # before the next step then gets the same block back whatever small allocations happen
-        # in between, which is what lets the step be replayed as a recorded graph
+        large, small, small_dst = self._take_slabs()
         out_by_buf = {}
-        offs, total = {}, 0
-        for bid, shape, dtype in plan.outputs:
-            if bid not in offs:
-                offs[bid] = total
-                n = 1
-                for d in shape:
-                    n *= d
-                total += (max(n, 1) * dtype.size_in_bytes + 255) & ~255
-        slab = torch.empty(max(total, 1 << 21), dtype=torch.uint8, device=ex.torch_device)
-        for oi, (bid, shape, dtype) in enumerate(plan.outputs):
-            if bid not in out_by_buf:
-                n = 1
-                for d in shape:
-                    n *= d
-                piece = slab[offs[bid]:offs[bid] + n * dtype.size_in_bytes]
-                out_by_buf[bid] = piece.view(dtype.to_torch()).reshape(shape)
-            outs[oi] = out_by_buf[bid]
+        for bid, (is_small, off, nbytes, shape, dtype) in self._out_layout.items():
+            piece = (small if is_small else large)[off:off + nbytes]
+            out_by_buf[bid] = piece.view(dtype.to_torch()).reshape(shape)
+        outs: list[torch.Tensor] = [out_by_buf[bid] for bid, _, _ in plan.outputs]
         for b in plan.bufs:
             if b.role == "input":
                 t = inputs[b.index]
@@ -344,25 +330,106 @@ class BoundPlan:
         base = self.base
         check = lib.check
         # Replay as a HIP graph: a step that runs again on the very buffers of an earlier
-        # run (inputs unchanged, the allocator handed the same output blocks back) is
+        # run (inputs unchanged, outputs in a slab of this plan that has come free again) is
         # recorded once and from then on costs one launch call instead of one per kernel.
         if ex.use_graphs and timer is None and not keep and len(self.calls) > 1 and not self._graph_off:
             key = tuple(base[b] for b in self.dynamic)
             g = self._graphs.get(key)
-            if g is None and key in self._seen and len(self._graphs) < 4:
+            if g is None and key in self._seen and len(self._graphs) < 8:
                 g = self._record(key)
             if g is not None:
                 check(ex.lib.nbk_graph_launch(g, stream))
                 ex.graph_replays += 1
                 if self.has_gather:
                     ex.status_dirty = True
-                return outs
+                return self._finish(outs, small_dst)
             if len(self._seen) < 64:
                 self._seen.add(key)
         self._issue(stream, timer)
         del keep
         if self.has_gather:
             ex.status_dirty = True
+        return self._finish(outs, small_dst)
+
+    # -- output storage ------------------------------------------------------------
+    #: results up to this many bytes (losses, counters, small bias gradients) live apart from
+    #: the large ones, so that a caller who keeps a loss keeps a few KB alive, not the step's
+    #: gradients
+    SMALL_OUTPUT_BYTES = 4096
+    POOL_SLABS = 4
+
+    def _layout_outputs(self) -> None:
+        """Offsets of every distinct output buffer inside the step's two allocations."""
+        self._out_layout: dict = {}
+        totals = [0, 0]
+        for bid, shape, dtype in self.plan.outputs:
+            if bid in self._out_layout:
+                continue
+            n = 1
+            for d in shape:
+                n *= d
+            nbytes = n * dtype.size_in_bytes
+            is_small = nbytes <= self.SMALL_OUTPUT_BYTES
+            self._out_layout[bid] = (is_small, totals[is_small], nbytes, tuple(shape), dtype)
+            totals[is_small] += (max(nbytes, 1) + 255) & ~255
+        self._out_bytes = (max(totals[0], 256), max(totals[1], 256))
+        self._pools: tuple = ([], [])   # per class: [slab, use count when nobody holds a view]
+        self._small_stage = None         # fixed small slab the kernels write once callers hoard
+        self._runs = 0
+
+    def _new_slab(self, nbytes: int):
+        return torch.empty(nbytes, dtype=torch.uint8, device=self.ex.torch_device)
+
+    @staticmethod
+    def _use_count(slab) -> int:
+        return torch._C._storage_Use_Count(slab.untyped_storage()._cdata)
+
+    def _from_pool(self, cls: int):
+        """A slab of this plan that no returned tensor (or anything made from one: views, DLPack
+        exports) refers to any more, a new pooled one while the pool has room, else None.  The
+        plan owns its slabs, so a step whose caller drops or overwrites the previous results
+        runs on the same addresses again whatever the allocator does in between, which is what
+        lets the step be replayed as a recorded graph."""
+        pool = self._pools[cls]
+        for slab, idle in pool:
+            if self._use_count(slab) == idle:
+                return slab
+        if len(pool) < self.POOL_SLABS:
+            slab = self._new_slab(self._out_bytes[cls])
+            pool.append((slab, self._use_count(slab)))
+            return slab
+        return None
+
+    def _take_slabs(self):
+        """(large slab, small slab the kernels write, small slab the caller gets or None)."""
+        self._runs += 1
+        if self._runs == 1:
+            # a plan that runs once (eager evaluation of a new expression) keeps nothing
+            return self._new_slab(self._out_bytes[0]), self._new_slab(self._out_bytes[1]), None
+        large = self._from_pool(0)
+        if large is None:  # the caller holds the results of POOL_SLABS steps: plain allocations
+            large = self._new_slab(self._out_bytes[0])
+        if self._small_stage is None:
+            small = self._from_pool(1)
+            if small is not None:
+                return large, small, None
+            # the caller keeps the small results of many steps (a list of losses): from now on
+            # the kernels write them to one fixed slab (same addresses every step, so the
+            # recorded step stays valid) and each step hands out a copy
+            self._small_stage = self._new_slab(self._out_bytes[1])
+        return large, self._small_stage, True
+
+    def _finish(self, outs, small_dst):
+        if small_dst is None:
+            return outs
+        copy = self._small_stage.clone()  # ordered behind the step on the current stream
+        done = {}
+        for oi, (bid, _, _) in enumerate(self.plan.outputs):
+            is_small, off, nbytes, shape, dtype = self._out_layout[bid]
+            if is_small:
+                if bid not in done:
+                    done[bid] = copy[off:off + nbytes].view(dtype.to_torch()).reshape(shape)
+                outs[oi] = done[bid]
         return outs
 
     def _record(self, key):
@@ -452,6 +519,7 @@ class HipExecutor:
         self.graph_replays = 0
         self.status_dirty = False        # a launched plan may have flagged a bad gather index
         self.force_interpreter = False   # plans bound while set never use specialised row kernels
+        self.launch_timer = None         # callable(step index, kind, stream) -> callable | None: measurement hook; plans run as plain launches while set
 
     def current_stream(self) -> int:
         return torch.cuda.current_stream(self.torch_device).cuda_stream

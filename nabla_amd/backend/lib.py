@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 MAX_RANK = 8
 
@@ -129,6 +129,7 @@ _SIGNATURES = {
     "nbk_graph_destroy": ([C.c_void_p], C.c_int),
     "nbk_rowprog_launch": ([C.POINTER(RowProg), C.c_void_p], C.c_int),
     "nbk_rowprog_is_specialized": ([C.POINTER(RowProg)], C.c_int),
+    "nbk_rowprog_hash": ([C.POINTER(RowProg)], C.c_uint64),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
                         C.c_int64, C.c_int32, C.c_void_p], C.c_int),
     "nbk_reduce_mid_batch": ([C.POINTER(ReduceTask), C.c_int32, C.c_void_p], C.c_int),

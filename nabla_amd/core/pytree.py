@@ -109,7 +109,10 @@ def tree_unflatten(treedef: PyTreeDef, leaves) -> Any:
             return _REGISTRY[d.kind][1](d.aux, kids)
         return d.kind(*kids)  # namedtuple
 
-    return go(treedef)
+    try:
+        return go(treedef)
+    finally:
+        go = None  # (self-referential closure holding `leaves`, as in tree_flatten)
 
 
 def tree_leaves(tree: Any, is_leaf=None) -> list:

@@ -522,6 +522,11 @@ extern "C" int nbk_rowprog_is_specialized(const nbk_rowprog* prog) {
   return (!rp_specs_disabled() && rp_find_spec(rp_program_hash(prog)) != nullptr) ? 1 : 0;
 }
 
+extern "C" uint64_t nbk_rowprog_hash(const nbk_rowprog* prog) {
+  if (rp_validate(prog) != NBK_OK) return 0;
+  return rp_program_hash(prog);
+}
+
 extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
   int rc = rp_validate(prog);
   if (rc != NBK_OK) return rc;

@@ -426,13 +426,9 @@ def test_adamw_and_sgd_steps_on_device(hip, dtype, tol):
 def test_graph_replay_matches_eager_every_time(hip):
     """A compiled step called again on the same buffers is recorded once and replayed; every
     replay is checked against the oracle, with unrelated eager work and synchronisation between
-    the replays, and a call on new buffers falls back to plain launches."""
-    import gc
-    import torch
-    # (a replay needs the allocator to hand the step the same output block again: start from
-    # an empty cache so that blocks left behind by earlier tests do not take turns)
-    torch.cuda.synchronize()
-    torch.cuda.empty_cache()
+    the replays, and a call on new buffers falls back to plain launches.  The plan owns the
+    slabs its results live in, so the replay does not depend on what the allocator hands out:
+    the caller just lets go of the previous results, as a training loop does."""
     t = oc.c1_inputs(64, 96, 48, 10, seed=31)
     t["b1"] = np.random.default_rng(2).uniform(-0.05, 0.05, t["b1"].shape).astype(np.float32)
     wl, wg = oc.c1_reference(**t)
@@ -446,11 +442,11 @@ def test_graph_replay_matches_eager_every_time(hip):
         assert abs(got[0] - wl) <= F32_TOL * abs(wl) + 1e-9, it
         for g, w in zip(got[1:], wg):
             assert relerr(g, w) < F32_TOL, it
-        del loss, grads, got
-        gc.collect()  # (graph nodes of the step form cycles: drop them now, not when the collector likes)
-        # unrelated work between replays
+        # unrelated work between replays (allocations of all sizes included)
         np.testing.assert_array_equal((other * 2.0 + float(it)).numpy(), np.arange(12) * 2.0 + it)
-    assert hip.graph_replays > before, "the repeated step was never replayed as a graph"
+        junk = torch.empty((it + 1) << 20, dtype=torch.uint8, device="cuda")
+        del junk
+    assert hip.graph_replays - before >= 3, "the repeated step was not replayed as a graph"
     # new input buffers: pointers differ, the recording must not be used
     t2 = oc.c1_inputs(64, 96, 48, 10, seed=32)
     wl2, wg2 = oc.c1_reference(**t2)
@@ -458,6 +454,43 @@ def test_graph_replay_matches_eager_every_time(hip):
     assert abs(loss.item() - wl2) <= F32_TOL * abs(wl2) + 1e-9
     for g, w in zip(grads, wg2):
         assert relerr(g.numpy(), w) < F32_TOL
+
+
+def test_kept_losses_stay_valid_and_do_not_pin_the_gradients(hip):
+    """A loop that keeps every loss tensor: each kept loss still reads its own step's value
+    after later steps ran (no slab is written while something refers to it), the gradients of
+    all those steps share a few recycled slabs instead of one allocation per kept loss, and
+    the step is still replayed as a graph once the inputs repeat."""
+    rng = np.random.default_rng(33)
+    w = rng.standard_normal((256, 384)).astype(np.float32)
+    W = T(w)
+
+    @nb.compile
+    def step(W, x):
+        return nb.value_and_grad(lambda W: nb.mean(nb.tanh(x @ W) ** 2))(W)
+
+    xs = [rng.standard_normal((32, 256)).astype(np.float32) for _ in range(9)]
+    want = [float(np.mean(np.tanh(x.astype(np.float64) @ w.astype(np.float64)) ** 2)) for x in xs]
+    kept, grad_ptrs = [], set()
+    for x in xs:
+        loss, g = step(W, T(x))
+        kept.append(loss)
+        grad_ptrs.add(g._impl._buffer.untyped_storage().data_ptr())
+        del g
+    for loss, wl in zip(kept, want):
+        assert abs(loss.item() - wl) <= F32_TOL * abs(wl)
+    assert len({l._impl._buffer.untyped_storage().data_ptr() for l in kept}) == len(kept)
+    assert len(grad_ptrs) <= 3, "dropped gradients must be recycled although the losses are kept"
+    # the same inputs again and again, still keeping the losses: replayed, values unchanged
+    X = T(xs[0])
+    before = hip.graph_replays
+    for _ in range(6):
+        loss, g = step(W, X)
+        kept.append(loss)
+        del g
+    assert hip.graph_replays - before >= 3
+    for loss in kept[-6:]:
+        assert abs(loss.item() - want[0]) <= F32_TOL * abs(want[0])
 
 
 # ---- avg_pool2d, silu -------------------------------------------------------------------------------
