@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 12
+#define NBK_ABI_VERSION 13
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -330,6 +330,23 @@ int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
                       const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                       const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
                       void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The same backward pass for callers that cannot allocate device memory or hand over a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  The row sums live in scratch that is
+ * part of the library image (NBK_ATTN_STATIC_ROWS floats = 4 MiB per GPU, held until the
+ * process ends); the call allocates nothing and fails with NBK_ERR_INVALID when
+ * B * H * S > NBK_ATTN_STATIC_ROWS.  Results are those of nbk_attention_bwd bit for bit.
+ * All calls on one GPU share that scratch: calls that overlap in time on one GPU (two streams)
+ * race; calls on one stream, or ordered by events, do not.  Nothing needs clearing between
+ * calls (each call writes every row it later reads). */
+#define NBK_ATTN_STATIC_ROWS (1 << 20)
+int nbk_attention_bwd_static(const nbk_attn_desc* d, const nbk_attn_tensor* q,
+                             const nbk_attn_tensor* k, const nbk_attn_tensor* v,
+                             const nbk_attn_tensor* o, const void* lse,
+                             const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                             const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
+                             void* stream);
 
 /* ===================================================================== */
 /*  Index ops (bit-exact)                                                 */

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 MAX_RANK = 8
 
@@ -155,6 +155,8 @@ _SIGNATURES = {
     "nbk_attention_bwd_workspace": ([C.POINTER(AttnDesc)], C.c_int64),
     "nbk_attention_bwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p] +
                           [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_int64, C.c_void_p], C.c_int),
+    "nbk_attention_bwd_static": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p] +
+                                 [C.POINTER(AttnTensor)] * 4 + [C.c_void_p], C.c_int),
     "nbk_gather": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64,
                     C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_scatter": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,

@@ -43,7 +43,7 @@ extern "C" int nbk_init(int device) {
                   prop.gcnArchName);
     return NBK_ERR_UNSUPPORTED;
   }
-  return NBK_OK;
+  return nbk_attention_static_setup();
 }
 
 // ---- events / stream sync ---------------------------------------------------

@@ -27,6 +27,7 @@
 //   transposed [hd rows][64 cols]  row pitch 68 elements: the 8-byte reads of 32
 //                                  consecutive rows fall on distinct banks per half
 #include "nbk_common.h"
+#include <mutex>
 
 #include <utility>
 
@@ -709,27 +710,11 @@ extern "C" int64_t nbk_attention_bwd_workspace(const nbk_attn_desc* d) {
   return d->B * d->H * d->S * (int64_t)sizeof(float);
 }
 
-extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
-                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
-                                 const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
-                                 const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, void* workspace,
-                                 int64_t workspace_bytes, void* stream) {
-  AttnArgs a = {};
-  int rc = attn_common(d, &a);
-  if (rc) return rc;
-  if ((rc = attn_tensor(q, "q", &a.q, true)) || (rc = attn_tensor(k, "k", &a.k, true)) ||
-      (rc = attn_tensor(v, "v", &a.v, true)) || (rc = attn_tensor(o, "o", &a.o, true)) ||
-      (rc = attn_tensor(dout, "dout", &a.dout, true)) || (rc = attn_tensor(dq, "dq", &a.dq, true)) ||
-      (rc = attn_tensor(dk, "dk", &a.dk, true)) || (rc = attn_tensor(dv, "dv", &a.dv, true)))
-    return rc;
-  NBK_REQUIRE(lse != nullptr, "attention: null lse");
-  NBK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 15) == 0 &&
-                  workspace_bytes >= nbk_attention_bwd_workspace(d),
-              "attention: backward needs %lld bytes of 16-byte aligned workspace",
-              (long long)nbk_attention_bwd_workspace(d));
-  a.lse = (float*)lse;
-  a.delta = (float*)workspace;
-  hipStream_t st = (hipStream_t)stream;
+// Launches of the backward pass once the arguments are checked; `delta` is B * H * S floats of
+// device scratch (one per score row).
+static int attn_bwd_launch(const nbk_attn_desc* d, AttnArgs& a, float* delta, hipStream_t st) {
+  int rc;
+  a.delta = delta;
   const int64_t rows = d->B * d->H * d->S;
   const dim3 grid((unsigned)(d->B * d->H), (unsigned)(d->S / 128));
   if (d->hd == 64) {
@@ -751,3 +736,89 @@ extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* 
   }
   return nbk_check_launch("attn_bwd kernels");
 }
+
+static int attn_bwd_args(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
+                         const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
+                         const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                         const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, AttnArgs* a) {
+  int rc = attn_common(d, a);
+  if (rc) return rc;
+  if ((rc = attn_tensor(q, "q", &a->q, true)) || (rc = attn_tensor(k, "k", &a->k, true)) ||
+      (rc = attn_tensor(v, "v", &a->v, true)) || (rc = attn_tensor(o, "o", &a->o, true)) ||
+      (rc = attn_tensor(dout, "dout", &a->dout, true)) || (rc = attn_tensor(dq, "dq", &a->dq, true)) ||
+      (rc = attn_tensor(dk, "dk", &a->dk, true)) || (rc = attn_tensor(dv, "dv", &a->dv, true)))
+    return rc;
+  NBK_REQUIRE(lse != nullptr, "attention: null lse");
+  a->lse = (float*)lse;
+  return NBK_OK;
+}
+
+extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
+                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
+                                 const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                                 const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, void* workspace,
+                                 int64_t workspace_bytes, void* stream) {
+  AttnArgs a = {};
+  int rc = attn_bwd_args(d, q, k, v, o, lse, dout, dq, dk, dv, &a);
+  if (rc) return rc;
+  NBK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 15) == 0 &&
+                  workspace_bytes >= nbk_attention_bwd_workspace(d),
+              "attention: backward needs %lld bytes of 16-byte aligned workspace",
+              (long long)nbk_attention_bwd_workspace(d));
+  return attn_bwd_launch(d, a, (float*)workspace, (hipStream_t)stream);
+}
+
+// ---- the backward pass for callers that cannot allocate ------------------------------------
+// Scratch of the library's own: one float per score row, NBK_ATTN_STATIC_ROWS of them, in a
+// file-scope device array (every GPU the library runs on holds its own copy, 4 MiB, until the
+// process ends).  In host code the array's name is only a handle: the device address is asked
+// for once per device and kept.
+static __device__ __align__(256) float attn_scratch[NBK_ATTN_STATIC_ROWS];
+#define NBK_MAX_DEVICES 64
+static float* g_attn_scratch_ptr[NBK_MAX_DEVICES] = {};
+static std::mutex g_attn_scratch_mu;
+
+// The address of this device's copy of the scratch array (the device must be current).
+static int attn_scratch_for_current_device(float** out) {
+  int dev = -1;
+  NBK_HIP(hipGetDevice(&dev));
+  NBK_REQUIRE(dev >= 0 && dev < NBK_MAX_DEVICES, "attention: device ordinal %d beyond %d", dev,
+              NBK_MAX_DEVICES);
+  std::lock_guard<std::mutex> lk(g_attn_scratch_mu);
+  if (g_attn_scratch_ptr[dev] == nullptr) {
+    float* ptr = nullptr;
+    NBK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(attn_scratch)));
+    NBK_REQUIRE(ptr != nullptr, "attention: no device address for the scratch array");
+    g_attn_scratch_ptr[dev] = ptr;
+  }
+  *out = g_attn_scratch_ptr[dev];
+  return NBK_OK;
+}
+
+// Called by nbk_init with the chosen device current.
+int nbk_attention_static_setup(void) {
+  float* ptr;
+  return attn_scratch_for_current_device(&ptr);
+}
+
+extern "C" int nbk_attention_bwd_static(const nbk_attn_desc* d, const nbk_attn_tensor* q,
+                                        const nbk_attn_tensor* k, const nbk_attn_tensor* v,
+                                        const nbk_attn_tensor* o, const void* lse,
+                                        const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
+                                        const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
+                                        void* stream) {
+  AttnArgs a = {};
+  int rc = attn_bwd_args(d, q, k, v, o, lse, dout, dq, dk, dv, &a);
+  if (rc) return rc;
+  const int64_t rows = d->B * d->H * d->S;
+  NBK_REQUIRE(rows <= NBK_ATTN_STATIC_ROWS,
+              "attention: B * H * S = %lld score rows exceed the %d rows of built-in scratch; use "
+              "nbk_attention_bwd with a workspace",
+              (long long)rows, NBK_ATTN_STATIC_ROWS);
+  float* delta = nullptr;
+  if ((rc = attn_scratch_for_current_device(&delta))) return rc;
+  // every row of the scratch that the kernels read is written first by the row-sum kernel of
+  // this call, so nothing has to be cleared between calls
+  return attn_bwd_launch(d, a, delta, (hipStream_t)stream);
+}
+

@@ -12,6 +12,9 @@
 void nbk_set_error(const char* fmt, ...);
 // Compute units of the current device (256 on MI355X); set by nbk_init, lazily otherwise.
 int nbk_num_cus(void);
+// Looks up the device address of the attention kernels' built-in scratch for the current
+// device (attention.hip); nbk_init calls it right after selecting the device.
+int nbk_attention_static_setup(void);
 
 #define NBK_REQUIRE(cond, ...)            \
   do {                                    \
