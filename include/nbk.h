@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 13
+#define NBK_ABI_VERSION 14
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -227,6 +227,11 @@ enum nbk_gemm_act { NBK_ACT_NONE = 0, NBK_ACT_RELU = 1, NBK_ACT_GELU = 2 };
 /* what the residual does to the result: added (x + r: a skip connection, an accumulated
  * gradient) or multiplied in (x * r: the saved derivative of an activation, a mask) */
 enum nbk_gemm_residual_op { NBK_RES_ADD = 0, NBK_RES_MUL = 1 };
+/* second result of the same launch: C_aux = act'(alpha * op(A) @ op(B) + bias), the derivative of
+ * the activation at the value the activation was applied to (what the backward pass of
+ * gelu(x @ W + b) multiplies the cotangent with: nabla/ops/unary.py:567-595), taken from the
+ * fp32 accumulator like C itself, so that the pre-activation never makes a trip through memory */
+enum nbk_gemm_aux_op { NBK_AUX_NONE = 0, NBK_AUX_ACT_GRAD = 1 };
 typedef struct nbk_gemm_desc {
   const void* A; const void* B; void* C;
   const void* bias;      /* NULL or [N] (dtype_c), added to every row        */
@@ -244,6 +249,9 @@ typedef struct nbk_gemm_desc {
   int32_t batch_reduce;
   float alpha;
   int32_t residual_op;   /* enum nbk_gemm_residual_op */
+  void* C_aux;           /* NULL or a second result in C's layout and dtype (see nbk_gemm_aux_op) */
+  int32_t aux_op;        /* enum nbk_gemm_aux_op; needs act != NBK_ACT_NONE and no residual */
+  int32_t reserved;
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
 

@@ -41,7 +41,7 @@ def _compile(src: Path, force: bool) -> Path:
     deps = [src, *CSRC.glob("*.h"), *INCLUDE.glob("*.h")]
     if not force and obj.exists() and all(obj.stat().st_mtime > d.stat().st_mtime for d in deps):
         return obj
-    cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *FLAGS, *os.environ.get("NBK_EXTRA_HIPCC_FLAGS", "").split(), "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{res.stderr[-4000:]}")

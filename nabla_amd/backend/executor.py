@@ -163,7 +163,14 @@ class BoundPlan:
                     raise TypeError(f"matmul operands differ in dtype: {ra.dtype} vs {rb.dtype}")
                 d.dtype_ab = ra.dtype.abi
                 d.dtype_c = rc.dtype.abi
-                d.act = 0
+                d.act = {None: 0, "relu": 1, "gelu": 2}[a.get("act")]
+                d.C_aux, d.aux_op = None, 0
+                if a.get("aux_dst") is not None:
+                    raux = a["aux_dst"]
+                    if raux.dtype is not rc.dtype:
+                        raise TypeError(f"matmul second result is {raux.dtype}, the first {rc.dtype}")
+                    ptr_field(d, "C_aux", raux.buf, raux.offset * raux.dtype.size_in_bytes)
+                    d.aux_op = 1
                 d.batch_reduce = 0
                 d.alpha = a.get("alpha", 1.0)
                 self.calls.append((L.nbk_gemm, [C.byref(d)], patches, d))

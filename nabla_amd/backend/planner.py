@@ -713,6 +713,44 @@ class Planner:
                 n.attrs = dict(mm.attrs or {}, bias_in=2)
                 break
 
+    def _fold_activation_into_matmul(self) -> None:
+        """``gelu(x @ W + b)`` whose pre-activation has no reader but the activation and, in a
+        training step, its derivative (``GeluOp``'s VJP multiplies the cotangent with
+        ``dgelu`` of the same value): both become results of the product itself, computed in
+        its epilogue from the fp32 accumulator, and the pre-activation never reaches memory.
+        The node of the two that comes first in program order turns into the product (its
+        inputs precede it, every reader of either result follows it)."""
+        nodes = self._live_nodes()
+        users: dict[int, list[ir.Node]] = {}
+        for n in nodes:
+            for i in n.inputs:
+                if not any(u is n for u in users.get(i.id, ())):
+                    users.setdefault(i.id, []).append(n)
+        out_ids = {v.id for v in self.outputs}
+        for mm in nodes:
+            if mm.kind != "matmul" or len(mm.outputs) != 1 or (mm.attrs or {}).get("act"):
+                continue
+            h = mm.outputs[0]
+            us = users.get(h.id, [])
+            if h.id in out_ids or not us:
+                continue
+            act = [u for u in us if u.kind == "ew" and u.fn == "gelu"]
+            der = [u for u in us if u.kind == "ew" and u.fn == "dgelu"]
+            if len(act) != 1 or len(der) > 1 or len(us) != 1 + len(der):
+                continue
+            a_out = act[0].outputs[0]
+            outs = [a_out] + [d.outputs[0] for d in der]
+            if not self._epilogue_ok(mm, a_out) or any(
+                    o.dtype is not a_out.dtype or o.shape != a_out.shape for o in outs):
+                continue
+            host = min(act + der, key=lambda n: n.pos)
+            host.kind, host.fn = "matmul", None
+            host.inputs = list(mm.inputs)
+            host.attrs = dict(mm.attrs or {}, act="gelu")
+            host.outputs = outs
+            for k, v in enumerate(outs):
+                v.node, v.index = host, k
+
     def _epilogue_ok(self, mm: ir.Node, out: ir.Value) -> bool:
         """The product ``mm`` may write ``out`` through its epilogue."""
         m = mm.outputs[0]
@@ -1109,6 +1147,10 @@ class Planner:
         at = n.attrs or {}
         if "bias_in" in at:
             epi["bias"] = self._contig(n.inputs[at["bias_in"]])
+        if at.get("act"):
+            epi["act"] = at["act"]
+            if len(n.outputs) > 1:
+                epi["aux_value"] = n.outputs[1]  # the activation's derivative, a second result
         ra, rb = self._resolve(a), self._resolve(b)
         if isinstance(ra, Const):
             ra = self._materialize(ra)
@@ -1138,7 +1180,7 @@ class Planner:
             self.skip_nodes.add(red.pos)
             self._emit_plain_gemm(ra, rb, pa, pb, M, N, K * batch, red.outputs[0])
             return
-        c_strides = self._matmul_out_layout(out)
+        c_strides = self._matmul_out_layout(out) if "aux_value" not in epi else contiguous_strides(out.shape)
         gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
         # one (outer, inner) split of the batch index has to serve A, B and C
         split = None
@@ -1185,7 +1227,11 @@ class Planner:
             buf = self._new_buf(out.shape, out.dtype, "temp", -1)
             dst = ViewRef(buf.id, 0, out.shape, c_strides, out.dtype)
             self.loc[out.id] = dst
-        self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), [dst.buf], dict(
+        writes = [dst.buf]
+        if "aux_value" in epi:
+            epi["aux_dst"] = self._alloc_value(epi.pop("aux_value"))
+            writes.append(epi["aux_dst"].buf)
+        self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), writes, dict(
             epi, a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
@@ -1214,9 +1260,13 @@ class Planner:
         dst = self._alloc_value(out)
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
-        epi = epi or {}
+        epi = dict(epi or {})
         if ks == 1 or epi:  # (a product with a folded epilogue is never split)
-            self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), [dst.buf],
+            writes = [dst.buf]
+            if "aux_value" in epi:
+                epi["aux_dst"] = self._alloc_value(epi.pop("aux_value"))
+                writes.append(epi["aux_dst"].buf)
+            self._emit(Step("gemm", [ra.buf, rb.buf] + self._epi_bufs(epi), writes,
                             dict(common, **epi, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
             return
         kc = K // ks
@@ -1840,6 +1890,9 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     pre = Planner(builder, outputs)
     pre._rematerialize_masks()
     pre._fold_bias_into_matmul()
+    from .. import config
+    if config.FOLD_ACTIVATION:
+        pre._fold_activation_into_matmul()
     outputs = pre.outputs
     for limit in (28, 16, 8, 4, 1):
         try:

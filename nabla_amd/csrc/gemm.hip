@@ -53,12 +53,33 @@ struct GemmArgs {
   float alpha;
   int32_t tiles_m, tiles_n;
   int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
+  void* C2;              // second result (derivative of the activation), or null
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
   if (act == NBK_ACT_RELU) return fmaxf(v, 0.f);
   if (act == NBK_ACT_GELU) return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
   return v;
+}
+
+// Activation and its derivative at the same point (the second result of a launch).  LOWP: the
+// results are stored as 16-bit floats, so hardware exp and a 1.5e-7 erf do (the same forms the
+// row kernels use for such results).
+template <bool LOWP>
+__device__ __forceinline__ void gemm_act_pair(float x, int act, float& y, float& dy) {
+  if (act == NBK_ACT_RELU) {
+    y = fmaxf(x, 0.f);
+    dy = x > 0.f ? 1.f : 0.f;
+  } else if (act == NBK_ACT_GELU) {
+    const float z = x * 0.70710678118654752440f;
+    const float e = LOWP ? __expf(-z * z) : expf(-z * z);
+    const float cdf = 0.5f * (1.f + (LOWP ? nbk_fast_erf_with(z, e) : erff(z)));
+    y = x * cdf;
+    dy = cdf + x * 0.39894228040143267794f * e;
+  } else {
+    y = x;
+    dy = 1.f;
+  }
 }
 
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
@@ -303,10 +324,37 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
             for (int e = 0; e < 8; ++e)
               if (col + e < g.N) res[e] = nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
           }
+          if (g.C2) {
+            // two results: the activation goes to C below, its derivative to C2 here
+            float d2[8];
+            if (out_f32) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float x = gemm_act(v[e] + bias_v[e], g.act);
-            v[e] = !g.residual ? x : (g.res_mul ? x * res[e] : x + res[e]);
+              for (int e = 0; e < 8; ++e) gemm_act_pair<false>(v[e] + bias_v[e], g.act, v[e], d2[e]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) gemm_act_pair<true>(v[e] + bias_v[e], g.act, v[e], d2[e]);
+            }
+            if (vec_store && !out_f32) {
+              uint4 o;
+              o.x = (uint32_t)nbk_f32_to_bf16(d2[0]) | ((uint32_t)nbk_f32_to_bf16(d2[1]) << 16);
+              o.y = (uint32_t)nbk_f32_to_bf16(d2[2]) | ((uint32_t)nbk_f32_to_bf16(d2[3]) << 16);
+              o.z = (uint32_t)nbk_f32_to_bf16(d2[4]) | ((uint32_t)nbk_f32_to_bf16(d2[5]) << 16);
+              o.w = (uint32_t)nbk_f32_to_bf16(d2[6]) | ((uint32_t)nbk_f32_to_bf16(d2[7]) << 16);
+              *(uint4*)((uint16_t*)g.C2 + idx) = o;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (col + e < g.N) {
+                  if (out_f32) ((float*)g.C2)[idx + e] = d2[e];
+                  else ((uint16_t*)g.C2)[idx + e] = nbk_f32_to_bf16(d2[e]);
+                }
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float x = gemm_act(v[e] + bias_v[e], g.act);
+              v[e] = !g.residual ? x : (g.res_mul ? x * res[e] : x + res[e]);
+            }
           }
         }
         if (vec_store && !out_f32) {
@@ -1086,8 +1134,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
       for (int r = 0; r < 16; ++r) {
         const int64_t row = m0 + wm + i * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
         if (row >= g.M) continue;
-        float v = gemm_act(acc[i][j][r] * g.alpha + bv, g.act);
         const int64_t idx = c_off + row * g.ldc + col;
+        float v, dv;
+        if (g.C2) {
+          gemm_act_pair<false>(acc[i][j][r] * g.alpha + bv, g.act, v, dv);
+          ((float*)g.C2)[idx] = dv;
+        } else {
+          v = gemm_act(acc[i][j][r] * g.alpha + bv, g.act);
+        }
         if (g.residual) v = g.res_mul ? v * ((const float*)g.residual)[idx] : v + ((const float*)g.residual)[idx];
         C[idx] = v;
       }
@@ -1183,8 +1237,15 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const GemmArgs g) {
     const int64_t row = m0 + r, col = n0 + c;
     if (row >= g.M || col >= g.N) continue;
     float v = (part[0][r][c] + part[1][r][c]) + (part[2][r][c] + part[3][r][c]);
-    v = gemm_act(v * g.alpha + (g.bias ? ((const float*)g.bias)[col] : 0.f), g.act);
     const int64_t idx = c_off + row * g.ldc + col;
+    const float x = v * g.alpha + (g.bias ? ((const float*)g.bias)[col] : 0.f);
+    if (g.C2) {
+      float dv;
+      gemm_act_pair<false>(x, g.act, v, dv);
+      ((float*)g.C2)[idx] = dv;
+    } else {
+      v = gemm_act(x, g.act);
+    }
     if (g.residual) v = g.res_mul ? v * ((const float*)g.residual)[idx] : v + ((const float*)g.residual)[idx];
     C[idx] = v;
   }
@@ -1299,6 +1360,12 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.b_bs2 = a.batch_inner > 1 ? d->b_bs2 : 0;
   a.c_bs2 = a.batch_inner > 1 ? d->c_bs2 : 0;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
+  NBK_REQUIRE(d->aux_op == NBK_AUX_NONE || d->aux_op == NBK_AUX_ACT_GRAD, "gemm: aux_op %d", d->aux_op);
+  NBK_REQUIRE((d->aux_op == NBK_AUX_NONE) == (d->C_aux == nullptr),
+              "gemm: C_aux and aux_op go together");
+  NBK_REQUIRE(d->aux_op == NBK_AUX_NONE || (d->act != NBK_ACT_NONE && d->residual == nullptr),
+              "gemm: the derivative of the activation needs an activation and no residual");
+  a.C2 = d->C_aux;
   NBK_REQUIRE(d->residual_op == NBK_RES_ADD || d->residual_op == NBK_RES_MUL,
               "gemm: residual_op %d", d->residual_op);
   a.res_mul = d->residual_op == NBK_RES_MUL;

@@ -65,6 +65,19 @@ __device__ __forceinline__ uint16_t nbk_f32_to_bf16(float f) {
   const __bf16 b = (__bf16)f;
   return __builtin_bit_cast(uint16_t, b);
 }
+// Five-term erf (Abramowitz & Stegun 7.1.26, 1.5e-7 absolute) on hardware rcp; e = exp(-x^2) is
+// passed in so that a caller that needs it anyway computes it once.  For results that are
+// stored as 16-bit floats.
+__device__ __forceinline__ float nbk_fast_erf_with(float x, float e) {
+  const float ax = fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, ax, 1.0f));
+  float p = fmaf(1.061405429f, t, -1.453152027f);
+  p = fmaf(p, t, 1.421413741f);
+  p = fmaf(p, t, -0.284496736f);
+  p = fmaf(p, t, 0.254829592f);
+  const float r = fmaf(-p * t, e, 1.0f);
+  return copysignf(r, x);
+}
 __device__ __forceinline__ float nbk_load_as_f32(const void* p, int64_t i, int dt) {
   switch (dt) {
     case NBK_F32: return ((const float*)p)[i];

@@ -169,16 +169,7 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
 // they take a fifth of the instructions of the correctly rounded library routines,
 // which is what bounds these kernels once their traffic is halved by the 16-bit I/O.
 // e = exp(-x^2), passed in so that a caller that needs it anyway computes it once
-__device__ __forceinline__ float rp_fast_erf_with(float x, float e) {
-  const float ax = fabsf(x);
-  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, ax, 1.0f));
-  float p = fmaf(1.061405429f, t, -1.453152027f);
-  p = fmaf(p, t, 1.421413741f);
-  p = fmaf(p, t, -0.284496736f);
-  p = fmaf(p, t, 0.254829592f);
-  const float r = fmaf(-p * t, e, 1.0f);
-  return copysignf(r, x);
-}
+__device__ __forceinline__ float rp_fast_erf_with(float x, float e) { return nbk_fast_erf_with(x, e); }
 __device__ __forceinline__ float rp_fast_erf(float x) { return rp_fast_erf_with(x, __expf(-x * x)); }
 __device__ __forceinline__ float rp_unary_lowp(int op, float a) {
   switch (op) {

@@ -200,6 +200,17 @@ def _gemm(a, mem):
     C = torch.matmul(A.double(), B.double()).float() * a.get("alpha", 1.0)
     if a.get("bias") is not None:  # added before the result is rounded, as in the kernel's epilogue
         C = C + _view(mem, a["bias"]).reshape(-1).float()
+    if a.get("act") is not None:
+        x = C.double()
+        if a["act"] == "gelu":
+            cdf = 0.5 * (1.0 + torch.erf(x / 2.0 ** 0.5))
+            act, dact = x * cdf, cdf + x * torch.exp(-0.5 * x * x) / (2.0 * torch.pi) ** 0.5
+        else:
+            act, dact = torch.relu(x), (x > 0).double()
+        if a.get("aux_dst") is not None:
+            aux = mat(a["aux_dst"], a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"])
+            aux.copy_(dact.to(aux.dtype))
+        C = act.float()
     if a.get("residual") is not None:
         res = a["residual"]
         R = mat(res, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"]).float()

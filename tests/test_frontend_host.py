@@ -579,3 +579,48 @@ def test_scatter_value_rules_and_embedding_table_gradient(emulator):
     np.testing.assert_allclose(gt.numpy(), wt, rtol=1e-6)
     with pytest.raises(Exception, match="updates of shape"):
         nb.scatter(T(x), I, T(upd[:2])).realize()
+
+
+def test_gelu_of_a_linear_layer_is_folded_into_the_product(emulator):
+    """gelu(x @ W + b) in a training step: the activation and its derivative are two results of
+    the product's own launch (no row program reads the pre-activation), and loss and gradients
+    still agree with the float64 oracle."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    from oracle import ops as O
+    tok = config.set_flag("FOLD_ACTIVATION", True)
+    try:
+        _check_gelu_fold(engine, O)
+    finally:
+        config.reset_flag("FOLD_ACTIVATION", tok)
+        engine.clear_plan_cache()
+
+
+def _check_gelu_fold(engine, O):
+    rng = np.random.default_rng(77)
+    x, w, b = rng.standard_normal((6, 40)), rng.standard_normal((40, 24)) * 0.3, rng.standard_normal((1, 24))
+    w2 = rng.standard_normal((24, 5))
+    T = lambda a: nb.Tensor.constant(a.astype(np.float32))
+
+    def loss_fn(w, b, w2):
+        return nb.mean(nb.gelu(T(x) @ w + b) @ w2)
+
+    engine.clear_plan_cache()
+    loss, grads = nb.value_and_grad(loss_fn, argnums=(0, 1, 2))(T(w), T(b), T(w2))
+    nb.realize_all(loss, *grads)
+    plan = list(engine._PLAN_CACHE.values())[-1].plan
+    fused = [st for st in plan.steps if st.kind == "gemm" and st.attrs.get("act") == "gelu"]
+    assert len(fused) == 1 and fused[0].attrs.get("aux_dst") is not None and fused[0].attrs.get("bias") is not None
+    assert not any("gelu" in m for st in plan.steps if st.kind == "rowprog" for m in st.attrs["members"])
+    vw, vb, vw2 = O.V(w), O.V(b), O.V(w2)
+    want = O.mean(O.matmul(O.gelu(O.matmul(O.V(x), vw) + vb), vw2))
+    wg = O.grad_of(want, [vw, vb, vw2])
+    assert abs(loss.item() - float(want.a)) <= 1e-5 * abs(float(want.a))
+    for g, w_ in zip(grads, wg):
+        assert np.abs(g.numpy() - w_).max() <= 1e-5 * np.abs(w_).max()
+    # forward only: the activation alone, one result
+    engine.clear_plan_cache()
+    y = nb.gelu(T(x) @ T(w) + T(b))
+    np.testing.assert_allclose(y.numpy(), O.gelu(O.matmul(O.V(x), O.V(w)) + O.V(b)).a, rtol=1e-5, atol=1e-6)
+    plan = list(engine._PLAN_CACHE.values())[-1].plan
+    assert [st.kind for st in plan.steps] == ["gemm"] and plan.steps[0].attrs.get("aux_dst") is None

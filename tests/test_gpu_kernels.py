@@ -232,6 +232,46 @@ def test_gemm_low_rank_product(hip, b_layout, out, shape):
         assert err.max() <= atol, (with_res, err.max())
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(512, 512, 256), (300, 136, 72), (64, 40, 24), (1024, 256, 512)])
+def test_gemm_activation_and_its_derivative_as_two_results(hip, dtype, shape):
+    """C = gelu(A @ B + bias) and C_aux = gelu'(A @ B + bias) from one launch, against float64
+    torch (exact erf form, nabla/ops/unary.py:567-595); every tile size and both dtypes."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(14)
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    A = torch.tensor(rng.standard_normal((M, K)) * 0.2, dtype=tdt)
+    B = torch.tensor(rng.standard_normal((K, N)) * 0.2, dtype=tdt)
+    bias = torch.tensor(rng.standard_normal((N,)), dtype=tdt)
+    x = (A.double() @ B.double() + bias.double()).requires_grad_(True)
+    y = torch.nn.functional.gelu(x)
+    (dy,) = torch.autograd.grad(y.sum(), x)
+    a_dev, b_dev, bias_dev = A.cuda(), B.cuda(), bias.cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    c2_dev = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    L = lib.load()
+    d = lib.GemmDesc()
+    d.A, d.B, d.C, d.bias = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr(), bias_dev.data_ptr()
+    d.C_aux, d.aux_op, d.act = c2_dev.data_ptr(), 1, 2
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs, d.b_rs, d.b_cs, d.ldc = K, 1, N, 1, N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
+    d.dtype_ab = d.dtype_c = 1 if dtype == "bf16" else 0
+    d.alpha = 1.0
+    print(f"gemm gelu + derivative {shape} {dtype}", flush=True)
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    rtol, atol = (2.0 ** -8, 2e-3) if dtype == "bf16" else (1e-5, 1e-5)
+    for got, want in ((c_dev, y.detach()), (c2_dev, dy)):
+        err = (got.double().cpu() - want).abs() - rtol * want.abs()
+        assert err.max().item() <= atol, err.max().item()
+    # the derivative without an activation, or together with a residual, is refused
+    d.act = 0
+    with pytest.raises(ValueError, match="derivative"):
+        lib.check(L.nbk_gemm(C.byref(d), None))
+
+
 def test_mlp_grads(hip):
     import nabla_amd as nb
     rng = np.random.default_rng(0)
