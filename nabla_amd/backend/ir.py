@@ -204,6 +204,16 @@ def cast(x: Value, dtype: DType) -> Value:
     return ew("mov", x, dtype=dtype)
 
 
+def pin_after(x: Value, dep: Value) -> Value:
+    """``x`` unchanged, but to the planner an elementwise function of ``x`` and ``dep``: whatever is
+    computed from the result cannot be scheduled before ``dep`` exists.  A backward op uses it on
+    a forward value it re-reads, with its cotangent as ``dep``: without it the planner, which
+    fuses a node into the group of its producers, would pull the cotangent-independent part of
+    the backward arithmetic into the forward kernel and store full-size intermediates there."""
+    d = dep if dep.shape == x.shape else broadcast_to(dep, x.shape)
+    return current().add("ew", [x, d], [(x.shape, x.dtype)], fn="mov", operands=(x,))[0]
+
+
 def tril(x: Value, k: int = 0, upper: bool = False) -> Value:
     """Zero everything above (below, if ``upper``) the k-th diagonal of the last two axes."""
     if x.rank < 2:
@@ -286,8 +296,12 @@ def fill(shape, dtype: DType, value: float) -> Value:
     return current().add("fill", [], [(tuple(shape), dtype)], value=float(value))[0]
 
 
-def iota(n: int, dtype: DType, start: float = 0.0, step: float = 1.0) -> Value:
-    return current().add("iota", [], [((int(n),), dtype)], start=float(start), step=float(step))[0]
+def iota(n: int, dtype: DType, start: float = 0.0, step: float = 1.0, lead=()) -> Value:
+    """``start + step * j`` along an axis of ``n`` entries; with ``lead`` the same row repeated
+    over leading dims ``lead`` (shape ``lead + (n,)``), which lets it sit inside the kernel of
+    whatever reads it instead of being a tensor of its own."""
+    shape = tuple(int(d) for d in lead) + (int(n),)
+    return current().add("iota", [], [(shape, dtype)], start=float(start), step=float(step))[0]
 
 
 # ---- contractions ---------------------------------------------------------------------

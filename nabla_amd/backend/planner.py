@@ -559,7 +559,9 @@ class Planner:
             c = Const(n.attrs["value"], v.shape, v.dtype)
             self.loc[v.id] = c
             return c
-        if n.kind in VIEW_KINDS and n.pos not in self.alias_nodes:
+        if n.kind in VIEW_KINDS:
+            # (also a broadcast that lives inside a group as an alias of a row value: whoever
+            # asks for its location reads it from outside the group, as a view of the stored row)
             base = self._resolve(n.inputs[0])
             if isinstance(base, Const):
                 r = Const(base.value, v.shape, v.dtype)
@@ -637,7 +639,7 @@ class Planner:
                     if _numel(i.shape) * 64 <= big:
                         continue  # a small leaf: read again by the copy
                     pn = i.node
-                    if pn.kind in ("broadcast", "reshape") or (pn.kind == "ew" and pn.fn in self._REMAT_FNS):
+                    if pn.kind in ("broadcast", "reshape", "iota") or (pn.kind == "ew" and pn.fn in self._REMAT_FNS):
                         stack.append(pn)
                     else:
                         ok = False
@@ -780,16 +782,25 @@ class Planner:
 
         # consumers outside the producing unit decide what must be stored
         self.need_store: set[int] = set()
+
+        def stored_source(v: ir.Value) -> ir.Value:
+            # a row value broadcast over its row inside a group (an alias node) and read from
+            # outside that group is not worth a full-size store: the row value is stored and
+            # the outside reader sees the broadcast as a view of it
+            while v.node.pos in self.alias_nodes:
+                v = v.node.inputs[0]
+            return v
+
         for n in nodes:
             cu = self._unit(n.pos)
             for i in n.inputs:
                 if n.kind in VIEW_KINDS and n.pos not in self.alias_nodes:
                     # a view forces its source into memory unless that is a view too
-                    self.need_store.add(i.id)
+                    self.need_store.add(stored_source(i).id)
                     continue
                 pu = self._unit(i.node.pos)
                 if pu is None or pu is not cu or not cu.fused:
-                    self.need_store.add(i.id)
+                    self.need_store.add(stored_source(i).id)
         # plan outputs: the first output that names a unit-produced value owns
         # that value's allocation; everything else is copied at the end
         self._out_pending: dict[int, int] = {}
