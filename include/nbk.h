@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 14
+#define NBK_ABI_VERSION 15
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -254,6 +254,26 @@ typedef struct nbk_gemm_desc {
   int32_t reserved;
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
+
+/* C = alpha * A @ W or alpha * A @ W^T for a weight W [w_rows, w_cols] that is stored NF4-coded
+ * as quantize_nf4 leaves it (nabla/nn/finetune/qlora.py:41-75): `codes`, one uint8 per weight in
+ * row-major order holding the index of one of the sixteen levels (18-38), and `scales`, one fp32
+ * per `block` consecutive codes.  Replaces dequantize_nf4 followed by matmul (77-113) and the
+ * input-gradient product of that matmul: the dense weight is never built, the kernel reads
+ * the codes, looks the levels up, applies the block scale and feeds the matrix cores (bf16: the
+ * product level * scale is rounded to bf16 once).  A is row-major [M, K] with leading dimension
+ * lda, C row-major [M, N]; dtype (NBK_BF16 or NBK_F32) is the type of A and C.  w_cols and block
+ * must be multiples of 8, codes 8-byte aligned. */
+typedef struct nbk_gemm_nf4_desc {
+  const void* A; const void* codes; const void* scales; void* C;
+  int64_t M, w_rows, w_cols;
+  int64_t lda, ldc;
+  int32_t block;
+  int32_t transpose_w;   /* 0: C = A @ W (K = w_rows), 1: C = A @ W^T (K = w_cols) */
+  int32_t dtype;
+  float alpha;
+} nbk_gemm_nf4_desc;
+int nbk_gemm_nf4(const nbk_gemm_nf4_desc* d, void* stream);
 
 /* ===================================================================== */
 /*  Convolution / pooling (NHWC x HWIO)                                   */

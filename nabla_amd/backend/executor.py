@@ -174,6 +174,25 @@ class BoundPlan:
                 d.batch_reduce = 0
                 d.alpha = a.get("alpha", 1.0)
                 self.calls.append((L.nbk_gemm, [C.byref(d)], patches, d))
+            elif k == "gemm_nf4":
+                d = lib.GemmNf4Desc()
+                rx, rcodes, rsc, rc = a["x"], a["codes"], a["scales"], a["dst"]
+                if rcodes.dtype is not DType.uint8 or rsc.dtype is not DType.float32:
+                    raise TypeError(f"matmul_nf4 wants uint8 codes and float32 scales, got {rcodes.dtype}, {rsc.dtype}")
+                if rx.dtype is not rc.dtype or rx.dtype not in (DType.bfloat16, DType.float32):
+                    raise TypeError(f"matmul_nf4 computes in bfloat16 or float32, got {rx.dtype} -> {rc.dtype}")
+                ptr_field(d, "A", rx.buf, rx.offset * rx.dtype.size_in_bytes)
+                ptr_field(d, "codes", rcodes.buf, rcodes.offset)
+                ptr_field(d, "scales", rsc.buf, rsc.offset * 4)
+                ptr_field(d, "C", rc.buf, rc.offset * rc.dtype.size_in_bytes)
+                d.M = a["M"]
+                d.w_rows, d.w_cols = a["w_shape"]
+                d.lda, d.ldc = a["K"], a["N"]
+                d.block = a["block"]
+                d.transpose_w = 1 if a["transpose"] else 0
+                d.dtype = rx.dtype.abi
+                d.alpha = 1.0
+                self.calls.append((L.nbk_gemm_nf4, [C.byref(d)], patches, d))
             elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
                 d = lib.ConvDesc()
                 xs, ws, ys = a["x_shape"], a["w_shape"], a["y_shape"]

@@ -317,6 +317,20 @@ def matmul(a: Value, b: Value) -> Value:
     return current().add("matmul", [a, b], [(shape, promote(a.dtype, b.dtype))])[0]
 
 
+def matmul_nf4(x: Value, codes: Value, scales: Value, w_shape, block: int, transpose: bool) -> Value:
+    """``x @ W`` (or ``x @ W^T``) for a weight of shape ``w_shape`` stored as NF4 codes (uint8, one per
+    weight, row-major) and one fp32 scale per ``block`` consecutive codes."""
+    rows, cols = (int(d) for d in w_shape)
+    k, n = (cols, rows) if transpose else (rows, cols)
+    if x.rank < 1 or x.shape[-1] != k:
+        raise ValueError(f"matmul_nf4: contraction mismatch {x.shape} against a weight {tuple(w_shape)}"
+                         f"{' transposed' if transpose else ''}")
+    if codes.numel() != rows * cols or scales.numel() * int(block) != rows * cols:
+        raise ValueError("matmul_nf4: codes / scales do not match the weight's shape and block length")
+    return current().add("matmul_nf4", [x, codes, scales], [(x.shape[:-1] + (n,), x.dtype)],
+                         w_shape=(rows, cols), block=int(block), transpose=bool(transpose))[0]
+
+
 def conv_out_size(n: int, k: int, stride: int, pad_lo: int, pad_hi: int) -> int:
     return (n + pad_lo + pad_hi - k) // stride + 1
 

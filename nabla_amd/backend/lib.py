@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 MAX_RANK = 8
 
@@ -68,6 +68,15 @@ class GemmDesc(C.Structure):
         ("act", C.c_int32), ("batch_reduce", C.c_int32),
         ("alpha", C.c_float), ("residual_op", C.c_int32),
         ("C_aux", C.c_void_p), ("aux_op", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class GemmNf4Desc(C.Structure):
+    _fields_ = [
+        ("A", C.c_void_p), ("codes", C.c_void_p), ("scales", C.c_void_p), ("C", C.c_void_p),
+        ("M", C.c_int64), ("w_rows", C.c_int64), ("w_cols", C.c_int64),
+        ("lda", C.c_int64), ("ldc", C.c_int64),
+        ("block", C.c_int32), ("transpose_w", C.c_int32), ("dtype", C.c_int32), ("alpha", C.c_float),
     ]
 
 
@@ -139,6 +148,7 @@ _SIGNATURES = {
                           C.c_void_p], C.c_int),
     "nbk_fill": ([C.c_void_p, C.c_int32, C.c_int64, C.c_double, C.c_void_p], C.c_int),
     "nbk_gemm": ([C.POINTER(GemmDesc), C.c_void_p], C.c_int),
+    "nbk_gemm_nf4": ([C.POINTER(GemmNf4Desc), C.c_void_p], C.c_int),
     "nbk_conv2d_fwd": ([C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                         C.c_void_p], C.c_int),
     "nbk_conv2d_dgrad": ([C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p],

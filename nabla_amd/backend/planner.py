@@ -940,6 +940,14 @@ class Planner:
                     attrs["workspace_bytes"] = nbytes
                     writes.append(wbuf.id)
             self._emit(Step(k, [i.buf for i in ins], writes, attrs))
+        elif k == "matmul_nf4":
+            x, codes, scales = (self._contig(i) for i in n.inputs)
+            dst = self._alloc_value(out)
+            kdim = n.inputs[0].shape[-1]
+            self._emit(Step("gemm_nf4", [x.buf, codes.buf, scales.buf], [dst.buf], dict(
+                x=x, codes=codes, scales=scales, dst=dst, M=_numel(n.inputs[0].shape[:-1]), K=kdim,
+                N=out.shape[-1], w_shape=n.attrs["w_shape"], block=n.attrs["block"],
+                transpose=n.attrs["transpose"])))
         elif k in ("attention", "attention_bwd"):
             self._lower_attention(n)
         elif k in ("maxpool2d", "maxpool2d_bwd", "avgpool2d", "avgpool2d_bwd"):

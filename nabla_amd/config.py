@@ -39,6 +39,11 @@ _LORA_LOW_RANK_ORDER: ContextVar[bool] = ContextVar("LORA_LOW_RANK_ORDER",
 _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
                                                 default=_env_flag("NBK_FOLD_ACTIVATION", False))
 
+# x @ W for an NF4-coded W as one product that reads the codes (one byte per weight) and
+# dequantises them on the way into LDS; off: dequantise into a dense weight first
+_FUSED_NF4_MATMUL: ContextVar[bool] = ContextVar("FUSED_NF4_MATMUL",
+                                                 default=_env_flag("NBK_FUSED_NF4_MATMUL", True))
+
 _FLAGS = {
     "EAGER_MAX_GRAPH": _EAGER_MAX_GRAPH,
     "VERIFY_EAGER_SHAPES": _VERIFY_EAGER_SHAPES,
@@ -46,6 +51,7 @@ _FLAGS = {
     "FUSED_ATTENTION": _FUSED_ATTENTION,
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
+    "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
 }
 
 

@@ -54,6 +54,8 @@ struct GemmArgs {
   int32_t tiles_m, tiles_n;
   int32_t a_vec, b_vec;  // 16-byte accesses are legal for this operand
   void* C2;              // second result (derivative of the activation), or null
+  const float* b_scales; // NF4-coded B only: one scale per `b_block` consecutive codes
+  int32_t b_block;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -124,6 +126,32 @@ __device__ __forceinline__ u32x4 ld8_bf16(const uint16_t* p, int64_t valid, bool
   return r;
 }
 
+// ---- NF4-coded B operand --------------------------------------------------------------------
+// The sixteen levels (nabla/nn/finetune/qlora.py:18-38), copied to LDS by the kernels that
+// dequantise: a lane looks up eight different entries per load.
+__device__ const float nbk_nf4_levels[16] = {-1.0f,    -0.6962f, -0.5251f, -0.3949f, -0.2844f, -0.1848f,
+                                             -0.0911f, 0.0f,     0.0796f,  0.1609f,  0.2461f,  0.3379f,
+                                             0.4407f,  0.5626f,  0.7230f,  1.0f};
+// Eight consecutive weights from their codes: level[code] * scale of the block the codes lie
+// in (`flat` is the index of the first code in the flattened weight, a multiple of 8, and the
+// block length is a multiple of 8, so the eight share a block); entries from `valid` on are 0.
+__device__ __forceinline__ void nf4_load8(const uint8_t* codes, const float* scales, int block,
+                                          const float* table, int64_t flat, int64_t valid, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = 0.f;
+  if (valid <= 0) return;
+  const float s = scales[flat / block];
+  uint64_t raw = 0;
+  if (valid >= 8) {
+    raw = *(const uint64_t*)(codes + flat);
+  } else {
+    for (int e = 0; e < valid; ++e) raw |= (uint64_t)codes[flat + e] << (8 * e);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (e < valid) out[e] = table[(raw >> (8 * e)) & 15] * s;
+}
+
 // ------------------------------------------------------- bf16, guarded register-staged loads
 // The general form: any alignment, any K, ragged edges.  Every access is guarded element by
 // element; it is kept out of the hot kernel because its code size alone would push the main
@@ -171,6 +199,34 @@ struct TileLoader {
         if (gk < K) reg[s] = ld8_bf16(base + gk * cs + gr, rows_total - gr, vec);
         else reg[s] = (u32x4){0u, 0u, 0u, 0u};
       }
+    }
+  }
+
+  // The same tile from NF4 codes: `codes` addressed like `base` above, dequantised in registers
+  // and rounded to bf16 once.
+  __device__ __forceinline__ void load_nf4(const uint8_t* codes, const float* scales, int block,
+                                           const float* table, int64_t rs, int64_t cs, int64_t row0,
+                                           int64_t rows_total, int64_t k0, int64_t K) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int s = 0; s < NREG; ++s) {
+      const int t = tid + s * NT;
+      float w[8];
+      if (KC) {
+        const int row = t >> 3, c = t & 7;
+        const int64_t gr = row0 + row, gk = k0 + c * 8;
+        nf4_load8(codes, scales, block, table, gr * rs + gk, gr < rows_total ? K - gk : 0, w);
+      } else {
+        const int k = t / NC, c = t % NC;
+        const int64_t gr = row0 + c * 8, gk = k0 + k;
+        nf4_load8(codes, scales, block, table, gk * cs + gr, gk < K ? rows_total - gr : 0, w);
+      }
+      u32x4 r;
+      r.x = (uint32_t)nbk_f32_to_bf16(w[0]) | ((uint32_t)nbk_f32_to_bf16(w[1]) << 16);
+      r.y = (uint32_t)nbk_f32_to_bf16(w[2]) | ((uint32_t)nbk_f32_to_bf16(w[3]) << 16);
+      r.z = (uint32_t)nbk_f32_to_bf16(w[4]) | ((uint32_t)nbk_f32_to_bf16(w[5]) << 16);
+      r.w = (uint32_t)nbk_f32_to_bf16(w[6]) | ((uint32_t)nbk_f32_to_bf16(w[7]) << 16);
+      reg[s] = r;
     }
   }
 
@@ -391,9 +447,16 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
 
 // NW waves: 4 as 2 x 2, or 8 as 2 x 4 (two waves per SIMD, each with half the accumulators:
 // they cover each other's waits at the price of 1.5 x the LDS fragment traffic).
-template <int BM, int BN, bool A_KC, bool B_KC, bool EPI, int NW>
+template <int BM, int BN, bool A_KC, bool B_KC, bool EPI, int NW, bool B_Q = false>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
   constexpr int NT = NW * 64, WGN = NW / 2;
+  // B_Q: B holds NF4 codes (one byte per weight, addressed like a dense B) and g.b_scales the
+  // block scales; the tile loader dequantises on the way into LDS
+  __shared__ float nf4_table[B_Q ? 16 : 1];
+  if (B_Q) {
+    if (threadIdx.x < 16) nf4_table[threadIdx.x] = nbk_nf4_levels[threadIdx.x];
+    __syncthreads();
+  }
   constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int CA = TileGeom<BM, A_KC>::CHUNKS, CB = TileGeom<BN, B_KC>::CHUNKS;
@@ -422,7 +485,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
   // A is rows = m; for the loader a K-contiguous operand has (rs = row stride, k unit),
   // a row-contiguous one has (cs = k stride, row unit).
   la.load(A, g.a_rs, g.a_cs, m0, g.M, 0, g.K, g.a_vec);
-  lb.load(B, g.b_cs, g.b_rs, n0, g.N, 0, g.K, g.b_vec);
+  if constexpr (B_Q) lb.load_nf4((const uint8_t*)g.B, g.b_scales, g.b_block, nf4_table, g.b_cs, g.b_rs, n0, g.N, 0, g.K);
+  else lb.load(B, g.b_cs, g.b_rs, n0, g.N, 0, g.K, g.b_vec);
   la.store(gemm_lds);
   lb.store(gemm_lds + CA);
   __syncthreads();
@@ -519,7 +583,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
   {
     const int64_t k1 = nk > 1 ? 64 : 0;  // a single-tile problem re-reads tile 0 (never stored)
     la.load(A, g.a_rs, g.a_cs, m0, g.M, k1, g.K, g.a_vec);
-    lb.load(B, g.b_cs, g.b_rs, n0, g.N, k1, g.K, g.b_vec);
+    if constexpr (B_Q) lb.load_nf4((const uint8_t*)g.B, g.b_scales, g.b_block, nf4_table, g.b_cs, g.b_rs, n0, g.N, k1, g.K);
+    else lb.load(B, g.b_cs, g.b_rs, n0, g.N, k1, g.K, g.b_vec);
   }
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
@@ -558,7 +623,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_kernel(const GemmArgs g) {
     {
       const int64_t k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * 64;
       la.load(A, g.a_rs, g.a_cs, m0, g.M, k2, g.K, g.a_vec);
-      lb.load(B, g.b_cs, g.b_rs, n0, g.N, k2, g.K, g.b_vec);
+      if constexpr (B_Q) lb.load_nf4((const uint8_t*)g.B, g.b_scales, g.b_block, nf4_table, g.b_cs, g.b_rs, n0, g.N, k2, g.K);
+      else lb.load(B, g.b_cs, g.b_rs, n0, g.N, k2, g.K, g.b_vec);
     }
     static_for<NMFMA / 2>([&](auto q) { mfma(S1{}, q); });
     {
@@ -1031,11 +1097,16 @@ __global__ __launch_bounds__(SKN_WAVES * 64) void gemm_skinny_n_kernel(const Gem
 
 // ---------------------------------------------------------------------------- fp32
 // 128 x 128 x 16 tile, LDS k-major ([k][rows], rows padded by 4 floats).
-template <bool A_KC, bool B_KC>
+template <bool A_KC, bool B_KC, bool B_Q = false>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
   constexpr int BM = 128, BN = 128, BK = 16, LD = 128 + 4;
   __shared__ float As[2][BK][LD];
   __shared__ float Bs[2][BK][LD];
+  __shared__ float nf4_table[B_Q ? 16 : 1];  // B_Q: B holds NF4 codes, g.b_scales the block scales
+  if (B_Q) {
+    if (threadIdx.x < 16) nf4_table[threadIdx.x] = nbk_nf4_levels[threadIdx.x];
+    __syncthreads();
+  }
   int tm_i, tn_i;
   gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
   const int64_t m0 = (int64_t)tm_i * BM, n0 = (int64_t)tn_i * BN;
@@ -1077,6 +1148,24 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
       }
     }
   };
+  // B from NF4 codes: the same eight elements per lane, dequantised
+  auto load_b = [&](int64_t k0, float* r) {
+    if constexpr (B_Q) {
+      if (B_KC) {
+        const int row = tid >> 1, kk = (tid & 1) * 8;
+        const int64_t gr = n0 + row, gk = k0 + kk;
+        nf4_load8((const uint8_t*)g.B, g.b_scales, g.b_block, nf4_table, gr * g.b_cs + gk,
+                  gr < g.N ? g.K - gk : 0, r);
+      } else {
+        const int kk = tid >> 4, rr = (tid & 15) * 8;
+        const int64_t gk = k0 + kk, gr = n0 + rr;
+        nf4_load8((const uint8_t*)g.B, g.b_scales, g.b_block, nf4_table, gk * g.b_rs + gr,
+                  gk < g.K ? g.N - gr : 0, r);
+      }
+    } else {
+      load_tile(B, g.b_cs, g.b_rs, n0, g.N, k0, B_KC, g.b_vec, r);
+    }
+  };
   auto store_tile = [&](float (*S)[LD], bool kc, const float* r) {
     if (kc) {
       const int row = tid >> 1, kk = (tid & 1) * 8;
@@ -1091,7 +1180,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
 
   const int64_t nk = (g.K + BK - 1) / BK;
   load_tile(A, g.a_rs, g.a_cs, m0, g.M, 0, A_KC, g.a_vec, ra);
-  load_tile(B, g.b_cs, g.b_rs, n0, g.N, 0, B_KC, g.b_vec, rb);
+  load_b(0, rb);
   store_tile(As[0], A_KC, ra);
   store_tile(Bs[0], B_KC, rb);
   __syncthreads();
@@ -1100,7 +1189,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     const bool more = kt + 1 < nk;
     if (more) {
       load_tile(A, g.a_rs, g.a_cs, m0, g.M, (kt + 1) * BK, A_KC, g.a_vec, ra);
-      load_tile(B, g.b_cs, g.b_rs, n0, g.N, (kt + 1) * BK, B_KC, g.b_vec, rb);
+      load_b((kt + 1) * BK, rb);
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 2; ++ks) {
@@ -1464,4 +1553,62 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   else if (bkc) hipLaunchKernelGGL((gemm_f32_kernel<false, true>), grid, dim3(256), 0, st, a);
   else hipLaunchKernelGGL((gemm_f32_kernel<false, false>), grid, dim3(256), 0, st, a);
   return nbk_check_launch("gemm_f32_kernel");
+}
+
+// ------------------------------------------------------------------ NF4-coded weights
+extern "C" int nbk_gemm_nf4(const nbk_gemm_nf4_desc* d, void* stream) {
+  NBK_REQUIRE(d != nullptr, "gemm_nf4: null descriptor");
+  NBK_REQUIRE(d->A && d->codes && d->scales && d->C, "gemm_nf4: null pointer");
+  NBK_REQUIRE(d->M > 0 && d->w_rows > 0 && d->w_cols > 0, "gemm_nf4: empty problem");
+  NBK_REQUIRE(d->dtype == NBK_BF16 || d->dtype == NBK_F32, "gemm_nf4: dtype %d", d->dtype);
+  NBK_REQUIRE(d->block > 0 && d->block % 8 == 0 && d->w_cols % 8 == 0,
+              "gemm_nf4: the block length (%d) and the weight's width (%lld) must be multiples of 8",
+              d->block, (long long)d->w_cols);
+  NBK_REQUIRE(((uintptr_t)d->codes & 7) == 0, "gemm_nf4: codes must be 8-byte aligned");
+  // C = A @ W (K = rows of W, N = its columns) or A @ W^T (K = columns of W, N = its rows)
+  const int64_t K = d->transpose_w ? d->w_cols : d->w_rows;
+  const int64_t N = d->transpose_w ? d->w_rows : d->w_cols;
+  NBK_REQUIRE(d->lda >= K && d->ldc >= N, "gemm_nf4: leading dimension too small");
+  GemmArgs a = {};
+  a.A = d->A; a.B = d->codes; a.C = d->C;
+  a.M = d->M; a.N = N; a.K = K;
+  a.a_rs = d->lda; a.a_cs = 1;
+  // the element (k, n) of the B operand is code k * b_rs + n * b_cs of the flattened weight
+  a.b_rs = d->transpose_w ? 1 : d->w_cols;
+  a.b_cs = d->transpose_w ? d->w_cols : 1;
+  a.ldc = d->ldc; a.batch_inner = 1;
+  a.dtype_c = d->dtype; a.act = NBK_ACT_NONE; a.alpha = d->alpha;
+  a.b_scales = (const float*)d->scales; a.b_block = d->block;
+  a.a_vec = ((uintptr_t)d->A % 16 == 0) && (d->lda % (d->dtype == NBK_F32 ? 4 : 8) == 0);
+  a.b_vec = 0;
+  a.tiles_m = (int)((a.M + 127) / 128);
+  a.tiles_n = (int)((a.N + 127) / 128);
+  NBK_REQUIRE((int64_t)a.tiles_m * a.tiles_n <= 0x7fffffffLL, "gemm_nf4: launch too large");
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), 1);
+  hipStream_t st = (hipStream_t)stream;
+  const bool bkc = d->transpose_w != 0;
+  if (d->dtype == NBK_F32) {
+    if (bkc) hipLaunchKernelGGL((gemm_f32_kernel<true, true, true>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_f32_kernel<true, false, true>), grid, dim3(256), 0, st, a);
+    return nbk_check_launch("gemm_f32_kernel (nf4)");
+  }
+  const size_t pipe = 2 * (size_t)(TileGeom<128, true>::CHUNKS +
+                                   (bkc ? TileGeom<128, true>::CHUNKS : TileGeom<128, false>::CHUNKS)) * 16;
+  const size_t slabs = 4 * 32 * (size_t)(64 + 4) * sizeof(float);
+  const size_t lds = pipe > slabs ? pipe : slabs;
+#define NBK_LAUNCH_NF4(BK_)                                                                   \
+  do {                                                                                        \
+    auto kern = gemm_bf16_kernel<128, 128, true, BK_, false, 4, true>;                        \
+    static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
+    if (!attr_set) {                                                                          \
+      NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                  (int)lds));                                                 \
+      attr_set = true;                                                                        \
+    }                                                                                         \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);                                    \
+  } while (0)
+  if (bkc) NBK_LAUNCH_NF4(true);
+  else NBK_LAUNCH_NF4(false);
+#undef NBK_LAUNCH_NF4
+  return nbk_check_launch("gemm_bf16_kernel (nf4)");
 }

@@ -1,46 +1,58 @@
-"""LoRA helpers (nabla/nn/finetune/lora.py): init_lora_adapter 16-52,
-lora_delta 55-69 = ``(A @ B) * (alpha / rank)``, lora_linear 72-79, merge / unmerge.
+"""LoRA adapters (nabla/nn/finetune/lora.py:16-127): an adapter is the plain dict
+``{"A": (in, rank), "B": (rank, out)}`` and stands for the update ``(alpha / rank) * A @ B`` of a
+frozen ``(in, out)`` weight.
 
-The reference writes ``lora_linear`` as ``x @ W + x @ delta``: a full ``[D, D]`` delta and
-a second full GEMM forward, and two more full GEMMs in the backward pass (``x^T dy`` and
-``dy delta^T``).  With ``config.LORA_LOW_RANK_ORDER`` (the default) the same function is
-evaluated as ``x @ W + ((x @ A) @ B) * (alpha / rank)``: every adapter product is rank-sized
-in both directions.  The two orders differ by rounding only; switch the flag off for the
-order as written."""
+``lora_linear`` is where this backend departs from the reference's arithmetic order.  The
+reference forms the full ``(in, out)`` update and multiplies the activations with it, a second
+full-size product forward and two more backward (``x^T dy`` and ``dy delta^T``).  With
+``config.LORA_LOW_RANK_ORDER`` (the default) the activations go through the two thin factors
+instead, ``((x @ A) @ B) * (alpha / rank)``: every adapter product is rank-sized in both
+directions, and the result differs from the reference's by rounding only.  Switch the flag off
+for the order as written there.
+"""
 from __future__ import annotations
 
 from ... import config
 from ...core.dtype import DType
+from ...core.pytree import tree_map
 from ...core.tensor import Tensor
 from ...ops.creation import zeros
 from ..functional.init import normal
 
 
+def _factors(adapter: dict[str, Tensor]) -> tuple[Tensor, Tensor, float]:
+    """(A, B, 1 / rank) of an adapter dict."""
+    down, up = adapter["A"], adapter["B"]
+    return down, up, 1.0 / float(int(down.shape[1]))
+
+
 def init_lora_adapter(weight: Tensor, rank: int, init_std: float = 0.01,
                       dtype: DType | None = None) -> dict[str, Tensor]:
+    """Fresh adapter for a 2-D ``weight``: Gaussian ``A``, zero ``B``, so that it starts as a no-op."""
     if len(weight.shape) != 2:
         raise ValueError("init_lora_adapter expects a 2D weight tensor")
     if rank <= 0:
         raise ValueError("rank must be > 0")
-    in_features, out_features = int(weight.shape[0]), int(weight.shape[1])
-    adapter_dtype = dtype or weight.dtype
-    A = normal((in_features, rank), 0.0, init_std, dtype=adapter_dtype)
-    B = zeros((rank, out_features), dtype=adapter_dtype, device=weight.device)
-    return {"A": A, "B": B}
+    fan_in, fan_out = (int(d) for d in weight.shape)
+    kind = weight.dtype if dtype is None else dtype
+    return {"A": normal((fan_in, rank), 0.0, init_std, dtype=kind),
+            "B": zeros((rank, fan_out), dtype=kind, device=weight.device)}
 
 
 def lora_delta(adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
-    A, B = adapter["A"], adapter["B"]
-    rank = int(A.shape[1])
-    return (A @ B) * (alpha / float(rank))
+    """The full-size update ``(alpha / rank) * A @ B``."""
+    down, up, inv_rank = _factors(adapter)
+    return (down @ up) * (alpha * inv_rank)
 
 
 def lora_linear(x: Tensor, frozen_weight: Tensor, adapter: dict[str, Tensor],
                 alpha: float = 1.0) -> Tensor:
-    if config.LORA_LOW_RANK_ORDER:
-        A, B = adapter["A"], adapter["B"]
-        return (x @ frozen_weight) + ((x @ A) @ B) * (alpha / float(int(A.shape[1])))
-    return (x @ frozen_weight) + (x @ lora_delta(adapter, alpha=alpha))
+    """``x @ (frozen_weight + delta)`` without ever adding the two weights."""
+    base = x @ frozen_weight
+    if not config.LORA_LOW_RANK_ORDER:
+        return base + x @ lora_delta(adapter, alpha=alpha)
+    down, up, inv_rank = _factors(adapter)
+    return base + ((x @ down) @ up) * (alpha * inv_rank)
 
 
 def merge_lora_weight(frozen_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
@@ -49,3 +61,11 @@ def merge_lora_weight(frozen_weight: Tensor, adapter: dict[str, Tensor], alpha: 
 
 def unmerge_lora_weight(merged_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
     return merged_weight - lora_delta(adapter, alpha=alpha)
+
+
+def tree_lora_delta(adapters, alpha: float = 1.0, *, is_leaf=None):
+    """Every adapter dict in a pytree replaced by its full-size update; other leaves untouched."""
+    is_adapter = lambda node: isinstance(node, dict) and "A" in node and "B" in node
+    stop = is_adapter if is_leaf is None else (lambda node: is_adapter(node) or is_leaf(node))
+    return tree_map(lambda leaf: lora_delta(leaf, alpha=alpha) if is_adapter(leaf) else leaf,
+                    adapters, is_leaf=stop)

@@ -220,6 +220,22 @@ def _gemm(a, mem):
     out.copy_(C.to(out.dtype))
 
 
+_NF4_LEVELS = torch.tensor([-1.0, -0.6962, -0.5251, -0.3949, -0.2844, -0.1848, -0.0911, 0.0, 0.0796,
+                            0.1609, 0.2461, 0.3379, 0.4407, 0.5626, 0.7230, 1.0], dtype=torch.float32)
+
+
+def _gemm_nf4(a, mem):
+    codes = _view(mem, a["codes"]).reshape(-1).long()
+    scales = _view(mem, a["scales"]).reshape(-1).float()
+    w = (_NF4_LEVELS[codes].reshape(-1, a["block"]) * scales[:, None]).reshape(a["w_shape"])
+    dst = _view(mem, a["dst"])
+    if dst.dtype == torch.bfloat16:  # level * scale is rounded to bf16 once, as in the kernel
+        w = w.to(torch.bfloat16).float()
+    x = _view(mem, a["x"]).reshape(a["M"], a["K"]).double()
+    w = w.double().t() if a["transpose"] else w.double()
+    dst.copy_((x @ w).reshape(dst.shape).to(dst.dtype))
+
+
 def _conv(kind, a, mem):
     import torch.nn.functional as F
     pt, pb, pl, pr = a["padding"]
@@ -367,6 +383,8 @@ class EmulatedPlan:
                     _store(mem[d.buf], d.offset + np.arange(t["outer"] * t["inner"]), np.asarray(r, dtype=_F32))
             elif k == "gemm":
                 _gemm(a, mem)
+            elif k == "gemm_nf4":
+                _gemm_nf4(a, mem)
             elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
                 _conv(k, a, mem)
             elif k in ("maxpool2d", "maxpool2d_bwd"):

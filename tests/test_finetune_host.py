@@ -137,3 +137,43 @@ def test_checkpoint_nested_trees_without_optimizer_and_errors(emulator, tmp_path
         ft.load_finetune_checkpoint(tmp_path / "nonexistent", lora_template=template)
     with pytest.raises(KeyError, match="Missing tensor key"):
         ft.load_finetune_checkpoint(ckpt, lora_template=template + [dict(template[0])])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_qlora_base_product_reads_the_codes(emulator, dtype):
+    """A weight whose width is a multiple of 8: qlora_linear's base product is one launch on the
+    NF4 codes (no dense weight in the plan), forward and, for the gradient with respect to the
+    activations, the same kernel on the transposed weight; values against the oracle."""
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(2031)
+    n, din, dout = 24, 40, 16
+    x = rng.standard_normal((2, n, din)).astype(np.float32)
+    w = rng.standard_normal((din, dout)).astype(np.float32)
+    dt = nb.DType.float32 if dtype == "f32" else nb.DType.bfloat16
+    tol = 2e-5 if dtype == "f32" else 2e-2
+    qw = ft.quantize_nf4(T(w), block_size=8)
+    adapter = {"A": T(rng.standard_normal((din, 4)).astype(np.float32) * 0.1),
+               "B": T(rng.standard_normal((4, dout)).astype(np.float32) * 0.1)}
+    wd = O.nf4_dequantize(O.nf4_quantize(w, 8)).astype(np.float64)
+    A, B = (adapter[k].to_numpy().astype(np.float64) for k in "AB")
+
+    def f(xt, p):
+        return nb.reduce_sum(ft.qlora_linear(xt, qw, p, alpha=2.0, compute_dtype=dt) ** 2)
+
+    engine.clear_plan_cache()
+    y = ft.qlora_linear(T(x), qw, adapter, alpha=2.0, compute_dtype=dt)
+    want = x.astype(np.float64) @ wd + x.astype(np.float64) @ ((A @ B) * 0.5)
+    got = y.to(nb.DType.float32).to_numpy()
+    assert np.abs(got - want).max() <= tol * np.abs(want).max()
+    kinds = [st.kind for st in list(engine._PLAN_CACHE.values())[-1].plan.steps]
+    assert kinds.count("gemm_nf4") == 1 and "gather" not in kinds
+    gx, gp = nb.grad(f, argnums=(0, 1))(T(x), adapter)
+    nb.realize_all(gx, gp["A"], gp["B"])
+    steps = list(engine._PLAN_CACHE.values())[-1].plan.steps
+    assert sorted(st.attrs["transpose"] for st in steps if st.kind == "gemm_nf4") == [False, True]
+    vx, vA, vB = O.V(x.astype(np.float64)), O.V(A), O.V(B)
+    out = O.matmul(vx, O.V(wd)) + O.matmul(vx, O.matmul(vA, vB) * 0.5)
+    wgx, wgA, wgB = O.grad_of(O.reduce_sum(out * out), [vx, vA, vB])
+    for g, wnt in ((gx, wgx), (gp["A"], wgA), (gp["B"], wgB)):
+        g = g.to(nb.DType.float32).to_numpy()
+        assert np.abs(g - wnt).max() <= (tol if dtype == "f32" else 4e-2) * np.abs(wnt).max()
