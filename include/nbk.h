@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 15
+#define NBK_ABI_VERSION 16
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -419,6 +419,50 @@ typedef int (*nbk_custom_fn)(const nbk_tensor* in, int n_in, nbk_tensor* out,
                              int n_out, void* stream);
 int nbk_custom(const char* library_path, const char* name, const nbk_tensor* in,
                int n_in, nbk_tensor* out, int n_out, void* stream);
+
+/* ===================================================================== */
+/*  Optimizer updates, all parameters in one launch                       */
+/* ===================================================================== */
+/* The reference updates a parameter pytree leaf by leaf with tensor arithmetic
+ * (sgd_step nabla/nn/optim/functional.py:14-39, adamw_step 116-162, mapped over the leaves by
+ * sgd_update 42-113 and adamw_update nabla/nn/optim/optimizer.py:242-305).  These two entry
+ * points take the whole list: `tensors` is a host array of n entries, every entry the pointers of
+ * one leaf -- all of them in `dtype` (NBK_F32 or NBK_BF16), contiguous, `numel` elements.  The
+ * *_out pointers may be the inputs themselves (an in-place step) or fresh storage (the
+ * functional form).  Arithmetic is fp32 in registers, one rounding per stored result.  One
+ * launch per NBK_OPT_MULTI_MAX tensors. */
+#define NBK_OPT_MULTI_MAX 48
+typedef struct nbk_opt_tensor {
+  const void* param; const void* grad;
+  const void* m;        /* AdamW first moment / SGD momentum buffer (unused without momentum) */
+  const void* v;        /* AdamW second moment (unused by SGD)                                 */
+  void* param_out; void* m_out; void* v_out;
+  int64_t numel;
+} nbk_opt_tensor;
+/* m' = beta1 m + (1-beta1) g;  v' = beta2 v + (1-beta2) g^2;
+ * p' = p - lr ((m'/c1) / (sqrt(v'/c2) + eps) + weight_decay p)        (decoupled decay)
+ * Bias corrections: with bias_correction == 0, c1 = c2 = 1.  Otherwise, when `step` is NULL the
+ * host passes c1 = 1 - beta1^t and c2 = 1 - beta2^t; when `step` points to a device fp32 scalar
+ * holding t (the counter is data inside a compiled step: optimizer.py:262-268), the kernel
+ * computes c = 1 - exp(t log beta) itself from log_beta1 / log_beta2. */
+typedef struct nbk_adamw_desc {
+  float lr, beta1, beta2, eps, weight_decay;
+  float c1, c2;
+  float log_beta1, log_beta2;
+  int32_t bias_correction;
+  const float* step;
+  int32_t dtype;
+  int32_t reserved;
+} nbk_adamw_desc;
+int nbk_adamw_multi(const nbk_adamw_desc* d, const nbk_opt_tensor* tensors, int32_t n, void* stream);
+/* dir = g + weight_decay p;  with momentum != 0: buf' = momentum buf + dir, dir = buf';
+ * p' = p - lr dir.  (A leaf without a buffer yet passes zeros: the first step then adopts the
+ * direction as the buffer, as functional.py:30-34 does.) */
+typedef struct nbk_sgd_desc {
+  float lr, momentum, weight_decay;
+  int32_t dtype;
+} nbk_sgd_desc;
+int nbk_sgd_multi(const nbk_sgd_desc* d, const nbk_opt_tensor* tensors, int32_t n, void* stream);
 
 /* ===================================================================== */
 /*  Measurement helpers                                                   */

@@ -12,6 +12,7 @@ same launch records.
 from __future__ import annotations
 
 import ctypes as C
+import math
 import os
 from typing import Any, Sequence
 
@@ -306,6 +307,39 @@ class BoundPlan:
                 self.calls.append((L.nbk_argmax_rows,
                                    [holder, ("p0", "p1"), src.dtype.abi, a["rows"], a["C"],
                                     1 if a["fn"] == "min" else 0], patches, None))
+            elif k in ("adamw_multi", "sgd_multi"):
+                entries = a["entries"]
+                table = (lib.OptTensor * len(entries))()
+                in_fields = ("param", "grad", "m", "v")
+                out_fields = ("param_out", "m_out", "v_out")
+                for t, e in zip(table, entries):
+                    for name, r in zip(in_fields, e["ins"]):
+                        ptr_field(t, name, r.buf, r.offset * r.dtype.size_in_bytes)
+                    for name, r in zip(out_fields, e["outs"]):
+                        ptr_field(t, name, r.buf, r.offset * r.dtype.size_in_bytes)
+                    t.numel = e["numel"]
+                if k == "adamw_multi":
+                    d = lib.AdamwDesc()
+                    d.lr, d.beta1, d.beta2, d.eps = a["lr"], a["beta1"], a["beta2"], a["eps"]
+                    d.weight_decay = a["weight_decay"]
+                    d.bias_correction = 1 if a["bias_correction"] else 0
+                    d.log_beta1 = math.log(a["beta1"]) if a["beta1"] > 0.0 else -math.inf
+                    d.log_beta2 = math.log(a["beta2"]) if a["beta2"] > 0.0 else -math.inf
+                    d.c1 = d.c2 = 1.0
+                    d.step = None
+                    if a["step"] is not None:
+                        d.c1 = 1.0 - a["beta1"] ** a["step"]
+                        d.c2 = 1.0 - a["beta2"] ** a["step"]
+                    else:
+                        r = a["step_ref"]
+                        ptr_field(d, "step", r.buf, r.offset * 4)
+                    fn = L.nbk_adamw_multi
+                else:
+                    d = lib.SgdDesc()
+                    d.lr, d.momentum, d.weight_decay = a["lr"], a["momentum"], a["weight_decay"]
+                    fn = L.nbk_sgd_multi
+                d.dtype = a["dtype"].abi
+                self.calls.append((fn, [C.byref(d), table, len(entries)], patches, (d, table)))
             elif k == "custom":
                 ins = (lib.TensorDesc * max(len(a["ins"]), 1))()
                 outs = (lib.TensorDesc * len(a["dsts"]))()

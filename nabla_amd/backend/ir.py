@@ -453,3 +453,53 @@ def attention_bwd(q: Value, k: Value, v: Value, o: Value, lse: Value, dout: Valu
     """Gradients (dq, dk, dv) of ``attention`` from its inputs, both outputs and d(output)."""
     return current().add("attention_bwd", [q, k, v, o, lse, dout], [(q.shape, q.dtype)] * 3,
                          scale=float(scale), causal=bool(causal))
+
+
+# ---- optimizer updates over a list of parameters ---------------------------------------------
+def _check_update_list(who: str, groups: Sequence[Sequence[Value]]) -> DType:
+    first = groups[0][0]
+    for vals in groups:
+        for v in vals:
+            if v.dtype is not first.dtype or v.shape != vals[0].shape:
+                raise ValueError(f"{who}: every tensor of a parameter shares its shape, and all of "
+                                 f"them one dtype; got {v.shape} {v.dtype} beside {vals[0].shape} "
+                                 f"{first.dtype}")
+    if first.dtype not in (DType.float32, DType.bfloat16):
+        raise TypeError(f"{who}: float32 or bfloat16 parameters, got {first.dtype}")
+    return first.dtype
+
+
+def adamw_multi(params: Sequence[Value], grads: Sequence[Value], ms: Sequence[Value],
+                vs: Sequence[Value], step: Value | float, *, lr: float, beta1: float, beta2: float,
+                eps: float, weight_decay: float, bias_correction: bool) -> list[Value]:
+    """One AdamW step for every parameter of the list: ``[p'_0, m'_0, v'_0, p'_1, ...]``.  ``step``
+    (the number of this step, from 1) is a number or a 0-d float32 value."""
+    groups = list(zip(params, grads, ms, vs))
+    _check_update_list("adamw_multi", groups)
+    inputs = [x for g in groups for x in g]
+    attrs = dict(lr=float(lr), beta1=float(beta1), beta2=float(beta2), eps=float(eps),
+                 weight_decay=float(weight_decay), bias_correction=bool(bias_correction),
+                 n=len(groups), step=None)
+    if isinstance(step, Value):
+        if step.numel() != 1 or step.dtype is not DType.float32:
+            raise TypeError(f"adamw_multi: the step counter is one float32 value, got {step}")
+        inputs.append(step)
+    else:
+        attrs["step"] = float(step)
+    outs = [(p.shape, p.dtype) for p in params for _ in range(3)]
+    return current().add("adamw_multi", inputs, outs, **attrs)
+
+
+def sgd_multi(params: Sequence[Value], grads: Sequence[Value], bufs: Sequence[Value] | None, *,
+              lr: float, momentum: float, weight_decay: float) -> list[Value]:
+    """One SGD step for every parameter of the list.  With momentum ``bufs`` holds the momentum
+    buffers and the result is ``[p'_0, buf'_0, p'_1, ...]``; without, ``[p'_0, p'_1, ...]``."""
+    with_mom = float(momentum) != 0.0
+    if with_mom and bufs is None:
+        raise ValueError("sgd_multi: momentum needs the momentum buffers")
+    groups = list(zip(params, grads, bufs)) if with_mom else list(zip(params, grads))
+    _check_update_list("sgd_multi", groups)
+    inputs = [x for g in groups for x in g]
+    outs = [(p.shape, p.dtype) for p in params for _ in range(2 if with_mom else 1)]
+    return current().add("sgd_multi", inputs, outs, lr=float(lr), momentum=float(momentum),
+                         weight_decay=float(weight_decay), n=len(groups))

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 MAX_RANK = 8
 
@@ -120,6 +120,27 @@ class ReduceTask(C.Structure):
     ]
 
 
+class OptTensor(C.Structure):
+    _fields_ = [
+        ("param", C.c_void_p), ("grad", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
+        ("param_out", C.c_void_p), ("m_out", C.c_void_p), ("v_out", C.c_void_p), ("numel", C.c_int64),
+    ]
+
+
+class AdamwDesc(C.Structure):
+    _fields_ = [
+        ("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("eps", C.c_float),
+        ("weight_decay", C.c_float), ("c1", C.c_float), ("c2", C.c_float),
+        ("log_beta1", C.c_float), ("log_beta2", C.c_float), ("bias_correction", C.c_int32),
+        ("step", C.c_void_p), ("dtype", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class SgdDesc(C.Structure):
+    _fields_ = [("lr", C.c_float), ("momentum", C.c_float), ("weight_decay", C.c_float),
+                ("dtype", C.c_int32)]
+
+
 class TensorDesc(C.Structure):
     _fields_ = [
         ("ptr", C.c_void_p), ("dtype", C.c_int32), ("rank", C.c_int32),
@@ -142,6 +163,8 @@ _SIGNATURES = {
     "nbk_rowprog_hash": ([C.POINTER(RowProg)], C.c_uint64),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
                         C.c_int64, C.c_int32, C.c_void_p], C.c_int),
+    "nbk_adamw_multi": ([C.POINTER(AdamwDesc), C.POINTER(OptTensor), C.c_int32, C.c_void_p], C.c_int),
+    "nbk_sgd_multi": ([C.POINTER(SgdDesc), C.POINTER(OptTensor), C.c_int32, C.c_void_p], C.c_int),
     "nbk_reduce_mid_batch": ([C.POINTER(ReduceTask), C.c_int32, C.c_void_p], C.c_int),
     "nbk_copy_strided": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
                           C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64),

@@ -988,8 +988,27 @@ class Planner:
             dsts = [self._alloc_value(o) for o in n.outputs]
             self._emit(Step("custom", [i.buf for i in ins], [d.buf for d in dsts], dict(
                 ins=ins, dsts=dsts, name=n.attrs["name"], library=n.attrs["library"])))
+        elif k in ("adamw_multi", "sgd_multi"):
+            self._lower_update_list(n)
         else:
             raise NotImplementedError(f"lowering: no rule for node kind '{k}'")
+
+    def _lower_update_list(self, n: ir.Node) -> None:
+        """An optimizer step over a list of parameters: one launch whose table holds, per
+        parameter, where its tensors are read and where the results go."""
+        count = n.attrs["n"]
+        per_in = (len(n.inputs) - (1 if n.kind == "adamw_multi" and n.attrs["step"] is None else 0)) // count
+        per_out = len(n.outputs) // count
+        ins = [self._contig(i) for i in n.inputs]
+        outs = [self._alloc_value(o) for o in n.outputs]
+        entries = [dict(ins=ins[i * per_in:(i + 1) * per_in], outs=outs[i * per_out:(i + 1) * per_out],
+                        numel=n.outputs[i * per_out].numel()) for i in range(count)]
+        attrs = {key: val for key, val in n.attrs.items() if key != "n"}
+        attrs["entries"] = entries
+        attrs["dtype"] = n.outputs[0].dtype
+        if n.kind == "adamw_multi" and n.attrs["step"] is None:
+            attrs["step_ref"] = ins[-1]
+        self._emit(Step(n.kind, [r.buf for r in ins], [r.buf for r in outs], attrs))
 
     def _copy_into(self, src, dst: ViewRef, starts, shape) -> None:
         off = dst.offset + sum(a * s for a, s in zip(starts, dst.strides))

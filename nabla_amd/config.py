@@ -44,6 +44,11 @@ _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
 _FUSED_NF4_MATMUL: ContextVar[bool] = ContextVar("FUSED_NF4_MATMUL",
                                                  default=_env_flag("NBK_FUSED_NF4_MATMUL", True))
 
+# optimizer steps over pytrees as one launch per dtype (ops.optim); off: a group of tensor ops
+# per leaf, as the reference writes them
+_MULTI_TENSOR_OPTIMIZER: ContextVar[bool] = ContextVar(
+    "MULTI_TENSOR_OPTIMIZER", default=_env_flag("NBK_MULTI_TENSOR_OPTIMIZER", True))
+
 _FLAGS = {
     "EAGER_MAX_GRAPH": _EAGER_MAX_GRAPH,
     "VERIFY_EAGER_SHAPES": _VERIFY_EAGER_SHAPES,
@@ -52,6 +57,7 @@ _FLAGS = {
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
+    "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,
 }
 
 

@@ -128,8 +128,8 @@ class ComputeGraph:
         parts = []
         for impl in leaves:
             parts.append(("L", impl.shape, impl.dtype))
-        n_leaves = len(leaves)
-        for ni, node in enumerate(order):
+        next_slot = len(leaves) + (1 << 40)
+        for node in order:
             ins = []
             for a in node.op_args:
                 if isinstance(a, TensorImpl):
@@ -143,9 +143,10 @@ class ComputeGraph:
             if kw is None:
                 kw = _freeze(node.op_kwargs) if node.op_kwargs else ()
             parts.append((node.op.name, kw, tuple(ins), len(node._refs)))
-            for oi, o in enumerate(node._refs):
+            for o in node._refs:  # (numbered whether alive or not: the number says which result it is)
                 if o is not None:
-                    slot[id(o)] = n_leaves + ni * 8 + oi + (1 << 40)
+                    slot[id(o)] = next_slot
+                next_slot += 1
         tk = tuple(leaf_ids[id(t)] if t._buffer is not None else slot[id(t)] for t in targets)
         return (tuple(parts), tk)
 

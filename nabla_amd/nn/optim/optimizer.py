@@ -9,9 +9,11 @@ from __future__ import annotations
 
 from typing import Any
 
-from ...core import is_tensor, realize_all, tree_flatten, tree_unflatten
+from ... import config
+from ...core import Tensor, is_tensor, realize_all, tree_flatten, tree_unflatten
+from ...core.dtype import DType
 from ...ops.creation import zeros_like
-from .functional import adamw_step, map_update, sgd_step, unrealized
+from .functional import adamw_over_trees, adamw_step, sgd_over_trees, sgd_step, unrealized
 
 
 def _zeros_tree(params: Any):
@@ -102,7 +104,12 @@ class AdamW(Optimizer):
             return adamw_step(p, g, m, v, self.step_count, lr=self.lr, beta1=self.beta1,
                               beta2=self.beta2, eps=self.eps, weight_decay=self.weight_decay)
 
-        self.params, self.m, self.v = map_update(one, self.params, grads, self.m, self.v)
+        # (the counter goes in as data: one plan serves every step)
+        step = Tensor.constant(float(self.step_count), dtype=DType.float32) \
+            if config.MULTI_TENSOR_OPTIMIZER else self.step_count
+        self.params, self.m, self.v = adamw_over_trees(
+            one, self.params, grads, self.m, self.v, step, lr=self.lr, beta1=self.beta1,
+            beta2=self.beta2, eps=self.eps, weight_decay=self.weight_decay)
         return self._finish(old, self.m, self.v)
 
 
@@ -128,7 +135,8 @@ class SGD(Optimizer):
             return sgd_step(p, g, buf, lr=self.lr, weight_decay=self.weight_decay,
                             momentum=self.momentum)
 
-        self.params, bufs = map_update(one, self.params, grads, self.momentum_buffers)
+        self.params, bufs = sgd_over_trees(one, self.params, grads, self.momentum_buffers, lr=self.lr,
+                                           momentum=self.momentum, weight_decay=self.weight_decay)
         if self.momentum != 0.0:
             self.momentum_buffers = bufs
             return self._finish(old, self.momentum_buffers)
@@ -154,7 +162,9 @@ def adamw_update(params: Any, grads: Any, state: dict[str, Any], *, lr: float,
         return adamw_step(p, g, m, v, step, lr=lr, beta1=beta1, beta2=beta2, eps=eps,
                           weight_decay=weight_decay, bias_correction=bias_correction)
 
-    new_params, new_m, new_v = map_update(one, params, grads, state["m"], state["v"])
+    new_params, new_m, new_v = adamw_over_trees(
+        one, params, grads, state["m"], state["v"], step, lr=lr, beta1=beta1, beta2=beta2, eps=eps,
+        weight_decay=weight_decay, bias_correction=bias_correction)
     do_realize = Optimizer._AUTO_REALIZE_UPDATED_PARAMS if realize is None else bool(realize)
     if do_realize:
         todo = unrealized(new_params)

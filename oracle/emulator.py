@@ -236,6 +236,34 @@ def _gemm_nf4(a, mem):
     dst.copy_((x @ w).reshape(dst.shape).to(dst.dtype))
 
 
+def _update_list(kind, a, mem):
+    """Optimizer step over a list of parameters, in float64 from the stored values
+    (nabla/nn/optim/functional.py:14-39 and 116-162)."""
+    for e in a["entries"]:
+        ins = [_view(mem, r).double() for r in e["ins"]]
+        outs = [_view(mem, r) for r in e["outs"]]
+        p, g = ins[0], ins[1]
+        if kind == "adamw_multi":
+            m, v = ins[2], ins[3]
+            b1, b2 = a["beta1"], a["beta2"]
+            step = a["step"] if a["step"] is not None else float(_view(mem, a["step_ref"]).reshape(-1)[0])
+            c1 = 1.0 - b1 ** step if a["bias_correction"] else 1.0
+            c2 = 1.0 - b2 ** step if a["bias_correction"] else 1.0
+            m_t = m * b1 + g * (1.0 - b1)
+            v_t = v * b2 + g * g * (1.0 - b2)
+            upd = (m_t / c1) / ((v_t / c2).sqrt() + a["eps"]) + p * a["weight_decay"]
+            results = [p - upd * a["lr"], m_t, v_t]
+        else:
+            direction = g + p * a["weight_decay"]
+            results = []
+            if a["momentum"] != 0.0:
+                direction = ins[2] * a["momentum"] + direction
+                results = [direction]
+            results.insert(0, p - direction * a["lr"])
+        for dst, val in zip(outs, results):
+            dst.copy_(val.to(dst.dtype))
+
+
 def _conv(kind, a, mem):
     import torch.nn.functional as F
     pt, pb, pl, pr = a["padding"]
@@ -385,6 +413,8 @@ class EmulatedPlan:
                 _gemm(a, mem)
             elif k == "gemm_nf4":
                 _gemm_nf4(a, mem)
+            elif k in ("adamw_multi", "sgd_multi"):
+                _update_list(k, a, mem)
             elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
                 _conv(k, a, mem)
             elif k in ("maxpool2d", "maxpool2d_bwd"):
