@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 16
+#define NBK_ABI_VERSION 17
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -118,8 +118,8 @@ enum nbk_rp_op {
   NBK_OP_LDR = 4,      /* prologue: sreg dst <- operand a at column 0          */
   NBK_OP_STR = 5,      /* prologue: operand dst <- sreg a (column 0, 1 lane)   */
   NBK_OP_IMM = 6,      /* prologue: sreg dst <- imm[a]                         */
-  NBK_OP_COLIDX = 7,   /* body: vreg dst <- column index as float              */
-  NBK_OP_LEADIDX = 8,  /* prologue: sreg dst <- index along leading dim a      */
+  NBK_OP_COLIDX = 7,   /* body: vreg dst <- column index, as float (a = 0) or int32 (a = 1) */
+  NBK_OP_LEADIDX = 8,  /* prologue: sreg dst <- index along leading dim a, as float (b = 0) or int32 (b = 1) */
   /* reductions over the row */
   NBK_OP_ACCINIT = 9,  /* prologue: acc dst <- identity of kind a              */
   NBK_OP_ACC = 10,     /* body: acc dst <- combine(acc, vreg a), kind b        */
@@ -142,7 +142,22 @@ enum nbk_rp_op {
   NBK_OP_FMA = 49,     /* dst <- a * b + c                                     */
   /* more unary ops (the block 16..31 is full) */
   NBK_OP_DGELU = 50,   /* derivative of the exact GELU: Phi(a) + a * phi(a)    */
-  NBK_OP_SIN = 51, NBK_OP_COS = 52 /* unary; the block 16..31 is full              */
+  NBK_OP_SIN = 51, NBK_OP_COS = 52, /* unary; the block 16..31 is full             */
+  /* Integer registers.  A register is 32 bits; the program decides what they mean.  Values of
+   * int32 / int64 tensors are loaded, held and stored as two's-complement int32 (LDG / LDR /
+   * STG / STR go by the operand's dtype; int64 storage passes through its low 32 bits, sign-
+   * extended on the way out), and these instructions compute on them exactly, wrapping modulo
+   * 2^32.  Floats, bool and uint8 are fp32 in registers.  MOV, WHERE (its payload) and IMM move
+   * bits and serve both; an integer immediate is stored in imm[] by its bit pattern. */
+  /* binary on int32 (comparisons produce a float 0 / 1, like their float forms) */
+  NBK_OP_IADD = 64, NBK_OP_ISUB = 65, NBK_OP_IMUL = 66, NBK_OP_IMAX = 67, NBK_OP_IMIN = 68,
+  NBK_OP_IGT = 69, NBK_OP_IGE = 70, NBK_OP_IEQ = 71, NBK_OP_INE = 72, NBK_OP_ILT = 73,
+  NBK_OP_ILE = 74,
+  /* unary on int32 */
+  NBK_OP_INEG = 80, NBK_OP_IABS = 81, NBK_OP_IRELU = 82,
+  NBK_OP_I2F = 83,     /* int32 -> float                                        */
+  NBK_OP_F2I = 84,     /* float -> int32, toward zero                           */
+  NBK_OP_INEZ = 85     /* int32 != 0 -> float 1 / 0                             */
 };
 
 enum nbk_red_kind { NBK_RED_SUM = 0, NBK_RED_MAX = 1, NBK_RED_MIN = 2 };

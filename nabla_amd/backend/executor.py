@@ -85,8 +85,12 @@ class BoundPlan:
                 rp.block = a["block"]
                 rp.n_stage = a["n_stage"]
                 rp.reserved = 1 if self.ex.force_interpreter else 0
+                imm_bits = C.cast(rp.imm, C.POINTER(C.c_int32))
                 for i, v in enumerate(a["imm"]):
-                    rp.imm[i] = v
+                    if isinstance(v, int):  # an integer register's immediate: its bit pattern
+                        imm_bits[i] = v
+                    else:
+                        rp.imm[i] = v
                 for i, o in enumerate(a["operands"]):
                     od = rp.operand[i]
                     for j, s in enumerate(o.lead_strides):

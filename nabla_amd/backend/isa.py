@@ -17,6 +17,16 @@ BINARY = {
     "eq": 40, "ne": 41, "lt": 42, "le": 43, "pow": 44, "and": 45, "or": 46,
 }
 TERNARY = {"where": 48, "fma": 49}
+# int32 registers (values of int32 / int64 tensors); comparisons give a float 0 / 1
+INT_BINARY = {"iadd": 64, "isub": 65, "imul": 66, "imax": 67, "imin": 68, "igt": 69, "ige": 70,
+              "ieq": 71, "ine": 72, "ilt": 73, "ile": 74}
+INT_UNARY = {"ineg": 80, "iabs": 81, "irelu": 82, "i2f": 83, "f2i": 84, "inez": 85}
+UNARY.update(INT_UNARY)
+BINARY.update(INT_BINARY)
+#: float elementwise function -> its form on integer registers
+INT_FORM = {"add": "iadd", "sub": "isub", "mul": "imul", "max": "imax", "min": "imin", "gt": "igt",
+            "ge": "ige", "eq": "ieq", "ne": "ine", "lt": "ilt", "le": "ile", "neg": "ineg",
+            "abs": "iabs", "relu": "irelu", "nez": "inez", "mov": "mov"}
 EW = {**UNARY, **BINARY, **TERNARY}
 EW_NAME = {v: k for k, v in EW.items()}
 

@@ -29,6 +29,8 @@ from ..core.dtype import DType
 from . import ir, isa
 
 FUSABLE = ("ew", "reduce", "tril", "iota")
+#: values of these types live in row-program registers as int32, not as fp32
+INT_REG_DTYPES = (DType.int32, DType.int64)
 VIEW_KINDS = ("reshape", "broadcast", "permute", "slice")
 
 
@@ -421,7 +423,10 @@ class Planner:
                         self.unit_of[node.pos] = g
                         self.alias_nodes.add(node.pos)
                 continue
-            if kind not in FUSABLE or (kind == "reduce" and node.attrs["axis"] != node.inputs[0].rank - 1):
+            # (integer reductions keep a 64-bit accumulator in a kernel of their own)
+            if kind not in FUSABLE or (kind == "reduce" and (
+                    node.attrs["axis"] != node.inputs[0].rank - 1 or
+                    node.inputs[0].dtype in INT_REG_DTYPES)):
                 u = new_unit(node, False)
                 for i in node.inputs:
                     pu = self._producer_unit(i)
@@ -1101,7 +1106,7 @@ class Planner:
         vec = 16 // x.dtype.size_in_bytes if inner % (16 // x.dtype.size_in_bytes) == 0 else 1
         blocks = outer * ((inner + 64 * vec - 1) // (64 * vec))
         split = 1
-        if blocks < 256 and red >= 256:
+        if blocks < 256 and red >= 256 and x.dtype.is_float():  # (partials are fp32)
             want = min(256, red // 64, max(1, 1024 // max(blocks, 1)))
             for s in range(want, 1, -1):
                 if red % s == 0 and outer * s <= 65535:
@@ -1432,11 +1437,16 @@ class Planner:
 
 # ------------------------------------------------------------------ row codegen
 class _VReg:
-    __slots__ = ("kind", "id")
+    __slots__ = ("kind", "id", "t")
 
-    def __init__(self, kind: str, vid: int):
+    def __init__(self, kind: str, vid: int, t: str = "f"):
         self.kind = kind  # 'v' vector | 's' scalar
         self.id = vid
+        self.t = t        # what the 32 bits hold: 'f' fp32 (floats, bool, uint8) | 'i' int32
+
+
+def _reg_type(dtype: DType) -> str:
+    return "i" if dtype in INT_REG_DTYPES else "f"
 
 
 class _RowCodegen:
@@ -1509,7 +1519,7 @@ class _RowCodegen:
             """('imm', value) or ('op', index, class) for an external input."""
             loc = p._resolve(v)
             if isinstance(loc, Const):
-                return ("imm", float(loc.value))
+                return ("imm", float(loc.value), _reg_type(v.dtype))
             lead_st, col = self._dom_strides(loc)
             key = (loc.buf, loc.offset, lead_st, col)
             idx = op_index.get(key)
@@ -1553,9 +1563,9 @@ class _RowCodegen:
         n_vregs = [0]
         imm_vals: list[float] = []
 
-        def new_v(kind: str) -> _VReg:
+        def new_v(kind: str, t: str = "f") -> _VReg:
             n_vregs[0] += 1
-            return _VReg(kind, n_vregs[0])
+            return _VReg(kind, n_vregs[0], t)
 
         sreg_of: dict[Any, _VReg] = {}   # row value id / ('op', idx) / ('imm', value) -> sreg
         out_operand: dict[int, int] = {}
@@ -1572,9 +1582,16 @@ class _RowCodegen:
                 out_operand[v.id] = idx
             return idx
 
-        def imm_index(val: float) -> int:
+        def imm_index(val) -> int:
+            """Slot of an immediate: a Python int is an integer register's (stored by its bits),
+            a float an fp32 one."""
             for i, x in enumerate(imm_vals):
-                if x == val or (x != x and val != val):
+                if type(x) is not type(val):
+                    continue
+                if isinstance(val, int):
+                    if x == val:
+                        return i
+                elif x == val or (x != x and val != val):
                     if math.copysign(1.0, x) == math.copysign(1.0, val) or x != x:
                         return i
             imm_vals.append(val)
@@ -1582,20 +1599,103 @@ class _RowCodegen:
 
         prologue: list[list] = []
 
-        def scalar_for(key, emit) -> _VReg:
+        def scalar_for(key, emit, t: str = "f") -> _VReg:
             r = sreg_of.get(key)
             if r is None:
-                r = new_v("s")
+                r = new_v("s", t)
                 sreg_of[key] = r
                 emit(r)
             return r
 
-        def scalar_imm(val: float) -> _VReg:
+        def scalar_imm(val: float, t: str = "f") -> _VReg:
+            if t == "i" and val == val and abs(val) != math.inf and val == int(val):
+                if not -2 ** 31 <= int(val) < 2 ** 31:
+                    raise NotImplementedError(
+                        f"the integer constant {int(val)} does not fit the 32-bit integer registers "
+                        "of a fused kernel")
+                return scalar_for(("imm", int(val), "i"), lambda r: prologue.append(
+                    [isa.IMM, r, imm_index(int(val)), 0, 0, 0]), "i")
             return scalar_for(("imm", val), lambda r: prologue.append(
-                [isa.IMM, r, imm_index(val), 0, 0, 0]))
+                [isa.IMM, r, imm_index(float(val)), 0, 0, 0]))
 
         def scalar_ext(idx: int) -> _VReg:
-            return scalar_for(("op", idx), lambda r: prologue.append([isa.LDR, r, idx, 0, 0, 0]))
+            return scalar_for(("op", idx), lambda r: prologue.append([isa.LDR, r, idx, 0, 0, 0]),
+                              _reg_type(operands[idx].dtype))
+
+        conv_v: dict = {}  # (register id, type) -> converted vector register, per phase
+
+        def as_type(r: _VReg, t: str, body: list) -> _VReg:
+            """``r`` as a register of type ``t``: itself, or its conversion (int32 <-> fp32, the
+            float -> int direction toward zero).  A scalar converts once per row, in the
+            prologue; a vector register in the body that asks."""
+            if r.t == t:
+                return r
+            op = isa.EW["i2f" if t == "f" else "f2i"]
+            if r.kind == "s":
+                return scalar_for(("conv", r.id, t), lambda o: prologue.append([op, o, r, 0, 0, 0]), t)
+            hit = conv_v.get((r.id, t))
+            if hit is None:
+                hit = new_v("v", t)
+                body.append([op, hit, r, 0, 0, 0])
+                conv_v[(r.id, t)] = hit
+            return hit
+
+        def truthy(r: _VReg, code: list, kind: str) -> _VReg:
+            """A 0 / 1 float for the condition held in ``r``."""
+            if r.t == "f":
+                return r
+            out = new_v(kind, "f")
+            code.append([isa.EW["inez"], out, r, 0, 0, 0])
+            return out
+
+        def emit_ew(n: ir.Node, get, code: list, kind: str) -> _VReg:
+            """Instructions for the elementwise node ``n`` into ``code``; ``get(x, t)`` gives the
+            register of operand ``x`` (a Python number becomes an immediate of type ``t``).  Which
+            form an operation takes follows the types: integer tensors compute in int32 where
+            the operation has an integer form, everything else in fp32 with conversions at the
+            edges."""
+            fn = n.fn
+            o = n.outputs[0]
+            ot = _reg_type(o.dtype)
+            xs = n.attrs["operands"]
+            vals = [x for x in xs if isinstance(x, ir.Value)]
+
+            def conv(r, t):
+                if kind == "s" and r.kind != "s":
+                    raise AssertionError("vector register in a row-scalar operation")
+                return as_type(r, t, code)
+
+            def out(name: str, regs, t: str) -> _VReg:
+                r = new_v(kind, t)
+                regs = list(regs) + [0] * (3 - len(regs))
+                code.append([isa.EW[name], r, regs[0], regs[1], regs[2], 0])
+                return r
+
+            if fn in ("mov", "trunc", "nez"):
+                src = get(xs[0], ot)
+                if fn == "nez":
+                    return out("inez" if src.t == "i" else "nez", [src], "f")
+                if src.t == ot:
+                    return out(fn if ot == "f" else "mov", [src], ot)
+                return out("i2f" if ot == "f" else "f2i", [src], ot)
+            if fn in ("gt", "ge", "eq", "ne", "lt", "le"):
+                whole = all(v.dtype.is_integral() or v.dtype is DType.bool for v in vals) and \
+                    all(isinstance(x, ir.Value) or float(x) == int(x) for x in xs)
+                ct = "i" if whole and any(_reg_type(v.dtype) == "i" for v in vals) else "f"
+                regs = [conv(get(x, ct), ct) for x in xs]
+                return out(isa.INT_FORM[fn] if ct == "i" else fn, regs, "f")
+            if fn in ("and", "or", "not"):
+                return out(fn, [truthy(get(x, "f"), code, kind) for x in xs], "f")
+            if fn == "where":
+                cond = truthy(get(xs[0], "f"), code, kind)
+                return out("where", [cond] + [conv(get(x, ot), ot) for x in xs[1:]], ot)
+            if ot == "i" and fn in isa.INT_FORM and \
+                    all(isinstance(x, ir.Value) or float(x) == int(x) for x in xs):
+                return out(isa.INT_FORM[fn], [conv(get(x, "i"), "i") for x in xs], "i")
+            r = out(fn, [conv(get(x, "f"), "f") for x in xs], "f")
+            if ot == "i":  # an operation without an integer form (div, pow ...): fp32, then back
+                r = out("f2i", [r], "i")
+            return r
 
         def resolve_alias(v: ir.Value) -> ir.Value:
             while v.node.pos in p.alias_nodes and v.node.pos in member_pos:
@@ -1620,6 +1720,7 @@ class _RowCodegen:
             prologue = []
             body: list[list] = []
             vreg_of: dict[Any, _VReg] = {}
+            conv_v.clear()
 
             # 1. reductions finished by the previous body
             for n in members:
@@ -1658,16 +1759,16 @@ class _RowCodegen:
                             stack.append(i2)
 
             # 3. row-scalar ops that become computable in this phase
-            def scalar_operand(x, emit_list):
+            def scalar_operand(x, t: str = "f"):
                 """Register of a row-class operand of a scalar op."""
                 if not isinstance(x, ir.Value):
-                    return scalar_imm(float(x))
+                    return scalar_imm(float(x), t)
                 if in_group(x):
                     x2 = resolve_alias(x)
                     return sreg_of[x2.id]
                 e = ext_operand(x)
                 if e[0] == "imm":
-                    return scalar_imm(e[1])
+                    return scalar_imm(e[1], e[2])
                 return scalar_ext(e[1])
 
             for n in members:
@@ -1678,11 +1779,7 @@ class _RowCodegen:
                     continue
                 if n.kind != "ew":
                     raise FusionLimit(f"row-class node of kind {n.kind}")
-                regs = [scalar_operand(x, prologue) for x in n.attrs["operands"]]
-                r = new_v("s")
-                sreg_of[o.id] = r
-                regs += [0] * (3 - len(regs))
-                prologue.append([isa.EW[n.fn], r, regs[0], regs[1], regs[2], 0])
+                sreg_of[o.id] = emit_ew(n, scalar_operand, prologue, "s")
             # stores of row values that became available in this phase
             for n in members:
                 o = n.outputs[0]
@@ -1691,9 +1788,9 @@ class _RowCodegen:
                     prologue.append([isa.STR, store_operand(o), sreg_of[o.id], 0, 0, 0])
 
             # 4. body: full-class ops in topological order
-            def vec_operand(x):
+            def vec_operand(x, t: str = "f"):
                 if not isinstance(x, ir.Value):
-                    return scalar_imm(float(x))
+                    return scalar_imm(float(x), t)
                 if in_group(x):
                     x2 = resolve_alias(x) if x.id not in vreg_of else x
                     if cls.get(x2.id) == "R":
@@ -1701,14 +1798,14 @@ class _RowCodegen:
                     return vreg_of[x2.id]
                 e = ext_operand(x)
                 if e[0] == "imm":
-                    return scalar_imm(e[1])
+                    return scalar_imm(e[1], e[2])
                 _, idx, c = e
                 if c in ("U", "R"):
                     return scalar_ext(idx)
                 key = ("op", idx)
                 r = vreg_of.get(key)
                 if r is None:
-                    r = new_v("v")
+                    r = new_v("v", _reg_type(operands[idx].dtype))
                     vreg_of[key] = r
                     body.append([isa.LDG, r, idx, 0, 0, 0])
                 return r
@@ -1718,7 +1815,7 @@ class _RowCodegen:
                 if n.kind == "reduce":
                     if ph[o.id] == phase:
                         x = n.inputs[0]
-                        src = vec_operand(x)
+                        src = as_type(vec_operand(x), "f", body)  # (accumulators are fp32)
                         if src.kind == "s":  # reducing a row scalar broadcast: materialise it
                             t = new_v("v")
                             body.append([isa.EW["mov"], t, src, 0, 0, 0])
@@ -1729,29 +1826,40 @@ class _RowCodegen:
                     continue
                 if n.pos in p.alias_nodes:
                     src = vec_operand(n.inputs[0])
-                    r = new_v("v")
+                    r = new_v("v", src.t)
                     body.append([isa.EW["mov"], r, src, 0, 0, 0])
                 elif n.kind == "ew":
-                    regs = [vec_operand(x) for x in n.attrs["operands"]]
-                    regs += [0] * (3 - len(regs))
-                    r = new_v("v")
-                    body.append([isa.EW[n.fn], r, regs[0], regs[1], regs[2], 0])
+                    r = emit_ew(n, vec_operand, body, "v")
                 elif n.kind == "tril":
                     lim = tril_setup(n)
                     x = vec_operand(n.inputs[0])
-                    zero = scalar_imm(0.0)
+                    zero = scalar_imm(0.0)  # (all bits clear: zero of either register type)
                     c = new_v("v")
                     body.append([isa.COLIDX, c, 0, 0, 0, 0])
                     m = new_v("v")
                     body.append([isa.EW["ge" if n.attrs["upper"] else "le"], m, c, lim, 0, 0])
-                    r = new_v("v")
+                    r = new_v("v", x.t)
                     body.append([isa.EW["where"], r, m, x, zero, 0])
                 elif n.kind == "iota":
-                    c = new_v("v")
-                    body.append([isa.COLIDX, c, 0, 0, 0, 0])
-                    r = new_v("v")
-                    body.append([isa.EW["fma"], r, c, scalar_imm(n.attrs["step"]),
-                                 scalar_imm(n.attrs["start"]), 0])
+                    start, step = n.attrs["start"], n.attrs["step"]
+                    if _reg_type(o.dtype) == "i" and start == int(start) and step == int(step):
+                        r = new_v("v", "i")
+                        body.append([isa.COLIDX, r, 1, 0, 0, 0])  # the column as an int32
+                        if step != 1:
+                            t = new_v("v", "i")
+                            body.append([isa.EW["imul"], t, r, scalar_imm(step, "i"), 0, 0])
+                            r = t
+                        if start != 0:
+                            t = new_v("v", "i")
+                            body.append([isa.EW["iadd"], t, r, scalar_imm(start, "i"), 0, 0])
+                            r = t
+                    else:
+                        c = new_v("v")
+                        body.append([isa.COLIDX, c, 0, 0, 0, 0])
+                        r = new_v("v")
+                        body.append([isa.EW["fma"], r, c, scalar_imm(n.attrs["step"]),
+                                     scalar_imm(n.attrs["start"]), 0])
+                        r = as_type(r, _reg_type(o.dtype), body)
                 else:
                     raise AssertionError(n.kind)
                 vreg_of[o.id] = r

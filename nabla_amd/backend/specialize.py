@@ -46,8 +46,8 @@ def program_bytes(a: dict) -> bytes:
                            o.stage_slot)
     for i in a["ins"]:
         out += struct.pack("<BBBBBBH", i[0], i[1], i[2], i[3], i[4], 0, i[5])
-    for v in a["imm"]:
-        out += struct.pack("<f", v)
+    for v in a["imm"]:  # (an int is an integer register's immediate: its bits)
+        out += struct.pack("<i", v) if isinstance(v, int) else struct.pack("<f", v)
     return out
 
 
@@ -87,7 +87,7 @@ def _ew_scalar(op: int, dst: int, a: int, b: int, c: int, lowp: bool = False) ->
     if name in isa.BINARY:
         return f"s{dst} = rp_binary{lp}({op}, s{a}, s{b});"
     if name == "where":
-        return f"s{dst} = s{a} != 0.f ? s{b} : s{c};"
+        return f"s{dst} = rp_where(s{a}, s{b}, s{c});"
     return f"s{dst} = fmaf(s{a}, s{b}, s{c});"
 
 
@@ -184,7 +184,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                 w(ind + f"  noff{k} = rp_row_offset(o{k}, nlead, 4);")
             w(ind + "}")
             for k in hoisted:
-                w(ind + f"nldr{k} = nbk_load_as_f32(o{k}.ptr, noff{k}, o{k}.dtype);")
+                w(ind + f"nldr{k} = rp_load1(o{k}.ptr, noff{k}, o{k}.dtype);")
             for k in inputs:
                 full_load = f"rp_load4(o{k}, noff{k}, colj[j], 4)"
                 if ops[k].dtype.abi == 0 and ops[k].vec_ok and ops[k].col_stride == 1:
@@ -228,7 +228,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         for k in hoisted:
             w(f"  const bool uni{k} = (o{k}.lead_stride[0] | o{k}.lead_stride[1] | o{k}.lead_stride[2] | "
               f"o{k}.lead_stride[3]) == 0;")
-            w(f"  const float pre{k} = uni{k} ? nbk_load_as_f32(o{k}.ptr, 0, o{k}.dtype) : 0.f;")
+            w(f"  const float pre{k} = uni{k} ? rp_load1(o{k}.ptr, 0, o{k}.dtype) : 0.f;")
         w("  const uint64_t stride = (uint64_t)gridDim.x * 256u;")
         w("  const bool small = total_chunks <= 0xffffffffull;  // 32-bit row arithmetic suffices")
         w("  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {")
@@ -248,7 +248,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
             for k in range(len(ops)):
                 w(f"    const int64_t off{k} = rp_row_offset(o{k}, lead_idx, 4);")
             for k in hoisted:
-                w(f"    const float ldr{k} = nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
+                w(f"    const float ldr{k} = rp_load1(o{k}.ptr, off{k}, o{k}.dtype);")
         else:
             # per-lane rows: with at most one leading dim an offset is one multiply-add
             w("    int64_t " + ", ".join(f"off{k}" for k in range(len(ops))) + ";")
@@ -260,7 +260,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                 w(f"      off{k} = rp_row_offset(o{k}, lead_idx, 4);")
             w("    }")
             for k in hoisted:
-                w(f"    const float ldr{k} = uni{k} ? pre{k} : nbk_load_as_f32(o{k}.ptr, off{k}, o{k}.dtype);")
+                w(f"    const float ldr{k} = uni{k} ? pre{k} : rp_load1(o{k}.ptr, off{k}, o{k}.dtype);")
         if block_mode and a["n_stage"] > 0:
             for k, o in enumerate(ops):
                 if o.stage_slot >= 0:
@@ -316,8 +316,7 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                 elif bop == isa.ACC:
                     w(ind + f"acc{bd} = rp_acc4(acc{bd}, {_as_vec(bx)}, {by}, valid);")
                 elif bop == isa.COLIDX:
-                    w(ind + f"v{bd} = make_float4((float)col, (float)col + 1.f, (float)col + 2.f, "
-                      "(float)col + 3.f);")
+                    w(ind + f"v{bd} = rp_colidx4(col, {'true' if bx else 'false'});")
                 else:
                     w(ind + _ew_vec(bop, bd, bx, by, bz, lowp))
             w("    }")
@@ -329,11 +328,11 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
             if x in hoisted:
                 w(f"    s{dst} = {hoisted[x]};")
             else:
-                w(f"    s{dst} = nbk_load_as_f32(o{x}.ptr, off{x}, o{x}.dtype);")
+                w(f"    s{dst} = rp_load1(o{x}.ptr, off{x}, o{x}.dtype);")
         elif op == isa.STR:
-            w(f"    if (writer) nbk_store_from_f32(o{dst}.ptr, off{dst}, o{dst}.dtype, s{x});")
+            w(f"    if (writer) rp_store1(o{dst}.ptr, off{dst}, o{dst}.dtype, s{x});")
         elif op == isa.LEADIDX:
-            w(f"    s{dst} = (float)lead_idx[{x}];")
+            w(f"    s{dst} = rp_ibits((int)lead_idx[{x}]);" if y else f"    s{dst} = (float)lead_idx[{x}];")
         elif op == isa.ACCINIT:
             w(f"    acc{dst} = rp_identity({x});")
         elif op == isa.RED:

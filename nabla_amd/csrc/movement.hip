@@ -277,6 +277,37 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
     }
   }
 }
+// Integer tensors: exact, with a 64-bit accumulator.  The same [outer, red, inner] layout and
+// strip of 64 columns per workgroup as above; the four waves split `red` and meet in LDS.
+__device__ __forceinline__ int64_t red_comb_i(int64_t a, int64_t b, int kind) {
+  return kind == NBK_RED_SUM ? a + b : (kind == NBK_RED_MAX ? (a > b ? a : b) : (a < b ? a : b));
+}
+__device__ __forceinline__ int64_t load_as_i64(const void* p, int64_t i, int dt) {
+  return dt == NBK_I64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
+}
+__global__ __launch_bounds__(256) void reduce_mid_int_kernel(const void* __restrict__ in,
+                                                             void* __restrict__ out, int dti, int dto,
+                                                             int64_t red, int64_t inner, int kind) {
+  __shared__ int64_t part[4][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t col = (int64_t)blockIdx.x * 64 + lane, o = blockIdx.y;
+  int64_t acc = kind == NBK_RED_SUM ? 0 : (kind == NBK_RED_MAX ? INT64_MIN : INT64_MAX);
+  if (col < inner) {
+    const int64_t base = o * red * inner + col;
+    for (int64_t r = w; r < red; r += 4) acc = red_comb_i(acc, load_as_i64(in, base + r * inner, dti), kind);
+  }
+  part[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && col < inner) {
+    const int64_t v = red_comb_i(red_comb_i(part[0][lane], part[1][lane], kind),
+                                 red_comb_i(part[2][lane], part[3][lane], kind), kind);
+    const int64_t at = o * inner + col;
+    if (dto == NBK_I64) ((int64_t*)out)[at] = v;
+    else if (dto == NBK_I32) ((int32_t*)out)[at] = (int32_t)v;
+    else nbk_store_from_f32(out, at, dto, (float)v);
+  }
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void reduce_mid_vec_kernel(const T* __restrict__ in,
                                                              void* __restrict__ out, int dto,
@@ -316,13 +347,35 @@ __global__ __launch_bounds__(256) void reduce_batch_kernel(const ReduceBatchArgs
 // how reductions are grouped into launches.)
 static int reduce_waves_across(int64_t chunks) { return chunks >= 256 ? 4 : (chunks >= 128 ? 2 : 1); }
 
+static int reduce_mid_slab(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
+                           int64_t red, int64_t inner, int32_t kind, void* stream);
+
 extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
                               int64_t red, int64_t inner, int32_t kind, void* stream) {
   NBK_REQUIRE(in && out, "reduce_mid: null pointer");
   NBK_REQUIRE(outer > 0 && red > 0 && inner > 0, "reduce_mid: empty extent");
   NBK_REQUIRE(kind >= NBK_RED_SUM && kind <= NBK_RED_MIN, "reduce_mid: kind %d", kind);
   NBK_REQUIRE(nbk_dtype_size(dti) > 0 && nbk_dtype_size(dto) > 0, "reduce_mid: bad dtype");
-  NBK_REQUIRE(outer <= 65535, "reduce_mid: outer %lld exceeds the grid limit", (long long)outer);
+  // `outer` rides on the grid's second dimension (65535 at most): longer ones go in slabs
+  const int64_t kSlab = 65535;
+  for (int64_t o0 = 0; o0 < outer; o0 += kSlab) {
+    const int64_t n = outer - o0 < kSlab ? outer - o0 : kSlab;
+    const int rc = reduce_mid_slab((const char*)in + o0 * red * inner * nbk_dtype_size(dti),
+                                   (char*)out + o0 * inner * nbk_dtype_size(dto), dti, dto, n, red,
+                                   inner, kind, stream);
+    if (rc != NBK_OK) return rc;
+  }
+  return NBK_OK;
+}
+
+static int reduce_mid_slab(const void* in, void* out, int32_t dti, int32_t dto, int64_t outer,
+                           int64_t red, int64_t inner, int32_t kind, void* stream) {
+  if (dti == NBK_I32 || dti == NBK_I64) {
+    dim3 grid((unsigned)((inner + 63) / 64), (unsigned)outer);
+    hipLaunchKernelGGL(reduce_mid_int_kernel, grid, dim3(256), 0, (hipStream_t)stream, in, out, dti,
+                       dto, red, inner, kind);
+    return nbk_check_launch("reduce_mid_int_kernel");
+  }
   const bool aligned = ((uintptr_t)in & 15) == 0;
   if (dti == NBK_BF16 && inner % 8 == 0 && aligned) {
     const int wc = reduce_waves_across(inner / 8);
@@ -346,6 +399,28 @@ extern "C" int nbk_reduce_mid(const void* in, void* out, int32_t dti, int32_t dt
 
 extern "C" int nbk_reduce_mid_batch(const nbk_reduce_task* tasks, int32_t n, void* stream) {
   NBK_REQUIRE(tasks != nullptr && n > 0, "reduce_mid_batch: no tasks");
+  for (int32_t i = 0; i < n; ++i)
+    if (tasks[i].dtype_in == NBK_I32 || tasks[i].dtype_in == NBK_I64) {
+      // integer tensors take the exact kernel, one launch each; the float ones share launches
+      int32_t n_float = 0;
+      nbk_reduce_task rest[NBK_REDUCE_BATCH_MAX];
+      for (int32_t j = 0; j < n; ++j) {
+        const nbk_reduce_task& t = tasks[j];
+        if (t.dtype_in == NBK_I32 || t.dtype_in == NBK_I64) {
+          const int rc = nbk_reduce_mid(t.in, t.out, t.dtype_in, t.dtype_out, t.outer, t.red, t.inner,
+                                        t.kind, stream);
+          if (rc != NBK_OK) return rc;
+        } else {
+          rest[n_float++] = t;
+          if (n_float == NBK_REDUCE_BATCH_MAX) {
+            const int rc = nbk_reduce_mid_batch(rest, n_float, stream);
+            if (rc != NBK_OK) return rc;
+            n_float = 0;
+          }
+        }
+      }
+      return n_float > 0 ? nbk_reduce_mid_batch(rest, n_float, stream) : NBK_OK;
+    }
   for (int32_t base = 0; base < n; base += NBK_REDUCE_BATCH_MAX) {
     ReduceBatchArgs B;
     B.n = n - base < NBK_REDUCE_BATCH_MAX ? n - base : NBK_REDUCE_BATCH_MAX;

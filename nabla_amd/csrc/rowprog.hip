@@ -52,7 +52,13 @@ __device__ __forceinline__ nbk_operand rp_operand(const nbk_rowprog& S, int i, i
 
 __host__ __device__ __forceinline__ bool rp_is_unary(int op) {
   return (op >= NBK_OP_MOV && op < NBK_OP_ADD) || op == NBK_OP_DGELU || op == NBK_OP_SIN ||
-         op == NBK_OP_COS;
+         op == NBK_OP_COS || (op >= NBK_OP_INEG && op <= NBK_OP_INEZ);
+}
+__host__ __device__ __forceinline__ bool rp_is_binary(int op) {
+  return (op >= NBK_OP_ADD && op < NBK_OP_WHERE) || (op >= NBK_OP_IADD && op <= NBK_OP_ILE);
+}
+__host__ __device__ __forceinline__ bool rp_is_ew(int op) {
+  return rp_is_unary(op) || rp_is_binary(op) || op == NBK_OP_WHERE || op == NBK_OP_FMA;
 }
 
 // One body instruction on one chunk.
@@ -61,7 +67,7 @@ __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins
                                              const IDX* lead_idx, int64_t col, int valid,
                                              const float* stage, int64_t c_pad, int n_lead) {
   const int op = in.op;
-  if (op >= NBK_OP_ADD && op < NBK_OP_WHERE) {
+  if (rp_is_binary(op)) {
     float4 a = rp_read(R, in.a), b = rp_read(R, in.b), r;
     switch (op) {  // the hot ones without a per-component switch
       case NBK_OP_ADD: r = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); break;
@@ -100,15 +106,13 @@ __device__ __forceinline__ void rp_exec_body(const nbk_rowprog& P, const nbk_ins
     R.acc[in.dst] = v;
   } else if (op == NBK_OP_WHERE) {
     float4 c = rp_read(R, in.a), a = rp_read(R, in.b), b = rp_read(R, in.c);
-    rp_write(R, in.dst, make_float4(c.x != 0.f ? a.x : b.x, c.y != 0.f ? a.y : b.y,
-                                    c.z != 0.f ? a.z : b.z, c.w != 0.f ? a.w : b.w));
+    rp_write(R, in.dst, rp_where4(c, a, b));
   } else if (op == NBK_OP_FMA) {
     float4 a = rp_read(R, in.a), b = rp_read(R, in.b), c = rp_read(R, in.c);
     rp_write(R, in.dst, make_float4(fmaf(a.x, b.x, c.x), fmaf(a.y, b.y, c.y),
                                     fmaf(a.z, b.z, c.z), fmaf(a.w, b.w, c.w)));
   } else if (op == NBK_OP_COLIDX) {
-    float c0 = (float)col;
-    rp_write(R, in.dst, make_float4(c0, c0 + 1.f, c0 + 2.f, c0 + 3.f));
+    rp_write(R, in.dst, rp_colidx4(col, in.a != 0));
   }
 }
 
@@ -123,26 +127,26 @@ __device__ __forceinline__ void rp_exec_scalar(const nbk_rowprog& P, const nbk_i
     R.s[d] = __uint_as_float(rp_sgpr(__float_as_uint(P.imm[in.a])));
   } else if (op == NBK_OP_LDR) {
     const nbk_operand o = rp_operand(P, in.a, n_lead);
-    R.s[d] = nbk_load_as_f32(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype);
+    R.s[d] = rp_load1(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype);
   } else if (op == NBK_OP_STR) {
     const nbk_operand o = rp_operand(P, in.dst, n_lead);
     if (writer) {
-      nbk_store_from_f32(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype,
-                         R.s[in.a - NBK_RP_NVEC]);
+      rp_store1(o.ptr, rp_row_offset(o, lead_idx, n_lead), o.dtype, R.s[in.a - NBK_RP_NVEC]);
     }
   } else if (op == NBK_OP_LEADIDX) {
     const int k = in.a;
-    R.s[d] = (float)(k == 0 ? lead_idx[0] : k == 1 ? lead_idx[1] : k == 2 ? lead_idx[2] : lead_idx[3]);
+    const int li = (int)(k == 0 ? lead_idx[0] : k == 1 ? lead_idx[1] : k == 2 ? lead_idx[2] : lead_idx[3]);
+    R.s[d] = in.b != 0 ? rp_ibits(li) : (float)li;
   } else if (op == NBK_OP_ACCINIT) {
     R.acc[in.dst] = rp_identity(in.a);
   } else if (op == NBK_OP_RED) {
     R.s[d] = rp_block_reduce(R.acc[in.a], in.b, red_buf);
-  } else if (op >= NBK_OP_ADD && op < NBK_OP_WHERE) {
+  } else if (rp_is_binary(op)) {
     R.s[d] = rp_binary(op, R.s[in.a - NBK_RP_NVEC], R.s[in.b - NBK_RP_NVEC]);
   } else if (rp_is_unary(op)) {
     R.s[d] = rp_unary(op, R.s[in.a - NBK_RP_NVEC]);
   } else if (op == NBK_OP_WHERE) {
-    R.s[d] = R.s[in.a - NBK_RP_NVEC] != 0.f ? R.s[in.b - NBK_RP_NVEC] : R.s[in.c - NBK_RP_NVEC];
+    R.s[d] = rp_where(R.s[in.a - NBK_RP_NVEC], R.s[in.b - NBK_RP_NVEC], R.s[in.c - NBK_RP_NVEC]);
   } else if (op == NBK_OP_FMA) {
     R.s[d] = fmaf(R.s[in.a - NBK_RP_NVEC], R.s[in.b - NBK_RP_NVEC], R.s[in.c - NBK_RP_NVEC]);
   }
@@ -379,7 +383,7 @@ static int rp_validate(const nbk_rowprog* p) {
                       "rowprog: bad ACC at %d", q);
         } else if (op == NBK_OP_COLIDX) {
           NBK_REQUIRE(b.dst < NBK_RP_NVEC, "rowprog: bad COLIDX at %d", q);
-        } else if ((op >= NBK_OP_MOV && op <= NBK_OP_FMA) || rp_is_unary(op)) {
+        } else if (rp_is_ew(op)) {
           NBK_REQUIRE(b.dst < NBK_RP_NVEC && b.a < 32 && b.b < 32 && b.c < 32,
                       "rowprog: bad register at %d", q);
         } else {
@@ -405,12 +409,12 @@ static int rp_validate(const nbk_rowprog* p) {
     } else if (op == NBK_OP_RED) {
       NBK_REQUIRE(p->has_reduce && sreg_dst && in.a < NBK_RP_NACC && in.b <= NBK_RED_MIN,
                   "rowprog: bad RED at %d", pc);
-    } else if ((op >= NBK_OP_MOV && op <= NBK_OP_FMA) || rp_is_unary(op)) {
+    } else if (rp_is_ew(op)) {
       NBK_REQUIRE(sreg_dst && in.a >= NBK_RP_NVEC && in.a < 32, "rowprog: bad scalar op at %d",
                   pc);
-      if (op >= NBK_OP_ADD && !rp_is_unary(op))
+      if (!rp_is_unary(op))
         NBK_REQUIRE(in.b >= NBK_RP_NVEC && in.b < 32, "rowprog: bad scalar op at %d", pc);
-      if (op >= NBK_OP_WHERE && !rp_is_unary(op))
+      if (op == NBK_OP_WHERE || op == NBK_OP_FMA)
         NBK_REQUIRE(in.c >= NBK_RP_NVEC && in.c < 32, "rowprog: bad scalar op at %d", pc);
     } else {
       NBK_REQUIRE(false, "rowprog: opcode %d not allowed in a prologue (at %d)", op, pc);

@@ -28,6 +28,25 @@ __device__ __forceinline__ void rp_store4_stream(float* p, float4 r) {
   __builtin_nontemporal_store(v, (rp_vf4*)p);
 }
 
+// Registers are 32 bits wide and typed by the program, not by the hardware: a value of an
+// integer tensor (int32, int64) is held as a two's-complement int32 in the register's bits and
+// computed with the integer instructions, so integers are exact over the whole int32 range
+// (int64 storage is read and written through its low 32 bits, sign-extended on the way out);
+// everything else -- floats, and bool / uint8 as 0.0, 1.0, ... -- is held as fp32.
+__device__ __forceinline__ float rp_ibits(int v) { return __int_as_float(v); }
+__device__ __forceinline__ int rp_int(float v) { return __float_as_int(v); }
+
+__device__ __forceinline__ float rp_load1(const void* p, int64_t i, int dt) {
+  if (dt == NBK_I32) return rp_ibits(((const int32_t*)p)[i]);
+  if (dt == NBK_I64) return rp_ibits((int)((const int64_t*)p)[i]);
+  return nbk_load_as_f32(p, i, dt);
+}
+__device__ __forceinline__ void rp_store1(void* p, int64_t i, int dt, float v) {
+  if (dt == NBK_I32) ((int32_t*)p)[i] = rp_int(v);
+  else if (dt == NBK_I64) ((int64_t*)p)[i] = (int64_t)rp_int(v);
+  else nbk_store_from_f32(p, i, dt, v);
+}
+
 __device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, int64_t col,
                                            int valid) {
   const int dt = o.dtype;
@@ -50,12 +69,11 @@ __device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, in
       float2 fa = __half22float2(a), fb = __half22float2(b);
       r = make_float4(fa.x, fa.y, fb.x, fb.y);
     } else if (dt == NBK_I32) {
-      int4 u = *(const int4*)((const int32_t*)o.ptr + e);
-      r = make_float4((float)u.x, (float)u.y, (float)u.z, (float)u.w);
+      r = *(const float4*)((const int32_t*)o.ptr + e);  // the bits as they are
     } else if (dt == NBK_I64) {
       const int64_t* p = (const int64_t*)o.ptr + e;
       longlong2 u0 = *(const longlong2*)p, u1 = *(const longlong2*)(p + 2);
-      r = make_float4((float)u0.x, (float)u0.y, (float)u1.x, (float)u1.y);
+      r = make_float4(rp_ibits((int)u0.x), rp_ibits((int)u0.y), rp_ibits((int)u1.x), rp_ibits((int)u1.y));
     } else {
       uint32_t u = *(const uint32_t*)((const uint8_t*)o.ptr + e);
       r = make_float4((float)(u & 0xff), (float)((u >> 8) & 0xff), (float)((u >> 16) & 0xff),
@@ -64,14 +82,14 @@ __device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, in
     return r;
   }
   const int64_t e0 = off + col * cs;
-  if (valid > 0) r.x = nbk_load_as_f32(o.ptr, e0, dt);
+  if (valid > 0) r.x = rp_load1(o.ptr, e0, dt);
   if (cs == 0) {
     r.y = r.z = r.w = r.x;
     return r;
   }
-  if (valid > 1) r.y = nbk_load_as_f32(o.ptr, e0 + cs, dt);
-  if (valid > 2) r.z = nbk_load_as_f32(o.ptr, e0 + 2 * cs, dt);
-  if (valid > 3) r.w = nbk_load_as_f32(o.ptr, e0 + 3 * cs, dt);
+  if (valid > 1) r.y = rp_load1(o.ptr, e0 + cs, dt);
+  if (valid > 2) r.z = rp_load1(o.ptr, e0 + 2 * cs, dt);
+  if (valid > 3) r.w = rp_load1(o.ptr, e0 + 3 * cs, dt);
   return r;
 }
 
@@ -95,10 +113,11 @@ __device__ __forceinline__ void rp_store4(const nbk_operand& o, int64_t off, int
       u.y = *(uint32_t*)&b;
       *(uint2*)((__half*)o.ptr + e) = u;
     } else if (dt == NBK_I32) {
-      *(int4*)((int32_t*)o.ptr + e) = make_int4((int)v.x, (int)v.y, (int)v.z, (int)v.w);
+      *(float4*)((int32_t*)o.ptr + e) = v;
     } else if (dt == NBK_I64) {
-      int64_t* p = (int64_t*)o.ptr + e;
-      p[0] = (int64_t)v.x; p[1] = (int64_t)v.y; p[2] = (int64_t)v.z; p[3] = (int64_t)v.w;
+      longlong2* p = (longlong2*)((int64_t*)o.ptr + e);
+      p[0] = make_longlong2((int64_t)rp_int(v.x), (int64_t)rp_int(v.y));
+      p[1] = make_longlong2((int64_t)rp_int(v.z), (int64_t)rp_int(v.w));
     } else {
       uint32_t u = (uint32_t)(v.x != 0.f) | ((uint32_t)(v.y != 0.f) << 8) |
                    ((uint32_t)(v.z != 0.f) << 16) | ((uint32_t)(v.w != 0.f) << 24);
@@ -107,10 +126,10 @@ __device__ __forceinline__ void rp_store4(const nbk_operand& o, int64_t off, int
     return;
   }
   const int64_t e0 = off + col * cs;
-  if (valid > 0) nbk_store_from_f32(o.ptr, e0, dt, v.x);
-  if (valid > 1) nbk_store_from_f32(o.ptr, e0 + cs, dt, v.y);
-  if (valid > 2) nbk_store_from_f32(o.ptr, e0 + 2 * cs, dt, v.z);
-  if (valid > 3) nbk_store_from_f32(o.ptr, e0 + 3 * cs, dt, v.w);
+  if (valid > 0) rp_store1(o.ptr, e0, dt, v.x);
+  if (valid > 1) rp_store1(o.ptr, e0 + cs, dt, v.y);
+  if (valid > 2) rp_store1(o.ptr, e0 + 2 * cs, dt, v.z);
+  if (valid > 3) rp_store1(o.ptr, e0 + 3 * cs, dt, v.w);
 }
 
 // ---- elementwise functions --------------------------------------------------
@@ -139,6 +158,13 @@ __device__ __forceinline__ float rp_unary(int op, float a) {
     case NBK_OP_NOT: return a != 0.0f ? 0.0f : 1.0f;
     case NBK_OP_TRUNC: return truncf(a);
     case NBK_OP_NEZ: return a != 0.0f ? 1.0f : 0.0f;
+    // integer registers
+    case NBK_OP_INEG: return rp_ibits(-rp_int(a));
+    case NBK_OP_IABS: return rp_ibits(rp_int(a) < 0 ? -rp_int(a) : rp_int(a));
+    case NBK_OP_IRELU: return rp_ibits(rp_int(a) > 0 ? rp_int(a) : 0);
+    case NBK_OP_I2F: return (float)rp_int(a);
+    case NBK_OP_F2I: return rp_ibits((int)a);
+    case NBK_OP_INEZ: return rp_int(a) != 0 ? 1.0f : 0.0f;
     default: return a;
   }
 }
@@ -159,6 +185,18 @@ __device__ __forceinline__ float rp_binary(int op, float a, float b) {
     case NBK_OP_POW: return powf(a, b);
     case NBK_OP_AND: return (a != 0.0f && b != 0.0f) ? 1.0f : 0.0f;
     case NBK_OP_OR: return (a != 0.0f || b != 0.0f) ? 1.0f : 0.0f;
+    // integer registers (wrap-around arithmetic; comparisons give a float 0 / 1)
+    case NBK_OP_IADD: return rp_ibits((int)((uint32_t)rp_int(a) + (uint32_t)rp_int(b)));
+    case NBK_OP_ISUB: return rp_ibits((int)((uint32_t)rp_int(a) - (uint32_t)rp_int(b)));
+    case NBK_OP_IMUL: return rp_ibits((int)((uint32_t)rp_int(a) * (uint32_t)rp_int(b)));
+    case NBK_OP_IMAX: return rp_ibits(rp_int(a) > rp_int(b) ? rp_int(a) : rp_int(b));
+    case NBK_OP_IMIN: return rp_ibits(rp_int(a) < rp_int(b) ? rp_int(a) : rp_int(b));
+    case NBK_OP_IGT: return rp_int(a) > rp_int(b) ? 1.0f : 0.0f;
+    case NBK_OP_IGE: return rp_int(a) >= rp_int(b) ? 1.0f : 0.0f;
+    case NBK_OP_IEQ: return rp_int(a) == rp_int(b) ? 1.0f : 0.0f;
+    case NBK_OP_INE: return rp_int(a) != rp_int(b) ? 1.0f : 0.0f;
+    case NBK_OP_ILT: return rp_int(a) < rp_int(b) ? 1.0f : 0.0f;
+    case NBK_OP_ILE: return rp_int(a) <= rp_int(b) ? 1.0f : 0.0f;
     default: return a;
   }
 }
@@ -314,9 +352,22 @@ __device__ __forceinline__ float4 rp_bin4(float4 a, float4 b) {
   return make_float4(rp_binary(OP, a.x, b.x), rp_binary(OP, a.y, b.y), rp_binary(OP, a.z, b.z),
                      rp_binary(OP, a.w, b.w));
 }
+// The choice moves register bits, whatever they hold.
+__device__ __forceinline__ float rp_where(float c, float a, float b) {
+  return rp_ibits(c != 0.f ? rp_int(a) : rp_int(b));
+}
 __device__ __forceinline__ float4 rp_where4(float4 c, float4 a, float4 b) {
-  return make_float4(c.x != 0.f ? a.x : b.x, c.y != 0.f ? a.y : b.y, c.z != 0.f ? a.z : b.z,
-                     c.w != 0.f ? a.w : b.w);
+  return make_float4(rp_where(c.x, a.x, b.x), rp_where(c.y, a.y, b.y), rp_where(c.z, a.z, b.z),
+                     rp_where(c.w, a.w, b.w));
+}
+// Column indices col .. col + 3 as floats or, for an integer register, as int32.
+__device__ __forceinline__ float4 rp_colidx4(int64_t col, bool as_int) {
+  if (as_int) {
+    const int c0 = (int)col;
+    return make_float4(rp_ibits(c0), rp_ibits(c0 + 1), rp_ibits(c0 + 2), rp_ibits(c0 + 3));
+  }
+  const float c0 = (float)col;
+  return make_float4(c0, c0 + 1.f, c0 + 2.f, c0 + 3.f);
 }
 __device__ __forceinline__ float4 rp_fma4(float4 a, float4 b, float4 c) {
   return make_float4(fmaf(a.x, b.x, c.x), fmaf(a.y, b.y, c.y), fmaf(a.z, b.z, c.z),

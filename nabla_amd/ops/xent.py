@@ -25,9 +25,8 @@ F32 = DType.float32
 
 def _label_mask(labels: ir.Value, full_shape) -> ir.Value:
     """1.0 where the column index equals the row's label, else 0.0 (never stored)."""
-    classes = ir.iota(full_shape[-1], F32, lead=full_shape[:-1])
-    # (integer labels are compared as they are: operands of a row program are widened to fp32 in
-    # registers, exact for class counts below 2^24)
+    # (an integer column index against the integer label: an exact comparison in int32 registers)
+    classes = ir.iota(full_shape[-1], labels.dtype, lead=full_shape[:-1])
     lab = ir.broadcast_to(ir.reshape(labels, tuple(labels.shape) + (1,)), full_shape)
     return ir.cast(ir.ew("eq", lab, classes), F32)
 

@@ -67,6 +67,52 @@ _BINARY = {
 }
 
 
+# Integer registers: values of int32 / int64 tensors are held as int32 in the 32 bits of a
+# register (here: in the bytes of a float32 array) and computed with the integer forms below.
+_I32 = np.int32
+
+
+def _ibits(a) -> np.ndarray:
+    """float32 array -> the int32 values its bytes hold."""
+    return np.ascontiguousarray(a, dtype=_F32).view(_I32)
+
+
+def _fbits(i) -> np.ndarray:
+    """int values (wrapped to int32) -> float32 array with those bytes."""
+    return np.ascontiguousarray(np.asarray(i).astype(_I32)).view(_F32)
+
+
+_UNARY.update({
+    "ineg": lambda a: _fbits(-_ibits(a)),
+    "iabs": lambda a: _fbits(np.abs(_ibits(a))),
+    "irelu": lambda a: _fbits(np.maximum(_ibits(a), 0)),
+    "i2f": lambda a: _ibits(a).astype(_F32),
+    "f2i": lambda a: _fbits(np.trunc(np.nan_to_num(a.astype(np.float64))).clip(-2.0 ** 31, 2.0 ** 31 - 1)
+                            .astype(np.int64)),
+    "inez": lambda a: (_ibits(a) != 0).astype(_F32),
+})
+_BINARY.update({
+    "iadd": lambda a, b: _fbits(_ibits(a).astype(np.int64) + _ibits(b)),
+    "isub": lambda a, b: _fbits(_ibits(a).astype(np.int64) - _ibits(b)),
+    "imul": lambda a, b: _fbits(_ibits(a).astype(np.int64) * _ibits(b)),
+    "imax": lambda a, b: _fbits(np.maximum(_ibits(a), _ibits(b))),
+    "imin": lambda a, b: _fbits(np.minimum(_ibits(a), _ibits(b))),
+    "igt": lambda a, b: (_ibits(a) > _ibits(b)).astype(_F32),
+    "ige": lambda a, b: (_ibits(a) >= _ibits(b)).astype(_F32),
+    "ieq": lambda a, b: (_ibits(a) == _ibits(b)).astype(_F32),
+    "ine": lambda a, b: (_ibits(a) != _ibits(b)).astype(_F32),
+    "ilt": lambda a, b: (_ibits(a) < _ibits(b)).astype(_F32),
+    "ile": lambda a, b: (_ibits(a) <= _ibits(b)).astype(_F32),
+})
+
+
+def _load_reg(t: torch.Tensor) -> np.ndarray:
+    """Elements of an operand as register contents."""
+    if t.dtype in (torch.int32, torch.int64):
+        return _fbits(t.numpy())
+    return _as_f32(t)
+
+
 def _as_f32(t: torch.Tensor) -> np.ndarray:
     if t.dtype == torch.bfloat16 or t.dtype == torch.float16:
         return t.float().numpy()
@@ -77,11 +123,13 @@ def _as_f32(t: torch.Tensor) -> np.ndarray:
 
 def _store(flat: torch.Tensor, idx: np.ndarray, vals: np.ndarray) -> None:
     """flat[idx] = vals with the destination's rounding."""
+    if flat.dtype in (torch.int32, torch.int64):  # an integer register: its bits are the value
+        v = torch.from_numpy(_ibits(vals).copy()).to(flat.dtype)
+        flat[torch.from_numpy(idx.reshape(-1))] = v.reshape(-1)
+        return
     v = torch.from_numpy(np.ascontiguousarray(vals.astype(_F32)))
     if flat.dtype == torch.bool:
         v = v != 0
-    elif flat.dtype in (torch.int32, torch.int64):
-        v = v.to(flat.dtype)  # truncation, as the kernel's float->int conversion
     else:
         v = v.to(flat.dtype)
     flat[torch.from_numpy(idx.reshape(-1))] = v.reshape(-1)
@@ -126,7 +174,7 @@ def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
                 if bop == isa.LDG:
                     o = ops[bx]
                     idx = row_off(o)[:, None] + cols[None, :] * o.col_stride
-                    V[bd] = _as_f32(mem[o.buf][torch.from_numpy(idx.reshape(-1))]).reshape(R, C)
+                    V[bd] = _load_reg(mem[o.buf][torch.from_numpy(idx.reshape(-1))]).reshape(R, C)
                 elif bop == isa.STG:
                     o = ops[bd]
                     idx = row_off(o)[:, None] + cols[None, :] * o.col_stride
@@ -137,7 +185,8 @@ def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
                     part = red(v, axis=1).astype(_F32)
                     ACC[bd] = {0: np.add, 1: np.maximum, 2: np.minimum}[by](ACC[bd], part).astype(_F32)
                 elif bop == isa.COLIDX:
-                    V[bd] = np.broadcast_to(cols.astype(_F32)[None, :], (R, C)).copy()
+                    as_reg = _fbits(cols) if bx else cols.astype(_F32)
+                    V[bd] = np.broadcast_to(as_reg[None, :], (R, C)).copy()
                 elif bop in isa.EW_NAME:
                     name = isa.EW_NAME[bop]
                     with np.errstate(all="ignore"):
@@ -146,7 +195,7 @@ def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
                         elif name in _BINARY:
                             r = _BINARY[name](rd(bx).astype(_F32), rd(by).astype(_F32))
                         elif name == "where":
-                            r = np.where(rd(bx) != 0, rd(by), rd(bz))
+                            r = _fbits(np.where(rd(bx) != 0, _ibits(rd(by)), _ibits(rd(bz))))  # moves bits
                         else:  # fma
                             r = (rd(bx).astype(np.float64) * rd(by) + rd(bz))
                     V[bd] = np.broadcast_to(np.asarray(r, dtype=_F32), (R, C)).copy()
@@ -155,15 +204,15 @@ def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
             pc += 1 + aux
             continue
         if op == isa.IMM:
-            S[dst] = np.full(R, imm[x], dtype=_F32)
+            S[dst] = _fbits(np.full(R, imm[x])) if isinstance(imm[x], int) else np.full(R, imm[x], dtype=_F32)
         elif op == isa.LDR:
             o = ops[x]
-            S[dst] = _as_f32(mem[o.buf][torch.from_numpy(row_off(o))])
+            S[dst] = _load_reg(mem[o.buf][torch.from_numpy(row_off(o))])
         elif op == isa.STR:
             o = ops[dst]
             _store(mem[o.buf], row_off(o), rs(x))
         elif op == isa.LEADIDX:
-            S[dst] = lead_idx[x].astype(_F32)
+            S[dst] = _fbits(lead_idx[x]) if y else lead_idx[x].astype(_F32)
         elif op == isa.ACCINIT:
             ACC[dst] = np.full(R, {0: 0.0, 1: -np.inf, 2: np.inf}[x], dtype=_F32)
         elif op == isa.RED:
@@ -176,7 +225,7 @@ def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
                 elif name in _BINARY:
                     S[dst] = np.asarray(_BINARY[name](rs(x), rs(y)), dtype=_F32)
                 elif name == "where":
-                    S[dst] = np.where(rs(x) != 0, rs(y), rs(z)).astype(_F32)
+                    S[dst] = _fbits(np.where(rs(x) != 0, _ibits(rs(y)), _ibits(rs(z))))
                 else:
                     S[dst] = (rs(x).astype(np.float64) * rs(y) + rs(z)).astype(_F32)
         else:
@@ -405,6 +454,14 @@ class EmulatedPlan:
             elif k in ("reduce_mid", "reduce_batch"):
                 for t in ([a] if k == "reduce_mid" else a["tasks"]):
                     src = mem[t["src"].buf][t["src"].offset:t["src"].offset + t["outer"] * t["red"] * t["inner"]]
+                    if src.dtype in (torch.int32, torch.int64):  # exact, 64-bit accumulator
+                        xi = src.numpy().astype(np.int64).reshape(t["outer"], t["red"], t["inner"])
+                        ri = {"sum": xi.sum(axis=1), "max": xi.max(axis=1), "min": xi.min(axis=1)}[t["fn"]]
+                        d = t["dst"]
+                        flat = mem[d.buf]
+                        vals = torch.from_numpy(ri.reshape(-1))
+                        flat[d.offset:d.offset + vals.numel()] = vals.to(flat.dtype)
+                        continue
                     x = _as_f32(src).reshape(t["outer"], t["red"], t["inner"])
                     r = {"sum": x.sum(axis=1, dtype=np.float64), "max": x.max(axis=1), "min": x.min(axis=1)}[t["fn"]]
                     d = t["dst"]

@@ -624,3 +624,9 @@ def _check_gelu_fold(engine, O):
     np.testing.assert_allclose(y.numpy(), O.gelu(O.matmul(O.V(x), O.V(w)) + O.V(b)).a, rtol=1e-5, atol=1e-6)
     plan = list(engine._PLAN_CACHE.values())[-1].plan
     assert [st.kind for st in plan.steps] == ["gemm"] and plan.steps[0].attrs.get("aux_dst") is None
+
+
+def test_integers_above_2_pow_24_are_exact(emulator):
+    """Integer tensors compute in integer registers: no value passes through fp32."""
+    from integer_cases import check_large_integers
+    check_large_integers(nb)

@@ -265,6 +265,12 @@ def test_integer_and_bool_elementwise_exact(hip):
     np.testing.assert_array_equal(nb.reduce_sum(T(a), axis=1).numpy(), a.sum(1))
 
 
+def test_integers_above_2_pow_24_are_exact(hip):
+    """The same cases as the emulator-backed host test, on the kernels."""
+    from integer_cases import check_large_integers
+    check_large_integers(nb)
+
+
 def test_slice_pad_concat_exact(hip):
     rng = np.random.default_rng(9)
     a = rng.standard_normal((6, 10, 12)).astype(np.float32)
