@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 17
+#define NBK_ABI_VERSION 18
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -434,6 +434,27 @@ typedef int (*nbk_custom_fn)(const nbk_tensor* in, int n_in, nbk_tensor* out,
                              int n_out, void* stream);
 int nbk_custom(const char* library_path, const char* name, const nbk_tensor* in,
                int n_in, nbk_tensor* out, int n_out, void* stream);
+
+/* ===================================================================== */
+/*  Random tensors                                                        */
+/* ===================================================================== */
+/* The reference's uniform / gaussian (nabla/ops/creation.py:152-183, 462-520) and the dropout
+ * mask built on them (nabla/nn/functional/layers.py:64-76: uniform(shape) > p) draw from MAX's
+ * generator and thread a seed value through every compiled graph (core/graph/engine.py:80,
+ * 610-611).  Here the generator is Philox4x32-10 and the state is two int64 in device memory
+ * owned by the caller: state[0] the seed, state[1] the number of steps drawn so far.  Element i
+ * of a tensor is word i % 4 of the block with counter (i / 4 low, i / 4 high, stream_id,
+ * state[1] low) and key (seed low, seed high): `stream_id` tells the random tensors of one step
+ * apart, nbk_rng_advance (state[1] += 1, as a kernel, so that it can be part of a recorded
+ * sequence) goes once at the end of a step that drew numbers.
+ *   NBK_RANDOM_UNIFORM: a + (b - a) u,  u = (word >> 8) 2^-24 in [0, 1)
+ *   NBK_RANDOM_NORMAL:  a + b z, Box-Muller on the word pairs (0, 1) and (2, 3) of a block
+ *   NBK_RANDOM_KEEP:    u > a as 1 / 0 (the keep mask of dropout with rate a); also into bool
+ * dtype: NBK_F32, NBK_BF16, NBK_F16 (NBK_U8 for KEEP). */
+enum nbk_random_mode { NBK_RANDOM_UNIFORM = 0, NBK_RANDOM_NORMAL = 1, NBK_RANDOM_KEEP = 2 };
+int nbk_random(void* out, int32_t dtype, int64_t n, int32_t mode, float a, float b,
+               const int64_t* state, uint32_t stream_id, void* stream);
+int nbk_rng_advance(int64_t* state, void* stream);
 
 /* ===================================================================== */
 /*  Optimizer updates, all parameters in one launch                       */

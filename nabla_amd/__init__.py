@@ -8,7 +8,7 @@ transformer / CNN / LoRA examples, ``grad`` / ``value_and_grad`` / ``vjp`` /
 from . import config
 from .core import (CPU, GRAPH, Accelerator, Device, DType, OpNode, PyTreeDef, Tensor, TensorImpl,
                    Trace, default_device, default_dtype, defaults, defaults_like, get_cache_stats,
-                   is_tensor, realize_all, register_pytree_node, tensor_leaves, trace,
+                   is_tensor, realize_all, register_pytree_node, set_seed, tensor_leaves, trace,
                    tree_flatten, tree_leaves, tree_map, tree_structure, tree_unflatten)
 from .core.backward import backward, backward_on_trace
 from .ops import *  # noqa: F401,F403

@@ -19,7 +19,7 @@ from typing import Any, Sequence
 import torch
 
 from ..core.dtype import DType
-from . import isa, lib
+from . import ir, isa, lib
 from .planner import Plan, Step, ViewRef
 
 _RED = {"sum": 0, "max": 1, "min": 2}
@@ -311,6 +311,18 @@ class BoundPlan:
                 self.calls.append((L.nbk_argmax_rows,
                                    [holder, ("p0", "p1"), src.dtype.abi, a["rows"], a["C"],
                                     1 if a["fn"] == "min" else 0], patches, None))
+            elif k == "random":
+                dst = a["dst"]
+                holder = _Ptrs(1)
+                ptr_field(holder, "p0", dst.buf, dst.offset * dst.dtype.size_in_bytes)
+                self.calls.append((L.nbk_random,
+                                   [holder, ("p0",), dst.dtype.abi, a["numel"],
+                                    ir.RANDOM_MODES.index(a["mode"]), C.c_float(a["a"]), C.c_float(a["b"]),
+                                    C.c_void_p(self.ex.rng_state.data_ptr()), C.c_uint32(a["stream"])],
+                                   patches, None))
+            elif k == "rng_advance":
+                self.calls.append((L.nbk_rng_advance, [C.c_void_p(self.ex.rng_state.data_ptr())],
+                                   patches, None))
             elif k in ("adamw_multi", "sgd_multi"):
                 entries = a["entries"]
                 table = (lib.OptTensor * len(entries))()
@@ -578,6 +590,8 @@ class HipExecutor:
         lib.check(self.lib.nbk_init(device))
         self.torch_device = torch.device("cuda", device)
         self.status_flag = torch.zeros(1, dtype=torch.int32, device=self.torch_device)
+        # generator state read by every random launch: [seed, steps drawn so far]
+        self.rng_state = torch.zeros(2, dtype=torch.int64, device=self.torch_device)
         self.use_graphs = os.environ.get("NBK_GRAPHS", "1") != "0"  # replay repeated steps as HIP graphs
         self._capture_stream = None
         self.graph_replays = 0
@@ -587,6 +601,11 @@ class HipExecutor:
 
     def current_stream(self) -> int:
         return torch.cuda.current_stream(self.torch_device).cuda_stream
+
+    def seed(self, value: int) -> None:
+        """Restart the random generator: the same seed gives the same numbers again."""
+        v = int(value) & 0xFFFFFFFFFFFFFFFF
+        self.rng_state.copy_(torch.tensor([v - (1 << 64) if v >= (1 << 63) else v, 0], dtype=torch.int64))
 
     def bind(self, plan: Plan) -> BoundPlan:
         return BoundPlan(plan, self)

@@ -455,6 +455,26 @@ def attention_bwd(q: Value, k: Value, v: Value, o: Value, lse: Value, dout: Valu
                          scale=float(scale), causal=bool(causal))
 
 
+# ---- random tensors -------------------------------------------------------------------------
+RANDOM_MODES = ("uniform", "normal", "keep")
+
+
+def random(shape, dtype: DType, mode: str, a: float, b: float = 0.0) -> Value:  # noqa: A001
+    """A tensor drawn from the device generator: ``uniform`` on [a, b), ``normal`` with mean a
+    and deviation b, or ``keep``: 1 where a uniform [0, 1) draw exceeds ``a``, else 0 (the mask
+    of dropout with rate a).  Every call is a stream of its own: two calls with equal
+    arguments give different tensors, and one value read in two places is one tensor."""
+    if mode not in RANDOM_MODES:
+        raise ValueError(f"random: unknown mode '{mode}'")
+    if not (dtype.is_float() or (mode == "keep" and dtype is DType.bool)):
+        raise TypeError(f"random.{mode}: cannot draw {dtype}")
+    shape = tuple(int(d) for d in shape)
+    bld = current()
+    stream = getattr(bld, "n_random", 0)
+    bld.n_random = stream + 1
+    return bld.add("random", [], [(shape, dtype)], mode=mode, a=float(a), b=float(b), stream=stream)[0]
+
+
 # ---- optimizer updates over a list of parameters ---------------------------------------------
 def _check_update_list(who: str, groups: Sequence[Sequence[Value]]) -> DType:
     first = groups[0][0]

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 MAX_RANK = 8
 
@@ -163,6 +163,9 @@ _SIGNATURES = {
     "nbk_rowprog_hash": ([C.POINTER(RowProg)], C.c_uint64),
     "nbk_reduce_mid": ([C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64,
                         C.c_int64, C.c_int32, C.c_void_p], C.c_int),
+    "nbk_random": ([C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_float, C.c_float, C.c_void_p,
+                    C.c_uint32, C.c_void_p], C.c_int),
+    "nbk_rng_advance": ([C.c_void_p, C.c_void_p], C.c_int),
     "nbk_adamw_multi": ([C.POINTER(AdamwDesc), C.POINTER(OptTensor), C.c_int32, C.c_void_p], C.c_int),
     "nbk_sgd_multi": ([C.POINTER(SgdDesc), C.POINTER(OptTensor), C.c_int32, C.c_void_p], C.c_int),
     "nbk_reduce_mid_batch": ([C.POINTER(ReduceTask), C.c_int32, C.c_void_p], C.c_int),

@@ -848,6 +848,10 @@ class Planner:
                 dst = ViewRef(b.id, 0, v.shape, contiguous_strides(v.shape), v.dtype)
                 self._emit(Step("copy", [src.buf], [b.id], dict(src=src, dst=dst)))
             outs.append((b.id, v.shape, v.dtype))
+        if any(st.kind == "random" for st in self.steps):
+            # the step drew random numbers: its last launch moves the generator on, so that
+            # the next run (a replay of the recording included) draws new ones
+            self._emit(Step("rng_advance", [], [], {}))
         arena = self._assign_arena()
         stats = {"steps": len(self.steps), "units": len(units),
                  "fused_groups": sum(1 for u in units if u.fused)}
@@ -995,6 +999,11 @@ class Planner:
                 ins=ins, dsts=dsts, name=n.attrs["name"], library=n.attrs["library"])))
         elif k in ("adamw_multi", "sgd_multi"):
             self._lower_update_list(n)
+        elif k == "random":
+            dst = self._alloc_value(out)
+            self._emit(Step("random", [], [dst.buf], dict(
+                dst=dst, numel=out.numel(), mode=n.attrs["mode"], a=n.attrs["a"], b=n.attrs["b"],
+                stream=n.attrs["stream"])))
         else:
             raise NotImplementedError(f"lowering: no rule for node kind '{k}'")
 

@@ -33,6 +33,13 @@ def get_cache_stats() -> dict:
     return dict(_STATS, size=len(_PLAN_CACHE))
 
 
+def set_seed(seed: int) -> None:
+    """Restart the device random generator (uniform, gaussian, dropout): after the same seed the
+    same sequence of steps draws the same numbers."""
+    from ..backend.executor import get_executor
+    get_executor().seed(int(seed))
+
+
 def clear_plan_cache() -> None:
     _PLAN_CACHE.clear()
     _STATS.update(hits=0, misses=0, lower_ms=0.0)
@@ -206,6 +213,14 @@ class ComputeGraph:
             return None
         t0 = time.perf_counter()
         order, leaves, leaf_ids = self._collect(targets)
+        # a random tensor is drawn once: whoever evaluates it first keeps it, so that a later
+        # evaluation that reads it too (the backward pass of a dropout) sees the same numbers
+        for node in order:
+            if getattr(node.op, "draws_random", False):
+                for o in node._refs:
+                    if o is not None and o._buffer is None and id(o) not in seen_t:
+                        seen_t.add(id(o))
+                        targets.append(o)
         key = self._structure_key(order, leaves, leaf_ids, targets)
         ex = get_executor()
         bound = _PLAN_CACHE.get(key)

@@ -5,8 +5,8 @@ from .comparison import (equal, greater, greater_equal, less, less_equal, logica
                          logical_not, logical_or, not_equal)
 from .control_flow import where
 from .convolution import conv2d, conv2d_transpose
-from .creation import (arange, constant, full, full_like, ones, ones_like, tril, triu, zeros,
-                       zeros_like)
+from .creation import (arange, constant, full, full_like, gaussian, normal, ones, ones_like, tril,
+                       triu, uniform, zeros, zeros_like)
 from .extra import (atanh, chunk, flip, floor, is_inf, is_nan, log1p, logical_xor, minmax, outer, split,
                     trunc, unbind)
 from .pooling import avg_pool2d, max_pool2d

@@ -1,7 +1,8 @@
 """Creation ops (nabla/ops/creation.py): full / zeros / ones 50-93 and 353-426,
 arange 96-149, tril / triu 225-274, constant 289-350, ``*_like`` 586-645.
-Random ops are not provided: the reference draws them from MAX's RNG stream,
-which cannot be reproduced; seeded host arrays are uploaded instead.
+``uniform`` / ``gaussian`` 152-183 and 462-511 draw from a device generator of this backend
+(Philox4x32-10): the reference's numbers come from MAX's generator, whose stream is not part of
+its sources, so values differ while distribution and reproducibility under a seed hold.
 """
 from __future__ import annotations
 
@@ -72,7 +73,30 @@ class TriuOp(_TriOp):
         return "triu"
 
 
+class RandomOp(CreationOperation):
+    """A tensor drawn from the device generator (``uniform`` / ``gaussian`` at
+    nabla/ops/creation.py:152-183).  Every evaluation draws anew: the generator's state lives on
+    the device and moves on with every step that uses it."""
+
+    draws_random = True  # (the engine keeps the result of the evaluation that draws it)
+
+    def __init__(self, mode: str, public_name: str):
+        self._mode, self._name = mode, public_name
+
+    @property
+    def name(self) -> str:
+        return self._name
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        return [tuple(kwargs["shape"])], [kwargs["dtype"]], [kwargs["device"]]
+
+    def kernel(self, args, kwargs):
+        return [ir.random(kwargs["shape"], kwargs["dtype"], self._mode, kwargs["a"], kwargs["b"])]
+
+
 _full_op, _arange_op, _tril_op, _triu_op = FullOp(), ArangeOp(), TrilOp(), TriuOp()
+_uniform_op, _gaussian_op = RandomOp("uniform", "uniform"), RandomOp("normal", "gaussian")
+_keep_mask_op = RandomOp("keep", "keep_mask")
 
 
 def _resolve(dtype, device):
@@ -108,6 +132,35 @@ def arange(start=0, stop=None, step=1, *, dtype=None, device=None) -> Tensor:
         raise ValueError("arange: step must not be zero")
     return _arange_op([], {"start": float(start), "stop": float(stop), "step": float(step),
                            "dtype": dtype, "device": device})[0]
+
+
+def _shape_tuple(shape) -> tuple[int, ...]:
+    return (int(shape),) if isinstance(shape, int) else tuple(int(d) for d in shape)
+
+
+def uniform(shape=(), low: float = 0.0, high: float = 1.0, *, dtype=None, device=None) -> Tensor:
+    """Samples of U[low, high) (creation.py:462-485)."""
+    dtype, device = _resolve(dtype, device)
+    return _uniform_op([], {"shape": _shape_tuple(shape), "a": float(low), "b": float(high),
+                            "dtype": dtype, "device": device})[0]
+
+
+def gaussian(shape=(), mean: float = 0.0, std: float = 1.0, *, dtype=None, device=None) -> Tensor:
+    """Samples of N(mean, std^2) (creation.py:488-511)."""
+    dtype, device = _resolve(dtype, device)
+    return _gaussian_op([], {"shape": _shape_tuple(shape), "a": float(mean), "b": float(std),
+                             "dtype": dtype, "device": device})[0]
+
+
+normal = gaussian
+
+
+def keep_mask(shape, p: float, *, dtype=None, device=None) -> Tensor:
+    """``uniform(shape) > p`` as 1 / 0 in ``dtype`` (bool allowed) without the uniform tensor in
+    between: the mask of dropout with rate ``p``."""
+    dtype, device = _resolve(dtype, device)
+    return _keep_mask_op([], {"shape": _shape_tuple(shape), "a": float(p), "b": 0.0,
+                              "dtype": dtype, "device": device})[0]
 
 
 def tril(x, k: int = 0) -> Tensor:

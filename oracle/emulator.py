@@ -421,8 +421,9 @@ def _avgpool(kind, a, mem):
 
 
 class EmulatedPlan:
-    def __init__(self, plan: Plan):
+    def __init__(self, plan: Plan, rng_state: list | None = None):
         self.plan = plan
+        self.rng_state = rng_state if rng_state is not None else [0, 0]  # [seed, runs], shared
 
     def run(self, inputs):
         plan = self.plan
@@ -472,6 +473,17 @@ class EmulatedPlan:
                 _gemm_nf4(a, mem)
             elif k in ("adamw_multi", "sgd_multi"):
                 _update_list(k, a, mem)
+            elif k == "random":
+                from . import philox
+                seed, run = self.rng_state
+                n = a["numel"]
+                vals = {"uniform": lambda: philox.uniform(n, a["a"], a["b"], seed, run, a["stream"]),
+                        "normal": lambda: philox.normal(n, a["a"], a["b"], seed, run, a["stream"]),
+                        "keep": lambda: philox.keep_mask(n, a["a"], seed, run, a["stream"])}[a["mode"]]()
+                dst = _view(mem, a["dst"])
+                dst.copy_(torch.from_numpy(np.ascontiguousarray(vals)).reshape(dst.shape).to(dst.dtype))
+            elif k == "rng_advance":
+                self.rng_state[1] += 1
             elif k in ("conv2d", "conv2d_dgrad", "conv2d_wgrad"):
                 _conv(k, a, mem)
             elif k in ("maxpool2d", "maxpool2d_bwd"):
@@ -517,9 +529,13 @@ class EmulatorExecutor:
 
     def __init__(self):
         self.torch_device = torch.device("cpu")
+        self.rng_state = [0, 0]
+
+    def seed(self, value: int) -> None:
+        self.rng_state[:] = [int(value) & 0xFFFFFFFFFFFFFFFF, 0]
 
     def bind(self, plan: Plan) -> EmulatedPlan:
-        return EmulatedPlan(plan)
+        return EmulatedPlan(plan, self.rng_state)
 
     def current_stream(self) -> int:
         return 0

@@ -600,3 +600,35 @@ def test_torch_steps_agree_with_the_numpy_oracle():
     for a, b in zip(gg, wg):
         assert np.abs(b).max() > 0
         _close(a, b, 1e-9)
+
+
+def test_philox_known_answers():
+    """Philox4x32 with 10 rounds against the known-answer vectors of the Random123 library
+    (zeros, all ones, and the digits of pi as counter and key)."""
+    from oracle.philox import philox4x32_10
+    u = lambda *w: np.array(w, dtype=np.uint32)
+    cases = [
+        (u(0, 0, 0, 0), u(0, 0), u(0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+        (u(*[0xFFFFFFFF] * 4), u(0xFFFFFFFF, 0xFFFFFFFF), u(0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+        (u(0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), u(0xA4093822, 0x299F31D0),
+         u(0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+    ]
+    for ctr, key, want in cases:
+        np.testing.assert_array_equal(philox4x32_10(ctr, key), want)
+    # vectorised over a batch of counters, the same words come out
+    ctrs = np.stack([c for c, _, _ in cases[:1]] * 3)
+    np.testing.assert_array_equal(philox4x32_10(ctrs, cases[0][1][None, :]), np.stack([cases[0][2]] * 3))
+
+
+def test_philox_streams_are_disjoint_and_uniform():
+    """Streams, runs and seeds give different words; the unit floats fill [0, 1) evenly and the
+    Box-Muller values have unit variance."""
+    from oracle import philox
+    base = philox.words(4096, 1, 0, 0)
+    for other in (philox.words(4096, 2, 0, 0), philox.words(4096, 1, 1, 0), philox.words(4096, 1, 0, 1)):
+        assert (base == other).mean() < 0.01
+    u = philox.unit_floats(philox.words(1 << 18, 3, 0, 0))
+    hist = np.histogram(u, bins=16, range=(0.0, 1.0))[0] / u.size
+    assert np.abs(hist - 1.0 / 16).max() < 2e-3
+    z = philox.normal(1 << 18, 0.0, 1.0, 3, 0, 0)
+    assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3
