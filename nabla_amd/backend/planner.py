@@ -530,6 +530,10 @@ class Planner:
         return b
 
     def _emit(self, step: Step) -> None:
+        if step.kind == "fill" and step.attrs["numel"] == 0:
+            return
+        if step.kind == "copy" and _numel(step.attrs["src"].shape) == 0:
+            return
         idx = len(self.steps)
         for r in step.reads:
             b = self.bufs[r]
@@ -2038,10 +2042,37 @@ class _RowCodegen:
         return out
 
 
+def _fold_empty(builder: ir.Builder) -> None:
+    """Tensors without elements never reach a kernel.  A node whose results are all empty needs
+    no work; a node that makes something out of nothing has a value that is known beforehand: a
+    sum over an empty axis and a product with an empty contraction are zero (a maximum or minimum
+    of nothing has no value and is an error, as in numpy).  Both kinds become constants here, so
+    the passes and kernels behind see non-empty operands only."""
+    for n in builder.nodes:
+        if n.kind in ("input", "fill"):
+            continue
+        if all(_numel(o.shape) == 0 for o in n.outputs):
+            value = 0.0
+        elif any(_numel(i.shape) == 0 for i in n.inputs):
+            if n.kind == "reduce" and n.fn != "sum":
+                raise ValueError(f"{n.fn} over an axis of length 0 has no value "
+                                 f"(input of shape {tuple(n.inputs[0].shape)})")
+            if n.kind not in ("reduce", "matmul", "matmul_nf4", "concat", "pad", "slice_update",
+                              "scatter"):
+                raise NotImplementedError(f"'{n.kind}' with an empty operand and a non-empty result")
+            if n.kind in ("concat", "pad", "slice_update", "scatter"):
+                continue  # (copies of the empty pieces are skipped when they are lowered)
+            value = 0.0
+        else:
+            continue
+        n.kind, n.fn, n.inputs, n.attrs = "fill", None, [], {"value": value}
+
+
 def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     """Plan with shrinking fusion limits until every group fits a row program."""
     last = None
     # graph rewrites happen once, before the attempts below share the builder
+    _fold_empty(builder)
     pre = Planner(builder, outputs)
     pre._rematerialize_masks()
     pre._fold_bias_into_matmul()

@@ -1,150 +1,167 @@
-"""``Module`` base class (nabla/nn/modules/base.py:106-337): parameters are
-tensors with ``requires_grad`` assigned as attributes, submodules are tracked,
-and every subclass is a pytree node (parameters, buffers, submodules are the
-children) so modules pass through grad / compile unchanged."""
+"""``Module``: the container layers are built from (interface of nabla/nn/modules/base.py:106-337).
+
+A module is an ordinary object whose attributes happen to include tensors and other modules.
+It keeps one record about them, ``_roles``: attribute name -> ``"parameter"`` (a tensor that
+required a gradient when it was assigned), ``"buffer"`` (any other tensor) or ``"module"``.
+Everything else is derived from that record and the attributes themselves: the ``_parameters``
+/ ``_buffers`` / ``_modules`` views, the iterators, the state dict, and the pytree form that
+lets a module pass through ``grad`` / ``compile`` / ``tree_map`` like a dict of its tensors
+(children = the attributes that have a role, in assignment order; everything else, with the
+roles and the training flag, is static structure).
+"""
 from __future__ import annotations
 
 from collections import OrderedDict
 from typing import Any, Iterator
 
 from ...core.pytree import is_tensor, register_pytree_node
-from ...core.tensor import Tensor, realize_all
+from ...core.tensor import Tensor
 
-_RESERVED = {"_parameters", "_buffers", "_modules", "_training"}
-
-
-def _module_tree_flatten(module: "Module"):
-    param_keys = tuple(module._parameters.keys())
-    buffer_keys = tuple(module._buffers.keys())
-    module_keys = tuple(module._modules.keys())
-    children = ([module._parameters[k] for k in param_keys] +
-                [module._buffers[k] for k in buffer_keys] +
-                [module._modules[k] for k in module_keys])
-    extras = []
-    for key, value in module.__dict__.items():
-        if key in _RESERVED or key in module._parameters or key in module._buffers \
-                or key in module._modules:
-            continue
-        extras.append((key, value))
-    aux = (type(module), param_keys, buffer_keys, module_keys,
-           tuple(sorted(extras, key=lambda kv: kv[0])), bool(module._training))
-    return children, aux
+PARAMETER, BUFFER, MODULE = "parameter", "buffer", "module"
+_OWN_STATE = ("_roles", "_training")
 
 
-def _module_tree_unflatten(aux, children) -> "Module":
-    cls, param_keys, buffer_keys, module_keys, extras, training = aux
-    obj = object.__new__(cls)
-    object.__setattr__(obj, "_parameters", OrderedDict())
-    object.__setattr__(obj, "_buffers", OrderedDict())
-    object.__setattr__(obj, "_modules", OrderedDict())
-    object.__setattr__(obj, "_training", training)
-    cursor = 0
-    for keys, store in ((param_keys, obj._parameters), (buffer_keys, obj._buffers),
-                        (module_keys, obj._modules)):
-        for key in keys:
-            value = children[cursor]
-            cursor += 1
-            store[key] = value
-            object.__setattr__(obj, key, value)
-    for key, value in extras:
-        object.__setattr__(obj, key, value)
-    return obj
+def _role_of(value: Any) -> str | None:
+    if isinstance(value, Module):
+        return MODULE
+    if is_tensor(value):
+        return PARAMETER if value.requires_grad else BUFFER
+    return None
+
+
+def _flatten_module(module: "Module"):
+    roles = module._roles
+    names = tuple(roles)
+    plain = tuple(sorted(((k, v) for k, v in vars(module).items()
+                          if k not in roles and k not in _OWN_STATE), key=lambda kv: kv[0]))
+    static = (type(module), names, tuple(roles[n] for n in names), plain, module._training)
+    return [getattr(module, n) for n in names], static
+
+
+def _unflatten_module(static, children) -> "Module":
+    cls, names, kinds, plain, training = static
+    module = object.__new__(cls)
+    state = vars(module)
+    state["_roles"] = dict(zip(names, kinds))  # roles travel with the structure, not the leaves
+    state["_training"] = training
+    state.update(zip(names, children))
+    state.update(plain)
+    return module
 
 
 class Module:
     def __init_subclass__(cls, **kwargs: Any) -> None:
         super().__init_subclass__(**kwargs)
-        register_pytree_node(cls, _module_tree_flatten, _module_tree_unflatten)
+        register_pytree_node(cls, _flatten_module, _unflatten_module)
 
     def __init__(self) -> None:
-        object.__setattr__(self, "_parameters", OrderedDict())
-        object.__setattr__(self, "_buffers", OrderedDict())
-        object.__setattr__(self, "_modules", OrderedDict())
-        object.__setattr__(self, "_training", True)
+        vars(self).update(_roles={}, _training=True)
 
+    # ---- attribute bookkeeping ---------------------------------------------------------------
     def __setattr__(self, name: str, value: Any) -> None:
-        if name in _RESERVED:
-            object.__setattr__(self, name, value)
+        if name in _OWN_STATE:
+            vars(self)[name] = value
             return
-        for store in (self._parameters, self._buffers, self._modules):
-            store.pop(name, None)
-        object.__setattr__(self, name, value)
-        if isinstance(value, Module):
-            self._modules[name] = value
-        elif is_tensor(value):
-            (self._parameters if value.requires_grad else self._buffers)[name] = value
+        roles = self._roles
+        roles.pop(name, None)  # a re-assigned attribute moves to the end, whatever it was before
+        role = _role_of(value)
+        if role is not None:
+            roles[name] = role
+        vars(self)[name] = value
+
+    def __delattr__(self, name: str) -> None:
+        self._roles.pop(name, None)
+        object.__delattr__(self, name)
+
+    def _having(self, role: str) -> "OrderedDict[str, Any]":
+        return OrderedDict((n, getattr(self, n)) for n, r in self._roles.items() if r == role)
+
+    @property
+    def _parameters(self) -> "OrderedDict[str, Tensor]":
+        return self._having(PARAMETER)
+
+    @property
+    def _buffers(self) -> "OrderedDict[str, Tensor]":
+        return self._having(BUFFER)
+
+    @property
+    def _modules(self) -> "OrderedDict[str, Module]":
+        return self._having(MODULE)
 
     def register_buffer(self, name: str, tensor: Tensor | None) -> None:
         setattr(self, name, tensor)
 
+    # ---- calling -----------------------------------------------------------------------------
     def forward(self, *args: Any, **kwargs: Any) -> Any:
         raise NotImplementedError
 
     def __call__(self, *args: Any, **kwargs: Any) -> Any:
         return self.forward(*args, **kwargs)
 
-    def parameters(self) -> Iterator[Tensor]:
-        for _, p in self.named_parameters():
-            yield p
+    # ---- walking -----------------------------------------------------------------------------
+    def _walk(self, role: str, prefix: str = "") -> Iterator[tuple[str, Any]]:
+        """(dotted name, value) of every attribute with ``role``, this module's first, then its
+        submodules' in assignment order."""
+        for name, value in self._having(role).items():
+            yield prefix + name, value
+        for name, sub in self._having(MODULE).items():
+            yield from sub._walk(role, f"{prefix}{name}.")
 
     def named_parameters(self, prefix: str = "") -> Iterator[tuple[str, Tensor]]:
-        for name, p in self._parameters.items():
-            yield (f"{prefix}{name}", p)
-        for mname, m in self._modules.items():
-            yield from m.named_parameters(prefix=f"{prefix}{mname}.")
-
-    def buffers(self) -> Iterator[Tensor]:
-        for _, b in self.named_buffers():
-            yield b
+        return self._walk(PARAMETER, prefix)
 
     def named_buffers(self, prefix: str = "") -> Iterator[tuple[str, Tensor]]:
-        for name, b in self._buffers.items():
-            yield (f"{prefix}{name}", b)
-        for mname, m in self._modules.items():
-            yield from m.named_buffers(prefix=f"{prefix}{mname}.")
+        return self._walk(BUFFER, prefix)
+
+    def parameters(self) -> Iterator[Tensor]:
+        return (p for _, p in self.named_parameters())
+
+    def buffers(self) -> Iterator[Tensor]:
+        return (b for _, b in self.named_buffers())
 
     def modules(self) -> Iterator["Module"]:
         yield self
-        for m in self._modules.values():
-            yield from m.modules()
+        for sub in self._having(MODULE).values():
+            yield from sub.modules()
+
+    # ---- modes and gradients -------------------------------------------------------------------
+    def _set_training(self, flag: bool) -> "Module":
+        for m in self.modules():
+            vars(m)["_training"] = flag
+        return self
 
     def train(self) -> "Module":
-        for m in self.modules():
-            object.__setattr__(m, "_training", True)
-        return self
+        return self._set_training(True)
 
     def eval(self) -> "Module":
-        for m in self.modules():
-            object.__setattr__(m, "_training", False)
-        return self
+        return self._set_training(False)
 
     def zero_grad(self) -> None:
         for p in self.parameters():
             p.grad = None
 
+    # ---- state -------------------------------------------------------------------------------
     def state_dict(self) -> "OrderedDict[str, Tensor]":
-        out: "OrderedDict[str, Tensor]" = OrderedDict()
-        for k, v in self.named_parameters():
-            out[k] = v
-        for k, v in self.named_buffers():
-            out[k] = v
-        return out
+        return OrderedDict([*self.named_parameters(), *self.named_buffers()])
 
     def load_state_dict(self, state_dict) -> None:
-        for name, value in state_dict.items():
-            obj = self
-            *path, leaf = name.split(".")
+        """Assign every entry to the attribute its dotted name leads to; a tensor that replaces
+        one keeps the old tensor's ``requires_grad`` (and with it the role)."""
+        for dotted, value in state_dict.items():
+            *path, leaf = dotted.split(".")
+            owner = self
             for part in path:
-                obj = obj._modules[part]
-            if obj.__dict__.get(leaf) is not None and is_tensor(obj.__dict__[leaf]):
-                value.requires_grad = obj.__dict__[leaf].requires_grad
-            setattr(obj, leaf, value)
+                owner = getattr(owner, part)
+            current = vars(owner).get(leaf)
+            if is_tensor(current):
+                value.requires_grad = current.requires_grad
+            setattr(owner, leaf, value)
 
+    # ---- display -----------------------------------------------------------------------------
     def extra_repr(self) -> str:
         return ""
 
     def __repr__(self) -> str:
-        lines = [f"{type(self).__name__}({self.extra_repr()}"]
-        for name, m in self._modules.items():
-            lines.append(f"  ({name}): {m!r}")
-        return "\n".join(lines) + ")"
+        head = f"{type(self).__name__}({self.extra_repr()}"
+        body = [f"  ({name}): {sub!r}" for name, sub in self._having(MODULE).items()]
+        return "\n".join([head, *body]) + ")"

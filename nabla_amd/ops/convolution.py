@@ -16,37 +16,70 @@ from ..core.tensor import Tensor
 from .base import Operation, ensure_tensor
 
 
-def _normalize_2tuple(value, name: str) -> tuple[int, int]:
+# What each window argument may look like and which values it may hold.  One table drives the
+# expansion to per-side integers and the range checks of both public functions; the wording of
+# the errors is the reference's (convolution.py:602-696), which user code may match on.
+_PADDING_FORMS = "padding must be int, (pad_h, pad_w), or (pad_top, pad_bottom, pad_left, pad_right)"
+_WINDOW_ARGS = {
+    # name: (entries after expansion, smallest allowed value)
+    "stride": (2, 1),
+    "dilation": (2, 1),
+    "padding": (4, 0),
+    "output_paddings": (2, 0),
+    "kernel_size": (2, 1),
+}
+
+
+def _expand_window_arg(name: str, value) -> tuple[int, ...]:
+    """An int or a short sequence -> one integer per side, checked against the argument's range."""
+    width, lowest = _WINDOW_ARGS[name]
+    seq = None
     if isinstance(value, int):
-        return (value, value)
-    if isinstance(value, (tuple, list)) and len(value) == 2:
-        return (int(value[0]), int(value[1]))
-    raise ValueError(f"{name} must be int or tuple/list of length 2, got {value}")
+        seq = (value,) * width
+    elif isinstance(value, (tuple, list)):
+        if len(value) == width:
+            seq = tuple(value)
+        elif width == 4 and len(value) == 2:  # (pad_h, pad_w): both sides of an axis alike
+            seq = (value[0], value[0], value[1], value[1])
+    if seq is None:
+        raise ValueError(_PADDING_FORMS if width == 4 else
+                         f"{name} must be int or tuple/list of length 2, got {value}")
+    out = tuple(int(v) for v in seq)
+    if min(out) < lowest:
+        bound = "> 0" if lowest == 1 else ">= 0"
+        raise ValueError(f"{name} values must be {bound}, got {out}")
+    return out
 
 
-def _normalize_4padding(padding) -> tuple[int, int, int, int]:
-    if isinstance(padding, int):
-        p = int(padding)
-        return (p, p, p, p)
-    if isinstance(padding, (tuple, list)):
-        if len(padding) == 2:
-            ph, pw = int(padding[0]), int(padding[1])
-            return (ph, ph, pw, pw)
-        if len(padding) == 4:
-            return tuple(int(v) for v in padding)
-    raise ValueError(
-        "padding must be int, (pad_h, pad_w), or (pad_top, pad_bottom, pad_left, pad_right)"
-    )
+def _window(**given) -> dict[str, tuple[int, ...]]:
+    """Expand every window argument first, then range-check in the order given (the order in
+    which the reference reports a call that is wrong in two ways)."""
+    shapes = {}
+    for name, value in given.items():  # malformed arguments are reported before out-of-range ones
+        width = _WINDOW_ARGS[name][0]
+        ok = isinstance(value, int) or (isinstance(value, (tuple, list)) and
+                                        (len(value) == width or (width == 4 and len(value) == 2)))
+        if not ok:
+            _expand_window_arg(name, value)  # raises with the form message
+        shapes[name] = value
+    return {name: _expand_window_arg(name, value) for name, value in shapes.items()}
 
 
-def _require_all_positive_2tuple(value, name: str) -> None:
-    if value[0] <= 0 or value[1] <= 0:
-        raise ValueError(f"{name} values must be > 0, got {value}")
+def _check_bias(who: str, bias, c_out: int) -> None:
+    if bias is None:
+        return
+    if len(bias.shape) != 1:
+        raise ValueError(f"{who} bias must be rank-1 [C_out], got shape={tuple(bias.shape)}")
+    if bias.shape[0] != c_out:
+        raise ValueError(f"{who} bias size ({bias.shape[0]}) must match filter C_out ({c_out})")
 
 
-def _require_all_nonnegative(value, name: str) -> None:
-    if any(v < 0 for v in value):
-        raise ValueError(f"{name} values must be >= 0, got {value}")
+def _rank4_operands(who: str, x, filter, bias):  # noqa: A002
+    x, filter = ensure_tensor(x), ensure_tensor(filter)
+    if len(x.shape) != 4 or len(filter.shape) != 4:
+        raise ValueError(f"{who} expects rank-4 tensors, got x={tuple(x.shape)}, "
+                         f"filter={tuple(filter.shape)}")
+    return x, filter, (None if bias is None else ensure_tensor(bias))
 
 
 def _out_hw(x_shape, w_shape, stride, padding) -> tuple[int, int]:
@@ -174,43 +207,24 @@ _conv2d_wgrad_op = Conv2DFilterGradOp()
 
 def conv2d(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0, 0, 0), groups: int = 1,
            bias=None, input_layout: Any = None, filter_layout: Any = None) -> Tensor:  # noqa: A002
-    x = ensure_tensor(x)
-    filter = ensure_tensor(filter)
-    bias_t = ensure_tensor(bias) if bias is not None else None
-    if len(x.shape) != 4 or len(filter.shape) != 4:
-        raise ValueError(
-            f"conv2d expects rank-4 tensors, got x={tuple(x.shape)}, filter={tuple(filter.shape)}"
-        )
+    x, filter, bias_t = _rank4_operands("conv2d", x, filter, bias)
     if input_layout is not None or filter_layout is not None:
         raise ValueError("conv2d currently supports only the default NHWC/RSCF layouts")
-    norm_stride = _normalize_2tuple(stride, "stride")
-    norm_dilation = _normalize_2tuple(dilation, "dilation")
-    norm_padding = _normalize_4padding(padding)
-    groups_i = int(groups)
-    _require_all_positive_2tuple(norm_stride, "stride")
-    _require_all_positive_2tuple(norm_dilation, "dilation")
-    _require_all_nonnegative(norm_padding, "padding")
-    if groups_i <= 0:
-        raise ValueError(f"groups must be > 0, got {groups_i}")
-    if norm_dilation != (1, 1):
+    win = _window(stride=stride, dilation=dilation, padding=padding)
+    n_groups = int(groups)
+    if n_groups <= 0:
+        raise ValueError(f"groups must be > 0, got {n_groups}")
+    if win["dilation"] != (1, 1):
         raise ValueError("conv2d currently supports only dilation=(1, 1)")
-    if groups_i != 1:
+    if n_groups != 1:
         raise ValueError("conv2d grouped mode is not exposed")
-    c_in, c_in_w, c_out = x.shape[-1], filter.shape[2], filter.shape[3]
-    if c_in != c_in_w * groups_i:
+    c_in, (_, _, c_in_w, c_out) = x.shape[-1], filter.shape
+    if c_in != c_in_w * n_groups:
         raise ValueError(
-            f"Input channels ({c_in}) must match filter channels*groups ({c_in_w * groups_i})"
-        )
-    if bias_t is not None:
-        if len(bias_t.shape) != 1:
-            raise ValueError(f"conv2d bias must be rank-1 [C_out], got shape={tuple(bias_t.shape)}")
-        if bias_t.shape[0] != c_out:
-            raise ValueError(
-                f"conv2d bias size ({bias_t.shape[0]}) must match filter C_out ({c_out})"
-            )
-    kwargs = {"stride": norm_stride, "padding": norm_padding}
-    args = [x, filter] if bias_t is None else [x, filter, bias_t]
-    return _conv2d_op(args, kwargs)[0]
+            f"Input channels ({c_in}) must match filter channels*groups ({c_in_w * n_groups})")
+    _check_bias("conv2d", bias_t, c_out)
+    operands = [x, filter] + ([bias_t] if bias_t is not None else [])
+    return _conv2d_op(operands, {"stride": win["stride"], "padding": win["padding"]})[0]
 
 
 def conv2d_transpose(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0, 0, 0),  # noqa: A002
@@ -220,36 +234,17 @@ def conv2d_transpose(x, filter, *, stride=(1, 1), dilation=(1, 1), padding=(0, 0
     [R,S,Cout,Cin] (channels the other way round than ``conv2d``), optional ``bias`` [Cout].
     The same argument checks and messages as the reference; dilation and output padding other
     than the defaults are rejected, as there (762-763 for the output padding)."""
-    x = ensure_tensor(x)
-    filter = ensure_tensor(filter)
-    bias_t = ensure_tensor(bias) if bias is not None else None
-    if len(x.shape) != 4 or len(filter.shape) != 4:
-        raise ValueError(
-            f"conv2d_transpose expects rank-4 tensors, got x={tuple(x.shape)}, filter={tuple(filter.shape)}"
-        )
+    x, filter, bias_t = _rank4_operands("conv2d_transpose", x, filter, bias)
     if input_layout is not None or filter_layout is not None:
         raise ValueError("conv2d_transpose currently supports only the default NHWC layouts")
-    norm_stride = _normalize_2tuple(stride, "stride")
-    norm_dilation = _normalize_2tuple(dilation, "dilation")
-    norm_padding = _normalize_4padding(padding)
-    norm_out_pad = _normalize_2tuple(output_paddings, "output_paddings")
-    _require_all_positive_2tuple(norm_stride, "stride")
-    _require_all_positive_2tuple(norm_dilation, "dilation")
-    _require_all_nonnegative(norm_padding, "padding")
-    _require_all_nonnegative(norm_out_pad, "output_paddings")
-    if norm_out_pad != (0, 0):
+    win = _window(stride=stride, dilation=dilation, padding=padding, output_paddings=output_paddings)
+    if win["output_paddings"] != (0, 0):
         raise ValueError("conv2d_transpose currently supports only output_paddings=(0, 0)")
-    if norm_dilation != (1, 1):
+    if win["dilation"] != (1, 1):
         raise ValueError("conv2d_transpose currently supports only dilation=(1, 1)")
-    c_in, c_out, c_in_w = x.shape[-1], filter.shape[2], filter.shape[3]
+    c_in, (_, _, c_out, c_in_w) = x.shape[-1], filter.shape
     if c_in != c_in_w:
         raise ValueError(f"Input channels ({c_in}) must match filter input channels ({c_in_w})")
-    if bias_t is not None:
-        if len(bias_t.shape) != 1:
-            raise ValueError(
-                f"conv2d_transpose bias must be rank-1 [C_out], got shape={tuple(bias_t.shape)}")
-        if bias_t.shape[0] != c_out:
-            raise ValueError(
-                f"conv2d_transpose bias size ({bias_t.shape[0]}) must match filter C_out ({c_out})")
-    y = _conv2d_transpose_op([x, filter], {"stride": norm_stride, "padding": norm_padding})[0]
+    _check_bias("conv2d_transpose", bias_t, c_out)
+    y = _conv2d_transpose_op([x, filter], {"stride": win["stride"], "padding": win["padding"]})[0]
     return y if bias_t is None else y + bias_t

@@ -64,18 +64,24 @@ def is_inf(x) -> Tensor:
 
 def log1p(x) -> Tensor:
     """``log(1 + x)`` without losing small ``x``: with u = 1 + x as rounded, log(u) * x / (u - 1)
-    corrects for the rounding of u, and x itself is returned where u == 1.  The derivative that
-    falls out of the parts equals the reference's 1 / (1 + x) up to that rounding."""
+    corrects for the rounding of u, x itself is returned where u == 1 and u where it is infinite
+    (the quotient would be inf / inf there).  The derivative that falls out of the parts equals the
+    reference's 1 / (1 + x) up to that rounding."""
     from .binary import add, div, mul, sub
     from .comparison import equal
     from .control_flow import where
     from .unary import log
+    from .comparison import logical_or
+    from .creation import ones_like
     x = ensure_tensor(x)
     u = add(x, 1.0)
     d = sub(u, 1.0)
     one = equal(d, 0.0)
-    safe = where(one, add(mul(x, 0.0), 1.0), d)      # a divisor of 1 where u == 1
-    return where(one, x, mul(log(u), div(x, safe)))
+    big = is_inf(u)                                   # x = +inf: the answer is u itself
+    ones = ones_like(x)
+    safe = where(logical_or(one, big), ones, d)       # a divisor of 1 where the quotient is unused
+    corrected = mul(log(where(big, ones, u)), div(where(big, ones, x), safe))
+    return where(one, x, where(big, u, corrected))
 
 
 def atanh(x) -> Tensor:

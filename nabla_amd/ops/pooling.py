@@ -13,8 +13,7 @@ from __future__ import annotations
 from ..backend import ir
 from ..core.tensor import Tensor
 from .base import Operation, ensure_tensor
-from .convolution import (_normalize_2tuple, _normalize_4padding, _require_all_nonnegative,
-                          _require_all_positive_2tuple)
+from .convolution import _window
 
 
 class MaxPool2DOp(Operation):
@@ -137,19 +136,15 @@ _avg_pool2d_grad_op = AvgPool2DGradOp()
 
 
 def _pool_args(x, kernel_size, stride, padding, dilation, what: str):
+    """The window of a pooling call as per-side integers (a missing stride is the kernel size)."""
     x = ensure_tensor(x)
     if len(x.shape) != 4:
         raise ValueError(f"{what} expects an NHWC rank-4 tensor, got shape {tuple(x.shape)}")
-    kernel = _normalize_2tuple(kernel_size, "kernel_size")
-    stride_n = _normalize_2tuple(stride if stride is not None else kernel, "stride")
-    padding_n = _normalize_4padding(padding)
-    dil = _normalize_2tuple(dilation, "dilation")
-    _require_all_positive_2tuple(kernel, "kernel_size")
-    _require_all_positive_2tuple(stride_n, "stride")
-    _require_all_nonnegative(padding_n, "padding")
-    if dil != (1, 1):
+    win = _window(kernel_size=kernel_size, stride=kernel_size if stride is None else stride,
+                  padding=padding, dilation=dilation)
+    if win["dilation"] != (1, 1):
         raise ValueError("pool2d currently supports only dilation=(1, 1)")
-    return x, {"kernel_size": kernel, "stride": stride_n, "padding": padding_n}
+    return x, {"kernel_size": win["kernel_size"], "stride": win["stride"], "padding": win["padding"]}
 
 
 def avg_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Tensor:
@@ -158,16 +153,5 @@ def avg_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Te
 
 
 def max_pool2d(x, *, kernel_size, stride=None, padding=0, dilation=(1, 1)) -> Tensor:
-    x = ensure_tensor(x)
-    if len(x.shape) != 4:
-        raise ValueError(f"max_pool2d expects an NHWC rank-4 tensor, got shape {tuple(x.shape)}")
-    kernel = _normalize_2tuple(kernel_size, "kernel_size")
-    stride_n = _normalize_2tuple(stride if stride is not None else kernel, "stride")
-    padding_n = _normalize_4padding(padding)
-    dil = _normalize_2tuple(dilation, "dilation")
-    _require_all_positive_2tuple(kernel, "kernel_size")
-    _require_all_positive_2tuple(stride_n, "stride")
-    _require_all_nonnegative(padding_n, "padding")
-    if dil != (1, 1):
-        raise ValueError("pool2d currently supports only dilation=(1, 1)")
-    return _max_pool2d_op([x], {"kernel_size": kernel, "stride": stride_n, "padding": padding_n})[0]
+    x, kw = _pool_args(x, kernel_size, stride, padding, dilation, "max_pool2d")
+    return _max_pool2d_op([x], kw)[0]

@@ -26,24 +26,70 @@ from ..core.pytree import PyTreeDef, tree_flatten, tree_unflatten
 from ..core.tensor import Tensor, TensorImpl
 
 
-@dataclass
 class CompilationStats:
-    hits: int = 0
-    misses: int = 0
-    fallbacks: int = 0
-    total_compile_time_ms: float = 0.0
-    total_cached_exec_time_ms: float = 0.0
-    cache_size: int = 0
-    specializations: int = 0  # plans built for new bindings of symbolic dims
+    """Counters of one compiled function, under the reference's names (compile.py:40-69): calls
+    answered from the cache (``hits``), signatures traced for the first time (``misses``), calls
+    that ran uncompiled (``fallbacks``), the milliseconds spent tracing and lowering, and those
+    spent in cached calls.  ``specializations`` counts plans built for a new binding of
+    symbolic dims inside a known signature."""
+
+    _COUNTERS = ("hits", "misses", "fallbacks", "specializations", "cache_size")
+    _CLOCKS = ("total_compile_time_ms", "total_cached_exec_time_ms")
+
+    def __init__(self) -> None:
+        for name in self._COUNTERS:
+            setattr(self, name, 0)
+        for name in self._CLOCKS:
+            setattr(self, name, 0.0)
+
+    def clock(self, name: str):
+        """Context manager that adds the time spent inside it to the clock ``name``."""
+        return _Stopwatch(self, name)
+
+    @property
+    def calls(self) -> int:
+        return self.hits + self.misses + self.fallbacks
 
     @property
     def hit_rate(self) -> float:
-        total = self.hits + self.misses + self.fallbacks
-        return (self.hits / total * 100) if total > 0 else 0.0
+        """Share of calls answered from the cache, in percent."""
+        return 100.0 * self.hits / self.calls if self.calls else 0.0
 
     def __repr__(self) -> str:
         return (f"CompilationStats(hits={self.hits}, misses={self.misses}, "
                 f"fallbacks={self.fallbacks}, hit_rate={self.hit_rate:.1f}%)")
+
+
+class _Stopwatch:
+    __slots__ = ("stats", "name", "t0")
+
+    def __init__(self, stats: CompilationStats, name: str):
+        self.stats, self.name = stats, name
+
+    def __enter__(self):
+        self.t0 = time.perf_counter()
+        return self
+
+    def __exit__(self, *exc) -> None:
+        spent = (time.perf_counter() - self.t0) * 1e3
+        setattr(self.stats, self.name, getattr(self.stats, self.name) + spent)
+
+
+def _static_key(value: Any) -> Any:
+    """A hashable stand-in for a non-tensor argument, equal for equal arguments: containers are
+    rebuilt from the stand-ins of their items (a dict as its sorted items, a set as a
+    frozenset), hashable objects stand for themselves, anything else for its type and repr."""
+    if isinstance(value, dict):
+        return ("dict", tuple(sorted((_static_key(k), _static_key(v)) for k, v in value.items())))
+    if isinstance(value, (set, frozenset)):
+        return ("set", frozenset(_static_key(v) for v in value))
+    if isinstance(value, (list, tuple)):
+        return tuple(_static_key(v) for v in value)
+    try:
+        hash(value)
+    except TypeError:
+        return (type(value).__qualname__, repr(value))
+    return value
 
 
 @dataclass(frozen=True)
@@ -90,22 +136,6 @@ class CompiledFunction:
         self._cache.clear()
 
     # ---- keys ---------------------------------------------------------------
-    def _make_hashable_static(self, value: Any) -> Any:
-        if isinstance(value, (str, bytes, int, float, bool, type(None))):
-            return value
-        if isinstance(value, (tuple, list)):
-            return tuple(self._make_hashable_static(v) for v in value)
-        if isinstance(value, dict):
-            return tuple(sorted((self._make_hashable_static(k), self._make_hashable_static(v))
-                                for k, v in value.items()))
-        if isinstance(value, (set, frozenset)):
-            return frozenset(self._make_hashable_static(v) for v in value)
-        try:
-            hash(value)
-            return value
-        except TypeError:
-            return (type(value).__qualname__, repr(value))
-
     def _tensor_signature(self, t: Tensor, arg_idx: int):
         shape: list = list(t.shape)
         if arg_idx in self.dynamic_dims:
@@ -123,7 +153,7 @@ class CompiledFunction:
                 concrete.append(tuple(x.shape))
                 ti += 1
             else:
-                statics.append(self._make_hashable_static(x))
+                statics.append(_static_key(x))
         return tuple(sigs), tuple(statics), tuple(concrete)
 
     # ---- call ---------------------------------------------------------------
@@ -135,31 +165,24 @@ class CompiledFunction:
         sigs, statics, concrete = self._build_keys(flat)
         key = _CacheKey(sigs, statics, treedef)
         entry = self._cache.get(key)
-        if entry is None:
+        known = entry is not None
+        if known:
+            self._cache.move_to_end(key)
+            self._stats.hits += 1
+        else:
             self._stats.misses += 1
-            entry = _CachedModel()
-            self._cache[key] = entry
+            entry = self._cache[key] = _CachedModel()
             if len(self._cache) > self.max_cache_size:
                 self._cache.popitem(last=False)
-            t0 = time.perf_counter()
-            spec = self._trace_and_compile(args, kwargs, flat)
-            entry.specializations[concrete] = spec
-            self._stats.total_compile_time_ms += (time.perf_counter() - t0) * 1e3
-            return spec._first_result
-        self._cache.move_to_end(key)
-        self._stats.hits += 1
         spec = entry.specializations.get(concrete)
-        if spec is None:
+        if spec is not None:
+            with self._stats.clock("total_cached_exec_time_ms"):
+                return self._execute_cached(spec, flat)
+        if known:
             self._stats.specializations += 1
-            t0 = time.perf_counter()
-            spec = self._trace_and_compile(args, kwargs, flat)
-            entry.specializations[concrete] = spec
-            self._stats.total_compile_time_ms += (time.perf_counter() - t0) * 1e3
-            return spec._first_result
-        t0 = time.perf_counter()
-        out = self._execute_cached(spec, flat)
-        self._stats.total_cached_exec_time_ms += (time.perf_counter() - t0) * 1e3
-        return out
+        with self._stats.clock("total_compile_time_ms"):
+            spec = entry.specializations[concrete] = self._trace_and_compile(args, kwargs, flat)
+        return spec._first_result
 
     # ---- miss ---------------------------------------------------------------
     def _trace_and_compile(self, args, kwargs, flat) -> _Specialization:

@@ -105,6 +105,16 @@ def vmap(func: Callable | None = None, in_axes: Any = 0, out_axes: Any = 0,
             sliced = tuple(_walk(lambda t, ax: t if ax is None else t[i], a, ax)
                            for a, ax in zip(fronted, in_ax))
             results.append(func(*sliced))
+        empty = size == 0
+        if empty:
+            # nothing to map over: one call on a stand-in element (zeros of an element's shape)
+            # tells the structure and the element shapes of the result, which then comes back
+            # with a mapped axis of length 0
+            from ..ops.creation import zeros
+            stand_in = tuple(_walk(lambda t, ax: t if ax is None else
+                                   zeros(tuple(t.shape[1:]), dtype=t.dtype, device=t.device), a, ax)
+                             for a, ax in zip(fronted, in_ax))
+            results.append(func(*stand_in))
 
         first = results[0]
         is_single = not isinstance(first, (list, tuple))
@@ -119,6 +129,11 @@ def vmap(func: Callable | None = None, in_axes: Any = 0, out_axes: Any = 0,
                     if sp is None:
                         return head
                     ax = sp if sp >= 0 else sp + len(head.shape) + 1
+                    if empty:
+                        from ..ops.creation import zeros
+                        shape = list(head.shape)
+                        shape.insert(ax, 0)
+                        return zeros(tuple(shape), dtype=head.dtype, device=head.device)
                     return stack(nodes, axis=ax)
                 if isinstance(head, dict):
                     return {key: rec([n[key] for n in nodes], sp[key] if isinstance(sp, dict) else sp)

@@ -517,7 +517,8 @@ class EmulatedPlan:
         by_buf = {}
         for oi, (bid, shape, dtype) in enumerate(plan.outputs):
             if bid not in by_buf:
-                by_buf[bid] = mem[bid].reshape(shape)
+                n = int(np.prod(shape)) if len(shape) else 1
+                by_buf[bid] = mem[bid][:n].reshape(shape)
             outs[oi] = by_buf[bid]
         return outs
 

@@ -96,3 +96,13 @@ def test_atanh(emulator):
     np.testing.assert_allclose(got, np.arctanh(x.astype(np.float64)), rtol=1e-6, atol=0)
     g = nb.grad(lambda t: nb.reduce_sum(nb.atanh(t)))(T(x[3:])).numpy()
     np.testing.assert_allclose(g, 1.0 / (1.0 - x[3:].astype(np.float64) ** 2), rtol=3e-4)
+
+
+def test_tensors_without_elements(emulator):
+    from edge_cases import check_empty_tensors
+    check_empty_tensors(nb)
+
+
+def test_log1p_and_atanh_at_the_edges(emulator):
+    from edge_cases import check_log1p_and_atanh_at_the_edges
+    check_log1p_and_atanh_at_the_edges(nb)

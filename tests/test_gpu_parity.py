@@ -271,6 +271,12 @@ def test_integers_above_2_pow_24_are_exact(hip):
     check_large_integers(nb)
 
 
+def test_tensors_without_elements_and_domain_edges(hip):
+    from edge_cases import check_empty_tensors, check_log1p_and_atanh_at_the_edges
+    check_empty_tensors(nb)
+    check_log1p_and_atanh_at_the_edges(nb)
+
+
 def test_slice_pad_concat_exact(hip):
     rng = np.random.default_rng(9)
     a = rng.standard_normal((6, 10, 12)).astype(np.float32)
