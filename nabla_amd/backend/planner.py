@@ -710,8 +710,10 @@ class Planner:
             out = n.outputs[0]
             for m, bb in ((n.inputs[0], n.inputs[1]), (n.inputs[1], n.inputs[0])):
                 mm = m.node
+                at = mm.attrs or {}
                 if not (bb.node.kind == "broadcast" and mm.kind == "matmul" and
-                        len(mm.inputs) == 2 and n_users.get(m.id) == 1 and m.id not in out_ids and
+                        len(mm.outputs) == 1 and "bias_in" not in at and not at.get("act") and
+                        n_users.get(m.id) == 1 and m.id not in out_ids and
                         self._epilogue_ok(mm, out)):
                     continue
                 src = bb.node.inputs[0]
@@ -721,7 +723,66 @@ class Planner:
                     continue
                 n.kind, n.fn = "matmul", None
                 n.inputs = list(mm.inputs) + [src]
-                n.attrs = dict(mm.attrs or {}, bias_in=2)
+                n.attrs = dict(at, bias_in=len(mm.inputs))
+                break
+
+    def _fold_sum_into_matmul(self) -> None:
+        """``r + (x @ W) * alpha`` with ``r`` of the product's shape (a skip connection, the base
+        product under a low-rank update, a gradient that two branches contribute to): the add
+        node turns into the product, which reads ``r`` in its epilogue and adds it to the fp32
+        accumulator before the one rounding of the result.  The scaled product and the sum
+        never make their own trips through memory.  A chain of such sums folds link by link:
+        the second product takes the first sum as its ``r``."""
+        nodes = self._live_nodes()
+        n_users: dict[int, int] = {}
+        for n in nodes:
+            for i in n.inputs:
+                n_users[i.id] = n_users.get(i.id, 0) + 1
+        out_ids = {v.id for v in self.outputs}
+
+        def single_use(v: ir.Value) -> bool:
+            return n_users.get(v.id) == 1 and v.id not in out_ids
+
+        def constant_of(x):
+            """The number an operand stands for: itself, or the fill behind a chain of views."""
+            if not isinstance(x, ir.Value):
+                return float(x)
+            while x.node.kind in ("broadcast", "reshape"):
+                x = x.node.inputs[0]
+            return float(x.node.attrs["value"]) if x.node.kind == "fill" else None
+
+        for n in nodes:
+            if not (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2 and
+                    all(isinstance(x, ir.Value) for x in n.attrs["operands"])):
+                continue
+            out = n.outputs[0]
+            for m, r in ((n.inputs[1], n.inputs[0]), (n.inputs[0], n.inputs[1])):
+                alpha, mm = 1.0, m.node
+                if mm.kind == "ew" and mm.fn == "mul" and single_use(m):
+                    # (x @ W) * c with c a number or a broadcast constant
+                    xs = mm.attrs["operands"]
+                    scaled = None
+                    for x, other in ((xs[0], xs[1]), (xs[1], xs[0])):
+                        if (isinstance(x, ir.Value) and x.node.kind == "matmul" and
+                                x.dtype is m.dtype and x.shape == m.shape and
+                                constant_of(other) is not None):
+                            scaled = (x, constant_of(other))
+                            break
+                    if scaled is None:
+                        continue
+                    m, alpha = scaled
+                    mm = m.node
+                at = mm.attrs or {}
+                if alpha != 1.0 and "bias_in" in at:
+                    continue  # (the kernel scales the product only, not a bias folded earlier)
+                if not (mm.kind == "matmul" and len(mm.outputs) == 1 and single_use(m) and
+                        "res_in" not in at and not at.get("act") and
+                        r.shape == out.shape and r.dtype is out.dtype and r.node.kind != "fill" and
+                        self._epilogue_ok(mm, out)):
+                    continue
+                n.kind, n.fn = "matmul", None
+                n.inputs = list(mm.inputs) + [r]
+                n.attrs = dict(at, res_in=len(mm.inputs), alpha=alpha * at.get("alpha", 1.0))
                 break
 
     def _fold_activation_into_matmul(self) -> None:
@@ -739,7 +800,8 @@ class Planner:
                     users.setdefault(i.id, []).append(n)
         out_ids = {v.id for v in self.outputs}
         for mm in nodes:
-            if mm.kind != "matmul" or len(mm.outputs) != 1 or (mm.attrs or {}).get("act"):
+            if (mm.kind != "matmul" or len(mm.outputs) != 1 or (mm.attrs or {}).get("act") or
+                    "res_in" in (mm.attrs or {})):  # (the residual joins after the activation)
                 continue
             h = mm.outputs[0]
             us = users.get(h.id, [])
@@ -1203,6 +1265,11 @@ class Planner:
         at = n.attrs or {}
         if "bias_in" in at:
             epi["bias"] = self._contig(n.inputs[at["bias_in"]])
+        if "res_in" in at:
+            epi["residual"] = self._contig(n.inputs[at["res_in"]])
+            epi["res_op"] = "add"
+        if at.get("alpha", 1.0) != 1.0:
+            epi["alpha"] = at["alpha"]
         if at.get("act"):
             epi["act"] = at["act"]
             if len(n.outputs) > 1:
@@ -1236,7 +1303,9 @@ class Planner:
             self.skip_nodes.add(red.pos)
             self._emit_plain_gemm(ra, rb, pa, pb, M, N, K * batch, red.outputs[0])
             return
-        c_strides = self._matmul_out_layout(out) if "aux_value" not in epi else contiguous_strides(out.shape)
+        # (a second result or a residual is laid out like the product: both plain row-major then)
+        c_strides = self._matmul_out_layout(out) if not ("aux_value" in epi or "residual" in epi) \
+            else contiguous_strides(out.shape)
         gc = self._batch_groups(out.shape[:-2], c_strides[:-2])
         # one (outer, inner) split of the batch index has to serve A, B and C
         split = None
@@ -1291,7 +1360,8 @@ class Planner:
             epi, a=ra, b=rb, dst=dst, M=M, N=N, K=K, batch=batch, batch_inner=inner,
             a_bs=a_bs, a_rs=pa[1], a_cs=pa[2], b_bs=b_bs, b_rs=pb[1], b_cs=pb[2],
             a_bs2=a_bs2, b_bs2=b_bs2, c_bs2=c_bs2,
-            ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N, alpha=1.0)))
+            ldc=c_strides[-2] if out.rank >= 2 else N, c_bs=c_bs if batch > 1 else M * N,
+            alpha=epi.get("alpha", 1.0))))
 
     @staticmethod
     def _split_k(M: int, N: int, K: int, dtype: DType, a_k_contiguous: bool = False) -> int:
@@ -1317,6 +1387,7 @@ class Planner:
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
         epi = dict(epi or {})
+        common["alpha"] = epi.get("alpha", 1.0)
         if ks == 1 or epi:  # (a product with a folded epilogue is never split)
             writes = [dst.buf]
             if "aux_value" in epi:
@@ -2077,6 +2148,9 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     pre._rematerialize_masks()
     pre._fold_bias_into_matmul()
     from .. import config
+    if config.FOLD_RESIDUAL:
+        pre._fold_sum_into_matmul()
+        pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)
     if config.FOLD_ACTIVATION:
         pre._fold_activation_into_matmul()
     outputs = pre.outputs

@@ -39,6 +39,13 @@ _LORA_LOW_RANK_ORDER: ContextVar[bool] = ContextVar("LORA_LOW_RANK_ORDER",
 _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
                                                 default=_env_flag("NBK_FOLD_ACTIVATION", False))
 
+# r + (x @ W) * alpha as one product whose epilogue reads r.  Off: measured on the LoRA decoder
+# step, the epilogue's read of a full-size r (it starts when a tile's matrix work is over and
+# nothing overlaps it) costs 33-41 us per 8192 x 2048 result where the separate sum kernel
+# takes 17 us (32.4 -> 33.8 ms per step with the fold on)
+_FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
+                                              default=_env_flag("NBK_FOLD_RESIDUAL", False))
+
 # x @ W for an NF4-coded W as one product that reads the codes (one byte per weight) and
 # dequantises them on the way into LDS; off: dequantise into a dense weight first
 _FUSED_NF4_MATMUL: ContextVar[bool] = ContextVar("FUSED_NF4_MATMUL",
@@ -56,6 +63,7 @@ _FLAGS = {
     "FUSED_ATTENTION": _FUSED_ATTENTION,
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
+    "FOLD_RESIDUAL": _FOLD_RESIDUAL,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
     "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,
 }

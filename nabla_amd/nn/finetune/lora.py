@@ -52,7 +52,9 @@ def lora_linear(x: Tensor, frozen_weight: Tensor, adapter: dict[str, Tensor],
     if not config.LORA_LOW_RANK_ORDER:
         return base + x @ lora_delta(adapter, alpha=alpha)
     down, up, inv_rank = _factors(adapter)
-    return base + ((x @ down) @ up) * (alpha * inv_rank)
+    # (the scale goes on the small factor, as the reference puts it on the update: the product
+    # with the activations then needs no pass of its own for it)
+    return base + (x @ down) @ (up * (alpha * inv_rank))
 
 
 def merge_lora_weight(frozen_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:

@@ -96,6 +96,6 @@ def qlora_linear(x: Tensor, qweight: dict[str, Any], adapter: dict[str, Tensor],
         down, up = cast_adapter["A"], cast_adapter["B"]
         scale = alpha / float(int(down.shape[1]))
         if config.LORA_LOW_RANK_ORDER:
-            return base + ((xc @ down) @ up) * scale
+            return base + (xc @ down) @ (up * scale)
         return base + xc @ ((down @ up) * scale)
     return lora_linear(xc, dequantize_nf4(qweight, dtype=compute_dtype), cast_adapter, alpha=alpha)

@@ -630,3 +630,28 @@ def test_integers_above_2_pow_24_are_exact(emulator):
     """Integer tensors compute in integer registers: no value passes through fp32."""
     from integer_cases import check_large_integers
     check_large_integers(nb)
+
+
+def test_sum_with_a_product_folds_into_its_epilogue_when_asked(emulator):
+    """``r + x @ W + b`` becomes one product that reads ``r`` and ``b`` in its epilogue under
+    ``FOLD_RESIDUAL`` (off by default: the epilogue read measured slower than the sum kernel);
+    the numbers are the unfused ones up to the rounding points that disappear."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(12)
+    x, w = rng.standard_normal((6, 40, 32)).astype(np.float32), rng.standard_normal((32, 24)).astype(np.float32)
+    r, b = rng.standard_normal((6, 40, 24)).astype(np.float32), rng.standard_normal((1, 24)).astype(np.float32)
+    want = r + x @ w + b
+
+    def f():
+        return T(r) + T(x) @ T(w) + T(b)
+
+    plain = f().numpy()
+    with config.flag("FOLD_RESIDUAL", True):
+        engine.clear_plan_cache()
+        folded = f().numpy()
+        kinds = [[s.kind for s in bp.plan.steps] for bp in engine._PLAN_CACHE.values()]
+    engine.clear_plan_cache()
+    assert ["gemm"] in kinds, kinds
+    np.testing.assert_allclose(plain, want, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(folded, want, rtol=1e-5, atol=1e-5)
