@@ -267,6 +267,21 @@ def launch_flops(step) -> float:
     return 0.0
 
 
+def rowprog_bytes(step) -> float:
+    """Algorithmic bytes of one row-program launch: every distinct operand read or written once
+    (an operand that is broadcast along an axis counts the elements it has, not the ones it is
+    read as)."""
+    a = step.attrs
+    total = 0.0
+    for o in a["operands"]:
+        n = a["C"] if o.col_stride != 0 else 1
+        for d, st in zip(a["lead"], o.lead_strides):
+            if st != 0:
+                n *= d
+        total += n * o.dtype.size_in_bytes
+    return total
+
+
 def launch_label(step) -> str:
     a, k = step.attrs, step.kind
     if k == "gemm":
@@ -331,12 +346,18 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
         spec.bound.run(inputs)
     sync()
     wall_plan = time.perf_counter() - t0
+    row_dur = {}
     if not single:
         n2 = min(steps, 20)
+        if w["bound"] == "mfma":
+            timer.kinds.add("rowprog")  # (reported beside the matrix kernels, not counted with them)
         for _ in range(n2):
             spec.bound.run(inputs, timer=timer)
         sync()
         dur = timer.durations_ms()
+        if w["bound"] == "mfma":
+            row_dur = {k: v for k, v in dur.items() if k[1] == "rowprog"}
+            dur = {k: v for k, v in dur.items() if k[1] != "rowprog"}
         kernel_timing = (f"second pass of {n2} steps, plain launches bracketed by HIP events on the "
                          "launch stream (the timed region replays the step as one HIP graph, inside "
                          "which events cannot be recorded)")
@@ -379,6 +400,26 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
                        "tflops": round(tf, 1), "frac": round(tf / peak, 4)})
         roofline["by_kernel"] = by[:12]
         roofline["counted_flops_per_step"] = sum(g[2] for g in groups.values())
+        if row_dur:
+            # the fused elementwise / normalisation / loss kernels of the same step against the
+            # HBM roofline: algorithmic bytes of each launch over its own duration
+            rows = []
+            for (si, _), ms in row_dur.items():
+                st = plan.steps[si]
+                rows.append((ms, rowprog_bytes(st), f"rows{tuple(st.attrs['lead'])} x {st.attrs['C']}, "
+                             f"{len(st.attrs['operands'])} operands, {len(st.attrs['ins'])} instructions"))
+            rows.sort(key=lambda r: -r[0])
+            big = [r for r in rows if r[1] >= 32e6]  # launches that move at least 32 MB
+            t_all, b_all = sum(r[0] for r in rows), sum(r[1] for r in rows)
+            t_big, b_big = sum(r[0] for r in big), sum(r[1] for r in big)
+            roofline["row_kernels"] = {
+                "launches_per_step": len(rows), "ms_per_step": round(t_all, 4),
+                "gb_per_s": round(b_all / (t_all * 1e-3) / 1e9, 1) if t_all else 0.0,
+                "launches_over_32MB": len(big),
+                "gb_per_s_over_32MB": round(b_big / (t_big * 1e-3) / 1e9, 1) if t_big else 0.0,
+                "frac_of_hbm_peak_over_32MB": round(b_big / (t_big * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if t_big else 0.0,
+                "slowest": [{"kernel": r[2], "us": round(r[0] * 1e3, 1), "gb_per_s": round(r[1] / (r[0] * 1e-3) / 1e9, 1)}
+                            for r in rows[:6]]}
     res = {"workload": w["name"], "value": round(steps / wall, 3), "unit": "steps/s",
            "ms_per_step": round(wall / steps * 1e3, 4),
            "plan_ms_per_step": round(wall_plan / steps * 1e3, 4),

@@ -46,6 +46,12 @@ _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
 _FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
                                               default=_env_flag("NBK_FOLD_RESIDUAL", False))
 
+# the backward pass of the exact GELU computes GELU'(x) from the kept pre-activation, in the
+# kernel that multiplies it with the cotangent; off: the forward kernel stores GELU'(x) as a
+# second full-size result and the backward kernel reads it
+_GELU_BACKWARD_FROM_INPUT: ContextVar[bool] = ContextVar(
+    "GELU_BACKWARD_FROM_INPUT", default=_env_flag("NBK_GELU_BACKWARD_FROM_INPUT", True))
+
 # x @ W for an NF4-coded W as one product that reads the codes (one byte per weight) and
 # dequantises them on the way into LDS; off: dequantise into a dense weight first
 _FUSED_NF4_MATMUL: ContextVar[bool] = ContextVar("FUSED_NF4_MATMUL",
@@ -64,6 +70,7 @@ _FLAGS = {
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
+    "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
     "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,
 }

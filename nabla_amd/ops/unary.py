@@ -12,7 +12,7 @@ import math
 from ..backend import ir
 from ..core.dtype import DType
 from ..core.tensor import Tensor
-from .base import AxisOp, UnaryOperation, ensure_tensor
+from .base import AxisOp, Operation, UnaryOperation, ensure_tensor
 
 
 def _ew1(fn: str):
@@ -228,6 +228,13 @@ class GeluOp(UnaryOperation):
         # kernel shares them too
         return _gelu_grad_op([primal], {})[0]
 
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        from .. import config
+        approx = kwargs.get("approximate", "none")
+        if config.GELU_BACKWARD_FROM_INPUT and approx in ("none", False):
+            return [_gelu_backward_op([primals[0], cotangents[0]], {})[0]]
+        return super().vjp_rule(primals, cotangents, outputs, kwargs)
+
 
 class GeluGradOp(UnaryOperation):
     """``Phi(x) + x * phi(x)``, the derivative of the exact GELU."""
@@ -244,6 +251,39 @@ class GeluGradOp(UnaryOperation):
         x = primal
         pdf = div(exp(neg(div(mul(x, x), 2.0))), math.sqrt(2.0 * math.pi))
         return mul(pdf, sub(2.0, mul(x, x)))
+
+
+class GeluBackwardOp(Operation):
+    """(x, g) -> g * GELU'(x), with the derivative computed where the cotangent is: the forward
+    kernel then writes the activation only, not a second tensor of the same size that holds the
+    derivative until the backward pass (the pre-activation is kept instead, which exists
+    anyway)."""
+
+    @property
+    def name(self) -> str:
+        return "gelu_backward"
+
+    def compute_physical_shape(self, args, kwargs, output_sharding=None):
+        x = args[0]
+        return [tuple(x.shape)], [x.dtype], [x.device]
+
+    def kernel(self, args, kwargs):
+        x, g = args
+        return [ir.ew("mul", g, ir.ew("dgelu", ir.pin_after(x, g)))]
+
+    def vjp_rule(self, primals, cotangents, outputs, kwargs):
+        from .binary import mul
+        x, g = primals
+        d1 = _gelu_grad_op([x], {})[0]
+        d2 = _gelu_grad_op._derivative(x, None)
+        return [mul(cotangents[0], mul(g, d2)), mul(cotangents[0], d1)]
+
+    def jvp_rule(self, primals, tangents, outputs, kwargs):
+        from .binary import add, mul
+        x, g = primals
+        d1 = _gelu_grad_op([x], {})[0]
+        d2 = _gelu_grad_op._derivative(x, None)
+        return [add(mul(tangents[0], mul(g, d2)), mul(tangents[1], d1))]
 
 
 def _softmax_ir(x, axis: int, log: bool):
@@ -346,6 +386,7 @@ _log_op, _sqrt_op, _rsqrt_op, _erf_op = LogOp(), SqrtOp(), RsqrtOp(), ErfOp()
 _tanh_op, _sigmoid_op, _gelu_op, _cast_op = TanhOp(), SigmoidOp(), GeluOp(), CastOp()
 _silu_op = SiluOp()
 _gelu_grad_op = GeluGradOp()
+_gelu_backward_op = GeluBackwardOp()
 _softmax_native, _logsoftmax_native = _SoftmaxNativeOp(), _LogSoftmaxNativeOp()
 
 

@@ -588,12 +588,13 @@ def test_gelu_of_a_linear_layer_is_folded_into_the_product(emulator):
     from nabla_amd import config
     from nabla_amd.core import engine
     from oracle import ops as O
-    tok = config.set_flag("FOLD_ACTIVATION", True)
-    try:
-        _check_gelu_fold(engine, O)
-    finally:
-        config.reset_flag("FOLD_ACTIVATION", tok)
-        engine.clear_plan_cache()
+    # (the fold keeps the derivative as the product's second result: the alternative to
+    # recomputing it from the pre-activation in the backward kernel)
+    with config.flag("FOLD_ACTIVATION", True), config.flag("GELU_BACKWARD_FROM_INPUT", False):
+        try:
+            _check_gelu_fold(engine, O)
+        finally:
+            engine.clear_plan_cache()
 
 
 def _check_gelu_fold(engine, O):
@@ -655,3 +656,32 @@ def test_sum_with_a_product_folds_into_its_epilogue_when_asked(emulator):
     assert ["gemm"] in kinds, kinds
     np.testing.assert_allclose(plain, want, rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(folded, want, rtol=1e-5, atol=1e-5)
+
+
+def test_gelu_backward_recomputes_the_derivative_where_the_cotangent_is(emulator):
+    """Two ways to get gelu's derivative to the backward pass -- recomputed from the pre-activation
+    where the cotangent is (the default), or stored by the forward kernel -- agree with the
+    float64 oracle, second order included."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    from oracle import ops as O
+    rng = np.random.default_rng(78)
+    x = rng.standard_normal((12, 40))
+
+    def loss_fn(t):
+        return nb.reduce_sum(nb.gelu(t * 1.5) * T(np.arange(40, dtype=np.float32)))
+
+    vx = O.V(x)
+    want = O.reduce_sum(O.gelu(vx * 1.5) * O.V(np.arange(40, dtype=np.float64)))
+    (wg,) = O.grad_of(want, [vx])
+    for flag in (True, False):
+        with config.flag("GELU_BACKWARD_FROM_INPUT", flag):
+            engine.clear_plan_cache()
+            loss, g = nb.value_and_grad(loss_fn)(T(x.astype(np.float32)))
+            nb.realize_all(loss, g)
+            np.testing.assert_allclose(g.numpy(), wg, rtol=2e-5, atol=2e-6)
+    engine.clear_plan_cache()
+    # second order: d/dx sum(gelu'(x)) = sum gelu''(x), gelu''(x) = phi(x) (2 - x^2)
+    h = nb.grad(lambda t: nb.reduce_sum(nb.grad(lambda u: nb.reduce_sum(nb.gelu(u)))(t)))(T(x.astype(np.float32)))
+    pdf = np.exp(-0.5 * x * x) / np.sqrt(2 * np.pi)
+    np.testing.assert_allclose(h.numpy(), pdf * (2 - x * x), rtol=2e-4, atol=2e-5)
