@@ -17,7 +17,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 
     L = lib.load()
     hdr = HEADER.read_text()
-    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(nbk_[a-z0-9_]+)\s*\(", hdr, re.M))
+    declared = set(re.findall(r"^\s*(?:int|int64_t|uint64_t|const char\*)\s+(nbk_[a-z0-9_]+)\s*\(", hdr, re.M))
     assert len(declared) >= 20
     for name in sorted(declared):
         assert hasattr(L, name), f"{name} is declared in nbk.h but not exported"
@@ -42,32 +42,43 @@ def test_isa_numbers_match_header():
     assert lim["NVEC"] == isa.NVEC and lim["NSCL"] == isa.NSCL and lim["NACC"] == isa.NACC
 
 
+#: every struct of the header and its ctypes mirror
+STRUCTS = {
+    "nbk_operand": "Operand", "nbk_ins": "Ins", "nbk_rowprog": "RowProg", "nbk_gemm_desc": "GemmDesc",
+    "nbk_gemm_nf4_desc": "GemmNf4Desc", "nbk_conv_desc": "ConvDesc", "nbk_pool_desc": "PoolDesc",
+    "nbk_attn_desc": "AttnDesc", "nbk_attn_tensor": "AttnTensor", "nbk_reduce_task": "ReduceTask",
+    "nbk_opt_tensor": "OptTensor", "nbk_adamw_desc": "AdamwDesc", "nbk_sgd_desc": "SgdDesc",
+    "nbk_tensor": "TensorDesc",
+}
+
+
 def test_struct_layouts_match_the_c_compiler(tmp_path):
+    """Size of every struct and offset of every field, as gcc lays the header out, against the
+    ctypes mirrors (a field named ``in`` in C is ``in_`` in Python)."""
     from nabla_amd.backend import lib
 
+    hdr = HEADER.read_text()
+    declared = set(re.findall(r"typedef struct (nbk_[a-z0-9_]+) \{", hdr))
+    assert declared == set(STRUCTS), declared ^ set(STRUCTS)
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "nbk.h"', "int main(void) {"]
+    for cname, pyname in STRUCTS.items():
+        cls = getattr(lib, pyname)
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for field, _ in cls._fields_:
+            cfield = field[:-1] if field.endswith("_") else field
+            lines.append(f'  printf("{cname}.{field} %zu\\n", offsetof({cname}, {cfield}));')
+    lines += ["  return 0;", "}"]
     src = tmp_path / "sizes.c"
-    src.write_text(
-        '#include <stdio.h>\n#include <stddef.h>\n#include "nbk.h"\n'
-        "int main(void) {\n"
-        '  printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(nbk_rowprog), sizeof(nbk_operand),\n'
-        "         sizeof(nbk_ins), sizeof(nbk_gemm_desc), sizeof(nbk_conv_desc), sizeof(nbk_pool_desc),\n"
-        "         sizeof(nbk_tensor));\n"
-        '  printf("%zu %zu %zu %zu\\n", offsetof(nbk_rowprog, imm), offsetof(nbk_rowprog, operand),\n'
-        "         offsetof(nbk_rowprog, ins), offsetof(nbk_gemm_desc, alpha));\n"
-        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(nbk_attn_desc), sizeof(nbk_attn_tensor),\n'
-        "         sizeof(nbk_reduce_task), offsetof(nbk_attn_desc, scale), offsetof(nbk_reduce_task, dtype_in));\n"
-        "  return 0;\n}\n")
+    src.write_text("\n".join(lines) + "\n")
     exe = tmp_path / "sizes"
     subprocess.run(["gcc", f"-I{ROOT / 'include'}", str(src), "-o", str(exe)], check=True)
-    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()
-    sizes = [int(x) for x in out]
-    assert sizes[:7] == [C.sizeof(lib.RowProg), C.sizeof(lib.Operand), C.sizeof(lib.Ins),
-                         C.sizeof(lib.GemmDesc), C.sizeof(lib.ConvDesc), C.sizeof(lib.PoolDesc),
-                         C.sizeof(lib.TensorDesc)]
-    assert sizes[7:11] == [lib.RowProg.imm.offset, lib.RowProg.operand.offset, lib.RowProg.ins.offset,
-                           lib.GemmDesc.alpha.offset]
-    assert sizes[11:] == [C.sizeof(lib.AttnDesc), C.sizeof(lib.AttnTensor), C.sizeof(lib.ReduceTask),
-                          lib.AttnDesc.scale.offset, lib.ReduceTask.dtype_in.offset]
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout
+    got = dict((k, int(v)) for k, v in (line.split() for line in out.splitlines()))
+    for cname, pyname in STRUCTS.items():
+        cls = getattr(lib, pyname)
+        assert got[cname] == C.sizeof(cls), (cname, got[cname], C.sizeof(cls))
+        for field, _ in cls._fields_:
+            assert got[f"{cname}.{field}"] == getattr(cls, field).offset, (cname, field)
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
