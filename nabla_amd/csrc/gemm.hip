@@ -21,6 +21,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 // 16-byte register / LDS unit.  A native vector (an SSA value), not the uint4 struct:
 // arrays of structs that are filled by loads and drained by stores are turned into
 // memcpy through a stack slot, which puts the staging registers in scratch.
@@ -294,19 +295,17 @@ extern __shared__ __align__(16) u32x4 gemm_lds[];
 // Epilogue shared by the bf16 kernels (the caller has passed a workgroup barrier: the tile
 // buffers are free).
 // EPI: 0 plain, 1 bias only (as lean as the plain form), 2 bias / activation / residual.
-template <int TM, int TN, int WN, bool FAST, int EPI>
-__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
-                                              int64_t n0, int wm, int wn, int64_t c_off, int wave,
-                                              int lane) {
-  const int li = lane & 31, kg = lane >> 5;
-  // Epilogue.  D[i][j] of a 32x32 MFMA tile lives in lane (j, (i / 4) % 2),
-  // register (i / 8) * 4 + i % 4.  Each wave passes its accumulators through a
-  // private LDS slab, 32 rows at a time, so that C is written as whole
-  // 16-byte (bf16) / 32-byte (fp32) pieces of a row: 8 columns per lane.
-  // The plain form (no bias / activation / residual) is a separate
-  // instantiation: the fused form carries erf() bodies, and an epilogue that does
-  // not fit the instruction cache costs more than the whole K loop of a short GEMM.
-  constexpr int SLAB_LD = WN + 4;  // floats per slab row (padding spreads the two row groups)
+// Each wave passes its accumulators through a private LDS slab, a band of 32 rows of its tile
+// at a time (`scatter(band, slab)` writes the band's accumulators there, row-major with a
+// pitch of WN + 4 floats), so that C is written as whole 16-byte (bf16) / 32-byte (fp32)
+// pieces of a row: 8 columns per lane.  The plain form (no bias / activation / residual)
+// is a separate instantiation: the fused form carries erf() bodies, and an epilogue that does
+// not fit the instruction cache costs more than the whole K loop of a short GEMM.
+template <int TM, int WN, bool FAST, int EPI, typename Scatter>
+__device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const GemmArgs& g, int64_t m0,
+                                                    int64_t n0, int wm, int wn, int64_t c_off, int wave,
+                                                    int lane) {
+  constexpr int SLAB_LD = WN + 4;  // floats per slab row (padding spreads the row groups)
   float* slab = (float*)gemm_lds + wave * (32 * SLAB_LD);
   const bool out_f32 = g.dtype_c == NBK_F32;
   constexpr int LANES_PER_ROW = WN / 8;        // each lane writes 8 consecutive columns
@@ -341,13 +340,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
   }
   static_for<TM>([&](auto ti) {
     constexpr int i = decltype(ti)::value;
-    static_for<TN>([&](auto tj) {
-      constexpr int j = decltype(tj)::value;
-      const f32x16 a = acc[i][j];
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        slab[((r >> 2) * 8 + kg * 4 + (r & 3)) * SLAB_LD + j * 32 + li] = a[r];
-    });
+    scatter(ti, slab);
     // the slab is private to the wave: no workgroup barrier, only LDS ordering
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     auto one_pass = [&](int pass, const uint4 u) {
@@ -443,6 +436,49 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // slab reads done before the next tile row overwrites it
   });
+}
+
+// 32x32 MFMA blocks: D[i][j] lives in lane (j, (i / 4) % 2), register (i / 8) * 4 + i % 4.
+template <int TM, int TN, int WN, bool FAST, int EPI>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
+                                              int64_t n0, int wm, int wn, int64_t c_off, int wave,
+                                              int lane) {
+  const int li = lane & 31, kg = lane >> 5;
+  gemm_epilogue_bands<TM, WN, FAST, EPI>(
+      [&](auto ti, float* slab) {
+        constexpr int i = decltype(ti)::value;
+        static_for<TN>([&](auto tj) {
+          constexpr int j = decltype(tj)::value;
+          const f32x16 a = acc[i][j];
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            slab[((r >> 2) * 8 + kg * 4 + (r & 3)) * (WN + 4) + j * 32 + li] = a[r];
+        });
+      },
+      g, m0, n0, wm, wn, c_off, wave, lane);
+}
+
+// 16x16 MFMA blocks: D[i][j] lives in lane (j, i / 4), register i % 4; a band is two block rows.
+// (Storing straight from the registers, with the product transposed so that a lane holds four
+// consecutive columns, was measured: the 32-byte row pieces it writes make the epilogue slower
+// than the slab round trip with its whole 128-byte lines.)
+template <int TM, int TN, int WN, bool FAST, int EPI>
+__device__ __forceinline__ void gemm_epilogue(f32x4 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
+                                              int64_t n0, int wm, int wn, int64_t c_off, int wave,
+                                              int lane) {
+  static_assert(TM % 2 == 0, "block rows per wave tile");
+  const int p = lane & 15, q = lane >> 4;
+  gemm_epilogue_bands<TM / 2, WN, FAST, EPI>(
+      [&](auto ti, float* slab) {
+        constexpr int i = decltype(ti)::value;
+        static_for<2 * TN>([&](auto tb) {
+          constexpr int ib = decltype(tb)::value / TN, j = decltype(tb)::value % TN;
+          const f32x4 a = acc[2 * i + ib][j];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) slab[(ib * 16 + 4 * q + r) * (WN + 4) + j * 16 + p] = a[r];
+        });
+      },
+      g, m0, n0, wm, wn, c_off, wave, lane);
 }
 
 // NW waves: 4 as 2 x 2, or 8 as 2 x 4 (two waves per SIMD, each with half the accumulators:
@@ -679,11 +715,17 @@ __device__ __forceinline__ int dl_swz_kc(int row, int c) {
   return row * 8 + (c ^ (row & 7) ^ ((row >> 3) & 1));
 }
 __device__ __forceinline__ int dl_seg_xor(int k) { return (k & 3) ^ (((k & 3) << 1) & 7); }
+// The 16x16x32 form reads k-rows k .. k + 3 and k + 8 .. k + 11 of one 32-byte segment in
+// half a wave: bit 3 of k joins the swizzle.
+template <bool MI16>
+__device__ __forceinline__ int dl_seg_xor_of(int k) {
+  return MI16 ? dl_seg_xor(k) ^ ((k >> 3) & 1) : dl_seg_xor(k);
+}
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void glb_void_t;
 
-template <int ROWS, bool KC, int NW>
+template <int ROWS, bool KC, int NW, bool MI16 = false>
 struct DirectLoader {
   // ROWS * 8 chunks, 64 per wave instruction, dealt to the waves in consecutive runs
   static constexpr int N = ROWS / (8 * NW);
@@ -715,7 +757,7 @@ struct DirectLoader {
 #pragma unroll
       for (int j = 0; j < N; ++j) {
         const int l = (first + j) * 64 + lane;
-        const int k = l / NC, c = (l % NC) ^ (dl_seg_xor(k) << 1);
+        const int k = l / NC, c = (l % NC) ^ (dl_seg_xor_of<MI16>(k) << 1);
         const int64_t r = c * 8 < last ? c * 8 : last;
         voff[j] = (int)(k * cs * 2 + r * 2);
       }
@@ -734,14 +776,21 @@ struct DirectLoader {
   }
 };
 
-// KSS: k-steps (of 16) per fragment set.  A step of KSS k-steps is multiplied out of one
+// MI16: the matrix instruction is v_mfma_f32_16x16x32_bf16 (blocks of 16 x 16, 32 deep) instead
+// of v_mfma_f32_32x32x16_bf16 (32 x 32, 16 deep).  Same LDS traffic and register budget; the
+// 16 x 16 form does the same arithmetic for about a tenth less power, and these products run at
+// the power limit (the clock under MFMA load settles where the limit puts it), so it is the
+// faster one with two waves per SIMD to keep its shorter instructions back to back.
+// KSS: k-steps (one MFMA deep) per fragment set.  A step of KSS k-steps is multiplied out of one
 // set while the other is filled for the next step; small wave tiles take 2, so that a read has
 // more than a handful of MFMAs to land.
-template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS>
+template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS, bool MI16>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g) {
   constexpr int WGN = NW / 2;
   constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
-  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int FM = MI16 ? 16 : 32;          // rows / columns of an MFMA block
+  constexpr int KQ = MI16 ? 32 : 16;          // depth of one MFMA
+  constexpr int TM = WM / FM, TN = WN / FM;
   constexpr int CA = BM * 8, TILE_CHUNKS = (BM + BN) * 8;
   int tm_i, tn_i;
   gemm_tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm_i, tn_i);
@@ -755,27 +804,48 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   const int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
   const int li = lane & 31, kg = lane >> 5;
 
-  f32x16 acc[TM][TN];
+  using Acc = std::conditional_t<MI16, f32x4, f32x16>;
+  Acc acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = (f32x16)(0.f);
+    for (int j = 0; j < TN; ++j) acc[i][j] = (Acc)(0.f);
 
-  DirectLoader<BM, A_KC, NW> la;
-  DirectLoader<BN, B_KC, NW> lb;
+  using LA = DirectLoader<BM, A_KC, NW, MI16>;
+  using LB = DirectLoader<BN, B_KC, NW, MI16>;
+  LA la;
+  LB lb;
   la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
   lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
   const int64_t nk = g.K / 64;
   la.issue(gemm_lds, 0);
   lb.issue(gemm_lds + CA, 0);
 
-  // Fragment addresses, one per 32-row block of the wave tile.
+  // Fragment addresses, one per block row / column of the wave tile.  32 x 32 x 16:
   //   K-contiguous: byte address 16 ((row * 8 | t) ^ (2 ks)), t = kg ^ (row % 8) ^ (row / 8 % 2);
   //   row-contiguous: byte address of this lane's 8 bytes in the transposing read of k-step 0,
   //     first half; the k-step and the half are constant offsets.  Lane p of group q = lane / 16
   //     points at k-row 8 (q / 2) + p / 4, rows 16 (q % 2) + 4 (p % 4) .. + 4 of the block.
+  // 16 x 16 x 32 (lane p of group q holds k = 8 q .. + 8 of row p):
+  //   K-contiguous: 16 ((row * 8 | t) ^ (4 ks)), t = q ^ (row % 8) ^ (row / 8 % 2);
+  //   row-contiguous: k-row 8 q + p / 4, rows 4 (p % 4) .. + 4 of the block.
   int a_addr[TM], b_addr[TN];
-  {
+  if constexpr (MI16) {
+    const int p = lane & 15, q = lane >> 4;
+    const int kl = 8 * q + (p >> 2), sx = dl_seg_xor_of<true>(kl);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm + i * 16 + p;
+      if (A_KC) a_addr[i] = (row * 8 + (q ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
+      else a_addr[i] = kl * (BM * 2) + ((((wm >> 4) + i) ^ sx) * 32) + 8 * (p & 3);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn + j * 16 + p;
+      if (B_KC) b_addr[j] = (CA + row * 8 + (q ^ (row & 7) ^ ((row >> 3) & 1))) * 16;
+      else b_addr[j] = CA * 16 + kl * (BN * 2) + ((((wn >> 4) + j) ^ sx) * 32) + 8 * (p & 3);
+    }
+  } else {
     const int p = lane & 15, q = lane >> 4;
     const int kl = 8 * (q >> 1) + (p >> 2), sx = dl_seg_xor(p >> 2);
 #pragma unroll
@@ -795,7 +865,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   }
 
   bf16x8 fa[2][KSS * TM], fb[2][KSS * TN];
-  constexpr int NSTEP = 4 / KSS;
+  constexpr int NSTEP = 64 / KQ / KSS;
   static_assert(NSTEP >= 2 && NSTEP % 2 == 0, "steps per tile");
   constexpr int NFRAG = KSS * (TM + TN), NMFMA = KSS * TM * TN;  // per step
   // read fragment r of step `step` from `tile` into set SET; order of use by the MFMAs
@@ -807,21 +877,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
     const int ks = step * KSS + KL;
     if constexpr (R < TM) {
       if constexpr (A_KC) {
-        int sel = ks * 32;
+        int sel = ks * (KQ * 2);
         asm volatile("" : "+s"(sel));  // recomputed at every read: hoisted variants would spill
         fa[SET][KL * TM + R] = lds_read_b128(lds_addr(tile) + (a_addr[R] ^ sel));
       } else {
         const uint32_t p = lds_addr(tile) + a_addr[R];
-        fa[SET][KL * TM + R] = lds_read_tr_pair(p, ks * 16 * (BM * 2), (ks * 16 + 4) * (BM * 2));
+        fa[SET][KL * TM + R] = lds_read_tr_pair(p, ks * KQ * (BM * 2), (ks * KQ + 4) * (BM * 2));
       }
     } else {
       if constexpr (B_KC) {
-        int sel = ks * 32;
+        int sel = ks * (KQ * 2);
         asm volatile("" : "+s"(sel));
         fb[SET][KL * TN + R - TM] = lds_read_b128(lds_addr(tile) + (b_addr[R - TM] ^ sel));
       } else {
         const uint32_t p = lds_addr(tile) + b_addr[R - TM];
-        fb[SET][KL * TN + R - TM] = lds_read_tr_pair(p, ks * 16 * (BN * 2), (ks * 16 + 4) * (BN * 2));
+        fb[SET][KL * TN + R - TM] = lds_read_tr_pair(p, ks * KQ * (BN * 2), (ks * KQ + 4) * (BN * 2));
       }
     }
   };
@@ -838,8 +908,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   auto mfma = [&](auto set, auto q) {
     constexpr int SET = decltype(set)::value, Q = decltype(q)::value;
     constexpr int kl = Q / (TM * TN), i = Q % (TM * TN) / TN, j = Q % TN;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kl * TM + i], fb[SET][kl * TN + j],
-                                                        acc[i][j], 0, 0, 0);
+    if constexpr (MI16)
+      acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[SET][kl * TM + i], fb[SET][kl * TN + j],
+                                                          acc[i][j], 0, 0, 0);
+    else
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kl * TM + i], fb[SET][kl * TN + j],
+                                                          acc[i][j], 0, 0, 0);
   };
   // step on fragment set SET while set 1 - SET is filled for step `step_next` of `tile`
   auto stage = [&](auto set, const u32x4* tile, int step_next) {
@@ -897,8 +971,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
       // and the reads both touch LDS, so the scheduler would otherwise leave the MFMAs last).
       // (the last pass has no tile kt + 2: it fetches tile nk - 1 again, into a buffer that
       // is not read any more, which keeps this block free of branches)
-      using LA = DirectLoader<BM, A_KC, NW>;
-      using LB = DirectLoader<BN, B_KC, NW>;
       constexpr int NL = LA::N + LB::N, H = NMFMA / 2;
       const int64_t k2 = kt + 2 < nk ? kt + 2 : nk - 1;
       const char* src_a = la.tile_src(k2);
@@ -1381,7 +1453,7 @@ static int launch_bf16(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hip
   return nbk_check_launch("gemm_bf16_kernel");
 }
 
-template <int BM, int BN, int NW, int KSS>
+template <int BM, int BN, int NW, int KSS, bool MI16>
 static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, hipStream_t st) {
   GemmArgs g = a;
   g.tiles_m = (int)((a.M + BM - 1) / BM);
@@ -1393,7 +1465,7 @@ static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, 
   const int epi = (a.residual != nullptr || a.act != NBK_ACT_NONE) ? 2 : (a.bias != nullptr ? 1 : 0);
 #define NBK_LAUNCH_DL(AK, BK_, EP)                                                            \
   do {                                                                                        \
-    auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS>;                                 \
+    auto kern = gemm_bf16_dl_kernel<BM, BN, AK, BK_, EP, NW, KSS, MI16>;                      \
     static bool attr_set = false; /* idempotent, so a race only repeats the call */          \
     if (!attr_set) {                                                                          \
       NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -1528,11 +1600,14 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     // 128 x 128 workgroups per CU overlap better than one 256 x 256)
     // (eight waves on the big tile: 8-16 % faster than four on every shape measured)
     if (big_tiles * 10 >= rounds * cus * 6 && d->M >= 256 && d->N >= 256 && d->K > 128)
-      return launch_bf16_dl<256, 256, 8, 2>(a, akc, bkc, d->batch, st);
+      return launch_bf16_dl<256, 256, 8, 1, true>(a, akc, bkc, d->batch, st);
     // (a 256 x 128 tile was measured and is no faster than 128 x 128 on mid-sized problems:
     // with one workgroup per CU a short K loop is bound by load latency, and two co-resident
     // 128 x 128 workgroups hide it better)
-    return launch_bf16_dl<128, 128, 4, 1>(a, akc, bkc, d->batch, st);
+    // (the 16 x 16 x 32 instruction is 3-8 % faster on every shape and layout of the big tile; on
+    // this one it gains 4-9 % with a row-contiguous operand and loses 5-10 % with two K-contiguous)
+    return !(akc && bkc) ? launch_bf16_dl<128, 128, 4, 1, true>(a, akc, bkc, d->batch, st)
+                         : launch_bf16_dl<128, 128, 4, 1, false>(a, akc, bkc, d->batch, st);
   }
   a.tiles_m = (int)((d->M + 127) / 128);
   a.tiles_n = (int)((d->N + 127) / 128);
