@@ -42,7 +42,7 @@ _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
 # r + (x @ W) * alpha as one product whose epilogue reads r.  Off: measured on the LoRA decoder
 # step, the epilogue's read of a full-size r (it starts when a tile's matrix work is over and
 # nothing overlaps it) costs 33-41 us per 8192 x 2048 result where the separate sum kernel
-# takes 17 us (32.4 -> 33.8 ms per step with the fold on)
+# takes 17 us (29.5 -> 44.9 ms per decoder step with the fold on)
 _FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
                                               default=_env_flag("NBK_FOLD_RESIDUAL", False))
 
