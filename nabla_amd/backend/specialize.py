@@ -135,6 +135,8 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         w("  const bool writer = threadIdx.x == 0;")
         w("  (void)c_pad;")
     else:
+        # FLAT: the launch has a single row (a flat array): no row arithmetic, every operand at offset 0
+        w("template <bool FLAT>")
         w(f"__global__ __launch_bounds__(256) void {name}(const nbk_rowprog P, uint32_t cpr, "
           "uint64_t total_chunks) {")
         w("  const int64_t C = P.C;")
@@ -233,12 +235,13 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         w("  const bool small = total_chunks <= 0xffffffffull;  // 32-bit row arithmetic suffices")
         w("  for (uint64_t g = (uint64_t)blockIdx.x * 256u + threadIdx.x; g < total_chunks; g += stride) {")
         w("    uint32_t row, cc;")
-        w("    if (cpr == 1) { row = (uint32_t)g; cc = 0; }")
+        w("    if (FLAT) { row = 0; cc = (uint32_t)g; }")
+        w("    else if (cpr == 1) { row = (uint32_t)g; cc = 0; }")
         w("    else if (total_chunks <= cpr) { row = 0; cc = (uint32_t)g; }")
         w("    else if (small) { row = (uint32_t)g / cpr; cc = (uint32_t)g - row * cpr; }")
         w("    else { row = (uint32_t)(g / cpr); cc = (uint32_t)(g - (uint64_t)row * cpr); }")
         w("    uint32_t lead_idx[4] = {0, 0, 0, 0};")
-        w("    if (P.n_lead > 0) " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
+        w("    if (!FLAT && P.n_lead > 0) " + decomp.replace("ROW", "row").replace("LI", "lead_idx"))
         w("    const bool writer = cc == 0;")
         w("    const int64_t col = (int64_t)cc << 2;")
         w("    const int64_t left = C - col;")
@@ -252,7 +255,9 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
         else:
             # per-lane rows: with at most one leading dim an offset is one multiply-add
             w("    int64_t " + ", ".join(f"off{k}" for k in range(len(ops))) + ";")
-            w("    if (P.n_lead <= 1) {")
+            w("    if (FLAT) {")
+            w("      " + " ".join(f"off{k} = 0;" for k in range(len(ops))))
+            w("    } else if (P.n_lead <= 1) {")
             for k in range(len(ops)):
                 w(f"      off{k} = (int64_t)lead_idx[0] * o{k}.lead_stride[0];")
             w("    } else {")
@@ -481,18 +486,20 @@ def write_sources(programs: dict[int, dict]) -> list[Path]:
         src.append(f"extern const rp_spec_entry rp_spec_table_{fi}[] = {{")
         for h, a in chunk:
             rv = resident_variants(a)
-            ks = [f"(const void*)rp_spec_{h:016x}"]
+            flat = not a["has_reduce"]
+            ks = [f"(const void*)rp_spec_{h:016x}" + ("<false>" if flat else "")]
             kf = ["nullptr"]
             kst = ["nullptr"]
             for c in (1, 2, 4, 8):
                 ks.append(f"(const void*)rp_spec_{h:016x}_c{c}<false, false>" if c in rv else "nullptr")
                 kf.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, false>" if c in rv else "nullptr")
                 kst.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, true>" if c in rv else "nullptr")
+            kflat = f"(const void*)rp_spec_{h:016x}<true>" if flat else "nullptr"
             src.append(f"  {{0x{h:016x}ULL, {{{', '.join(ks)}}}, {{{', '.join(kf)}}}, "
-                       f"{{{', '.join(kst)}}}, {1 if a['has_reduce'] else 0}}},")
+                       f"{{{', '.join(kst)}}}, {kflat}, {1 if a['has_reduce'] else 0}}},")
         src.append("  {0ULL, {nullptr, nullptr, nullptr, nullptr, nullptr}, "
                    "{nullptr, nullptr, nullptr, nullptr, nullptr}, "
-                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, 0}};")
+                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, nullptr, 0}};")
         src.append(f"extern const int rp_spec_count_{fi} = {len(chunk)};")
         path = CSRC / f"rowprog_spec_gen{fi}.hip"
         path.write_text("\n".join(src) + "\n")

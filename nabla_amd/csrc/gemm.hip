@@ -66,8 +66,7 @@ __device__ __forceinline__ float gemm_act(float v, int act) {
 }
 
 // Activation and its derivative at the same point (the second result of a launch).  LOWP: the
-// results are stored as 16-bit floats, so hardware exp and a 1.5e-7 erf do (the same forms the
-// row kernels use for such results).
+// results are stored as 16-bit floats, so hardware exp and a 1.5e-7 erf do.
 template <bool LOWP>
 __device__ __forceinline__ void gemm_act_pair(float x, int act, float& y, float& dy) {
   if (act == NBK_ACT_RELU) {

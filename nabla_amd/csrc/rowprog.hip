@@ -461,6 +461,7 @@ struct RpSpec {
   const void* kernel[5];
   const void* kernel_full[5];
   const void* kernel_stream[5];
+  const void* kernel_flat;
   int block_mode;
   bool lds_attr_set;
 };
@@ -484,6 +485,7 @@ static RpSpec* rp_find_spec(uint64_t h) {
           e.kernel_full[k] = tabs[t][i].kernel_full[k];
           e.kernel_stream[k] = tabs[t][i].kernel_stream[k];
         }
+        e.kernel_flat = tabs[t][i].kernel_flat;
         e.block_mode = tabs[t][i].block_mode;
         e.lds_attr_set = false;
         (*g_specs)[tabs[t][i].hash] = e;
@@ -626,7 +628,8 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     uint32_t cpr_arg = (uint32_t)cpr;
     uint64_t total_arg = total;
     void* args[3] = {(void*)p, (void*)&cpr_arg, (void*)&total_arg};
-    NBK_HIP(hipLaunchKernel(spec->kernel[0], dim3((unsigned)blocks), dim3(256), args, 0, st));
+    const void* fn = (rows == 1 && spec->kernel_flat) ? spec->kernel_flat : spec->kernel[0];
+    NBK_HIP(hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(256), args, 0, st));
     return NBK_OK;
   }
   hipLaunchKernelGGL(rp_flat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, *p, (uint32_t)cpr,

@@ -17,6 +17,9 @@ struct rp_spec_entry {
   // [1..4]: kernel_full with non-temporal loads and stores, for launches that move
   // more bytes than the last-level cache holds.
   const void* kernel_stream[5];
+  // programs without reductions: the generic form compiled for launches of a single row (a flat
+  // array: no row arithmetic per chunk); nullptr for reduction programs.
+  const void* kernel_flat;
   int block_mode;
 };
 

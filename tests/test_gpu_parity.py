@@ -631,6 +631,25 @@ def test_small_composite_ops_on_device(hip):
     np.testing.assert_allclose(g.numpy(), np.cos(2 * a.astype(np.float64)), rtol=0, atol=2e-6)
 
 
+def test_gelu_bf16_over_its_whole_range(hip):
+    """GELU of bf16 tensors takes a cheaper form in the kernels (the upper tail of the normal
+    distribution as 2^polynomial instead of erf): every element within one bf16 step of the
+    float64 value, from the far negative tail (where the result is all tail) to large arguments."""
+    from scipy.special import ndtr
+    a = oc.to_bf16_grid(np.concatenate([np.linspace(-12.0, 12.0, 1 << 16), [-30.0, 30.0, 0.0, -0.0, 1e-20, -1e-20]])
+                        .astype(np.float32))
+    got = nb.gelu(T(a, dtype=nb.DType.bfloat16))
+    assert got.dtype == nb.DType.bfloat16
+    got = got.numpy().astype(np.float64)
+    want = a.astype(np.float64) * ndtr(a.astype(np.float64))
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-14)
+    # and its gradient (the erf form, from the kept input) against the closed form
+    g = nb.grad(lambda t: nb.reduce_sum(nb.cast(nb.gelu(t), nb.DType.float32)))(T(a[:4096], dtype=nb.DType.bfloat16))
+    x = a[:4096].astype(np.float64)
+    dwant = ndtr(x) + x * np.exp(-0.5 * x * x) / np.sqrt(2 * np.pi)
+    assert np.all(np.abs(g.numpy().astype(np.float64) - dwant) <= 2.0 ** -7 * np.abs(dwant) + 1e-6)
+
+
 # ---- scatter ----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_scatter_on_device_is_exact_and_deterministic(hip, dtype):
