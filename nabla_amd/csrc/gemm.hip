@@ -57,6 +57,7 @@ struct GemmArgs {
   void* C2;              // second result (derivative of the activation), or null
   const float* b_scales; // NF4-coded B only: one scale per `b_block` consecutive codes
   int32_t b_block;
+  int32_t c_stream;      // C is larger than the last-level cache: store it with the non-temporal hint
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -411,7 +412,12 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
           o.y = (uint32_t)nbk_f32_to_bf16(v[2]) | ((uint32_t)nbk_f32_to_bf16(v[3]) << 16);
           o.z = (uint32_t)nbk_f32_to_bf16(v[4]) | ((uint32_t)nbk_f32_to_bf16(v[5]) << 16);
           o.w = (uint32_t)nbk_f32_to_bf16(v[6]) | ((uint32_t)nbk_f32_to_bf16(v[7]) << 16);
-          *(uint4*)((uint16_t*)g.C + idx) = o;
+          if (g.c_stream) {
+            const u32x4 ov = {o.x, o.y, o.z, o.w};
+            __builtin_nontemporal_store(ov, (u32x4*)((uint16_t*)g.C + idx));
+          } else {
+            *(uint4*)((uint16_t*)g.C + idx) = o;
+          }
         } else if (vec_store && out_f32) {
           float4* dst = (float4*)((float*)g.C + idx);
           dst[0] = make_float4(v[0], v[1], v[2], v[3]);
@@ -1535,6 +1541,11 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   a.b_bs2 = a.batch_inner > 1 ? d->b_bs2 : 0;
   a.c_bs2 = a.batch_inner > 1 ? d->c_bs2 : 0;
   a.dtype_c = d->dtype_c; a.act = d->act; a.alpha = d->alpha;
+  // A result beyond the 256 MiB last-level cache does not survive until its consumer runs: it is
+  // streamed (non-temporal stores), which leaves the cache to the operands.  Smaller results are
+  // stored normally: measured inside the decoder step, streaming them takes as much from the
+  // kernels that read them next as it gives the product.
+  a.c_stream = d->M * d->N * d->batch * (d->dtype_c == NBK_F32 ? 4 : 2) > (256ll << 20) ? 1 : 0;
   NBK_REQUIRE(d->aux_op == NBK_AUX_NONE || d->aux_op == NBK_AUX_ACT_GRAD, "gemm: aux_op %d", d->aux_op);
   NBK_REQUIRE((d->aux_op == NBK_AUX_NONE) == (d->C_aux == nullptr),
               "gemm: C_aux and aux_op go together");
