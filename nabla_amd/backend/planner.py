@@ -785,6 +785,45 @@ class Planner:
                 n.attrs = dict(at, res_in=len(mm.inputs), alpha=alpha * at.get("alpha", 1.0))
                 break
 
+    def _fold_scale_into_matmul(self) -> None:
+        """``(x @ W) * c`` with ``c`` a number: the multiply node turns into the product with
+        ``alpha = c`` (applied to the fp32 accumulator, also of K-split partial products, before
+        the one rounding of the result).  The low-rank adapters put their ``alpha / rank`` on a
+        [tokens, rank] product this way, and their backward pass on two more."""
+        nodes = self._live_nodes()
+        n_users: dict[int, int] = {}
+        for n in nodes:
+            for i in n.inputs:
+                n_users[i.id] = n_users.get(i.id, 0) + 1
+        out_ids = {v.id for v in self.outputs}
+
+        def constant_of(x):
+            if not isinstance(x, ir.Value):
+                return float(x)
+            while x.node.kind in ("broadcast", "reshape"):
+                x = x.node.inputs[0]
+            return float(x.node.attrs["value"]) if x.node.kind == "fill" else None
+
+        for n in nodes:
+            if not (n.kind == "ew" and n.fn == "mul" and len(n.attrs["operands"]) == 2):
+                continue
+            out = n.outputs[0]
+            xs = n.attrs["operands"]
+            for x, other in ((xs[0], xs[1]), (xs[1], xs[0])):
+                if not (isinstance(x, ir.Value) and x.node.kind == "matmul"):
+                    continue
+                c = constant_of(other)
+                mm, at = x.node, x.node.attrs or {}
+                if (c is None or len(mm.outputs) != 1 or n_users.get(x.id) != 1 or x.id in out_ids or
+                        x.dtype is not out.dtype or x.shape != out.shape or
+                        out.dtype not in (DType.float32, DType.bfloat16) or
+                        "bias_in" in at or "res_in" in at or at.get("act")):
+                    continue
+                n.kind, n.fn = "matmul", None
+                n.inputs = list(mm.inputs)
+                n.attrs = dict(at, alpha=c * at.get("alpha", 1.0))
+                break
+
     def _fold_activation_into_matmul(self) -> None:
         """``gelu(x @ W + b)`` whose pre-activation has no reader but the activation and, in a
         training step, its derivative (``GeluOp``'s VJP multiplies the cotangent with
@@ -1388,7 +1427,7 @@ class Planner:
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
         epi = dict(epi or {})
         common["alpha"] = epi.get("alpha", 1.0)
-        if ks == 1 or epi:  # (a product with a folded epilogue is never split)
+        if ks == 1 or set(epi) - {"alpha"}:  # (only a scale survives the split: it goes on the partial products)
             writes = [dst.buf]
             if "aux_value" in epi:
                 epi["aux_dst"] = self._alloc_value(epi.pop("aux_value"))
@@ -2146,8 +2185,10 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     _fold_empty(builder)
     pre = Planner(builder, outputs)
     pre._rematerialize_masks()
-    pre._fold_bias_into_matmul()
     from .. import config
+    if config.FOLD_SCALE:
+        pre._fold_scale_into_matmul()
+    pre._fold_bias_into_matmul()
     if config.FOLD_RESIDUAL:
         pre._fold_sum_into_matmul()
         pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)

@@ -39,6 +39,10 @@ _LORA_LOW_RANK_ORDER: ContextVar[bool] = ContextVar("LORA_LOW_RANK_ORDER",
 _FOLD_ACTIVATION: ContextVar[bool] = ContextVar("FOLD_ACTIVATION",
                                                 default=_env_flag("NBK_FOLD_ACTIVATION", False))
 
+# (x @ W) * c with c a constant of the graph as one product with alpha = c (how the low-rank
+# adapters carry alpha / rank: no multiply kernel of its own in either direction)
+_FOLD_SCALE: ContextVar[bool] = ContextVar("FOLD_SCALE", default=_env_flag("NBK_FOLD_SCALE", True))
+
 # r + (x @ W) * alpha as one product whose epilogue reads r.  Off: measured on the LoRA decoder
 # step, the epilogue's read of a full-size r (it starts when a tile's matrix work is over and
 # nothing overlaps it) costs 33-41 us per 8192 x 2048 result where the separate sum kernel
@@ -70,6 +74,7 @@ _FLAGS = {
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
+    "FOLD_SCALE": _FOLD_SCALE,
     "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
     "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,

@@ -16,7 +16,7 @@ from ... import config
 from ...core.dtype import DType
 from ...core.pytree import tree_map
 from ...core.tensor import Tensor
-from ...ops.creation import zeros
+from ...ops.creation import full, zeros
 from ..functional.init import normal
 
 
@@ -39,6 +39,12 @@ def init_lora_adapter(weight: Tensor, rank: int, init_std: float = 0.01,
             "B": zeros((rank, fan_out), dtype=kind, device=weight.device)}
 
 
+def _scale_constant(value: float, like: Tensor) -> Tensor:
+    """The scale as a constant of the graph (a lazy ``full``), not as a realized scalar: the
+    planner can then read its value and fold it into the neighbouring product."""
+    return full((), float(value), dtype=like.dtype, device=like.device)
+
+
 def lora_delta(adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:
     """The full-size update ``(alpha / rank) * A @ B``."""
     down, up, inv_rank = _factors(adapter)
@@ -52,9 +58,10 @@ def lora_linear(x: Tensor, frozen_weight: Tensor, adapter: dict[str, Tensor],
     if not config.LORA_LOW_RANK_ORDER:
         return base + x @ lora_delta(adapter, alpha=alpha)
     down, up, inv_rank = _factors(adapter)
-    # (the scale goes on the small factor, as the reference puts it on the update: the product
-    # with the activations then needs no pass of its own for it)
-    return base + (x @ down) @ (up * (alpha * inv_rank))
+    # (the scale goes on the [tokens, rank] product, where the planner folds it into that
+    # product's alpha, and the same happens to its two mirror images in the backward pass: no
+    # kernel of its own anywhere)
+    return base + ((x @ down) * _scale_constant(alpha * inv_rank, x)) @ up
 
 
 def merge_lora_weight(frozen_weight: Tensor, adapter: dict[str, Tensor], alpha: float = 1.0) -> Tensor:

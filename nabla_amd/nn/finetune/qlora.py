@@ -23,6 +23,7 @@ from ... import config
 from ...core.dtype import DType
 from ...core.tensor import Tensor
 from ...ops.unary import cast
+from .lora import _scale_constant
 from ...ops.view import gather, reshape, unsqueeze
 
 #: the sixteen NF4 levels as the reference tabulates them (four decimals)
@@ -96,6 +97,6 @@ def qlora_linear(x: Tensor, qweight: dict[str, Any], adapter: dict[str, Tensor],
         down, up = cast_adapter["A"], cast_adapter["B"]
         scale = alpha / float(int(down.shape[1]))
         if config.LORA_LOW_RANK_ORDER:
-            return base + (xc @ down) @ (up * scale)
+            return base + ((xc @ down) * _scale_constant(scale, xc)) @ up
         return base + xc @ ((down @ up) * scale)
     return lora_linear(xc, dequantize_nf4(qweight, dtype=compute_dtype), cast_adapter, alpha=alpha)

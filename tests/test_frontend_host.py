@@ -658,6 +658,45 @@ def test_sum_with_a_product_folds_into_its_epilogue_when_asked(emulator):
     np.testing.assert_allclose(folded, want, rtol=1e-5, atol=1e-5)
 
 
+def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
+    """``(x @ W) * c`` with ``c`` a constant of the graph is one product with ``alpha = c`` (the
+    way the low-rank adapters carry ``alpha / rank``, forward and backward); a realized scalar
+    tensor is a run-time value and keeps its own multiply."""
+    from nabla_amd.core import engine
+    from nabla_amd.nn.finetune import lora_linear
+    rng = np.random.default_rng(21)
+    x, w = rng.standard_normal((5, 24, 32)).astype(np.float32), rng.standard_normal((32, 16)).astype(np.float32)
+    engine.clear_plan_cache()
+    got = (T(x) @ T(w)) * nb.full((), 2.5)
+    got.realize()
+    steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+    assert [s.kind for s in steps] == ["gemm"] and steps[0].attrs["alpha"] == 2.5
+    np.testing.assert_allclose(got.numpy(), (x @ w) * 2.5, rtol=1e-5, atol=1e-5)
+    engine.clear_plan_cache()
+    kept = (T(x) @ T(w)) * 2.5
+    kept.realize()
+    assert sorted(s.kind for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps) == ["gemm", "rowprog"]
+    np.testing.assert_allclose(kept.numpy(), (x @ w) * 2.5, rtol=1e-5, atol=1e-5)
+    # an adapter with alpha / rank = 3: value and gradients against numpy, no multiply of its own
+    a, b = rng.standard_normal((32, 4)).astype(np.float32) * 0.1, rng.standard_normal((4, 16)).astype(np.float32) * 0.1
+
+    def loss(ad):
+        return nb.reduce_sum(lora_linear(T(x), T(w), ad, alpha=12.0) * T(np.ones((5, 24, 16), np.float32)))
+
+    engine.clear_plan_cache()
+    val, grads = nb.value_and_grad(loss)({"A": T(a), "B": T(b)})
+    nb.realize_all(val, grads["A"], grads["B"])
+    kinds = [s.kind for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+    alphas = sorted(s.attrs.get("alpha", 1.0) for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps
+                    if s.kind == "gemm")
+    engine.clear_plan_cache()
+    assert alphas.count(3.0) >= 2, (kinds, alphas)
+    x2 = x.reshape(-1, 32)
+    np.testing.assert_allclose(val.numpy(), (x2 @ w + 3.0 * (x2 @ a) @ b).sum(), rtol=1e-4)
+    np.testing.assert_allclose(grads["B"].numpy(), 3.0 * (x2 @ a).T @ np.ones((120, 16), np.float32), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(grads["A"].numpy(), 3.0 * x2.T @ (np.ones((120, 16), np.float32) @ b.T), rtol=1e-4, atol=1e-4)
+
+
 def test_gelu_backward_recomputes_the_derivative_where_the_cotangent_is(emulator):
     """Two ways to get gelu's derivative to the backward pass -- recomputed from the pre-activation
     where the cotangent is (the default), or stored by the forward kernel -- agree with the
