@@ -726,13 +726,19 @@ class Planner:
                 n.attrs = dict(at, bias_in=len(mm.inputs))
                 break
 
-    def _fold_sum_into_matmul(self) -> None:
+    def _fold_sum_into_matmul(self, thin_only: bool = False) -> None:
         """``r + (x @ W) * alpha`` with ``r`` of the product's shape (a skip connection, the base
         product under a low-rank update, a gradient that two branches contribute to): the add
         node turns into the product, which reads ``r`` in its epilogue and adds it to the fp32
         accumulator before the one rounding of the result.  The scaled product and the sum
         never make their own trips through memory.  A chain of such sums folds link by link:
-        the second product takes the first sum as its ``r``."""
+        the second product takes the first sum as its ``r``.
+
+        ``thin_only``: only products with a contraction of at most 16 (the update of a low-rank
+        adapter on top of its base product).  Their kernel is all memory traffic, many
+        workgroups to a CU, and reads ``r`` for less than the separate sum kernel costs; the
+        large products pay more for it than that kernel (one workgroup per CU, nothing runs
+        beside its epilogue), so for them the fold stays behind ``config.FOLD_RESIDUAL``."""
         nodes = self._live_nodes()
         n_users: dict[int, int] = {}
         for n in nodes:
@@ -775,6 +781,12 @@ class Planner:
                 at = mm.attrs or {}
                 if alpha != 1.0 and "bias_in" in at:
                     continue  # (the kernel scales the product only, not a bias folded earlier)
+                # (and only on top of another product, the adapter's base: a sum with anything
+                # else usually sits inside a fused row kernel already and would be cut out of it)
+                if thin_only and not (mm.kind == "matmul" and mm.inputs[0].shape[-1] <= 16 and
+                                      m.dtype is DType.bfloat16 and m.shape[-1] % 8 == 0 and
+                                      r.node.kind == "matmul"):
+                    continue
                 if not (mm.kind == "matmul" and len(mm.outputs) == 1 and single_use(m) and
                         "res_in" not in at and not at.get("act") and
                         r.shape == out.shape and r.dtype is out.dtype and r.node.kind != "fill" and
@@ -2189,8 +2201,8 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     if config.FOLD_SCALE:
         pre._fold_scale_into_matmul()
     pre._fold_bias_into_matmul()
-    if config.FOLD_RESIDUAL:
-        pre._fold_sum_into_matmul()
+    if config.FOLD_RESIDUAL or config.FOLD_THIN_RESIDUAL:
+        pre._fold_sum_into_matmul(thin_only=not config.FOLD_RESIDUAL)
         pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)
     if config.FOLD_ACTIVATION:
         pre._fold_activation_into_matmul()

@@ -50,6 +50,11 @@ _FOLD_SCALE: ContextVar[bool] = ContextVar("FOLD_SCALE", default=_env_flag("NBK_
 _FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
                                               default=_env_flag("NBK_FOLD_RESIDUAL", False))
 
+# the same fold for products with a contraction of at most 16 only (a low-rank adapter's update
+# on top of its base product): on: their kernel reads r for less than the sum kernel costs
+_FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
+    "FOLD_THIN_RESIDUAL", default=_env_flag("NBK_FOLD_THIN_RESIDUAL", True))
+
 # the backward pass of the exact GELU computes GELU'(x) from the kept pre-activation, in the
 # kernel that multiplies it with the cotangent; off: the forward kernel stores GELU'(x) as a
 # second full-size result and the backward kernel reads it
@@ -74,6 +79,7 @@ _FLAGS = {
     "LORA_LOW_RANK_ORDER": _LORA_LOW_RANK_ORDER,
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
+    "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
     "FOLD_SCALE": _FOLD_SCALE,
     "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,

@@ -294,7 +294,9 @@ extern __shared__ __align__(16) u32x4 gemm_lds[];
 
 // Epilogue shared by the bf16 kernels (the caller has passed a workgroup barrier: the tile
 // buffers are free).
-// EPI: 0 plain, 1 bias only (as lean as the plain form), 2 bias / activation / residual.
+// EPI: 0 plain, 1 bias only (as lean as the plain form), 2 bias / activation / residual (the
+// residual requested for the whole wave tile up front), 3 bias and an added residual read pass by
+// pass (for kernels whose occupancy hides that latency and must not lose it to registers).
 // Each wave passes its accumulators through a private LDS slab, a band of 32 rows of its tile
 // at a time (`scatter(band, slab)` writes the band's accumulators there, row-major with a
 // pitch of WN + 4 floats), so that C is written as whole 16-byte (bf16) / 32-byte (fp32)
@@ -318,9 +320,17 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
 #pragma unroll
   for (int e = 0; e < 8; ++e) bias_v[e] = 0.f;
   if (EPI != 0 && g.bias) {
+    if (!out_f32 && col + 8 <= g.N && (((uintptr_t)g.bias + 2 * (uintptr_t)col) & 15) == 0) {
+      const uint4 bu = *(const uint4*)((const uint16_t*)g.bias + col);  // eight 16-bit values at once
+      bias_v[0] = __uint_as_float(bu.x << 16); bias_v[1] = __uint_as_float(bu.x & 0xffff0000u);
+      bias_v[2] = __uint_as_float(bu.y << 16); bias_v[3] = __uint_as_float(bu.y & 0xffff0000u);
+      bias_v[4] = __uint_as_float(bu.z << 16); bias_v[5] = __uint_as_float(bu.z & 0xffff0000u);
+      bias_v[6] = __uint_as_float(bu.w << 16); bias_v[7] = __uint_as_float(bu.w & 0xffff0000u);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      if (col + e < g.N) bias_v[e] = nbk_load_as_f32(g.bias, col + e, g.dtype_c);
+      for (int e = 0; e < 8; ++e)
+        if (col + e < g.N) bias_v[e] = nbk_load_as_f32(g.bias, col + e, g.dtype_c);
+    }
   }
   constexpr int NP = 32 / ROWS_PER_PASS;
   const bool res_vec = EPI == 2 && g.residual && vec_store && !out_f32;
@@ -355,9 +365,22 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
         const int64_t idx = c_off + row * g.ldc + col;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
-        if (EPI == 1) {
+        if (EPI == 1 || EPI == 3) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
+        }
+        if (EPI == 3 && g.residual) {
+          if (vec_store && !out_f32) {
+            const uint4 ru = *(const uint4*)((const uint16_t*)g.residual + idx);
+            v[0] += __uint_as_float(ru.x << 16); v[1] += __uint_as_float(ru.x & 0xffff0000u);
+            v[2] += __uint_as_float(ru.y << 16); v[3] += __uint_as_float(ru.y & 0xffff0000u);
+            v[4] += __uint_as_float(ru.z << 16); v[5] += __uint_as_float(ru.z & 0xffff0000u);
+            v[6] += __uint_as_float(ru.w << 16); v[7] += __uint_as_float(ru.w & 0xffff0000u);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < g.N) v[e] += nbk_load_as_f32(g.residual, idx + e, g.dtype_c);
+          }
         }
         if (EPI == 2) {
           float res[8];
@@ -1033,7 +1056,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
 // low-rank adapter): one MFMA deep, all memory traffic.  No K loop and no operand tiles in
 // LDS: every lane reads its 8 k-values of an A row / a B column straight from global memory
 // into the MFMA fragment, and the tile leaves through the shared epilogue.
-template <bool B_KC, bool EPI>
+template <bool B_KC, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
   constexpr int TM = 2, TN = 2, WN = 64;
   int tm_i, tn_i;
@@ -1079,7 +1102,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], (f32x16)(0.f), 0, 0, 0);
-  gemm_epilogue<TM, TN, WN, true, EPI ? 2 : 0>(acc, g, m0, n0, wm, wn, 0, wave, lane);
+  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane);
 }
 
 // ------------------------------------------------------------------- bf16, N <= 32
@@ -1600,11 +1623,19 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     a.tiles_n = (int)((d->N + 127) / 128);
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
     const size_t lds = 4 * 32 * (size_t)(64 + 4) * sizeof(float);
-    const bool epi = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
-    if (bkc && epi) hipLaunchKernelGGL((gemm_skinny_k_kernel<true, true>), grid, dim3(256), lds, st, a);
-    else if (bkc) hipLaunchKernelGGL((gemm_skinny_k_kernel<true, false>), grid, dim3(256), lds, st, a);
-    else if (epi) hipLaunchKernelGGL((gemm_skinny_k_kernel<false, true>), grid, dim3(256), lds, st, a);
-    else hipLaunchKernelGGL((gemm_skinny_k_kernel<false, false>), grid, dim3(256), lds, st, a);
+    // 0 plain; 3 a bias and / or an added residual (the adapter's update on top of the base
+    // product: all memory traffic, so the lean epilogue that keeps four waves per SIMD); 2 the rest
+    const bool any = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
+    const int epi = !any ? 0 : ((a.act == NBK_ACT_NONE && a.C2 == nullptr && !a.res_mul) ? 3 : 2);
+#define NBK_LAUNCH_SKK(BK_)                                                                        \
+  do {                                                                                             \
+    if (epi == 0) hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 0>), grid, dim3(256), lds, st, a); \
+    else if (epi == 3) hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 3>), grid, dim3(256), lds, st, a); \
+    else hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 2>), grid, dim3(256), lds, st, a);         \
+  } while (0)
+    if (bkc) NBK_LAUNCH_SKK(true);
+    else NBK_LAUNCH_SKK(false);
+#undef NBK_LAUNCH_SKK
     return nbk_check_launch("gemm_skinny_k_kernel");
   }
   if (d->dtype_ab == NBK_BF16) {

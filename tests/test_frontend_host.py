@@ -658,6 +658,41 @@ def test_sum_with_a_product_folds_into_its_epilogue_when_asked(emulator):
     np.testing.assert_allclose(folded, want, rtol=1e-5, atol=1e-5)
 
 
+def test_an_adapter_update_folds_into_the_sum_with_its_base_product(emulator):
+    """``x @ W + h @ B`` with a contraction of at most 16 in the second product (a low-rank
+    adapter's update) is two products and no sum kernel: the thin product's epilogue reads the
+    base product.  A sum with anything that is not a product keeps its row kernel."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(31)
+    x, w = rng.standard_normal((4, 16, 32)).astype(np.float32), rng.standard_normal((32, 24)).astype(np.float32)
+    h, b = rng.standard_normal((4, 16, 8)).astype(np.float32), rng.standard_normal((8, 24)).astype(np.float32)
+    r = rng.standard_normal((4, 16, 24)).astype(np.float32)
+    bf = nb.DType.bfloat16
+
+    def steps_of(f):
+        engine.clear_plan_cache()
+        out = f().numpy()
+        steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+        engine.clear_plan_cache()
+        return out, steps
+
+    got, steps = steps_of(lambda: nb.cast(T(x, dtype=bf) @ T(w, dtype=bf) + T(h, dtype=bf) @ T(b, dtype=bf),
+                                          nb.DType.float32))
+    assert sorted(s.kind for s in steps).count("gemm") == 2
+    assert sum("residual" in s.attrs for s in steps if s.kind == "gemm") == 1, \
+        [s.attrs for s in steps]
+    want = _bf16_round(x) @ _bf16_round(w) + _bf16_round(h) @ _bf16_round(b)
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2)
+    with config.flag("FOLD_THIN_RESIDUAL", False):
+        off, steps_off = steps_of(lambda: nb.cast(
+            T(x, dtype=bf) @ T(w, dtype=bf) + T(h, dtype=bf) @ T(b, dtype=bf), nb.DType.float32))
+    assert not any("residual" in s.attrs for s in steps_off if s.kind == "gemm")
+    np.testing.assert_allclose(off, want, rtol=2e-2, atol=2e-2)
+    _, steps_r = steps_of(lambda: nb.cast(T(r, dtype=bf) + T(h, dtype=bf) @ T(b, dtype=bf), nb.DType.float32))
+    assert not any("residual" in s.attrs for s in steps_r if s.kind == "gemm")
+
+
 def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
     """``(x @ W) * c`` with ``c`` a constant of the graph is one product with ``alpha = c`` (the
     way the low-rank adapters carry ``alpha / rank``, forward and backward); a realized scalar
