@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 18
+#define NBK_ABI_VERSION 19
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -267,6 +267,14 @@ typedef struct nbk_gemm_desc {
   void* C_aux;           /* NULL or a second result in C's layout and dtype (see nbk_gemm_aux_op) */
   int32_t aux_op;        /* enum nbk_gemm_aux_op; needs act != NBK_ACT_NONE and no residual */
   int32_t reserved;
+  /* NULL, or [batch][N] in dtype_c: sum over k of B[b][k][n], a third result of the same launch.
+   * With A = x^T and B = dy the product is the weight gradient of a linear layer and this is its
+   * bias gradient (the reduction of the cotangent to the bias' shape,
+   * nabla/core/autograd/backward.py:31-54), taken from the B fragments the product has in
+   * registers, so dy is read once.  bf16 operands, both row-contiguous (a_rs == b_cs == 1) and
+   * 16-byte aligned, K % 64 == 0, M % 8 == 0, N % 8 == 0, alpha 1, no bias / residual / activation,
+   * one batch level; anything else is an error. */
+  void* colsum;
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
 

@@ -178,6 +178,12 @@ class BoundPlan:
                     d.aux_op = 1
                 d.batch_reduce = 0
                 d.alpha = a.get("alpha", 1.0)
+                d.colsum = None
+                if a.get("colsum") is not None:
+                    rcs = a["colsum"]
+                    if rcs.dtype is not rc.dtype:
+                        raise TypeError(f"matmul column sums are {rcs.dtype}, the product {rc.dtype}")
+                    ptr_field(d, "colsum", rcs.buf, rcs.offset * rcs.dtype.size_in_bytes)
                 self.calls.append((L.nbk_gemm, [C.byref(d)], patches, d))
             elif k == "gemm_nf4":
                 d = lib.GemmNf4Desc()

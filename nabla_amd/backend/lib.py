@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 MAX_RANK = 8
 
@@ -68,6 +68,7 @@ class GemmDesc(C.Structure):
         ("act", C.c_int32), ("batch_reduce", C.c_int32),
         ("alpha", C.c_float), ("residual_op", C.c_int32),
         ("C_aux", C.c_void_p), ("aux_op", C.c_int32), ("reserved", C.c_int32),
+        ("colsum", C.c_void_p),
     ]
 
 

@@ -259,6 +259,8 @@ class Planner:
         self.loc: dict[int, Any] = {}  # value id -> ViewRef | Const
         self.unit_of: dict[int, Unit] = {}  # node pos -> unit
         self.alias_nodes: set[int] = set()  # broadcast nodes fused as row->full aliases
+        from .. import config
+        self.fold_column_sums = bool(config.FOLD_COLUMN_SUMS)
 
     # ................................................................ liveness
     def _live_nodes(self) -> list[ir.Node]:
@@ -1163,7 +1165,46 @@ class Planner:
         else:
             self._emit(step)
 
+    def _fold_column_sums(self) -> None:
+        """Deferred column sums whose matrix is the right operand of a product that was emitted
+        with room for them (``colsum_key`` on both) become a result of that product's launch:
+        the matrix is read once.  A product split along K leaves one row of partial sums per
+        slice, which the second stage adds up as it would have the first stage's."""
+        hosts = {}
+        for idx, st in enumerate(self.steps):
+            key = st.attrs.get("colsum_key") if st.kind == "gemm" else None
+            if key is not None and key not in hosts:
+                hosts[key] = idx
+        first, second = self._deferred_reduces
+        for task in list(first):
+            key = task.attrs.get("colsum_key")
+            idx = hosts.pop(key, None) if key is not None else None
+            if idx is None:
+                continue
+            host = self.steps[idx]
+            ks, n = host.attrs["batch"], host.attrs["N"]
+            stage2 = task.attrs.get("second")
+            final = (stage2 or task).attrs["dst"]
+            first.remove(task)
+            if ks == 1:
+                if stage2 is not None:
+                    second.remove(stage2)
+                target = ViewRef(final.buf, final.offset, (1, n), (n, 1), final.dtype)
+            else:
+                tmp = self._new_buf((ks, n), DType.float32)
+                target = ViewRef(tmp.id, 0, (ks, n), (n, 1), DType.float32)
+                if stage2 is not None:
+                    second.remove(stage2)
+                second.append(Step("reduce_mid", [tmp.id], [final.buf], dict(
+                    src=target, dst=final, outer=1, red=ks, inner=n, fn="sum")))
+            host.attrs["colsum"] = target
+            host.writes.append(target.buf)
+            b = self.bufs[target.buf]
+            b.first, b.last = min(b.first, idx), max(b.last, idx)
+
     def _flush_reduces(self) -> None:
+        if self.fold_column_sums:
+            self._fold_column_sums()
         for tasks in self._deferred_reduces:
             if len(tasks) == 1:
                 self._emit(tasks[0])
@@ -1239,19 +1280,29 @@ class Planner:
                     split = s
                     break
         terminal = self._terminal(out)
+        # the column sums of a matrix that a product also reads as its row-contiguous right
+        # operand (a bias gradient beside the weight gradient) can ride on that product
+        fold = {}
+        if (terminal and self.fold_column_sums and kind == "sum" and outer == 1 and
+                x.dtype is DType.bfloat16 and out.dtype is DType.bfloat16):
+            fold = dict(colsum_key=(src.buf, src.offset, red, inner))
         if split > 1:
             tmp = self._new_buf((outer, split, inner), DType.float32)
             tref = ViewRef(tmp.id, 0, (outer, split, inner),
                            contiguous_strides((outer, split, inner)), DType.float32)
-            self._emit_reduce(Step("reduce_mid", [src.buf], [tmp.id], dict(
-                src=src, dst=tref, outer=outer * split, red=red // split, inner=inner, fn=kind)), 0, terminal)
             dst = self._alloc_value(out)
-            self._emit_reduce(Step("reduce_mid", [tmp.id], [dst.buf], dict(
-                src=tref, dst=dst, outer=outer, red=split, inner=inner, fn=kind)), 1, terminal)
+            second = Step("reduce_mid", [tmp.id], [dst.buf], dict(
+                src=tref, dst=dst, outer=outer, red=split, inner=inner, fn=kind))
+            if fold:
+                fold["second"] = second
+            self._emit_reduce(Step("reduce_mid", [src.buf], [tmp.id], dict(
+                fold, src=src, dst=tref, outer=outer * split, red=red // split, inner=inner, fn=kind)),
+                0, terminal)
+            self._emit_reduce(second, 1, terminal)
             return
         dst = self._alloc_value(out)
         self._emit_reduce(Step("reduce_mid", [src.buf], [dst.buf], dict(
-            src=src, dst=dst, outer=outer, red=red, inner=inner, fn=kind)), 0, terminal)
+            fold, src=src, dst=dst, outer=outer, red=red, inner=inner, fn=kind)), 0, terminal)
 
     # ................................................................ matmul
     @staticmethod
@@ -1428,6 +1479,26 @@ class Planner:
             ks *= 2
         return ks
 
+    @staticmethod
+    def _colsum_key(ra: ViewRef, rb: ViewRef, pa, pb, M: int, N: int, K: int, ks: int, epi: dict):
+        """What a deferred column sum must name to ride on this product (one launch, or ``ks``
+        slices of K): the right operand is a whole row-major [K, N] bf16 matrix, the left one is
+        row-contiguous too, and the launch is one that takes the 128 x 128 tile anyway (the
+        kernel that carries the sums), with the alignment its direct loads ask for."""
+        if epi or ra.dtype is not DType.bfloat16 or rb.dtype is not DType.bfloat16:
+            return None
+        if not (pa[1] == 1 and pa[2] != 1 and pb[2] == 1 and pb[1] == N):
+            return None
+        if M % 8 or N % 8 or M < 8 or N < 8 or K % (64 * ks) or K // ks <= 16:
+            return None
+        if pa[2] % 8 or pa[2] >= 1 << 22 or N >= 1 << 22 or ra.offset % 8 or rb.offset % 8:
+            return None
+        big = -(-M // 256) * -(-N // 256) * ks
+        rounds = -(-big // 256)
+        if big * 10 >= rounds * 256 * 6 and M >= 256 and N >= 256 and K // ks > 128:
+            return None  # the 256 x 256 tile is the faster launch here
+        return (rb.buf, rb.offset, K, N)
+
     def _emit_plain_gemm(self, ra: ViewRef, rb: ViewRef, pa, pb, M: int, N: int, K: int,
                          out: ir.Value, epi: dict | None = None) -> None:
         """One unbatched product into contiguous storage for ``out``; split along K into fp32
@@ -1439,7 +1510,12 @@ class Planner:
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
         epi = dict(epi or {})
         common["alpha"] = epi.get("alpha", 1.0)
-        if ks == 1 or set(epi) - {"alpha"}:  # (only a scale survives the split: it goes on the partial products)
+        if ks > 1 and set(epi) - {"alpha"}:
+            ks = 1  # (only a scale survives the split: it goes on the partial products)
+        key = self._colsum_key(ra, rb, pa, pb, M, N, K, ks, epi) if self.fold_column_sums else None
+        if key is not None:
+            common["colsum_key"] = key
+        if ks == 1:
             writes = [dst.buf]
             if "aux_value" in epi:
                 epi["aux_dst"] = self._alloc_value(epi.pop("aux_value"))

@@ -55,6 +55,11 @@ _FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
 _FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
     "FOLD_THIN_RESIDUAL", default=_env_flag("NBK_FOLD_THIN_RESIDUAL", True))
 
+# the column sums of dy (a bias gradient) as one more result of the weight-gradient product
+# x^T dy that reads dy anyway; off: the reduction kernels read dy a second time
+_FOLD_COLUMN_SUMS: ContextVar[bool] = ContextVar(
+    "FOLD_COLUMN_SUMS", default=_env_flag("NBK_FOLD_COLUMN_SUMS", True))
+
 # the backward pass of the exact GELU computes GELU'(x) from the kept pre-activation, in the
 # kernel that multiplies it with the cotangent; off: the forward kernel stores GELU'(x) as a
 # second full-size result and the backward kernel reads it
@@ -81,6 +86,7 @@ _FLAGS = {
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
     "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
     "FOLD_SCALE": _FOLD_SCALE,
+    "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
     "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
     "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,

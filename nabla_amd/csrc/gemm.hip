@@ -58,6 +58,7 @@ struct GemmArgs {
   const float* b_scales; // NF4-coded B only: one scale per `b_block` consecutive codes
   int32_t b_block;
   int32_t c_stream;      // C is larger than the last-level cache: store it with the non-temporal hint
+  void* colsum;          // null, or [batch][N] in C's dtype: the column sums of B over K
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -827,7 +828,11 @@ struct DirectLoader {
 // KSS: k-steps (one MFMA deep) per fragment set.  A step of KSS k-steps is multiplied out of one
 // set while the other is filled for the next step; small wave tiles take 2, so that a read has
 // more than a handful of MFMAs to land.
-template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS, bool MI16>
+// COLSUM: the launch also leaves sum_k B[k][n] (the bias gradient beside a weight gradient
+// x^T dy, which reads dy anyway): the waves that hold the first block row of the first tile row
+// multiply a fragment of ones into one more accumulator per block column, from the B fragments
+// that are in registers for the product -- no byte is read twice.
+template <int BM, int BN, bool A_KC, bool B_KC, int EPI, int NW, int KSS, bool MI16, bool COLSUM = false>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g) {
   constexpr int WGN = NW / 2;
   constexpr int WM = BM / 2, WN = BN / WGN;  // wave tile
@@ -853,6 +858,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (Acc)(0.f);
+
+  static_assert(!COLSUM || MI16, "column sums ride on the 16 x 16 x 32 instruction");
+  f32x4 cs[COLSUM ? TN : 1];
+  bool do_cs = false;
+  if constexpr (COLSUM) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) cs[j] = (f32x4)(0.f);
+    do_cs = tm_i == 0 && wm == 0;  // (uniform over the wave)
+  }
 
   using LA = DirectLoader<BM, A_KC, NW, MI16>;
   using LB = DirectLoader<BN, B_KC, NW, MI16>;
@@ -958,6 +972,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kl * TM + i], fb[SET][kl * TN + j],
                                                           acc[i][j], 0, 0, 0);
   };
+  // column sums of the step whose B fragments are in set SET (still whole: reads fill the other)
+  auto colsum_step = [&](auto set) {
+    if constexpr (COLSUM) {
+      constexpr int SET = decltype(set)::value;
+      if (do_cs) {
+        const uint32_t one2 = 0x3f803f80u;  // two bf16 ones
+        const u32x4 ones4 = {one2, one2, one2, one2};
+        const bf16x8 ones = __builtin_bit_cast(bf16x8, ones4);
+#pragma unroll
+        for (int kl = 0; kl < KSS; ++kl)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            cs[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, fb[SET][kl * TN + j], cs[j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   // step on fragment set SET while set 1 - SET is filled for step `step_next` of `tile`
   auto stage = [&](auto set, const u32x4* tile, int step_next) {
     constexpr int SET = decltype(set)::value;
@@ -975,6 +1006,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
       if constexpr (Q < SPREAD) __builtin_amdgcn_sched_barrier(0);
     });
     __builtin_amdgcn_sched_barrier(0);
+    colsum_step(set);
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
@@ -1036,6 +1068,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
       });
     }
     __builtin_amdgcn_sched_barrier(0);
+    colsum_step(S1{});
   }
   {
     const u32x4* cur = gemm_lds + ((nk - 1) & 1) * TILE_CHUNKS;
@@ -1045,6 +1078,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
     });
     frags_ready(S1{});
     static_for<NMFMA>([&](auto q) { mfma(S1{}, q); });
+    colsum_step(S1{});
+  }
+  if constexpr (COLSUM) {
+    // every row of a block holds the same sums: lanes 0..15 have row 0 of their column
+    if (do_cs && lane < 16) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t col = n0 + wn + j * 16 + lane;
+        if (col < g.N) {
+          const int64_t at = (int64_t)blockIdx.y * g.N + col;
+          if (g.dtype_c == NBK_F32) ((float*)g.colsum)[at] = cs[j][0];
+          else ((uint16_t*)g.colsum)[at] = nbk_f32_to_bf16(cs[j][0]);
+        }
+      }
+    }
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no copy may land in a slab
   __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
@@ -1532,6 +1580,27 @@ static int launch_bf16_dl(const GemmArgs& a, bool akc, bool bkc, int64_t batch, 
   return nbk_check_launch("gemm_bf16_dl_kernel");
 }
 
+// The same launch with the column sums of B as a second result (both operands row-contiguous,
+// no epilogue: the weight gradient x^T dy beside the bias gradient).
+template <int BM, int BN, int NW>
+static int launch_bf16_dl_colsum(const GemmArgs& a, int64_t batch, hipStream_t st) {
+  GemmArgs g = a;
+  g.tiles_m = (int)((a.M + BM - 1) / BM);
+  g.tiles_n = (int)((a.N + BN - 1) / BN);
+  dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
+  const size_t pipe = 2 * (size_t)(BM + BN) * 8 * 16;
+  const size_t slabs = NW * 32 * (size_t)(BN / (NW / 2) + 4) * sizeof(float);
+  const size_t lds = pipe > slabs ? pipe : slabs;
+  auto kern = gemm_bf16_dl_kernel<BM, BN, false, false, 0, NW, 1, true, true>;
+  static bool attr_set = false; /* idempotent, so a race only repeats the call */
+  if (!attr_set) {
+    NBK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, st, g);
+  return nbk_check_launch("gemm_bf16_dl_kernel (column sums)");
+}
+
 extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   NBK_REQUIRE(d != nullptr, "gemm: null descriptor");
   NBK_REQUIRE(d->A && d->B && d->C, "gemm: null operand pointer");
@@ -1578,6 +1647,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   NBK_REQUIRE(d->residual_op == NBK_RES_ADD || d->residual_op == NBK_RES_MUL,
               "gemm: residual_op %d", d->residual_op);
   a.res_mul = d->residual_op == NBK_RES_MUL;
+  a.colsum = d->colsum;
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;
@@ -1588,6 +1658,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   };
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs, a.a_bs2);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs, a.b_bs2);
+  NBK_REQUIRE(d->colsum == nullptr || d->dtype_ab == NBK_BF16, "gemm: column sums need bf16 operands");
   if (d->dtype_ab == NBK_BF16 && d->N <= 32 && d->M >= 1024 && d->K >= 256 && d->K % 64 == 0 &&
       akc && a.a_vec && d->batch == 1 && d->bias == nullptr && d->residual == nullptr &&
       d->act == NBK_ACT_NONE && (bkc ? (bool)a.b_vec : (d->b_cs == 1 && d->N % 8 == 0 && a.b_vec))) {
@@ -1645,6 +1716,13 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8 &&
                       a_stride >= 0 && b_stride >= 0 && a_stride < (1 << 22) && b_stride < (1 << 22);
+    if (d->colsum != nullptr) {
+      NBK_REQUIRE(fast && !akc && !bkc && a.batch_inner == 1 && d->bias == nullptr &&
+                      d->residual == nullptr && d->act == NBK_ACT_NONE && d->alpha == 1.f,
+                  "gemm: column sums go with a plain bf16 product of two row-contiguous, 16-byte "
+                  "aligned operands (K %% 64 == 0, M %% 8 == 0, N %% 8 == 0, one batch level)");
+      return launch_bf16_dl_colsum<128, 128, 4>(a, d->batch, st);
+    }
     if (!fast) return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);
     // 256 x 256 tiles run at about twice the rate of 128 x 128 ones per CU, one workgroup
     // per CU at a time: take them when the rounds of workgroups they need are at least

@@ -267,6 +267,9 @@ def _gemm(a, mem):
     dst = a["dst"]
     out = mat(dst, a["c_bs"], a.get("c_bs2", 0), a["ldc"], 1, a["M"], a["N"])
     out.copy_(C.to(out.dtype))
+    if a.get("colsum") is not None:  # sum over k of B, one row per batch slice, in C's dtype
+        cs = _view(mem, a["colsum"]).reshape(a["batch"], a["N"])
+        cs.copy_(B.double().sum(dim=2).reshape(a["batch"], a["N"]).to(cs.dtype))
 
 
 _NF4_LEVELS = torch.tensor([-1.0, -0.6962, -0.5251, -0.3949, -0.2844, -0.1848, -0.0911, 0.0, 0.0796,

@@ -693,6 +693,40 @@ def test_an_adapter_update_folds_into_the_sum_with_its_base_product(emulator):
     assert not any("residual" in s.attrs for s in steps_r if s.kind == "gemm")
 
 
+def test_a_bias_gradient_rides_on_the_weight_gradient_product(emulator):
+    """The column sums of dy (the cotangent's reduction to the bias' shape) become a result of
+    the launch that computes x^T dy, whole or split along K; the numbers are those of the
+    separate reduction, and ``FOLD_COLUMN_SUMS`` switches the fold off."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(3)
+    bf = nb.DType.bfloat16
+    for (B, S, D, N), split in (((2, 64, 32, 48), False), ((4, 256, 128, 128), True)):
+        x, w = rng.standard_normal((B, S, D)).astype(np.float32), rng.standard_normal((D, N)).astype(np.float32) * 0.1
+        b, g = rng.standard_normal((N,)).astype(np.float32), rng.standard_normal((B, S, N)).astype(np.float32)
+
+        def loss(p):
+            return nb.reduce_sum(nb.relu(T(x, dtype=bf) @ p["w"] + p["b"]) * T(g, dtype=bf))
+
+        got = {}
+        for on in (True, False):
+            with config.flag("FOLD_COLUMN_SUMS", on):
+                engine.clear_plan_cache()
+                val, grads = nb.value_and_grad(loss)({"w": T(w, dtype=bf), "b": T(b, dtype=bf)})
+                nb.realize_all(val, grads["w"], grads["b"])
+                steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+                hosts = [s for s in steps if s.kind == "gemm" and s.attrs.get("colsum") is not None]
+                assert len(hosts) == (1 if on else 0)
+                if on:
+                    assert (hosts[0].attrs["batch"] > 1) == split
+                got[on] = (nb.cast(grads["b"], nb.DType.float32).numpy(), nb.cast(grads["w"], nb.DType.float32).numpy())
+        engine.clear_plan_cache()
+        np.testing.assert_array_equal(got[True][1], got[False][1])
+        np.testing.assert_allclose(got[True][0], got[False][0], rtol=2e-2, atol=2e-2)
+        dy = _bf16_round(g) * (_bf16_round(x) @ _bf16_round(w * 1.0) + _bf16_round(b) > 0)
+        np.testing.assert_allclose(got[True][0], dy.reshape(-1, N).sum(0), rtol=3e-2, atol=0.3)
+
+
 def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
     """``(x @ W) * c`` with ``c`` a constant of the graph is one product with ``alpha = c`` (the
     way the low-rank adapters carry ``alpha / rank``, forward and backward); a realized scalar

@@ -115,6 +115,63 @@ def test_gemm_long_k_small_output(hip, layout, shape):
     assert err.max() <= 2e-2, err.max()
 
 
+@pytest.mark.parametrize("shape,ks", [((1024, 1024, 2048), 1), ((256, 136, 512), 1), ((1024, 520, 4096), 4),
+                                      ((8, 8, 64), 1), ((4096, 1024, 1024), 1)])
+def test_gemm_column_sums(hip, shape, ks):
+    """The weight gradient x^T dy with the column sums of dy (the bias gradient) as a second
+    result of the same launch: whole, and split along K into fp32 partial products and partial
+    sums.  The product must be what the launch without the sums gives, bit for bit; the sums
+    are checked against fp64 with the rounding of their dtype and accumulation length."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(8)
+    xt = torch.tensor(rng.standard_normal((K, M)), dtype=torch.bfloat16).cuda()   # x, read as x^T
+    dy = torch.tensor(rng.standard_normal((K, N)) + 0.25, dtype=torch.bfloat16).cuda()
+    odt = torch.bfloat16 if ks == 1 else torch.float32
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(with_sums):
+        c = torch.full((ks, M, N), float("nan"), dtype=odt, device="cuda")
+        cs = torch.full((ks, N), float("nan"), dtype=odt, device="cuda")
+        d = lib.GemmDesc()
+        d.A, d.B, d.C = xt.data_ptr(), dy.data_ptr(), c.data_ptr()
+        d.M, d.N, d.K = M, N, K // ks
+        d.a_rs, d.a_cs, d.b_rs, d.b_cs, d.ldc = 1, M, N, 1, N
+        d.batch, d.a_bs, d.b_bs, d.c_bs, d.batch_inner = ks, (K // ks) * M, (K // ks) * N, M * N, 1
+        d.dtype_ab, d.dtype_c, d.alpha = 1, (1 if ks == 1 else 0), 1.0
+        d.colsum = cs.data_ptr() if with_sums else None
+        lib.check(L.nbk_gemm(C.byref(d), st))
+        torch.cuda.synchronize()
+        return c, cs
+
+    c0, _ = run(False)
+    c1, cs = run(True)
+    ref_c = (xt.double().t().cpu() @ dy.double().cpu()).numpy()
+    got_c = c1.double().sum(0).cpu().numpy()
+    assert (np.abs(got_c - ref_c) - 2.0 ** -8 * np.abs(ref_c)).max() <= 2e-2
+    if K // ks > 16 and not (M >= 256 and N >= 256 and -(-M // 256) * -(-N // 256) * ks * 10 >= 256 * 6):
+        # (the same kernel and tile with and without the sums: identical products)
+        assert torch.equal(c0, c1)
+    ref_s = dy.double().cpu().reshape(ks, K // ks, N).sum(1).numpy()
+    got_s = cs.double().cpu().numpy()
+    tol = 2.0 ** -8 * np.abs(ref_s) + 1e-4 * np.sqrt(K / ks)
+    assert (np.abs(got_s - ref_s) <= tol).all(), np.abs(got_s - ref_s).max()
+
+
+def test_gemm_column_sums_refuses_what_the_kernel_does_not_cover(hip):
+    from nabla_amd.backend import lib
+    a = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    cs = torch.zeros((64,), dtype=torch.bfloat16, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C, d.colsum = a.data_ptr(), a.data_ptr(), a.data_ptr(), cs.data_ptr()
+    d.M = d.N = d.K = 64
+    d.a_rs, d.a_cs, d.b_rs, d.b_cs, d.ldc = 64, 1, 64, 1, 64      # A K-contiguous: not covered
+    d.batch, d.batch_inner, d.dtype_ab, d.dtype_c, d.alpha = 1, 1, 1, 1, 1.0
+    L = lib.load()
+    assert L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)) != 0
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("act", [0, 1, 2])
 @pytest.mark.parametrize("shape", [(256, 384, 128),      # 128 x 128 tiles
