@@ -297,17 +297,39 @@ extern __shared__ __align__(16) u32x4 gemm_lds[];
 // buffers are free).
 // EPI: 0 plain, 1 bias only (as lean as the plain form), 2 bias / activation / residual (the
 // residual requested for the whole wave tile up front), 3 bias and an added residual read pass by
-// pass (for kernels whose occupancy hides that latency and must not lose it to registers).
+// pass (for kernels whose occupancy hides that latency and must not lose it to registers), 4 bias
+// and an added bf16 residual that the caller requested before its product (`pre`: the 16-byte
+// piece of every pass of every band, in this function's lane layout -- gemm_residual_prefetch).
 // Each wave passes its accumulators through a private LDS slab, a band of 32 rows of its tile
 // at a time (`scatter(band, slab)` writes the band's accumulators there, row-major with a
 // pitch of WN + 4 floats), so that C is written as whole 16-byte (bf16) / 32-byte (fp32)
 // pieces of a row: 8 columns per lane.  The plain form (no bias / activation / residual)
 // is a separate instantiation: the fused form carries erf() bodies, and an epilogue that does
 // not fit the instruction cache costs more than the whole K loop of a short GEMM.
+// The residual pieces this lane adds in an EPI 4 epilogue, requested up front (rows and columns
+// past the edge read a valid address and are never used).  The caller has checked that C is
+// bf16 and that residual, ldc and N allow 16-byte pieces.
+template <int TM, int WN>
+__device__ __forceinline__ void gemm_residual_prefetch(const GemmArgs& g, int64_t m0, int64_t n0, int wm,
+                                                       int wn, int lane, uint4 (&pre)[TM * (WN / 16)]) {
+  constexpr int LANES_PER_ROW = WN / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW, NP = 32 / ROWS_PER_PASS;
+  const int sub_r = lane / LANES_PER_ROW, sub_c = (lane % LANES_PER_ROW) * 8;
+  int64_t col = n0 + wn + sub_c;
+  col = col + 8 <= g.N ? col : 0;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int pass = 0; pass < NP; ++pass) {
+      int64_t row = m0 + wm + i * 32 + pass * ROWS_PER_PASS + sub_r;
+      row = row < g.M ? row : g.M - 1;
+      pre[i * NP + pass] = *(const uint4*)((const uint16_t*)g.residual + row * g.ldc + col);
+    }
+}
+
 template <int TM, int WN, bool FAST, int EPI, typename Scatter>
 __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const GemmArgs& g, int64_t m0,
                                                     int64_t n0, int wm, int wn, int64_t c_off, int wave,
-                                                    int lane) {
+                                                    int lane, const uint4* pre = nullptr) {
   constexpr int SLAB_LD = WN + 4;  // floats per slab row (padding spreads the row groups)
   float* slab = (float*)gemm_lds + wave * (32 * SLAB_LD);
   const bool out_f32 = g.dtype_c == NBK_F32;
@@ -366,9 +388,15 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
         const int64_t idx = c_off + row * g.ldc + col;
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
-        if (EPI == 1 || EPI == 3) {
+        if (EPI == 1 || EPI == 3 || EPI == 4) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] += bias_v[e];
+        }
+        if (EPI == 4) {
+          v[0] += __uint_as_float(u.x << 16); v[1] += __uint_as_float(u.x & 0xffff0000u);
+          v[2] += __uint_as_float(u.y << 16); v[3] += __uint_as_float(u.y & 0xffff0000u);
+          v[4] += __uint_as_float(u.z << 16); v[5] += __uint_as_float(u.z & 0xffff0000u);
+          v[6] += __uint_as_float(u.w << 16); v[7] += __uint_as_float(u.w & 0xffff0000u);
         }
         if (EPI == 3 && g.residual) {
           if (vec_store && !out_f32) {
@@ -459,6 +487,9 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
     if constexpr (EPI == 2) {
 #pragma unroll
       for (int pass = 0; pass < NP; ++pass) one_pass(pass, rpre[i][pass]);
+    } else if constexpr (EPI == 4) {
+#pragma unroll
+      for (int pass = 0; pass < NP; ++pass) one_pass(pass, pre[i * NP + pass]);
     } else {
 #pragma unroll 1
       for (int pass = 0; pass < NP; ++pass) one_pass(pass, make_uint4(0u, 0u, 0u, 0u));
@@ -471,7 +502,7 @@ __device__ __forceinline__ void gemm_epilogue_bands(Scatter&& scatter, const Gem
 template <int TM, int TN, int WN, bool FAST, int EPI>
 __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmArgs& g, int64_t m0,
                                               int64_t n0, int wm, int wn, int64_t c_off, int wave,
-                                              int lane) {
+                                              int lane, const uint4* pre = nullptr) {
   const int li = lane & 31, kg = lane >> 5;
   gemm_epilogue_bands<TM, WN, FAST, EPI>(
       [&](auto ti, float* slab) {
@@ -484,7 +515,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const GemmA
             slab[((r >> 2) * 8 + kg * 4 + (r & 3)) * (WN + 4) + j * 32 + li] = a[r];
         });
       },
-      g, m0, n0, wm, wn, c_off, wave, lane);
+      g, m0, n0, wm, wn, c_off, wave, lane, pre);
 }
 
 // 16x16 MFMA blocks: D[i][j] lives in lane (j, i / 4), register i % 4; a band is two block rows.
@@ -1131,6 +1162,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
     }
     return *(const bf16x8*)&u;
   };
+  // (EPI 4: the residual is on its way before the operands are, one memory latency for both)
+  uint4 pre[TM * (WN / 16)];
+  if constexpr (EPI == 4) gemm_residual_prefetch<TM, WN>(g, m0, n0, wm, wn, lane, pre);
   bf16x8 fa[TM], fb[TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -1150,7 +1184,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], (f32x16)(0.f), 0, 0, 0);
-  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane);
+  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane, EPI == 4 ? pre : nullptr);
 }
 
 // ------------------------------------------------------------------- bf16, N <= 32
@@ -1697,10 +1731,13 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     // 0 plain; 3 a bias and / or an added residual (the adapter's update on top of the base
     // product: all memory traffic, so the lean epilogue that keeps four waves per SIMD); 2 the rest
     const bool any = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
-    const int epi = !any ? 0 : ((a.act == NBK_ACT_NONE && a.C2 == nullptr && !a.res_mul) ? 3 : 2);
+    // (4: the same with the residual requested before the operands -- bf16 results only)
+    const int epi = !any ? 0 : ((a.act == NBK_ACT_NONE && a.C2 == nullptr && !a.res_mul)
+                                    ? (a.residual != nullptr && d->dtype_c == NBK_BF16 ? 4 : 3) : 2);
 #define NBK_LAUNCH_SKK(BK_)                                                                        \
   do {                                                                                             \
     if (epi == 0) hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 0>), grid, dim3(256), lds, st, a); \
+    else if (epi == 4) hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 4>), grid, dim3(256), lds, st, a); \
     else if (epi == 3) hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 3>), grid, dim3(256), lds, st, a); \
     else hipLaunchKernelGGL((gemm_skinny_k_kernel<BK_, 2>), grid, dim3(256), lds, st, a);         \
   } while (0)
