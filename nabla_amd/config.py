@@ -60,6 +60,10 @@ _FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
 _FOLD_COLUMN_SUMS: ContextVar[bool] = ContextVar(
     "FOLD_COLUMN_SUMS", default=_env_flag("NBK_FOLD_COLUMN_SUMS", True))
 
+# vmap runs the mapped function once on tensors with a hidden leading axis where every op it
+# uses has a batching rule; off (or an op without a rule): one trace per element, stacked
+_VMAP_BATCHED: ContextVar[bool] = ContextVar("VMAP_BATCHED", default=_env_flag("NBK_VMAP_BATCHED", True))
+
 # the backward pass of the exact GELU computes GELU'(x) from the kept pre-activation, in the
 # kernel that multiplies it with the cotangent; off: the forward kernel stores GELU'(x) as a
 # second full-size result and the backward kernel reads it
@@ -87,6 +91,7 @@ _FLAGS = {
     "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
     "FOLD_SCALE": _FOLD_SCALE,
     "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
+    "VMAP_BATCHED": _VMAP_BATCHED,
     "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,
     "MULTI_TENSOR_OPTIMIZER": _MULTI_TENSOR_OPTIMIZER,

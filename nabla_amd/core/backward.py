@@ -11,7 +11,7 @@ from __future__ import annotations
 from typing import Any
 
 from .pytree import tree_leaves
-from .tensor import Tensor, TensorImpl
+from .tensor import BatchedTensor, Tensor, TensorImpl
 from .tracing import OpNode, Trace
 
 
@@ -52,9 +52,10 @@ class BackwardEngine:
         if len(outs) != len(cots):
             raise ValueError(f"backward: {len(outs)} outputs but {len(cots)} cotangents")
         for o, c in zip(outs, cots):
-            if tuple(o.shape) != tuple(c.shape):
+            # (stored shapes: inside vmap both carry the hidden batch dimensions)
+            if tuple(o._impl.shape) != tuple(c._impl.shape):
                 raise ValueError(f"cotangent shape {c.shape} does not match output shape {o.shape}")
-            _accumulate_cotangent(self.cotangent_map, o._impl, c)
+            _accumulate_cotangent(self.cotangent_map, o._impl, Tensor(impl=c._impl))
 
     def run(self) -> dict:
         for node in reversed(self.trace.nodes):
@@ -109,7 +110,9 @@ class BackwardEngine:
             if not isinstance(inp, Tensor):
                 continue
             c = self.cotangent_map.get(inp._impl)
-            grads[inp] = Tensor(impl=c) if c is not None else zeros_like(inp)
+            g = Tensor(impl=c) if c is not None else zeros_like(Tensor(impl=inp._impl))
+            # the gradient of a tensor seen from inside vmap hides the same dimensions
+            grads[inp] = BatchedTensor(g, inp._bd) if isinstance(inp, BatchedTensor) else g
         return grads
 
 

@@ -404,6 +404,46 @@ class Tensor:
         return getitem(self, key)
 
 
+class BatchedTensor(Tensor):
+    """What a function sees of a mapped argument inside ``vmap``: the tensor with its first
+    ``_bd`` (hidden) dimensions taken away.  The storage keeps them, in front; ``shape``,
+    ``rank`` and the axis arguments of every op are those of one element, and each op call
+    that meets such a tensor runs once on the whole batch with its axes shifted
+    (nabla_amd/ops/batching.py).  Plays the part of the ``batch_dims`` counter of the
+    reference's tensors (nabla/core/tensor/impl.py, nabla/ops/view/batch.py)."""
+
+    __slots__ = ("_bd",)
+
+    def __init__(self, physical: Tensor, batch_dims: int):
+        Tensor.__init__(self, impl=physical._impl)
+        self._bd = int(batch_dims)
+
+    def physical(self) -> Tensor:
+        """The same storage with the hidden dimensions in view."""
+        return Tensor(impl=self._impl)
+
+    @property
+    def batch_shape(self) -> tuple[int, ...]:
+        return tuple(self._impl.shape[:self._bd])
+
+    @property
+    def shape(self) -> tuple[int, ...]:
+        return tuple(self._impl.shape[self._bd:])
+
+    @property
+    def rank(self) -> int:
+        return len(self._impl.shape) - self._bd
+
+    ndim = rank
+
+    def dim(self) -> int:
+        return len(self._impl.shape) - self._bd
+
+    def __repr__(self) -> str:
+        return (f"BatchedTensor(shape={self.shape}, batch={self.batch_shape}, "
+                f"dtype={self.dtype.name})")
+
+
 def _ensure_tensor(value: Any, like: Tensor) -> Tensor:
     if isinstance(value, Tensor):
         return value

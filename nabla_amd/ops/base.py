@@ -21,7 +21,7 @@ from typing import Any
 from .. import config
 from ..core.dtype import DType, promote
 from ..core.pytree import PyTreeDef, _K_LEAF
-from ..core.tensor import Tensor, TensorImpl
+from ..core.tensor import BatchedTensor, Tensor, TensorImpl
 from ..core.tracing import OpNode
 
 _LEAF_DEF = PyTreeDef(_K_LEAF, None, (), 1)
@@ -87,6 +87,10 @@ class Operation(ABC):
     # -- call pipeline ----------------------------------------------------------------
     def __call__(self, args: OpArgs, kwargs: OpKwargs) -> OpResult:
         kwargs = kwargs or {}
+        for a in args:
+            if type(a) is BatchedTensor:  # inside vmap: once for the whole batch, axes shifted
+                from . import batching
+                return batching.dispatch(self, args, kwargs)
         tensors = [a for a in args if isinstance(a, Tensor)]
         any_traced = False
         for t in tensors:

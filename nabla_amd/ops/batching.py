@@ -1,0 +1,184 @@
+"""Batching rules: how an op call that meets a ``BatchedTensor`` runs once on the whole batch.
+
+The reference gives every tensor a ``batch_dims`` counter and lets each op translate its
+logical axes to physical ones (nabla/ops/base.py:294-395 ``adapt_kwargs``,
+nabla/ops/view/batch.py, nabla/transforms/vmap.py:153-288).  Here the same translation sits in
+one place.  ``Operation.__call__`` hands a call over to :func:`dispatch` when one of its tensor
+arguments is batched; the rule for the op's class
+
+* brings every tensor argument to the same number of leading hidden dimensions (a tensor from
+  an outer ``vmap`` level gets size-1 dimensions behind its own, an unmapped tensor in front
+  of its shape) and broadcasts them to the batch sizes -- views, nothing is copied,
+* shifts the axes that the keyword arguments name past the hidden dimensions (negative axes
+  count from the end and stay as they are) and puts the batch sizes in front of shapes,
+* runs the op on the plain tensors and wraps its results again.
+
+An op without a rule raises :class:`NoBatchRule`; ``vmap`` then maps the function element by
+element instead, which is always possible.  Backward passes never come through here: a VJP rule
+replays on the plain tensors of the recorded ops, which form a valid program of their own.
+"""
+from __future__ import annotations
+
+from typing import Any, Callable
+
+from ..core.tensor import BatchedTensor, Tensor
+
+
+class NoBatchRule(Exception):
+    """The op has no batching rule (or not for this combination of arguments)."""
+
+
+# sizes of the hidden dimensions of the vmap calls that are being traced, outermost first
+_LEVELS: list[int] = []
+
+
+def current_level() -> int:
+    return len(_LEVELS)
+
+
+def push_level(size: int) -> None:
+    _LEVELS.append(int(size))
+
+
+def pop_level() -> None:
+    _LEVELS.pop()
+
+
+def plain(t: Tensor) -> Tensor:
+    return t.physical() if isinstance(t, BatchedTensor) else t
+
+
+def batch_dims_of(t: Any) -> int:
+    return t._bd if isinstance(t, BatchedTensor) else 0
+
+
+def lift(t: Tensor, bd: int, sizes: tuple[int, ...], logical_rank: int | None = None) -> Tensor:
+    """``t`` as a plain tensor of shape ``sizes + (1,) * pad + t.shape``: hidden dimensions it
+    does not have are size-1 dimensions broadcast to ``sizes``; ``logical_rank`` pads the
+    element's own shape with leading 1s (numpy alignment of operands of different rank)."""
+    from . import view
+
+    own = batch_dims_of(t)
+    phys = plain(t)
+    lshape = tuple(phys.shape[own:])
+    pad = 0 if logical_rank is None else logical_rank - len(lshape)
+    if pad < 0:
+        raise NoBatchRule("operand rank exceeds the result's")
+    have = tuple(phys.shape[:own]) + (1,) * (bd - own)
+    want_shape = have + (1,) * pad + lshape
+    if tuple(phys.shape) != want_shape:
+        phys = view.reshape(phys, want_shape)
+    full = tuple(sizes) + (1,) * pad + lshape
+    if want_shape != full:
+        phys = view.broadcast_to(phys, full)
+    return phys
+
+
+def _shift(axis: int, bd: int) -> int:
+    return axis if axis < 0 else axis + bd
+
+
+# ------------------------------------------------------------------------------ rules
+# rule(op, args, kwargs, bd, sizes) -> (plain args, physical kwargs)
+def _rule_same_shape(op, args, kwargs, bd, sizes):
+    """Elementwise ops whose operands already have one (logical) shape, reductions and other
+    ops that name at most an ``axis``: lift everything, shift the axis."""
+    out = [lift(a, bd, sizes) if isinstance(a, Tensor) else a for a in args]
+    kw = dict(kwargs)
+    if isinstance(kw.get("axis"), int):
+        kw["axis"] = _shift(kw["axis"], bd)
+    return out, kw
+
+
+def _rule_broadcast_to(op, args, kwargs, bd, sizes):
+    shape = tuple(kwargs["shape"])
+    x = lift(args[0], bd, sizes, logical_rank=len(shape))
+    return [x], dict(kwargs, shape=tuple(sizes) + shape)
+
+
+def _rule_reshape(op, args, kwargs, bd, sizes):
+    return [lift(args[0], bd, sizes)], dict(kwargs, shape=tuple(sizes) + tuple(kwargs["shape"]))
+
+
+def _rule_permute(op, args, kwargs, bd, sizes):
+    order = [int(o) for o in kwargs["order"]]
+    rank = len(order)
+    order = [o + rank if o < 0 else o for o in order]
+    return [lift(args[0], bd, sizes)], dict(kwargs, order=tuple(range(bd)) + tuple(o + bd for o in order))
+
+
+def _rule_slice(op, args, kwargs, bd, sizes):
+    out = [lift(a, bd, sizes) if isinstance(a, Tensor) else a for a in args]
+    return out, dict(kwargs, start=(0,) * bd + tuple(kwargs["start"]),
+                     size=tuple(sizes) + tuple(kwargs["size"]))
+
+
+def _rule_pad(op, args, kwargs, bd, sizes):
+    pads = tuple((int(a), int(b)) for a, b in kwargs["paddings"])
+    return [lift(args[0], bd, sizes)], dict(kwargs, paddings=((0, 0),) * bd + pads)
+
+
+def _rule_layer_norm(op, args, kwargs, bd, sizes):
+    # the statistics are per row either way; weight and bias are vectors over the last axis and
+    # must be the same for every element of the batch
+    if any(isinstance(a, BatchedTensor) for a in args[1:]):
+        raise NoBatchRule("layer_norm with mapped weight or bias")
+    return [lift(args[0], bd, sizes)] + list(args[1:]), dict(kwargs)
+
+
+def _rules() -> list[tuple[type, Callable]]:
+    from . import binary, comparison, control_flow, creation, normalization, reduction, unary, view
+    from .base import BinaryOperation, ReduceOperation, UnaryOperation
+
+    return [
+        (view.BroadcastToOp, _rule_broadcast_to),
+        (view.ReshapeOp, _rule_reshape),
+        (view.PermuteOp, _rule_permute),
+        (view.SliceTensorOp, _rule_slice),
+        (view.SliceUpdateOp, _rule_slice),
+        (view.PadOp, _rule_pad),
+        (view.ConcatenateOp, _rule_same_shape),
+        (normalization.LayerNormOp, _rule_layer_norm),
+        (binary.MatmulOp, _rule_same_shape),
+        (control_flow.WhereOp, _rule_same_shape),
+        (unary.GeluBackwardOp, _rule_same_shape),
+        (BinaryOperation, _rule_same_shape),
+        (ReduceOperation, _rule_same_shape),
+        (UnaryOperation, _rule_same_shape),
+    ]
+
+
+_RULES: list[tuple[type, Callable]] | None = None
+
+
+def _rule_for(op) -> Callable | None:
+    global _RULES
+    if _RULES is None:
+        _RULES = _rules()
+    for cls, rule in _RULES:
+        if isinstance(op, cls):
+            return rule
+    return None
+
+
+def dispatch(op, args: list, kwargs: dict) -> list:
+    """Run ``op`` on arguments of which at least one is batched."""
+    rule = _rule_for(op)
+    if rule is None:
+        raise NoBatchRule(f"op '{op.name}' has no batching rule")
+    batched = [a for a in args if isinstance(a, BatchedTensor)]
+    bd = max(a._bd for a in batched)
+    sizes = [1] * bd
+    for a in batched:
+        for i, d in enumerate(a.batch_shape):
+            if d != 1:
+                if sizes[i] not in (1, d):
+                    raise ValueError(f"vmap: mapped axes of sizes {sizes[i]} and {d} meet in '{op.name}'")
+                sizes[i] = d
+    phys_args, phys_kwargs = rule(op, list(args), dict(kwargs or {}), bd, tuple(sizes))
+    outs = op(phys_args, phys_kwargs)
+    return [BatchedTensor(o, bd) for o in outs]
+
+
+__all__ = ["NoBatchRule", "dispatch", "lift", "plain", "batch_dims_of", "current_level",
+           "push_level", "pop_level"]

@@ -10,14 +10,37 @@ from ..core.tracing import trace
 from .utils import select_argnums
 
 
+def lift_to_vmap_level(args):
+    """Inside ``vmap``, a derivative is taken per element of the batch, also with respect to an
+    argument that is the same for every element: such an argument is given the hidden
+    dimensions of the running ``vmap`` calls (a broadcast view) before the function is traced,
+    so that its gradient comes back with one slice per element instead of their sum."""
+    from ..core.tensor import BatchedTensor
+    from ..ops import batching
+
+    level = batching.current_level()
+    if not level:
+        return args
+    sizes = tuple(batching._LEVELS)
+
+    def up(t):
+        if isinstance(t, Tensor) and batching.batch_dims_of(t) < level:
+            return BatchedTensor(batching.lift(t, level, sizes), level)
+        return t
+
+    return pytree.tree_map(up, args)
+
+
 def _run(fun, argnums, create_graph, realize, args, kwargs, with_value: bool):
     from ..ops.creation import ones_like
 
+    args = lift_to_vmap_level(args)
     t = trace(fun, *args, **kwargs)
     output = t.outputs
     if not isinstance(output, Tensor):
         raise TypeError(f"grad: output must be a Tensor, got {type(output)}")
-    grads_map = backward_on_trace(t, ones_like(output), create_graph=create_graph)
+    seed = ones_like(Tensor(impl=output._impl))  # (with the hidden dimensions, inside vmap)
+    grads_map = backward_on_trace(t, seed, create_graph=create_graph)
     leaves = pytree.tree_leaves(args)
     grad_leaves = []
     for inp in leaves:

@@ -34,12 +34,17 @@ def jvp(fn: Callable, primals: tuple, tangents: tuple, *, has_aux: bool = False,
             aux_box.append(aux)
         return out
 
+    from ..core.tensor import BatchedTensor
+    from .grad import lift_to_vmap_level
+    # (inside vmap: primals and tangents carry the same hidden dimensions, see there)
+    primals, tangents = lift_to_vmap_level(primals), lift_to_vmap_level(tangents)
     t = trace(wrapped, *primals)
     tmap = forward_on_trace(t, tangents, create_graph=create_graph)
 
     def tangent_of(x: Any) -> Any:
         if isinstance(x, Tensor):
-            return Tensor(impl=tmap[x._impl]) if x._impl in tmap else zeros_like(x)
+            g = Tensor(impl=tmap[x._impl]) if x._impl in tmap else zeros_like(Tensor(impl=x._impl))
+            return BatchedTensor(g, x._bd) if isinstance(x, BatchedTensor) else g
         return x
 
     out_tangents = pytree.tree_map(tangent_of, t.outputs)

@@ -20,10 +20,13 @@ def vjp(fun: Callable, *primals: Any, has_aux: bool = False, create_graph: bool 
             aux_box.append(aux)
         return out
 
+    from .grad import lift_to_vmap_level
+    primals = lift_to_vmap_level(primals)  # (inside vmap: per-element gradients, see there)
     t = trace(wrapped, *primals)
     output = t.outputs
 
     def vjp_fn(cotangent: Any):
+        cotangent = lift_to_vmap_level(cotangent)
         grads_map = backward_on_trace(t, cotangent, create_graph=create_graph)
         leaves = pytree.tree_leaves(primals)
         gl = [grads_map.get(x) if isinstance(x, Tensor) else None for x in leaves]

@@ -1,12 +1,18 @@
 """``vmap`` (nabla/transforms/vmap.py:291-362): map a function over one axis of its arguments.
 
-The reference gives every tensor hidden batch dimensions and every op a batching rule.  This
-backend has no batch dimensions: the mapped function is traced once per batch element on slices
-of the arguments and the per-element results are stacked, all inside one lazy graph, so the
-planner still sees a single program (B copies of the body; elementwise bodies fuse back into
-one row program per group).  Results and composition (``grad`` of ``vmap``, ``vmap`` of ``grad``,
-nesting) are those of the reference; the cost grows with the batch size, so it is meant for
-the small batch sizes of per-example gradients and Jacobians, not as a way to batch a model.
+Two ways to run the mapped function, with the same results:
+
+* **batched** (the reference's way: hidden batch dimensions and a batching rule per op).  The
+  mapped axis goes to the front, the function is called ONCE on ``BatchedTensor`` views that
+  hide that axis, and every op call translates its axes and runs on the whole batch
+  (nabla_amd/ops/batching.py).  The cost does not grow with the batch size: per-example
+  gradients of a model are one forward and one backward pass over the batch.
+* **element by element**: the function is traced once per batch element on slices of the
+  arguments and the results are stacked, all inside one lazy graph.  Used when the function
+  reaches an op that has no batching rule (gathers, convolutions, pooling, the fused attention
+  and cross-entropy ops, custom kernels) or when ``config.VMAP_BATCHED`` is off.
+
+Composition (``grad`` of ``vmap``, ``vmap`` of ``grad``, nesting) is the reference's either way.
 
 ``in_axes`` / ``out_axes`` follow the reference (vmap.py:44-60, 63-150): an int or ``None`` for
 every argument, a tuple / list with one entry per argument, and an entry may itself be a
@@ -80,6 +86,8 @@ def vmap(func: Callable | None = None, in_axes: Any = 0, out_axes: Any = 0,
                                   "this one-GPU backend")
 
     def vectorized(*args: Any) -> Any:
+        from .. import config
+        from ..ops.batching import NoBatchRule
         from ..ops.view import moveaxis, stack
 
         if not args:
@@ -96,6 +104,11 @@ def vmap(func: Callable | None = None, in_axes: Any = 0, out_axes: Any = 0,
             size = dims[0]
             if axis_size is not None and int(axis_size) != size:
                 raise ValueError(f"axis_size={axis_size} doesn't match inferred {size}")
+        if config.VMAP_BATCHED and size > 0:
+            try:
+                return _run_batched(func, args, in_ax, out_axes, size)
+            except NoBatchRule:
+                pass  # an op of the function has no batching rule: map element by element
 
         # the mapped axis goes to the front once, then element i is a leading-index view
         fronted = tuple(_walk(lambda t, ax: t if ax is None else moveaxis(t, ax, 0), a, ax)
@@ -149,6 +162,62 @@ def vmap(func: Callable | None = None, in_axes: Any = 0, out_axes: Any = 0,
         return stacked[0] if is_single else type(first)(stacked)
 
     return vectorized
+
+
+def _run_batched(func: Callable, args: tuple, in_ax: tuple, out_axes: Any, size: int) -> Any:
+    """One call of ``func`` on views that hide the mapped axis (see the module docstring)."""
+    from ..core.tensor import BatchedTensor
+    from ..ops import batching
+    from ..ops.view import broadcast_to, moveaxis, reshape
+
+    outer = batching.current_level()
+    level = outer + 1
+
+    def hide(t: Tensor, ax):
+        if ax is None:
+            return t
+        # the mapped axis becomes the last hidden dimension: behind those of the vmap calls
+        # this one is nested in (which a tensor that does not come from them lacks: size 1)
+        own = batching.batch_dims_of(t)
+        front = moveaxis(t, ax, 0)  # (a logical move: hidden dimensions stay in front)
+        phys = batching.plain(front)
+        if own < outer:
+            shape = tuple(phys.shape)
+            phys = reshape(phys, shape[:own] + (1,) * (outer - own) + shape[own:])
+        return BatchedTensor(phys, level)
+
+    wrapped = tuple(_walk(hide, a, ax) for a, ax in zip(args, in_ax))
+    batching.push_level(size)
+    try:
+        result = func(*wrapped)
+    finally:
+        batching.pop_level()
+
+    is_single = not isinstance(result, (list, tuple))
+    outs = [result] if is_single else list(result)
+    out_ax = _broadcast_to_args(out_axes, len(outs))
+
+    def show(t: Tensor, ax):
+        own = batching.batch_dims_of(t)
+        if own < level:
+            # does not depend on the mapped arguments: the same for every element
+            if ax is None:
+                return t
+            lshape = tuple(t.shape)
+            rep = broadcast_to(reshape(t, (1,) + lshape), (size,) + lshape)
+            return moveaxis(rep, 0, ax if ax >= 0 else ax + len(lshape) + 1)
+        if ax is None:
+            raise ValueError("vmap: out_axes is None for a result that depends on a mapped argument")
+        phys = batching.plain(t)
+        if phys.shape[outer] != size:  # a size-1 hidden dimension that was never broadcast
+            shape = tuple(phys.shape)
+            phys = broadcast_to(phys, shape[:outer] + (size,) + shape[outer + 1:])
+        seen = BatchedTensor(phys, outer) if outer > 0 else phys
+        nd = len(seen.shape)
+        return moveaxis(seen, 0, ax if ax >= 0 else ax + nd)
+
+    shown = [_walk(show, o, ax) for o, ax in zip(outs, out_ax)]
+    return shown[0] if is_single else type(result)(shown)
 
 
 __all__ = ["vmap"]

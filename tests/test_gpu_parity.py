@@ -606,6 +606,40 @@ def test_vmap_per_example_gradients_on_device(hip):
     assert relerr(total.numpy(), want.sum(axis=0)) <= F32_TOL
 
 
+def test_vmap_batched_per_example_gradients_of_a_block_on_device(hip):
+    """Per-example gradients of a two-layer block with layer norm over 256 examples: vmap runs
+    the function once on the batch (its launches do not grow with the batch), and the result is
+    the float64 closed form per example, computed by looping in numpy."""
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(50)
+    n, s, d, h = 256, 8, 32, 64
+    X, Y = rng.standard_normal((n, s, d)), rng.standard_normal((n, s, d))
+    W1, W2 = rng.standard_normal((d, h)) / np.sqrt(d), rng.standard_normal((h, d)) / np.sqrt(h)
+    F = nb.nn.functional
+    calls = []
+
+    def loss(p, x, y):
+        calls.append(1)
+        z = F.layer_norm(x, None, None)
+        return nb.mean((nb.tanh(z @ p["w1"]) @ p["w2"] - y) ** 2.0)
+
+    f32 = lambda a: T(a.astype(np.float32))
+    engine.clear_plan_cache()
+    g = nb.vmap(nb.grad(loss), in_axes=(None, 0, 0))({"w1": f32(W1), "w2": f32(W2)}, f32(X), f32(Y))
+    got = {k: v.numpy() for k, v in g.items()}
+    steps = sum(len(bp.plan.steps) for bp in engine._PLAN_CACHE.values())
+    engine.clear_plan_cache()
+    assert len(calls) == 1 and steps < 40
+    mu, var = X.mean(-1, keepdims=True), X.var(-1, keepdims=True)
+    Z = (X - mu) / np.sqrt(var + 1e-5)
+    A = np.tanh(Z @ W1)
+    R = 2.0 * (A @ W2 - Y) / (s * d)
+    want2 = np.einsum("nsh,nsd->nhd", A, R)
+    want1 = np.einsum("nsd,nsh->ndh", Z, (R @ W2.T) * (1.0 - A * A))
+    assert got["w1"].shape == want1.shape and got["w2"].shape == want2.shape
+    assert relerr(got["w2"], want2) <= 5e-5 and relerr(got["w1"], want1) <= 5e-5
+
+
 def test_small_composite_ops_on_device(hip):
     """trunc / floor / is_nan / is_inf / flip exactly and log1p to fp32 rounding on the device
     (NaN and infinity must survive the kernels' compare instructions)."""

@@ -85,3 +85,129 @@ def test_errors(emulator):
         nb.vmap(lambda: x)()
     with pytest.raises(NotImplementedError, match="mesh"):
         nb.vmap(lambda a: a, spmd_axis_name="dp")
+
+
+# ---- the batched way: one call of the function, hidden batch dimension ----------------------
+def _both_ways(fn, *args, **kw):
+    """Result of ``vmap(fn, **kw)(*args)`` run batched and element by element, and how often each
+    way called ``fn``."""
+    from nabla_amd import config
+    calls = []
+
+    def counted(*a):
+        calls.append(1)
+        return fn(*a)
+
+    out = {}
+    for batched in (True, False):
+        calls.clear()
+        with config.flag("VMAP_BATCHED", batched):
+            r = nb.vmap(counted, **kw)(*args)
+        leaves = r if isinstance(r, (list, tuple)) else [r]
+        out[batched] = ([t.numpy() for t in leaves], len(calls))
+    return out
+
+
+_X = RNG.standard_normal((6, 4, 5))
+_Y = RNG.standard_normal((6, 5))
+_CASES = {
+    "rank mix": (lambda a, b: a * b + 1.0, (_X, _Y), {}),                      # [4,5] * [5]
+    "unmapped higher rank": (lambda a, b: a + b, (_Y, _X), {"in_axes": (0, None)}),  # [5] + [6,4,5]
+    "matvec both orders": (lambda a, v: (a @ v, v @ a.T), (_X, _Y), {}),
+    "reductions": (lambda a: (nb.reduce_sum(a, axis=0), nb.reduce_max(a, axis=-1, keepdims=True),
+                              nb.mean(a), nb.cast(nb.argmax(a, axis=1), nb.DType.float32)), (_X,), {}),
+    "softmax and where": (lambda a: nb.where(nb.greater(a, 0.0), nb.softmax(a, axis=0), nb.exp(a)), (_X,), {}),
+    "views": (lambda a: (a.T, a.reshape(5, 4), a[1:3, ::1], a[2], nb.unsqueeze(a, 1),
+                         nb.flatten(a), nb.permute(a, (1, 0))), (_X,), {}),
+    "pad concat stack": (lambda a, b: (nb.pad(a, [(1, 0), (0, 2)]), nb.concatenate([a, a * 2.0], axis=1),
+                                       nb.stack([b, b + 1.0], axis=0)), (_X, _Y), {}),
+    "layer norm": (lambda a: nb.nn.functional.layer_norm(a, T(np.linspace(0.5, 1.5, 5)), T(np.ones(5) * 0.1)),
+                   (_X,), {}),
+    "mapped axis in the middle, result axis last": (lambda a: nb.tanh(a) * 2.0, (_X,),
+                                                    {"in_axes": 1, "out_axes": -1}),
+    "constant result": (lambda a: (nb.ones((2,)), a), (_Y,), {"out_axes": (0, 0)}),
+    "slice_update": (lambda a, b: nb.slice_update(a, nb.unsqueeze(b, 0), (1, 0), (1, 5)), (_X, _Y), {}),
+    "tril": (lambda a: nb.tril(a @ a.T), (_X,), {}),
+}
+
+
+@pytest.mark.parametrize("name", sorted(_CASES))
+def test_batched_way_calls_the_function_once_and_agrees(emulator, name):
+    fn, arrays, kw = _CASES[name]
+    got = _both_ways(fn, *[T(a) for a in arrays], **kw)
+    (batched, n_b), (mapped, n_m) = got[True], got[False]
+    assert n_b == 1 and n_m > 1  # (once against once per element of the mapped axis)
+    assert len(batched) == len(mapped)
+    for a, b in zip(batched, mapped):
+        assert a.shape == b.shape
+        np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_per_example_gradients_cost_one_pass(emulator):
+    """vmap(grad(f)) with the parameters unmapped: one forward and one backward over the batch,
+    the same launches for 4 and for 32 examples, results those of the element-wise map."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    W, B = RNG.standard_normal((5, 7)), RNG.standard_normal((7,))
+
+    def loss(p, x, y):
+        return nb.mean((nb.tanh(x @ p["w"] + p["b"]) - y) ** 2.0)
+
+    steps = {}
+    for n in (4, 32):
+        X, Y = RNG.standard_normal((n, 3, 5)), RNG.standard_normal((n, 3, 7))
+        res = {}
+        for batched in (True, False):
+            with config.flag("VMAP_BATCHED", batched):
+                engine.clear_plan_cache()
+                g = nb.vmap(nb.grad(loss), in_axes=(None, 0, 0))({"w": T(W), "b": T(B)}, T(X), T(Y))
+                res[batched] = {k: v.numpy() for k, v in g.items()}
+                if batched:
+                    steps[n] = sum(len(bp.plan.steps) for bp in engine._PLAN_CACHE.values())
+        engine.clear_plan_cache()
+        assert res[True]["w"].shape == (n, 5, 7) and res[True]["b"].shape == (n, 7)
+        for k in res[True]:
+            np.testing.assert_allclose(res[True][k], res[False][k], rtol=1e-5, atol=1e-6)
+        h = np.tanh(X @ W + B)
+        dz = 2.0 * (h - Y) / 21.0 * (1.0 - h * h)
+        np.testing.assert_allclose(res[True]["w"], np.einsum("nsi,nsj->nij", X, dz), rtol=1e-4, atol=1e-5)
+    assert steps[4] == steps[32]
+
+
+def test_nested_batched_maps_and_vjp_inside(emulator):
+    A, Bm = RNG.standard_normal((4, 5)), RNG.standard_normal((3, 5))
+    pair = nb.vmap(nb.vmap(lambda a, b: nb.reduce_sum(a * b), in_axes=(0, None)), in_axes=(None, 0))
+    close(pair(T(A), T(Bm)), Bm @ A.T)
+    # an inner map over a tensor that does not come from the outer one
+    mixed = nb.vmap(lambda b: nb.vmap(lambda a: nb.reduce_sum(a * b))(T(A)))
+    close(mixed(T(Bm)), Bm @ A.T)
+
+    def pulled(x):
+        out, back = nb.vjp(lambda v: nb.exp(v) * 2.0, x)
+        return back(nb.ones_like(out))[0]
+
+    close(nb.vmap(pulled)(T(A)), 2.0 * np.exp(A), 1e-4)
+
+
+def test_ops_without_a_batching_rule_fall_back_to_the_map(emulator):
+    table, idx = RNG.standard_normal((7, 3)), np.array([[1, 2], [6, 0], [3, 3]])
+    calls = []
+
+    def look_up(i):
+        calls.append(1)
+        return nb.nn.functional.embedding(i, T(table)) * 2.0
+
+    got = nb.vmap(look_up)(nb.Tensor.constant(idx.astype(np.int64)))
+    assert len(calls) == 1 + 3  # the batched attempt, then one call per element
+    close(got, 2.0 * table[idx])
+
+
+def test_forward_mode_inside_a_batched_map(emulator):
+    X, V, W = RNG.standard_normal((5, 3)), RNG.standard_normal((5, 3)), RNG.standard_normal((3, 4))
+
+    def pushed(x, v):
+        return nb.jvp(lambda a: nb.tanh(a @ T(W)), (x,), (v,))
+
+    out, tan = nb.vmap(pushed)(T(X), T(V))
+    close(out, np.tanh(X @ W), 1e-5)
+    close(tan, (1.0 - np.tanh(X @ W) ** 2) * (V @ W), 1e-5)
