@@ -100,7 +100,27 @@ def full_inputs(a: dict) -> list[int]:
     return sorted({i[2] for i in a["ins"] if i[0] == isa.LDG})
 
 
-def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
+def stage16_operand(a: dict) -> int | None:
+    """The input whose row the LDS-staged generic form keeps: reduction programs over rows no
+    register-resident form can hold, with a 16-bit, unit-stride input that at least two
+    phases read.  (The row length a kernel meets at run time may differ from the one planned
+    here; the launch checks it again.)"""
+    if not a["has_reduce"] or a.get("n_stage", 0) or a["C"] % 4 or a["C"] * 2 > 64000:
+        return None
+    if (a["C"] + 3) // 4 <= 8 * 512:
+        return None
+    loads: dict[int, int] = {}
+    for i in a["ins"]:
+        if i[0] == isa.LDG:
+            loads[i[2]] = loads.get(i[2], 0) + 1
+    for k, n in sorted(loads.items()):
+        o = a["operands"][k]
+        if n >= 2 and o.dtype.abi in (1, 2) and o.vec_ok and o.col_stride == 1 and not o.is_output:
+            return k
+    return None
+
+
+def generate_kernel(a: dict, name: str, cpt: int = 0, stage16: int | None = None) -> str:
     """HIP source of one specialised kernel for the row program ``a``.
 
     ``cpt`` = 0: generic form, chunk loops with a run-time trip count, rows that
@@ -270,6 +290,8 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
             for k, o in enumerate(ops):
                 if o.stage_slot >= 0:
                     w(f"    rp_stage_row(o{k}, off{k}, rp_stage_lds + {o.stage_slot} * c_pad, C, n_chunks);")
+        if stage16 is not None:
+            w(f"    rp_stage_row16(o{stage16}, off{stage16}, (uint2*)rp_stage_lds, n_chunks);")
     if used_s:
         w("    float " + ", ".join(f"s{r} = 0.f" for r in used_s) + ";")
     w("    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;")
@@ -307,6 +329,8 @@ def generate_kernel(a: dict, name: str, cpt: int = 0) -> str:
                         w(ind + f"v{bd} = r{bx}[j];")
                     elif block_mode and o.stage_slot >= 0:
                         w(ind + f"v{bd} = *(const float4*)(rp_stage_lds + {o.stage_slot} * c_pad + col);")
+                    elif stage16 is not None and bx == stage16:
+                        w(ind + f"v{bd} = rp_staged16((const uint2*)rp_stage_lds, col, {o.dtype.abi});")
                     else:
                         w(ind + f"v{bd} = rp_load4(o{bx}, off{bx}, col, valid);")
                 elif bop == isa.STG:
@@ -482,6 +506,8 @@ def write_sources(programs: dict[int, dict]) -> list[Path]:
             src.append(generate_kernel(a, f"rp_spec_{h:016x}"))
             for c in resident_variants(a):
                 src.append(generate_kernel(a, f"rp_spec_{h:016x}_c{c}", cpt=c))
+            if stage16_operand(a) is not None:
+                src.append(generate_kernel(a, f"rp_spec_{h:016x}_s16", stage16=stage16_operand(a)))
             src.append("")
         src.append(f"extern const rp_spec_entry rp_spec_table_{fi}[] = {{")
         for h, a in chunk:
@@ -495,11 +521,12 @@ def write_sources(programs: dict[int, dict]) -> list[Path]:
                 kf.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, false>" if c in rv else "nullptr")
                 kst.append(f"(const void*)rp_spec_{h:016x}_c{c}<true, true>" if c in rv else "nullptr")
             kflat = f"(const void*)rp_spec_{h:016x}<true>" if flat else "nullptr"
+            k16 = f"(const void*)rp_spec_{h:016x}_s16" if stage16_operand(a) is not None else "nullptr"
             src.append(f"  {{0x{h:016x}ULL, {{{', '.join(ks)}}}, {{{', '.join(kf)}}}, "
-                       f"{{{', '.join(kst)}}}, {kflat}, {1 if a['has_reduce'] else 0}}},")
+                       f"{{{', '.join(kst)}}}, {kflat}, {k16}, {1 if a['has_reduce'] else 0}}},")
         src.append("  {0ULL, {nullptr, nullptr, nullptr, nullptr, nullptr}, "
                    "{nullptr, nullptr, nullptr, nullptr, nullptr}, "
-                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, nullptr, 0}};")
+                   "{nullptr, nullptr, nullptr, nullptr, nullptr}, nullptr, nullptr, 0}};")
         src.append(f"extern const int rp_spec_count_{fi} = {len(chunk)};")
         path = CSRC / f"rowprog_spec_gen{fi}.hip"
         path.write_text("\n".join(src) + "\n")

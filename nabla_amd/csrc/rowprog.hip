@@ -462,8 +462,10 @@ struct RpSpec {
   const void* kernel_full[5];
   const void* kernel_stream[5];
   const void* kernel_flat;
+  const void* kernel_stage16;
   int block_mode;
   bool lds_attr_set;
+  bool lds16_attr_set;
 };
 static std::mutex g_spec_mu;
 static std::unordered_map<uint64_t, RpSpec>* g_specs = nullptr;
@@ -486,8 +488,10 @@ static RpSpec* rp_find_spec(uint64_t h) {
           e.kernel_stream[k] = tabs[t][i].kernel_stream[k];
         }
         e.kernel_flat = tabs[t][i].kernel_flat;
+        e.kernel_stage16 = tabs[t][i].kernel_stage16;
         e.block_mode = tabs[t][i].block_mode;
         e.lds_attr_set = false;
+        e.lds16_attr_set = false;
         (*g_specs)[tabs[t][i].hash] = e;
       }
   }
@@ -602,6 +606,20 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
         int64_t g2 = (int64_t)nbk_num_cus() * per_cu;
         if (g2 > rows) g2 = rows;
         NBK_HIP(hipLaunchKernel(fn, dim3((unsigned)g2), dim3(block), args, 0, st));
+        return NBK_OK;
+      }
+      if (spec->kernel_stage16 && p->n_stage == 0 && (p->C & 3) == 0 && c_pad * 2 <= 64000) {
+        // a long 16-bit row that several phases read: one copy in LDS as stored, two
+        // workgroups per CU so that one row's traffic overlaps the other's arithmetic
+        if (!spec->lds16_attr_set) {
+          NBK_HIP(hipFuncSetAttribute(spec->kernel_stage16, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      64 * 1024));
+          spec->lds16_attr_set = true;
+        }
+        int64_t g2 = (int64_t)nbk_num_cus() * 2;
+        if (g2 > rows) g2 = rows;
+        NBK_HIP(hipLaunchKernel(spec->kernel_stage16, dim3((unsigned)g2), dim3(block), args,
+                                (size_t)c_pad * 2, st));
         return NBK_OK;
       }
       if (lds > 32 * 1024 && !spec->lds_attr_set) {

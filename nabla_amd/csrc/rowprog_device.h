@@ -398,6 +398,42 @@ __device__ __forceinline__ float rp_acc4(float acc, float4 a, int kind, int vali
   return acc;
 }
 
+// Copy one row of a 16-bit operand (unit column stride, C % 4 == 0) into LDS as it is stored.
+// A lane copies the 4-element chunks it reads back later (chunk index = lane + j * workgroup
+// size), so no barrier separates staging from use; eight loads are in flight per lane.
+__device__ __forceinline__ void rp_stage_row16(const nbk_operand& o, int64_t off, uint2* dst,
+                                               int64_t n_chunks) {
+  const uint16_t* base = (const uint16_t*)o.ptr + off;
+  const int64_t bd = blockDim.x;
+  int64_t ch = threadIdx.x;
+  if ((((uintptr_t)base) & 7) == 0) {
+    const uint2* src = (const uint2*)base;
+    for (; ch + 7 * bd < n_chunks; ch += 8 * bd) {
+      uint2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[ch + u * bd];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) dst[ch + u * bd] = v[u];
+    }
+    for (; ch < n_chunks; ch += bd) dst[ch] = src[ch];
+  } else {
+    for (; ch < n_chunks; ch += bd) {
+      const uint16_t* q = base + (ch << 2);
+      dst[ch] = make_uint2((uint32_t)q[0] | ((uint32_t)q[1] << 16), (uint32_t)q[2] | ((uint32_t)q[3] << 16));
+    }
+  }
+}
+// Four elements of a row staged by rp_stage_row16, as registers.
+__device__ __forceinline__ float4 rp_staged16(const uint2* stage, int64_t col, int dt) {
+  const uint2 u = stage[col >> 2];
+  if (dt == NBK_BF16)
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+  __half2 a = *(const __half2*)&u.x, b = *(const __half2*)&u.y;
+  const float2 fa = __half22float2(a), fb = __half22float2(b);
+  return make_float4(fa.x, fa.y, fb.x, fb.y);
+}
+
 // Copy one row of an operand into LDS as fp32.  Every lane stages exactly the
 // chunks it reads back later (chunk index = lane + j * workgroup size), so no
 // barrier separates staging from use.

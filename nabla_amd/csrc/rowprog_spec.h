@@ -20,6 +20,11 @@ struct rp_spec_entry {
   // programs without reductions: the generic form compiled for launches of a single row (a flat
   // array: no row arithmetic per chunk); nullptr for reduction programs.
   const void* kernel_flat;
+  // reduction programs over rows too long for a register-resident form, with a 16-bit input that
+  // several phases read: the generic form with that row copied into LDS once, as it is stored
+  // (2 bytes per element: a 32 000-element row and two workgroups fit a CU), and every phase
+  // reading it from there; nullptr where not generated.
+  const void* kernel_stage16;
   int block_mode;
 };
 
