@@ -79,7 +79,8 @@ def _shift(axis: int, bd: int) -> int:
 
 
 # ------------------------------------------------------------------------------ rules
-# rule(op, args, kwargs, bd, sizes) -> (plain args, physical kwargs)
+# rule(op, args, kwargs, bd, sizes) -> (plain args, physical kwargs[, post]); ``post`` turns the
+# op's plain results into plain tensors with the hidden dimensions in front
 def _rule_same_shape(op, args, kwargs, bd, sizes):
     """Elementwise ops whose operands already have one (logical) shape, reductions and other
     ops that name at most an ``axis``: lift everything, shift the axis."""
@@ -126,11 +127,77 @@ def _rule_layer_norm(op, args, kwargs, bd, sizes):
     return [lift(args[0], bd, sizes)] + list(args[1:]), dict(kwargs)
 
 
+def _fold(t: Tensor, bd: int) -> Tensor:
+    """The hidden dimensions and the first logical one as one dimension (ops whose kernels are
+    written for a fixed rank with a leading batch: images, attention heads)."""
+    from . import view
+    shape = tuple(t.shape)
+    n = 1
+    for d in shape[:bd + 1]:
+        n *= d
+    return view.reshape(t, (n,) + shape[bd + 1:])
+
+
+def _unfold(sizes: tuple[int, ...]):
+    def post(outs):
+        from . import view
+        return [view.reshape(o, tuple(sizes) + (o.shape[0] // _prod(sizes),) + tuple(o.shape[1:]))
+                for o in outs]
+    return post
+
+
+def _prod(dims) -> int:
+    n = 1
+    for d in dims:
+        n *= d
+    return n
+
+
+def _rule_fold_leading(op, args, kwargs, bd, sizes):
+    """Pooling windows and fused attention: every tensor argument has the element's leading batch
+    axis; the hidden dimensions join it."""
+    out = [_fold(lift(a, bd, sizes), bd) if isinstance(a, Tensor) else a for a in args]
+    return out, dict(kwargs), _unfold(sizes)
+
+
+def _rule_conv(op, args, kwargs, bd, sizes):
+    # the images carry the batch; one filter for all of them
+    if isinstance(args[1], BatchedTensor):
+        raise NoBatchRule("convolution with a mapped filter")
+    return [_fold(lift(args[0], bd, sizes), bd), args[1]], dict(kwargs), _unfold(sizes)
+
+
+def _rule_gather(op, args, kwargs, bd, sizes):
+    """Mapped indices into one table: the gathered axis is replaced by the indices' whole shape,
+    hidden dimensions included, which then move to the front."""
+    from . import view
+    x, idx = args
+    if isinstance(x, BatchedTensor):
+        raise NoBatchRule("gather from a mapped table")
+    rank = len(x.shape)
+    axis = int(kwargs.get("axis", 0))
+    axis = axis + rank if axis < 0 else axis
+
+    def post(outs):
+        o = outs[0]
+        order = list(range(axis, axis + bd)) + [i for i in range(len(o.shape)) if not axis <= i < axis + bd]
+        return [view.permute(o, order) if axis else o]
+
+    return [x, lift(idx, bd, sizes)], dict(kwargs, axis=axis), post
+
+
 def _rules() -> list[tuple[type, Callable]]:
-    from . import binary, comparison, control_flow, creation, normalization, reduction, unary, view
+    from . import (attention, binary, control_flow, convolution, normalization, pooling, unary, view,
+                   xent)
     from .base import BinaryOperation, ReduceOperation, UnaryOperation
 
     return [
+        (view.GatherOp, _rule_gather),
+        (convolution.Conv2DOp, _rule_conv),
+        (pooling.MaxPool2DOp, _rule_fold_leading),
+        (pooling.AvgPool2DOp, _rule_fold_leading),
+        (attention.FusedAttentionOp, _rule_fold_leading),
+        (xent.SoftmaxCrossEntropyOp, _rule_same_shape),
         (view.BroadcastToOp, _rule_broadcast_to),
         (view.ReshapeOp, _rule_reshape),
         (view.PermuteOp, _rule_permute),
@@ -175,8 +242,10 @@ def dispatch(op, args: list, kwargs: dict) -> list:
                 if sizes[i] not in (1, d):
                     raise ValueError(f"vmap: mapped axes of sizes {sizes[i]} and {d} meet in '{op.name}'")
                 sizes[i] = d
-    phys_args, phys_kwargs = rule(op, list(args), dict(kwargs or {}), bd, tuple(sizes))
-    outs = op(phys_args, phys_kwargs)
+    got = rule(op, list(args), dict(kwargs or {}), bd, tuple(sizes))
+    outs = op(got[0], got[1])
+    if len(got) > 2:
+        outs = got[2](outs)
     return [BatchedTensor(o, bd) for o in outs]
 
 

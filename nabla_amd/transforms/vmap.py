@@ -9,8 +9,9 @@ Two ways to run the mapped function, with the same results:
   gradients of a model are one forward and one backward pass over the batch.
 * **element by element**: the function is traced once per batch element on slices of the
   arguments and the results are stacked, all inside one lazy graph.  Used when the function
-  reaches an op that has no batching rule (gathers, convolutions, pooling, the fused attention
-  and cross-entropy ops, custom kernels) or when ``config.VMAP_BATCHED`` is off.
+  reaches an op that has no batching rule (scatters, gathers from a mapped table, convolutions
+  with a mapped filter, the backward ops when called directly, custom kernels, optimizer and
+  random ops) or when ``config.VMAP_BATCHED`` is off.
 
 Composition (``grad`` of ``vmap``, ``vmap`` of ``grad``, nesting) is the reference's either way.
 

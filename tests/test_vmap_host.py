@@ -190,24 +190,43 @@ def test_nested_batched_maps_and_vjp_inside(emulator):
 
 
 def test_ops_without_a_batching_rule_fall_back_to_the_map(emulator):
-    table, idx = RNG.standard_normal((7, 3)), np.array([[1, 2], [6, 0], [3, 3]])
+    """A gather from a table that is itself mapped has no batching rule: the function is tried
+    once, then mapped element by element, with the right result either way."""
+    tables, idx = RNG.standard_normal((3, 7, 2)), np.array([1, 6, 3, 3])
     calls = []
 
-    def look_up(i):
+    def look_up(tab):
         calls.append(1)
-        return nb.nn.functional.embedding(i, T(table)) * 2.0
+        return nb.gather(tab, nb.Tensor.constant(idx.astype(np.int64)), axis=0) * 2.0
 
-    got = nb.vmap(look_up)(nb.Tensor.constant(idx.astype(np.int64)))
+    got = nb.vmap(look_up)(T(tables))
     assert len(calls) == 1 + 3  # the batched attempt, then one call per element
-    close(got, 2.0 * table[idx])
+    close(got, 2.0 * tables[:, idx])
 
 
-def test_forward_mode_inside_a_batched_map(emulator):
-    X, V, W = RNG.standard_normal((5, 3)), RNG.standard_normal((5, 3)), RNG.standard_normal((3, 4))
-
-    def pushed(x, v):
-        return nb.jvp(lambda a: nb.tanh(a @ T(W)), (x,), (v,))
-
-    out, tan = nb.vmap(pushed)(T(X), T(V))
-    close(out, np.tanh(X @ W), 1e-5)
-    close(tan, (1.0 - np.tanh(X @ W) ** 2) * (V @ W), 1e-5)
+def test_window_index_and_fused_ops_join_the_hidden_axis(emulator):
+    """Convolution and pooling (one filter, mapped images), gathers from one table with mapped
+    indices, row-wise cross-entropy and the fused attention op run once on the batch: the hidden
+    axis joins the op's own leading axis (or, for a gather, moves out of the middle)."""
+    F = nb.nn.functional
+    img, filt = RNG.standard_normal((3, 2, 8, 8, 4)), RNG.standard_normal((3, 3, 4, 5))
+    table = RNG.standard_normal((7, 3))
+    idx = nb.Tensor.constant(np.array([[1, 2], [6, 0], [3, 3]], dtype=np.int64))
+    logits = RNG.standard_normal((3, 4, 9))
+    labels = nb.Tensor.constant(RNG.integers(0, 9, (3, 4)).astype(np.int64))
+    heads = nb.Tensor.constant(RNG.standard_normal((2, 1, 2, 128, 64)).astype(np.float32), dtype=nb.DType.bfloat16)
+    cases = [
+        (lambda x: nb.avg_pool2d(nb.max_pool2d(nb.relu(nb.conv2d(x, T(filt), padding=(1, 1, 1, 1))),
+                                               kernel_size=2), kernel_size=2), (T(img),)),
+        (lambda i: F.embedding(i, T(table)) * 2.0, (idx,)),
+        (lambda i: nb.gather(T(table.T), i, axis=1), (idx,)),
+        (lambda lg, lb: F.cross_entropy_loss(lg, lb), (T(logits), labels)),
+        (lambda a: nb.cast(F.scaled_dot_product_attention(a, a, a, is_causal=True), nb.DType.float32), (heads,)),
+    ]
+    for fn, args in cases:
+        got = _both_ways(fn, *args)
+        (batched, n_b), (mapped, n_m) = got[True], got[False]
+        assert n_b == 1 and n_m == args[0].shape[0]
+        for a, b in zip(batched, mapped):
+            assert a.shape == b.shape
+            np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
