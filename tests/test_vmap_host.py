@@ -230,3 +230,14 @@ def test_window_index_and_fused_ops_join_the_hidden_axis(emulator):
         for a, b in zip(batched, mapped):
             assert a.shape == b.shape
             np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_forward_mode_inside_a_batched_map(emulator):
+    X, V, W = RNG.standard_normal((5, 3)), RNG.standard_normal((5, 3)), RNG.standard_normal((3, 4))
+
+    def pushed(x, v):
+        return nb.jvp(lambda a: nb.tanh(a @ T(W)), (x,), (v,))
+
+    out, tan = nb.vmap(pushed)(T(X), T(V))
+    close(out, np.tanh(X @ W), 1e-5)
+    close(tan, (1.0 - np.tanh(X @ W) ** 2) * (V @ W), 1e-5)
