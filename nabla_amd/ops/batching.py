@@ -19,6 +19,7 @@ replays on the plain tensors of the recorded ops, which form a valid program of 
 """
 from __future__ import annotations
 
+from contextvars import ContextVar
 from typing import Any, Callable
 
 from ..core.tensor import BatchedTensor, Tensor
@@ -29,19 +30,24 @@ class NoBatchRule(Exception):
 
 
 # sizes of the hidden dimensions of the vmap calls that are being traced, outermost first
-_LEVELS: list[int] = []
+# (per context: two threads that trace at the same time do not see each other's levels)
+_LEVELS: ContextVar[tuple[int, ...]] = ContextVar("vmap_levels", default=())
 
 
 def current_level() -> int:
-    return len(_LEVELS)
+    return len(_LEVELS.get())
+
+
+def level_sizes() -> tuple[int, ...]:
+    return _LEVELS.get()
 
 
 def push_level(size: int) -> None:
-    _LEVELS.append(int(size))
+    _LEVELS.set(_LEVELS.get() + (int(size),))
 
 
 def pop_level() -> None:
-    _LEVELS.pop()
+    _LEVELS.set(_LEVELS.get()[:-1])
 
 
 def plain(t: Tensor) -> Tensor:
@@ -249,5 +255,5 @@ def dispatch(op, args: list, kwargs: dict) -> list:
     return [BatchedTensor(o, bd) for o in outs]
 
 
-__all__ = ["NoBatchRule", "dispatch", "lift", "plain", "batch_dims_of", "current_level",
+__all__ = ["NoBatchRule", "dispatch", "lift", "plain", "batch_dims_of", "current_level", "level_sizes",
            "push_level", "pop_level"]

@@ -21,7 +21,7 @@ def lift_to_vmap_level(args):
     level = batching.current_level()
     if not level:
         return args
-    sizes = tuple(batching._LEVELS)
+    sizes = batching.level_sizes()
 
     def up(t):
         if isinstance(t, Tensor) and batching.batch_dims_of(t) < level:
