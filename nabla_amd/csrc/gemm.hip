@@ -1692,7 +1692,9 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   };
   a.a_vec = vec_ok(d->A, akc ? d->a_rs : d->a_cs, d->a_bs, a.a_bs2);
   a.b_vec = vec_ok(d->B, bkc ? d->b_cs : d->b_rs, d->b_bs, a.b_bs2);
-  NBK_REQUIRE(d->colsum == nullptr || d->dtype_ab == NBK_BF16, "gemm: column sums need bf16 operands");
+  // (checked before any kernel is chosen: no path may take the product and drop the sums)
+  NBK_REQUIRE(d->colsum == nullptr || (d->dtype_ab == NBK_BF16 && !akc && !bkc),
+              "gemm: column sums need bf16 operands that are both row-contiguous (a_rs == b_cs == 1)");
   if (d->dtype_ab == NBK_BF16 && d->N <= 32 && d->M >= 1024 && d->K >= 256 && d->K % 64 == 0 &&
       akc && a.a_vec && d->batch == 1 && d->bias == nullptr && d->residual == nullptr &&
       d->act == NBK_ACT_NONE && (bkc ? (bool)a.b_vec : (d->b_cs == 1 && d->N % 8 == 0 && a.b_vec))) {
