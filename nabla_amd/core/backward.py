@@ -34,10 +34,7 @@ def _accumulate_cotangent(cot_map: dict, target: TensorImpl, cot: Tensor) -> Non
     from ..ops.binary import add
 
     existing = cot_map.get(target)
-    if existing is not None:
-        cot_map[target] = add(Tensor(impl=existing), cot)._impl
-    else:
-        cot_map[target] = cot._impl
+    cot_map[target] = add(existing, cot) if existing is not None else cot
 
 
 class BackwardEngine:
@@ -46,16 +43,22 @@ class BackwardEngine:
     def __init__(self, trace: Trace, cotangents: Any, create_graph: bool = False):
         self.trace = trace
         self.create_graph = create_graph
-        self.cotangent_map: dict[TensorImpl, TensorImpl] = {}
+        # value (by its impl) -> cotangent.  The cotangents are kept as the tensors they are: one
+        # that comes from inside ``vmap`` (a whole basis of directions pulled back over a trace
+        # made outside it) keeps its hidden dimensions through every VJP rule
+        self.cotangent_map: dict[TensorImpl, Tensor] = {}
         outs = [t for t in tree_leaves(trace.outputs) if isinstance(t, Tensor)]
         cots = [c for c in tree_leaves(cotangents) if isinstance(c, Tensor)]
         if len(outs) != len(cots):
             raise ValueError(f"backward: {len(outs)} outputs but {len(cots)} cotangents")
         for o, c in zip(outs, cots):
-            # (stored shapes: inside vmap both carry the hidden batch dimensions)
-            if tuple(o._impl.shape) != tuple(c._impl.shape):
+            if tuple(o._impl.shape) == tuple(c._impl.shape):
+                # the same storage shape (inside vmap: both with their hidden dimensions, and the
+                # replay below runs on the stored tensors as they are)
+                c = Tensor(impl=c._impl)
+            elif isinstance(o, BatchedTensor) or tuple(o.shape) != tuple(c.shape):
                 raise ValueError(f"cotangent shape {c.shape} does not match output shape {o.shape}")
-            _accumulate_cotangent(self.cotangent_map, o._impl, Tensor(impl=c._impl))
+            _accumulate_cotangent(self.cotangent_map, o._impl, c)
 
     def run(self) -> dict:
         for node in reversed(self.trace.nodes):
@@ -74,7 +77,7 @@ class BackwardEngine:
             if o is None:
                 cots.append(None)
             elif o in self.cotangent_map:
-                cots.append(Tensor(impl=self.cotangent_map[o]))
+                cots.append(self.cotangent_map[o])
             else:
                 from ..ops.creation import zeros_like
                 cots.append(zeros_like(Tensor(impl=o)))
@@ -110,9 +113,11 @@ class BackwardEngine:
             if not isinstance(inp, Tensor):
                 continue
             c = self.cotangent_map.get(inp._impl)
-            g = Tensor(impl=c) if c is not None else zeros_like(Tensor(impl=inp._impl))
+            g = c if c is not None else zeros_like(Tensor(impl=inp._impl))
             # the gradient of a tensor seen from inside vmap hides the same dimensions
-            grads[inp] = BatchedTensor(g, inp._bd) if isinstance(inp, BatchedTensor) else g
+            if isinstance(inp, BatchedTensor) and not isinstance(g, BatchedTensor):
+                g = BatchedTensor(g, inp._bd)
+            grads[inp] = g
         return grads
 
 
@@ -143,10 +148,9 @@ def backward(output: Tensor, gradient: Tensor | None = None, *, retain_graph: bo
         eng._process_node(node)
     new_grads = []
     for leaf in tr.gradient_leaves:
-        c = eng.cotangent_map.get(leaf)
-        if c is None:
+        g = eng.cotangent_map.get(leaf)
+        if g is None:
             continue
-        g = Tensor(impl=c)
         if leaf.cotangent is not None:
             g = add(Tensor(impl=leaf.cotangent), g)
         leaf.cotangent = g._impl

@@ -1,10 +1,14 @@
 """``jacrev`` and ``jacfwd`` (nabla/transforms/jacrev.py:27-115, jacfwd.py:32-119).
 
-Both walk the standard basis one direction at a time, as the reference does (jacrev.py:78-82
-calls the pullback once per output element, jacfwd.py:81-104 calls ``jvp`` once per input
-element), and stack the results.  Here the forward trace is captured once for ``jacrev``
-(one ``vjp``) and every pullback is a replay over it; all rows are realised together, so
-the backward programs of all directions land in one plan.
+The reference walks the standard basis one direction at a time (jacrev.py:78-82 calls the
+pullback once per output element, jacfwd.py:81-104 calls ``jvp`` once per input element) and
+stacks the results.  ``jacrev`` here sends the whole basis through at once: it captures the
+forward trace once (one ``vjp``) and maps its pullback over the identity with ``vmap``, so the
+backward pass runs once on cotangents with a hidden axis of one direction per output element.
+Where an op on the way has no batching rule ``vmap`` walks the directions one by one, which is the
+reference's loop, and so does ``jacrev`` when it is itself called inside a ``vmap``.  ``jacfwd``
+calls ``jvp`` once per input element as the reference does.  Either way all rows are realised
+together in one plan.
 
 The Jacobian of a function with one output tensor has shape ``(*out_shape, *in_shape)``;
 several differentiated arguments give a tuple of Jacobians.  Several output tensors raise
@@ -75,6 +79,14 @@ def _one_hot_like(t: Tensor, j: int | None) -> Tensor:
     return Tensor.constant(a.reshape(sh), dtype=t.dtype)
 
 
+def _identity_like(t: Tensor) -> Tensor:
+    """The standard basis of ``t``'s space as one tensor ``(numel, *t.shape)``: slice ``j`` is the
+    direction that selects element ``j`` (row-major)."""
+    sh = tuple(int(d) for d in t.shape)
+    n = max(int(np.prod(sh, dtype=np.int64)), 1)
+    return Tensor.constant(np.eye(n, dtype=np.float32).reshape((n,) + sh), dtype=t.dtype)
+
+
 def _basis(flat: list[Tensor]):
     """For every element of every tensor in ``flat``, the list of per-tensor directions that
     selects it."""
@@ -90,7 +102,9 @@ _MULTI_OUT = ("{} with multiple output tensors is not yet supported. "
 
 def jacrev(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
     """Jacobian by reverse mode: one pullback per output element."""
+    from ..ops import batching
     from ..ops.view import reshape, stack
+    from .vmap import vmap
 
     def jacrev_fn(*args: Any) -> Any:
         diff_args, partial_func = _partial(fn, argnums, args)
@@ -107,17 +121,24 @@ def jacrev(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
             raise NotImplementedError("jacrev: every differentiated argument must be one tensor")
         out_shape = tuple(int(d) for d in flat_out[0].shape)
 
-        rows: list[list[Tensor]] = [[] for _ in flat_in]
-        for direction in _basis(flat_out):
-            grads = pullback(pytree.tree_unflatten(out_td, direction))
-            g_flat, _ = _tensor_leaves(grads)
-            for k, g in enumerate(g_flat):
-                rows[k].append(g)
+        def pull(ct: Tensor):
+            grads = pullback(pytree.tree_unflatten(out_td, [ct]))
+            return tuple(_tensor_leaves(grads)[0])
 
+        if batching.current_level() == 0:
+            # the whole basis at once: cotangents with a hidden axis over a trace without one
+            stacked = vmap(pull)(_identity_like(flat_out[0]))  # each (n_out, *in_shape)
+        else:
+            # inside a vmap the trace has hidden axes of its own, which a recorded op no longer
+            # tells from the others: one replay per direction, as the reference does
+            rows: list[list[Tensor]] = [[] for _ in flat_in]
+            for direction in _basis(flat_out):
+                for k, g in enumerate(pull(direction[0])):
+                    rows[k].append(g)
+            stacked = [r[0] if len(r) == 1 and not out_shape else stack(r, axis=0) for r in rows]
         jacs = []
-        for r, x in zip(rows, flat_in):
+        for j, x in zip(stacked, flat_in):
             in_shape = tuple(int(d) for d in x.shape)
-            j = r[0] if len(r) == 1 else stack(r, axis=0)
             jacs.append(reshape(j, out_shape + in_shape))
         jac = jacs[0] if len(jacs) == 1 else tuple(jacs)
         return (jac, aux) if has_aux else jac

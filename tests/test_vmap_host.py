@@ -241,3 +241,28 @@ def test_forward_mode_inside_a_batched_map(emulator):
     out, tan = nb.vmap(pushed)(T(X), T(V))
     close(out, np.tanh(X @ W), 1e-5)
     close(tan, (1.0 - np.tanh(X @ W) ** 2) * (V @ W), 1e-5)
+
+
+def test_jacobian_by_one_batched_pullback(emulator):
+    """jacrev maps the pullback over the identity: the launches of a two-layer Jacobian do not
+    grow with the number of outputs, and the result is the chain rule in numpy."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    W1, W2, x = RNG.standard_normal((5, 16)), RNG.standard_normal((16, 12)), RNG.standard_normal((5,))
+    f = lambda v: nb.tanh(nb.tanh(v @ T(W1)) @ T(W2))
+    h = np.tanh(x @ W1)
+    y = np.tanh(h @ W2)
+    want = ((1 - y ** 2)[:, None] * W2.T) @ ((1 - h ** 2)[:, None] * W1.T)
+    steps = {}
+    for batched in (True, False):
+        with config.flag("VMAP_BATCHED", batched):
+            engine.clear_plan_cache()
+            J = nb.jacrev(f)(T(x))
+            close(J, want, 1e-4)
+            steps[batched] = sum(len(bp.plan.steps) for bp in engine._PLAN_CACHE.values())
+    engine.clear_plan_cache()
+    assert steps[True] * 3 < steps[False]
+    H = nb.jacrev(nb.grad(lambda v: nb.reduce_sum(nb.tanh(v @ T(W1)) ** 2.0)))(T(x))
+    t = np.tanh(x @ W1)
+    d2 = 2.0 * ((1 - t ** 2) ** 2 - 2.0 * t * t * (1 - t ** 2))
+    close(H, (W1 * d2) @ W1.T, 1e-4)
