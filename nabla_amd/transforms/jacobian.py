@@ -7,8 +7,8 @@ forward trace once (one ``vjp``) and maps its pullback over the identity with ``
 backward pass runs once on cotangents with a hidden axis of one direction per output element.
 Where an op on the way has no batching rule ``vmap`` walks the directions one by one, which is the
 reference's loop, and so does ``jacrev`` when it is itself called inside a ``vmap``.  ``jacfwd``
-calls ``jvp`` once per input element as the reference does.  Either way all rows are realised
-together in one plan.
+does the same with ``jvp``: the identity of an input as tangents with a hidden axis, one call per
+input tensor.  Either way all rows are realised together in one plan.
 
 The Jacobian of a function with one output tensor has shape ``(*out_shape, *in_shape)``;
 several differentiated arguments give a tuple of Jacobians.  Several output tensors raise
@@ -147,8 +147,12 @@ def jacrev(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
 
 
 def jacfwd(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
-    """Jacobian by forward mode: one ``jvp`` per input element."""
+    """Jacobian by forward mode: one ``jvp`` per input tensor over its whole basis (per input
+    element where ``vmap`` cannot batch the function, inside a ``vmap``, or with ``has_aux``)."""
+    from ..ops import batching
+    from ..ops.creation import zeros_like
     from ..ops.view import permute, reshape, stack
+    from .vmap import vmap
 
     def jacfwd_fn(*args: Any) -> Any:
         diff_args, partial_func = _partial(fn, argnums, args)
@@ -157,30 +161,47 @@ def jacfwd(fn: Callable, argnums=None, has_aux: bool = False) -> Callable:
             raise NotImplementedError("jacfwd: every differentiated argument must be one tensor")
         sizes = [_numel(t) for t in flat_in]
 
-        cols: list[Tensor] = []
         aux = None
         out_shape: tuple[int, ...] = ()
-        for direction in _basis(flat_in):
-            tangents = pytree.tree_unflatten(in_td, direction)
-            if not isinstance(tangents, tuple):
-                tangents = (tangents,)
-            if has_aux:
-                out, tan, aux = jvp(partial_func, tuple(diff_args), tangents, has_aux=True)
-            else:
-                out, tan = jvp(partial_func, tuple(diff_args), tangents)
-            t_flat, _ = _tensor_leaves(tan)
-            if len(t_flat) != 1:
-                raise NotImplementedError(_MULTI_OUT.format("jacfwd"))
-            out_shape = tuple(int(d) for d in t_flat[0].shape)
-            cols.append(t_flat[0])
+        per_input: list[Tensor] = []  # for every input: (numel(input), *out_shape)
+        if batching.current_level() == 0 and not has_aux:
+            # one jvp per input tensor, its whole basis at once as tangents with a hidden axis
+            for k, x in enumerate(flat_in):
+                def push(tang: Tensor, k=k):
+                    tangents = tuple(tang if i == k else zeros_like(t) for i, t in enumerate(flat_in))
+                    _, tan = jvp(partial_func, tuple(diff_args), tangents)
+                    t_flat, _ = _tensor_leaves(tan)
+                    if len(t_flat) != 1:
+                        raise NotImplementedError(_MULTI_OUT.format("jacfwd"))
+                    return t_flat[0]
+
+                col = vmap(push)(_identity_like(x))
+                out_shape = tuple(int(d) for d in col.shape[1:])
+                per_input.append(col)
+        else:
+            cols: list[Tensor] = []
+            for direction in _basis(flat_in):
+                tangents = pytree.tree_unflatten(in_td, direction)
+                if not isinstance(tangents, tuple):
+                    tangents = (tangents,)
+                if has_aux:
+                    out, tan, aux = jvp(partial_func, tuple(diff_args), tangents, has_aux=True)
+                else:
+                    out, tan = jvp(partial_func, tuple(diff_args), tangents)
+                t_flat, _ = _tensor_leaves(tan)
+                if len(t_flat) != 1:
+                    raise NotImplementedError(_MULTI_OUT.format("jacfwd"))
+                out_shape = tuple(int(d) for d in t_flat[0].shape)
+                cols.append(t_flat[0])
+            off = 0
+            for n in sizes:
+                chunk = cols[off:off + n]
+                off += n
+                per_input.append(stack(chunk, axis=0))
 
         jacs = []
-        off = 0
-        for x, n in zip(flat_in, sizes):
+        for x, j in zip(flat_in, per_input):
             in_shape = tuple(int(d) for d in x.shape)
-            chunk = cols[off:off + n]
-            off += n
-            j = chunk[0] if n == 1 else stack(chunk, axis=0)
             j = reshape(j, in_shape + out_shape)
             if in_shape and out_shape:
                 ni, no = len(in_shape), len(out_shape)

@@ -266,3 +266,36 @@ def test_jacobian_by_one_batched_pullback(emulator):
     t = np.tanh(x @ W1)
     d2 = 2.0 * ((1 - t ** 2) ** 2 - 2.0 * t * t * (1 - t ** 2))
     close(H, (W1 * d2) @ W1.T, 1e-4)
+
+
+def test_forward_mode_jacobian_and_hessian_by_one_batched_pass(emulator):
+    """jacfwd pushes the identity of its input through one jvp; forward over reverse gives the
+    Hessian in one pass as well.  Launches against the per-direction loop, values against numpy."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    W1, W2, x = RNG.standard_normal((5, 16)), RNG.standard_normal((16, 12)), RNG.standard_normal((5,))
+    f = lambda v: nb.tanh(nb.tanh(v @ T(W1)) @ T(W2))
+    h = np.tanh(x @ W1)
+    y = np.tanh(h @ W2)
+    want = ((1 - y ** 2)[:, None] * W2.T) @ ((1 - h ** 2)[:, None] * W1.T)
+    steps = {}
+    for batched in (True, False):
+        with config.flag("VMAP_BATCHED", batched):
+            engine.clear_plan_cache()
+            close(nb.jacfwd(f)(T(x)), want, 1e-4)
+            steps[batched] = sum(len(bp.plan.steps) for bp in engine._PLAN_CACHE.values())
+    engine.clear_plan_cache()
+    assert steps[True] * 3 < steps[False]
+    H = nb.jacfwd(nb.grad(lambda v: nb.reduce_sum(nb.tanh(v @ T(W1)) ** 2.0)))(T(x))
+    t = np.tanh(x @ W1)
+    d2 = 2.0 * ((1 - t ** 2) ** 2 - 2.0 * t * t * (1 - t ** 2))
+    close(H, (W1 * d2) @ W1.T, 1e-4)
+    # two differentiated arguments: one Jacobian each
+    A, B = RNG.standard_normal((3, 4)), RNG.standard_normal((4,))
+    ja, jb = nb.jacfwd(lambda a, b: nb.tanh(a @ b), argnums=(0, 1))(T(A), T(B))
+    s = 1 - np.tanh(A @ B) ** 2
+    want_a = np.zeros((3, 3, 4))
+    for i in range(3):
+        want_a[i, i] = s[i] * B
+    close(ja, want_a, 1e-4)
+    close(jb, s[:, None] * A, 1e-4)
