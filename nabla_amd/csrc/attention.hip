@@ -345,35 +345,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
 }
 
 // ------------------------------------------------------------------------------ backward
-// delta[b, h, q] = sum_d dO[q, d] * O[q, d]: one lane per (row, 8-wide slice), reduced
-// over the HD / 8 lanes of a row.
-template <int HD>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs g) {
-  constexpr int LPR = HD / 8;  // lanes per row
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = idx / LPR;
-  const int c = (int)(idx % LPR);
-  const int64_t rows = (int64_t)g.B * g.H * g.S;
-  float s = 0.f;
-  if (row < rows) {
-    const int q = (int)(row % g.S);
-    const int64_t bh = row / g.S;
-    const int hh = (int)(bh % g.H), b = (int)(bh / g.H);
-    const uint16_t* o = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)q * g.o.ss + c * 8;
-    const uint16_t* d = g.dout.p + (int64_t)b * g.dout.sb + (int64_t)hh * g.dout.sh +
-                        (int64_t)q * g.dout.ss + c * 8;
-    const at_u32x4 uo = *(const at_u32x4*)o, ud = *(const at_u32x4*)d;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      s += __uint_as_float(uo[e] << 16) * __uint_as_float(ud[e] << 16);
-      s += __uint_as_float(uo[e] & 0xffff0000u) * __uint_as_float(ud[e] & 0xffff0000u);
-    }
-  }
-#pragma unroll
-  for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-  if (row < rows && c == 0) g.delta[row] = s;
-}
-
 // dK, dV.  Grid: (B * H, S / 128).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
 // and walks the query tiles that can see them.
 //   S[q, key]  = Q K^T          (A: Q tile rows, B: the wave's K fragments)
@@ -757,16 +728,28 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_tr_kernel(const AttnArgs g)
   const float my_lse = g.lse[((int64_t)b * g.H + hh) * g.S + my_q] * AT_LOG2E;
   const int wq0 = q0 + wave * 32;  // first query of the wave
   const float c = g.scale * AT_LOG2E;
-  const float my_delta = g.delta[((int64_t)b * g.H + hh) * g.S + my_q];
 
+  // delta[q] = sum_d dO[q, d] O[q, d] comes out of the dO fragments this kernel loads anyway and
+  // the matching pieces of O (a lane pair holds one row); it is left in g.delta for the dK / dV
+  // kernel, which runs after this one.
+  const uint16_t* O = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh;
   at_bf16x8 qf[KSTEPS], dof[KSTEPS];
+  float my_delta = 0.f;
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
     const at_u32x4 uq = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
     const at_u32x4 ud = *(const at_u32x4*)(DO + (int64_t)my_q * g.dout.ss + s * 16 + h * 8);
+    const at_u32x4 uo = *(const at_u32x4*)(O + (int64_t)my_q * g.o.ss + s * 16 + h * 8);
     qf[s] = __builtin_bit_cast(at_bf16x8, uq);
     dof[s] = __builtin_bit_cast(at_bf16x8, ud);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      my_delta += __uint_as_float(uo[e] << 16) * __uint_as_float(ud[e] << 16);
+      my_delta += __uint_as_float(uo[e] & 0xffff0000u) * __uint_as_float(ud[e] & 0xffff0000u);
+    }
   }
+  my_delta += at_xhalf(my_delta);
+  if (h == 0) g.delta[((int64_t)b * g.H + hh) * g.S + my_q] = my_delta;
   at_f32x16 dq_acc[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d) dq_acc[d] = (at_f32x16)(0.f);
@@ -950,24 +933,22 @@ extern "C" int64_t nbk_attention_bwd_workspace(const nbk_attn_desc* d) {
 static int attn_bwd_launch(const nbk_attn_desc* d, AttnArgs& a, float* delta, hipStream_t st) {
   int rc;
   a.delta = delta;
-  const int64_t rows = d->B * d->H * d->S;
   const dim3 grid((unsigned)(d->B * d->H), (unsigned)(d->S / 128));
   if (d->hd == 64) {
     // (the eight-wave dK / dV form was measured on this head size too: 70 against 68 us on the
     // transformer block's shape, so 64-wide heads keep the four-wave kernel, which fits twice on a CU)
-    hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)((rows * 8 + 255) / 256)), dim3(256), 0, st, a);
+    // (the dQ kernel first: it leaves delta, the row sums of dO * O, for the dK / dV kernel)
     const size_t lds_kv = 2 * (2 * 64 * 64 * 2 + 2 * 64 * AT_TP * 2 + 2 * 64 * 4);
     const size_t lds_qtr = 2 * (2 * 64 * 64 * 2);
     if ((rc = attn_set_lds(attn_bwd_kv_kernel<64>, lds_kv))) return rc;
-    hipLaunchKernelGGL(attn_bwd_kv_kernel<64>, grid, dim3(256), lds_kv, st, a);
     hipLaunchKernelGGL(attn_bwd_q_tr_kernel<64>, grid, dim3(256), lds_qtr, st, a);
+    hipLaunchKernelGGL(attn_bwd_kv_kernel<64>, grid, dim3(256), lds_kv, st, a);
   } else {
-    hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st, a);
     const size_t lds_kv8 = 2 * (128 * 128 * 2) + 2 * (2 * 64 * 128 * 2 + 2 * 64 * 4);
     const size_t lds_qtr = 2 * (2 * 64 * 128 * 2);
     if ((rc = attn_set_lds(attn_bwd_kv8_kernel<128>, lds_kv8))) return rc;
-    hipLaunchKernelGGL(attn_bwd_kv8_kernel<128>, grid, dim3(512), lds_kv8, st, a);
     hipLaunchKernelGGL(attn_bwd_q_tr_kernel<128>, grid, dim3(256), lds_qtr, st, a);
+    hipLaunchKernelGGL(attn_bwd_kv8_kernel<128>, grid, dim3(512), lds_kv8, st, a);
   }
   return nbk_check_launch("attn_bwd kernels");
 }
