@@ -1033,7 +1033,7 @@ extern "C" int nbk_attention_bwd_static(const nbk_attn_desc* d, const nbk_attn_t
               (long long)rows, NBK_ATTN_STATIC_ROWS);
   float* delta = nullptr;
   if ((rc = attn_scratch_for_current_device(&delta))) return rc;
-  // every row of the scratch that the kernels read is written first by the row-sum kernel of
+  // every row of the scratch that the dK / dV kernel reads is written first by the dQ kernel of
   // this call, so nothing has to be cleared between calls
   return attn_bwd_launch(d, a, delta, (hipStream_t)stream);
 }

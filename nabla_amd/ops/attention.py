@@ -4,7 +4,7 @@ The reference builds attention from primitive ops -- matmul, mul by the scale, a
 ``where`` against a ``tril`` mask, softmax, matmul (nabla/nn/functional/layers.py:106-153)
 -- and differentiates it through the VJP rules of those ops, which stores the S x S
 scores and probabilities several times over.  Here the same function is one op with one
-kernel forward and three backward; the probabilities are recomputed from the per-row
+kernel forward and two backward; the probabilities are recomputed from the per-row
 log-sum-exp the forward keeps.
 
 ``FusedAttentionOp`` takes heads-first tensors ``[B, H, S, hd]`` (what
