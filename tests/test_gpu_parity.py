@@ -107,6 +107,52 @@ def test_specialised_kernels_match_interpreter(hip):
     np.testing.assert_allclose(gx_s.numpy(), gx_i.numpy(), rtol=2e-6, atol=1e-30)
 
 
+@pytest.mark.parametrize("rows,vocab", [(96, 32000), (700, 24000), (40, 20004)])
+def test_cross_entropy_over_long_rows_staged_in_lds(hip, rows, vocab):
+    """Cross-entropy and its gradient over bf16 rows too long for a register-resident kernel: the
+    specialised kernel that keeps the row in LDS (row lengths other than the benchmark's too; a
+    length that is no multiple of 4 takes the form that re-reads the row) against the interpreter
+    and against float64."""
+    from nabla_amd.backend import lib
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(77)
+    logits = (rng.standard_normal((rows, vocab)) * 3.0).astype(np.float32)
+    labels = rng.integers(0, vocab, (rows,)).astype(np.int64)
+    F = nb.nn.functional
+
+    def run():
+        x = T(logits, dtype=nb.DType.bfloat16)
+        lab = nb.Tensor.constant(labels)
+        loss, g = nb.value_and_grad(lambda z: F.cross_entropy_loss(z, lab))(x)
+        nb.realize_all(loss, g)
+        return loss.item(), nb.cast(g, nb.DType.float32).numpy()
+
+    engine.clear_plan_cache()
+    loss_s, g_s = run()
+    L = lib.load()
+    n_spec = sum(int(L.nbk_rowprog_is_specialized(C.byref(call[3])))
+                 for bound in engine._PLAN_CACHE.values() for call in bound.calls
+                 if call[0] is L.nbk_rowprog_launch)
+    assert n_spec >= 1, "the loss program of the decoder step must hit its specialised kernel"
+    engine.clear_plan_cache()
+    hip.force_interpreter = True
+    try:
+        loss_i, g_i = run()
+    finally:
+        hip.force_interpreter = False
+        engine.clear_plan_cache()
+    assert abs(loss_s - loss_i) <= 1e-5 * abs(loss_i)
+    np.testing.assert_allclose(g_s, g_i, rtol=2e-2, atol=1e-8)
+    x64 = torch.tensor(logits).to(torch.bfloat16).double().numpy()
+    m = x64.max(1, keepdims=True)
+    lse = m[:, 0] + np.log(np.exp(x64 - m).sum(1))
+    want_loss = float((lse - x64[np.arange(rows), labels]).mean())
+    p = np.exp(x64 - lse[:, None])
+    p[np.arange(rows), labels] -= 1.0
+    assert abs(loss_s - want_loss) <= 2.0 ** -8 * abs(want_loss)  # (the loss comes back in bf16)
+    assert relerr(g_s, p / rows) <= BF16_TOL
+
+
 # ---- C3 ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape,heads", [((2, 16, 32, 64), 4), ((2, 128, 256, 512), 4), ((1, 72, 64, 96), 2)])
 def test_c3_block_fp32(hip, shape, heads):
