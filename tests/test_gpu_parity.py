@@ -284,6 +284,72 @@ def test_argmax_ties_and_nan(hip):
     assert got.dtype == np.int64
 
 
+def test_argmin_ties_nan_and_axes(hip):
+    """argmin (nabla/ops/reduction.py:739-811, 880-896): int64, the first minimum on ties, a NaN
+    counts as the minimum (numpy / torch convention), along the last, a middle and the leading
+    axis, with and without keepdims, flattened for axis=None, f32 and bf16 -- exact."""
+    a = np.ones((7, 300), np.float32)
+    a[0, [5, 9, 250]] = -3.0          # first minimum wins
+    a[1, :] = 2.0                     # all equal -> 0
+    a[2, 299] = -1.0                  # last column
+    a[3, 17] = -np.inf
+    a[4, [100, 200]] = [-2.0, np.nan]  # NaN counts as the minimum
+    a[5, 0] = np.inf
+    a[6, [64, 128]] = [np.nan, np.nan]  # two NaNs in different lanes' strides: the first one
+    want = torch.from_numpy(a).argmin(-1).numpy()
+    np.testing.assert_array_equal(want, np.argmin(a, -1))
+    got = nb.argmin(T(a), axis=-1).numpy()
+    assert got.dtype == np.int64
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(nb.argmin(T(a), axis=0).numpy(), np.argmin(a, 0))
+    np.testing.assert_array_equal(nb.argmin(T(a), axis=-1, keepdims=True).numpy(), want[:, None])
+    rng = np.random.default_rng(21)
+    b = rng.standard_normal((5, 33, 70)).astype(np.float32)
+    for axis in (0, 1, 2, -2):
+        np.testing.assert_array_equal(nb.argmin(T(b), axis=axis).numpy(), np.argmin(b, axis))
+        np.testing.assert_array_equal(nb.argmax(T(b), axis=axis).numpy(), np.argmax(b, axis))
+    np.testing.assert_array_equal(nb.argmin(T(b), axis=None).numpy(), np.argmin(b))
+    # bf16 rounds many entries onto one value: ties resolve to the lowest index there too
+    bb = torch.from_numpy(b).to(torch.bfloat16)
+    got16 = nb.argmin(T(b).cast(nb.DType.bfloat16), axis=-1).numpy()
+    np.testing.assert_array_equal(got16, bb.float().argmin(-1).numpy())
+    # argmin(x) is argmax(-x) wherever no NaN is involved
+    np.testing.assert_array_equal(nb.argmin(T(b), axis=1).numpy(), nb.argmax(-T(b), axis=1).numpy())
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", F32_TOL), ("bf16", BF16_TOL)])
+def test_sigmoid_value_and_gradient(hip, dtype, tol):
+    """sigmoid (nabla/ops/unary.py SigmoidOp; derivative out * (1 - out)) against float64:
+    values over the range where fp32 saturates either way, and the gradient under a random
+    cotangent; sigmoid(x) + sigmoid(-x) = 1 as the invariant."""
+    rng = np.random.default_rng(22)
+    x = np.concatenate([rng.standard_normal(4000) * 3.0, np.linspace(-100.0, 100.0, 96)]).astype(np.float32)
+    x = x.reshape(64, 64)
+    w = rng.standard_normal(x.shape).astype(np.float32)
+    dt = nb.DType.bfloat16 if dtype == "bf16" else nb.DType.float32
+    if dtype == "bf16":
+        x = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+        w = torch.from_numpy(w).to(torch.bfloat16).float().numpy()
+    X, W = T(x).cast(dt), T(w).cast(dt)
+    y = nb.sigmoid(X)
+    g = nb.grad(lambda t: nb.reduce_sum(nb.sigmoid(t) * W))(X)
+    s = nb.sigmoid(X) + nb.sigmoid(-X)
+    nb.realize_all(y, g, s)
+    x64 = x.astype(np.float64)
+    want = np.where(x64 >= 0, 1.0 / (1.0 + np.exp(-np.abs(x64))), np.exp(-np.abs(x64)) / (1.0 + np.exp(-np.abs(x64))))
+    tx = torch.tensor(x64, requires_grad=True)
+    (torch.sigmoid(tx) * torch.tensor(w, dtype=torch.float64)).sum().backward()
+    yn = y.cast(nb.DType.float32).numpy().astype(np.float64)
+    gn = g.cast(nb.DType.float32).numpy().astype(np.float64)
+    assert np.isfinite(yn).all() and np.isfinite(gn).all()
+    assert relerr(yn, want) < tol
+    assert relerr(gn, tx.grad.numpy()) < tol
+    assert np.abs(s.cast(nb.DType.float32).numpy() - 1.0).max() < (2e-2 if dtype == "bf16" else 1e-6)
+    if dtype == "f32":
+        # elementwise, not only against the tensor's largest entry
+        assert (np.abs(yn - want) <= 1e-6 * want + 1e-37).all()
+
+
 def test_gather_rows_and_out_of_range(hip):
     rng = np.random.default_rng(7)
     table = rng.standard_normal((50, 24)).astype(np.float32)

@@ -572,6 +572,87 @@ def test_slice_tensor_window_and_zero_padded_vjp():
     assert g2[0, 0, 0] == 1.0 and g2[1, 0, 0] == 2.0 and g2[2, 0, 0] == 1.0 and g2[3, 0, 0] == 0.0
 
 
+def test_broadcast_to_values_and_summed_vjp():
+    """broadcast_to: numpy's right-aligned rule on odd shapes (new leading axes and size-1
+    axes stretched at once), and the VJP sums the cotangent over every axis that was added or
+    stretched (view/shape.py:131-152) -- torch's `expand` is the independent check; summing
+    over the wrong axes, or forgetting keepdims on a stretched axis, fails it."""
+    x = RNG.standard_normal((3, 1, 5))
+    shape = (2, 7, 3, 4, 5)
+    v = O.V(x)
+    out = O.broadcast_to(v, shape)
+    assert out.a.shape == shape
+    for a in range(2):
+        for b in range(7):
+            for j in range(4):
+                assert np.array_equal(out.a[a, b, :, j, :], x[:, 0, :])
+    w = RNG.standard_normal(shape)
+    (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+    t = _t(x)
+    (t.expand(*shape) * torch.tensor(w)).sum().backward()
+    _close(g, t.grad.numpy())
+    _close(g, w.sum(axis=(0, 1, 3)).reshape(3, 1, 5))
+    # a 0-d value goes everywhere and collects everything
+    s = O.V(np.array(1.5))
+    o0 = O.broadcast_to(s, (3, 2))
+    assert o0.a.shape == (3, 2) and (o0.a == 1.5).all()
+    w0 = RNG.standard_normal((3, 2))
+    (g0,) = O.grad_of(O.reduce_sum(o0 * w0), [s])
+    assert g0.shape == () and abs(g0 - w0.sum()) < 1e-12
+
+
+def test_pad_values_and_sliced_vjp():
+    """pad: (before, after) per axis with a constant fill (view/shape.py:1313-1398), checked
+    element by element and against torch's F.pad (whose argument order is last axis first);
+    the VJP is the window of the cotangent that starts at `before` and has the input's size
+    (1385-1390) -- unequal before/after widths, so that swapping them fails."""
+    x = RNG.standard_normal((2, 3, 4))
+    paddings = [(1, 0), (0, 2), (3, 1)]
+    v = O.V(x)
+    out = O.pad(v, paddings, value=-2.5)
+    assert out.a.shape == (3, 5, 8)
+    for i in range(3):
+        for j in range(5):
+            for k in range(8):
+                inside = 1 <= i < 3 and j < 3 and 3 <= k < 7
+                assert out.a[i, j, k] == (x[i - 1, j, k - 3] if inside else -2.5)
+    t = _t(x)
+    tp = TF.pad(t, (3, 1, 0, 2, 1, 0), value=-2.5)
+    assert np.array_equal(out.a, tp.detach().numpy())
+    w = RNG.standard_normal(out.a.shape)
+    (g,) = O.grad_of(O.reduce_sum(out * w), [v])
+    (tp * torch.tensor(w)).sum().backward()
+    _close(g, t.grad.numpy())
+    assert np.array_equal(g, w[1:3, 0:3, 3:7])
+    # default fill is zero
+    assert O.pad(v, [(0, 1), (0, 0), (0, 0)]).a[2].max() == 0.0
+
+
+def test_concatenate_values_and_split_vjp():
+    """concatenate: pieces of unequal length along a middle axis, in order (view/shape.py:821-980);
+    the VJP hands each input its own slab of the cotangent -- checked against torch.cat and
+    explicit slices, with three different lengths so that a wrong offset fails."""
+    parts = [RNG.standard_normal((2, n, 3)) for n in (1, 4, 2)]
+    vs = [O.V(p) for p in parts]
+    out = O.concatenate(vs, axis=1)
+    assert out.a.shape == (2, 7, 3)
+    assert np.array_equal(out.a[:, 0:1], parts[0]) and np.array_equal(out.a[:, 1:5], parts[1]) \
+        and np.array_equal(out.a[:, 5:7], parts[2])
+    w = RNG.standard_normal(out.a.shape)
+    gs = O.grad_of(O.reduce_sum(out * w), vs)
+    ts = [_t(p) for p in parts]
+    (torch.cat(ts, dim=1) * torch.tensor(w)).sum().backward()
+    for g, t in zip(gs, ts):
+        _close(g, t.grad.numpy())
+    assert np.array_equal(gs[0], w[:, 0:1]) and np.array_equal(gs[1], w[:, 1:5]) and np.array_equal(gs[2], w[:, 5:7])
+    # negative axis, and one tensor used twice accumulates both slabs
+    o2 = O.concatenate([vs[0], vs[0]], axis=-1)
+    assert o2.a.shape == (2, 1, 6)
+    w2 = RNG.standard_normal(o2.a.shape)
+    (g2,) = O.grad_of(O.reduce_sum(o2 * w2), [vs[0]])
+    _close(g2, w2[..., :3] + w2[..., 3:])
+
+
 def test_torch_steps_agree_with_the_numpy_oracle():
     """oracle/torch_steps.py (the full-size checker of the transformer and decoder steps) against
     oracle/configs.py in float64: loss and every gradient, non-trivial biases, norm weights and
