@@ -52,6 +52,21 @@ class FusionLimit(Exception):
 
 
 # --------------------------------------------------------------------------- data
+def _as_stored(value: float, dtype: DType) -> float:
+    """``value`` after one rounding to ``dtype`` (what a kernel reading the stored constant sees)."""
+    import numpy as np
+    if dtype is DType.bfloat16:
+        bits = np.array([value], np.float32).view(np.uint32)
+        if np.isfinite(value):
+            bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & np.uint32(0xFFFF0000)
+        return float(bits.astype(np.uint32).view(np.float32)[0])
+    if dtype is DType.float16:
+        return float(np.float16(value))
+    if dtype is DType.float32:
+        return float(np.float32(value))
+    return value
+
+
 def _numel(shape) -> int:
     n = 1
     for d in shape:
@@ -757,7 +772,10 @@ class Planner:
                 return float(x)
             while x.node.kind in ("broadcast", "reshape"):
                 x = x.node.inputs[0]
-            return float(x.node.attrs["value"]) if x.node.kind == "fill" else None
+            if x.node.kind != "fill":
+                return None
+            # the unfused multiply would read the constant as stored: round it the same way
+            return _as_stored(float(x.node.attrs["value"]), x.dtype)
 
         for n in nodes:
             if not (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2 and
@@ -816,7 +834,10 @@ class Planner:
                 return float(x)
             while x.node.kind in ("broadcast", "reshape"):
                 x = x.node.inputs[0]
-            return float(x.node.attrs["value"]) if x.node.kind == "fill" else None
+            if x.node.kind != "fill":
+                return None
+            # the unfused multiply would read the constant as stored: round it the same way
+            return _as_stored(float(x.node.attrs["value"]), x.dtype)
 
         for n in nodes:
             if not (n.kind == "ew" and n.fn == "mul" and len(n.attrs["operands"]) == 2):
@@ -1399,11 +1420,13 @@ class Planner:
                 users[0].kind == "reduce" and users[0].fn == "sum" and users[0].attrs["axis"] == 0 and
                 users[0].pos not in self.skip_nodes and self._unit(users[0].pos) is not None and
                 not self._unit(users[0].pos).fused and
+                not (set(epi) - {"alpha"}) and  # a scale commutes with the sum; a bias, a residual
+                                                # or an activation per batch element does not
                 len(pa[0]) == 1 and len(pb[0]) == 1 and
                 pa[0][0] == (batch, K * pa[2]) and pb[0][0] == (batch, K * pb[1])):
             red = users[0]
             self.skip_nodes.add(red.pos)
-            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K * batch, red.outputs[0])
+            self._emit_plain_gemm(ra, rb, pa, pb, M, N, K * batch, red.outputs[0], epi)
             return
         # (a second result or a residual is laid out like the product: both plain row-major then)
         c_strides = self._matmul_out_layout(out) if not ("aux_value" in epi or "residual" in epi) \

@@ -170,7 +170,10 @@ def _rule_conv(op, args, kwargs, bd, sizes):
     # the images carry the batch; one filter for all of them
     if isinstance(args[1], BatchedTensor):
         raise NoBatchRule("convolution with a mapped filter")
-    return [_fold(lift(args[0], bd, sizes), bd), args[1]], dict(kwargs), _unfold(sizes)
+    # a bias (third operand) is one vector per output channel for every image
+    if any(isinstance(a, BatchedTensor) for a in args[2:]):
+        raise NoBatchRule("convolution with a mapped bias")
+    return [_fold(lift(args[0], bd, sizes), bd), args[1]] + list(args[2:]), dict(kwargs), _unfold(sizes)
 
 
 def _rule_gather(op, args, kwargs, bd, sizes):

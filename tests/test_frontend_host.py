@@ -766,6 +766,45 @@ def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
     np.testing.assert_allclose(grads["A"].numpy(), 3.0 * x2.T @ (np.ones((120, 16), np.float32) @ b.T), rtol=1e-4, atol=1e-4)
 
 
+def test_a_batch_summed_product_keeps_what_was_folded_onto_it(emulator):
+    """sum_b A[b] @ B[b] becomes one product over (b, k).  A scale folded onto the batched product
+    commutes with the sum and rides along as alpha; a bias or a residual added per batch element
+    does not, so those products stay batched and are summed afterwards.  Values against numpy."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(31)
+    xt = rng.standard_normal((3, 8, 16)).astype(np.float32)   # the weight-gradient form x^T @ dy
+    a = np.ascontiguousarray(np.swapaxes(xt, 1, 2))
+    b = rng.standard_normal((3, 8, 5)).astype(np.float32)
+    bias = rng.standard_normal((1, 5)).astype(np.float32)
+    res = rng.standard_normal((3, 16, 8)).astype(np.float32)
+    w2 = rng.standard_normal((8, 5)).astype(np.float32)
+    prod = np.einsum("bik,bkn->bin", a, b)
+    A = lambda: nb.swap_axes(T(xt), 1, 2)
+    engine.clear_plan_cache()
+    got = nb.reduce_sum((A() @ T(b)) * nb.full((), 0.5), axis=0)
+    got.realize()
+    steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+    assert [s.kind for s in steps] == ["gemm"] and steps[0].attrs["alpha"] == 0.5, [s.kind for s in steps]
+    np.testing.assert_allclose(got.numpy(), 0.5 * prod.sum(0), rtol=1e-5, atol=1e-5)
+    engine.clear_plan_cache()
+    got = nb.reduce_sum(A() @ T(b) + T(bias), axis=0)
+    np.testing.assert_allclose(got.numpy(), (prod + bias).sum(0), rtol=1e-5, atol=1e-5)
+    for flag in ("FOLD_RESIDUAL", "FOLD_THIN_RESIDUAL"):
+        with config.flag(flag, True):
+            engine.clear_plan_cache()
+            got = nb.reduce_sum((T(res) @ T(w2)) + A() @ T(b), axis=0)
+            np.testing.assert_allclose(got.numpy(), (res @ w2 + prod).sum(0), rtol=1e-5, atol=1e-5)
+    engine.clear_plan_cache()
+    # a bf16 constant is folded as stored: bf16(0.3), not 0.3
+    x16 = nb.Tensor.constant(a[0], dtype=nb.DType.bfloat16)
+    w16 = nb.Tensor.constant(b[0], dtype=nb.DType.bfloat16)
+    (x16 @ w16 * nb.full((), 0.3, dtype=nb.DType.bfloat16)).realize()
+    alphas = [s.attrs.get("alpha") for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps if s.kind == "gemm"]
+    engine.clear_plan_cache()
+    assert alphas == [0.30078125], alphas
+
+
 def test_gelu_backward_recomputes_the_derivative_where_the_cotangent_is(emulator):
     """Two ways to get gelu's derivative to the backward pass -- recomputed from the pre-activation
     where the cotangent is (the default), or stored by the forward kernel -- agree with the

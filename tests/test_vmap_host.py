@@ -232,6 +232,31 @@ def test_window_index_and_fused_ops_join_the_hidden_axis(emulator):
             np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
 
 
+def test_convolution_with_a_bias_under_vmap(emulator):
+    """conv2d(x, k, bias=b) mapped over images: the bias is the third operand of the op and has
+    to survive the batching rule -- values against numpy's own sum (the no-bias result plus b),
+    batched and element by element; a mapped bias has no rule and falls back to the element map,
+    with the same values."""
+    img, filt = RNG.standard_normal((3, 2, 6, 6, 4)), RNG.standard_normal((3, 3, 4, 5))
+    bias = RNG.standard_normal((5,)) + 2.0
+    f_nb = lambda x: nb.conv2d(x, T(filt), padding=(1, 1, 1, 1))
+    f_b = lambda x: nb.conv2d(x, T(filt), padding=(1, 1, 1, 1), bias=T(bias))
+    plain = _both_ways(f_nb, T(img))[True][0][0]
+    got = _both_ways(f_b, T(img))
+    (batched, n_b), (mapped, n_m) = got[True], got[False]
+    assert n_b == 1 and n_m == 3
+    np.testing.assert_allclose(batched[0], plain + bias, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(mapped[0], plain + bias, rtol=1e-5, atol=1e-5)
+    # gradient with respect to the images through the biased convolution, per element
+    g = _both_ways(nb.grad(lambda x: nb.reduce_sum(nb.relu(f_b(x)))), T(img))
+    np.testing.assert_allclose(g[True][0][0], g[False][0][0], rtol=1e-5, atol=1e-5)
+    # one bias per element of the batch
+    biases = RNG.standard_normal((3, 5))
+    got = _both_ways(lambda x, b: nb.conv2d(x, T(filt), padding=(1, 1, 1, 1), bias=b), T(img), T(biases))
+    for way in (True, False):
+        np.testing.assert_allclose(got[way][0][0], plain + biases[:, None, None, None, :], rtol=1e-5, atol=1e-5)
+
+
 def test_forward_mode_inside_a_batched_map(emulator):
     X, V, W = RNG.standard_normal((5, 3)), RNG.standard_normal((5, 3)), RNG.standard_normal((3, 4))
 
