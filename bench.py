@@ -252,6 +252,22 @@ def committed_traffic(workload: str, kernel_hashes: set):
     return z.get("traffic_bytes_per_launch"), f"profiles/hbm_traffic_{workload}.json (rocprofv3 --pmc, kernel {z.get('kernel')})"
 
 
+def result_digest(nb, out) -> dict:
+    """What a step returned, condensed on the host: its first leaf's first element (the loss of
+    the training steps), the sum of magnitudes over every leaf, and whether all are finite."""
+    leaves, _ = nb.tree_flatten(out)
+    head, total, finite = None, 0.0, True
+    for leaf in leaves:
+        if not isinstance(leaf, nb.Tensor):
+            continue
+        a = np.asarray(leaf.numpy(), dtype=np.float64)
+        if head is None:
+            head = float(a.reshape(-1)[0])
+        finite = finite and bool(np.isfinite(a).all())
+        total += float(np.abs(a).sum())
+    return {"head": head, "abs_sum": total, "finite": finite}
+
+
 def launch_flops(step) -> float:
     """Algorithmic flops of one MFMA launch of the plan (attention counted causal-aware)."""
     a, k = step.attrs, step.kind
@@ -301,6 +317,7 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
     cf = nb.compile(w["fn"])
     args = w["args"]
     out = cf(*args)  # miss: trace, lower, bind
+    first = result_digest(nb, out)  # (read now: the plan hands its result slabs out again)
     spec = next(iter(next(iter(cf._cache.values())).specializations.values()))
     plan = spec.bound.plan
     flat, _ = nb.tree_flatten((args, {}))
@@ -336,7 +353,16 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
     if single:
         kernel_timing = "HIP events around the launch, inside the timed region"
         dur = timer.durations_ms()
+    # the step that was timed (a graph replay for the multi-launch steps) still computes what the
+    # first, plainly launched call computed
+    last = result_digest(nb, out)
     del out
+    if not (first["finite"] and last["finite"]):
+        raise RuntimeError(f"{w['name']}: a result of the timed step is not finite: {first} / {last}")
+    if abs(first["head"] - last["head"]) > 1e-6 * abs(first["head"]) + 1e-12 or \
+            abs(first["abs_sum"] - last["abs_sum"]) > 1e-5 * abs(first["abs_sum"]) + 1e-12:
+        raise RuntimeError(f"{w['name']}: the timed step's results differ from the first call's: "
+                           f"{first} / {last}")
     # the same plan one layer below the public call
     for _ in range(min(warmup, 3)):
         spec.bound.run(inputs)
@@ -420,7 +446,8 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
                 "frac_of_hbm_peak_over_32MB": round(b_big / (t_big * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if t_big else 0.0,
                 "slowest": [{"kernel": r[2], "us": round(r[0] * 1e3, 1), "gb_per_s": round(r[1] / (r[0] * 1e-3) / 1e9, 1)}
                             for r in rows[:6]]}
-    res = {"workload": w["name"], "value": round(steps / wall, 3), "unit": "steps/s",
+    res = {"self_check": {"first_result": first["head"], "same_after_timed_region": True, "finite": True},
+           "workload": w["name"], "value": round(steps / wall, 3), "unit": "steps/s",
            "ms_per_step": round(wall / steps * 1e3, 4),
            "plan_ms_per_step": round(wall_plan / steps * 1e3, 4),
            "dtype": w["dtype"], "graph_replays_in_timed_region": replays,
@@ -468,22 +495,57 @@ def main() -> int:
         gc.collect()
         torch.cuda.empty_cache()
     head = results[names[-1]]  # c5 (the largest configuration) when all five run
+    # The one line stays small enough to be read whole from the end of a log: the headline
+    # configuration with its three slowest product shapes, then one compact object per
+    # configuration, last.  Everything else (every product shape, the slowest row kernels, plan
+    # statistics, the CPU samples) goes to a side file.
+    details = os.environ.get("NBK_BENCH_DETAILS", os.path.join(ROOT, "gpurun_out", "bench_details.json"))
+    try:
+        os.makedirs(os.path.dirname(details), exist_ok=True)
+        with open(details, "w") as f:
+            json.dump({"host": host, "configs": results}, f, indent=1)
+    except OSError:
+        details = None
+
+    def brief_roofline(r: dict, shapes: int) -> dict:
+        keep = {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel",
+                                  "kernel_ms_per_step", "launches_per_step", "algorithmic_per_step")
+                if k in r}
+        if shapes and "by_kernel" in r:
+            keep["by_kernel"] = r["by_kernel"][:shapes]
+        if "row_kernels" in r:
+            rk = r["row_kernels"]
+            keep["row_kernels"] = {k: rk[k] for k in ("launches_per_step", "ms_per_step", "gb_per_s_over_32MB",
+                                                     "frac_of_hbm_peak_over_32MB")}
+        return keep
+
+    def brief_config(v: dict) -> dict:
+        r = v["roofline"]
+        c = {"ms_per_step": v["ms_per_step"], "value": v["value"], "dtype": v["dtype"],
+             "roofline": {"bound": r["bound"], "frac": r["frac"], "achieved": r["achieved"], "unit": r["unit"],
+                          "kernel_ms_per_step": r["kernel_ms_per_step"], "traffic": r["traffic"]}}
+        if "row_kernels" in r:
+            c["row_kernels_frac_of_hbm_peak_over_32MB"] = r["row_kernels"]["frac_of_hbm_peak_over_32MB"]
+        if "cpu_baseline" in v:
+            c["cpu_baseline"] = {"value": v["cpu_baseline"]["value"], "cores": v["cpu_baseline"]["cores"]}
+        return c
+
     line = {
         "metric": METRIC, "value": head["value"], "unit": "steps/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
         "config": {"workload": head["workload"],
                    "step": "public compiled call: forward + gradients, inputs resident in HBM",
-                   "plan_ms_per_step": head["plan_ms_per_step"], "plan": head["plan"],
-                   "graph_replays_in_timed_region": head["graph_replays_in_timed_region"]},
-        "roofline": head["roofline"], "cpu_baseline": head.get("cpu_baseline"),
+                   "plan_ms_per_step": head["plan_ms_per_step"], "launches_per_step": head["plan"]["steps"],
+                   "graph_replays_in_timed_region": head["graph_replays_in_timed_region"],
+                   "self_check": head["self_check"]},
+        "roofline": brief_roofline(head["roofline"], 3), "cpu_baseline": head.get("cpu_baseline"),
+        "host": {"cpu_model": host["cpu_model"], "os_cpu_count": host["os_cpu_count"]},
+        "details_file": os.path.relpath(details, ROOT) if details else None,
     }
+    line["roofline"]["kernel_timing"] = head["roofline"]["kernel_timing"]
     if len(names) > 1:
-        line["configs"] = {k: {kk: v[kk] for kk in ("workload", "value", "unit", "ms_per_step",
-                                                    "plan_ms_per_step", "dtype", "roofline",
-                                                    "cpu_baseline") if kk in v}
-                           for k, v in results.items()}
-        line["host"] = host
+        line["configs"] = {k: brief_config(v) for k, v in results.items()}
     print(json.dumps(line))
     return 0
 

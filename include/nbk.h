@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 19
+#define NBK_ABI_VERSION 20
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -442,6 +442,24 @@ typedef int (*nbk_custom_fn)(const nbk_tensor* in, int n_in, nbk_tensor* out,
                              int n_out, void* stream);
 int nbk_custom(const char* library_path, const char* name, const nbk_tensor* in,
                int n_in, nbk_tensor* out, int n_out, void* stream);
+
+/* ===================================================================== */
+/*  Elementwise arithmetic on 64-bit integers                             */
+/* ===================================================================== */
+/* out = op(in[0] [, in[1] [, in[2]]]) element by element in int64 arithmetic; replaces the MAX
+ * elementwise ops behind nabla/ops/binary.py:18-156 (add/sub/mul/div), comparison.py:63-106,
+ * control_flow.py:21-141 (where) and the casts of unary.py:660-697 whenever an operand or the
+ * result is int64 (argmax results, token ids, labels, counters).  The fused row programs hold
+ * integers in 32-bit registers, so the lowering sends these operations here instead: exact
+ * over the whole int64 range, sums / differences / products wrap modulo 2^64 as numpy's do,
+ * division rounds toward zero (x / 0 gives 0).  `op` is one of the NBK_OP_* elementwise codes
+ * MOV TRUNC NEG ABS RELU NOT NEZ ADD..OR WHERE FMA.  Every operand has the result's rank and
+ * shape (broadcast axes have stride 0; strides in elements) and any dtype: integers and bool
+ * widen to int64, floats are cut toward zero.  An operand with ptr == NULL is the constant
+ * imm[k].  The result is stored as out->dtype: int64, int32 (low 32 bits), bool (!= 0) or a
+ * float type (nearest). */
+int nbk_ew_int64(int32_t op, const nbk_tensor* in, const int64_t* imm, int32_t n_in,
+                 const nbk_tensor* out, void* stream);
 
 /* ===================================================================== */
 /*  Random tensors                                                        */

@@ -362,6 +362,28 @@ class BoundPlan:
                     fn = L.nbk_sgd_multi
                 d.dtype = a["dtype"].abi
                 self.calls.append((fn, [C.byref(d), table, len(entries)], patches, (d, table)))
+            elif k == "ew64":
+                refs = a["operands"]
+                ins = (lib.TensorDesc * len(refs))()
+                imm = (C.c_int64 * len(refs))()
+                out = lib.TensorDesc()
+                dst = a["dst"]
+                for t, r in list(zip(ins, refs)) + [(out, dst)]:
+                    if isinstance(r, int):
+                        continue  # (ptr stays NULL: the operand is the immediate)
+                    t.dtype = r.dtype.abi
+                    t.rank = len(r.shape)
+                    for j, (d_, s_) in enumerate(zip(r.shape, r.strides)):
+                        t.shape[j] = d_
+                        t.stride[j] = s_
+                    ptr_field(t, "ptr", r.buf, r.offset * r.dtype.size_in_bytes)
+                for i, r in enumerate(refs):
+                    if isinstance(r, int):
+                        imm[i] = r
+                        ins[i].rank = len(dst.shape)
+                self.calls.append((L.nbk_ew_int64,
+                                   [C.c_int32(isa.EW[a["fn"]]), ins, imm, len(refs), C.byref(out)],
+                                   patches, (ins, imm, out)))
             elif k == "custom":
                 ins = (lib.TensorDesc * max(len(a["ins"]), 1))()
                 outs = (lib.TensorDesc * len(a["dsts"]))()

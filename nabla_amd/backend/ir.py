@@ -190,6 +190,18 @@ def ew(fn: str, *xs: Value | float | int, dtype: DType | None = None) -> Value:
             dtype = tensors[0].dtype
             for t in tensors[1:]:
                 dtype = promote(dtype, t.dtype)
+    # int64 values meet floats as floats: an int64 operand of a floating-point operation or of a
+    # comparison with a float is converted first (its own exact step), so that whatever touches
+    # int64 storage afterwards is either pure integer work or a plain float kernel
+    if fn == "where" and isinstance(xs[0], Value) and xs[0].dtype is DType.int64:
+        xs = (cast(xs[0], DType.bool),) + tuple(xs[1:])
+        tensors = [x for x in xs if isinstance(x, Value)]
+    floats = [t.dtype for t in tensors if t.dtype.is_float()]
+    if fn not in ("mov", "trunc", "nez") and any(t.dtype is DType.int64 for t in tensors) and \
+            (dtype.is_float() or (fn in BOOL_FNS and floats)):
+        to = dtype if dtype.is_float() else floats[0]
+        xs = tuple(cast(x, to) if isinstance(x, Value) and x.dtype is DType.int64 else x for x in xs)
+        tensors = [x for x in xs if isinstance(x, Value)]
     operands = tuple(x if isinstance(x, Value) else float(x) for x in xs)
     return current().add("ew", tensors, [(shape, dtype)], fn=fn, operands=operands)[0]
 

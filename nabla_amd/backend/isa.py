@@ -27,6 +27,9 @@ BINARY.update(INT_BINARY)
 INT_FORM = {"add": "iadd", "sub": "isub", "mul": "imul", "max": "imax", "min": "imin", "gt": "igt",
             "ge": "ige", "eq": "ieq", "ne": "ine", "lt": "ilt", "le": "ile", "neg": "ineg",
             "abs": "iabs", "relu": "irelu", "nez": "inez", "mov": "mov"}
+#: elementwise functions of the 64-bit integer kernel (nbk_ew_int64), under their float codes
+INT64_FNS = ("mov", "trunc", "neg", "abs", "relu", "not", "nez", "add", "sub", "mul", "div", "max", "min",
+             "gt", "ge", "eq", "ne", "lt", "le", "pow", "and", "or", "where", "fma")
 EW = {**UNARY, **BINARY, **TERNARY}
 EW_NAME = {v: k for k, v in EW.items()}
 

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 MAX_RANK = 8
 
@@ -203,6 +203,8 @@ _SIGNATURES = {
                          C.c_void_p], C.c_int),
     "nbk_custom": ([C.c_char_p, C.c_char_p, C.POINTER(TensorDesc), C.c_int,
                     C.POINTER(TensorDesc), C.c_int, C.c_void_p], C.c_int),
+    "nbk_ew_int64": ([C.c_int32, C.POINTER(TensorDesc), C.POINTER(C.c_int64), C.c_int32,
+                      C.POINTER(TensorDesc), C.c_void_p], C.c_int),
     "nbk_event_create": ([C.POINTER(C.c_void_p)], C.c_int),
     "nbk_event_record": ([C.c_void_p, C.c_void_p], C.c_int),
     "nbk_event_elapsed_ms": ([C.c_void_p, C.c_void_p, C.POINTER(C.c_float)], C.c_int),

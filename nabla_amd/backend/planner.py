@@ -313,6 +313,84 @@ class Planner:
     def _is_member_value(self, v: ir.Value) -> bool:
         return v.node.kind in FUSABLE or v.node.pos in self.alias_nodes
 
+    # ................................................................ int64
+    _I32_OPEN = (-(2 ** 31) + 1, 2 ** 31 - 2)  # strictly inside the int32 range
+    _COMPARISONS = ("eq", "ne", "gt", "ge", "lt", "le")
+
+    def _inside_int32(self, x) -> bool:
+        """Is ``x`` (an operand of an ew node) an index or constant made inside the kernel whose
+        every value lies strictly inside the int32 range?"""
+        lo, hi = self._I32_OPEN
+        if not isinstance(x, ir.Value):
+            return float(x) == int(x) and lo <= int(x) <= hi
+        while x.node.kind in VIEW_KINDS:
+            x = x.node.inputs[0]
+        n = x.node
+        if n.kind == "fill":
+            v = n.attrs["value"]
+            return v == int(v) and lo <= int(v) <= hi
+        if n.kind == "iota":
+            first = n.attrs["start"]
+            last = first + n.attrs["step"] * max(x.shape[-1] - 1, 0)
+            return lo <= min(first, last) and max(first, last) <= hi
+        return False
+
+    def _wants_int64_kernel(self, node: ir.Node) -> bool:
+        """Does this fusable node have to run in the 64-bit integer kernel?  Row programs hold
+        integers in 32-bit registers and read int64 storage saturated to the int32 range.
+        That is exact for exactly one use of an int64 tensor: a comparison with an index or
+        constant strictly inside the int32 range (labels against a class index, ids against a
+        position), because saturation moves no value across such a bound.  Everything else
+        that reads or makes int64 values -- arithmetic, selects, copies, casts, comparisons of
+        two stored tensors -- is exact only in 64 bits."""
+        i64 = DType.int64
+        if node.kind == "iota":
+            if node.outputs[0].dtype is i64 and not self._inside_int32(node.outputs[0]):
+                raise NotImplementedError(
+                    "an int64 index sequence that leaves the int32 range has no kernel; "
+                    "build it on the host (Tensor.constant(numpy.arange(...)))")
+            return False
+        if node.kind == "tril":
+            if node.outputs[0].dtype is i64:
+                raise NotImplementedError("tril / triu of an int64 tensor: cast it to int32 or a "
+                                          "floating-point type first")
+            return False
+        if node.kind != "ew":
+            return False
+        if node.outputs[0].dtype is not i64 and not any(i.dtype is i64 for i in node.inputs):
+            return False
+        xs = node.attrs["operands"]
+        if node.fn in self._COMPARISONS and any(self._inside_int32(x) for x in xs):
+            return False
+        if node.fn not in isa.INT64_FNS:
+            raise NotImplementedError(
+                f"'{node.fn}' has no integer form: cast the int64 tensor to a floating-point type first")
+        return True
+
+    def _lower_int64_ew(self, n: ir.Node) -> None:
+        """One launch of the 64-bit integer kernel for an elementwise node (operands as strided
+        views of the result's shape, constants as immediates)."""
+        out = n.outputs[0]
+        ops = []
+        for x in n.attrs["operands"]:
+            if not isinstance(x, ir.Value):
+                ops.append(int(x))
+                continue
+            ref = self._resolve(x)
+            if isinstance(ref, Const):
+                if ref.value != int(ref.value):
+                    ref = self._materialize(ref)
+                else:
+                    ops.append(int(ref.value))
+                    continue
+            ops.append(ref)
+        if all(isinstance(o, int) for o in ops):  # (a kernel needs one operand in memory)
+            first = next(x for x in n.attrs["operands"] if isinstance(x, ir.Value))
+            ops[list(n.attrs["operands"]).index(first)] = self._materialize(self._resolve(first))
+        dst = self._alloc_value(out)
+        self._emit(Step("ew64", [o.buf for o in ops if isinstance(o, ViewRef)], [dst.buf],
+                        dict(fn=n.fn, operands=ops, dst=dst)))
+
     def _depends(self, u: Unit, g: Unit, skip: "Unit | None" = None) -> bool:
         """Does unit ``u`` (transitively) need ``g`` to have run?  Paths through
         ``skip`` are ignored (used when ``skip`` is about to be merged with g)."""
@@ -440,10 +518,11 @@ class Planner:
                         self.unit_of[node.pos] = g
                         self.alias_nodes.add(node.pos)
                 continue
-            # (integer reductions keep a 64-bit accumulator in a kernel of their own)
+            # (integer reductions keep a 64-bit accumulator in a kernel of their own, and so does
+            # elementwise work on int64 values: row-program registers are 32 bits wide)
             if kind not in FUSABLE or (kind == "reduce" and (
                     node.attrs["axis"] != node.inputs[0].rank - 1 or
-                    node.inputs[0].dtype in INT_REG_DTYPES)):
+                    node.inputs[0].dtype in INT_REG_DTYPES)) or self._wants_int64_kernel(node):
                 u = new_unit(node, False)
                 for i in node.inputs:
                     pu = self._producer_unit(i)
@@ -1027,6 +1106,8 @@ class Planner:
         out = n.outputs[0]
         if k == "matmul":
             self._lower_matmul(n)
+        elif k == "ew":
+            self._lower_int64_ew(n)
         elif k == "reduce":
             self._lower_reduce_mid(n)
         elif k == "argreduce":

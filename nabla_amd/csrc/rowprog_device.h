@@ -31,14 +31,20 @@ __device__ __forceinline__ void rp_store4_stream(float* p, float4 r) {
 // Registers are 32 bits wide and typed by the program, not by the hardware: a value of an
 // integer tensor (int32, int64) is held as a two's-complement int32 in the register's bits and
 // computed with the integer instructions, so integers are exact over the whole int32 range
-// (int64 storage is read and written through its low 32 bits, sign-extended on the way out);
+// (an int64 operand is read saturated to the int32 range and written sign-extended: the lowering
+// keeps int64 tensors in these programs only where they are compared with an index or constant
+// strictly inside that range, which saturation leaves exact, and sends every other operation
+// on int64 values to the 64-bit elementwise kernel);
 // everything else -- floats, and bool / uint8 as 0.0, 1.0, ... -- is held as fp32.
 __device__ __forceinline__ float rp_ibits(int v) { return __int_as_float(v); }
 __device__ __forceinline__ int rp_int(float v) { return __float_as_int(v); }
 
+__device__ __forceinline__ int rp_sat32(int64_t v) {
+  return v > 2147483647LL ? 2147483647 : (v < -2147483648LL ? (int)(-2147483647 - 1) : (int)v);
+}
 __device__ __forceinline__ float rp_load1(const void* p, int64_t i, int dt) {
   if (dt == NBK_I32) return rp_ibits(((const int32_t*)p)[i]);
-  if (dt == NBK_I64) return rp_ibits((int)((const int64_t*)p)[i]);
+  if (dt == NBK_I64) return rp_ibits(rp_sat32(((const int64_t*)p)[i]));
   return nbk_load_as_f32(p, i, dt);
 }
 __device__ __forceinline__ void rp_store1(void* p, int64_t i, int dt, float v) {
@@ -73,7 +79,8 @@ __device__ __forceinline__ float4 rp_load4(const nbk_operand& o, int64_t off, in
     } else if (dt == NBK_I64) {
       const int64_t* p = (const int64_t*)o.ptr + e;
       longlong2 u0 = *(const longlong2*)p, u1 = *(const longlong2*)(p + 2);
-      r = make_float4(rp_ibits((int)u0.x), rp_ibits((int)u0.y), rp_ibits((int)u1.x), rp_ibits((int)u1.y));
+      r = make_float4(rp_ibits(rp_sat32(u0.x)), rp_ibits(rp_sat32(u0.y)), rp_ibits(rp_sat32(u1.x)),
+                      rp_ibits(rp_sat32(u1.y)));
     } else {
       uint32_t u = *(const uint32_t*)((const uint8_t*)o.ptr + e);
       r = make_float4((float)(u & 0xff), (float)((u >> 8) & 0xff), (float)((u >> 16) & 0xff),

@@ -107,8 +107,10 @@ _BINARY.update({
 
 
 def _load_reg(t: torch.Tensor) -> np.ndarray:
-    """Elements of an operand as register contents."""
-    if t.dtype in (torch.int32, torch.int64):
+    """Elements of an operand as register contents (int64 storage saturates to the int32 range)."""
+    if t.dtype == torch.int64:
+        return _fbits(np.clip(t.numpy(), -2 ** 31, 2 ** 31 - 1))
+    if t.dtype == torch.int32:
         return _fbits(t.numpy())
     return _as_f32(t)
 
@@ -133,6 +135,62 @@ def _store(flat: torch.Tensor, idx: np.ndarray, vals: np.ndarray) -> None:
     else:
         v = v.to(flat.dtype)
     flat[torch.from_numpy(idx.reshape(-1))] = v.reshape(-1)
+
+
+def _ew_int64(a: dict, mem: list[torch.Tensor]) -> None:
+    """The 64-bit integer elementwise kernel: operands widen to int64 (floats are cut toward
+    zero), the arithmetic wraps modulo 2^64, division rounds toward zero."""
+    dst = _view(mem, a["dst"])
+
+    def widen(o):
+        if isinstance(o, int):
+            return np.int64(o)
+        t = _view(mem, o)
+        if t.dtype.is_floating_point:
+            x = np.nan_to_num(np.trunc(t.double().numpy()), nan=0.0)
+            return np.clip(x, -2.0 ** 63, 2.0 ** 63 - 1025).astype(np.int64)
+        return t.numpy().astype(np.int64)
+
+    def div(p, q):
+        safe = np.where(q == 0, 1, q)
+        r = np.abs(p) // np.abs(safe) * np.sign(p) * np.sign(safe)
+        return np.where(q == 0, 0, r).astype(np.int64)
+
+    def ipow(b, e):
+        b, e = np.broadcast_arrays(np.asarray(b, np.int64), np.asarray(e, np.int64))
+        out = np.empty(b.shape, np.int64)
+        for idx in np.ndindex(b.shape):
+            bb, ee = int(b[idx]), int(e[idx])
+            if ee < 0:
+                v = 1 if bb == 1 else ((-1 if ee & 1 else 1) if bb == -1 else 0)
+            else:
+                v = pow(bb, ee, 2 ** 64)
+                v = v - 2 ** 64 if v >= 2 ** 63 else v
+            out[idx] = v
+        return out
+
+    xs = [widen(o) for o in a["operands"]]
+    fn = a["fn"]
+    with np.errstate(over="ignore"):
+        r = {
+            "mov": lambda p: p, "trunc": lambda p: p, "neg": lambda p: -p, "abs": lambda p: np.abs(p),
+            "relu": lambda p: np.maximum(p, 0), "not": lambda p: p == 0, "nez": lambda p: p != 0,
+            "add": lambda p, q: p + q, "sub": lambda p, q: p - q, "mul": lambda p, q: p * q, "div": div,
+            "max": np.maximum, "min": np.minimum, "gt": lambda p, q: p > q, "ge": lambda p, q: p >= q,
+            "eq": lambda p, q: p == q, "ne": lambda p, q: p != q, "lt": lambda p, q: p < q,
+            "le": lambda p, q: p <= q, "pow": ipow, "and": lambda p, q: (p != 0) & (q != 0),
+            "or": lambda p, q: (p != 0) | (q != 0), "where": lambda c, p, q: np.where(c != 0, p, q),
+            "fma": lambda p, q, c: p * q + c,
+        }[fn](*xs)
+    r = np.broadcast_to(np.asarray(r), tuple(dst.shape)).astype(np.int64)
+    if dst.dtype == torch.bool:
+        dst.copy_(torch.from_numpy(r != 0))
+    elif dst.dtype == torch.int32:
+        dst.copy_(torch.from_numpy(r.astype(np.int32)))
+    elif dst.dtype == torch.int64:
+        dst.copy_(torch.from_numpy(r.copy()))
+    else:
+        dst.copy_(torch.from_numpy(r.astype(np.float32)).to(dst.dtype))
 
 
 def run_rowprog(a: dict, mem: list[torch.Tensor]) -> None:
@@ -511,7 +569,15 @@ class EmulatedPlan:
                 ix = torch.where(ix < 0, ix + a["axis_len"], ix)
                 for j in range(a["n_idx"]):  # in order: the last write to a row wins
                     dst[:, int(ix[j]), :] = up[:, j, :]
+            elif k == "ew64":
+                _ew_int64(a, mem)
             elif k == "argreduce":
+                src = _view(mem, a["src"])
+                if src.dtype in (torch.int32, torch.int64):  # integers compare exactly
+                    xi = src.numpy().astype(np.int64).reshape(a["rows"], a["C"])
+                    r = np.argmin(xi, axis=1) if a["fn"] == "min" else np.argmax(xi, axis=1)
+                    _view(mem, a["dst"]).copy_(torch.from_numpy(r.astype(np.int64)).reshape(a["dst"].shape))
+                    continue
                 x = _as_f32(_view(mem, a["src"])).reshape(a["rows"], a["C"])
                 r = np.argmin(x, axis=1) if a["fn"] == "min" else np.argmax(x, axis=1)
                 _view(mem, a["dst"]).copy_(torch.from_numpy(r.astype(np.int64)).reshape(a["dst"].shape))

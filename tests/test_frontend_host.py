@@ -633,6 +633,13 @@ def test_integers_above_2_pow_24_are_exact(emulator):
     check_large_integers(nb)
 
 
+def test_int64_beyond_the_int32_range_is_exact(emulator):
+    """Arithmetic, comparisons, selects and casts on int64 values outside the int32 range run in
+    the 64-bit integer kernel; the label-against-class-index comparison stays fused and exact."""
+    from integer_cases import check_int64_beyond_int32
+    check_int64_beyond_int32(nb)
+
+
 def test_sum_with_a_product_folds_into_its_epilogue_when_asked(emulator):
     """``r + x @ W + b`` becomes one product that reads ``r`` and ``b`` in its epilogue under
     ``FOLD_RESIDUAL`` (off by default: the epilogue read measured slower than the sum kernel);

@@ -383,6 +383,13 @@ def test_integers_above_2_pow_24_are_exact(hip):
     check_large_integers(nb)
 
 
+def test_int64_beyond_the_int32_range_is_exact(hip):
+    """Arithmetic, comparisons, selects and casts on int64 values outside the int32 range run in
+    the 64-bit integer kernel; the label-against-class-index comparison stays fused and exact."""
+    from integer_cases import check_int64_beyond_int32
+    check_int64_beyond_int32(nb)
+
+
 def test_tensors_without_elements_and_domain_edges(hip):
     from edge_cases import check_empty_tensors, check_log1p_and_atanh_at_the_edges
     check_empty_tensors(nb)
@@ -508,6 +515,42 @@ def test_compiled_train_step_on_device(hip):
         assert relerr(p[k].numpy(), ref[k]) < F32_TOL
 
 
+def test_compiled_step_with_a_dynamic_batch_on_device(hip):
+    """`compile(dynamic_dims={4: {0: "batch"}})` (nabla/transforms/compile.py:207-268, 508-555;
+    the key counts the tensor leaves of the flattened arguments: four parameters, then x): one
+    signature serves every batch size.  The MLP step is called with three batch sizes, back to
+    the first, and repeatedly on one size (so that a replayed recording is among the calls);
+    every loss and gradient is checked against the oracle at that size, and the statistics
+    show a single miss."""
+    from nabla_amd.core import engine
+    t0 = oc.c1_inputs(8, 48, 24, 5, seed=12)
+    t0["b1"] = np.random.default_rng(3).uniform(-0.05, 0.05, t0["b1"].shape).astype(np.float32)
+    names = ("W1", "b1", "W2", "b2")
+    params = {k: T(t0[k]) for k in names}
+
+    @nb.compile(dynamic_dims={4: {0: "batch"}})
+    def step(p, x):
+        return nb.value_and_grad(lambda q: nb.mean(nb.relu(x @ q["W1"] + q["b1"]) @ q["W2"] + q["b2"]))(p)
+
+    rng = np.random.default_rng(13)
+    xs = {n: rng.uniform(-0.05, 0.05, (n, 48)).astype(np.float32) for n in (8, 37, 128, 1)}
+    dev = {n: T(a) for n, a in xs.items()}
+    plans_before = len(engine._PLAN_CACHE)
+    calls = 0
+    for n in (8, 37, 128, 8, 8, 8, 37, 1, 128, 37):
+        loss, g = step(params, dev[n])
+        calls += 1
+        wl, wg = oc.c1_reference(xs[n], *[t0[k] for k in names])
+        assert abs(loss.item() - wl) <= F32_TOL * abs(wl) + 1e-9, n
+        for k, w in zip(names, wg):
+            assert g[k].shape == w.shape
+            assert relerr(g[k].numpy(), w) < F32_TOL, (n, k)
+        del loss, g
+    assert step.stats.misses == 1 and step.stats.hits == calls - 1, step.stats
+    # one launch plan per batch size that was seen, not per call
+    assert len(engine._PLAN_CACHE) - plans_before <= len(xs)
+
+
 # ---- optimizer step (next row after the hot path: nn/optim) ---------------------------------------
 @pytest.mark.parametrize("dtype,tol", [("f32", 2e-5), ("bf16", 2e-2)])
 def test_adamw_and_sgd_steps_on_device(hip, dtype, tol):
@@ -553,6 +596,8 @@ def test_graph_replay_matches_eager_every_time(hip):
     the replays, and a call on new buffers falls back to plain launches.  The plan owns the
     slabs its results live in, so the replay does not depend on what the allocator hands out:
     the caller just lets go of the previous results, as a training loop does."""
+    if not hip.use_graphs:
+        pytest.skip("graph replay is switched off (NBK_GRAPHS=0): nothing to replay")
     t = oc.c1_inputs(64, 96, 48, 10, seed=31)
     t["b1"] = np.random.default_rng(2).uniform(-0.05, 0.05, t["b1"].shape).astype(np.float32)
     wl, wg = oc.c1_reference(**t)
@@ -722,7 +767,11 @@ def test_vmap_batched_per_example_gradients_of_a_block_on_device(hip):
     """Per-example gradients of a two-layer block with layer norm over 256 examples: vmap runs
     the function once on the batch (its launches do not grow with the batch), and the result is
     the float64 closed form per example, computed by looping in numpy."""
+    from nabla_amd import config
     from nabla_amd.core import engine
+    if not config.VMAP_BATCHED:
+        pytest.skip("batched vmap is switched off (NBK_VMAP_BATCHED=0): the element-by-element map "
+                    "is covered by test_vmap_per_example_gradients_on_device")
     rng = np.random.default_rng(50)
     n, s, d, h = 256, 8, 32, 64
     X, Y = rng.standard_normal((n, s, d)), rng.standard_normal((n, s, d))
