@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 20
+#define NBK_ABI_VERSION 21
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -369,15 +369,23 @@ typedef struct nbk_attn_tensor {
   void* ptr;
   int64_t sb, ss, sh;
 } nbk_attn_tensor;
+/* `o_lo` (may be NULL, or have ptr == NULL): a second bf16 tensor of O's shape that receives
+ * what rounding O to bf16 cut off, O_fp32 - O_bf16.  The backward pass forms
+ * delta = rowsum(dO * O) and then dS = P * (dP - delta); where the keys a query sees have
+ * values with a large common part, dP - delta cancels most of dP and a delta taken from bf16 O
+ * alone puts errors of several percent on dQ and dK (measured: 2-4 % on the query-side
+ * gradients of a 12-layer decoder against 0.5-1 % on the value side).  Handing the same tensor
+ * to the backward pass brings delta to about 16 bits. */
 int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
                       const nbk_attn_tensor* k, const nbk_attn_tensor* v,
-                      const nbk_attn_tensor* o, void* lse, void* stream);
+                      const nbk_attn_tensor* o, const nbk_attn_tensor* o_lo, void* lse,
+                      void* stream);
 /* Backward needs nbk_attention_bwd_workspace(d) bytes of caller scratch (one
  * fp32 per score row: rowsum(dO * O)). */
 int64_t nbk_attention_bwd_workspace(const nbk_attn_desc* d);
 int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
                       const nbk_attn_tensor* k, const nbk_attn_tensor* v,
-                      const nbk_attn_tensor* o, const void* lse,
+                      const nbk_attn_tensor* o, const nbk_attn_tensor* o_lo, const void* lse,
                       const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                       const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
                       void* workspace, int64_t workspace_bytes, void* stream);
@@ -394,7 +402,8 @@ int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q,
 #define NBK_ATTN_STATIC_ROWS (1 << 20)
 int nbk_attention_bwd_static(const nbk_attn_desc* d, const nbk_attn_tensor* q,
                              const nbk_attn_tensor* k, const nbk_attn_tensor* v,
-                             const nbk_attn_tensor* o, const void* lse,
+                             const nbk_attn_tensor* o, const nbk_attn_tensor* o_lo,
+                             const void* lse,
                              const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                              const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
                              void* stream);

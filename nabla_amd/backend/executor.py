@@ -276,15 +276,16 @@ class BoundPlan:
 
                 holder = _Ptrs(2)
                 ptr_field(holder, "p0", a["lse"].buf, a["lse"].offset * 4)
+                o_lo = heads(a["o_lo"]) if a.get("o_lo") is not None else None
                 if k == "attention":
                     args = [_LATE, C.byref(d), heads(a["q"]), heads(a["k"]), heads(a["v"]), heads(a["o"]),
-                            _Late(holder, "p0")]
+                            o_lo, _Late(holder, "p0")]
                     self.calls.append((L.nbk_attention_fwd, args, patches, keep_alive))
                 else:
                     ws = a["workspace"]
                     ptr_field(holder, "p1", ws.buf, ws.offset * 4)
                     args = [_LATE, C.byref(d), heads(a["q"]), heads(a["k"]), heads(a["v"]), heads(a["o"]),
-                            _Late(holder, "p0"), heads(a["dout"]), heads(a["dq"]), heads(a["dk"]),
+                            o_lo, _Late(holder, "p0"), heads(a["dout"]), heads(a["dq"]), heads(a["dk"]),
                             heads(a["dv"]), _Late(holder, "p1"), C.c_int64(a["workspace_bytes"])]
                     self.calls.append((L.nbk_attention_bwd, args, patches, keep_alive))
             elif k == "gather":

@@ -452,18 +452,20 @@ def custom(name: str, library: str, inputs: Sequence[Value], out_types: Sequence
 
 # ---- fused attention ----------------------------------------------------------------------
 def attention(q: Value, k: Value, v: Value, scale: float, causal: bool) -> list[Value]:
-    """[B, H, S, hd] heads -> (output [B, H, S, hd], log-sum-exp of the score rows [B, H, S])."""
+    """[B, H, S, hd] heads -> (output [B, H, S, hd], log-sum-exp of the score rows [B, H, S],
+    what rounding the output to its 16-bit type cut off [B, H, S, hd], for the backward pass)."""
     if not (q.shape == k.shape == v.shape) or q.rank != 4:
         raise ValueError(f"attention: q, k, v must share one [B, H, S, hd] shape, got "
                          f"{q.shape}, {k.shape}, {v.shape}")
-    return current().add("attention", [q, k, v], [(q.shape, q.dtype), (q.shape[:-1], DType.float32)],
+    return current().add("attention", [q, k, v],
+                         [(q.shape, q.dtype), (q.shape[:-1], DType.float32), (q.shape, q.dtype)],
                          scale=float(scale), causal=bool(causal))
 
 
-def attention_bwd(q: Value, k: Value, v: Value, o: Value, lse: Value, dout: Value, scale: float,
-                  causal: bool) -> list[Value]:
-    """Gradients (dq, dk, dv) of ``attention`` from its inputs, both outputs and d(output)."""
-    return current().add("attention_bwd", [q, k, v, o, lse, dout], [(q.shape, q.dtype)] * 3,
+def attention_bwd(q: Value, k: Value, v: Value, o: Value, lse: Value, o_lo: Value, dout: Value,
+                  scale: float, causal: bool) -> list[Value]:
+    """Gradients (dq, dk, dv) of ``attention`` from its inputs, its three outputs and d(output)."""
+    return current().add("attention_bwd", [q, k, v, o, lse, o_lo, dout], [(q.shape, q.dtype)] * 3,
                          scale=float(scale), causal=bool(causal))
 
 

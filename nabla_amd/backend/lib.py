@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 MAX_RANK = 8
 
@@ -188,12 +188,12 @@ _SIGNATURES = {
                            C.c_void_p], C.c_int),
     "nbk_avgpool2d_fwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
     "nbk_avgpool2d_bwd": ([C.POINTER(PoolDesc), C.c_void_p, C.c_void_p, C.c_void_p], C.c_int),
-    "nbk_attention_fwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_void_p],
+    "nbk_attention_fwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 5 + [C.c_void_p, C.c_void_p],
                           C.c_int),
     "nbk_attention_bwd_workspace": ([C.POINTER(AttnDesc)], C.c_int64),
-    "nbk_attention_bwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p] +
+    "nbk_attention_bwd": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 5 + [C.c_void_p] +
                           [C.POINTER(AttnTensor)] * 4 + [C.c_void_p, C.c_int64, C.c_void_p], C.c_int),
-    "nbk_attention_bwd_static": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 4 + [C.c_void_p] +
+    "nbk_attention_bwd_static": ([C.POINTER(AttnDesc)] + [C.POINTER(AttnTensor)] * 5 + [C.c_void_p] +
                                  [C.POINTER(AttnTensor)] * 4 + [C.c_void_p], C.c_int),
     "nbk_gather": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64,
                     C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p], C.c_int),

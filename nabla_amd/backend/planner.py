@@ -1685,18 +1685,23 @@ class Planner:
             q, k, v = (self._heads_operand(i) for i in n.inputs)
             o = self._heads_result(n.outputs[0])
             lse = self._alloc_value(n.outputs[1])
-            self._emit(Step("attention", [q.buf, k.buf, v.buf], [o.buf, lse.buf],
-                            dict(common, q=q, k=k, v=v, o=o, lse=lse)))
+            # the rounding remainder of the output is only written where something reads it
+            rest = n.outputs[2]
+            o_lo = self._alloc_value(rest) if (self.users.get(rest.id) or rest.id in self._out_pending) else None
+            self._emit(Step("attention", [q.buf, k.buf, v.buf],
+                            [o.buf, lse.buf] + ([o_lo.buf] if o_lo is not None else []),
+                            dict(common, q=q, k=k, v=v, o=o, lse=lse, o_lo=o_lo)))
             return
         q, k, v, o = (self._heads_operand(i) for i in n.inputs[:4])
         lse = self._contig(n.inputs[4])
-        dout = self._heads_operand(n.inputs[5])
+        o_lo = self._heads_operand(n.inputs[5])
+        dout = self._heads_operand(n.inputs[6])
         dq, dk, dv = (self._heads_result(t) for t in n.outputs)
         wbuf = self._new_buf((B * H * S,), DType.float32, "temp", -1)
         ws = ViewRef(wbuf.id, 0, (B * H * S,), (1,), DType.float32)
-        self._emit(Step("attention_bwd", [q.buf, k.buf, v.buf, o.buf, lse.buf, dout.buf],
+        self._emit(Step("attention_bwd", [q.buf, k.buf, v.buf, o.buf, lse.buf, o_lo.buf, dout.buf],
                         [dq.buf, dk.buf, dv.buf, wbuf.id],
-                        dict(common, q=q, k=k, v=v, o=o, lse=lse, dout=dout, dq=dq, dk=dk, dv=dv,
+                        dict(common, q=q, k=k, v=v, o=o, lse=lse, o_lo=o_lo, dout=dout, dq=dq, dk=dk, dv=dv,
                              workspace=ws, workspace_bytes=B * H * S * 4)))
 
     # ................................................................ groups

@@ -55,6 +55,7 @@ struct AttnTensor {
 
 struct AttnArgs {
   AttnTensor q, k, v, o, dout, dq, dk, dv;
+  AttnTensor o_lo;  // optional: what rounding O to bf16 cut off, itself as bf16 (p == nullptr: none)
   float* lse;    // [B, H, S]
   float* delta;  // [B, H, S]: rowsum(dO * O), backward only
   int32_t B, H, S;
@@ -241,6 +242,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
 #pragma unroll
   for (int d = 0; d < DT; ++d) o_acc[d] = (at_f32x16)(0.f);
   float m_i = at_neg_big(), l_i = 0.f;
+  // The output is normalised by the sum of the probabilities as the matrix cores saw them
+  // (rounded to bf16), so that it is an exact convex combination of the values: a part common to
+  // all values then passes through unchanged, which the backward pass's dP - delta relies on.
+  // That sum comes out of the same MFMAs, with a row of ones in the place of V^T (every row of
+  // l_mm holds it); l_i, the sum before rounding, goes into the log-sum-exp, with which the
+  // probabilities that the backward pass recomputes sum to one as well.
+  at_f32x16 l_mm = (at_f32x16)(0.f);
+  at_bf16x8 ones_frag;
+  {
+    const at_u32x4 u = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    ones_frag = __builtin_bit_cast(at_bf16x8, u);
+  }
 
   const int n_tiles = g.causal ? (q0 + 128) / 64 : g.S / 64;
   RowT kl;
@@ -296,6 +309,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
         m_i = m_new;
 #pragma unroll
         for (int d = 0; d < DT; ++d) o_acc[d] *= alpha;
+        l_mm *= alpha;
       }
       float sum = 0.f;
 #pragma unroll
@@ -317,6 +331,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
           for (int d = 0; d < DT; ++d)
             o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
                                                                o_acc[d], 0, 0, 0);
+          l_mm = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_frag, pf, l_mm, 0, 0, 0);
         }
     };
     // keys of this tile against the wave's queries: all visible, some, or none
@@ -330,7 +345,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   }
   // normalise and write: register r of tile d is O[my_q][32 d + (r/4)*8 + 4h + r%4]
   l_i += at_xhalf(l_i);
-  const float inv = 1.0f / l_i;
+  const float inv = 1.0f / l_mm[0];
   uint16_t* O = (uint16_t*)g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)my_q * g.o.ss;
 #pragma unroll
   for (int d = 0; d < DT; ++d)
@@ -341,6 +356,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
       w.y = at_pack2(o_acc[d][gq * 4 + 2] * inv, o_acc[d][gq * 4 + 3] * inv);
       *(at_u32x2*)(O + d * 32 + gq * 8 + 4 * h) = w;
     }
+  if (g.o_lo.p != nullptr) {
+    // The backward pass needs delta = rowsum(dO * O) to more digits than bf16 O has (dS is
+    // P * (dP - delta), and with many keys of similar value dP - delta cancels almost
+    // everything): the part of O that the rounding above cut off goes out as a second bf16 tensor.
+    uint16_t* OL = (uint16_t*)g.o_lo.p + (int64_t)b * g.o_lo.sb + (int64_t)hh * g.o_lo.sh + (int64_t)my_q * g.o_lo.ss;
+    auto rest = [&](float x) { return x - __uint_as_float((uint32_t)nbk_f32_to_bf16(x) << 16); };
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        at_u32x2 w;
+        w.x = at_pack2(rest(o_acc[d][gq * 4 + 0] * inv), rest(o_acc[d][gq * 4 + 1] * inv));
+        w.y = at_pack2(rest(o_acc[d][gq * 4 + 2] * inv), rest(o_acc[d][gq * 4 + 3] * inv));
+        *(at_u32x2*)(OL + d * 32 + gq * 8 + 4 * h) = w;
+      }
+  }
   if (h == 0) g.lse[((int64_t)b * g.H + hh) * g.S + my_q] = m_i * AT_LN2 + __logf(l_i);
 }
 
@@ -732,7 +763,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_tr_kernel(const AttnArgs g)
   // delta[q] = sum_d dO[q, d] O[q, d] comes out of the dO fragments this kernel loads anyway and
   // the matching pieces of O (a lane pair holds one row); it is left in g.delta for the dK / dV
   // kernel, which runs after this one.
+  // With the forward pass's second tensor (what bf16 O lost) the sum runs over O to about 16
+  // bits: a delta off by 2^-9 of |dO| |O| would be a visible share of dP - delta wherever the
+  // keys a query sees have values with a large common part.
   const uint16_t* O = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh;
+  const uint16_t* OL = g.o_lo.p == nullptr ? nullptr
+                                           : g.o_lo.p + (int64_t)b * g.o_lo.sb + (int64_t)hh * g.o_lo.sh;
   at_bf16x8 qf[KSTEPS], dof[KSTEPS];
   float my_delta = 0.f;
 #pragma unroll
@@ -740,12 +776,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_tr_kernel(const AttnArgs g)
     const at_u32x4 uq = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
     const at_u32x4 ud = *(const at_u32x4*)(DO + (int64_t)my_q * g.dout.ss + s * 16 + h * 8);
     const at_u32x4 uo = *(const at_u32x4*)(O + (int64_t)my_q * g.o.ss + s * 16 + h * 8);
+    at_u32x4 ul = {0u, 0u, 0u, 0u};
+    if (OL != nullptr) ul = *(const at_u32x4*)(OL + (int64_t)my_q * g.o_lo.ss + s * 16 + h * 8);
     qf[s] = __builtin_bit_cast(at_bf16x8, uq);
     dof[s] = __builtin_bit_cast(at_bf16x8, ud);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      my_delta += __uint_as_float(uo[e] << 16) * __uint_as_float(ud[e] << 16);
-      my_delta += __uint_as_float(uo[e] & 0xffff0000u) * __uint_as_float(ud[e] & 0xffff0000u);
+      my_delta += (__uint_as_float(uo[e] << 16) + __uint_as_float(ul[e] << 16)) * __uint_as_float(ud[e] << 16);
+      my_delta += (__uint_as_float(uo[e] & 0xffff0000u) + __uint_as_float(ul[e] & 0xffff0000u)) *
+                  __uint_as_float(ud[e] & 0xffff0000u);
     }
   }
   my_delta += at_xhalf(my_delta);
@@ -897,13 +936,14 @@ static int attn_set_lds(Kern kern, size_t bytes) {
 }
 
 extern "C" int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
-                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, void* lse,
-                                 void* stream) {
+                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o,
+                                 const nbk_attn_tensor* o_lo, void* lse, void* stream) {
   AttnArgs a = {};
   int rc = attn_common(d, &a);
   if (rc) return rc;
   if ((rc = attn_tensor(q, "q", &a.q, true)) || (rc = attn_tensor(k, "k", &a.k, true)) ||
-      (rc = attn_tensor(v, "v", &a.v, true)) || (rc = attn_tensor(o, "o", &a.o, true)))
+      (rc = attn_tensor(v, "v", &a.v, true)) || (rc = attn_tensor(o, "o", &a.o, true)) ||
+      (rc = attn_tensor(o_lo, "o_lo", &a.o_lo, false)))
     return rc;
   NBK_REQUIRE(lse != nullptr, "attention: null lse");
   a.lse = (float*)lse;
@@ -954,13 +994,15 @@ static int attn_bwd_launch(const nbk_attn_desc* d, AttnArgs& a, float* delta, hi
 }
 
 static int attn_bwd_args(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
-                         const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
+                         const nbk_attn_tensor* v, const nbk_attn_tensor* o,
+                         const nbk_attn_tensor* o_lo, const void* lse,
                          const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                          const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, AttnArgs* a) {
   int rc = attn_common(d, a);
   if (rc) return rc;
   if ((rc = attn_tensor(q, "q", &a->q, true)) || (rc = attn_tensor(k, "k", &a->k, true)) ||
       (rc = attn_tensor(v, "v", &a->v, true)) || (rc = attn_tensor(o, "o", &a->o, true)) ||
+      (rc = attn_tensor(o_lo, "o_lo", &a->o_lo, false)) ||
       (rc = attn_tensor(dout, "dout", &a->dout, true)) || (rc = attn_tensor(dq, "dq", &a->dq, true)) ||
       (rc = attn_tensor(dk, "dk", &a->dk, true)) || (rc = attn_tensor(dv, "dv", &a->dv, true)))
     return rc;
@@ -970,12 +1012,13 @@ static int attn_bwd_args(const nbk_attn_desc* d, const nbk_attn_tensor* q, const
 }
 
 extern "C" int nbk_attention_bwd(const nbk_attn_desc* d, const nbk_attn_tensor* q, const nbk_attn_tensor* k,
-                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o, const void* lse,
+                                 const nbk_attn_tensor* v, const nbk_attn_tensor* o,
+                                 const nbk_attn_tensor* o_lo, const void* lse,
                                  const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                                  const nbk_attn_tensor* dk, const nbk_attn_tensor* dv, void* workspace,
                                  int64_t workspace_bytes, void* stream) {
   AttnArgs a = {};
-  int rc = attn_bwd_args(d, q, k, v, o, lse, dout, dq, dk, dv, &a);
+  int rc = attn_bwd_args(d, q, k, v, o, o_lo, lse, dout, dq, dk, dv, &a);
   if (rc) return rc;
   NBK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 15) == 0 &&
                   workspace_bytes >= nbk_attention_bwd_workspace(d),
@@ -1019,12 +1062,13 @@ int nbk_attention_static_setup(void) {
 
 extern "C" int nbk_attention_bwd_static(const nbk_attn_desc* d, const nbk_attn_tensor* q,
                                         const nbk_attn_tensor* k, const nbk_attn_tensor* v,
-                                        const nbk_attn_tensor* o, const void* lse,
+                                        const nbk_attn_tensor* o, const nbk_attn_tensor* o_lo,
+                                        const void* lse,
                                         const nbk_attn_tensor* dout, const nbk_attn_tensor* dq,
                                         const nbk_attn_tensor* dk, const nbk_attn_tensor* dv,
                                         void* stream) {
   AttnArgs a = {};
-  int rc = attn_bwd_args(d, q, k, v, o, lse, dout, dq, dk, dv, &a);
+  int rc = attn_bwd_args(d, q, k, v, o, o_lo, lse, dout, dq, dk, dv, &a);
   if (rc) return rc;
   const int64_t rows = d->B * d->H * d->S;
   NBK_REQUIRE(rows <= NBK_ATTN_STATIC_ROWS,

@@ -9,7 +9,9 @@ log-sum-exp the forward keeps.
 
 ``FusedAttentionOp`` takes heads-first tensors ``[B, H, S, hd]`` (what
 ``MultiHeadAttention`` passes, nabla/nn/modules/layers.py) and returns
-``(output, lse)``.  ``fused_attention_applies`` says whether the kernels cover a call;
+``(output, lse, remainder)``: the third result is what rounding the output to bf16 cut off,
+kept for the backward pass, whose row sums ``sum(d output * output)`` need more digits than
+bf16 holds (a forward pass that nobody differentiates does not compute it).  ``fused_attention_applies`` says whether the kernels cover a call;
 ``scaled_dot_product_attention`` keeps the composition of primitive ops for every other
 case.  Second-order derivatives go through primitive ops as well: the VJP rule of the
 gradient op differentiates the matmul / softmax expression of the same gradients.
@@ -50,19 +52,19 @@ class FusedAttentionOp(Operation):
     def compute_physical_shape(self, args, kwargs, output_sharding=None):
         q = args[0]
         shape = tuple(q.shape)
-        return [shape, shape[:-1]], [q.dtype, DType.float32], [q.device, q.device]
+        return [shape, shape[:-1], shape], [q.dtype, DType.float32, q.dtype], [q.device] * 3
 
     def kernel(self, args, kwargs):
         return list(ir.attention(args[0], args[1], args[2], kwargs["scale"], kwargs["is_causal"]))
 
     def vjp_rule(self, primals, cotangents, outputs, kwargs):
         q, k, v = primals
-        out, lse = outputs
-        return _fused_attention_grad_op([q, k, v, out, lse, cotangents[0]], dict(kwargs))
+        out, lse, out_lo = outputs
+        return _fused_attention_grad_op([q, k, v, out, lse, out_lo, cotangents[0]], dict(kwargs))
 
 
 class FusedAttentionGradOp(Operation):
-    """(dq, dk, dv) from (q, k, v, output, lse, d output)."""
+    """(dq, dk, dv) from (q, k, v, output, lse, output's rounding remainder, d output)."""
 
     multiple_results = True
 
@@ -76,18 +78,18 @@ class FusedAttentionGradOp(Operation):
         return [shape] * 3, [q.dtype] * 3, [q.device] * 3
 
     def kernel(self, args, kwargs):
-        return list(ir.attention_bwd(*args[:6], kwargs["scale"], kwargs["is_causal"]))
+        return list(ir.attention_bwd(*args[:7], kwargs["scale"], kwargs["is_causal"]))
 
     def vjp_rule(self, primals, cotangents, outputs, kwargs):
         # As a function of (q, k, v, d output) these gradients equal the ones the primitive ops
         # give (output and lse are themselves functions of q, k, v), so the second-order rule
         # differentiates that expression.
         from ..transforms.vjp import vjp
-        q, k, v, _, _, g = primals
+        q, k, v, _, _, _, g = primals
         scale, causal = kwargs["scale"], kwargs["is_causal"]
         _, pull = vjp(lambda q, k, v, g: tuple(_composite_vjp(q, k, v, g, scale, causal)), q, k, v, g)
         dq, dk, dv, dg = pull(tuple(cotangents))
-        return [dq, dk, dv, None, None, dg]
+        return [dq, dk, dv, None, None, None, dg]
 
 
 def _composite_vjp(q, k, v, g, scale, causal):

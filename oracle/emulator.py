@@ -449,6 +449,9 @@ def _attention(kind, a, mem):
         dst = _view(mem, a["o"])
         dst.copy_(o.float().to(dst.dtype))
         _view(mem, a["lse"]).copy_(lse.float())
+        if a.get("o_lo") is not None:  # what the rounding of o cut off, rounded the same way
+            lo = _view(mem, a["o_lo"])
+            lo.copy_((o.float() - dst.float()).to(lo.dtype))
         return
     q, k, v = (t.clone().requires_grad_(True) for t in (q, k, v))
     o, _ = forward(q, k, v)

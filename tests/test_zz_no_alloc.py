@@ -28,15 +28,16 @@ def _both_ways(lib, L, shape, causal, seed):
     lse = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
     d = lib.AttnDesc()
     d.B, d.H, d.S, d.hd, d.scale, d.causal, d.dtype = B, H, S, hd, 1.0 / math.sqrt(hd), int(causal), 1
-    tq, tk, tv, to, tg = (_desc(lib, t) for t in (q, k, v, o, g))
+    o_lo = torch.empty_like(q)
+    tq, tk, tv, to, tg, tol = (_desc(lib, t) for t in (q, k, v, o, g, o_lo))
     print(f"attention fwd {shape} causal={causal}", flush=True)
     lib.check(L.nbk_attention_fwd(C.byref(d), C.byref(tq), C.byref(tk), C.byref(tv), C.byref(to),
-                                  C.c_void_p(lse.data_ptr()), st))
+                                  C.byref(tol), C.c_void_p(lse.data_ptr()), st))
     want = [torch.full(shape, float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(3)]
     ws = torch.empty(L.nbk_attention_bwd_workspace(C.byref(d)), dtype=torch.uint8, device="cuda")
     print(f"nbk_attention_bwd {shape}", flush=True)
     lib.check(L.nbk_attention_bwd(C.byref(d), C.byref(tq), C.byref(tk), C.byref(tv), C.byref(to),
-                                  C.c_void_p(lse.data_ptr()), C.byref(tg),
+                                  C.byref(tol), C.c_void_p(lse.data_ptr()), C.byref(tg),
                                   *[C.byref(_desc(lib, t)) for t in want],
                                   C.c_void_p(ws.data_ptr()), ws.numel(), st))
     got = [torch.full(shape, float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(3)]
@@ -44,7 +45,7 @@ def _both_ways(lib, L, shape, causal, seed):
     before = torch.cuda.memory_allocated()
     print(f"nbk_attention_bwd_static {shape}", flush=True)
     lib.check(L.nbk_attention_bwd_static(C.byref(d), C.byref(tq), C.byref(tk), C.byref(tv), C.byref(to),
-                                         C.c_void_p(lse.data_ptr()), C.byref(tg),
+                                         C.byref(tol), C.c_void_p(lse.data_ptr()), C.byref(tg),
                                          *[C.byref(_desc(lib, t)) for t in got], st))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
@@ -73,5 +74,5 @@ def test_attention_backward_without_allocation_rejects_what_does_not_fit(hip):
     # launched: the check comes before any kernel, so the tensors need not be that large.
     d.B, d.H, d.S, d.hd, d.scale, d.causal, d.dtype = 8193, 1, 128, 64, 0.125, 1, 1
     with pytest.raises(ValueError, match="exceed"):
-        lib.check(L.nbk_attention_bwd_static(C.byref(d), *([C.byref(a)] * 4), C.c_void_p(lse.data_ptr()),
+        lib.check(L.nbk_attention_bwd_static(C.byref(d), *([C.byref(a)] * 4), None, C.c_void_p(lse.data_ptr()),
                                              *([C.byref(a)] * 4), None))
