@@ -174,6 +174,16 @@ __device__ __forceinline__ at_bf16x8 at_regs_frag(const at_f32x16& s, int t) {
 
 __device__ __forceinline__ float at_xhalf(float v) { return __shfl_xor(v, 32, 64); }
 
+// acc + the sum of eight packed bf16 values
+__device__ __forceinline__ float at_sum_bf16x8(at_bf16x8 v, float acc) {
+  const at_u32x4 u = __builtin_bit_cast(at_u32x4, v);
+  const at_bf16x2 ones = __builtin_bit_cast(at_bf16x2, 0x3f803f80u);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(at_bf16x2, u[i]), ones, acc, false);
+  return acc;
+}
+
 // Swizzle of the [rows][16 chunks] tiles that are read both by rows and through the transposing
 // LDS read (the kernels for 128-wide heads; the layout is described at the dK / dV kernel).
 template <int NCH>
@@ -245,15 +255,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   // The output is normalised by the sum of the probabilities as the matrix cores saw them
   // (rounded to bf16), so that it is an exact convex combination of the values: a part common to
   // all values then passes through unchanged, which the backward pass's dP - delta relies on.
-  // That sum comes out of the same MFMAs, with a row of ones in the place of V^T (every row of
-  // l_mm holds it); l_i, the sum before rounding, goes into the log-sum-exp, with which the
-  // probabilities that the backward pass recomputes sum to one as well.
-  at_f32x16 l_mm = (at_f32x16)(0.f);
-  at_bf16x8 ones_frag;
-  {
-    const at_u32x4 u = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-    ones_frag = __builtin_bit_cast(at_bf16x8, u);
-  }
+  // That sum (l_r) is taken from the packed bf16 pairs on their way to the second product, one
+  // v_dot2c_f32_bf16 against a pair of ones each; l_i, the sum before rounding, goes into the
+  // log-sum-exp, with which the probabilities that the backward pass recomputes sum to one too.
+  float l_r = 0.f;
 
   const int n_tiles = g.causal ? (q0 + 128) / 64 : g.S / 64;
   RowT kl;
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
         m_i = m_new;
 #pragma unroll
         for (int d = 0; d < DT; ++d) o_acc[d] *= alpha;
-        l_mm *= alpha;
+        l_r *= alpha;
       }
       float sum = 0.f;
 #pragma unroll
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
           for (int d = 0; d < DT; ++d)
             o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
                                                                o_acc[d], 0, 0, 0);
-          l_mm = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_frag, pf, l_mm, 0, 0, 0);
+          l_r = at_sum_bf16x8(pf, l_r);
         }
     };
     // keys of this tile against the wave's queries: all visible, some, or none
@@ -345,7 +350,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   }
   // normalise and write: register r of tile d is O[my_q][32 d + (r/4)*8 + 4h + r%4]
   l_i += at_xhalf(l_i);
-  const float inv = 1.0f / l_mm[0];
+  l_r += at_xhalf(l_r);
+  const float inv = 1.0f / l_r;
   uint16_t* O = (uint16_t*)g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh + (int64_t)my_q * g.o.ss;
 #pragma unroll
   for (int d = 0; d < DT; ++d)
