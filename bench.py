@@ -424,7 +424,7 @@ def measure(nb, L, ex, w, steps, warmup, with_cpu, host, calibrate_copy=False):
             tf = fl / (ms * 1e-3) / 1e12 if ms else 0.0
             by.append({"kernel": label, "launches": n, "avg_us": round(ms / n * 1e3, 2),
                        "tflops": round(tf, 1), "frac": round(tf / peak, 4)})
-        roofline["by_kernel"] = by[:12]
+        roofline["by_kernel"] = by[:16]
         roofline["counted_flops_per_step"] = sum(g[2] for g in groups.values())
         if row_dur:
             # the fused elementwise / normalisation / loss kernels of the same step against the

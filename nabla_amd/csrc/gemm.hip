@@ -1162,29 +1162,58 @@ __global__ __launch_bounds__(256) void gemm_skinny_k_kernel(const GemmArgs g) {
     }
     return *(const bf16x8*)&u;
   };
+  // The two 32-row bands of a wave's tile are worked off one after the other (not unrolled), so
+  // that one band's accumulators, residual pieces and epilogue registers are all a lane holds:
+  // four workgroups then fit a CU, and the 1024 tiles of an 8192 x 2048 result are resident at
+  // once instead of leaving a quarter of them to a second, mostly empty round.
   // (EPI 4: the residual is on its way before the operands are, one memory latency for both)
-  uint4 pre[TM * (WN / 16)];
-  if constexpr (EPI == 4) gemm_residual_prefetch<TM, WN>(g, m0, n0, wm, wn, lane, pre);
-  bf16x8 fa[TM], fb[TN];
+  bf16x8 fb[TN];
+  uint4 pre[WN / 16];
+  u32x4 b_piece = {0u, 0u, 0u, 0u};
+  if (!B_KC && g.b_vec) {
+    const int k = threadIdx.x >> 4;
+    const int64_t col = n0 + (threadIdx.x & 15) * 8;
+    if (k < g.K && col + 8 <= g.N) b_piece = *(const u32x4*)(B + (int64_t)k * g.b_rs + col);
+  }
+  if constexpr (EPI == 4) gemm_residual_prefetch<1, WN>(g, m0, n0, wm, wn, lane, pre);
+  if (!B_KC && g.b_vec) {
+    // B given as [K][N] with whole 16-byte pieces of its rows readable: the workgroup's 16 x 128
+    // piece goes to LDS k-major (one coalesced 16-byte load per lane, zeros past K and N; it was
+    // requested above, ahead of the first band's residual) and
+    // the fragments come out through the transposing read -- instead of eight strided 2-byte
+    // loads per lane and column block.
+    char* bst = (char*)gemm_lds + 4 * 32 * (64 + 4) * sizeof(float);
+    *(u32x4*)(bst + (threadIdx.x >> 4) * 256 + (threadIdx.x & 15) * 16) = b_piece;
+    __syncthreads();
+    const int p = lane & 15, q = lane >> 4;
+    const char* tr = bst + (8 * (q >> 1) + (p >> 2)) * 256 + (wn + 16 * (q & 1) + 4 * (p & 3)) * 2;
 #pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const s16x4 lo = lds_read_tr(tr + j * 64), hi = lds_read_tr(tr + j * 64 + 4 * 256);
+      const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      fb[j] = *(const bf16x8*)&u;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int64_t col = n0 + wn + j * 32 + li;
+      col = col < g.N ? col : g.N - 1;
+      fb[j] = B_KC ? frag8(B + col * g.b_cs, 1, g.b_vec) : frag8(B + col, g.b_rs, false);
+    }
+  }
+#pragma unroll 1
   for (int i = 0; i < TM; ++i) {
+    if (EPI == 4 && i > 0) gemm_residual_prefetch<1, WN>(g, m0, n0, wm + i * 32, wn, lane, pre);
     int64_t row = m0 + wm + i * 32 + li;
     row = row < g.M ? row : g.M - 1;
-    fa[i] = frag8(A + row * g.a_rs, 1, g.a_vec);
-  }
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int64_t col = n0 + wn + j * 32 + li;
-    col = col < g.N ? col : g.N - 1;
-    fb[j] = B_KC ? frag8(B + col * g.b_cs, 1, g.b_vec) : frag8(B + col, g.b_rs, false);
-  }
-  f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
+    const bf16x8 fa = frag8(A + row * g.a_rs, 1, g.a_vec);
+    f32x16 acc[1][TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], (f32x16)(0.f), 0, 0, 0);
-  gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, 0, wave, lane, EPI == 4 ? pre : nullptr);
+      acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[j], (f32x16)(0.f), 0, 0, 0);
+    gemm_epilogue<1, TN, WN, true, EPI>(acc, g, m0, n0, wm + i * 32, wn, 0, wave, lane,
+                                        EPI == 4 ? pre : nullptr);
+  }
 }
 
 // ------------------------------------------------------------------- bf16, N <= 32
@@ -1211,8 +1240,6 @@ __global__ __launch_bounds__(SKN_WAVES * 64) void gemm_skinny_n_kernel(const Gem
   const uint16_t* A = (const uint16_t*)g.A;
   const uint16_t* B = (const uint16_t*)g.B;
   const int64_t row0 = (int64_t)blockIdx.x * 32;
-  const int64_t arow = row0 + li < g.M ? row0 + li : g.M - 1;
-  const uint16_t* ap = A + arow * g.a_rs + 8 * kg;
   // this wave's 64-wide K chunks
   const int chunks = (int)(g.K >> 6);
   const int per = (chunks + SKN_WAVES - 1) / SKN_WAVES;
@@ -1227,14 +1254,7 @@ __global__ __launch_bounds__(SKN_WAVES * 64) void gemm_skinny_n_kernel(const Gem
     const int64_t col = li < g.N ? li : g.N - 1;
     bp = B + col * g.b_cs + 8 * kg;
   } else {
-    // stage rows [64 c_begin, 64 c_end) of B; a k-row holds N / 8 chunks (pitch_chunks >= that)
-    const int nch = (int)(g.N >> 3);
-    const int rows = (c_end - c_begin) * 64;
-    for (int t = lane; t < rows * nch; t += 64) {
-      const int k = t / nch, c = t - k * nch;
-      const int64_t gk = (int64_t)c_begin * 64 + k;
-      *(u32x4*)(stage + (size_t)gk * pitch + c * 16) = *(const u32x4*)(B + gk * g.b_rs + c * 8);
-    }
+    // (rows [64 c_begin, 64 c_end) of B are staged below, behind the first requests for A)
     // lane p of group q = lane / 16: k-row 8 (q / 2) + p / 4, columns 16 (q % 2) + 4 (p % 4) .. + 4
     // (every lane of a group takes part in the exchange, also those that point at padding)
     const int p = lane & 15, q = lane >> 4;
@@ -1242,40 +1262,105 @@ __global__ __launch_bounds__(SKN_WAVES * 64) void gemm_skinny_n_kernel(const Gem
     tr_ptr = stage + (8 * (q >> 1) + (p >> 2)) * pitch + col0 * 2;
   }
   f32x16 acc = (f32x16)(0.f);
-  // the rows of the next chunk are requested before the MFMAs of this one
-  u32x4 an[4], bn[4];
-  auto fetch = [&](int c) {
+  // A streams through a 4 KB slab per wave (the bytes that later hold this wave's partial tile):
+  // a 32-row x 64-k chunk arrives in four fully coalesced loads (eight lanes per 128-byte row
+  // piece; fetching the 32-byte pieces of 32 rows that an MFMA fragment consists of straight
+  // from memory runs at a quarter of that rate), is written to the slab swizzled and read back
+  // as fragments.  The slab belongs to one wave, whose LDS accesses execute in order, so no
+  // workgroup barrier is involved.  Three chunks are in flight in registers.
+  u32x4* slab = (u32x4*)(red + wave * 16 * 64);
+  const int lrow = lane >> 3, lch = lane & 7;
+  const uint16_t* arow_p[4];
+  int w_at[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int r = p * 8 + lrow;
+    const int64_t gr = row0 + r < g.M ? row0 + r : g.M - 1;
+    arow_p[p] = A + gr * g.a_rs + 8 * lch;
+    w_at[p] = r * 8 + (lch ^ dl_kc_xor<false>(r));
+  }
+  const int r_at = li * 8, r_x = dl_kc_xor<false>(li);
+  constexpr int AHEAD = 3;
+  u32x4 an[AHEAD][4], bn[AHEAD][4];
+  auto fetch = [&](auto slot, int c) {
+    constexpr int J = decltype(slot)::value;
     const int64_t k0 = (int64_t)c * 64;
 #pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) an[s4] = *(const u32x4*)(ap + k0 + 16 * s4);
+    for (int p = 0; p < 4; ++p) an[J][p] = *(const u32x4*)(arow_p[p] + k0);
     if (B_KC) {
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) bn[s4] = *(const u32x4*)(bp + k0 + 16 * s4);
+      for (int s4 = 0; s4 < 4; ++s4) bn[J][s4] = *(const u32x4*)(bp + k0 + 16 * s4);
     }
   };
-  if (c_begin < c_end) fetch(c_begin);
-  for (int c = c_begin; c < c_end; ++c) {
-    const int64_t k0 = (int64_t)c * 64;
-    bf16x8 fa[4], fb[4];
+  static_for<AHEAD>([&](auto j) {
+    if (c_begin + decltype(j)::value < c_end) fetch(j, c_begin + decltype(j)::value);
+  });
+  if (!B_KC) {
+    // stage rows [64 c_begin, 64 c_end) of B; a k-row holds N / 8 chunks (pitch_chunks >= that);
+    // four pieces per lane are on their way at a time
+    const int nch = (int)(g.N >> 3);
+    const int total = (c_end - c_begin) * 64 * nch;
+    for (int t0 = 0; t0 < total; t0 += 256) {
+      u32x4 piece[4];
 #pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) fa[s4] = *(const bf16x8*)&an[s4];
-    if (B_KC) {
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * 64 + lane;
+        const int k = t / nch, c = t - k * nch;
+        const int64_t gk = (int64_t)c_begin * 64 + k;
+        if (t < total) piece[u] = *(const u32x4*)(B + gk * g.b_rs + c * 8);
+      }
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) fb[s4] = *(const bf16x8*)&bn[s4];
-    } else {
-#pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) {
-        const char* a0 = tr_ptr + (k0 + 16 * s4) * pitch;
-        const s16x4 lo = lds_read_tr(a0), hi = lds_read_tr(a0 + 4 * pitch);
-        const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        fb[s4] = *(const bf16x8*)&u;
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * 64 + lane;
+        const int k = t / nch, c = t - k * nch;
+        const int64_t gk = (int64_t)c_begin * 64 + k;
+        if (t < total) *(u32x4*)(stage + (size_t)gk * pitch + c * 16) = piece[u];
       }
     }
-    if (c + 1 < c_end) fetch(c + 1);
-#pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s4], fb[s4], acc, 0, 0, 0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
+  for (int c = c_begin; c < c_end; c += AHEAD) {
+    static_for<AHEAD>([&](auto j) {
+      constexpr int J = decltype(j)::value;
+      const int cc = c + J;
+      if (cc < c_end) {  // (uniform over the wave)
+        const int64_t k0 = (int64_t)cc * 64;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) slab[w_at[p]] = an[J][p];
+        bf16x8 fa[4], fb[4];
+        if (B_KC) {
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) fb[s4] = *(const bf16x8*)&bn[J][s4];
+        } else {
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) {
+            const char* a0 = tr_ptr + (k0 + 16 * s4) * pitch;
+            const s16x4 lo = lds_read_tr(a0), hi = lds_read_tr(a0 + 4 * pitch);
+            const s16x8 u = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            fb[s4] = *(const bf16x8*)&u;
+          }
+        }
+        if (cc + AHEAD < c_end) fetch(j, cc + AHEAD);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+          const u32x4 u = slab[r_at + ((2 * s4 + kg) ^ r_x)];
+          fa[s4] = *(const bf16x8*)&u;
+        }
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s4], fb[s4], acc, 0, 0, 0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+    });
+  }
+  // (the slab is this wave's part of the reduction area: its last fragments are in registers)
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
   __syncthreads();
@@ -1725,11 +1810,13 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
       (d->K == 16 ? a.a_vec : d->K == 8 && (d->a_rs % 8 == 0) && ((uintptr_t)d->A & 15) == 0)) {
     // (the vector path reads whole 16-byte pieces of A rows: K = 16 or 8)
     a.a_vec = 1;
-    a.b_vec = bkc && (d->K == 16 ? a.b_vec : (d->b_cs % 8 == 0) && ((uintptr_t)d->B & 15) == 0);
+    // (K-contiguous B: whole fragments from memory; row-contiguous B: whole row pieces into LDS)
+    a.b_vec = bkc ? (d->K == 16 ? a.b_vec : (d->b_cs % 8 == 0) && ((uintptr_t)d->B & 15) == 0)
+                  : (d->b_cs == 1 && d->b_rs % 8 == 0 && ((uintptr_t)d->B & 15) == 0);
     a.tiles_m = (int)((d->M + 127) / 128);
     a.tiles_n = (int)((d->N + 127) / 128);
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
-    const size_t lds = 4 * 32 * (size_t)(64 + 4) * sizeof(float);
+    const size_t lds = 4 * 32 * (size_t)(64 + 4) * sizeof(float) + 16 * 256;  // slabs + a B piece
     // 0 plain; 3 a bias and / or an added residual (the adapter's update on top of the base
     // product: all memory traffic, so the lean epilogue that keeps four waves per SIMD); 2 the rest
     const bool any = a.bias != nullptr || a.residual != nullptr || a.act != NBK_ACT_NONE;
