@@ -176,11 +176,15 @@ __device__ __forceinline__ float at_xhalf(float v) { return __shfl_xor(v, 32, 64
 
 // acc + the sum of eight packed bf16 values
 __device__ __forceinline__ float at_sum_bf16x8(at_bf16x8 v, float acc) {
+  // (written as the instruction itself: __builtin_amdgcn_fdot2_f32_bf16 in an unrolled loop over
+  // the elements of a vector came out of hipcc 7.2 as four reads of the first element)
   const at_u32x4 u = __builtin_bit_cast(at_u32x4, v);
-  const at_bf16x2 ones = __builtin_bit_cast(at_bf16x2, 0x3f803f80u);
+  const uint32_t ones = 0x3f803f80u;  // two bf16 ones
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(at_bf16x2, u[i]), ones, acc, false);
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t w = u[i];
+    asm("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(acc) : "v"(ones), "v"(w));
+  }
   return acc;
 }
 
@@ -766,35 +770,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_tr_kernel(const AttnArgs g)
   const int wq0 = q0 + wave * 32;  // first query of the wave
   const float c = g.scale * AT_LOG2E;
 
-  // delta[q] = sum_d dO[q, d] O[q, d] comes out of the dO fragments this kernel loads anyway and
-  // the matching pieces of O (a lane pair holds one row); it is left in g.delta for the dK / dV
-  // kernel, which runs after this one.
-  // With the forward pass's second tensor (what bf16 O lost) the sum runs over O to about 16
-  // bits: a delta off by 2^-9 of |dO| |O| would be a visible share of dP - delta wherever the
-  // keys a query sees have values with a large common part.
-  const uint16_t* O = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh;
-  const uint16_t* OL = g.o_lo.p == nullptr ? nullptr
-                                           : g.o_lo.p + (int64_t)b * g.o_lo.sb + (int64_t)hh * g.o_lo.sh;
-  at_bf16x8 qf[KSTEPS], dof[KSTEPS];
-  float my_delta = 0.f;
-#pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
-    const at_u32x4 uq = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
-    const at_u32x4 ud = *(const at_u32x4*)(DO + (int64_t)my_q * g.dout.ss + s * 16 + h * 8);
-    const at_u32x4 uo = *(const at_u32x4*)(O + (int64_t)my_q * g.o.ss + s * 16 + h * 8);
-    at_u32x4 ul = {0u, 0u, 0u, 0u};
-    if (OL != nullptr) ul = *(const at_u32x4*)(OL + (int64_t)my_q * g.o_lo.ss + s * 16 + h * 8);
-    qf[s] = __builtin_bit_cast(at_bf16x8, uq);
-    dof[s] = __builtin_bit_cast(at_bf16x8, ud);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      my_delta += (__uint_as_float(uo[e] << 16) + __uint_as_float(ul[e] << 16)) * __uint_as_float(ud[e] << 16);
-      my_delta += (__uint_as_float(uo[e] & 0xffff0000u) + __uint_as_float(ul[e] & 0xffff0000u)) *
-                  __uint_as_float(ud[e] & 0xffff0000u);
-    }
-  }
-  my_delta += at_xhalf(my_delta);
-  if (h == 0) g.delta[((int64_t)b * g.H + hh) * g.S + my_q] = my_delta;
   at_f32x16 dq_acc[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d) dq_acc[d] = (at_f32x16)(0.f);
@@ -838,9 +813,49 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_q_tr_kernel(const AttnArgs g)
     return at_tr_pair(base + tr_lo + ((tr_x_lo ^ (dd << 2)) << 4), base + tr_hi + ((tr_x_hi ^ (dd << 2)) << 4));
   };
 
+  // delta[q] = sum_d dO[q, d] O[q, d] comes out of the dO fragments this kernel loads anyway and
+  // the matching pieces of O (a lane pair holds one row); it is left in g.delta for the dK / dV
+  // kernel, which runs after this one.
+  // With the forward pass's second tensor (what bf16 O lost) the sum runs over O to about 16
+  // bits: a delta off by 2^-9 of |dO| |O| would be a visible share of dP - delta wherever the
+  // keys a query sees have values with a large common part.
+  // Order of the requests: the first K / V tile, then Q and dO, then O and its remainder -- the
+  // tile is waited for first (to go to LDS), and the pieces of O, which only delta needs, are
+  // still on their way while the tile is stored and the workgroup meets at the barrier.
+  const uint16_t* O = g.o.p + (int64_t)b * g.o.sb + (int64_t)hh * g.o.sh;
+  const uint16_t* OL = g.o_lo.p == nullptr ? nullptr
+                                           : g.o_lo.p + (int64_t)b * g.o_lo.sb + (int64_t)hh * g.o_lo.sh;
+  at_bf16x8 qf[KSTEPS], dof[KSTEPS];
+  at_u32x4 uo[KSTEPS], ul[KSTEPS];
   load_all(0);
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const at_u32x4 uq = *(const at_u32x4*)(Q + (int64_t)my_q * g.q.ss + s * 16 + h * 8);
+    const at_u32x4 ud = *(const at_u32x4*)(DO + (int64_t)my_q * g.dout.ss + s * 16 + h * 8);
+    qf[s] = __builtin_bit_cast(at_bf16x8, uq);
+    dof[s] = __builtin_bit_cast(at_bf16x8, ud);
+  }
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    uo[s] = *(const at_u32x4*)(O + (int64_t)my_q * g.o.ss + s * 16 + h * 8);
+    ul[s] = (at_u32x4){0u, 0u, 0u, 0u};
+    if (OL != nullptr) ul[s] = *(const at_u32x4*)(OL + (int64_t)my_q * g.o_lo.ss + s * 16 + h * 8);
+  }
   store_all(0);
   __syncthreads();
+  float my_delta = 0.f;
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const at_u32x4 ud = __builtin_bit_cast(at_u32x4, dof[s]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      my_delta += (__uint_as_float(uo[s][e] << 16) + __uint_as_float(ul[s][e] << 16)) * __uint_as_float(ud[e] << 16);
+      my_delta += (__uint_as_float(uo[s][e] & 0xffff0000u) + __uint_as_float(ul[s][e] & 0xffff0000u)) *
+                  __uint_as_float(ud[e] & 0xffff0000u);
+    }
+  }
+  my_delta += at_xhalf(my_delta);
+  if (h == 0) g.delta[((int64_t)b * g.H + hh) * g.S + my_q] = my_delta;
   for (int kt = 0; kt < n_tiles; ++kt) {
     const int cur = kt & 1;
     const bool more = kt + 1 < n_tiles;
