@@ -29,6 +29,14 @@ class NoBatchRule(Exception):
     """The op has no batching rule (or not for this combination of arguments)."""
 
 
+class Done:
+    """What a rule returns when it has computed the batched result itself (plain tensors with the
+    hidden dimensions in front), as a composition of ops that do have kernels for it."""
+
+    def __init__(self, outs):
+        self.outs = list(outs)
+
+
 # sizes of the hidden dimensions of the vmap calls that are being traced, outermost first
 # (per context: two threads that trace at the same time do not see each other's levels)
 _LEVELS: ContextVar[tuple[int, ...]] = ContextVar("vmap_levels", default=())
@@ -167,13 +175,49 @@ def _rule_fold_leading(op, args, kwargs, bd, sizes):
 
 
 def _rule_conv(op, args, kwargs, bd, sizes):
-    # the images carry the batch; one filter for all of them
     if isinstance(args[1], BatchedTensor):
-        raise NoBatchRule("convolution with a mapped filter")
-    # a bias (third operand) is one vector per output channel for every image
+        return _conv_with_a_filter_per_element(args, kwargs, bd, sizes)
+    # the images carry the batch; one filter for all of them.  A bias (third operand) is one
+    # vector per output channel for every image
     if any(isinstance(a, BatchedTensor) for a in args[2:]):
         raise NoBatchRule("convolution with a mapped bias")
     return [_fold(lift(args[0], bd, sizes), bd), args[1]] + list(args[2:]), dict(kwargs), _unfold(sizes)
+
+
+def _conv_with_a_filter_per_element(args, kwargs, bd, sizes):
+    """conv2d where every element of the batch has a filter of its own (what per-example
+    gradients with respect to a shared filter look like once the filter has been lifted to the
+    batch): the kernels take one filter per launch, so the windows are laid out explicitly --
+    pad, one shifted view of the images per filter tap, joined along the channel axis -- and
+    the contraction over (tap, channel) is ONE batched matrix product whose batch is the hidden
+    axis.  Every op of that composition has a kernel and a VJP rule for batched operands, so
+    the launches do not grow with the batch, forward or backward.  Unit strides only (a strided
+    window is not a view here): other strides leave it to the element-by-element map."""
+    from . import binary, view
+    x, w = args[0], args[1]
+    (sh, sw), (pt, pb, pl, pr) = kwargs["stride"], kwargs["padding"]
+    if (sh, sw) != (1, 1):
+        raise NoBatchRule("convolution with a mapped filter and a stride")
+    xl, wl = lift(x, bd, sizes), lift(w, bd, sizes)
+    n, hh, ww, cin = xl.shape[bd:]
+    r, s_, _, cout = wl.shape[bd:]
+    ho, wo = hh + pt + pb - r + 1, ww + pl + pr - s_ + 1
+    lead = tuple(sizes)
+    if pt or pb or pl or pr:
+        xl = view.pad(xl, [(0, 0)] * (bd + 1) + [(pt, pb), (pl, pr), (0, 0)])
+    taps = []
+    for i in range(r):
+        for j in range(s_):
+            start = (0,) * (bd + 1) + (i, j, 0)
+            taps.append(view.slice_tensor(xl, start=start, size=lead + (n, ho, wo, cin)))
+    cols = taps[0] if len(taps) == 1 else view.concatenate(taps, axis=-1)
+    cols = view.reshape(cols, lead + (n * ho * wo, r * s_ * cin))
+    y = binary.matmul(cols, view.reshape(wl, lead + (r * s_ * cin, cout)))
+    y = view.reshape(y, lead + (n, ho, wo, cout))
+    if len(args) > 2:
+        b = lift(args[2], bd, sizes)                       # [*sizes, Cout]
+        y = binary.add(y, view.reshape(b, lead + (1, 1, 1, cout)))
+    return Done([y])
 
 
 def _rule_gather(op, args, kwargs, bd, sizes):
@@ -182,7 +226,7 @@ def _rule_gather(op, args, kwargs, bd, sizes):
     from . import view
     x, idx = args
     if isinstance(x, BatchedTensor):
-        raise NoBatchRule("gather from a mapped table")
+        return _gather_from_a_table_per_element(x, idx, kwargs, bd, sizes)
     rank = len(x.shape)
     axis = int(kwargs.get("axis", 0))
     axis = axis + rank if axis < 0 else axis
@@ -195,6 +239,70 @@ def _rule_gather(op, args, kwargs, bd, sizes):
     return [x, lift(idx, bd, sizes)], dict(kwargs, axis=axis), post
 
 
+def _row_numbers(idx: Tensor, rows: int, bd: int, sizes) -> Tensor:
+    """Indices into the rows of one table per batch element -> indices into all the tables laid
+    end to end: ``idx + element * rows`` (negative indices wrap once first, as gather does), and
+    whatever falls outside its own table goes to the first row past the last table, where the
+    kernels' range check sees it."""
+    from . import binary, comparison, control_flow, creation, view
+    from ..core.dtype import DType
+    il = lift(idx, bd, sizes)
+    if il.dtype is not DType.int64:
+        from .unary import cast
+        il = cast(il, DType.int64)
+    total = _prod(sizes)
+    n = _prod(il.shape[bd:])
+    il = view.reshape(il, (total, n))
+    const = lambda v: creation.full((total, n), v, dtype=DType.int64)  # (int64 throughout: exact)
+    wrapped = control_flow.where(comparison.less(il, const(0)), binary.add(il, const(rows)), il)
+    first = view.broadcast_to(view.reshape(creation.arange(0, total * rows, rows, dtype=DType.int64),
+                                           (total, 1)), (total, n))
+    inside = comparison.logical_and(comparison.greater_equal(wrapped, const(0)),
+                                    comparison.less(wrapped, const(rows)))
+    outside = control_flow.where(inside, binary.add(wrapped, first), const(total * rows))
+    return view.reshape(outside, (total * n,))
+
+
+def _gather_from_a_table_per_element(x, idx, kwargs, bd, sizes):
+    """gather where every element of the batch has a table of its own: the tables are laid end
+    to end (a view) and the indices shifted to their own table, so one launch serves the batch.
+    Along the first axis only (what an embedding does); other axes are mapped element by element."""
+    from . import view
+    xl = lift(x, bd, sizes)
+    rank = len(xl.shape) - bd
+    axis = int(kwargs.get("axis", 0))
+    axis = axis + rank if axis < 0 else axis
+    if axis != 0:
+        raise NoBatchRule("gather from a mapped table along an inner axis")
+    rows, rest = xl.shape[bd], tuple(xl.shape[bd + 1:])
+    total = _prod(sizes)
+    idx_shape = tuple(plain(idx).shape[batch_dims_of(idx):])
+    flat_idx = _row_numbers(idx, rows, bd, sizes)
+    out = view.gather(view.reshape(xl, (total * rows,) + rest), flat_idx, axis=0)
+    return Done([view.reshape(out, tuple(sizes) + idx_shape + rest)])
+
+
+def _rule_scatter(op, args, kwargs, bd, sizes):
+    """scatter with mapped operands: as for a gather from a table per element, the tables are
+    laid end to end and the indices shifted; rows of different elements never meet, and within
+    one element the updates keep their order, so a row named twice still takes its last update."""
+    from . import view
+    x, idx, upd = args
+    xl, ul = lift(x, bd, sizes), lift(upd, bd, sizes)
+    rank = len(xl.shape) - bd
+    axis = int(kwargs.get("axis", 0))
+    axis = axis + rank if axis < 0 else axis
+    if axis != 0:
+        raise NoBatchRule("scatter along an inner axis with mapped operands")
+    rows, rest = xl.shape[bd], tuple(xl.shape[bd + 1:])
+    total = _prod(sizes)
+    flat_idx = _row_numbers(idx, rows, bd, sizes)
+    n = flat_idx.shape[0] // total
+    out = view.scatter(view.reshape(xl, (total * rows,) + rest), flat_idx,
+                       view.reshape(ul, (total * n,) + rest), axis=0)
+    return Done([view.reshape(out, tuple(sizes) + (rows,) + rest)])
+
+
 def _rules() -> list[tuple[type, Callable]]:
     from . import (attention, binary, control_flow, convolution, normalization, pooling, unary, view,
                    xent)
@@ -202,6 +310,7 @@ def _rules() -> list[tuple[type, Callable]]:
 
     return [
         (view.GatherOp, _rule_gather),
+        (view.ScatterOp, _rule_scatter),
         (convolution.Conv2DOp, _rule_conv),
         (pooling.MaxPool2DOp, _rule_fold_leading),
         (pooling.AvgPool2DOp, _rule_fold_leading),
@@ -252,6 +361,8 @@ def dispatch(op, args: list, kwargs: dict) -> list:
                     raise ValueError(f"vmap: mapped axes of sizes {sizes[i]} and {d} meet in '{op.name}'")
                 sizes[i] = d
     got = rule(op, list(args), dict(kwargs or {}), bd, tuple(sizes))
+    if isinstance(got, Done):  # the rule computed the result itself, out of other ops
+        return [BatchedTensor(o, bd) for o in got.outs]
     outs = op(got[0], got[1])
     if len(got) > 2:
         outs = got[2](outs)

@@ -801,6 +801,49 @@ def test_vmap_batched_per_example_gradients_of_a_block_on_device(hip):
     assert relerr(got["w2"], want2) <= 5e-5 and relerr(got["w1"], want1) <= 5e-5
 
 
+def test_vmap_per_example_gradients_of_the_cnn_on_device(hip):
+    """Per-example gradients of the CNN step (conv - relu - conv - relu - maxpool - conv - relu -
+    mean - linear - cross-entropy) with respect to all eight shared parameters, as
+    vmap(grad(loss), in_axes=(None, 0, 0)): the filters are lifted to the batch, so every
+    convolution has a filter per element (windows laid out, one batched product), and the
+    whole thing is one forward and one backward pass whose launches do not grow with the
+    batch.  Values: the float64 oracle on each example alone."""
+    from nabla_amd.core import engine
+    F = nb.nn.functional
+    names = oc.C4_PARAMS
+
+    def one(params, img, label):
+        logits = nb.workloads.c4_logits(params, nb.unsqueeze(img, 0))
+        return F.cross_entropy_loss(logits, nb.unsqueeze(label, 0))
+
+    steps = {}
+    for n in (4, 12):
+        t = oc.c4_inputs(batch=n, hw=8, c=(3, 8, 16, 24), classes=5, seed=40 + n)
+        rng = np.random.default_rng(n)
+        for k in ("c1b", "c2b", "c3b", "bl"):
+            t[k] = (0.1 * rng.standard_normal(t[k].shape)).astype(np.float32)
+        params = {k: T(t[k]) for k in names}
+        engine.clear_plan_cache()
+        calls = []
+
+        def counted(p, img, label):
+            calls.append(1)
+            return nb.grad(one)(p, img, label)
+
+        g = nb.vmap(counted, in_axes=(None, 0, 0))(params, T(t["img"]), T(t["labels"]))
+        got = {k: g[k].numpy() for k in names}
+        steps[n] = sum(len(bp.plan.steps) for bp in engine._PLAN_CACHE.values())
+        engine.clear_plan_cache()
+        assert len(calls) == 1, "the function was mapped element by element"
+        for i in range(n):
+            single = dict(t, img=t["img"][i:i + 1], labels=t["labels"][i:i + 1])
+            _, wg, _, _ = oc.c4_reference(single)
+            for k in names:
+                assert got[k].shape == (n,) + wg[k].shape
+                assert relerr(got[k][i], wg[k], floor=1e-6) < 5e-5, (n, i, k, relerr(got[k][i], wg[k]))
+    assert steps[4] == steps[12], steps
+
+
 def test_small_composite_ops_on_device(hip):
     """trunc / floor / is_nan / is_inf / flip exactly and log1p to fp32 rounding on the device
     (NaN and infinity must survive the kernels' compare instructions)."""

@@ -190,18 +190,71 @@ def test_nested_batched_maps_and_vjp_inside(emulator):
 
 
 def test_ops_without_a_batching_rule_fall_back_to_the_map(emulator):
-    """A gather from a table that is itself mapped has no batching rule: the function is tried
-    once, then mapped element by element, with the right result either way."""
-    tables, idx = RNG.standard_normal((3, 7, 2)), np.array([1, 6, 3, 3])
+    """A gather along an inner axis of a table that is itself mapped has no batching rule: the
+    function is tried once, then mapped element by element, with the right result either way."""
+    tables, idx = RNG.standard_normal((3, 2, 7)), np.array([1, 6, 3, 3])
     calls = []
 
     def look_up(tab):
         calls.append(1)
-        return nb.gather(tab, nb.Tensor.constant(idx.astype(np.int64)), axis=0) * 2.0
+        return nb.gather(tab, nb.Tensor.constant(idx.astype(np.int64)), axis=1) * 2.0
 
     got = nb.vmap(look_up)(T(tables))
     assert len(calls) == 1 + 3  # the batched attempt, then one call per element
-    close(got, 2.0 * tables[:, idx])
+    close(got, 2.0 * tables[:, :, idx])
+
+
+def test_tables_and_filters_of_their_own_per_element(emulator):
+    """Rules for operands that used to force the element-by-element map: a convolution whose
+    filter (and bias) is mapped, a gather from a mapped table (mapped or shared indices, negative
+    ones wrapping inside their own table), a scatter with mapped operands (a row named twice
+    keeps its last update).  One call of the function each, values against numpy and against
+    the element-by-element map, gradients included: per-example gradients with respect to a
+    shared filter are one batched pass."""
+    img, filt = RNG.standard_normal((3, 2, 6, 6, 4)), RNG.standard_normal((3, 3, 3, 4, 5))
+    bias = RNG.standard_normal((3, 5))
+
+    def check(fn, *args, **kw):
+        got = _both_ways(fn, *args, **kw)
+        (batched, n_b), (mapped, n_m) = got[True], got[False]
+        assert n_b == 1 and n_m == 3, (n_b, n_m)
+        for a, b in zip(batched, mapped):
+            assert a.shape == b.shape
+            np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-5)
+        return batched
+
+    check(lambda x, k, b: nb.conv2d(x, k, padding=(1, 1, 0, 2), bias=b), T(img), T(filt), T(bias))
+    check(lambda k: nb.conv2d(T(img[0]), k), T(filt))
+
+    def loss(k, b, x):
+        return nb.reduce_sum(nb.relu(nb.conv2d(x, k, padding=(1, 1, 1, 1), bias=b)) ** 2.0)
+
+    gk, gb = check(nb.grad(loss, argnums=(0, 1)), T(filt[0]), T(bias[0]), T(img), in_axes=(None, None, 0))
+    assert gk.shape == (3, 3, 3, 4, 5) and gb.shape == (3, 5)
+    # a strided convolution with a mapped filter still takes the element-by-element map
+    got = _both_ways(lambda k: nb.conv2d(T(img[0]), k, stride=(2, 1)), T(filt))
+    assert got[True][1] == 1 + 3
+    np.testing.assert_allclose(got[True][0][0], got[False][0][0], rtol=1e-5, atol=1e-5)
+
+    tables = RNG.standard_normal((3, 7, 2))
+    idx = np.array([[1, 6, -1, 3], [0, 0, 2, 5], [6, -7, 3, 3]], dtype=np.int64)
+    I = nb.Tensor.constant(idx)
+    (got,) = check(lambda t, i: nb.gather(t, i, axis=0) * 2.0, T(tables), I)
+    np.testing.assert_allclose(got, 2.0 * np.stack([tables[b][idx[b]] for b in range(3)]), rtol=1e-6)
+    check(lambda t: nb.gather(t, nb.Tensor.constant(idx[0]), axis=0), T(tables))
+    check(nb.grad(lambda t, i: nb.reduce_sum(nb.gather(t, i, axis=0) ** 2.0)), T(tables), I)
+    upd = RNG.standard_normal((3, 4, 2))
+    (got,) = check(lambda t, i, u: nb.scatter(t, i, u, axis=0), T(tables), I, T(upd))
+    want = tables.astype(np.float32).copy()
+    for b in range(3):
+        for j in range(4):
+            want[b, idx[b, j]] = upd[b, j]
+    np.testing.assert_allclose(got, want, rtol=1e-6)
+    # an index outside its own table is an error, not a row of the neighbouring table
+    bad = idx.copy()
+    bad[0, 0] = 7
+    with pytest.raises(IndexError):
+        nb.vmap(lambda t, i: nb.gather(t, i, axis=0))(T(tables), nb.Tensor.constant(bad)).numpy()
 
 
 def test_window_index_and_fused_ops_join_the_hidden_axis(emulator):
