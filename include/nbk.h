@@ -144,11 +144,14 @@ enum nbk_rp_op {
   NBK_OP_DGELU = 50,   /* derivative of the exact GELU: Phi(a) + a * phi(a)    */
   NBK_OP_SIN = 51, NBK_OP_COS = 52, /* unary; the block 16..31 is full             */
   /* Integer registers.  A register is 32 bits; the program decides what they mean.  Values of
-   * int32 / int64 tensors are loaded, held and stored as two's-complement int32 (LDG / LDR /
-   * STG / STR go by the operand's dtype; int64 storage passes through its low 32 bits, sign-
-   * extended on the way out), and these instructions compute on them exactly, wrapping modulo
-   * 2^32.  Floats, bool and uint8 are fp32 in registers.  MOV, WHERE (its payload) and IMM move
-   * bits and serve both; an integer immediate is stored in imm[] by its bit pattern. */
+   * integer tensors are loaded, held and stored as two's-complement int32 (LDG / LDR / STG /
+   * STR go by the operand's dtype), and these instructions compute on them exactly, wrapping
+   * modulo 2^32.  An int64 operand is read SATURATED to the int32 range and written sign-
+   * extended: exact for comparisons with an index or constant strictly inside that range,
+   * which is the one use of int64 tensors the lowering leaves in row programs; arithmetic on
+   * int64 values belongs to nbk_ew_int64.  Floats, bool and uint8 are fp32 in registers.  MOV,
+   * WHERE (its payload) and IMM move bits and serve both; an integer immediate is stored in
+   * imm[] by its bit pattern. */
   /* binary on int32 (comparisons produce a float 0 / 1, like their float forms) */
   NBK_OP_IADD = 64, NBK_OP_ISUB = 65, NBK_OP_IMUL = 66, NBK_OP_IMAX = 67, NBK_OP_IMIN = 68,
   NBK_OP_IGT = 69, NBK_OP_IGE = 70, NBK_OP_IEQ = 71, NBK_OP_INE = 72, NBK_OP_ILT = 73,
