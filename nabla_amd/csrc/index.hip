@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256) void ew_int64_kernel(const Ew64Args A) {
 
 extern "C" int nbk_ew_int64(int32_t op, const nbk_tensor* in, const int64_t* imm, int32_t n_in,
                             const nbk_tensor* out, void* stream) {
-  NBK_REQUIRE(in && out && out->ptr, "ew_int64: null pointer");
+  NBK_REQUIRE(in && out, "ew_int64: null pointer");
   NBK_REQUIRE(n_in >= 1 && n_in <= 3, "ew_int64: %d operands", n_in);
   const bool known =
       op == NBK_OP_MOV || op == NBK_OP_TRUNC || op == NBK_OP_NEG || op == NBK_OP_ABS ||
@@ -333,6 +333,8 @@ extern "C" int nbk_ew_int64(int32_t op, const nbk_tensor* in, const int64_t* imm
     A.out_stride[d] = out->stride[d];
     A.n *= out->shape[d];
   }
+  if (A.n == 0) return NBK_OK;  // (nothing to compute: an empty result may come without memory)
+  NBK_REQUIRE(out->ptr != nullptr, "ew_int64: null result pointer");
   for (int k = 0; k < n_in; ++k) {
     if (in[k].ptr == nullptr) {
       NBK_REQUIRE(imm != nullptr, "ew_int64: operand %d has neither memory nor an immediate", k);
@@ -350,7 +352,6 @@ extern "C" int nbk_ew_int64(int32_t op, const nbk_tensor* in, const int64_t* imm
       A.stride[k][d] = in[k].stride[d];
     }
   }
-  if (A.n == 0) return NBK_OK;
   int64_t blocks = (A.n + 255) / 256;
   const int64_t cap = (int64_t)nbk_num_cus() * 16;
   if (blocks > cap) blocks = cap;

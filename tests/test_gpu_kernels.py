@@ -563,3 +563,112 @@ def test_conv_wgrad_workspace_and_fallback(hip):
     scale = ref.abs().max().item()
     assert (dw1.cpu().double() - ref).abs().max().item() <= 1e-5 * scale
     assert (dw2.cpu().double() - ref).abs().max().item() <= 1e-5 * scale
+
+
+def _tensor_desc(lib, t, shape=None, strides=None):
+    d = lib.TensorDesc()
+    d.ptr = t.data_ptr()
+    d.dtype = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2, torch.int32: 3, torch.int64: 4,
+               torch.bool: 5, torch.uint8: 5}[t.dtype]
+    shape = tuple(t.shape) if shape is None else shape
+    strides = tuple(t.stride()) if strides is None else strides
+    d.rank = len(shape)
+    for i, (n, st) in enumerate(zip(shape, strides)):
+        d.shape[i], d.stride[i] = n, st
+    return d
+
+
+def test_int64_elementwise_kernel_through_the_c_abi(hip):
+    """nbk_ew_int64: every operation on values beyond 2^31 and 2^53 against numpy's int64
+    arithmetic (wrapping sums and products, division toward zero, powers modulo 2^64), operands
+    of every integer type, broadcast through zero strides, a permuted operand, immediates, all
+    four kinds of result, a rank-0 and an empty problem, and the argument errors."""
+    from nabla_amd.backend import isa, lib
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(91)
+    shape = (5, 7, 9)
+    a = rng.integers(-2 ** 62, 2 ** 62, shape).astype(np.int64)
+    a.reshape(-1)[:4] = [2 ** 31, -(2 ** 31) - 1, 2 ** 53 + 1, -(2 ** 63)]
+    b = rng.integers(-2 ** 33, 2 ** 33, shape).astype(np.int64)
+    b.reshape(-1)[:4] = [-1, 0, 3, -1]
+    small = rng.integers(0, 6, shape).astype(np.int64)
+
+    def run(fn, ins, out_dtype=torch.int64, imm=None, out_shape=shape):
+        devs = [None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in ins]
+        out = torch.empty(out_shape, dtype=out_dtype, device="cuda")
+        descs = (lib.TensorDesc * len(ins))()
+        for i, t in enumerate(devs):
+            if t is None:
+                descs[i].rank = len(out_shape)
+                continue
+            bshape = tuple(t.shape)
+            strides = tuple(0 if n == 1 and m != 1 else s for n, m, s in zip(bshape, out_shape, t.stride()))
+            descs[i] = _tensor_desc(lib, t, out_shape, strides)
+        imms = (C.c_int64 * len(ins))(*([0] * len(ins)))
+        for i, v in enumerate(imm or []):
+            if v is not None:
+                imms[i] = v
+        od = _tensor_desc(lib, out)
+        lib.check(L.nbk_ew_int64(isa.EW[fn], descs, imms, len(ins), C.byref(od), st))
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(run("add", [a, b]), a + b)
+        np.testing.assert_array_equal(run("sub", [a, b]), a - b)
+        np.testing.assert_array_equal(run("mul", [a, b]), a * b)
+        np.testing.assert_array_equal(run("fma", [a, b, small]), a * b + small)
+        np.testing.assert_array_equal(run("neg", [a]), -a)
+        np.testing.assert_array_equal(run("abs", [a]), np.abs(a))
+        want_pow = np.empty(shape, np.int64)
+        for idx in np.ndindex(shape):
+            v = pow(int(b[idx]), int(small[idx]), 2 ** 64)
+            want_pow[idx] = v - 2 ** 64 if v >= 2 ** 63 else v
+        np.testing.assert_array_equal(run("pow", [b, small]), want_pow)
+    q = np.where(b == 0, 0, np.sign(a) * np.sign(b) * (np.abs(a.astype(object)) // np.maximum(np.abs(b.astype(object)), 1)))
+    q = np.where((a == -(2 ** 63)) & (b == -1), -(2 ** 63), q).astype(np.int64)
+    np.testing.assert_array_equal(run("div", [a, b]), q)
+    np.testing.assert_array_equal(run("relu", [a]), np.maximum(a, 0))
+    np.testing.assert_array_equal(run("max", [a, b]), np.maximum(a, b))
+    np.testing.assert_array_equal(run("min", [a, b]), np.minimum(a, b))
+    for fn, op in (("gt", np.greater), ("ge", np.greater_equal), ("eq", np.equal), ("ne", np.not_equal),
+                   ("lt", np.less), ("le", np.less_equal)):
+        np.testing.assert_array_equal(run(fn, [a, a + (small - 2) * 2 ** 32], torch.bool), op(a, a + (small - 2) * 2 ** 32))
+    np.testing.assert_array_equal(run("where", [small > 2, a, b]), np.where(small > 2, a, b))
+    np.testing.assert_array_equal(run("and", [small, b], torch.bool), (small != 0) & (b != 0))
+    np.testing.assert_array_equal(run("not", [small * 2 ** 40], torch.bool), small == 0)
+    # operand types: int32 and bool widen; a float is cut toward zero
+    i32 = rng.integers(-2 ** 31, 2 ** 31, shape).astype(np.int32)
+    np.testing.assert_array_equal(run("add", [a, i32]), a + i32)
+    f = (rng.standard_normal(shape) * 1e15).astype(np.float32)
+    np.testing.assert_array_equal(run("trunc", [f]), np.trunc(f).astype(np.int64))
+    # results: int32 keeps the low bits, floats round to nearest
+    np.testing.assert_array_equal(run("mov", [a], torch.int32), a.astype(np.int32))
+    np.testing.assert_array_equal(run("mov", [a], torch.float32), a.astype(np.float32))
+    # broadcast operands (zero strides), an immediate, a permuted view
+    row = rng.integers(-2 ** 40, 2 ** 40, (1, 7, 1)).astype(np.int64)
+    np.testing.assert_array_equal(run("add", [a, row]), a + row)
+    np.testing.assert_array_equal(run("mul", [a, None], imm=[None, -3]), a * -3)
+    at = torch.from_numpy(a).cuda()
+    perm = at.permute(2, 0, 1)                                   # [9, 5, 7] view of [5, 7, 9] storage
+    out = torch.empty((9, 5, 7), dtype=torch.int64, device="cuda")
+    descs = (lib.TensorDesc * 2)()
+    descs[0] = _tensor_desc(lib, perm, tuple(perm.shape), tuple(perm.stride()))
+    descs[1].rank = 3
+    imms = (C.c_int64 * 2)(0, 2 ** 40)
+    lib.check(L.nbk_ew_int64(isa.EW["sub"], descs, imms, 2, C.byref(_tensor_desc(lib, out)), st))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), np.transpose(a, (2, 0, 1)) - 2 ** 40)
+    # rank 0 and empty
+    np.testing.assert_array_equal(run("add", [np.int64(2 ** 62), np.int64(2 ** 62)], out_shape=()), np.int64(-(2 ** 63)))
+    assert run("add", [np.zeros((0, 3), np.int64), np.zeros((0, 3), np.int64)], out_shape=(0, 3)).shape == (0, 3)
+    # errors: an operation without an integer form, a wrong operand count, a shape mismatch
+    od = _tensor_desc(lib, out)
+    with pytest.raises(ValueError, match="no 64-bit integer form"):
+        lib.check(L.nbk_ew_int64(isa.EW["exp"], descs, imms, 1, C.byref(od), st))
+    with pytest.raises(ValueError, match="takes 2 operands"):
+        lib.check(L.nbk_ew_int64(isa.EW["add"], descs, imms, 1, C.byref(od), st))
+    bad = _tensor_desc(lib, at)
+    with pytest.raises(ValueError, match="differs from the result"):
+        lib.check(L.nbk_ew_int64(isa.EW["neg"], (lib.TensorDesc * 1)(bad), imms, 1, C.byref(od), st))
