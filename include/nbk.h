@@ -183,8 +183,10 @@ typedef struct nbk_rowprog {
 
 int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream);
 /* 1 if the library carries a straight-line (ahead-of-time specialised) kernel
- * for this program, 0 if the interpreter will run it.  Results are the same
- * either way; setting NBK_ROWPROG_INTERPRET=1 forces the interpreter. */
+ * for this program, 2 if it also carries a hand-scheduled kernel that this launch
+ * (row length, alignment) would take, 0 if the interpreter will run it.  Results
+ * are the same to rounding either way; NBK_ROWPROG_INTERPRET=1 forces the
+ * interpreter, NBK_ROWPROG_HAND=0 the generated kernels. */
 int nbk_rowprog_is_specialized(const nbk_rowprog* prog);
 /* The 64-bit hash (FNV-1a over header, operand classes, instructions, immediates; pointers,
  * strides and extents excluded) by which a program finds its specialised kernel.  That

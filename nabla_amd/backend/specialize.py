@@ -477,6 +477,16 @@ def collect_programs() -> dict[int, dict]:
                     return job()
             return run
 
+        # the loss over a batch too small for its label mask to be recomputed per reader (the
+        # planner keeps one mask below 2^22 elements: the same program in another order)
+        xs = nb.Tensor._from_torch(torch.empty((64, 32000), dtype=bf16))
+        ls = nb.Tensor._from_torch(torch.zeros((64,), dtype=i64))
+
+        def small_batch_loss():
+            loss, g = nb.value_and_grad(lambda z: nb.nn.functional.cross_entropy_loss(z, ls))(xs)
+            return [loss, g]
+
+        jobs.append(small_batch_loss)
         jobs.append(with_flags(jobs[2], FUSED_ATTENTION=False))
         jobs.append(with_flags(jobs[4], FUSED_ATTENTION=False, LORA_LOW_RANK_ORDER=False))
         for job in jobs:

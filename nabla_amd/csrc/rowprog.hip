@@ -463,6 +463,7 @@ struct RpSpec {
   const void* kernel_stream[5];
   const void* kernel_flat;
   const void* kernel_stage16;
+  const rp_hand_entry* hand;
   int block_mode;
   bool lds_attr_set;
   bool lds16_attr_set;
@@ -492,8 +493,14 @@ static RpSpec* rp_find_spec(uint64_t h) {
         e.block_mode = tabs[t][i].block_mode;
         e.lds_attr_set = false;
         e.lds16_attr_set = false;
+        e.hand = nullptr;
         (*g_specs)[tabs[t][i].hash] = e;
       }
+    // (a hand-scheduled kernel stands beside generated ones, which take the launches it declines)
+    for (int i = 0; i < rp_hand_count; ++i) {
+      auto it = g_specs->find(rp_hand_table[i].hash);
+      if (it != g_specs->end()) it->second.hand = &rp_hand_table[i];
+    }
   }
   auto it = g_specs->find(h);
   return it == g_specs->end() ? nullptr : &it->second;
@@ -527,9 +534,21 @@ static bool rp_specs_disabled() {
   return v == 1;
 }
 
+// 1: generated kernels only (comparison of a hand-scheduled kernel with them); read once.
+static bool rp_hand_disabled() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("NBK_ROWPROG_HAND");
+    v = (e && e[0] == '0') ? 1 : 0;
+  }
+  return v == 1;
+}
+
 extern "C" int nbk_rowprog_is_specialized(const nbk_rowprog* prog) {
-  if (rp_validate(prog) != NBK_OK) return 0;
-  return (!rp_specs_disabled() && rp_find_spec(rp_program_hash(prog)) != nullptr) ? 1 : 0;
+  if (rp_validate(prog) != NBK_OK || rp_specs_disabled()) return 0;
+  RpSpec* spec = rp_find_spec(rp_program_hash(prog));
+  if (!spec) return 0;
+  return (spec->hand && !rp_hand_disabled() && spec->hand->fits(prog)) ? 2 : 1;
 }
 
 extern "C" uint64_t nbk_rowprog_hash(const nbk_rowprog* prog) {
@@ -580,6 +599,19 @@ extern "C" int nbk_rowprog_launch(const nbk_rowprog* prog, void* stream) {
     if (spec) {
       int64_t rows_arg = rows;
       void* args[2] = {(void*)p, (void*)&rows_arg};
+      if (spec->hand && !rp_hand_disabled() && spec->hand->fits(p)) {
+        int64_t bytes = 0;
+        for (int i = 0; i < p->n_operands; ++i)
+          if (p->operand[i].col_stride != 0)
+            bytes += rows * p->C * (int64_t)nbk_dtype_size(p->operand[i].dtype);
+        const void* fn = bytes > (256ll << 20) ? spec->hand->kernel_stream : spec->hand->kernel;
+        int per_cu = 0;
+        { const int orc = rp_occupancy(fn, spec->hand->block, &per_cu); if (orc != NBK_OK) return orc; }
+        int64_t g2 = (int64_t)nbk_num_cus() * per_cu;
+        if (g2 > rows) g2 = rows;
+        NBK_HIP(hipLaunchKernel(fn, dim3((unsigned)g2), dim3(spec->hand->block), args, 0, st));
+        return NBK_OK;
+      }
       // register-resident form: lanes own ceil(chunks / block) chunks each
       const int64_t n_chunks = c_pad >> 2;
       const int64_t need = (n_chunks + block - 1) / block;

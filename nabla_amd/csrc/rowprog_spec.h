@@ -3,6 +3,7 @@
 // hash of the program it is asked to launch.
 #pragma once
 #include <stdint.h>
+#include "nbk.h"
 
 struct rp_spec_entry {
   uint64_t hash;
@@ -27,6 +28,20 @@ struct rp_spec_entry {
   const void* kernel_stage16;
   int block_mode;
 };
+
+// A hand-scheduled kernel for one program (rowprog_hand.hip), attached by hash to that program's
+// entry above.  Signature of rp_block_kernel; launched with `block` lanes per row when
+// `fits(program)` holds, `kernel_stream` (non-temporal loads and stores) for launches that move
+// more than the last-level cache holds.
+struct rp_hand_entry {
+  uint64_t hash;
+  const void* kernel;
+  const void* kernel_stream;
+  int block;
+  bool (*fits)(const nbk_rowprog*);
+};
+extern const rp_hand_entry rp_hand_table[];
+extern const int rp_hand_count;
 
 #define NBK_RP_SPEC_FILES 4
 extern const rp_spec_entry rp_spec_table_0[];

@@ -126,25 +126,58 @@ def test_specialised_program_hash_matches_between_python_and_c(emulator):
 
     progs = [s for s in plan.steps if s.kind == "rowprog"]
     assert progs
-    # build the ctypes record exactly as the executor does and ask the library
     for st in progs:
-        a = st.attrs
-        rp = lib.RowProg()
-        rp.n_lead = len(a["lead"])
-        for i, d in enumerate(a["lead"]):
-            rp.lead_dim[i] = d
-        rp.C, rp.n_operands, rp.n_ins, rp.n_imm = a["C"], len(a["operands"]), len(a["ins"]), len(a["imm"])
-        rp.has_reduce, rp.block, rp.n_stage = int(a["has_reduce"]), a["block"], a["n_stage"]
-        for i, v in enumerate(a["imm"]):
-            rp.imm[i] = v
-        for i, o in enumerate(a["operands"]):
-            od = rp.operand[i]
-            od.ptr = 4096  # any non-null, aligned address; nothing is launched
-            od.col_stride, od.dtype, od.vec_ok, od.stage_slot = o.col_stride, o.dtype.abi, int(o.vec_ok), o.stage_slot
-            for j, s_ in enumerate(o.lead_strides):
-                od.lead_stride[j] = s_
-        for i, ins in enumerate(a["ins"]):
-            d = rp.ins[i]
-            d.op, d.dst, d.a, d.b, d.c, d.aux = ins
-        assert L.nbk_rowprog_is_specialized(C.byref(rp)) == 1, \
-            f"hash {specialize.program_hash(a):016x} not found in the library's table"
+        assert L.nbk_rowprog_is_specialized(C.byref(_program_record(st.attrs))) == 1, \
+            f"hash {specialize.program_hash(st.attrs):016x} not found in the library's table"
+
+
+def _program_record(a):
+    """The ctypes record of a planned row program, built as the executor builds it (operands at
+    an aligned dummy address: nothing is launched)."""
+    from nabla_amd.backend import lib
+    rp = lib.RowProg()
+    rp.n_lead = len(a["lead"])
+    for i, d in enumerate(a["lead"]):
+        rp.lead_dim[i] = d
+    rp.C, rp.n_operands, rp.n_ins, rp.n_imm = a["C"], len(a["operands"]), len(a["ins"]), len(a["imm"])
+    rp.has_reduce, rp.block, rp.n_stage = int(a["has_reduce"]), a["block"], a["n_stage"]
+    for i, v in enumerate(a["imm"]):
+        rp.imm[i] = v
+    for i, o in enumerate(a["operands"]):
+        od = rp.operand[i]
+        od.ptr = 4096
+        od.col_stride, od.dtype, od.vec_ok, od.stage_slot = o.col_stride, o.dtype.abi, int(o.vec_ok), o.stage_slot
+        for j, s_ in enumerate(o.lead_strides):
+            od.lead_stride[j] = s_
+    for i, ins in enumerate(a["ins"]):
+        d = rp.ins[i]
+        d.op, d.dst, d.a, d.b, d.c, d.aux = ins
+    return rp
+
+
+def test_the_loss_program_over_long_bf16_rows_has_its_hand_scheduled_kernel(emulator, monkeypatch):
+    """The hand-scheduled cross-entropy kernel is attached to its row program by the program's
+    hash: if the planner ever emits that program differently, the library would quietly fall
+    back to the generated kernel.  Planned here as the decoder plans it (bf16 logits in memory,
+    int64 labels, mean over the rows) and asked of the library, without a launch."""
+    import numpy as np
+    import torch
+    import nabla_amd as nb
+    from nabla_amd.backend import lib
+    from nabla_amd.core.engine import _PLAN_CACHE, clear_plan_cache
+    monkeypatch.delenv("NBK_ROWPROG_HAND", raising=False)
+    clear_plan_cache()
+    rows, vocab = 8, 32000
+    x = nb.Tensor.from_dlpack(torch.zeros(rows, vocab, dtype=torch.bfloat16))
+    lab = nb.Tensor.constant(np.zeros((rows,), np.int64))
+    loss, g = nb.value_and_grad(lambda z: nb.nn.functional.cross_entropy_loss(z, lab))(x)
+    nb.realize_all(loss, g)
+    plan = list(_PLAN_CACHE.values())[-1].plan
+    long_rows = [s for s in plan.steps if s.kind == "rowprog" and s.attrs["C"] == vocab]
+    assert len(long_rows) == 1, "loss and gradient are one row program"
+    L = lib.load()
+    rp = _program_record(long_rows[0].attrs)
+    assert L.nbk_rowprog_is_specialized(C.byref(rp)) == 2
+    rp.C = vocab + 4      # not whole 16-byte pieces: the generated kernels take it
+    assert L.nbk_rowprog_is_specialized(C.byref(rp)) == 1
+    clear_plan_cache()

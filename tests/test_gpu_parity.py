@@ -107,12 +107,30 @@ def test_specialised_kernels_match_interpreter(hip):
     np.testing.assert_allclose(gx_s.numpy(), gx_i.numpy(), rtol=2e-6, atol=1e-30)
 
 
-@pytest.mark.parametrize("rows,vocab", [(96, 32000), (700, 24000), (40, 20004)])
-def test_cross_entropy_over_long_rows_staged_in_lds(hip, rows, vocab):
-    """Cross-entropy and its gradient over bf16 rows too long for a register-resident kernel: the
-    specialised kernel that keeps the row in LDS (row lengths other than the benchmark's too; a
-    length that is no multiple of 4 takes the form that re-reads the row) against the interpreter
-    and against float64."""
+def _row_program_kinds():
+    """What nbk_rowprog_is_specialized says of every row program of the cached plans."""
+    from nabla_amd.backend import lib
+    from nabla_amd.core import engine
+    L = lib.load()
+    return [int(L.nbk_rowprog_is_specialized(C.byref(call[3])))
+            for bound in engine._PLAN_CACHE.values() for call in bound.calls
+            if call[0] is L.nbk_rowprog_launch]
+
+
+def _hand_kernels_on():
+    import os
+    return os.environ.get("NBK_ROWPROG_HAND", "1") != "0" and os.environ.get("NBK_ROWPROG_INTERPRET", "0") != "1"
+
+
+@pytest.mark.parametrize("rows,vocab", [(96, 32000), (700, 24000), (40, 20004), (33, 32768), (19, 16392),
+                                        (300, 4104), (9, 32776), (64, 16384)])
+def test_cross_entropy_over_long_rows(hip, rows, vocab):
+    """Cross-entropy and its gradient over long bf16 rows against the interpreter and against
+    float64.  Rows of whole 16-byte pieces, longer than the 16384 elements the planner stages in
+    LDS as fp32 and up to 32768, take the hand-scheduled kernel (the row in registers: the
+    benchmark's length, the longest and the shortest it takes, lengths whose last piece only some
+    lanes hold); the others the generated kernels or the interpreter: the row staged in LDS, or
+    re-read where its length is no multiple of 4."""
     from nabla_amd.backend import lib
     from nabla_amd.core import engine
     rng = np.random.default_rng(77)
@@ -120,8 +138,10 @@ def test_cross_entropy_over_long_rows_staged_in_lds(hip, rows, vocab):
     labels = rng.integers(0, vocab, (rows,)).astype(np.int64)
     F = nb.nn.functional
 
+    stored = torch.tensor(logits).to(torch.bfloat16).cuda()  # (logits that are bf16 in memory, as the decoder's)
+
     def run():
-        x = T(logits, dtype=nb.DType.bfloat16)
+        x = nb.Tensor.from_dlpack(stored)
         lab = nb.Tensor.constant(labels)
         loss, g = nb.value_and_grad(lambda z: F.cross_entropy_loss(z, lab))(x)
         nb.realize_all(loss, g)
@@ -129,11 +149,10 @@ def test_cross_entropy_over_long_rows_staged_in_lds(hip, rows, vocab):
 
     engine.clear_plan_cache()
     loss_s, g_s = run()
-    L = lib.load()
-    n_spec = sum(int(L.nbk_rowprog_is_specialized(C.byref(call[3])))
-                 for bound in engine._PLAN_CACHE.values() for call in bound.calls
-                 if call[0] is L.nbk_rowprog_launch)
-    assert n_spec >= 1, "the loss program of the decoder step must hit its specialised kernel"
+    kinds = _row_program_kinds()
+    assert max(kinds) >= 1, "the loss program of the decoder step must hit its specialised kernel"
+    if _hand_kernels_on():
+        assert (2 in kinds) == (vocab % 8 == 0 and 16384 < vocab <= 32768), kinds
     engine.clear_plan_cache()
     hip.force_interpreter = True
     try:
@@ -151,6 +170,59 @@ def test_cross_entropy_over_long_rows_staged_in_lds(hip, rows, vocab):
     p[np.arange(rows), labels] -= 1.0
     assert abs(loss_s - want_loss) <= 2.0 ** -8 * abs(want_loss)  # (the loss comes back in bf16)
     assert relerr(g_s, p / rows) <= BF16_TOL
+
+
+def test_cross_entropy_rows_with_infinities_nans_and_labels_out_of_range(hip):
+    """What the hand-scheduled cross-entropy kernel makes of rows the arithmetic breaks down on is
+    what the interpreter makes of them: a row with +inf or NaN, or of nothing but -inf, is NaN in
+    all of its gradient; -inf among finite logits has probability 0; a label outside [0, V)
+    picks nothing (the row's gradient is its softmax)."""
+    from nabla_amd.core import engine
+    rows, vocab = 8, 16416
+    rng = np.random.default_rng(5)
+    logits = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    labels = rng.integers(0, vocab, (rows,)).astype(np.int64)
+    labels[0], labels[1] = -1, vocab
+    logits[2, 77] = np.inf
+    logits[3, 16000] = np.nan
+    logits[4, :] = -np.inf
+    logits[5, 5:900] = -np.inf
+    labels[5] = 3
+    logits[6, labels[6]] = -np.inf          # the label's own logit: an infinite loss, finite gradient
+    F = nb.nn.functional
+
+    stored = torch.tensor(logits).to(torch.bfloat16).cuda()  # (logits that are bf16 in memory, as the decoder's)
+
+    def run():
+        x = nb.Tensor.from_dlpack(stored)
+        lab = nb.Tensor.constant(labels)
+        loss, g = nb.value_and_grad(lambda z: F.cross_entropy_loss(z, lab))(x)
+        nb.realize_all(loss, g)
+        return loss.item(), nb.cast(g, nb.DType.float32).numpy()
+
+    engine.clear_plan_cache()
+    loss_s, g_s = run()
+    if _hand_kernels_on():
+        assert 2 in _row_program_kinds()
+    engine.clear_plan_cache()
+    hip.force_interpreter = True
+    try:
+        loss_i, g_i = run()
+    finally:
+        hip.force_interpreter = False
+        engine.clear_plan_cache()
+    assert np.isnan(loss_s) and np.isnan(loss_i)
+    assert np.array_equal(np.isnan(g_s), np.isnan(g_i))
+    assert np.isnan(g_s[2]).all() and np.isnan(g_s[3]).all() and np.isnan(g_s[4]).all()
+    fine = [0, 1, 5, 6, 7]
+    np.testing.assert_allclose(g_s[fine], g_i[fine], rtol=2e-2, atol=1e-9)
+    assert (g_s[5, 5:900] == 0).all()
+    x64 = torch.tensor(logits[fine]).to(torch.bfloat16).double()
+    p = torch.softmax(x64, 1).numpy()
+    for i, r in enumerate(fine):
+        if 0 <= labels[r] < vocab:
+            p[i, labels[r]] -= 1.0
+    assert relerr(g_s[fine], p / rows) <= BF16_TOL
 
 
 # ---- C3 ------------------------------------------------------------------------------------------
