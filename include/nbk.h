@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 21
+#define NBK_ABI_VERSION 22
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -280,6 +280,17 @@ typedef struct nbk_gemm_desc {
    * 16-byte aligned, K % 64 == 0, M % 8 == 0, N % 8 == 0, alpha 1, no bias / residual / activation,
    * one batch level; anything else is an error. */
   void* colsum;
+  /* K2 > 0: a second, shallow operand pair whose product joins the accumulator before the
+   * epilogue, C = act(alpha * (A @ B + A2 @ B2) + bias) ...: A2 is M x K2 with strides
+   * (a2_rs, a2_cs), B2 is K2 x N with (b2_rs, b2_cs), one unit stride each.  This is the update
+   * of a low-rank adapter inside its base product, x @ W + (x @ A) @ B
+   * (nabla/nn/finetune/lora.py:55-79): the sum is rounded once and the base product makes no
+   * trip through memory.  bf16 operands, batch 1, no column sums.  Where the pair is laid out like
+   * A and B, 16-byte aligned and K2 <= 64, K2 % 8 == 0, it is one more K tile of the same launch;
+   * otherwise two launches give the same sum (plain products only: no bias, residual,
+   * activation or alpha then). */
+  const void* A2; const void* B2;
+  int64_t K2, a2_rs, a2_cs, b2_rs, b2_cs;
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
 

@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 MAX_RANK = 8
 
@@ -69,6 +69,9 @@ class GemmDesc(C.Structure):
         ("alpha", C.c_float), ("residual_op", C.c_int32),
         ("C_aux", C.c_void_p), ("aux_op", C.c_int32), ("reserved", C.c_int32),
         ("colsum", C.c_void_p),
+        ("A2", C.c_void_p), ("B2", C.c_void_p),
+        ("K2", C.c_int64), ("a2_rs", C.c_int64), ("a2_cs", C.c_int64), ("b2_rs", C.c_int64),
+        ("b2_cs", C.c_int64),
     ]
 
 

@@ -896,6 +896,62 @@ class Planner:
                 n.attrs = dict(at, res_in=len(mm.inputs), alpha=alpha * at.get("alpha", 1.0))
                 break
 
+    def _fold_thin_pair_into_matmul(self) -> None:
+        """``x @ W + u @ V`` with ``u @ V`` at most one K tile deep (the update of a low-rank
+        adapter on top of its base product, already folded by `_fold_sum_into_matmul` into a
+        thin product that reads the base product as its residual): the node turns into the base
+        product with ``(u, V)`` as a second operand pair (``attrs["pair_in"]``), which the
+        kernel multiplies as one more K tile into the same accumulator.  The base product no
+        longer makes a trip through memory (one write and one read of the result saved, and
+        the thin product's launch), and the sum is rounded once.  Only plain products on both
+        sides (no activation, scale, second result; the base may carry a bias) of one bf16 dtype
+        whose base has no other reader; the operands' layouts are checked when the node is lowered, and a pair the
+        kernel cannot take runs as the two launches it replaced."""
+        nodes = self._live_nodes()
+        n_users: dict[int, int] = {}
+        for n in nodes:
+            for i in n.inputs:
+                n_users[i.id] = n_users.get(i.id, 0) + 1
+        out_ids = {v.id for v in self.outputs}
+        def one_matrix(w: ir.Value) -> bool:
+            """A 2-D right operand, or one broadcast over the batch axes of the left one."""
+            while w.rank > 2:
+                m = w.node
+                if m.kind == "permute":  # (the transpose of the backward pass)
+                    perm = tuple(m.attrs["perm"])
+                    if perm[:-2] != tuple(range(w.rank - 2)):
+                        return False
+                    w = m.inputs[0]
+                elif m.kind == "broadcast" and m.inputs[0].rank == 2 and \
+                        tuple(m.inputs[0].shape) == tuple(w.shape[-2:]):
+                    return True
+                else:
+                    return False
+            return True
+
+        for n in nodes:
+            at = n.attrs or {}
+            if not (n.kind == "matmul" and at.get("res_in") == 2 and len(n.inputs) == 3 and
+                    len(n.outputs) == 1 and not at.get("act") and "bias_in" not in at and
+                    at.get("alpha", 1.0) == 1.0):
+                continue
+            u, v, r = n.inputs
+            base = r.node
+            bat = base.attrs or {}
+            k2 = u.shape[-1]
+            if not (base.kind == "matmul" and len(base.outputs) == 1 and
+                    len(base.inputs) == (3 if "bias_in" in bat else 2) and
+                    not (set(bat) & {"res_in", "act", "pair_in"}) and
+                    bat.get("alpha", 1.0) == 1.0 and
+                    n_users.get(r.id) == 1 and r.id not in out_ids and
+                    k2 <= 64 and k2 % 8 == 0 and one_matrix(v) and one_matrix(base.inputs[1]) and
+                    base.inputs[0].shape[-1] % 64 == 0 and
+                    u.shape[:-1] == base.inputs[0].shape[:-1] and
+                    all(x.dtype is DType.bfloat16 for x in (u, v, r, *base.inputs, n.outputs[0]))):
+                continue
+            n.inputs = list(base.inputs) + [u, v]
+            n.attrs = dict(bat, pair_in=len(base.inputs))
+
     def _fold_scale_into_matmul(self) -> None:
         """``(x @ W) * c`` with ``c`` a number: the multiply node turns into the product with
         ``alpha = c`` (applied to the fp32 accumulator, also of K-split partial products, before
@@ -1493,6 +1549,43 @@ class Planner:
             pb = self._mat_operand(rb)
         M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
         batch = _numel(out.shape[:-2])
+        if "pair_in" in at:
+            # x[.., M, K] @ W + u[.., M, K2] @ V with 2-D W and V: one unbatched product over all
+            # rows, for which x and u are read as whole row-major blocks (copied if they are not)
+            u, v = n.inputs[at["pair_in"]], n.inputs[at["pair_in"] + 1]
+
+            def rows_of(val, ref):
+                if isinstance(ref, Const):
+                    ref = self._materialize(ref)
+                po = self._mat_operand(ref)
+                whole = po is not None and (val.rank == 2 or (
+                    len(po[0]) <= 1 and po[2] == 1 and
+                    all(g == (_numel(val.shape[:-2]), val.shape[-2] * po[1]) for g in po[0])))
+                if not whole:
+                    ref = self._materialize(ref)
+                    po = self._mat_operand(ref)
+                return ref, po
+
+            ra, pa = rows_of(a, ra)
+            ru, pu = rows_of(u, self._resolve(u))
+            def one_matrix(val, ref):
+                if isinstance(ref, Const):
+                    ref = self._materialize(ref)
+                if val.rank > 2:  # (broadcast over the batch axes: any one of the copies)
+                    if any(st != 0 for d, st in zip(ref.shape[:-2], ref.strides[:-2]) if d > 1):
+                        raise AssertionError("paired product: the right operand is not one matrix")
+                    ref = ViewRef(ref.buf, ref.offset, ref.shape[-2:], ref.strides[-2:], ref.dtype)
+                po = self._mat_operand(ref)
+                if po is None:
+                    ref = self._materialize(ref)
+                    po = self._mat_operand(ref)
+                return ref, po
+
+            rb, pb = one_matrix(b, rb)
+            rv, pv = one_matrix(v, self._resolve(v))
+            epi.update(a2=ru, b2=rv, K2=u.shape[-1], a2_rs=pu[1], a2_cs=pu[2], b2_rs=pv[1], b2_cs=pv[2])
+            self._emit_plain_gemm(ra, rb, pa, pb, M * batch, N, K, out, epi)
+            return
         # sum_b A[b] @ B[b] (the weight gradient x^T dy of a layer applied to a batch) is one
         # product over the contraction index (b, k) when both operands step through it with
         # one stride: no per-batch products to store and add up, fp32 accumulation throughout
@@ -1637,7 +1730,7 @@ class Planner:
 
     @staticmethod
     def _epi_bufs(epi: dict) -> list[int]:
-        return [epi[k].buf for k in ("bias", "residual") if k in epi]
+        return [epi[k].buf for k in ("bias", "residual", "a2", "b2") if k in epi]
 
     # ................................................................ attention
     def _heads_operand(self, v: ir.Value) -> ViewRef:
@@ -2388,6 +2481,8 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
     pre._fold_bias_into_matmul()
     if config.FOLD_RESIDUAL or config.FOLD_THIN_RESIDUAL:
         pre._fold_sum_into_matmul(thin_only=not config.FOLD_RESIDUAL)
+        if config.FOLD_THIN_PAIR:
+            pre._fold_thin_pair_into_matmul()
         pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)
     if config.FOLD_ACTIVATION:
         pre._fold_activation_into_matmul()

@@ -55,6 +55,12 @@ _FOLD_RESIDUAL: ContextVar[bool] = ContextVar("FOLD_RESIDUAL",
 _FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
     "FOLD_THIN_RESIDUAL", default=_env_flag("NBK_FOLD_THIN_RESIDUAL", True))
 
+# x @ W + u @ V with u @ V at most one K tile deep (a low-rank adapter's update folded onto its
+# base product by the fold above) as ONE product with two operand pairs: the base result makes
+# no trip through memory; off: the thin product reads the base result as its residual
+_FOLD_THIN_PAIR: ContextVar[bool] = ContextVar(
+    "FOLD_THIN_PAIR", default=_env_flag("NBK_FOLD_THIN_PAIR", True))
+
 # the column sums of dy (a bias gradient) as one more result of the weight-gradient product
 # x^T dy that reads dy anyway; off: the reduction kernels read dy a second time
 _FOLD_COLUMN_SUMS: ContextVar[bool] = ContextVar(
@@ -89,6 +95,7 @@ _FLAGS = {
     "FOLD_ACTIVATION": _FOLD_ACTIVATION,
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
     "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
+    "FOLD_THIN_PAIR": _FOLD_THIN_PAIR,
     "FOLD_SCALE": _FOLD_SCALE,
     "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
     "VMAP_BATCHED": _VMAP_BATCHED,

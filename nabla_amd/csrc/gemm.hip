@@ -59,6 +59,10 @@ struct GemmArgs {
   int32_t b_block;
   int32_t c_stream;      // C is larger than the last-level cache: store it with the non-temporal hint
   void* colsum;          // null, or [batch][N] in C's dtype: the column sums of B over K
+  // a second, shallow operand pair whose product joins the accumulator: C = A B + A2 B2
+  // (K2 <= 64 deep; oriented like A and B; 0 = none).  Direct-to-LDS kernels only.
+  const void* A2; const void* B2;
+  int64_t K2, a2_rs, a2_cs, b2_rs, b2_cs;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -838,6 +842,39 @@ struct DirectLoader {
       }
     }
   }
+  // One K tile of a second, shallower operand (only k < kvalid of the tile's 64 k-rows exist),
+  // laid out in `region` like any other tile: a lane whose chunk lies beyond kvalid writes zeros
+  // to its LDS slot instead of fetching.  Keeps no state; (rs, cs) as for init.
+  __device__ __forceinline__ static void issue_tail(u32x4* region, const uint16_t* op, int64_t rs,
+                                                    int64_t cs, int64_t row0, int64_t rows_total,
+                                                    int kvalid, int wave, int lane) {
+    const int first_ = wave * N;
+    static_for<N>([&](auto jj) {
+      constexpr int j = decltype(jj)::value;
+      const char* src;
+      bool there;
+      if (KC) {
+        const int64_t last = rows_total - 1 - row0;
+        const int row = (first_ + j) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ dl_kc_xor<MI16>(row);
+        const int64_t r = row < last ? row : last;
+        src = (const char*)(op + row0 * rs) + (r * rs * 2 + c * 16);
+        there = c * 8 < kvalid;
+      } else {
+        const int64_t last = rows_total - 8 - row0;
+        const int l = (first_ + j) * 64 + lane;
+        const int k = l / NC, c = (l % NC) ^ (dl_seg_xor_of<MI16>(k) << 1);
+        const int64_t r = c * 8 < last ? c * 8 : last;
+        src = (const char*)(op + row0) + (k * cs * 2 + r * 2);
+        there = k < kvalid;
+      }
+      if (there)
+        __builtin_amdgcn_global_load_lds((glb_void_t*)src, (lds_void_t*)(region + (first_ + j) * 64),
+                                         16, 0, 0);
+      else
+        region[(first_ + j) * 64 + lane] = (u32x4)(0u);
+    });
+  }
   // start the copy of K tile `kt` into `region` (this operand's part of a tile buffer)
   __device__ __forceinline__ const char* tile_src(int64_t kt) const { return base + kt * kstep; }
   template <int J>
@@ -903,11 +940,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   using LB = DirectLoader<BN, B_KC, NW, MI16>;
   LA la;
   LB lb;
-  la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
-  lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
-  const int64_t nk = g.K / 64;
-  la.issue(gemm_lds, 0);
-  lb.issue(gemm_lds + CA, 0);
+  int64_t nk = g.K / 64;
+  if (g.K2 > 0) {
+    // the shallow second pair is K tile 0 (its offsets are dead before the loop's are made);
+    // the tiles of A and B follow as tiles 1 .. K / 64
+    LA::issue_tail(gemm_lds, (const uint16_t*)g.A2, g.a2_rs, g.a2_cs, m0, g.M, (int)g.K2, wave, lane);
+    LB::issue_tail(gemm_lds + CA, (const uint16_t*)g.B2, g.b2_cs, g.b2_rs, n0, g.N, (int)g.K2, wave,
+                   lane);
+    la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
+    lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
+    la.base -= la.kstep;
+    lb.base -= lb.kstep;
+    nk += 1;
+  } else {
+    la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
+    lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
+    la.issue(gemm_lds, 0);
+    lb.issue(gemm_lds + CA, 0);
+  }
 
   // Fragment addresses, one per block row / column of the wave tile.  32 x 32 x 16:
   //   K-contiguous: byte address 16 ((row * 8 | t) ^ (2 ks)), t = kg ^ (row % 8) ^ (row / 8 % 2);
@@ -1740,7 +1790,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   NBK_REQUIRE(d->ldc >= d->N, "gemm: ldc %lld < N %lld", (long long)d->ldc, (long long)d->N);
   NBK_REQUIRE(d->batch_reduce == 0, "gemm: batch_reduce is folded into K by the caller");
   hipStream_t st = (hipStream_t)stream;
-  GemmArgs a;
+  GemmArgs a = {};
   a.A = d->A; a.B = d->B; a.C = d->C; a.bias = d->bias; a.residual = d->residual;
   a.M = d->M; a.N = d->N; a.K = d->K;
   a.a_rs = d->a_rs; a.a_cs = d->a_cs; a.b_rs = d->b_rs; a.b_cs = d->b_cs; a.ldc = d->ldc;
@@ -1770,6 +1820,14 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;
+  const bool tail = d->K2 > 0;
+  if (tail) {
+    NBK_REQUIRE(d->A2 && d->B2, "gemm: K2 = %lld without A2 / B2", (long long)d->K2);
+    NBK_REQUIRE(d->dtype_ab == NBK_BF16 && d->batch == 1 && d->colsum == nullptr,
+                "gemm: a second operand pair goes with one bf16 product without column sums");
+    NBK_REQUIRE(d->a2_rs == 1 || d->a2_cs == 1, "gemm: A2 needs a unit stride");
+    NBK_REQUIRE(d->b2_rs == 1 || d->b2_cs == 1, "gemm: B2 needs a unit stride");
+  }
   const int esz = d->dtype_ab == NBK_F32 ? 4 : 2;
   auto vec_ok = [&](const void* p, int64_t other_stride, int64_t bs, int64_t bs2) {
     const int64_t q = 16 / esz;
@@ -1780,7 +1838,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   // (checked before any kernel is chosen: no path may take the product and drop the sums)
   NBK_REQUIRE(d->colsum == nullptr || (d->dtype_ab == NBK_BF16 && !akc && !bkc),
               "gemm: column sums need bf16 operands that are both row-contiguous (a_rs == b_cs == 1)");
-  if (d->dtype_ab == NBK_BF16 && d->N <= 32 && d->M >= 1024 && d->K >= 256 && d->K % 64 == 0 &&
+  if (!tail && d->dtype_ab == NBK_BF16 && d->N <= 32 && d->M >= 1024 && d->K >= 256 && d->K % 64 == 0 &&
       akc && a.a_vec && d->batch == 1 && d->bias == nullptr && d->residual == nullptr &&
       d->act == NBK_ACT_NONE && (bkc ? (bool)a.b_vec : (d->b_cs == 1 && d->N % 8 == 0 && a.b_vec))) {
     // 32 rows per workgroup, K split over its eight waves
@@ -1805,7 +1863,7 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
       return nbk_check_launch("gemm_skinny_n_kernel");
     }
   }
-  if (d->dtype_ab == NBK_BF16 && d->K <= 16 && akc && d->batch == 1 && d->N % 8 == 0 &&
+  if (!tail && d->dtype_ab == NBK_BF16 && d->K <= 16 && akc && d->batch == 1 && d->N % 8 == 0 &&
       d->ldc % 8 == 0 && ((uintptr_t)d->C & 15) == 0 && ((uintptr_t)d->residual & 15) == 0 &&
       (d->K == 16 ? a.a_vec : d->K == 8 && (d->a_rs % 8 == 0) && ((uintptr_t)d->A & 15) == 0)) {
     // (the vector path reads whole 16-byte pieces of A rows: K = 16 or 8)
@@ -1842,6 +1900,37 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
     const bool fast = a.a_vec && a.b_vec && (d->K % 64 == 0) && (akc || d->M % 8 == 0) &&
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8 &&
                       a_stride >= 0 && b_stride >= 0 && a_stride < (1 << 22) && b_stride < (1 << 22);
+    if (tail) {
+      // In the accumulator of the direct-to-LDS kernels when the pair is laid out like A and B,
+      // at most one K tile deep and 16-byte aligned; otherwise as a second product that adds
+      // itself to the first (a plain one only: the epilogue would have to wait for it).
+      const bool a2kc = d->a2_cs == 1, b2kc = d->b2_rs == 1;
+      const int64_t a2_stride = a2kc ? d->a2_rs : d->a2_cs, b2_stride = b2kc ? d->b2_cs : d->b2_rs;
+      const bool inside = fast && a2kc == akc && b2kc == bkc && d->K2 <= 64 && d->K2 % 8 == 0 &&
+                          ((uintptr_t)d->A2 % 16 == 0) && ((uintptr_t)d->B2 % 16 == 0) &&
+                          a2_stride % 8 == 0 && b2_stride % 8 == 0 && a2_stride >= 0 &&
+                          b2_stride >= 0 && a2_stride < (1 << 22) && b2_stride < (1 << 22) &&
+                          d->M >= 128 && d->N >= 128;
+      if (inside) {
+        a.A2 = d->A2; a.B2 = d->B2; a.K2 = d->K2;
+        a.a2_rs = d->a2_rs; a.a2_cs = d->a2_cs; a.b2_rs = d->b2_rs; a.b2_cs = d->b2_cs;
+      } else {
+        NBK_REQUIRE(d->bias == nullptr && d->residual == nullptr && d->act == NBK_ACT_NONE &&
+                        d->C_aux == nullptr && d->alpha == 1.f,
+                    "gemm: a second operand pair outside the direct kernels' conditions goes with a "
+                    "plain product only");
+        nbk_gemm_desc first = *d;
+        first.A2 = nullptr; first.B2 = nullptr; first.K2 = 0;
+        const int rc = nbk_gemm(&first, stream);
+        if (rc != NBK_OK) return rc;
+        nbk_gemm_desc second = first;
+        second.A = d->A2; second.B = d->B2; second.K = d->K2;
+        second.a_rs = d->a2_rs; second.a_cs = d->a2_cs; second.b_rs = d->b2_rs; second.b_cs = d->b2_cs;
+        second.residual = d->C;  // (every kernel reads a residual element in the lane that writes it)
+        second.residual_op = NBK_RES_ADD;
+        return nbk_gemm(&second, stream);
+      }
+    }
     if (d->colsum != nullptr) {
       NBK_REQUIRE(fast && !akc && !bkc && a.batch_inner == 1 && d->bias == nullptr &&
                       d->residual == nullptr && d->act == NBK_ACT_NONE && d->alpha == 1.f,

@@ -85,6 +85,110 @@ def test_gemm(hip, dtype, layout, shape):
 
 
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape,k2,how", [
+    ((512, 384, 256), 16, "same"),      # one more K tile of the launch (128 x 128 tiles)
+    ((1024, 1024, 512), 8, "same"),     # 256 x 256 tiles; a single 16-byte piece per row of the pair
+    ((4000, 2600, 192), 64, "same"),    # a whole tile deep, ragged edges
+    ((1000, 520, 128), 24, "same"),
+    ((512, 384, 256), 16, "bias"),      # the epilogue sees the sum of both products
+    ((512, 384, 256), 12, "same"),      # K2 % 8 != 0: two launches give the sum
+    ((512, 384, 256), 80, "same"),      # deeper than a tile: two launches
+    ((512, 384, 256), 16, "other"),     # the pair laid out the other way round: two launches
+    ((512, 384, 256), 16, "offset"),    # the pair not 16-byte aligned: two launches
+    ((200, 136, 72), 16, "same"),       # K % 64 != 0: the guarded kernel, two launches
+])
+def test_gemm_with_a_second_operand_pair(hip, layout, shape, k2, how):
+    """C = A @ B + A2 @ B2 (the update of a low-rank adapter inside its base product) through
+    the C ABI against float64 of the same bf16 operands: where the pair meets the direct-to-LDS
+    kernels' conditions it is one more K tile of the launch, elsewhere the library runs the two
+    products one after the other, the second adding itself to the first."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(11)
+    bf = torch.bfloat16
+    A = torch.tensor(rng.standard_normal((M, K)), dtype=bf)
+    B = torch.tensor(rng.standard_normal((K, N)), dtype=bf)
+    A2 = torch.tensor(rng.standard_normal((M, k2)) * 3.0, dtype=bf)
+    B2 = torch.tensor(rng.standard_normal((k2, N)) * 3.0, dtype=bf)
+    bias = torch.tensor(rng.standard_normal((N,)) * 4.0, dtype=bf)
+    first = (A.double() @ B.double()).numpy()
+    ref = first + (A2.double() @ B2.double()).numpy()
+    if how == "bias":
+        ref = ref + bias.double().numpy()
+    lay2 = layout if how != "other" else ("t" if layout[0] == "n" else "n") + ("t" if layout[1] == "n" else "n")
+
+    def put(t, transposed, shift=0):
+        t = t.t().contiguous() if transposed else t.contiguous()
+        if not shift:
+            return t.cuda(), 0
+        flat = torch.zeros(t.numel() + 8, dtype=bf)
+        flat[shift:shift + t.numel()] = t.reshape(-1)
+        return flat.cuda(), shift * 2
+
+    a_dev, _ = put(A, layout[0] == "t")
+    b_dev, _ = put(B, layout[1] == "t")
+    shift = 3 if how == "offset" else 0
+    a2_dev, a2_off = put(A2, lay2[0] == "t", shift)
+    b2_dev, b2_off = put(B2, lay2[1] == "t", shift)
+    bias_dev = bias.cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=bf, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = a_dev.data_ptr(), b_dev.data_ptr(), c_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.a_rs, d.a_cs = (K, 1) if layout[0] == "n" else (1, M)
+    d.b_rs, d.b_cs = (N, 1) if layout[1] == "n" else (1, K)
+    d.A2, d.B2, d.K2 = a2_dev.data_ptr() + a2_off, b2_dev.data_ptr() + b2_off, k2
+    d.a2_rs, d.a2_cs = (k2, 1) if lay2[0] == "n" else (1, M)
+    d.b2_rs, d.b2_cs = (N, 1) if lay2[1] == "n" else (1, k2)
+    d.ldc = N
+    d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
+    d.dtype_ab = d.dtype_c = 1
+    d.alpha = 1.0
+    if how == "bias":
+        d.bias = bias_dev.data_ptr()
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    # (two launches round the first product to bf16 before the second is added: one more
+    # rounding, of a value that may be larger than the sum)
+    err = np.abs(got - ref) - 2.0 ** -8 * (np.abs(ref) + np.abs(first))
+    assert err.max() <= 2e-2, err.max()
+
+
+def test_gemm_second_pair_errors(hip):
+    """What the second operand pair does not go with is refused, not dropped."""
+    from nabla_amd.backend import lib
+    bf = torch.bfloat16
+    x = torch.zeros((256, 256), dtype=bf, device="cuda")
+    x32 = torch.zeros((256, 256), dtype=torch.float32, device="cuda")
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def desc(t=x, **kw):
+        d = lib.GemmDesc()
+        d.A = d.B = d.C = t.data_ptr()
+        d.M = d.N = d.K = 256
+        d.a_rs, d.a_cs, d.b_rs, d.b_cs, d.ldc = 256, 1, 256, 1, 256
+        d.batch = 1
+        d.dtype_ab = d.dtype_c = 1 if t is x else 0
+        d.alpha = 1.0
+        d.A2, d.B2, d.K2 = x.data_ptr(), x.data_ptr(), 16
+        d.a2_rs, d.a2_cs, d.b2_rs, d.b2_cs = 16, 1, 256, 1
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return d
+
+    assert L.nbk_gemm(C.byref(desc()), st) == 0
+    for bad in (desc(A2=None), desc(batch=2), desc(t=x32), desc(a2_rs=16, a2_cs=2),
+                desc(K2=12, act=1),                 # two launches cannot carry an epilogue
+                desc(colsum=x.data_ptr(), a_rs=1, a_cs=256)):
+        assert L.nbk_gemm(C.byref(bad), st) != 0
+        assert b"gemm" in L.nbk_last_error()
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
 @pytest.mark.parametrize("shape", [(384, 256, 2048), (1000, 520, 4096)])
 def test_gemm_long_k_small_output(hip, layout, shape):
     """bf16 products with a long contraction and few 128 x 128 tiles (the shapes the planner
