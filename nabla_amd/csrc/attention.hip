@@ -26,9 +26,11 @@
 //                                  fragment reads of 16 consecutive rows hit distinct banks
 //   transposed [hd rows][64 cols]  row pitch 68 elements: the 8-byte reads of 32
 //                                  consecutive rows fall on distinct banks per half
-// The dQ kernel and the dK/dV kernel for 128-wide heads keep no transposed tiles: they take
-// the A operand of the second MFMA out of the row-major tile with ds_read_b64_tr_b16 (the
-// swizzle at_sw serves both kinds of read).
+// The forward kernel, the dQ kernel and the dK/dV kernel for 128-wide heads keep no transposed
+// tiles: they take the A operand of the second MFMA out of the row-major tile with
+// ds_read_b64_tr_b16 (the swizzle at_sw serves both kinds of read).  The forward kernel's tiles
+// go from memory into LDS directly (global_load_lds: no staging registers, which lets four
+// waves per SIMD run with 64-wide heads).
 #include "nbk_common.h"
 #include <mutex>
 
@@ -197,6 +199,8 @@ __device__ __forceinline__ int at_sw(int row) {
   else return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
 }
 
+typedef __attribute__((address_space(3))) void at_lds_void;
+typedef __attribute__((address_space(1))) const void at_glb_void;
 typedef short at_s16x4 __attribute__((ext_vector_type(4)));
 typedef short at_s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) at_s16x4 at_lds_s16x4;
@@ -221,14 +225,12 @@ constexpr float AT_LOG2E = 1.4426950408889634f;
 constexpr float AT_LN2 = 0.6931471805599453f;
 
 template <int HD>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
-  using RowT = AtRowTile<HD>;
-  using TrT = AtTransTile<HD>;
-  constexpr int KSTEPS = HD / 16, DT = HD / 32;
-  constexpr int ROW_BYTES = 64 * HD * 2, TR_BYTES = HD * AT_TP * 2;
+__global__ __launch_bounds__(256, HD == 64 ? 4 : 2) void attn_fwd_kernel(const AttnArgs g) {
+  constexpr int KSTEPS = HD / 16, DT = HD / 32, NCH = HD / 8;
+  constexpr int TILE = 64 * HD * 2, STAGE = 2 * TILE;
   extern __shared__ __align__(16) unsigned char at_lds[];
-  auto k_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * (ROW_BYTES + TR_BYTES)); };
-  auto v_tile = [&](int buf) { return (uint16_t*)(at_lds + buf * (ROW_BYTES + TR_BYTES) + ROW_BYTES); };
+  auto k_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE); };
+  auto v_tile = [&](int buf) { return (at_u32x4*)(at_lds + buf * STAGE + TILE); };
 
   // Grid (B * H, tiles): workgroups are handed out along x first, so every (batch, head) runs
   // its longest causal rows before any runs a shorter one, and the tail of the launch consists
@@ -265,22 +267,60 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   float l_r = 0.f;
 
   const int n_tiles = g.causal ? (q0 + 128) / 64 : g.S / 64;
-  RowT kl;
-  TrT vl;
-  kl.load(K, g.k.ss, 0);
-  vl.load(V, g.v.ss, 0);
-  kl.store(k_tile(0));
-  vl.store(v_tile(0));
-  __syncthreads();
+  // K and V tiles go from memory into LDS without passing through registers: a wave instruction
+  // deposits 64 x 16 bytes in a row (four rows of a 128-wide tile, eight of a 64-wide one), so
+  // the swizzle is applied to the address each lane fetches from.
+  constexpr int PER_WAVE = 64 * NCH / 64 / 4;  // instructions per wave and tile
+  int src_off_k[PER_WAVE], src_off_v[PER_WAVE];  // element offsets of this lane's chunks in a tile
+#pragma unroll
+  for (int j = 0; j < PER_WAVE; ++j) {
+    const int slot = (wave * PER_WAVE + j) * 64 + lane, row = slot / NCH, c = (slot % NCH) ^ at_sw<NCH>(row);
+    src_off_k[j] = row * (int)g.k.ss + c * 8;
+    src_off_v[j] = row * (int)g.v.ss + c * 8;
+  }
+  auto request = [&](int kt, int buf) {
+    const uint16_t* ks = K + (int64_t)kt * 64 * g.k.ss;
+    const uint16_t* vs = V + (int64_t)kt * 64 * g.v.ss;
+#pragma unroll
+    for (int j = 0; j < PER_WAVE; ++j) {
+      __builtin_amdgcn_global_load_lds((at_glb_void*)(ks + src_off_k[j]),
+                                       (at_lds_void*)(k_tile(buf) + (wave * PER_WAVE + j) * 64), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((at_glb_void*)(vs + src_off_v[j]),
+                                       (at_lds_void*)(v_tile(buf) + (wave * PER_WAVE + j) * 64), 16, 0, 0);
+    }
+  };
+  // a workgroup barrier behind which every wave's copies have landed
+  auto tile_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  };
+  auto frag = [&](const at_u32x4* tile, int row, int chunk) {
+    return __builtin_bit_cast(at_bf16x8, tile[row * NCH + (chunk ^ at_sw<NCH>(row))]);
+  };
+  int tr_lo, tr_hi, tr_x_lo, tr_x_hi;  // the transposing read of V, as the dQ kernel reads K
+  {
+    const int p = lane & 15, G = lane >> 4;
+    const int kl = 4 * (G >> 1) + (p >> 2);
+    const int d0 = 16 * (G & 1) + 4 * (p & 3);
+    tr_x_lo = (d0 >> 3) ^ at_sw<NCH>(kl);
+    tr_x_hi = (d0 >> 3) ^ at_sw<NCH>(kl + 8);
+    tr_lo = kl * (HD * 2) + (d0 & 7) * 2;
+    tr_hi = (kl + 8) * (HD * 2) + (d0 & 7) * 2;
+  }
+  auto tr_frag = [&](const at_u32x4* tile, int dd, int k16) {
+    const unsigned char* base = (const unsigned char*)tile + k16 * 16 * (HD * 2);
+    return at_tr_pair(base + tr_lo + ((tr_x_lo ^ (dd << 2)) << 4), base + tr_hi + ((tr_x_hi ^ (dd << 2)) << 4));
+  };
+  request(0, 0);
+  tile_barrier();
   for (int kt = 0; kt < n_tiles; ++kt) {
     const int cur = kt & 1;
     const bool more = kt + 1 < n_tiles;
-    if (more) {
-      kl.load(K, g.k.ss, (kt + 1) * 64);
-      vl.load(V, g.v.ss, (kt + 1) * 64);
-    }
+    if (more) request(kt + 1, cur ^ 1);
     const at_u32x4* Ks = k_tile(cur);
-    const uint16_t* Vs = v_tile(cur);
+    const at_u32x4* Vs = v_tile(cur);
     const int k0 = kt * 64;
     auto tile = [&](auto masked) {
       constexpr bool MASK = decltype(masked)::value;
@@ -291,7 +331,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
         // all fragments of the 32 keys are requested before the first MFMA waits for one
         at_bf16x8 kfr[KSTEPS];
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) kfr[s] = RowT::frag(Ks, kt2 * 32 + li, 2 * s + h);
+        for (int s = 0; s < KSTEPS; ++s) kfr[s] = frag(Ks, kt2 * 32 + li, 2 * s + h);
         __builtin_amdgcn_sched_barrier(0);  // keeps the scheduler from sinking each read to its MFMA
         at_f32x16 acc = (at_f32x16)(0.f);
 #pragma unroll
@@ -338,19 +378,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
           const at_bf16x8 pf = at_regs_frag(st[kt2], t);
 #pragma unroll
           for (int d = 0; d < DT; ++d)
-            o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TrT::frag(Vs, d * 32 + li, kt2, t, h), pf,
-                                                               o_acc[d], 0, 0, 0);
+            o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag(Vs, d, 2 * kt2 + t), pf, o_acc[d], 0, 0, 0);
           l_r = at_sum_bf16x8(pf, l_r);
         }
     };
     // keys of this tile against the wave's queries: all visible, some, or none
     if (!g.causal || k0 + 63 <= wq0) tile(std::false_type{});
     else if (k0 <= wq0 + 31) tile(std::true_type{});
-    if (more) {
-      kl.store(k_tile(cur ^ 1));
-      vl.store(v_tile(cur ^ 1));
-    }
-    __syncthreads();
+    tile_barrier();
   }
   // normalise and write: register r of tile d is O[my_q][32 d + (r/4)*8 + 4h + r%4]
   l_i += at_xhalf(l_i);
@@ -384,6 +419,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs g) {
   }
   if (h == 0) g.lse[((int64_t)b * g.H + hh) * g.S + my_q] = m_i * AT_LN2 + __logf(l_i);
 }
+
 
 // ------------------------------------------------------------------------------ backward
 // dK, dV.  Grid: (B * H, S / 128).  Wave w owns keys k0 + 32w .. + 31 (one per lane pair)
@@ -970,14 +1006,12 @@ extern "C" int nbk_attention_fwd(const nbk_attn_desc* d, const nbk_attn_tensor* 
   a.lse = (float*)lse;
   const dim3 grid((unsigned)(d->B * d->H), (unsigned)(d->S / 128));
   hipStream_t st = (hipStream_t)stream;
+  // two stages of a row-major K and V tile each
+  const size_t lds = 2 * 2 * 64 * (size_t)d->hd * 2;
   if (d->hd == 64) {
-    const size_t lds = 2 * (64 * 64 * 2 + 64 * AT_TP * 2);
     if ((rc = attn_set_lds(attn_fwd_kernel<64>, lds))) return rc;
     hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, dim3(256), lds, st, a);
   } else {
-    // (reading V through the transposing LDS read, as the backward kernels for this head size
-    // do, was measured here too: same time, so the forward keeps its transposed copy)
-    const size_t lds = 2 * (64 * 128 * 2 + 128 * AT_TP * 2);
     if ((rc = attn_set_lds(attn_fwd_kernel<128>, lds))) return rc;
     hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, dim3(256), lds, st, a);
   }
