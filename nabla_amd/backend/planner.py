@@ -952,6 +952,64 @@ class Planner:
             n.inputs = list(base.inputs) + [u, v]
             n.attrs = dict(bat, pair_in=len(base.inputs))
 
+        # ``(X + u @ V) + x @ W``: contributions to one gradient arrive in the order of the
+        # backward pass, and a thin product whose base product comes one link later in the chain
+        # of sums was not folded above.  The base product takes the pair where it stands (``u``
+        # and ``V`` exist before the thin product, which comes earlier) and the outer sum reads
+        # ``X`` instead of the inner one; the thin product and the inner sum lose their readers.
+        nodes = self._live_nodes()
+        users: dict[int, list[ir.Node]] = {}
+        for n in nodes:
+            for i in n.inputs:
+                users.setdefault(i.id, []).append(n)
+
+        def only_reader(val: ir.Value):
+            us = users.get(val.id, [])
+            return us[0] if len(us) == 1 and val.id not in out_ids else None
+
+        def plain_add(n: ir.Node) -> bool:
+            return (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2 and
+                    all(isinstance(x, ir.Value) for x in n.attrs["operands"]))
+
+        for thin in nodes:
+            tat = thin.attrs or {}
+            if not (thin.kind == "matmul" and len(thin.inputs) == 2 and len(thin.outputs) == 1 and
+                    not (set(tat) & {"res_in", "bias_in", "act", "pair_in"}) and
+                    tat.get("alpha", 1.0) == 1.0):
+                continue
+            u, v = thin.inputs
+            k2 = u.shape[-1]
+            t_out = thin.outputs[0]
+            if not (k2 <= 64 and k2 % 8 == 0 and one_matrix(v)):
+                continue
+            inner = only_reader(t_out)
+            if inner is None or not plain_add(inner):
+                continue
+            x_val = inner.inputs[1] if inner.inputs[0].id == t_out.id else inner.inputs[0]
+            outer = only_reader(inner.outputs[0])
+            if outer is None or not plain_add(outer) or x_val.id == t_out.id:
+                continue
+            b_out = outer.inputs[1] if outer.inputs[0].id == inner.outputs[0].id else outer.inputs[0]
+            base = b_out.node
+            bat = base.attrs or {}
+            if not (base.kind == "matmul" and base is not thin and len(base.outputs) == 1 and
+                    len(base.inputs) == 2 and not (set(bat) & {"res_in", "bias_in", "act", "pair_in"}) and
+                    bat.get("alpha", 1.0) == 1.0 and only_reader(b_out) is outer and
+                    base.pos > thin.pos and base.inputs[0].shape[-1] % 64 == 0 and
+                    one_matrix(base.inputs[1]) and u.shape[:-1] == base.inputs[0].shape[:-1] and
+                    b_out.shape == t_out.shape == x_val.shape and
+                    all(z.dtype is DType.bfloat16 for z in (u, v, t_out, b_out, x_val, *base.inputs,
+                                                             inner.outputs[0], outer.outputs[0]))):
+                continue
+            base.inputs = list(base.inputs) + [u, v]
+            base.attrs = dict(bat, pair_in=2)
+            outer.inputs = [x_val, b_out]
+            outer.attrs = dict(outer.attrs, operands=(x_val, b_out))
+            users[b_out.id] = [outer]
+            users[x_val.id] = [z for z in users.get(x_val.id, []) if z is not inner] + [outer]
+            users[t_out.id] = []
+            users[inner.outputs[0].id] = []
+
     def _fold_scale_into_matmul(self) -> None:
         """``(x @ W) * c`` with ``c`` a number: the multiply node turns into the product with
         ``alpha = c`` (applied to the fp32 accumulator, also of K-split partial products, before

@@ -474,7 +474,10 @@ def collect_programs() -> dict[int, dict]:
                 with contextlib.ExitStack() as es:
                     for name, value in flags.items():
                         es.enter_context(config.flag(name, value))
-                    return job()
+                    res = job()
+                    # (planned here: a flag of the planner is read when the step is realized)
+                    nb.realize_all(*[x for x in nb.tree_leaves(res) if isinstance(x, nb.Tensor)])
+                    return res
             return run
 
         # the loss over a batch too small for its label mask to be recomputed per reader (the
@@ -489,6 +492,7 @@ def collect_programs() -> dict[int, dict]:
         jobs.append(small_batch_loss)
         jobs.append(with_flags(jobs[2], FUSED_ATTENTION=False))
         jobs.append(with_flags(jobs[4], FUSED_ATTENTION=False, LORA_LOW_RANK_ORDER=False))
+        jobs.append(with_flags(jobs[4], FOLD_THIN_PAIR=False))
         for job in jobs:
             clear_plan_cache()
             res = job()

@@ -131,6 +131,21 @@ def test_specialised_program_hash_matches_between_python_and_c(emulator):
             f"hash {specialize.program_hash(st.attrs):016x} not found in the library's table"
 
 
+def test_generated_kernels_cover_every_row_program_of_the_benchmark_steps():
+    """The five benchmark steps (and the other evaluation orders the generator plans) are planned
+    as the generator plans them, and every row program that comes out must have its
+    ahead-of-time kernel in the library: a planner change that alters a program without
+    `python -m nabla_amd.backend.specialize` being run again would leave that program to the
+    interpreter (correct, and ten times slower on the decoder's layer-norm backward)."""
+    from nabla_amd.backend import lib, specialize
+    programs = specialize.collect_programs()
+    assert len(programs) >= 30
+    L = lib.load()
+    missing = [f"{h:016x} ({' '.join(a.get('members', []))[:60]})" for h, a in programs.items()
+               if L.nbk_rowprog_is_specialized(C.byref(_program_record(a))) < 1]
+    assert not missing, "row programs without a specialised kernel: " + "; ".join(missing)
+
+
 def _program_record(a):
     """The ctypes record of a planned row program, built as the executor builds it (operands at
     an aligned dummy address: nothing is launched)."""

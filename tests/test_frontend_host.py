@@ -773,6 +773,43 @@ def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
     np.testing.assert_allclose(grads["A"].numpy(), 3.0 * x2.T @ (np.ones((120, 16), np.float32) @ b.T), rtol=1e-4, atol=1e-4)
 
 
+def test_adapter_updates_ride_inside_their_base_products(emulator):
+    """`x @ W + (x @ A) @ B` and its mirror image in the backward pass are ONE product with two
+    operand pairs each (`nbk_gemm_desc.A2 / B2 / K2`): in a two-layer decoder the four forward
+    updates fold onto their base products directly, the two backward ones of the second layer
+    also where the base product comes one link later in the chain of sums.  No thin product is
+    left that reads a base result, the gradients are those of the plan without the fold, and a
+    rank that is no multiple of 8 keeps the thin products."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+
+    def step(rank):
+        engine.clear_plan_cache()
+        t = oc.c5_inputs(layers=2, batch=2, seq=64, d_model=128, d_ff=256, vocab=300, rank=rank, seed=3,
+                         b_zero=False, bf16=True)
+        loss, grads = oc.c5_program(nb, oc.upload(nb, t, dtype=nb.DType.bfloat16), num_heads=4)
+        flat = [ad[k] for ad in grads for k in ("qA", "qB", "vA", "vB")]
+        nb.realize_all(loss, *flat)
+        gemms = [s.attrs for s in list(engine._PLAN_CACHE.values())[-1].plan.steps if s.kind == "gemm"]
+        return loss.item(), [g.numpy() for g in flat], gemms
+
+    loss_on, g_on, gemms = step(16)
+    paired = [a for a in gemms if a.get("a2") is not None]
+    assert len(paired) == 6
+    assert all(a["K2"] == 16 and a["K"] == 128 and a["batch"] == 1 and a["M"] == 128 for a in paired)
+    assert not [a for a in gemms if a["K"] <= 16 and a["N"] > 16]      # every update found its base
+    with config.flag("FOLD_THIN_PAIR", False):
+        loss_off, g_off, gemms_off = step(16)
+    assert not [a for a in gemms_off if a.get("a2") is not None]
+    assert len(gemms_off) == len(gemms) + 6
+    assert abs(loss_on - loss_off) <= 2e-2 * abs(loss_off)
+    for a, b in zip(g_on, g_off):
+        assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max()
+    _, _, gemms4 = step(4)
+    assert not [a for a in gemms4 if a.get("a2") is not None]
+    engine.clear_plan_cache()
+
+
 def test_a_batch_summed_product_keeps_what_was_folded_onto_it(emulator):
     """sum_b A[b] @ B[b] becomes one product over (b, k).  A scale folded onto the batched product
     commutes with the sum and rides along as alpha; a bias or a residual added per batch element
