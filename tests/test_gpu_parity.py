@@ -172,6 +172,44 @@ def test_cross_entropy_over_long_rows(hip, rows, vocab):
     assert relerr(g_s, p / rows) <= BF16_TOL
 
 
+def test_cross_entropy_over_rows_behind_two_leading_axes_and_a_row_pitch(hip):
+    """The hand-scheduled kernel finds its rows through the program's leading strides: logits
+    [batch, sequence, V] (two leading axes), and logits that are the first V columns of a wider
+    buffer (a row pitch that is not the row length), against float64."""
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(8)
+    B, S, V, wide = 3, 7, 16392, 16392 + 40
+    full = (rng.standard_normal((B, S, wide)) * 2.5).astype(np.float32)
+    labels = rng.integers(0, V, (B, S)).astype(np.int64)
+    stored = torch.tensor(full).to(torch.bfloat16).cuda()
+    F = nb.nn.functional
+
+    for sliced in (False, True):
+        engine.clear_plan_cache()
+        src = nb.Tensor.from_dlpack(stored if sliced else stored[:, :, :V].contiguous())
+        lab = nb.Tensor.constant(labels)
+
+        def loss_of(z):
+            logits = nb.slice_tensor(z, [0, 0, 0], [B, S, V]) if sliced else z
+            return F.cross_entropy_loss(logits, lab)
+
+        loss, g = nb.value_and_grad(loss_of)(src)
+        nb.realize_all(loss, g)
+        if _hand_kernels_on():
+            assert 2 in _row_program_kinds(), (sliced, _row_program_kinds())
+        x64 = stored[:, :, :V].double().cpu().numpy().reshape(B * S, V)
+        lse = torch.logsumexp(torch.tensor(x64), 1).numpy()
+        want_loss = float((lse - x64[np.arange(B * S), labels.reshape(-1)]).sum() / B)
+        p = np.exp(x64 - lse[:, None])
+        p[np.arange(B * S), labels.reshape(-1)] -= 1.0
+        got = nb.cast(g, nb.DType.float32).numpy()
+        assert abs(loss.item() - want_loss) <= 2.0 ** -8 * abs(want_loss)
+        assert relerr(got[:, :, :V].reshape(B * S, V), p / B) <= BF16_TOL
+        if sliced:
+            assert (got[:, :, V:] == 0).all()      # columns the loss never saw
+    engine.clear_plan_cache()
+
+
 def test_cross_entropy_rows_with_infinities_nans_and_labels_out_of_range(hip):
     """What the hand-scheduled cross-entropy kernel makes of rows the arithmetic breaks down on is
     what the interpreter makes of them: a row with +inf or NaN, or of nothing but -inf, is NaN in
