@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 22
+#define NBK_ABI_VERSION 23
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -252,6 +252,11 @@ enum nbk_gemm_residual_op { NBK_RES_ADD = 0, NBK_RES_MUL = 1 };
  * gelu(x @ W + b) multiplies the cotangent with: nabla/ops/unary.py:567-595), taken from the
  * fp32 accumulator like C itself, so that the pre-activation never makes a trip through memory */
 enum nbk_gemm_aux_op { NBK_AUX_NONE = 0, NBK_AUX_ACT_GRAD = 1 };
+#define NBK_GEMM_MAX_TERMS 4
+typedef struct nbk_gemm_term {
+  const void* A; const void* B;
+  int64_t K, a_rs, a_cs, b_rs, b_cs;
+} nbk_gemm_term;
 typedef struct nbk_gemm_desc {
   const void* A; const void* B; void* C;
   const void* bias;      /* NULL or [N] (dtype_c), added to every row        */
@@ -280,17 +285,23 @@ typedef struct nbk_gemm_desc {
    * 16-byte aligned, K % 64 == 0, M % 8 == 0, N % 8 == 0, alpha 1, no bias / residual / activation,
    * one batch level; anything else is an error. */
   void* colsum;
-  /* K2 > 0: a second, shallow operand pair whose product joins the accumulator before the
-   * epilogue, C = act(alpha * (A @ B + A2 @ B2) + bias) ...: A2 is M x K2 with strides
-   * (a2_rs, a2_cs), B2 is K2 x N with (b2_rs, b2_cs), one unit stride each.  This is the update
-   * of a low-rank adapter inside its base product, x @ W + (x @ A) @ B
-   * (nabla/nn/finetune/lora.py:55-79): the sum is rounded once and the base product makes no
-   * trip through memory.  bf16 operands, batch 1, no column sums.  Where the pair is laid out like
-   * A and B, 16-byte aligned and K2 <= 64, K2 % 8 == 0, it is one more K tile of the same launch;
-   * otherwise two launches give the same sum (plain products only: no bias, residual,
-   * activation or alpha then). */
-  const void* A2; const void* B2;
-  int64_t K2, a2_rs, a2_cs, b2_rs, b2_cs;
+  /* n_terms > 0: more operand pairs whose products join the accumulator before the epilogue,
+   *   C = act(alpha * (A @ B + sum_i term[i].A @ term[i].B) + bias) ...
+   * term[i].A is M x term[i].K with strides (a_rs, a_cs), term[i].B is term[i].K x N with
+   * (b_rs, b_cs), one unit stride each.  Two uses: the update of a low-rank adapter inside its
+   * base product, x @ W + (x @ A) @ B (nabla/nn/finetune/lora.py:55-79), and a gradient that
+   * several products contribute to, dq @ Wq^T + dk @ Wk^T + dv @ Wv^T (the cotangent
+   * accumulation of nabla/core/autograd/backward.py:31-54 over MatmulOp.vjp_rule,
+   * nabla/ops/binary.py:303-314): the sum is rounded once and no partial result makes a trip
+   * through memory.  bf16 operands, batch 1, no column sums.  Inside one launch when every pair
+   * is laid out like A and B (same unit-stride side) and 16-byte aligned, with at most two
+   * shallow pairs (K <= 64, K % 8 == 0: one K tile each) and at most two deep ones (K % 64 == 0
+   * and exactly the strides of A and B: their tiles follow those of A and B); otherwise one
+   * launch per pair, each adding itself to the result of the one before (plain products only:
+   * no bias, residual, activation or alpha then). */
+  int32_t n_terms;
+  int32_t reserved2;
+  nbk_gemm_term term[NBK_GEMM_MAX_TERMS];
 } nbk_gemm_desc;
 int nbk_gemm(const nbk_gemm_desc* d, void* stream);
 

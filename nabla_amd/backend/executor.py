@@ -184,15 +184,17 @@ class BoundPlan:
                     if rcs.dtype is not rc.dtype:
                         raise TypeError(f"matmul column sums are {rcs.dtype}, the product {rc.dtype}")
                     ptr_field(d, "colsum", rcs.buf, rcs.offset * rcs.dtype.size_in_bytes)
-                d.A2, d.B2, d.K2 = None, None, 0
-                if a.get("a2") is not None:
-                    ra2, rb2 = a["a2"], a["b2"]
-                    if ra2.dtype is not ra.dtype or rb2.dtype is not ra.dtype:
-                        raise TypeError(f"matmul second pair is {ra2.dtype} / {rb2.dtype}, the first {ra.dtype}")
-                    ptr_field(d, "A2", ra2.buf, ra2.offset * ra2.dtype.size_in_bytes)
-                    ptr_field(d, "B2", rb2.buf, rb2.offset * rb2.dtype.size_in_bytes)
-                    d.K2 = a["K2"]
-                    d.a2_rs, d.a2_cs, d.b2_rs, d.b2_cs = a["a2_rs"], a["a2_cs"], a["b2_rs"], a["b2_cs"]
+                d.n_terms = 0
+                for ti, term in enumerate(a.get("terms") or ()):
+                    ta, tb = term["a"], term["b"]
+                    if ta.dtype is not ra.dtype or tb.dtype is not ra.dtype:
+                        raise TypeError(f"matmul term {ti} is {ta.dtype} / {tb.dtype}, the first pair {ra.dtype}")
+                    t = d.term[ti]
+                    ptr_field(t, "A", ta.buf, ta.offset * ta.dtype.size_in_bytes)
+                    ptr_field(t, "B", tb.buf, tb.offset * tb.dtype.size_in_bytes)
+                    t.K = term["K"]
+                    t.a_rs, t.a_cs, t.b_rs, t.b_cs = term["a_rs"], term["a_cs"], term["b_rs"], term["b_cs"]
+                    d.n_terms = ti + 1
                 self.calls.append((L.nbk_gemm, [C.byref(d)], patches, d))
             elif k == "gemm_nf4":
                 d = lib.GemmNf4Desc()

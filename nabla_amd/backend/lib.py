@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 22
+ABI_VERSION = 23
 
 MAX_RANK = 8
 
@@ -55,6 +55,13 @@ class RowProg(C.Structure):
     ]
 
 
+class GemmTerm(C.Structure):
+    _fields_ = [
+        ("A", C.c_void_p), ("B", C.c_void_p),
+        ("K", C.c_int64), ("a_rs", C.c_int64), ("a_cs", C.c_int64), ("b_rs", C.c_int64), ("b_cs", C.c_int64),
+    ]
+
+
 class GemmDesc(C.Structure):
     _fields_ = [
         ("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p),
@@ -69,9 +76,8 @@ class GemmDesc(C.Structure):
         ("alpha", C.c_float), ("residual_op", C.c_int32),
         ("C_aux", C.c_void_p), ("aux_op", C.c_int32), ("reserved", C.c_int32),
         ("colsum", C.c_void_p),
-        ("A2", C.c_void_p), ("B2", C.c_void_p),
-        ("K2", C.c_int64), ("a2_rs", C.c_int64), ("a2_cs", C.c_int64), ("b2_rs", C.c_int64),
-        ("b2_cs", C.c_int64),
+        ("n_terms", C.c_int32), ("reserved2", C.c_int32),
+        ("term", GemmTerm * 4),
     ]
 
 

@@ -900,7 +900,8 @@ class Planner:
         """``x @ W + u @ V`` with ``u @ V`` at most one K tile deep (the update of a low-rank
         adapter on top of its base product, already folded by `_fold_sum_into_matmul` into a
         thin product that reads the base product as its residual): the node turns into the base
-        product with ``(u, V)`` as a second operand pair (``attrs["pair_in"]``), which the
+        product with ``(u, V)`` as one more operand pair (``attrs["terms_in"]``: the index of the first of the
+        pairs that follow the base product's own inputs), which the
         kernel multiplies as one more K tile into the same accumulator.  The base product no
         longer makes a trip through memory (one write and one read of the result saved, and
         the thin product's launch), and the sum is rounded once.  Only plain products on both
@@ -941,7 +942,7 @@ class Planner:
             k2 = u.shape[-1]
             if not (base.kind == "matmul" and len(base.outputs) == 1 and
                     len(base.inputs) == (3 if "bias_in" in bat else 2) and
-                    not (set(bat) & {"res_in", "act", "pair_in"}) and
+                    not (set(bat) & {"res_in", "act", "terms_in"}) and
                     bat.get("alpha", 1.0) == 1.0 and
                     n_users.get(r.id) == 1 and r.id not in out_ids and
                     k2 <= 64 and k2 % 8 == 0 and one_matrix(v) and one_matrix(base.inputs[1]) and
@@ -950,7 +951,7 @@ class Planner:
                     all(x.dtype is DType.bfloat16 for x in (u, v, r, *base.inputs, n.outputs[0]))):
                 continue
             n.inputs = list(base.inputs) + [u, v]
-            n.attrs = dict(bat, pair_in=len(base.inputs))
+            n.attrs = dict(bat, terms_in=len(base.inputs))
 
         # ``(X + u @ V) + x @ W``: contributions to one gradient arrive in the order of the
         # backward pass, and a thin product whose base product comes one link later in the chain
@@ -974,7 +975,7 @@ class Planner:
         for thin in nodes:
             tat = thin.attrs or {}
             if not (thin.kind == "matmul" and len(thin.inputs) == 2 and len(thin.outputs) == 1 and
-                    not (set(tat) & {"res_in", "bias_in", "act", "pair_in"}) and
+                    not (set(tat) & {"res_in", "bias_in", "act", "terms_in"}) and
                     tat.get("alpha", 1.0) == 1.0):
                 continue
             u, v = thin.inputs
@@ -993,7 +994,7 @@ class Planner:
             base = b_out.node
             bat = base.attrs or {}
             if not (base.kind == "matmul" and base is not thin and len(base.outputs) == 1 and
-                    len(base.inputs) == 2 and not (set(bat) & {"res_in", "bias_in", "act", "pair_in"}) and
+                    len(base.inputs) == 2 and not (set(bat) & {"res_in", "bias_in", "act", "terms_in"}) and
                     bat.get("alpha", 1.0) == 1.0 and only_reader(b_out) is outer and
                     base.pos > thin.pos and base.inputs[0].shape[-1] % 64 == 0 and
                     one_matrix(base.inputs[1]) and u.shape[:-1] == base.inputs[0].shape[:-1] and
@@ -1002,13 +1003,133 @@ class Planner:
                                                              inner.outputs[0], outer.outputs[0]))):
                 continue
             base.inputs = list(base.inputs) + [u, v]
-            base.attrs = dict(bat, pair_in=2)
+            base.attrs = dict(bat, terms_in=2)
             outer.inputs = [x_val, b_out]
             outer.attrs = dict(outer.attrs, operands=(x_val, b_out))
             users[b_out.id] = [outer]
             users[x_val.id] = [z for z in users.get(x_val.id, []) if z is not inner] + [outer]
             users[t_out.id] = []
             users[inner.outputs[0].id] = []
+
+    def _fold_product_sums(self) -> None:
+        """``x1 @ W1 + x2 @ W2 (+ x3 @ W3)``: a value that several products contribute to (the
+        gradient of an activation that feeds the query, key and value projections:
+        ``dq @ Wq^T + dk @ Wk^T + dv @ Wv^T``) is ONE product over the contraction indices of all
+        pairs (`nbk_gemm_desc.term`): one launch with one prologue and one epilogue instead of
+        three, one result instead of three results and the kernel that adds them.  Two shapes of
+        the sum are folded, repeatedly: ``P + Q`` (the add node becomes the product) and
+        ``(X + P) + Q`` with anything for ``X`` (contributions arrive in the order of the
+        backward pass; the later product takes the earlier one's pairs where it stands and the
+        outer sum reads ``X``).  Only plain bf16 products with one reader each, whose right
+        operands are one matrix; at most three pairs a K tile or more deep and two shallower
+        ones (what one launch takes; the kernel wants the deep pairs laid out alike, which
+        holds for the projections of one activation and is checked by the library, which runs
+        one launch per pair otherwise)."""
+        out_ids = {v.id for v in self.outputs}
+
+        def one_matrix(w: ir.Value) -> bool:
+            while w.rank > 2:
+                m = w.node
+                if m.kind == "permute":
+                    perm = tuple(m.attrs["perm"])
+                    if perm[:-2] != tuple(range(w.rank - 2)):
+                        return False
+                    w = m.inputs[0]
+                elif m.kind == "broadcast" and m.inputs[0].rank == 2 and \
+                        tuple(m.inputs[0].shape) == tuple(w.shape[-2:]):
+                    return True
+                else:
+                    return False
+            return True
+
+        def plain_add(n: ir.Node) -> bool:
+            return (n.kind == "ew" and n.fn == "add" and len(n.inputs) == 2 and
+                    all(isinstance(x, ir.Value) for x in n.attrs["operands"]))
+
+        def pairs_of(mm: ir.Node):
+            ins = mm.inputs
+            return [(ins[0], ins[1])] + list(zip(ins[2::2], ins[3::2]))
+
+        changed = True
+        while changed:
+            changed = False
+            nodes = self._live_nodes()
+            users: dict[int, list[ir.Node]] = {}
+            for n in nodes:
+                for i in n.inputs:
+                    users.setdefault(i.id, []).append(n)
+
+            def only_reader(val: ir.Value):
+                us = users.get(val.id, [])
+                return us[0] if len(us) == 1 and val.id not in out_ids else None
+
+            def product(val: ir.Value, reader: ir.Node) -> bool:
+                mm = val.node
+                at = mm.attrs or {}
+                if not (mm.kind == "matmul" and len(mm.outputs) == 1 and only_reader(val) is reader and
+                        not (set(at) - {"terms_in", "alpha"}) and at.get("alpha", 1.0) == 1.0 and
+                        at.get("terms_in", 2) == 2 and len(mm.inputs) % 2 == 0 and
+                        val.dtype is DType.bfloat16):
+                    return False
+                for u, v in pairs_of(mm):
+                    if not (u.dtype is DType.bfloat16 and v.dtype is DType.bfloat16 and one_matrix(v) and
+                            u.shape[:-1] == mm.inputs[0].shape[:-1] and u.shape[-1] % 8 == 0):
+                        return False
+                return mm.inputs[0].shape[-1] % 64 == 0
+
+            def fits(pairs) -> bool:
+                deep = [u for u, _ in pairs if u.shape[-1] > 64]
+                shallow = [u for u, _ in pairs if u.shape[-1] <= 64]
+                return (1 <= len(deep) <= 3 and len(shallow) <= 2 and
+                        all(u.shape[-1] % 64 == 0 for u in deep))
+
+            def merged_inputs(first: ir.Node, second: ir.Node):
+                """Pairs of both products, a deep one of the product that stays first."""
+                pairs = pairs_of(first) + pairs_of(second)
+                return [x for pair in pairs for x in pair] if fits(pairs) else None
+
+            for n in nodes:
+                if not plain_add(n):
+                    continue
+                x, y = n.inputs
+                if x.shape != y.shape or x.shape != n.outputs[0].shape:
+                    continue
+                # P + Q: the add node becomes the product
+                if product(x, n) and product(y, n) and x.node is not y.node:
+                    ins = merged_inputs(x.node, y.node)
+                    if ins is not None:
+                        n.kind, n.fn = "matmul", None
+                        n.inputs = ins
+                        n.attrs = dict(terms_in=2)
+                        changed = True
+                        break
+                # (X + P) + Q, either way round
+                done = False
+                for inner_v, q in ((x, y), (y, x)):
+                    inner = inner_v.node
+                    if not (plain_add(inner) and only_reader(inner_v) is n and product(q, n)):
+                        continue
+                    for p_v, other in ((inner.inputs[0], inner.inputs[1]), (inner.inputs[1], inner.inputs[0])):
+                        if not (product(p_v, inner) and p_v.node is not q.node and
+                                other.shape == n.outputs[0].shape and other.id != q.id):
+                            continue
+                        first, second = (q.node, p_v.node)       # the later one keeps its place
+                        later = first if first.pos > second.pos else second
+                        earlier = second if later is first else first
+                        ins = merged_inputs(later, earlier)
+                        if ins is None:
+                            continue
+                        later.inputs = ins
+                        later.attrs = dict(terms_in=2)
+                        keep = later.outputs[0]
+                        n.inputs = [other, keep]
+                        n.attrs = dict(n.attrs, operands=(other, keep))
+                        changed = done = True
+                        break
+                    if done:
+                        break
+                if done:
+                    break
 
     def _fold_scale_into_matmul(self) -> None:
         """``(x @ W) * c`` with ``c`` a number: the multiply node turns into the product with
@@ -1607,11 +1728,10 @@ class Planner:
             pb = self._mat_operand(rb)
         M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
         batch = _numel(out.shape[:-2])
-        if "pair_in" in at:
-            # x[.., M, K] @ W + u[.., M, K2] @ V with 2-D W and V: one unbatched product over all
-            # rows, for which x and u are read as whole row-major blocks (copied if they are not)
-            u, v = n.inputs[at["pair_in"]], n.inputs[at["pair_in"] + 1]
-
+        if "terms_in" in at:
+            # x[.., M, K] @ W + sum_i u_i[.., M, K_i] @ V_i with 2-D W and V_i: one unbatched
+            # product over all rows, for which x and the u_i are read as whole row-major blocks
+            # (copied if they are not)
             def rows_of(val, ref):
                 if isinstance(ref, Const):
                     ref = self._materialize(ref)
@@ -1624,14 +1744,12 @@ class Planner:
                     po = self._mat_operand(ref)
                 return ref, po
 
-            ra, pa = rows_of(a, ra)
-            ru, pu = rows_of(u, self._resolve(u))
             def one_matrix(val, ref):
                 if isinstance(ref, Const):
                     ref = self._materialize(ref)
                 if val.rank > 2:  # (broadcast over the batch axes: any one of the copies)
                     if any(st != 0 for d, st in zip(ref.shape[:-2], ref.strides[:-2]) if d > 1):
-                        raise AssertionError("paired product: the right operand is not one matrix")
+                        raise AssertionError("product with several operand pairs: a right operand is not one matrix")
                     ref = ViewRef(ref.buf, ref.offset, ref.shape[-2:], ref.strides[-2:], ref.dtype)
                 po = self._mat_operand(ref)
                 if po is None:
@@ -1639,9 +1757,15 @@ class Planner:
                     po = self._mat_operand(ref)
                 return ref, po
 
+            ra, pa = rows_of(a, ra)
             rb, pb = one_matrix(b, rb)
-            rv, pv = one_matrix(v, self._resolve(v))
-            epi.update(a2=ru, b2=rv, K2=u.shape[-1], a2_rs=pu[1], a2_cs=pu[2], b2_rs=pv[1], b2_cs=pv[2])
+            terms = []
+            extra = n.inputs[at["terms_in"]:]
+            for u, v in zip(extra[0::2], extra[1::2]):
+                ru, pu = rows_of(u, self._resolve(u))
+                rv, pv = one_matrix(v, self._resolve(v))
+                terms.append(dict(a=ru, b=rv, K=u.shape[-1], a_rs=pu[1], a_cs=pu[2], b_rs=pv[1], b_cs=pv[2]))
+            epi["terms"] = terms
             self._emit_plain_gemm(ra, rb, pa, pb, M * batch, N, K, out, epi)
             return
         # sum_b A[b] @ B[b] (the weight gradient x^T dy of a layer applied to a batch) is one
@@ -1788,7 +1912,8 @@ class Planner:
 
     @staticmethod
     def _epi_bufs(epi: dict) -> list[int]:
-        return [epi[k].buf for k in ("bias", "residual", "a2", "b2") if k in epi]
+        return [epi[k].buf for k in ("bias", "residual") if k in epi] + \
+            [t[k].buf for t in epi.get("terms", ()) for k in ("a", "b")]
 
     # ................................................................ attention
     def _heads_operand(self, v: ir.Value) -> ViewRef:
@@ -2541,6 +2666,8 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
         pre._fold_sum_into_matmul(thin_only=not config.FOLD_RESIDUAL)
         if config.FOLD_THIN_PAIR:
             pre._fold_thin_pair_into_matmul()
+            if config.FOLD_PRODUCT_SUMS:
+                pre._fold_product_sums()
         pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)
     if config.FOLD_ACTIVATION:
         pre._fold_activation_into_matmul()

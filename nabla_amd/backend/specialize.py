@@ -493,6 +493,8 @@ def collect_programs() -> dict[int, dict]:
         jobs.append(with_flags(jobs[2], FUSED_ATTENTION=False))
         jobs.append(with_flags(jobs[4], FUSED_ATTENTION=False, LORA_LOW_RANK_ORDER=False))
         jobs.append(with_flags(jobs[4], FOLD_THIN_PAIR=False))
+        jobs.append(with_flags(jobs[4], FOLD_PRODUCT_SUMS=False))
+        jobs.append(with_flags(jobs[2], FOLD_PRODUCT_SUMS=False))
         for job in jobs:
             clear_plan_cache()
             res = job()

@@ -61,6 +61,12 @@ _FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
 _FOLD_THIN_PAIR: ContextVar[bool] = ContextVar(
     "FOLD_THIN_PAIR", default=_env_flag("NBK_FOLD_THIN_PAIR", True))
 
+# x1 @ W1 + x2 @ W2 (+ x3 @ W3), products that contribute to one value (the gradient of an
+# activation that feeds several projections), as ONE product over all their contraction indices
+# (`nbk_gemm_desc.term`); off: one product each and the kernel that adds them
+_FOLD_PRODUCT_SUMS: ContextVar[bool] = ContextVar(
+    "FOLD_PRODUCT_SUMS", default=_env_flag("NBK_FOLD_PRODUCT_SUMS", True))
+
 # the column sums of dy (a bias gradient) as one more result of the weight-gradient product
 # x^T dy that reads dy anyway; off: the reduction kernels read dy a second time
 _FOLD_COLUMN_SUMS: ContextVar[bool] = ContextVar(
@@ -96,6 +102,7 @@ _FLAGS = {
     "FOLD_RESIDUAL": _FOLD_RESIDUAL,
     "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
     "FOLD_THIN_PAIR": _FOLD_THIN_PAIR,
+    "FOLD_PRODUCT_SUMS": _FOLD_PRODUCT_SUMS,
     "FOLD_SCALE": _FOLD_SCALE,
     "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
     "VMAP_BATCHED": _VMAP_BATCHED,

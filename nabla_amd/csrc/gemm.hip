@@ -59,10 +59,15 @@ struct GemmArgs {
   int32_t b_block;
   int32_t c_stream;      // C is larger than the last-level cache: store it with the non-temporal hint
   void* colsum;          // null, or [batch][N] in C's dtype: the column sums of B over K
-  // a second, shallow operand pair whose product joins the accumulator: C = A B + A2 B2
-  // (K2 <= 64 deep; oriented like A and B; 0 = none).  Direct-to-LDS kernels only.
-  const void* A2; const void* B2;
-  int64_t K2, a2_rs, a2_cs, b2_rs, b2_cs;
+  // More operand pairs whose products join the accumulator: C = A B + sum_i A_i B_i, all
+  // oriented like A and B.  Direct-to-LDS kernels only.
+  //   shallow pairs (n_shallow <= 2; K <= 64 each, own strides): one K tile each, the first tiles
+  //   of the launch;
+  //   deep pairs (n_deep <= 2; K % 64 == 0, the strides of A and B): their K tiles follow those
+  //   of A and B.
+  struct Shallow { const void* A; const void* B; int64_t K, a_rs, a_cs, b_rs, b_cs; } shallow[2];
+  struct Deep { const void* A; const void* B; int64_t K; } deep[2];
+  int32_t n_shallow, n_deep;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act) {
@@ -940,23 +945,55 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   using LB = DirectLoader<BN, B_KC, NW, MI16>;
   LA la;
   LB lb;
-  int64_t nk = g.K / 64;
-  if (g.K2 > 0) {
-    // the shallow second pair is K tile 0 (its offsets are dead before the loop's are made);
-    // the tiles of A and B follow as tiles 1 .. K / 64
-    LA::issue_tail(gemm_lds, (const uint16_t*)g.A2, g.a2_rs, g.a2_cs, m0, g.M, (int)g.K2, wave, lane);
-    LB::issue_tail(gemm_lds + CA, (const uint16_t*)g.B2, g.b2_cs, g.b2_rs, n0, g.N, (int)g.K2, wave,
-                   lane);
-    la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
-    lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
-    la.base -= la.kstep;
-    lb.base -= lb.kstep;
-    nk += 1;
-  } else {
-    la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
-    lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
-    la.issue(gemm_lds, 0);
-    lb.issue(gemm_lds + CA, 0);
+  // K tiles of the launch: the shallow pairs (one tile each; their offsets are dead before the
+  // loop's are made), then A and B, then the deep pairs, which share the loop's lane offsets and
+  // differ in the wave-uniform base only.  src_a(t) / src_b(t): where tile t starts in memory.
+  // (tile numbers are 32-bit: the scalar unit compares those, 64-bit ones go through vector registers)
+  const int ns = g.n_shallow;
+  const int e0 = ns + (int)(g.K / 64);                                   // first tile past A and B
+  const int e1 = e0 + (g.n_deep > 0 ? (int)(g.deep[0].K / 64) : 0);      // ... past the first deep pair
+  const int nk = e1 + (g.n_deep > 1 ? (int)(g.deep[1].K / 64) : 0);
+  if (ns > 0) {
+    const auto& t0 = g.shallow[0];
+    LA::issue_tail(gemm_lds, (const uint16_t*)t0.A, t0.a_rs, t0.a_cs, m0, g.M, (int)t0.K, wave, lane);
+    LB::issue_tail(gemm_lds + CA, (const uint16_t*)t0.B, t0.b_cs, t0.b_rs, n0, g.N, (int)t0.K, wave, lane);
+  }
+  if (ns > 1) {
+    const auto& t1 = g.shallow[1];
+    LA::issue_tail(gemm_lds + TILE_CHUNKS, (const uint16_t*)t1.A, t1.a_rs, t1.a_cs, m0, g.M, (int)t1.K,
+                   wave, lane);
+    LB::issue_tail(gemm_lds + TILE_CHUNKS + CA, (const uint16_t*)t1.B, t1.b_cs, t1.b_rs, n0, g.N,
+                   (int)t1.K, wave, lane);
+  }
+  la.init(A, g.a_rs, g.a_cs, m0, g.M, wave, lane);
+  lb.init(B, g.b_cs, g.b_rs, n0, g.N, wave, lane);
+  // base of every run of tiles, moved back by the tiles before it, so that tile t of the launch
+  // is at base + t * kstep whichever run it belongs to (wave-uniform values, held in scalar
+  // registers as 64-bit integers: the K loop has no vector register to spare)
+  auto uniform = [](const char* p) {
+    const uint64_t b = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  };
+  const uint64_t a_run0 = uniform(la.base - ns * la.kstep), b_run0 = uniform(lb.base - ns * lb.kstep);
+  uint64_t a_run1 = a_run0, b_run1 = b_run0, a_run2 = a_run0, b_run2 = b_run0;
+  if (g.n_deep > 0) {
+    a_run1 = uniform(la.base + ((const char*)g.deep[0].A - (const char*)A) - (int64_t)e0 * la.kstep);
+    b_run1 = uniform(lb.base + ((const char*)g.deep[0].B - (const char*)B) - (int64_t)e0 * lb.kstep);
+  }
+  if (g.n_deep > 1) {
+    a_run2 = uniform(la.base + ((const char*)g.deep[1].A - (const char*)A) - (int64_t)e1 * la.kstep);
+    b_run2 = uniform(lb.base + ((const char*)g.deep[1].B - (const char*)B) - (int64_t)e1 * lb.kstep);
+  }
+  const int64_t a_kstep = la.kstep, b_kstep = lb.kstep;
+#define GEMM_SRC_A(t) ((const char*)(((t) < e0 ? a_run0 : ((t) < e1 ? a_run1 : a_run2)) + (uint64_t)((int64_t)(t) * a_kstep)))
+#define GEMM_SRC_B(t) ((const char*)(((t) < e0 ? b_run0 : ((t) < e1 ? b_run1 : b_run2)) + (uint64_t)((int64_t)(t) * b_kstep)))
+  if (ns == 0) {
+    const char* sa = GEMM_SRC_A(0);
+    const char* sb = GEMM_SRC_B(0);
+    static_for<LA::N>([&](auto j) { la.template issue_one<decltype(j)::value>(gemm_lds, sa); });
+    static_for<LB::N>([&](auto j) { lb.template issue_one<decltype(j)::value>(gemm_lds + CA, sb); });
   }
 
   // Fragment addresses, one per block row / column of the wave tile.  32 x 32 x 16:
@@ -1107,11 +1144,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   // have the whole of tile kt + 1 to land.
   tile_barrier();
   static_for<NFRAG>([&](auto r) { read_frag(S0{}, r, gemm_lds, 0); });
-  if (nk > 1) {
-    la.issue(gemm_lds + TILE_CHUNKS, 1);
-    lb.issue(gemm_lds + TILE_CHUNKS + CA, 1);
+  if (nk > 1 && ns < 2) {
+    const char* sa = GEMM_SRC_A(1);
+    const char* sb = GEMM_SRC_B(1);
+    static_for<LA::N>([&](auto j) { la.template issue_one<decltype(j)::value>(gemm_lds + TILE_CHUNKS, sa); });
+    static_for<LB::N>([&](auto j) { lb.template issue_one<decltype(j)::value>(gemm_lds + TILE_CHUNKS + CA, sb); });
   }
-  for (int64_t kt = 0; kt + 1 < nk; ++kt) {
+  for (int kt = 0; kt + 1 < nk; ++kt) {
     u32x4* cur = gemm_lds + (kt & 1) * TILE_CHUNKS;
     const u32x4* nxt = gemm_lds + ((kt + 1) & 1) * TILE_CHUNKS;
     static_for<NSTEP - 1>([&](auto st) {
@@ -1128,9 +1167,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
       // (the last pass has no tile kt + 2: it fetches tile nk - 1 again, into a buffer that
       // is not read any more, which keeps this block free of branches)
       constexpr int NL = LA::N + LB::N, H = NMFMA / 2;
-      const int64_t k2 = kt + 2 < nk ? kt + 2 : nk - 1;
-      const char* src_a = la.tile_src(k2);
-      const char* src_b = lb.tile_src(k2);
+      const int k2 = kt + 2 < nk ? kt + 2 : nk - 1;
+      const char* src_a2 = GEMM_SRC_A(k2);
+      const char* src_b2 = GEMM_SRC_B(k2);
       static_for<H>([&](auto q) {
         constexpr int Q = decltype(q)::value;
         static_for<NFRAG>([&](auto r) {
@@ -1140,8 +1179,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
         static_for<NL>([&](auto l) {
           constexpr int L = decltype(l)::value;
           if constexpr (L >= NL * Q / H && L < NL * (Q + 1) / H) {
-            if constexpr (L < LA::N) la.template issue_one<L>(cur, src_a);
-            else lb.template issue_one<L - LA::N>(cur + CA, src_b);
+            if constexpr (L < LA::N) la.template issue_one<L>(cur, src_a2);
+            else lb.template issue_one<L - LA::N>(cur + CA, src_b2);
           }
         });
         mfma(S1{}, std::integral_constant<int, Q + H>{});
@@ -1178,6 +1217,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_dl_kernel(const GemmArgs g)
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no copy may land in a slab
   __syncthreads();  // the epilogue reuses the tile buffers as per-wave slabs
   gemm_epilogue<TM, TN, WN, true, EPI>(acc, g, m0, n0, wm, wn, c_off, wave, lane);
+#undef GEMM_SRC_A
+#undef GEMM_SRC_B
 }
 
 // ------------------------------------------------------------------- bf16, K <= 16
@@ -1820,13 +1861,17 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
   // K-contiguous when the stride along k is 1 (ties: a single row / column counts as K-contiguous)
   const bool akc = d->a_cs == 1;
   const bool bkc = d->b_rs == 1;
-  const bool tail = d->K2 > 0;
+  NBK_REQUIRE(d->n_terms >= 0 && d->n_terms <= NBK_GEMM_MAX_TERMS, "gemm: n_terms %d", d->n_terms);
+  const bool tail = d->n_terms > 0;
   if (tail) {
-    NBK_REQUIRE(d->A2 && d->B2, "gemm: K2 = %lld without A2 / B2", (long long)d->K2);
     NBK_REQUIRE(d->dtype_ab == NBK_BF16 && d->batch == 1 && d->colsum == nullptr,
-                "gemm: a second operand pair goes with one bf16 product without column sums");
-    NBK_REQUIRE(d->a2_rs == 1 || d->a2_cs == 1, "gemm: A2 needs a unit stride");
-    NBK_REQUIRE(d->b2_rs == 1 || d->b2_cs == 1, "gemm: B2 needs a unit stride");
+                "gemm: more operand pairs go with one bf16 product without column sums");
+    for (int i = 0; i < d->n_terms; ++i) {
+      const nbk_gemm_term& t = d->term[i];
+      NBK_REQUIRE(t.A && t.B && t.K > 0, "gemm: term %d is empty", i);
+      NBK_REQUIRE(t.a_rs == 1 || t.a_cs == 1, "gemm: A of term %d needs a unit stride", i);
+      NBK_REQUIRE(t.b_rs == 1 || t.b_cs == 1, "gemm: B of term %d needs a unit stride", i);
+    }
   }
   const int esz = d->dtype_ab == NBK_F32 ? 4 : 2;
   auto vec_ok = [&](const void* p, int64_t other_stride, int64_t bs, int64_t bs2) {
@@ -1901,34 +1946,50 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
                       (bkc || d->N % 8 == 0) && d->M >= 8 && d->N >= 8 &&
                       a_stride >= 0 && b_stride >= 0 && a_stride < (1 << 22) && b_stride < (1 << 22);
     if (tail) {
-      // In the accumulator of the direct-to-LDS kernels when the pair is laid out like A and B,
-      // at most one K tile deep and 16-byte aligned; otherwise as a second product that adds
-      // itself to the first (a plain one only: the epilogue would have to wait for it).
-      const bool a2kc = d->a2_cs == 1, b2kc = d->b2_rs == 1;
-      const int64_t a2_stride = a2kc ? d->a2_rs : d->a2_cs, b2_stride = b2kc ? d->b2_cs : d->b2_rs;
-      const bool inside = fast && a2kc == akc && b2kc == bkc && d->K2 <= 64 && d->K2 % 8 == 0 &&
-                          ((uintptr_t)d->A2 % 16 == 0) && ((uintptr_t)d->B2 % 16 == 0) &&
-                          a2_stride % 8 == 0 && b2_stride % 8 == 0 && a2_stride >= 0 &&
-                          b2_stride >= 0 && a2_stride < (1 << 22) && b2_stride < (1 << 22) &&
-                          d->M >= 128 && d->N >= 128;
-      if (inside) {
-        a.A2 = d->A2; a.B2 = d->B2; a.K2 = d->K2;
-        a.a2_rs = d->a2_rs; a.a2_cs = d->a2_cs; a.b2_rs = d->b2_rs; a.b2_cs = d->b2_cs;
-      } else {
+      // In the accumulator of the direct-to-LDS kernels when every pair is laid out like A and B
+      // and 16-byte aligned: shallow pairs (one K tile each, at most two) and deep pairs with
+      // exactly the strides of A and B (at most two); otherwise one product after the other,
+      // each adding itself to the result so far (plain products only: an epilogue would have to
+      // wait for the last one).
+      bool inside = fast && d->M >= 128 && d->N >= 128;
+      a.n_shallow = 0;
+      a.n_deep = 0;
+      for (int i = 0; inside && i < d->n_terms; ++i) {
+        const nbk_gemm_term& t = d->term[i];
+        const bool tkc_a = t.a_cs == 1, tkc_b = t.b_rs == 1;
+        const int64_t sa = tkc_a ? t.a_rs : t.a_cs, sb = tkc_b ? t.b_cs : t.b_rs;
+        if (tkc_a != akc || tkc_b != bkc || ((uintptr_t)t.A & 15) || ((uintptr_t)t.B & 15) || sa % 8 ||
+            sb % 8 || sa < 0 || sb < 0 || sa >= (1 << 22) || sb >= (1 << 22)) {
+          inside = false;
+        } else if (t.K <= 64 && t.K % 8 == 0 && a.n_shallow < 2) {
+          GemmArgs::Shallow& sh = a.shallow[a.n_shallow++];
+          sh.A = t.A; sh.B = t.B; sh.K = t.K;
+          sh.a_rs = t.a_rs; sh.a_cs = t.a_cs; sh.b_rs = t.b_rs; sh.b_cs = t.b_cs;
+        } else if (t.K % 64 == 0 && a.n_deep < 2 && t.a_rs == d->a_rs && t.a_cs == d->a_cs &&
+                   t.b_rs == d->b_rs && t.b_cs == d->b_cs) {
+          GemmArgs::Deep& dp = a.deep[a.n_deep++];
+          dp.A = t.A; dp.B = t.B; dp.K = t.K;
+        } else {
+          inside = false;
+        }
+      }
+      if (!inside) {
         NBK_REQUIRE(d->bias == nullptr && d->residual == nullptr && d->act == NBK_ACT_NONE &&
                         d->C_aux == nullptr && d->alpha == 1.f,
-                    "gemm: a second operand pair outside the direct kernels' conditions goes with a "
-                    "plain product only");
-        nbk_gemm_desc first = *d;
-        first.A2 = nullptr; first.B2 = nullptr; first.K2 = 0;
-        const int rc = nbk_gemm(&first, stream);
-        if (rc != NBK_OK) return rc;
-        nbk_gemm_desc second = first;
-        second.A = d->A2; second.B = d->B2; second.K = d->K2;
-        second.a_rs = d->a2_rs; second.a_cs = d->a2_cs; second.b_rs = d->b2_rs; second.b_cs = d->b2_cs;
-        second.residual = d->C;  // (every kernel reads a residual element in the lane that writes it)
-        second.residual_op = NBK_RES_ADD;
-        return nbk_gemm(&second, stream);
+                    "gemm: operand pairs outside the direct kernels' conditions go with a plain "
+                    "product only");
+        nbk_gemm_desc one = *d;
+        one.n_terms = 0;
+        int rc = nbk_gemm(&one, stream);
+        for (int i = 0; rc == NBK_OK && i < d->n_terms; ++i) {
+          const nbk_gemm_term& t = d->term[i];
+          one.A = t.A; one.B = t.B; one.K = t.K;
+          one.a_rs = t.a_rs; one.a_cs = t.a_cs; one.b_rs = t.b_rs; one.b_cs = t.b_cs;
+          one.residual = d->C;  // (every kernel reads a residual element in the lane that writes it)
+          one.residual_op = NBK_RES_ADD;
+          rc = nbk_gemm(&one, stream);
+        }
+        return rc;
       }
     }
     if (d->colsum != nullptr) {

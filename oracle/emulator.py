@@ -305,10 +305,10 @@ def _gemm(a, mem):
     A = mat(a["a"], a["a_bs"], a.get("a_bs2", 0), a["a_rs"], a["a_cs"], a["M"], a["K"]).float()
     B = mat(a["b"], a["b_bs"], a.get("b_bs2", 0), a["b_rs"], a["b_cs"], a["K"], a["N"]).float()
     prod = torch.matmul(A.double(), B.double())
-    if a.get("a2") is not None:  # a second, shallow pair in the same accumulator (batch 1)
-        A2 = torch.as_strided(mem[a["a2"].buf], (a["M"], a["K2"]), (a["a2_rs"], a["a2_cs"]), a["a2"].offset)
-        B2 = torch.as_strided(mem[a["b2"].buf], (a["K2"], a["N"]), (a["b2_rs"], a["b2_cs"]), a["b2"].offset)
-        prod = prod + torch.matmul(A2.double(), B2.double())
+    for t in a.get("terms") or ():  # more operand pairs in the same accumulator (batch 1)
+        At = torch.as_strided(mem[t["a"].buf], (a["M"], t["K"]), (t["a_rs"], t["a_cs"]), t["a"].offset)
+        Bt = torch.as_strided(mem[t["b"].buf], (t["K"], a["N"]), (t["b_rs"], t["b_cs"]), t["b"].offset)
+        prod = prod + torch.matmul(At.double(), Bt.double())
     C = prod.float() * a.get("alpha", 1.0)
     if a.get("bias") is not None:  # added before the result is rounded, as in the kernel's epilogue
         C = C + _view(mem, a["bias"]).reshape(-1).float()

@@ -48,7 +48,7 @@ STRUCTS = {
     "nbk_gemm_nf4_desc": "GemmNf4Desc", "nbk_conv_desc": "ConvDesc", "nbk_pool_desc": "PoolDesc",
     "nbk_attn_desc": "AttnDesc", "nbk_attn_tensor": "AttnTensor", "nbk_reduce_task": "ReduceTask",
     "nbk_opt_tensor": "OptTensor", "nbk_adamw_desc": "AdamwDesc", "nbk_sgd_desc": "SgdDesc",
-    "nbk_tensor": "TensorDesc",
+    "nbk_tensor": "TensorDesc", "nbk_gemm_term": "GemmTerm",
 }
 
 

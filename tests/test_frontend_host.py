@@ -773,13 +773,15 @@ def test_a_constant_scale_folds_into_the_product_it_multiplies(emulator):
     np.testing.assert_allclose(grads["A"].numpy(), 3.0 * x2.T @ (np.ones((120, 16), np.float32) @ b.T), rtol=1e-4, atol=1e-4)
 
 
-def test_adapter_updates_ride_inside_their_base_products(emulator):
-    """`x @ W + (x @ A) @ B` and its mirror image in the backward pass are ONE product with two
-    operand pairs each (`nbk_gemm_desc.A2 / B2 / K2`): in a two-layer decoder the four forward
-    updates fold onto their base products directly, the two backward ones of the second layer
-    also where the base product comes one link later in the chain of sums.  No thin product is
-    left that reads a base result, the gradients are those of the plan without the fold, and a
-    rank that is no multiple of 8 keeps the thin products."""
+def test_adapter_updates_and_gradient_sums_are_one_product(emulator):
+    """`x @ W + (x @ A) @ B` and its mirror image in the backward pass are ONE product with
+    several operand pairs (`nbk_gemm_desc.term`), and so is a gradient that several products
+    contribute to: in a two-layer decoder the four forward updates fold onto their base products,
+    and the gradient of the second layer's normalised input,
+    `dq Wq^T + (dq Bq^T) Aq^T + dk Wk^T + dv Wv^T + (dv Bv^T) Av^T`, is one launch with three deep
+    and two shallow pairs.  No thin product is left that reads a base result, the gradients are
+    those of the plans without the folds, and a rank that is no multiple of 8 keeps the thin
+    products."""
     from nabla_amd import config
     from nabla_amd.core import engine
 
@@ -793,20 +795,30 @@ def test_adapter_updates_ride_inside_their_base_products(emulator):
         gemms = [s.attrs for s in list(engine._PLAN_CACHE.values())[-1].plan.steps if s.kind == "gemm"]
         return loss.item(), [g.numpy() for g in flat], gemms
 
-    loss_on, g_on, gemms = step(16)
-    paired = [a for a in gemms if a.get("a2") is not None]
-    assert len(paired) == 6
-    assert all(a["K2"] == 16 and a["K"] == 128 and a["batch"] == 1 and a["M"] == 128 for a in paired)
+    def same(got, want):
+        assert abs(got[0] - want[0]) <= 2e-2 * abs(want[0])
+        for a, b in zip(got[1], want[1]):
+            assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max()
+
+    on = step(16)
+    gemms = on[2]
+    with_terms = [a for a in gemms if a.get("terms")]
+    assert sorted(len(a["terms"]) for a in with_terms) == [1, 1, 1, 1, 4]
+    assert all(a["batch"] == 1 and a["M"] == 128 and a["K"] == 128 for a in with_terms)
+    big = [a for a in with_terms if len(a["terms"]) == 4][0]
+    assert sorted(t["K"] for t in big["terms"]) == [16, 16, 128, 128]
     assert not [a for a in gemms if a["K"] <= 16 and a["N"] > 16]      # every update found its base
+    with config.flag("FOLD_PRODUCT_SUMS", False):
+        pairs_only = step(16)
+    assert sorted(len(a["terms"]) for a in pairs_only[2] if a.get("terms")) == [1] * 6
+    assert len(pairs_only[2]) == len(gemms) + 2
+    same(on, pairs_only)
     with config.flag("FOLD_THIN_PAIR", False):
-        loss_off, g_off, gemms_off = step(16)
-    assert not [a for a in gemms_off if a.get("a2") is not None]
-    assert len(gemms_off) == len(gemms) + 6
-    assert abs(loss_on - loss_off) <= 2e-2 * abs(loss_off)
-    for a, b in zip(g_on, g_off):
-        assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max()
-    _, _, gemms4 = step(4)
-    assert not [a for a in gemms4 if a.get("a2") is not None]
+        off = step(16)
+    assert not [a for a in off[2] if a.get("terms")]
+    assert len(off[2]) == len(gemms) + 8
+    same(on, off)
+    assert not [a for a in step(4)[2] if a.get("terms") and any(t["K"] < 64 for t in a["terms"])]
     engine.clear_plan_cache()
 
 

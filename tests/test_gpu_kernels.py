@@ -137,9 +137,11 @@ def test_gemm_with_a_second_operand_pair(hip, layout, shape, k2, how):
     d.M, d.N, d.K = M, N, K
     d.a_rs, d.a_cs = (K, 1) if layout[0] == "n" else (1, M)
     d.b_rs, d.b_cs = (N, 1) if layout[1] == "n" else (1, K)
-    d.A2, d.B2, d.K2 = a2_dev.data_ptr() + a2_off, b2_dev.data_ptr() + b2_off, k2
-    d.a2_rs, d.a2_cs = (k2, 1) if lay2[0] == "n" else (1, M)
-    d.b2_rs, d.b2_cs = (N, 1) if lay2[1] == "n" else (1, k2)
+    d.n_terms = 1
+    t = d.term[0]
+    t.A, t.B, t.K = a2_dev.data_ptr() + a2_off, b2_dev.data_ptr() + b2_off, k2
+    t.a_rs, t.a_cs = (k2, 1) if lay2[0] == "n" else (1, M)
+    t.b_rs, t.b_cs = (N, 1) if lay2[1] == "n" else (1, k2)
     d.ldc = N
     d.batch, d.a_bs, d.b_bs, d.c_bs = 1, 0, 0, 0
     d.dtype_ab = d.dtype_c = 1
@@ -153,6 +155,80 @@ def test_gemm_with_a_second_operand_pair(hip, layout, shape, k2, how):
     # (two launches round the first product to bf16 before the second is added: one more
     # rounding, of a value that may be larger than the sum)
     err = np.abs(got - ref) - 2.0 ** -8 * (np.abs(ref) + np.abs(first))
+    assert err.max() <= 2e-2, err.max()
+
+
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("shape,ks,how", [
+    ((512, 384, 256), (256, 128), "same"),            # two deep pairs behind A and B (128 x 128 tiles)
+    ((1024, 1024, 512), (512, 512, 16, 8), "same"),   # 256 x 256 tiles; two deep, two shallow: all four terms
+    ((4000, 2600, 192), (64, 24), "same"),            # ragged edges; a deep pair of one tile and a shallow one
+    ((1024, 1024, 512), (512, 16), "bias"),
+    ((512, 384, 256), (256, 128, 64), "same"),        # three deep pairs: the third runs as a launch of its own
+    ((512, 384, 256), (256,), "pitch"),               # a deep pair with another row pitch: launch of its own
+    ((512, 384, 256), (16, 16, 8), "same"),           # three shallow pairs: launches of their own
+])
+def test_gemm_with_several_operand_pairs(hip, layout, shape, ks, how):
+    """C = A @ B + sum_i A_i @ B_i through the C ABI (a gradient that several products
+    contribute to, with or without low-rank updates) against float64 of the same bf16 operands:
+    up to two deep pairs laid out like A and B and two shallow ones run inside one launch, whatever
+    else is asked for as one launch per pair that adds itself to the result so far."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(13)
+    bf = torch.bfloat16
+
+    def operands(k, pitch=0):
+        A = torch.tensor(rng.standard_normal((M, k)), dtype=bf)
+        B = torch.tensor(rng.standard_normal((k, N)), dtype=bf)
+        if layout[0] == "n":
+            a_dev = torch.zeros((M, k + pitch), dtype=bf)
+            a_dev[:, :k] = A
+            a_str = (k + pitch, 1)
+        else:
+            a_dev = torch.zeros((k, M + pitch), dtype=bf)
+            a_dev[:, :M] = A.t()
+            a_str = (1, M + pitch)
+        if layout[1] == "n":
+            b_dev = torch.zeros((k, N + pitch), dtype=bf)
+            b_dev[:, :N] = B
+            b_str = (N + pitch, 1)
+        else:
+            b_dev = torch.zeros((N, k + pitch), dtype=bf)
+            b_dev[:, :k] = B.t()
+            b_str = (1, k + pitch)
+        return A, B, a_dev.cuda(), b_dev.cuda(), a_str, b_str
+
+    main = operands(K)
+    terms = [operands(k, 8 if how == "pitch" else 0) for k in ks]
+    parts = [(main[0].double() @ main[1].double()).numpy()] + [(t[0].double() @ t[1].double()).numpy() for t in terms]
+    ref = sum(parts)
+    bias = torch.tensor(rng.standard_normal((N,)) * 4.0, dtype=bf)
+    if how == "bias":
+        ref = ref + bias.double().numpy()
+    bias_dev = bias.cuda()
+    c_dev = torch.full((M, N), float("nan"), dtype=bf, device="cuda")
+    d = lib.GemmDesc()
+    d.A, d.B, d.C = main[2].data_ptr(), main[3].data_ptr(), c_dev.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    (d.a_rs, d.a_cs), (d.b_rs, d.b_cs) = main[4], main[5]
+    d.ldc = N
+    d.batch = 1
+    d.dtype_ab = d.dtype_c = 1
+    d.alpha = 1.0
+    d.n_terms = len(terms)
+    for i, (t, k) in enumerate(zip(terms, ks)):
+        d.term[i].A, d.term[i].B, d.term[i].K = t[2].data_ptr(), t[3].data_ptr(), k
+        (d.term[i].a_rs, d.term[i].a_cs), (d.term[i].b_rs, d.term[i].b_cs) = t[4], t[5]
+    if how == "bias":
+        d.bias = bias_dev.data_ptr()
+    L = lib.load()
+    lib.check(L.nbk_gemm(C.byref(d), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = c_dev.double().cpu().numpy()
+    # (launches of their own round the result so far to bf16 before they add to it)
+    running = np.abs(np.cumsum(np.stack(parts), axis=0)).sum(axis=0)
+    err = np.abs(got - ref) - 2.0 ** -8 * (np.abs(ref) + running)
     assert err.max() <= 2e-2, err.max()
 
 
@@ -173,15 +249,19 @@ def test_gemm_second_pair_errors(hip):
         d.batch = 1
         d.dtype_ab = d.dtype_c = 1 if t is x else 0
         d.alpha = 1.0
-        d.A2, d.B2, d.K2 = x.data_ptr(), x.data_ptr(), 16
-        d.a2_rs, d.a2_cs, d.b2_rs, d.b2_cs = 16, 1, 256, 1
+        d.n_terms = 1
+        d.term[0].A, d.term[0].B, d.term[0].K = x.data_ptr(), x.data_ptr(), 16
+        d.term[0].a_rs, d.term[0].a_cs, d.term[0].b_rs, d.term[0].b_cs = 16, 1, 256, 1
         for k, v in kw.items():
-            setattr(d, k, v)
+            if k.startswith("t0_"):
+                setattr(d.term[0], k[3:], v)
+            else:
+                setattr(d, k, v)
         return d
 
     assert L.nbk_gemm(C.byref(desc()), st) == 0
-    for bad in (desc(A2=None), desc(batch=2), desc(t=x32), desc(a2_rs=16, a2_cs=2),
-                desc(K2=12, act=1),                 # two launches cannot carry an epilogue
+    for bad in (desc(t0_A=None), desc(batch=2), desc(t=x32), desc(t0_a_rs=16, t0_a_cs=2), desc(n_terms=5),
+                desc(t0_K=12, act=1),               # two launches cannot carry an epilogue
                 desc(colsum=x.data_ptr(), a_rs=1, a_cs=256)):
         assert L.nbk_gemm(C.byref(bad), st) != 0
         assert b"gemm" in L.nbk_last_error()
