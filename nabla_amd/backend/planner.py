@@ -1845,7 +1845,8 @@ class Planner:
             alpha=epi.get("alpha", 1.0))))
 
     @staticmethod
-    def _split_k(M: int, N: int, K: int, dtype: DType, a_k_contiguous: bool = False) -> int:
+    def _split_k(M: int, N: int, K: int, dtype: DType, a_k_contiguous: bool = False,
+                 rows_contiguous: bool = False) -> int:
         """Slices of the contraction axis for a product whose output has too few 128 x 128
         tiles to occupy the GPU while K is long (weight gradients: K = batch x sequence)."""
         if dtype is not DType.bfloat16:
@@ -1853,6 +1854,14 @@ class Planner:
         if a_k_contiguous and N <= 32 and M >= 1024 and K % 64 == 0:
             return 1  # tall products with a few columns have a kernel that splits K by itself
         tiles = ((M + 127) // 128) * ((N + 127) // 128)
+        if rows_contiguous and 128 <= tiles <= 256 and K >= 4096 and K % 128 == 0:
+            # x^T dy with one workgroup per CU at most: every workgroup walks the same rows of
+            # both operands at the same time, and on operands that come from memory (written
+            # long before) the launch takes a third longer than on cached ones, whatever the
+            # depth of its prefetch.  Two halves of K put two workgroups on a CU that read 40 MB
+            # apart: 1024 x 4096 x 8192 113 -> 82 us, plus 10 us for the sum of the halves (four
+            # slices: 67 us and 25)
+            return 2
         ks = 1
         while tiles * ks < 512 and tiles < 128 and K % (ks * 2 * 64) == 0 and K // (ks * 2) >= 512:
             ks *= 2
@@ -1883,7 +1892,8 @@ class Planner:
         """One unbatched product into contiguous storage for ``out``; split along K into fp32
         partial products plus their sum when the output alone gives too few workgroups."""
         ks = self._split_k(M, N, K, ra.dtype if ra.dtype is rb.dtype else DType.float32,
-                           a_k_contiguous=pa[2] == 1)
+                           a_k_contiguous=pa[2] == 1,
+                           rows_contiguous=pa[1] == 1 and pa[2] != 1 and pb[2] == 1 and pb[1] != 1)
         dst = self._alloc_value(out)
         common = dict(a=ra, b=rb, M=M, N=N, a_rs=pa[1], a_cs=pa[2], b_rs=pb[1], b_cs=pb[2],
                       batch_inner=1, a_bs2=0, b_bs2=0, c_bs2=0, ldc=N, c_bs=M * N, alpha=1.0)
