@@ -282,8 +282,9 @@ typedef struct nbk_gemm_desc {
    * bias gradient (the reduction of the cotangent to the bias' shape,
    * nabla/core/autograd/backward.py:31-54), taken from the B fragments the product has in
    * registers, so dy is read once.  bf16 operands, both row-contiguous (a_rs == b_cs == 1) and
-   * 16-byte aligned, K % 64 == 0, M % 8 == 0, N % 8 == 0, alpha 1, no bias / residual / activation,
-   * one batch level; anything else is an error. */
+   * 16-byte aligned, K % 64 == 0, M % 8 == 0, N % 8 == 0, alpha 1, no bias / residual / activation;
+   * anything else is an error.  Row b of the sums belongs to batch index b of the launch, also with
+   * two batch levels (b = outer * batch_inner + inner). */
   void* colsum;
   /* n_terms > 0: more operand pairs whose products join the accumulator before the epilogue,
    *   C = act(alpha * (A @ B + sum_i term[i].A @ term[i].B) + bias) ...

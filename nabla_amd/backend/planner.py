@@ -276,6 +276,8 @@ class Planner:
         self.alias_nodes: set[int] = set()  # broadcast nodes fused as row->full aliases
         from .. import config
         self.fold_column_sums = bool(config.FOLD_COLUMN_SUMS)
+        self.group_siblings = bool(config.GROUP_SIBLING_PRODUCTS)
+        self._sibling_groups: dict[int, list] = {}  # id(gemm step) -> members of its launch
 
     # ................................................................ liveness
     def _live_nodes(self) -> list[ir.Node]:
@@ -1507,35 +1509,43 @@ class Planner:
         with room for them (``colsum_key`` on both) become a result of that product's launch:
         the matrix is read once.  A product split along K leaves one row of partial sums per
         slice, which the second stage adds up as it would have the first stage's."""
-        hosts = {}
+        hosts = {}  # key -> (step, member of a joined launch)
         for idx, st in enumerate(self.steps):
-            key = st.attrs.get("colsum_key") if st.kind == "gemm" else None
-            if key is not None and key not in hosts:
-                hosts[key] = idx
+            if st.kind != "gemm":
+                continue
+            keys = st.attrs.get("colsum_keys") or [st.attrs.get("colsum_key")]
+            for member, key in enumerate(keys):
+                if key is not None and key not in hosts:
+                    hosts[key] = (idx, member)
         first, second = self._deferred_reduces
         for task in list(first):
             key = task.attrs.get("colsum_key")
-            idx = hosts.pop(key, None) if key is not None else None
+            idx, member = hosts.pop(key, (None, 0)) if key is not None else (None, 0)
             if idx is None:
                 continue
             host = self.steps[idx]
-            ks, n = host.attrs["batch"], host.attrs["N"]
+            batch, n = host.attrs["batch"], host.attrs["N"]
+            ks = host.attrs["batch_inner"] if "colsum_keys" in host.attrs else batch
             stage2 = task.attrs.get("second")
             final = (stage2 or task).attrs["dst"]
             first.remove(task)
-            if ks == 1:
-                if stage2 is not None:
-                    second.remove(stage2)
+            if stage2 is not None:
+                second.remove(stage2)
+            if batch == 1:
                 target = ViewRef(final.buf, final.offset, (1, n), (n, 1), final.dtype)
             else:
-                tmp = self._new_buf((ks, n), DType.float32)
-                target = ViewRef(tmp.id, 0, (ks, n), (n, 1), DType.float32)
-                if stage2 is not None:
-                    second.remove(stage2)
-                second.append(Step("reduce_mid", [tmp.id], [final.buf], dict(
-                    src=target, dst=final, outer=1, red=ks, inner=n, fn="sum")))
-            host.attrs["colsum"] = target
-            host.writes.append(target.buf)
+                # one row of partial sums per batch index of the launch; a joined launch writes
+                # the rows of all its members, wanted or not
+                target = host.attrs.get("colsum")
+                if target is None:
+                    tmp = self._new_buf((batch, n), DType.float32)
+                    target = ViewRef(tmp.id, 0, (batch, n), (n, 1), DType.float32)
+                rows = ViewRef(target.buf, member * ks * n, (ks, n), (n, 1), DType.float32)
+                second.append(Step("reduce_mid", [target.buf], [final.buf], dict(
+                    src=rows, dst=final, outer=1, red=ks, inner=n, fn="sum")))
+            if host.attrs.get("colsum") is None:
+                host.attrs["colsum"] = target
+                host.writes.append(target.buf)
             b = self.bufs[target.buf]
             b.first, b.last = min(b.first, idx), max(b.last, idx)
 
@@ -1913,12 +1923,92 @@ class Planner:
                             dict(common, **epi, dst=dst, K=K, batch=1, a_bs=0, b_bs=0)))
             return
         kc = K // ks
+        terminal = self._terminal(out)
+        if terminal and not epi and self.group_siblings and \
+                self._join_sibling_product(ra, rb, common, kc, ks, key, dst):
+            return
         tmp = self._new_buf((ks, M, N), DType.float32)
         tref = ViewRef(tmp.id, 0, (ks, M, N), contiguous_strides((ks, M, N)), DType.float32)
-        self._emit(Step("gemm", [ra.buf, rb.buf], [tmp.id], dict(
-            common, dst=tref, K=kc, batch=ks, a_bs=kc * pa[2], b_bs=kc * pb[1])))
-        self._emit_reduce(Step("reduce_mid", [tmp.id], [dst.buf], dict(
-            src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum")), 1, self._terminal(out))
+        step = Step("gemm", [ra.buf, rb.buf], [tmp.id], dict(
+            common, dst=tref, K=kc, batch=ks, a_bs=kc * pa[2], b_bs=kc * pb[1]))
+        self._emit(step)
+        red = Step("reduce_mid", [tmp.id], [dst.buf], dict(
+            src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum"))
+        self._emit_reduce(red, 1, terminal)
+        if terminal and not epi and common["alpha"] == 1.0:
+            # (more may join: _join_sibling_product)
+            self._sibling_groups[id(step)] = [dict(off=rb.offset, key=key, reduce=red)]
+
+    def _join_sibling_product(self, ra: ViewRef, rb: ViewRef, common: dict, kc: int, ks: int, key,
+                              dst: ViewRef) -> bool:
+        """A K-split product A^T B' whose left operand, shape and slices are those of a product
+        among the launches just emitted (nothing but products since), with B' in the same buffer
+        as that one's right operand(s) and equally spaced with them, joins that launch as one
+        more batch member: the batch index becomes (member, slice), the partial products of all
+        members lie in one buffer, and the left operand is read once per cache for all of them
+        (the weight gradients of the q, k and v projections: three launches -> one)."""
+        M, N = common["M"], common["N"]
+        for idx in range(len(self.steps) - 1, -1, -1):
+            st = self.steps[idx]
+            if st.kind != "gemm":
+                return False
+            members = self._sibling_groups.get(id(st))
+            if members is None:
+                continue
+            h = st.attrs
+            n = len(members)
+            ks_h = h["batch_inner"] if n > 1 else h["batch"]
+            hb = h["b"]
+            same = (h["a"] == ra and h["M"] == M and h["N"] == N and h["K"] * ks_h == kc * ks and
+                    all(h[f] == common[f] for f in ("a_rs", "a_cs", "b_rs", "b_cs", "ldc", "alpha")) and
+                    hb.buf == rb.buf and hb.dtype is rb.dtype and
+                    (members[0]["key"] is not None) == (key is not None))
+            if not same:
+                continue
+            # members in the order of their addresses, equally spaced
+            order = sorted(members + [dict(off=rb.offset, key=key, reduce=None)], key=lambda m: m["off"])
+            spacing = order[1]["off"] - order[0]["off"]
+            if spacing <= 0 or spacing % 8 or any(
+                    order[j + 1]["off"] - order[j]["off"] != spacing for j in range(n)):
+                continue
+            # nothing emitted since may write what this member reads
+            if any(w in (ra.buf, rb.buf) for later in self.steps[idx + 1:] for w in later.writes):
+                return False
+            # the launch has the tiles of all its members: fewer slices of K give it three
+            # workgroups for two CUs, and fewer partial products go through memory (three
+            # members of 64 tiles in the transformer block: 8, 4, 2 slices measured, two is best)
+            tiles = -(-M // 128) * -(-N // 128) * (n + 1)
+            k_all, ks_new = kc * ks, 2
+            while tiles * ks_new < 384 and ks_new < ks:
+                ks_new *= 2
+            ks = ks_new if (ks_new < ks and k_all % (ks_new * 64) == 0) else ks
+            kc = k_all // ks
+            tmp = self.bufs[h["dst"].buf]
+            tmp.numel = (n + 1) * ks * M * N
+            tmp.shape = (n + 1, ks, M, N)
+            h.pop("colsum_key", None)
+            h.update(K=kc, batch_inner=ks, a_bs2=kc * common["a_cs"], b_bs2=kc * common["b_rs"],
+                     c_bs2=M * N, a_bs=0, c_bs=ks * M * N)
+            h.update(batch=(n + 1) * ks, b_bs=spacing,
+                     b=ViewRef(hb.buf, order[0]["off"], hb.shape, hb.strides, hb.dtype),
+                     dst=ViewRef(tmp.id, 0, ((n + 1) * ks, M, N),
+                                 contiguous_strides(((n + 1) * ks, M, N)), DType.float32))
+            if key is not None:
+                h["colsum_keys"] = [m["key"] for m in order]
+            for b in (self.bufs[ra.buf], self.bufs[rb.buf]):
+                b.first, b.last = min(b.first, idx), max(b.last, idx)
+            for j, m in enumerate(order):
+                tref = ViewRef(tmp.id, j * ks * M * N, (ks, M, N), contiguous_strides((ks, M, N)),
+                               DType.float32)
+                if m["reduce"] is None:
+                    m["reduce"] = Step("reduce_mid", [tmp.id], [dst.buf], dict(
+                        src=tref, dst=dst, outer=1, red=ks, inner=M * N, fn="sum"))
+                    self._emit_reduce(m["reduce"], 1, True)
+                else:
+                    m["reduce"].attrs.update(src=tref, red=ks)
+            self._sibling_groups[id(st)] = order
+            return True
+        return False
 
     @staticmethod
     def _epi_bufs(epi: dict) -> list[int]:
@@ -1939,10 +2029,10 @@ class Planner:
                 ok = False
         return ref if ok else self._materialize(ref)
 
-    def _heads_result(self, out: ir.Value) -> ViewRef:
-        """Storage for a [B, H, S, hd] result.  When it is read through one permute that keeps
-        hd last (the transpose back to [B, S, H, hd]) it is written in that order, and the
-        permute becomes a contiguous view."""
+    def _heads_layout(self, out: ir.Value):
+        """Strides in which a [B, H, S, hd] result is written, or None for plain contiguous
+        storage.  When it is read through one permute that keeps hd last (the transpose back to
+        [B, S, H, hd]) it is written in that order, and the permute becomes a contiguous view."""
         strides = contiguous_strides(out.shape)
         users = self.users.get(out.id, ())
         perms = [u for u in users if u.kind == "permute"]
@@ -1958,11 +2048,35 @@ class Planner:
                 cand[p] = pst[i]
             strides = tuple(cand)
         if strides == contiguous_strides(out.shape) or any(s % 8 for s in strides[:-1]):
+            return None
+        return strides
+
+    def _heads_result(self, out: ir.Value) -> ViewRef:
+        """Storage for a [B, H, S, hd] result (see ``_heads_layout``)."""
+        strides = self._heads_layout(out)
+        if strides is None:
             return self._alloc_value(out)
         buf = self._new_buf(out.shape, out.dtype, "temp", -1)
         dst = ViewRef(buf.id, 0, out.shape, strides, out.dtype)
         self.loc[out.id] = dst
         return dst
+
+    def _heads_results_side_by_side(self, outs) -> list[ViewRef]:
+        """Storage for dq, dk and dv.  Where all three are written in the transposed order they
+        share one buffer, equally spaced: the weight gradients x^T dq, x^T dk, x^T dv of three
+        projections of one input can then be one batched launch (``_join_sibling_product``)."""
+        lay = [self._heads_layout(t) for t in outs]
+        same = all(l is not None and l == lay[0] for l in lay) and \
+            all(t.shape == outs[0].shape and t.dtype is outs[0].dtype for t in outs)
+        n = _numel(outs[0].shape)
+        if not (self.group_siblings and same and n % 8 == 0):
+            return [self._heads_result(t) for t in outs]
+        buf = self._new_buf((len(outs),) + tuple(outs[0].shape), outs[0].dtype, "temp", -1)
+        refs = []
+        for i, t in enumerate(outs):
+            refs.append(ViewRef(buf.id, i * n, t.shape, lay[0], t.dtype))
+            self.loc[t.id] = refs[-1]
+        return refs
 
     def _lower_attention(self, n: ir.Node) -> None:
         B, H, S, hd = n.inputs[0].shape
@@ -1982,11 +2096,11 @@ class Planner:
         lse = self._contig(n.inputs[4])
         o_lo = self._heads_operand(n.inputs[5])
         dout = self._heads_operand(n.inputs[6])
-        dq, dk, dv = (self._heads_result(t) for t in n.outputs)
+        dq, dk, dv = self._heads_results_side_by_side(n.outputs)
         wbuf = self._new_buf((B * H * S,), DType.float32, "temp", -1)
         ws = ViewRef(wbuf.id, 0, (B * H * S,), (1,), DType.float32)
         self._emit(Step("attention_bwd", [q.buf, k.buf, v.buf, o.buf, lse.buf, o_lo.buf, dout.buf],
-                        [dq.buf, dk.buf, dv.buf, wbuf.id],
+                        sorted({dq.buf, dk.buf, dv.buf}) + [wbuf.id],
                         dict(common, q=q, k=k, v=v, o=o, lse=lse, o_lo=o_lo, dout=dout, dq=dq, dk=dk, dv=dv,
                              workspace=ws, workspace_bytes=B * H * S * 4)))
 

@@ -67,6 +67,11 @@ _FOLD_THIN_PAIR: ContextVar[bool] = ContextVar(
 _FOLD_PRODUCT_SUMS: ContextVar[bool] = ContextVar(
     "FOLD_PRODUCT_SUMS", default=_env_flag("NBK_FOLD_PRODUCT_SUMS", True))
 
+# x^T dy1, x^T dy2, x^T dy3 (the weight gradients of projections that share their input), each
+# split along K, as ONE batched launch that reads x once per cache; off: one launch each
+_GROUP_SIBLING_PRODUCTS: ContextVar[bool] = ContextVar(
+    "GROUP_SIBLING_PRODUCTS", default=_env_flag("NBK_GROUP_SIBLING_PRODUCTS", True))
+
 # the column sums of dy (a bias gradient) as one more result of the weight-gradient product
 # x^T dy that reads dy anyway; off: the reduction kernels read dy a second time
 _FOLD_COLUMN_SUMS: ContextVar[bool] = ContextVar(
@@ -105,6 +110,7 @@ _FLAGS = {
     "FOLD_PRODUCT_SUMS": _FOLD_PRODUCT_SUMS,
     "FOLD_SCALE": _FOLD_SCALE,
     "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
+    "GROUP_SIBLING_PRODUCTS": _GROUP_SIBLING_PRODUCTS,
     "VMAP_BATCHED": _VMAP_BATCHED,
     "GELU_BACKWARD_FROM_INPUT": _GELU_BACKWARD_FROM_INPUT,
     "FUSED_NF4_MATMUL": _FUSED_NF4_MATMUL,

@@ -1993,10 +1993,10 @@ extern "C" int nbk_gemm(const nbk_gemm_desc* d, void* stream) {
       }
     }
     if (d->colsum != nullptr) {
-      NBK_REQUIRE(fast && !akc && !bkc && a.batch_inner == 1 && d->bias == nullptr &&
+      NBK_REQUIRE(fast && !akc && !bkc && d->bias == nullptr &&
                       d->residual == nullptr && d->act == NBK_ACT_NONE && d->alpha == 1.f,
                   "gemm: column sums go with a plain bf16 product of two row-contiguous, 16-byte "
-                  "aligned operands (K %% 64 == 0, M %% 8 == 0, N %% 8 == 0, one batch level)");
+                  "aligned operands (K %% 64 == 0, M %% 8 == 0, N %% 8 == 0)");
       return launch_bf16_dl_colsum<128, 128, 4>(a, d->batch, st);
     }
     if (!fast) return launch_bf16<128, 128>(a, akc, bkc, d->batch, st);

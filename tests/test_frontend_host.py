@@ -822,6 +822,47 @@ def test_adapter_updates_and_gradient_sums_are_one_product(emulator):
     engine.clear_plan_cache()
 
 
+def test_weight_gradients_of_projections_that_share_their_input_are_one_launch(emulator):
+    """x^T dq, x^T dk and x^T dv (the weight gradients of the q, k and v projections of a
+    transformer block, each split along K = batch x sequence) are ONE batched launch: dq, dk and
+    dv lie side by side in one buffer, the batch index of the launch is (projection, slice), and
+    the three bias gradients are rows of its column sums.  Gradients as without the grouping."""
+    from nabla_amd import config
+    from nabla_amd.core import engine
+
+    def step():
+        engine.clear_plan_cache()
+        t = oc.c3_inputs(2, 1024, 128, 256, seed=5, bf16=True)
+        loss, grads = oc.c3_program(nb, oc.upload(nb, t, nb.DType.bfloat16), num_heads=2)
+        nb.realize_all(loss, *grads.values())
+        steps = list(engine._PLAN_CACHE.values())[-1].plan.steps
+        return loss.item(), {k: g.numpy().astype(np.float64) for k, g in grads.items()}, steps, t
+
+    on = step()
+    wgrads = [s.attrs for s in on[2] if s.kind == "gemm" and s.attrs["a_rs"] == 1 and s.attrs["M"] == 128 and s.attrs["N"] == 128]
+    joined = [a for a in wgrads if a.get("batch_inner", 1) > 1]
+    assert len(joined) == 1 and len(wgrads) == 2, [(a["batch"], a.get("batch_inner")) for a in wgrads]
+    a = joined[0]
+    ks = a["batch_inner"]
+    assert ks > 1 and a["batch"] == 3 * ks and a["a_bs"] == 0 and a["b_bs"] == 2 * 1024 * 128
+    assert a["c_bs"] == ks * 128 * 128 and a["c_bs2"] == 128 * 128 and len(a["colsum_keys"]) == 3
+    assert a["colsum"].shape == (3 * ks, 128)
+    bwd = [s.attrs for s in on[2] if s.kind == "attention_bwd"][0]
+    assert bwd["dq"].buf == bwd["dk"].buf == bwd["dv"].buf
+    assert (bwd["dq"].offset, bwd["dk"].offset, bwd["dv"].offset) == (0, 2 * 1024 * 128, 2 * 2 * 1024 * 128)
+    with config.flag("GROUP_SIBLING_PRODUCTS", False):
+        off = step()
+    assert not [s for s in off[2] if s.kind == "gemm" and s.attrs.get("batch_inner", 1) > 1 and s.attrs["a_bs"] == 0]
+    assert len([s for s in off[2] if s.kind == "gemm"]) == len([s for s in on[2] if s.kind == "gemm"]) + 2
+    want_loss, want = oc.c3_reference(on[3], num_heads=2)
+    assert abs(on[0] - want_loss) <= 2e-2 * abs(want_loss)
+    for k in on[1]:
+        np.testing.assert_array_equal(on[1][k], off[1][k], err_msg=k)   # same sums in the same order
+        scale = max(np.abs(want[k]).max(), np.abs(want["bq"]).max() if k == "bk" else 0.0)
+        assert np.abs(on[1][k] - want[k]).max() <= 2e-2 * scale, k
+    engine.clear_plan_cache()
+
+
 def test_a_batch_summed_product_keeps_what_was_folded_onto_it(emulator):
     """sum_b A[b] @ B[b] becomes one product over (b, k).  A scale folded onto the batched product
     commutes with the sum and rides along as alpha; a bias or a residual added per batch element

@@ -343,6 +343,54 @@ def test_gemm_column_sums(hip, shape, ks):
     assert (np.abs(got_s - ref_s) <= tol).all(), np.abs(got_s - ref_s).max()
 
 
+@pytest.mark.parametrize("shape,members,ks", [((1024, 1024, 2048), 3, 4), ((256, 136, 1024), 2, 2),
+                                              ((128, 128, 512), 3, 1)])
+def test_gemm_column_sums_over_two_batch_levels(hip, shape, members, ks):
+    """x^T dy_m for several dy_m that lie equally spaced in one buffer, each split along K, as ONE
+    launch: batch index (member, slice), the left operand shared (batch stride 0), partial
+    products and partial column sums in (member, slice) order.  Every slice must be what the
+    launch of that member alone gives, bit for bit."""
+    from nabla_amd.backend import lib
+    M, N, K = shape
+    rng = np.random.default_rng(9)
+    xt = torch.tensor(rng.standard_normal((K, M)), dtype=torch.bfloat16).cuda()
+    gap = K * N + 64                                       # elements between members
+    dys = torch.zeros(members * gap, dtype=torch.bfloat16, device="cuda")
+    for m in range(members):
+        dys[m * gap:m * gap + K * N] = torch.tensor(rng.standard_normal(K * N) + 0.25, dtype=torch.bfloat16).cuda()
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    kc = K // ks
+
+    def run(first, count):
+        c = torch.full((count * ks, M, N), float("nan"), dtype=torch.float32, device="cuda")
+        cs = torch.full((count * ks, N), float("nan"), dtype=torch.float32, device="cuda")
+        d = lib.GemmDesc()
+        d.A, d.B, d.C = xt.data_ptr(), dys.data_ptr() + first * gap * 2, c.data_ptr()
+        d.M, d.N, d.K = M, N, kc
+        d.a_rs, d.a_cs, d.b_rs, d.b_cs, d.ldc = 1, M, N, 1, N
+        d.batch, d.batch_inner = count * ks, ks
+        d.a_bs, d.b_bs, d.c_bs = 0, gap, ks * M * N
+        d.a_bs2, d.b_bs2, d.c_bs2 = kc * M, kc * N, M * N
+        d.dtype_ab, d.dtype_c, d.alpha = 1, 0, 1.0
+        d.colsum = cs.data_ptr()
+        lib.check(L.nbk_gemm(C.byref(d), st))
+        torch.cuda.synchronize()
+        return c, cs
+
+    c_all, cs_all = run(0, members)
+    for m in range(members):
+        c_one, cs_one = run(m, 1)
+        assert torch.equal(c_all[m * ks:(m + 1) * ks], c_one), m
+        assert torch.equal(cs_all[m * ks:(m + 1) * ks], cs_one), m
+        dy = dys[m * gap:m * gap + K * N].reshape(K, N)
+        ref_c = (xt.double().t().cpu() @ dy.double().cpu()).numpy()
+        got_c = c_one.double().sum(0).cpu().numpy()
+        assert np.abs(got_c - ref_c).max() <= 1e-3 * np.abs(ref_c).max()
+        ref_s = dy.double().cpu().reshape(ks, kc, N).sum(1).numpy()
+        assert np.abs(cs_one.double().cpu().numpy() - ref_s).max() <= 1e-4 * np.sqrt(kc)
+
+
 def test_gemm_column_sums_refuses_what_the_kernel_does_not_cover(hip):
     from nabla_amd.backend import lib
     a = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
