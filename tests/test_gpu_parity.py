@@ -767,7 +767,8 @@ def test_kept_losses_stay_valid_and_do_not_pin_the_gradients(hip):
         loss, g = step(W, X)
         kept.append(loss)
         del g
-    assert hip.graph_replays - before >= 3
+    if hip.use_graphs:  # (NBK_GRAPHS=0: plain launches, the values are checked all the same)
+        assert hip.graph_replays - before >= 3
     for loss in kept[-6:]:
         assert abs(loss.item() - want[0]) <= F32_TOL * abs(want[0])
 

@@ -66,7 +66,8 @@ def test_dropout_inside_a_replayed_graph_draws_new_masks(hip):
         y = step(x, w)
         outs.append(y.numpy().copy())
         del y
-    assert hip.graph_replays > before
+    if hip.use_graphs:  # (NBK_GRAPHS=0: plain launches, the values are checked all the same)
+        assert hip.graph_replays > before
     for a, b in zip(outs, outs[1:]):
         assert not np.array_equal(a, b)
     nb.set_seed(3)
