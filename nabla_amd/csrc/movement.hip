@@ -277,6 +277,72 @@ __device__ __forceinline__ void reduce_mid_vec_body(const T* __restrict__ in, vo
     }
   }
 }
+// A few rows of a long fp32 row (the partial products of a GEMM split along K): one 16-byte piece
+// per lane and row, as above, is too little work per lane and leaves two loads in flight.  Here a
+// lane sums FEW_CPL pieces of the row, two rows of all of them requested at once, and stores
+// whole pieces.  Same order of summation as above (row 0 first), so the same results.
+constexpr int FEW_CPL = 4;
+__device__ __forceinline__ void reduce_few_rows_body(const float* __restrict__ in, void* __restrict__ out,
+                                                     int dto, int64_t red, int64_t inner, int kind,
+                                                     int64_t bx, int64_t o) {
+  const int64_t chunks = inner >> 2;
+  const float4* base = (const float4*)(in + o * red * inner);
+  const float ident = kind == NBK_RED_SUM ? 0.f : (kind == NBK_RED_MAX ? -INFINITY : INFINITY);
+  int64_t c[FEW_CPL];
+  float4 acc[FEW_CPL];
+#pragma unroll
+  for (int j = 0; j < FEW_CPL; ++j) {
+    c[j] = bx * (256 * FEW_CPL) + j * 256 + threadIdx.x;
+    acc[j] = make_float4(ident, ident, ident, ident);
+  }
+  auto add = [&](float4& a, const float4 v) {
+    a.x = red_comb(a.x, v.x, kind); a.y = red_comb(a.y, v.y, kind);
+    a.z = red_comb(a.z, v.z, kind); a.w = red_comb(a.w, v.w, kind);
+  };
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  int64_t r = 0;
+  for (; r + 1 < red; r += 2) {
+    float4 v0[FEW_CPL], v1[FEW_CPL];
+#pragma unroll
+    for (int j = 0; j < FEW_CPL; ++j) {
+      v0[j] = c[j] < chunks ? base[r * chunks + c[j]] : zero;
+      v1[j] = c[j] < chunks ? base[(r + 1) * chunks + c[j]] : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < FEW_CPL; ++j) { add(acc[j], v0[j]); add(acc[j], v1[j]); }
+  }
+  if (r < red) {
+#pragma unroll
+    for (int j = 0; j < FEW_CPL; ++j) add(acc[j], c[j] < chunks ? base[r * chunks + c[j]] : zero);
+  }
+#pragma unroll
+  for (int j = 0; j < FEW_CPL; ++j) {
+    if (c[j] >= chunks) continue;
+    const int64_t at = o * chunks + c[j];  // in pieces of four elements
+    if (dto == NBK_F32) {
+      ((float4*)out)[at] = acc[j];
+    } else if (dto == NBK_BF16) {
+      uint2 u;
+      u.x = (uint32_t)nbk_f32_to_bf16(acc[j].x) | ((uint32_t)nbk_f32_to_bf16(acc[j].y) << 16);
+      u.y = (uint32_t)nbk_f32_to_bf16(acc[j].z) | ((uint32_t)nbk_f32_to_bf16(acc[j].w) << 16);
+      ((uint2*)out)[at] = u;
+    } else {
+      nbk_store_from_f32(out, at * 4 + 0, dto, acc[j].x); nbk_store_from_f32(out, at * 4 + 1, dto, acc[j].y);
+      nbk_store_from_f32(out, at * 4 + 2, dto, acc[j].z); nbk_store_from_f32(out, at * 4 + 3, dto, acc[j].w);
+    }
+  }
+}
+// what a reduction must look like for the body above
+static bool reduce_few_rows_fits(const void* in, const void* out, int dti, int64_t red, int64_t inner) {
+  return dti == NBK_F32 && red <= 8 && inner % 4 == 0 && inner >= 65536 &&
+         ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0;
+}
+__global__ __launch_bounds__(256) void reduce_few_rows_kernel(const float* __restrict__ in,
+                                                              void* __restrict__ out, int dto, int64_t red,
+                                                              int64_t inner, int kind) {
+  reduce_few_rows_body(in, out, dto, red, inner, kind, blockIdx.x, blockIdx.y);
+}
+
 // Integer tensors: exact, with a 64-bit accumulator.  The same [outer, red, inner] layout and
 // strip of 64 columns per workgroup as above; the four waves split `red` and meet in LDS.
 __device__ __forceinline__ int64_t red_comb_i(int64_t a, int64_t b, int kind) {
@@ -323,7 +389,7 @@ struct ReduceBatchArgs {
   int32_t n;
   int32_t first_block[NBK_REDUCE_BATCH_MAX + 1];
   int32_t blocks_x[NBK_REDUCE_BATCH_MAX];
-  int32_t mode[NBK_REDUCE_BATCH_MAX];  // 0: element-wise, 1: bf16 x 8, 2: fp32 x 4
+  int32_t mode[NBK_REDUCE_BATCH_MAX];  // 0: element-wise, 1: bf16 x 8, 2: fp32 x 4, 3: few fp32 rows
   int32_t wc[NBK_REDUCE_BATCH_MAX];    // waves side by side along the row (vector modes)
   nbk_reduce_task t[NBK_REDUCE_BATCH_MAX];
 };
@@ -338,6 +404,8 @@ __global__ __launch_bounds__(256) void reduce_batch_kernel(const ReduceBatchArgs
     reduce_mid_vec_body<uint16_t, 8>((const uint16_t*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o, B.wc[i]);
   else if (B.mode[i] == 2)
     reduce_mid_vec_body<float, 4>((const float*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o, B.wc[i]);
+  else if (B.mode[i] == 3)
+    reduce_few_rows_body((const float*)t.in, t.out, t.dtype_out, t.red, t.inner, t.kind, bx, o);
   else
     reduce_mid_body(t.in, t.out, t.dtype_in, t.dtype_out, t.red, t.inner, t.kind, bx, o);
 }
@@ -377,6 +445,12 @@ static int reduce_mid_slab(const void* in, void* out, int32_t dti, int32_t dto, 
     return nbk_check_launch("reduce_mid_int_kernel");
   }
   const bool aligned = ((uintptr_t)in & 15) == 0;
+  if (reduce_few_rows_fits(in, out, dti, red, inner)) {
+    dim3 grid((unsigned)((inner / 4 + 256 * FEW_CPL - 1) / (256 * FEW_CPL)), (unsigned)outer);
+    hipLaunchKernelGGL(reduce_few_rows_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const float*)in,
+                       out, dto, red, inner, kind);
+    return nbk_check_launch("reduce_few_rows_kernel");
+  }
   if (dti == NBK_BF16 && inner % 8 == 0 && aligned) {
     const int wc = reduce_waves_across(inner / 8);
     dim3 grid((unsigned)((inner / 8 + 64 * wc - 1) / (64 * wc)), (unsigned)outer);
@@ -438,7 +512,11 @@ extern "C" int nbk_reduce_mid_batch(const nbk_reduce_task* tasks, int32_t n, voi
       if (t.dtype_in == NBK_BF16 && t.inner % 8 == 0 && aligned) { B.mode[i] = 1; vec = 8; }
       else if (t.dtype_in == NBK_F32 && t.inner % 4 == 0 && aligned) { B.mode[i] = 2; vec = 4; }
       B.wc[i] = vec > 1 ? reduce_waves_across(t.inner / vec) : 1;
-      const int64_t bx = (t.inner / vec + 64 * B.wc[i] - 1) / (64 * B.wc[i]);
+      int64_t bx = (t.inner / vec + 64 * B.wc[i] - 1) / (64 * B.wc[i]);
+      if (reduce_few_rows_fits(t.in, t.out, t.dtype_in, t.red, t.inner)) {
+        B.mode[i] = 3;
+        bx = (t.inner / 4 + 256 * FEW_CPL - 1) / (256 * FEW_CPL);
+      }
       B.blocks_x[i] = (int32_t)bx;
       B.first_block[i] = (int32_t)blocks;
       blocks += bx * t.outer;

@@ -729,6 +729,45 @@ def test_reduce_mid_direct(hip, dtype, outer, red, inner):
             assert torch.equal(out.cpu().double(), ref)
 
 
+@pytest.mark.parametrize("outer,red,inner", [(1, 2, 4194304), (3, 3, 65536 + 4 * 257), (1, 8, 65536), (2, 1, 70000),
+                                             (1, 2, 65532)])
+def test_reduce_mid_over_a_few_long_fp32_rows(hip, outer, red, inner):
+    """The partial products of a GEMM split along K: a few fp32 rows of millions of elements
+    (several pieces of the row per lane; rows shorter than 65536 take the general kernel).  Sums
+    are exactly the fp32 sums in row order, with fp32 and with bf16 results; one launch for
+    several such reductions gives the same bits."""
+    from nabla_amd.backend import lib
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((outer, red, inner)).astype(np.float32)
+    xd = torch.tensor(x).cuda()
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    acc = np.zeros((outer, inner), np.float32)
+    for r in range(red):
+        acc = acc + x[:, r]
+    want = {0: acc, 1: x.max(1), 2: x.min(1)}
+    tasks = (lib.ReduceTask * 6)()
+    outs = []
+    for i, (kind, dto) in enumerate([(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (2, 1)]):
+        tdt = torch.float32 if dto == 0 else torch.bfloat16
+        out = torch.full((outer, inner), float("nan"), dtype=tdt, device="cuda")
+        lib.check(L.nbk_reduce_mid(C.c_void_p(xd.data_ptr()), C.c_void_p(out.data_ptr()), 0, dto,
+                                   outer, red, inner, kind, st))
+        torch.cuda.synchronize()
+        ref = torch.tensor(want[kind]).to(tdt)
+        assert torch.equal(out.cpu(), ref), (kind, dto)
+        again = torch.full_like(out, float("nan"))
+        t = tasks[i]
+        t.in_, t.out = xd.data_ptr(), again.data_ptr()
+        t.outer, t.red, t.inner = outer, red, inner
+        t.dtype_in, t.dtype_out, t.kind = 0, dto, kind
+        outs.append((out, again))
+    lib.check(L.nbk_reduce_mid_batch(tasks, 6, st))
+    torch.cuda.synchronize()
+    for out, again in outs:
+        assert torch.equal(out, again)
+
+
 def test_reduce_mid_batch_matches_single_launches(hip):
     """One launch for many reductions: mixed dtypes, kinds, vector and element-wise shapes, more
     tasks than one launch holds; every result equals the single-task entry point's bit for bit."""
