@@ -822,6 +822,25 @@ def test_adapter_updates_and_gradient_sums_are_one_product(emulator):
     engine.clear_plan_cache()
 
 
+def test_slices_of_the_contraction_axis():
+    """How the planner splits K: products with fewer than 128 tiles of 128 x 128 and a long K
+    until the launch has 512 workgroups; weight gradients x^T dy (both operands row-contiguous)
+    with one workgroup per CU at most in two halves; nothing else, and fp32 never."""
+    from nabla_amd.backend.planner import Planner
+    bf16, f32 = nb.DType.bfloat16, nb.DType.float32
+    split = Planner._split_k
+    assert split(1024, 1024, 8192, bf16) == 8                    # 64 tiles
+    assert split(1024, 1024, 8192, bf16, rows_contiguous=True) == 8
+    assert split(2048, 16, 8192, bf16) == 16                     # 16 tiles, slices of 512
+    assert split(1024, 4096, 8192, bf16) == 1                    # 256 tiles: whole ...
+    assert split(1024, 4096, 8192, bf16, rows_contiguous=True) == 2   # ... but x^T dy in halves
+    assert split(2048, 2048, 8192, bf16, rows_contiguous=True) == 2
+    assert split(1024, 4096, 2048, bf16, rows_contiguous=True) == 1   # a short K stays whole
+    assert split(2048, 4096, 8192, bf16, rows_contiguous=True) == 1   # 512 tiles: two per CU anyway
+    assert split(8192, 16, 2048, bf16, a_k_contiguous=True) == 1      # the tall kernel splits K itself
+    assert split(1024, 1024, 8192, f32) == 1
+
+
 def test_weight_gradients_of_projections_that_share_their_input_are_one_launch(emulator):
     """x^T dq, x^T dk and x^T dv (the weight gradients of the q, k and v projections of a
     transformer block, each split along K = batch x sequence) are ONE batched launch: dq, dk and
