@@ -102,9 +102,15 @@ __device__ __forceinline__ void conv_ld8(const float* p, bool ok, float* r) {
 // workgroup tile, 1 for 128 x 64 (channel counts up to 64 would waste half of the wider tile).
 template <int MODE, bool FAST, int NJ>
 __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
-  constexpr int BK = 16, LD = 128 + 4, BN = 64 * NJ;
+  // Tiles sit in LDS k-major, [k][128 rows], with the rows of k-row k rotated by 32 places when
+  // (k ^ k / 8) is odd.  The two halves of a wave read k-rows 2 ks and 2 ks + 1 of one MFMA
+  // step, and the two lanes of a pixel store k-rows e and 8 + e: either way the halves land
+  // 32 banks apart (a padded pitch of 132 serves the stores only: 77-87 % of the LDS cycles of
+  // these kernels were bank conflicts).
+  constexpr int BK = 16, LD = 128, BN = 64 * NJ;
   __shared__ float As[2][BK][LD];
   __shared__ float Bs[2][BK][LD];
+  auto rot = [](int k, int col) { return (col + 32 * ((k ^ (k >> 3)) & 1)) & 127; };
   const nbk_conv_desc& d = g.d;
   const int tm_i = blockIdx.x % g.tiles_m, tn_i = blockIdx.x / g.tiles_m;
   const int64_t m0 = (int64_t)tm_i * 128, n0 = (int64_t)tn_i * BN;
@@ -156,6 +162,40 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
   }
 
   float ra[8], rb[8];
+  const bool unit_stride = d.stride_h == 1 && d.stride_w == 1;
+  // forward / dgrad, FAST: the filter tap (t_r, t_s) and the first channel t_c of the K step
+  // that is loaded next (uniform; kept as running counters: a 64-bit division per K step and
+  // operand otherwise)
+  int t_r = 0, t_s = 0, t_c = 0;
+  if (FAST && MODE != CONV_WGRAD) {
+    const int ck = MODE == CONV_FWD ? (int)d.Cin : (int)d.Cout;
+    const int tap = (int)(k_begin / ck);
+    t_c = (int)(k_begin - (int64_t)tap * ck);
+    t_r = tap / (int)d.S;
+    t_s = tap - t_r * (int)d.S;
+  }
+  // forward: row, column and number of the lane's input pixel at tap (0, 0); dgrad with unit
+  // stride: the same for its output pixel
+  int q_h0 = 0, q_w0 = 0, q_pix0 = 0;
+  if (MODE == CONV_FWD) {
+    q_h0 = p_y * d.stride_h - d.pad_t;
+    q_w0 = p_x * d.stride_w - d.pad_l;
+    q_pix0 = (p_n * (int)d.H + q_h0) * (int)d.W + q_w0;
+  } else if (MODE == CONV_DGRAD) {
+    q_h0 = p_y + d.pad_t;
+    q_w0 = p_x + d.pad_l;
+    q_pix0 = (p_n * (int)d.Ho + q_h0) * (int)d.Wo + q_w0;
+  }
+  auto next_tap = [&]() {
+    if (FAST && MODE != CONV_WGRAD) {
+      const int ck = MODE == CONV_FWD ? (int)d.Cin : (int)d.Cout;
+      t_c += BK;
+      if (t_c >= ck) {
+        t_c -= ck;
+        if (++t_s == (int)d.S) { t_s = 0; ++t_r; }
+      }
+    }
+  };
   auto load_a = [&](int64_t k0) {
     if (MODE == CONV_WGRAD) {
       // pixel (p_n, p_y, p_x) is column k0 + w_kk; taps of rows m0 + w_rr .. + 7
@@ -175,14 +215,18 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
         if (++p_y >= d.Ho) { p_y = 0; ++p_n; }
       }
     } else if (FAST) {
-      const int ck = MODE == CONV_FWD ? (int)d.Cin : (int)d.Cout;
-      const int tap = (int)(k0 / ck), c0 = (int)(k0 - (int64_t)tap * ck) + a_kk;
-      const int r = tap / (int)d.S, s = tap - r * (int)d.S;
+      const int c0 = t_c + a_kk, r = t_r, s = t_s;
       if (MODE == CONV_FWD) {
-        const int h = p_y * d.stride_h - d.pad_t + r, w = p_x * d.stride_w - d.pad_l + s;
+        // (the lane's pixel at tap (0, 0) is a constant of the lane; the tap adds a uniform
+        // number of pixels; pixel numbers fit 32 bits, checked on the host)
+        const int h = q_h0 + r, w = q_w0 + s;
         const bool ok = p_ok && h >= 0 && h < d.H && w >= 0 && w < d.W;
-        conv_ld8(g.a + (((int64_t)p_n * d.H + h) * d.W + w) * d.Cin + c0, ok, ra);
-      } else {
+        conv_ld8(g.a + (int64_t)(q_pix0 + r * (int)d.W + s) * d.Cin + c0, ok, ra);
+      } else if (unit_stride) {
+        const int ho = q_h0 - r, wo = q_w0 - s;
+        const bool ok = p_ok && ho >= 0 && wo >= 0 && ho < d.Ho && wo < d.Wo;
+        conv_ld8(g.a + (int64_t)(q_pix0 - r * (int)d.Wo - s) * d.Cout + c0, ok, ra);
+      } else {  // (two integer divisions per lane and K step)
         const int hn = p_y + d.pad_t - r, wn = p_x + d.pad_l - s;
         const int ho = hn / d.stride_h, wo = wn / d.stride_w;
         const bool ok = p_ok && hn >= 0 && wn >= 0 && ho * d.stride_h == hn &&
@@ -197,10 +241,10 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
   auto store_a = [&](float (*S)[LD]) {
     if (MODE == CONV_WGRAD) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[w_kk][w_rr + e] = ra[e];
+      for (int e = 0; e < 8; ++e) S[w_kk][rot(w_kk, w_rr) + e] = ra[e];
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[a_kk + e][a_row] = ra[e];
+      for (int e = 0; e < 8; ++e) S[a_kk + e][rot(a_kk + e, a_row)] = ra[e];
     }
   };
   auto load_b = [&](int64_t k0) {
@@ -208,7 +252,7 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
       // w[r, s, j, co]: contiguous along k = co for a fixed input channel j
       const int64_t j = n0 + a_row;
       if (FAST) {
-        const int tap = (int)(k0 / d.Cout), co = (int)(k0 - (int64_t)tap * d.Cout) + a_kk;
+        const int tap = t_r * (int)d.S + t_s, co = t_c + a_kk;
         conv_ld8(g.b + ((int64_t)tap * d.Cin + j) * d.Cout + co, j < g.Ng, rb);
       } else {
 #pragma unroll
@@ -228,16 +272,17 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
   auto store_b = [&](float (*S)[LD]) {
     if (MODE == CONV_DGRAD) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[a_kk + e][a_row] = rb[e];
+      for (int e = 0; e < 8; ++e) S[a_kk + e][rot(a_kk + e, a_row)] = rb[e];
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) S[w_kk][w_rr + e] = rb[e];
+      for (int e = 0; e < 8; ++e) S[w_kk][rot(w_kk, w_rr) + e] = rb[e];
     }
   };
 
   const int64_t nk = (k_end - k_begin + BK - 1) / BK;
   load_a(k_begin);
   load_b(k_begin);
+  next_tap();
   store_a(As[0]);
   store_b(Bs[0]);
   __syncthreads();
@@ -247,15 +292,16 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
     if (more) {
       load_a(k_begin + (kt + 1) * BK);
       load_b(k_begin + (kt + 1) * BK);
+      next_tap();
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 2; ++ks) {
       const int k = ks * 2 + kg;
       float fa[2], fb[NJ];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = As[cur][k][wm + i * 32 + li];
+      for (int i = 0; i < 2; ++i) fa[i] = As[cur][k][rot(k, wm + i * 32 + li)];
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) fb[j] = Bs[cur][k][wn + j * 32 + li];
+      for (int j = 0; j < NJ; ++j) fb[j] = Bs[cur][k][rot(k, wn + j * 32 + li)];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
