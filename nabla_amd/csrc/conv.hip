@@ -37,42 +37,47 @@ struct ConvArgs {
 };
 
 // ---- element-wise gather (any channel count) ----------------------------------------------
+// (every extent that is divided here fits 32 bits, checked on the host: 64-bit divisions would
+// cost ten times the instructions, eight times per element)
 template <int MODE>
-__device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m, int64_t k, int64_t k_end) {
+__device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m64, int64_t k64, int64_t k_end) {
   const nbk_conv_desc& d = g.d;
-  if (m >= g.M || k >= k_end) return 0.f;
+  if (m64 >= g.M || k64 >= k_end) return 0.f;
+  const int m = (int)m64, k = (int)k64;
+  const int Cin = (int)d.Cin, Cout = (int)d.Cout, S = (int)d.S, H = (int)d.H, W = (int)d.W,
+            Ho = (int)d.Ho, Wo = (int)d.Wo;
   if (MODE == CONV_FWD) {
-    const int64_t c = k % d.Cin;
-    const int64_t rs = k / d.Cin;
-    const int64_t s = rs % d.S, r = rs / d.S;
-    const int64_t wo = m % d.Wo;
-    const int64_t t = m / d.Wo;
-    const int64_t ho = t % d.Ho, n = t / d.Ho;
-    const int64_t h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
-    if (h < 0 || h >= d.H || w < 0 || w >= d.W) return 0.f;
-    return g.a[((n * d.H + h) * d.W + w) * d.Cin + c];
+    const int c = k % Cin;
+    const int rs = k / Cin;
+    const int s = rs % S, r = rs / S;
+    const int wo = m % Wo;
+    const int t = m / Wo;
+    const int ho = t % Ho, n = t / Ho;
+    const int h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
+    if (h < 0 || h >= H || w < 0 || w >= W) return 0.f;
+    return g.a[(int64_t)((n * H + h) * W + w) * Cin + c];
   } else if (MODE == CONV_DGRAD) {
-    const int64_t co = k % d.Cout;
-    const int64_t rs = k / d.Cout;
-    const int64_t s = rs % d.S, r = rs / d.S;
-    const int64_t w = m % d.W;
-    const int64_t t = m / d.W;
-    const int64_t h = t % d.H, n = t / d.H;
-    const int64_t hn = h + d.pad_t - r, wn = w + d.pad_l - s;
+    const int co = k % Cout;
+    const int rs = k / Cout;
+    const int s = rs % S, r = rs / S;
+    const int w = m % W;
+    const int t = m / W;
+    const int h = t % H, n = t / H;
+    const int hn = h + d.pad_t - r, wn = w + d.pad_l - s;
     if (hn < 0 || wn < 0 || hn % d.stride_h != 0 || wn % d.stride_w != 0) return 0.f;
-    const int64_t ho = hn / d.stride_h, wo = wn / d.stride_w;
-    if (ho >= d.Ho || wo >= d.Wo) return 0.f;
-    return g.a[((n * d.Ho + ho) * d.Wo + wo) * d.Cout + co];
+    const int ho = hn / d.stride_h, wo = wn / d.stride_w;
+    if (ho >= Ho || wo >= Wo) return 0.f;
+    return g.a[(int64_t)((n * Ho + ho) * Wo + wo) * Cout + co];
   } else {
-    const int64_t c = m % d.Cin;
-    const int64_t rs = m / d.Cin;
-    const int64_t s = rs % d.S, r = rs / d.S;
-    const int64_t wo = k % d.Wo;
-    const int64_t t = k / d.Wo;
-    const int64_t ho = t % d.Ho, n = t / d.Ho;
-    const int64_t h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
-    if (h < 0 || h >= d.H || w < 0 || w >= d.W) return 0.f;
-    return g.a[((n * d.H + h) * d.W + w) * d.Cin + c];
+    const int c = m % Cin;
+    const int rs = m / Cin;
+    const int s = rs % S, r = rs / S;
+    const int wo = k % Wo;
+    const int t = k / Wo;
+    const int ho = t % Ho, n = t / Ho;
+    const int h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
+    if (h < 0 || h >= H || w < 0 || w >= W) return 0.f;
+    return g.a[(int64_t)((n * H + h) * W + w) * Cin + c];
   }
 }
 
@@ -82,8 +87,8 @@ __device__ __forceinline__ float conv_load_b(const ConvArgs& g, int64_t k, int64
   if (k >= k_end || j >= g.Ng) return 0.f;
   if (MODE == CONV_FWD) return g.b[k * d.Cout + j];  // w viewed as [R*S*Cin, Cout]
   if (MODE == CONV_DGRAD) {
-    const int64_t co = k % d.Cout, rs = k / d.Cout;
-    return g.b[(rs * d.Cin + j) * d.Cout + co];
+    const int co = (int)k % (int)d.Cout, rs = (int)k / (int)d.Cout;
+    return g.b[((int64_t)rs * d.Cin + j) * d.Cout + co];
   }
   return g.b[k * d.Cout + j];  // dy viewed as [N*Ho*Wo, Cout]
 }

@@ -638,6 +638,53 @@ def test_conv_pool_grads(hip):
         assert np.abs(g.numpy() - ref).max() <= 1e-5 * np.abs(ref).max() + 1e-8
 
 
+@pytest.mark.parametrize("shape,kernel,stride,pad", [((3, 12, 12, 16), (2, 2), (2, 2), (0, 0)),
+                                                     ((2, 9, 11, 8), (3, 3), (2, 2), (1, 1)),
+                                                     ((2, 8, 8, 12), (3, 2), (1, 1), (1, 0)),
+                                                     ((2, 7, 7, 6), (2, 2), (2, 2), (0, 0))])
+def test_max_pool_through_the_c_abi(hip, shape, kernel, stride, pad):
+    """nbk_maxpool2d_fwd / _bwd against the oracle: channel counts that take the four-channel
+    form (16-byte accesses) and one that does not, overlapping windows, clipped borders, and
+    ties (values from a small set, so several elements of a window are its maximum and each
+    takes the window's cotangent).  The four-channel form and the general form (the same tensors
+    at addresses that are not 16-byte aligned) must agree bit for bit."""
+    from nabla_amd.backend import lib
+    from oracle import ops as O
+    N, H, W, Cc = shape
+    (kh, kw), (sh, sw), (pt, pl) = kernel, stride, pad
+    rng = np.random.default_rng(21)
+    x = rng.integers(-3, 4, shape).astype(np.float32) * 0.5
+    vx = O.V(x)
+    vy = O.max_pool2d(vx, kernel, stride, (pt, pt, pl, pl))
+    Ho, Wo = vy.a.shape[1:3]
+    g = rng.standard_normal(vy.a.shape).astype(np.float32)
+    (want_gx,) = vy.vjp(g)
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    d = lib.PoolDesc()
+    d.N, d.H, d.W, d.C, d.Ho, d.Wo = N, H, W, Cc, Ho, Wo
+    d.kh, d.kw, d.stride_h, d.stride_w, d.pad_t, d.pad_l, d.dtype = kh, kw, sh, sw, pt, pl, 0
+    results = []
+    for shift in (0, 1):     # element offset of every tensor inside its allocation
+        def dev(a):
+            buf = torch.zeros(a.size + 4, dtype=torch.float32, device="cuda")
+            buf[shift:shift + a.size] = torch.tensor(a.reshape(-1))
+            return buf, buf[shift:shift + a.size]
+        xb, xd = dev(x)
+        yb, yd = dev(np.full(vy.a.shape, np.nan, np.float32))
+        gb, gd = dev(g)
+        dxb, dxd = dev(np.full(shape, np.nan, np.float32))
+        lib.check(L.nbk_maxpool2d_fwd(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(yd.data_ptr()), st))
+        lib.check(L.nbk_maxpool2d_bwd(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(yd.data_ptr()),
+                                      C.c_void_p(gd.data_ptr()), C.c_void_p(dxd.data_ptr()), st))
+        torch.cuda.synchronize()
+        results.append((yd.cpu().numpy().reshape(vy.a.shape), dxd.cpu().numpy().reshape(shape)))
+    for y, dx in results:
+        np.testing.assert_array_equal(y, vy.a)
+        np.testing.assert_allclose(dx, want_gx, rtol=1e-6, atol=1e-6)
+    np.testing.assert_array_equal(results[0][1], results[1][1])
+
+
 def test_gather_argmax_views(hip):
     import nabla_amd as nb
     rng = np.random.default_rng(5)
