@@ -41,7 +41,7 @@ def _wgrad_workspace_bytes(xs, ws, ys, n_cus: int = 256) -> int:
     r, s_, cin, cout = ws
     m, k = r * s_ * cin, ys[0] * ys[1] * ys[2]
     tiles = ((m + 127) // 128) * ((cout + 127) // 128)
-    want = max(1, min((2 * n_cus + tiles - 1) // tiles, max(k // 64, 1)))
+    want = max(1, min(2 * n_cus // tiles, max(k // 64, 1)))
     kps = ((k + want - 1) // want + 15) // 16 * 16
     splits = (k + kps - 1) // kps
     return 0 if splits <= 1 else splits * m * cout * 4

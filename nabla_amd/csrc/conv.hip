@@ -420,12 +420,14 @@ extern "C" int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const vo
   return conv_launch<CONV_DGRAD>(a, fast, (hipStream_t)stream);
 }
 
-// K split of the filter-gradient product: enough workgroups to fill the GPU twice over,
-// at least four K steps each.
+// K split of the filter-gradient product: as many workgroups as the GPU holds at once (two per
+// CU) and no more -- a handful beyond that would run as a second round behind the first and
+// nearly double the launch (515 workgroups for 512 places: 129 us, 500: 90) --, at least four
+// K steps each.
 static void wgrad_split(const nbk_conv_desc* d, int* splits, int64_t* k_per_split) {
   const int64_t M = d->R * d->S * d->Cin, K = d->N * d->Ho * d->Wo;
   const int64_t tiles = ((M + 127) / 128) * ((d->Cout + 127) / 128);
-  int64_t want = (2 * (int64_t)nbk_num_cus() + tiles - 1) / tiles;
+  int64_t want = 2 * (int64_t)nbk_num_cus() / tiles;
   const int64_t most = K / 64 > 0 ? K / 64 : 1;
   if (want > most) want = most;
   if (want < 1) want = 1;
