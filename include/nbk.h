@@ -54,7 +54,7 @@ int nbk_init(int device);
 const char* nbk_last_error(void);
 /* ABI version of this header; the ctypes shim refuses a mismatch. */
 int nbk_abi_version(void);
-#define NBK_ABI_VERSION 23
+#define NBK_ABI_VERSION 24
 
 /* ===================================================================== */
 /*  Row programs: fused elementwise chains + last-axis reductions         */
@@ -339,7 +339,11 @@ typedef struct nbk_conv_desc {
   int32_t stride_h, stride_w;
   int32_t pad_t, pad_b, pad_l, pad_r;
   int32_t dtype;      /* NBK_F32 */
-  int32_t reserved;
+  /* forward only: NBK_ACT_NONE, or NBK_ACT_RELU for y = max(conv(x, w) + bias, 0) -- the relu that
+   * follows a convolution layer (nabla/ops/unary.py:31-42), applied to the accumulator on its way
+   * out; its mask in the backward pass, (pre-activation > 0), equals (y > 0).  The two gradient
+   * entry points want NBK_ACT_NONE. */
+  int32_t act;
 } nbk_conv_desc;
 int nbk_conv2d_fwd(const nbk_conv_desc* d, const void* x, const void* w,
                    const void* bias, void* y, void* stream);

@@ -224,6 +224,7 @@ class BoundPlan:
                 d.stride_h, d.stride_w = a["stride"]
                 d.pad_t, d.pad_b, d.pad_l, d.pad_r = a["padding"]
                 d.dtype = a["dst"].dtype.abi
+                d.act = {None: 0, "relu": 1}[a.get("act")]
                 n_ptr = 4 if k == "conv2d" else 3
                 holder = _Ptrs(4)
                 refs = list(a["ins"])

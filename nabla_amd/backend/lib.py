@@ -14,7 +14,7 @@ from pathlib import Path
 from . import isa
 
 LIB_PATH = Path(__file__).resolve().parents[1] / "csrc" / "libnbk.so"
-ABI_VERSION = 23
+ABI_VERSION = 24
 
 MAX_RANK = 8
 
@@ -97,7 +97,7 @@ class ConvDesc(C.Structure):
         ("Wo", C.c_int64),
         ("stride_h", C.c_int32), ("stride_w", C.c_int32),
         ("pad_t", C.c_int32), ("pad_b", C.c_int32), ("pad_l", C.c_int32), ("pad_r", C.c_int32),
-        ("dtype", C.c_int32), ("reserved", C.c_int32),
+        ("dtype", C.c_int32), ("act", C.c_int32),
     ]
 
 

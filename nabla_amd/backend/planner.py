@@ -1214,6 +1214,54 @@ class Planner:
             for k, v in enumerate(outs):
                 v.node, v.index = host, k
 
+    def _fold_relu_into_producer(self) -> None:
+        """``relu(conv2d(x, w) + b)`` or ``relu(x @ W + b)`` whose pre-activation has no reader
+        but the relu and, in a training step, the comparisons ``pre-activation > 0`` of the
+        relu's VJP: the convolution / product applies the relu to its accumulator on the way
+        out, and the comparisons read the result instead (max(h, 0) > 0 exactly where h > 0).
+        The pre-activation never reaches memory and the relu's row kernel is gone."""
+        nodes = self._live_nodes()
+        users: dict[int, list[ir.Node]] = {}
+        for n in nodes:
+            for i in n.inputs:
+                if not any(u is n for u in users.get(i.id, ())):
+                    users.setdefault(i.id, []).append(n)
+        out_ids = {v.id for v in self.outputs}
+        for cv in nodes:
+            at = cv.attrs or {}
+            if cv.kind not in ("conv2d", "matmul") or len(cv.outputs) != 1 or at.get("act"):
+                continue
+            if cv.kind == "matmul" and ("res_in" in at or "terms_in" in at):
+                continue  # (a residual joins after the activation)
+            h = cv.outputs[0]
+            us = users.get(h.id, [])
+            if h.id in out_ids or not us:
+                continue
+            act = [u for u in us if u.kind == "ew" and u.fn == "relu"]
+            def is_zero(x) -> bool:
+                if not isinstance(x, ir.Value):
+                    return float(x) == 0.0
+                while x.node.kind in ("broadcast", "reshape"):
+                    x = x.node.inputs[0]
+                return x.node.kind == "fill" and float(x.node.attrs["value"]) == 0.0
+
+            masks = [u for u in us if u.kind == "ew" and u.fn == "gt" and
+                     len(u.attrs["operands"]) == 2 and u.attrs["operands"][0] is h and
+                     is_zero(u.attrs["operands"][1])]
+            if len(act) != 1 or len(us) != 1 + len(masks):
+                continue
+            y = act[0].outputs[0]
+            if y.dtype is not h.dtype or y.shape != h.shape:
+                continue
+            if cv.kind == "matmul" and not self._epilogue_ok(cv, y):
+                continue
+            cv.attrs = dict(cv.attrs or {}, act="relu")
+            cv.outputs = [y]
+            y.node, y.index = cv, 0
+            for m in masks:
+                m.inputs = [y if i is h else i for i in m.inputs]
+                m.attrs["operands"] = [y if o is h else o for o in m.attrs["operands"]]
+
     def _epilogue_ok(self, mm: ir.Node, out: ir.Value) -> bool:
         """The product ``mm`` may write ``out`` through its epilogue."""
         m = mm.outputs[0]
@@ -1397,7 +1445,7 @@ class Planner:
                 xs, ws, ys = n.inputs[0].shape, out.shape, n.inputs[1].shape
             attrs = dict(ins=ins, dst=dst, x_shape=xs, w_shape=ws, y_shape=ys,
                          stride=n.attrs["stride"], padding=n.attrs["padding"],
-                         has_bias=n.attrs.get("has_bias", False))
+                         has_bias=n.attrs.get("has_bias", False), act=n.attrs.get("act"))
             writes = [dst.buf]
             if k == "conv2d_wgrad":
                 nbytes = _wgrad_workspace_bytes(xs, ws, ys)
@@ -2795,6 +2843,8 @@ def plan_graph(builder: ir.Builder, outputs: Sequence[ir.Value]) -> Plan:
         pre._fold_bias_into_matmul()  # (a bias on top of a sum that has just become a product)
     if config.FOLD_ACTIVATION:
         pre._fold_activation_into_matmul()
+    if config.FOLD_RELU:
+        pre._fold_relu_into_producer()
     outputs = pre.outputs
     for limit in (28, 16, 8, 4, 1):
         try:

@@ -495,6 +495,8 @@ def collect_programs() -> dict[int, dict]:
         jobs.append(with_flags(jobs[4], FOLD_THIN_PAIR=False))
         jobs.append(with_flags(jobs[4], FOLD_PRODUCT_SUMS=False))
         jobs.append(with_flags(jobs[2], FOLD_PRODUCT_SUMS=False))
+        jobs.append(with_flags(jobs[0], FOLD_RELU=False))
+        jobs.append(with_flags(jobs[3], FOLD_RELU=False))
         for job in jobs:
             clear_plan_cache()
             res = job()

@@ -61,6 +61,11 @@ _FOLD_THIN_RESIDUAL: ContextVar[bool] = ContextVar(
 _FOLD_THIN_PAIR: ContextVar[bool] = ContextVar(
     "FOLD_THIN_PAIR", default=_env_flag("NBK_FOLD_THIN_PAIR", True))
 
+# relu(conv2d(x, w) + b) and relu(x @ W + b) as the epilogue of the convolution / product itself
+# (`nbk_conv_desc.act`, `nbk_gemm_desc.act`); the relu's mask in the backward pass reads the
+# result instead of the pre-activation; off: a row program after the producer
+_FOLD_RELU: ContextVar[bool] = ContextVar("FOLD_RELU", default=_env_flag("NBK_FOLD_RELU", True))
+
 # x1 @ W1 + x2 @ W2 (+ x3 @ W3), products that contribute to one value (the gradient of an
 # activation that feeds several projections), as ONE product over all their contraction indices
 # (`nbk_gemm_desc.term`); off: one product each and the kernel that adds them
@@ -108,6 +113,7 @@ _FLAGS = {
     "FOLD_THIN_RESIDUAL": _FOLD_THIN_RESIDUAL,
     "FOLD_THIN_PAIR": _FOLD_THIN_PAIR,
     "FOLD_PRODUCT_SUMS": _FOLD_PRODUCT_SUMS,
+    "FOLD_RELU": _FOLD_RELU,
     "FOLD_SCALE": _FOLD_SCALE,
     "FOLD_COLUMN_SUMS": _FOLD_COLUMN_SUMS,
     "GROUP_SIBLING_PRODUCTS": _GROUP_SIBLING_PRODUCTS,

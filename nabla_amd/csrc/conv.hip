@@ -326,10 +326,12 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs g) {
       const int64_t col = n0 + wn + j * 32 + li;
       const bool col_ok = col < g.Ng;
       const float bv = (g.bias && col_ok) ? g.bias[col] : 0.f;
+      const bool relu = MODE == CONV_FWD && d.act == NBK_ACT_RELU;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t row = m0 + wm + i * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
-        if (col_ok && row < g.M) out[row * g.Ng + col] = acc[i][j][r] + bv;
+        const float v = acc[i][j][r] + bv;
+        if (col_ok && row < g.M) out[row * g.Ng + col] = relu ? fmaxf(v, 0.f) : v;
       }
     }
 }
@@ -358,6 +360,7 @@ static int conv_check(const nbk_conv_desc* d) {
   NBK_REQUIRE(d->N > 0 && d->H > 0 && d->W > 0 && d->Cin > 0 && d->R > 0 && d->S > 0 &&
                   d->Cout > 0 && d->Ho > 0 && d->Wo > 0,
               "conv2d: empty extent");
+  NBK_REQUIRE(d->act == NBK_ACT_NONE || d->act == NBK_ACT_RELU, "conv2d: act %d", d->act);
   NBK_REQUIRE(d->stride_h > 0 && d->stride_w > 0, "stride values must be > 0");
   NBK_REQUIRE(d->pad_t >= 0 && d->pad_b >= 0 && d->pad_l >= 0 && d->pad_r >= 0,
               "padding values must be >= 0");
@@ -411,6 +414,7 @@ extern "C" int nbk_conv2d_dgrad(const nbk_conv_desc* d, const void* dy, const vo
   int rc = conv_check(d);
   if (rc) return rc;
   NBK_REQUIRE(dy && w && dx, "conv2d: null pointer");
+  NBK_REQUIRE(d->act == NBK_ACT_NONE, "conv2d: an activation goes with the forward product only");
   ConvArgs a;
   a.d = *d;
   a.a = (const float*)dy; a.b = (const float*)w; a.bias = nullptr; a.out = (float*)dx;
@@ -451,6 +455,7 @@ extern "C" int nbk_conv2d_wgrad(const nbk_conv_desc* d, const void* x, const voi
   int rc = conv_check(d);
   if (rc) return rc;
   NBK_REQUIRE(x && dy && dw, "conv2d: null pointer");
+  NBK_REQUIRE(d->act == NBK_ACT_NONE, "conv2d: an activation goes with the forward product only");
   ConvArgs a;
   a.d = *d;
   a.a = (const float*)x; a.b = (const float*)dy; a.bias = nullptr; a.out = (float*)dw;

@@ -33,13 +33,16 @@ class ReluOp(UnaryOperation):
         from .comparison import greater
         from .control_flow import where
         from .creation import zeros_like
-        mask = greater(primals[0], 0.0)
+        # (the zero is a creation op, not a scalar leaf: the planner sees the comparison's constant
+        # and can let it read relu's result where the pre-activation is not stored)
+        mask = greater(primals[0], zeros_like(primals[0]))
         return [where(mask, cotangents[0], zeros_like(cotangents[0]))]
 
     def jvp_rule(self, primals, tangents, outputs, kwargs):
         from .binary import mul
         from .comparison import greater
-        return [mul(tangents[0], greater(primals[0], 0.0))]
+        from .creation import zeros_like
+        return [mul(tangents[0], greater(primals[0], zeros_like(primals[0])))]
 
 
 class ExpOp(UnaryOperation):

@@ -822,6 +822,64 @@ def test_adapter_updates_and_gradient_sums_are_one_product(emulator):
     engine.clear_plan_cache()
 
 
+def test_relu_after_a_convolution_is_its_epilogue(emulator):
+    """`relu(conv2d(x, w) + b)`: the convolution applies the relu itself (`nbk_conv_desc.act`), the
+    pre-activation is not stored, and the `pre-activation > 0` masks of the backward pass read the
+    result.  Values and gradients as without the fold, and against torch in float64; a
+    convolution whose pre-activation something else reads keeps its relu kernel."""
+    import torch
+    import torch.nn.functional as TF
+    from nabla_amd import config
+    from nabla_amd.core import engine
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((2, 9, 9, 4)).astype(np.float32)
+    w1 = (rng.standard_normal((3, 3, 4, 8)) * 0.3).astype(np.float32)
+    b1 = (rng.standard_normal((8,)) * 0.2).astype(np.float32)
+    w2 = (rng.standard_normal((3, 3, 8, 6)) * 0.3).astype(np.float32)
+
+    def loss_fn(w1, b1, w2, x):
+        h = nb.relu(nb.conv2d(x, w1, padding=1, bias=b1))
+        h = nb.relu(nb.conv2d(h, w2, stride=(2, 1), padding=(1, 0, 1, 1)))
+        return nb.mean(h * h)
+
+    def step():
+        engine.clear_plan_cache()
+        l, gs = nb.value_and_grad(loss_fn, argnums=(0, 1, 2, 3))(T(w1), T(b1), T(w2), T(x))
+        nb.realize_all(l, *gs)
+        steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+        return l.item(), [g.numpy() for g in gs], steps
+
+    on = step()
+    convs = [s.attrs for s in on[2] if s.kind == "conv2d"]
+    assert [a["act"] for a in convs] == ["relu", "relu"]
+    with config.flag("FOLD_RELU", False):
+        off = step()
+    assert [s.attrs["act"] for s in off[2] if s.kind == "conv2d"] == [None, None]
+    assert len(on[2]) < len(off[2])
+    assert on[0] == off[0]
+    for a, b in zip(on[1], off[1]):
+        np.testing.assert_array_equal(a, b)
+    tw1, tb1, tw2, tx = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (w1, b1, w2, x)]
+    h = torch.relu(TF.conv2d(tx.permute(0, 3, 1, 2), tw1.permute(3, 2, 0, 1), tb1, padding=1))
+    h = torch.relu(TF.conv2d(TF.pad(h, (1, 1, 1, 0)), tw2.permute(3, 2, 0, 1), stride=(2, 1)))
+    tl = (h * h).mean()
+    tl.backward()
+    assert abs(on[0] - tl.item()) <= 1e-5 * abs(tl.item())
+    for g, t in zip(on[1], (tw1, tb1, tw2, tx)):
+        assert np.abs(g - t.grad.numpy()).max() <= 1e-5 * np.abs(t.grad.numpy()).max() + 1e-8
+    # the pre-activation has another reader: no fold
+    engine.clear_plan_cache()
+    pre = nb.conv2d(T(x), T(w1), padding=1, bias=T(b1))
+    both = nb.relu(pre) + pre * 0.5
+    both.realize()
+    steps = [s for bp in engine._PLAN_CACHE.values() for s in bp.plan.steps]
+    assert [s.attrs["act"] for s in steps if s.kind == "conv2d"] == [None]
+    ref = TF.conv2d(torch.tensor(x).double().permute(0, 3, 1, 2), torch.tensor(w1).double().permute(3, 2, 0, 1),
+                    torch.tensor(b1).double(), padding=1).permute(0, 2, 3, 1)
+    np.testing.assert_allclose(both.numpy(), (torch.relu(ref) + 0.5 * ref).numpy(), rtol=1e-5, atol=1e-5)
+    engine.clear_plan_cache()
+
+
 def test_slices_of_the_contraction_axis():
     """How the planner splits K: products with fewer than 128 tiles of 128 x 128 and a long K
     until the launch has 512 workgroups; weight gradients x^T dy (both operands row-contiguous)
