@@ -847,6 +847,49 @@ def test_reduce_mid_batch_matches_single_launches(hip):
         lib.check(L.nbk_reduce_mid_batch(tasks, 0, st))
 
 
+@pytest.mark.parametrize("cin,cout,stride", [(16, 24, 1), (3, 8, 2), (32, 64, 1)])
+def test_conv_forward_with_relu_through_the_c_abi(hip, cin, cout, stride):
+    """`nbk_conv_desc.act = NBK_ACT_RELU`: max(conv(x, w) + bias, 0), bit for bit the relu of what
+    the same launch without the activation stores, against torch in float64; the two gradient
+    entry points refuse an activation."""
+    import torch.nn.functional as F
+    from nabla_amd.backend import lib
+    rng = np.random.default_rng(17)
+    N, H, W = 4, 11, 9
+    x = torch.tensor(rng.standard_normal((N, H, W, cin)), dtype=torch.float32)
+    w = torch.tensor(rng.standard_normal((3, 3, cin, cout)) * 0.3, dtype=torch.float32)
+    b = torch.tensor(rng.standard_normal((cout,)), dtype=torch.float32)
+    Ho, Wo = (H + 2 - 3) // stride + 1, (W + 2 - 3) // stride + 1
+    d = lib.ConvDesc()
+    d.N, d.H, d.W, d.Cin, d.R, d.S, d.Cout, d.Ho, d.Wo = N, H, W, cin, 3, 3, cout, Ho, Wo
+    d.stride_h = d.stride_w = stride
+    d.pad_t = d.pad_b = d.pad_l = d.pad_r = 1
+    d.dtype = 0
+    L = lib.load()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    outs = []
+    for act in (0, 1):
+        d.act = act
+        y = torch.full((N, Ho, Wo, cout), float("nan"), dtype=torch.float32, device="cuda")
+        lib.check(L.nbk_conv2d_fwd(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(wd.data_ptr()),
+                                   C.c_void_p(bd.data_ptr()), C.c_void_p(y.data_ptr()), st))
+        torch.cuda.synchronize()
+        outs.append(y.cpu())
+    assert torch.equal(outs[1], torch.relu(outs[0]))
+    ref = F.conv2d(x.double().permute(0, 3, 1, 2), w.double().permute(3, 2, 0, 1), b.double(),
+                   stride=stride, padding=1).permute(0, 2, 3, 1)
+    assert (outs[1].double() - torch.relu(ref)).abs().max().item() <= 1e-5 * ref.abs().max().item()
+    d.act = 1
+    dx = torch.empty_like(xd)
+    assert L.nbk_conv2d_dgrad(C.byref(d), C.c_void_p(outs[0].cuda().data_ptr()), C.c_void_p(wd.data_ptr()),
+                              C.c_void_p(dx.data_ptr()), st) != 0
+    d.act = 7
+    y = torch.empty((N, Ho, Wo, cout), dtype=torch.float32, device="cuda")
+    assert L.nbk_conv2d_fwd(C.byref(d), C.c_void_p(xd.data_ptr()), C.c_void_p(wd.data_ptr()),
+                            C.c_void_p(bd.data_ptr()), C.c_void_p(y.data_ptr()), st) != 0
+
+
 def test_conv_wgrad_workspace_and_fallback(hip):
     """The K-split filter gradient (with workspace) and the unsplit one (workspace NULL)
     agree to summation-order noise, and both match a float64 reference."""
