@@ -25,6 +25,29 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 enum { CONV_FWD = 0, CONV_DGRAD = 1, CONV_WGRAD = 2 };
 
+// Division of a number below 2^31 by a divisor fixed for the launch as a multiplication: the
+// host finds mul = ceil(2^(31 + shift) / d) with shift = ceil(log2 d), which fits 32 bits, and
+// n / d = (n * mul) >> (31 + shift) exactly for 0 <= n < 2^31 (five instructions where the
+// division takes twenty-odd).
+struct ConvDiv {
+  uint32_t mul, shift, d, pad;
+  __host__ void set(int64_t div) {
+    d = (uint32_t)div;
+    shift = 0;
+    while ((1ull << shift) < (uint64_t)div) ++shift;
+    mul = (uint32_t)(((1ull << (31 + shift)) + (uint64_t)div - 1) / (uint64_t)div);
+  }
+  __device__ __forceinline__ int quot(int n) const {
+    return (int)(((uint64_t)(uint32_t)n * mul) >> (31 + shift));
+  }
+  // quotient and remainder of n >= 0
+  __device__ __forceinline__ int divmod(int n, int& rem) const {
+    const int q = quot(n);
+    rem = n - q * (int)d;
+    return q;
+  }
+};
+
 struct ConvArgs {
   nbk_conv_desc d;
   const float* a;     // x (fwd, wgrad) or dy (dgrad)
@@ -34,6 +57,11 @@ struct ConvArgs {
   int64_t M, Ng, K;
   int64_t k_per_split;  // multiple of 16
   int32_t tiles_m, tiles_n, splits;
+  ConvDiv by_cin, by_cout, by_s, by_w, by_h, by_wo, by_ho;
+  __host__ void set_divisors() {
+    by_cin.set(d.Cin); by_cout.set(d.Cout); by_s.set(d.S);
+    by_w.set(d.W); by_h.set(d.H); by_wo.set(d.Wo); by_ho.set(d.Ho);
+  }
 };
 
 // ---- element-wise gather (any channel count) ----------------------------------------------
@@ -47,34 +75,31 @@ __device__ __forceinline__ float conv_load_a(const ConvArgs& g, int64_t m64, int
   const int Cin = (int)d.Cin, Cout = (int)d.Cout, S = (int)d.S, H = (int)d.H, W = (int)d.W,
             Ho = (int)d.Ho, Wo = (int)d.Wo;
   if (MODE == CONV_FWD) {
-    const int c = k % Cin;
-    const int rs = k / Cin;
-    const int s = rs % S, r = rs / S;
-    const int wo = m % Wo;
-    const int t = m / Wo;
-    const int ho = t % Ho, n = t / Ho;
+    int c, s, wo, ho;
+    const int rs = g.by_cin.divmod(k, c);
+    const int r = g.by_s.divmod(rs, s);
+    const int t = g.by_wo.divmod(m, wo);
+    const int n = g.by_ho.divmod(t, ho);
     const int h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
     if (h < 0 || h >= H || w < 0 || w >= W) return 0.f;
     return g.a[(int64_t)((n * H + h) * W + w) * Cin + c];
   } else if (MODE == CONV_DGRAD) {
-    const int co = k % Cout;
-    const int rs = k / Cout;
-    const int s = rs % S, r = rs / S;
-    const int w = m % W;
-    const int t = m / W;
-    const int h = t % H, n = t / H;
+    int co, s, w, h;
+    const int rs = g.by_cout.divmod(k, co);
+    const int r = g.by_s.divmod(rs, s);
+    const int t = g.by_w.divmod(m, w);
+    const int n = g.by_h.divmod(t, h);
     const int hn = h + d.pad_t - r, wn = w + d.pad_l - s;
     if (hn < 0 || wn < 0 || hn % d.stride_h != 0 || wn % d.stride_w != 0) return 0.f;
     const int ho = hn / d.stride_h, wo = wn / d.stride_w;
     if (ho >= Ho || wo >= Wo) return 0.f;
     return g.a[(int64_t)((n * Ho + ho) * Wo + wo) * Cout + co];
   } else {
-    const int c = m % Cin;
-    const int rs = m / Cin;
-    const int s = rs % S, r = rs / S;
-    const int wo = k % Wo;
-    const int t = k / Wo;
-    const int ho = t % Ho, n = t / Ho;
+    int c, s, wo, ho;
+    const int rs = g.by_cin.divmod(m, c);
+    const int r = g.by_s.divmod(rs, s);
+    const int t = g.by_wo.divmod(k, wo);
+    const int n = g.by_ho.divmod(t, ho);
     const int h = ho * d.stride_h - d.pad_t + r, w = wo * d.stride_w - d.pad_l + s;
     if (h < 0 || h >= H || w < 0 || w >= W) return 0.f;
     return g.a[(int64_t)((n * H + h) * W + w) * Cin + c];
@@ -87,7 +112,8 @@ __device__ __forceinline__ float conv_load_b(const ConvArgs& g, int64_t k, int64
   if (k >= k_end || j >= g.Ng) return 0.f;
   if (MODE == CONV_FWD) return g.b[k * d.Cout + j];  // w viewed as [R*S*Cin, Cout]
   if (MODE == CONV_DGRAD) {
-    const int co = (int)k % (int)d.Cout, rs = (int)k / (int)d.Cout;
+    int co;
+    const int rs = g.by_cout.divmod((int)k, co);
     return g.b[((int64_t)rs * d.Cin + j) * d.Cout + co];
   }
   return g.b[k * d.Cout + j];  // dy viewed as [N*Ho*Wo, Cout]
@@ -380,6 +406,7 @@ template <int MODE>
 static int conv_launch(ConvArgs& a, bool fast, hipStream_t st) {
   // the narrow workgroup tile when the last 128-wide column tile would be at most half full,
   // or when the wide tiling gives fewer workgroups than the GPU has CUs
+  a.set_divisors();
   const int64_t wide = ((a.M + 127) / 128) * ((a.Ng + 127) / 128) * a.splits;
   const bool narrow = (a.Ng - 1) % 128 < 64 || wide < nbk_num_cus();
   const int bn = narrow ? 64 : 128;
