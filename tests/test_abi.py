@@ -146,6 +146,19 @@ def test_generated_kernels_cover_every_row_program_of_the_benchmark_steps():
     assert not missing, "row programs without a specialised kernel: " + "; ".join(missing)
 
 
+def test_the_committed_traffic_counters_belong_to_the_kernel_the_stress_step_runs():
+    """`bench.py` reports the HBM traffic of the stress step from `profiles/hbm_traffic_c2.json`,
+    which names the kernel (by program hash) whose counters it holds.  A planner or op change
+    that alters that row program must come with new counter runs, or the bench line would
+    silently lose the figure."""
+    import json
+    from nabla_amd.backend import specialize
+    with open(ROOT / "profiles" / "hbm_traffic_c2.json") as f:
+        named = json.load(f)["kernel"]
+    hashes = [f"{h:016x}" for h in specialize.collect_programs()]
+    assert any(h in named for h in hashes), f"{named} is not a row program of the benchmark steps"
+
+
 def _program_record(a):
     """The ctypes record of a planned row program, built as the executor builds it (operands at
     an aligned dummy address: nothing is launched)."""
